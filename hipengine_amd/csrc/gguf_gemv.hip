@@ -1,0 +1,193 @@
+// C entry points of the dense q8_1 decode GEMV (Q4_K / Q6_K / Q8_0, batch 1..8)
+// and the launch planner that maps a shape to a workgroup layout.
+// The kernel body lives in gguf_gemv.hpp.
+
+#include "gguf_gemv.hpp"
+
+#include "../../include/hipengine_gfx950.h"
+
+namespace {
+
+using namespace hipengine_gfx950;
+
+// Workgroup size cap per instantiation: the weight registers of a chunk
+// (R*CB blocks) plus the per-batch-row activation reads have to fit the VGPR
+// budget that the cap implies (128 registers at 1024 threads, 256 at 512).
+template <int QT, int B, int R, int CB>
+constexpr int gemv_max_threads() {
+  return (R * CB * GemvTraits<QT>::REGS <= 64 && B <= 2) ? 1024 : 512;
+}
+
+template <int QT, int B, int R, int CB>
+__global__ void __launch_bounds__((gemv_max_threads<QT, B, R, CB>())) gemv_kernel(GemvArgs a) {
+  extern __shared__ __align__(16) uint8_t smem[];
+  gemv_workgroup<QT, B, R, CB>(a, a.w, blockIdx.x * a.nrg * 16 * R, smem);
+}
+
+using KernelFn = void (*)(GemvArgs);
+
+struct Variant {
+  int b, r, cb;
+  int max_threads;
+  KernelFn fn;
+};
+
+#define GEMV_VARIANT(QT, B, R, CB) \
+  Variant { B, R, CB, gemv_max_threads<QT, B, R, CB>(), gemv_kernel<QT, B, R, CB> }
+
+#define GEMV_VARIANTS_FOR(QT)                                                              \
+  GEMV_VARIANT(QT, 1, 1, 1), GEMV_VARIANT(QT, 1, 1, 2), GEMV_VARIANT(QT, 1, 1, 5),          \
+  GEMV_VARIANT(QT, 1, 2, 1), GEMV_VARIANT(QT, 1, 2, 2), GEMV_VARIANT(QT, 1, 2, 5),          \
+  GEMV_VARIANT(QT, 2, 1, 1), GEMV_VARIANT(QT, 2, 1, 2), GEMV_VARIANT(QT, 2, 1, 5),          \
+  GEMV_VARIANT(QT, 2, 2, 1), GEMV_VARIANT(QT, 2, 2, 2), GEMV_VARIANT(QT, 2, 2, 5),          \
+  GEMV_VARIANT(QT, 4, 1, 1), GEMV_VARIANT(QT, 4, 1, 2), GEMV_VARIANT(QT, 4, 1, 5),          \
+  GEMV_VARIANT(QT, 4, 2, 1), GEMV_VARIANT(QT, 4, 2, 2), GEMV_VARIANT(QT, 4, 2, 5),          \
+  GEMV_VARIANT(QT, 8, 1, 1), GEMV_VARIANT(QT, 8, 1, 2), GEMV_VARIANT(QT, 8, 1, 5),          \
+  GEMV_VARIANT(QT, 8, 2, 1), GEMV_VARIANT(QT, 8, 2, 2), GEMV_VARIANT(QT, 8, 2, 5)
+
+const Variant kQ4K[] = {GEMV_VARIANTS_FOR(GGML_Q4_K)};
+const Variant kQ6K[] = {GEMV_VARIANTS_FOR(GGML_Q6_K)};
+const Variant kQ80[] = {GEMV_VARIANTS_FOR(GGML_Q8_0)};
+constexpr int kVariants = 24;
+
+const Variant* find_variant(int qt, int b, int r, int cb) {
+  const Variant* table = qt == GGML_Q4_K ? kQ4K : qt == GGML_Q6_K ? kQ6K : qt == GGML_Q8_0 ? kQ80 : nullptr;
+  if (!table) return nullptr;
+  for (int i = 0; i < kVariants; ++i)
+    if (table[i].b == b && table[i].r == r && table[i].cb == cb) return &table[i];
+  return nullptr;
+}
+
+int batch_bucket(int rows) { return rows <= 1 ? 1 : rows <= 2 ? 2 : rows <= 4 ? 4 : 8; }
+
+struct Plan {
+  int b, r, cb, ks, nrg;
+};
+
+// Default layout for a shape.  ks K-slices of CB blocks each cover one chunk;
+// the row-group count is lowered until the launch has at least ~2 workgroups
+// per CU (256 CUs) or reaches one row group.
+Plan default_plan(int qt, int rows, int64_t K, int64_t N) {
+  Plan p;
+  const int nb = static_cast<int>(K / QK_K);
+  p.b = batch_bucket(rows);
+  p.r = p.b == 4 ? 2 : 1;
+  p.ks = nb >= 4 ? 4 : nb;
+  const int per_wave = (nb + p.ks - 1) / p.ks;
+  p.cb = per_wave >= 5 ? 5 : per_wave >= 2 ? 2 : 1;
+  if (p.r == 2 && p.cb > 2) p.cb = 2;   // keep R*CB blocks of weights within the register budget
+  const Variant* v = find_variant(qt, p.b, p.r, p.cb);
+  const int max_threads = v ? v->max_threads : 512;
+  int nrg = max_threads / 64 / p.ks;
+  if (nrg < 1) nrg = 1;
+  while (nrg > 1 && (N + nrg * 16 * p.r - 1) / (nrg * 16 * p.r) < 512) nrg >>= 1;
+  p.nrg = nrg;
+  return p;
+}
+
+int launch_gemv(int qt, const void* x, int x_kind, const uint8_t* w, void* out, int out_kind, int64_t rows, int64_t K,
+                int64_t N, const Plan* forced, hipStream_t stream) {
+  if (!x || !w || !out || rows <= 0 || K <= 0 || N <= 0 || (K % QK_K) != 0 || K > (1 << 24) || N > (1 << 30)) {
+    return static_cast<int>(hipErrorInvalidValue);
+  }
+  const int64_t x_row_bytes = x_kind == KIND_Q8_1 ? K / 32 * Q8_1_BYTES : K * (x_kind == KIND_F32 ? 4 : 2);
+  const int64_t out_elem = out_kind == KIND_F32 ? 4 : 2;
+  for (int64_t r0 = 0; r0 < rows; r0 += 8) {
+    const int chunk = static_cast<int>(rows - r0 < 8 ? rows - r0 : 8);
+    Plan p = forced ? *forced : default_plan(qt, chunk, K, N);
+    if (forced) p.b = batch_bucket(chunk);
+    const Variant* v = find_variant(qt, p.b, p.r, p.cb);
+    if (!v || p.ks < 1 || p.nrg < 1 || p.ks * p.nrg * 64 > v->max_threads) {
+      return static_cast<int>(hipErrorInvalidValue);
+    }
+    GemvArgs a;
+    a.x = static_cast<const uint8_t*>(x) + r0 * x_row_bytes;
+    a.w = w;
+    a.out = static_cast<uint8_t*>(out) + r0 * N * out_elem;
+    a.x_kind = x_kind;
+    a.out_kind = out_kind;
+    a.rows = chunk;
+    a.K = static_cast<int>(K);
+    a.N = static_cast<int>(N);
+    a.ks = p.ks;
+    a.nrg = p.nrg;
+    const int rows_wg = p.nrg * 16 * p.r;
+    const unsigned grid = static_cast<unsigned>((N + rows_wg - 1) / rows_wg);
+    const size_t lds = gemv_lds_bytes(qt, p.b, p.r, p.cb, p.ks, p.nrg);
+    if (lds > 64 * 1024) return static_cast<int>(hipErrorInvalidValue);
+    hipLaunchKernelGGL(v->fn, dim3(grid), dim3(p.ks * p.nrg * 64), lds, stream, a);
+    const hipError_t err = hipGetLastError();
+    if (err != hipSuccess) return static_cast<int>(err);
+  }
+  return static_cast<int>(hipSuccess);
+}
+
+}  // namespace
+
+// ---- fused: float activations in, q8_1 quantization inside the kernel -------
+
+#define DEFINE_FUSED(QNAME, QT, ANAME, AKIND, ONAME, OKIND)                                              \
+  extern "C" int hipengine_gguf_##QNAME##_q8_1_fused_gemv_##ANAME##_##ONAME##_out(                        \
+      const void* x, const uint8_t* qweight, void* out, int64_t rows, int64_t in_features,                \
+      int64_t out_features, int64_t threads, hipStream_t stream) {                                        \
+    (void)threads;                                                                                        \
+    return launch_gemv(QT, x, AKIND, qweight, out, OKIND, rows, in_features, out_features, nullptr,       \
+                       stream);                                                                           \
+  }
+
+#define DEFINE_FUSED_ALL(QNAME, QT)                       \
+  DEFINE_FUSED(QNAME, QT, f32, KIND_F32, f32, KIND_F32)   \
+  DEFINE_FUSED(QNAME, QT, bf16, KIND_BF16, f32, KIND_F32) \
+  DEFINE_FUSED(QNAME, QT, bf16, KIND_BF16, bf16, KIND_BF16) \
+  DEFINE_FUSED(QNAME, QT, bf16, KIND_BF16, fp16, KIND_F16) \
+  DEFINE_FUSED(QNAME, QT, fp16, KIND_F16, f32, KIND_F32)  \
+  DEFINE_FUSED(QNAME, QT, fp16, KIND_F16, fp16, KIND_F16)
+
+DEFINE_FUSED_ALL(q4_k, GGML_Q4_K)
+DEFINE_FUSED_ALL(q6_k, GGML_Q6_K)
+DEFINE_FUSED_ALL(q8_0, GGML_Q8_0)
+
+// ---- pre-quantized q8_1 activations (36-byte blocks) ------------------------
+
+#define DEFINE_Q8_1(SYMBOL, QT, OKIND)                                                                   \
+  extern "C" int SYMBOL(const void* xq, const uint8_t* qweight, void* out, int64_t rows,                 \
+                        int64_t in_features, int64_t out_features, hipStream_t stream) {                 \
+    return launch_gemv(QT, xq, KIND_Q8_1, qweight, out, OKIND, rows, in_features, out_features, nullptr, \
+                       stream);                                                                          \
+  }
+
+DEFINE_Q8_1(hipengine_gguf_q4_k_q8_1_dp4a_vdr_bf16_f32_out, GGML_Q4_K, KIND_F32)
+DEFINE_Q8_1(hipengine_gguf_q4_k_q8_1_dp4a_vdr_bf16_bf16_out, GGML_Q4_K, KIND_BF16)
+DEFINE_Q8_1(hipengine_gguf_q6_k_q8_1_dp4a_gemv_bf16_f32_out, GGML_Q6_K, KIND_F32)
+DEFINE_Q8_1(hipengine_gguf_q6_k_q8_1_dp4a_gemv_bf16_bf16_out, GGML_Q6_K, KIND_BF16)
+DEFINE_Q8_1(hipengine_gguf_q8_0_dp4a_gemv_f32_f32_out, GGML_Q8_0, KIND_F32)
+DEFINE_Q8_1(hipengine_gguf_q8_0_dp4a_gemv_bf16_bf16_out, GGML_Q8_0, KIND_BF16)
+
+// ---- explicit layout, for tuning sweeps --------------------------------------
+
+extern "C" int hipengine_gfx950_gguf_q8_1_fused_gemv_tuned(
+    int32_t ggml_type, const void* x, int32_t x_kind, const uint8_t* qweight, void* out, int32_t out_kind,
+    int64_t rows, int64_t in_features, int64_t out_features, int32_t k_slices, int32_t row_groups,
+    int32_t blocks_per_wave, int32_t rows_per_lane, hipStream_t stream) {
+  if (x_kind < KIND_F32 || x_kind > KIND_Q8_1 || out_kind < KIND_F32 || out_kind > KIND_F16 || rows > 8) {
+    return static_cast<int>(hipErrorInvalidValue);
+  }
+  Plan p;
+  p.b = 0;
+  p.r = rows_per_lane;
+  p.cb = blocks_per_wave;
+  p.ks = k_slices;
+  p.nrg = row_groups;
+  return launch_gemv(ggml_type, x, x_kind, qweight, out, out_kind, rows, in_features, out_features, &p, stream);
+}
+
+extern "C" int hipengine_gfx950_gguf_gemv_default_plan(int32_t ggml_type, int64_t rows, int64_t in_features,
+                                                       int64_t out_features, int32_t* plan5) {
+  if (!plan5 || rows <= 0 || in_features <= 0 || (in_features % QK_K) != 0 || out_features <= 0 ||
+      !find_variant(ggml_type, 1, 1, 1)) {
+    return static_cast<int>(hipErrorInvalidValue);
+  }
+  const Plan p = default_plan(ggml_type, static_cast<int>(rows < 8 ? rows : 8), in_features, out_features);
+  plan5[0] = p.b; plan5[1] = p.r; plan5[2] = p.cb; plan5[3] = p.ks; plan5[4] = p.nrg;
+  return static_cast<int>(hipSuccess);
+}

@@ -1,0 +1,163 @@
+// Stand-alone q8_1 activation quantizers for gfx950: the 36-byte GEMV
+// convention, the 144-byte DS4 (MMQ) convention and the 160-byte D4S4 one.
+// Eight lanes share a 32-value group (four consecutive values per lane, one
+// 16-byte or 8-byte load), so a wave covers eight groups per pass and the
+// group reductions are DPP only.
+
+#include "gguf_common.hpp"
+
+#include "../../include/hipengine_gfx950.h"
+
+namespace {
+
+using namespace hipengine_gfx950;
+
+__device__ __forceinline__ void load4_values(const void* x, int kind, int64_t idx, float (&v)[4]) {
+  if (kind == KIND_F32) {
+    const float4 t = *reinterpret_cast<const float4*>(static_cast<const float*>(x) + idx);
+    v[0] = t.x; v[1] = t.y; v[2] = t.z; v[3] = t.w;
+  } else {
+    const uint2 t = *reinterpret_cast<const uint2*>(static_cast<const uint16_t*>(x) + idx);
+    if (kind == KIND_BF16) {
+      v[0] = bf16_bits_to_float(t.x & 0xFFFFu); v[1] = bf16_bits_to_float(t.x >> 16);
+      v[2] = bf16_bits_to_float(t.y & 0xFFFFu); v[3] = bf16_bits_to_float(t.y >> 16);
+    } else {
+      v[0] = f16_bits_to_float(t.x & 0xFFFFu); v[1] = f16_bits_to_float(t.x >> 16);
+      v[2] = f16_bits_to_float(t.y & 0xFFFFu); v[3] = f16_bits_to_float(t.y >> 16);
+    }
+  }
+}
+
+__device__ __forceinline__ uint32_t pack_i8x4(int a, int b, int c, int d) {
+  return (a & 0xFF) | ((b & 0xFF) << 8) | ((c & 0xFF) << 16) | (static_cast<uint32_t>(d & 0xFF) << 24);
+}
+
+// 36-byte blocks.  Grid: x = ceil(groups / 32), 256 threads = 32 groups.
+__global__ void __launch_bounds__(256) quantize_q8_1_kernel(const void* __restrict__ x, int kind,
+                                                            uint8_t* __restrict__ xq, int64_t total_groups) {
+  const int64_t g = static_cast<int64_t>(blockIdx.x) * 32 + (threadIdx.x >> 3);
+  const int e = threadIdx.x & 7;
+  if (g >= total_groups) return;   // uniform for the 8 lanes of a group
+  float v[4];
+  load4_values(x, kind, g * 32 + e * 4, v);
+  const float amax = oct_max(fmaxf(fmaxf(fabsf(v[0]), fabsf(v[1])), fmaxf(fabsf(v[2]), fabsf(v[3]))));
+  const float sum = oct_tree_sum32(v[0], v[1], v[2], v[3]);
+  const float d = amax / 127.0f;
+  uint32_t packed = 0;
+  if (amax != 0.0f) {
+    packed = pack_i8x4(max(-128, min(127, static_cast<int>(roundf(v[0] / d)))),
+                       max(-128, min(127, static_cast<int>(roundf(v[1] / d)))),
+                       max(-128, min(127, static_cast<int>(roundf(v[2] / d)))),
+                       max(-128, min(127, static_cast<int>(roundf(v[3] / d)))));
+  }
+  uint8_t* blk = xq + g * Q8_1_BYTES;
+  *reinterpret_cast<uint32_t*>(blk + 4 + 4 * e) = packed;
+  if (e == 0) {
+    *reinterpret_cast<uint32_t*>(blk) =
+        static_cast<uint32_t>(float_to_f16_bits(d)) | (static_cast<uint32_t>(float_to_f16_bits(sum)) << 16);
+  }
+}
+
+constexpr float kFp16Max = 65504.0f;
+
+// DS4 (ties-to-even, clamp +-127, fp16 scale and sum) or D4S4 (ties away,
+// clamp -128..127, float32 scale and sum).  One group of 8 lanes per 32 values;
+// a 128-value block is four consecutive groups.
+template <bool D4S4>
+__global__ void __launch_bounds__(256) pack_mmq_kernel(const uint16_t* __restrict__ x, uint8_t* __restrict__ out,
+                                                       int64_t total_groups) {
+  const int64_t g = static_cast<int64_t>(blockIdx.x) * 32 + (threadIdx.x >> 3);
+  const int e = threadIdx.x & 7;
+  if (g >= total_groups) return;
+  float v[4];
+  load4_values(x, KIND_BF16, g * 32 + e * 4, v);
+  const float amax = oct_max(fmaxf(fmaxf(fabsf(v[0]), fabsf(v[1])), fmaxf(fabsf(v[2]), fabsf(v[3]))));
+  const int64_t blk_idx = g >> 2;
+  const int grp = static_cast<int>(g & 3);
+  if constexpr (D4S4) {
+    // four sequential adds per lane, then an xor tree over the 8 lanes (4, 2, 1)
+    float s = ((v[0] + v[1]) + v[2]) + v[3];
+    s += dpp_f<DPP_ROW_SHL4>(s);
+    s += dpp_f<DPP_ROW_SHL2>(s);
+    s += dpp_f<DPP_ROW_SHL1>(s);
+    const float d = amax == 0.0f ? 0.0f : amax / 127.0f;
+    uint32_t packed = 0;
+    if (d != 0.0f) {
+      packed = pack_i8x4(max(-128, min(127, static_cast<int>(roundf(v[0] / d)))),
+                         max(-128, min(127, static_cast<int>(roundf(v[1] / d)))),
+                         max(-128, min(127, static_cast<int>(roundf(v[2] / d)))),
+                         max(-128, min(127, static_cast<int>(roundf(v[3] / d)))));
+    }
+    uint8_t* blk = out + blk_idx * D4S4_BYTES;
+    *reinterpret_cast<uint32_t*>(blk + 32 + grp * 32 + 4 * e) = packed;
+    if (e == 0) {
+      *reinterpret_cast<float*>(blk + 4 * grp) = d;
+      *reinterpret_cast<float*>(blk + 16 + 4 * grp) = s;
+    }
+  } else {
+    const float sum = fminf(kFp16Max, fmaxf(-kFp16Max, oct_tree_sum32(v[0], v[1], v[2], v[3])));
+    const float scale = fminf(kFp16Max, amax / 127.0f);
+    uint32_t packed = 0;
+    if (scale > 0.0f) {
+      packed = pack_i8x4(static_cast<int>(fminf(127.0f, fmaxf(-127.0f, rintf(v[0] / scale)))),
+                         static_cast<int>(fminf(127.0f, fmaxf(-127.0f, rintf(v[1] / scale)))),
+                         static_cast<int>(fminf(127.0f, fmaxf(-127.0f, rintf(v[2] / scale)))),
+                         static_cast<int>(fminf(127.0f, fmaxf(-127.0f, rintf(v[3] / scale)))));
+    }
+    uint8_t* blk = out + blk_idx * DS4_BYTES;
+    *reinterpret_cast<uint32_t*>(blk + 16 + grp * 32 + 4 * e) = packed;
+    if (e == 0) {
+      *reinterpret_cast<uint32_t*>(blk + 4 * grp) =
+          static_cast<uint32_t>(float_to_f16_bits(scale)) | (static_cast<uint32_t>(float_to_f16_bits(sum)) << 16);
+    }
+  }
+}
+
+int launch_q8_1(const void* x, int kind, void* xq, int64_t rows, int64_t in_features, hipStream_t stream) {
+  if (!x || !xq || rows <= 0 || in_features <= 0 || (in_features % 32) != 0) {
+    return static_cast<int>(hipErrorInvalidValue);
+  }
+  const int64_t groups = rows * (in_features / 32);
+  const int64_t grid = (groups + 31) / 32;
+  if (grid > 0x7FFFFFFF) return static_cast<int>(hipErrorInvalidValue);
+  hipLaunchKernelGGL(quantize_q8_1_kernel, dim3(static_cast<unsigned>(grid)), dim3(256), 0, stream, x, kind,
+                     static_cast<uint8_t*>(xq), groups);
+  return static_cast<int>(hipGetLastError());
+}
+
+template <bool D4S4>
+int launch_pack(const void* x, void* out, int64_t rows, int64_t hidden, hipStream_t stream) {
+  if (!x || !out || rows <= 0 || hidden <= 0 || (hidden % 128) != 0) {
+    return static_cast<int>(hipErrorInvalidValue);
+  }
+  const int64_t groups = rows * (hidden / 32);
+  const int64_t grid = (groups + 31) / 32;
+  if (grid > 0x7FFFFFFF) return static_cast<int>(hipErrorInvalidValue);
+  hipLaunchKernelGGL(pack_mmq_kernel<D4S4>, dim3(static_cast<unsigned>(grid)), dim3(256), 0, stream,
+                     static_cast<const uint16_t*>(x), static_cast<uint8_t*>(out), groups);
+  return static_cast<int>(hipGetLastError());
+}
+
+}  // namespace
+
+extern "C" int hipengine_gfx950_abi_version(void) { return 1; }
+
+extern "C" int hipengine_gguf_q4_k_quantize_f32_q8_1(const void* x, void* xq, int64_t rows, int64_t in_features,
+                                                     hipStream_t stream) {
+  return launch_q8_1(x, KIND_F32, xq, rows, in_features, stream);
+}
+
+extern "C" int hipengine_gguf_q4_k_quantize_bf16_q8_1(const void* x, void* xq, int64_t rows, int64_t in_features,
+                                                      hipStream_t stream) {
+  return launch_q8_1(x, KIND_BF16, xq, rows, in_features, stream);
+}
+
+extern "C" int hipengine_gguf_q8_1_mmq_ds4_pack_bf16(const void* x, void* out, int64_t rows, int64_t hidden,
+                                                     hipStream_t stream) {
+  return launch_pack<false>(x, out, rows, hidden, stream);
+}
+
+extern "C" int hipengine_gguf_q8_1_d4s4_f32_quantize_bf16(const void* x, void* out, int64_t rows, int64_t hidden,
+                                                          hipStream_t stream) {
+  return launch_pack<true>(x, out, rows, hidden, stream);
+}

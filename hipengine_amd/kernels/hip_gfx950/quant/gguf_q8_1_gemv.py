@@ -1,0 +1,130 @@
+"""Decode GEMV wrappers (batch 1..8 per launch) for Q4_K / Q6_K / Q8_0 weights
+with q8_1 activations.
+
+Two families, both with hipEngine's dense wrapper signature
+``fn(x_ptr, qweight_ptr, out_ptr, rows, in_features, out_features, *, threads,
+stream, library, runtime)`` (``kernels/hip_gfx1100/quant/gguf_q4_k_gemv.py:115-142``):
+
+* ``gguf_<q>_q8_1_fused_gemv_<act>_<out>_out`` take float activations and
+  quantize them to q8_1 inside the kernel;
+* ``gguf_q4_k_q8_1_dp4a_vdr_*``, ``gguf_q6_k_q8_1_dp4a_gemv_*`` and
+  ``gguf_q8_0_dp4a_gemv_*`` take pre-quantized 36-byte q8_1 blocks, as
+  hipEngine's ``gguf_q4_k_q8_1_dp4a_vdr_gemv.py`` / ``gguf_q8_0_dp4a_gemv.py`` do.
+"""
+
+from __future__ import annotations
+
+import ctypes
+
+from hipengine_amd.core.hip import HipRuntime
+from hipengine_amd.kernels.hip_gfx950._launch import (
+    I32,
+    I64,
+    KIND_BF16,
+    KIND_F16,
+    KIND_F32,
+    KIND_Q8_1,
+    QUANT_KEY_TO_GGML,
+    VOID,
+    check_launch,
+    entry,
+    validate_linear,
+    validate_pointers,
+)
+from hipengine_amd.kernels.registry import KernelKey, register
+
+_FUSED_ARGS = [VOID, VOID, VOID, I64, I64, I64, I64, VOID]
+_Q8_1_ARGS = [VOID, VOID, VOID, I64, I64, I64, VOID]
+_QUANTS = ("q4_k", "q6_k", "q8_0")
+_FUSED_DTYPES = (("f32", "f32"), ("bf16", "f32"), ("bf16", "bf16"), ("bf16", "fp16"), ("fp16", "f32"), ("fp16", "fp16"))
+_KINDS = {"f32": KIND_F32, "bf16": KIND_BF16, "fp16": KIND_F16, "q8_1": KIND_Q8_1}
+
+
+def _make_fused(quant: str, act: str, out: str):
+    symbol = f"hipengine_gguf_{quant}_q8_1_fused_gemv_{act}_{out}_out"
+
+    def wrapper(x_ptr: int, qweight_ptr: int, out_ptr: int, rows: int, in_features: int, out_features: int, *,
+                threads: int = 128, stream: int = 0, library: ctypes.CDLL | None = None,
+                runtime: HipRuntime | None = None) -> None:
+        validate_linear(rows, in_features, out_features, threads)
+        validate_pointers(x_ptr=x_ptr, qweight_ptr=qweight_ptr, out_ptr=out_ptr)
+        code = entry(symbol, _FUSED_ARGS, library)(x_ptr, qweight_ptr, out_ptr, rows, in_features, out_features,
+                                                   threads, stream)
+        check_launch(code, runtime)
+
+    wrapper.__name__ = f"gguf_{quant}_q8_1_fused_gemv_{act}_{out}_out"
+    wrapper.__doc__ = (f"GGUF {quant.upper()} GEMV, {act} activations quantized to q8_1 in the kernel, {out} output "
+                       f"(C symbol ``{symbol}``).")
+    return wrapper
+
+
+def _make_q8_1(name: str, symbol: str):
+    def wrapper(xq_ptr: int, qweight_ptr: int, out_ptr: int, rows: int, in_features: int, out_features: int, *,
+                threads: int = 128, stream: int = 0, library: ctypes.CDLL | None = None,
+                runtime: HipRuntime | None = None) -> None:
+        validate_linear(rows, in_features, out_features, threads)
+        validate_pointers(xq_ptr=xq_ptr, qweight_ptr=qweight_ptr, out_ptr=out_ptr)
+        check_launch(entry(symbol, _Q8_1_ARGS, library)(xq_ptr, qweight_ptr, out_ptr, rows, in_features, out_features,
+                                                        stream), runtime)
+
+    wrapper.__name__ = name
+    wrapper.__doc__ = f"GGUF GEMV over pre-quantized 36-byte q8_1 activation blocks (C symbol ``{symbol}``)."
+    return wrapper
+
+
+FUSED: dict[tuple[str, str, str], object] = {}
+for _q in _QUANTS:
+    for _a, _o in _FUSED_DTYPES:
+        _fn = _make_fused(_q, _a, _o)
+        FUSED[(_q, _a, _o)] = _fn
+        globals()[_fn.__name__] = _fn
+
+gguf_q4_k_q8_1_dp4a_vdr_bf16_f32_out = _make_q8_1(
+    "gguf_q4_k_q8_1_dp4a_vdr_bf16_f32_out", "hipengine_gguf_q4_k_q8_1_dp4a_vdr_bf16_f32_out")
+gguf_q4_k_q8_1_dp4a_vdr_bf16_bf16_out = _make_q8_1(
+    "gguf_q4_k_q8_1_dp4a_vdr_bf16_bf16_out", "hipengine_gguf_q4_k_q8_1_dp4a_vdr_bf16_bf16_out")
+gguf_q6_k_q8_1_dp4a_gemv_bf16_f32_out = _make_q8_1(
+    "gguf_q6_k_q8_1_dp4a_gemv_bf16_f32_out", "hipengine_gguf_q6_k_q8_1_dp4a_gemv_bf16_f32_out")
+gguf_q6_k_q8_1_dp4a_gemv_bf16_bf16_out = _make_q8_1(
+    "gguf_q6_k_q8_1_dp4a_gemv_bf16_bf16_out", "hipengine_gguf_q6_k_q8_1_dp4a_gemv_bf16_bf16_out")
+gguf_q8_0_dp4a_gemv_f32_f32_out = _make_q8_1(
+    "gguf_q8_0_dp4a_gemv_f32_f32_out", "hipengine_gguf_q8_0_dp4a_gemv_f32_f32_out")
+gguf_q8_0_dp4a_gemv_bf16_bf16_out = _make_q8_1(
+    "gguf_q8_0_dp4a_gemv_bf16_bf16_out", "hipengine_gguf_q8_0_dp4a_gemv_bf16_bf16_out")
+
+_TUNED_ARGS = [I32, VOID, I32, VOID, VOID, I32, I64, I64, I64, I32, I32, I32, I32, VOID]
+
+
+def gguf_q8_1_fused_gemv_tuned(quant_key: str, x_ptr: int, x_kind: str, qweight_ptr: int, out_ptr: int, out_kind: str,
+                               rows: int, in_features: int, out_features: int, *, k_slices: int, row_groups: int,
+                               blocks_per_wave: int, rows_per_lane: int, stream: int = 0,
+                               library: ctypes.CDLL | None = None, runtime: HipRuntime | None = None) -> None:
+    """The fused GEMV with an explicit workgroup layout (tuning sweeps only)."""
+    validate_linear(rows, in_features, out_features)
+    fn = entry("hipengine_gfx950_gguf_q8_1_fused_gemv_tuned", _TUNED_ARGS, library)
+    check_launch(fn(QUANT_KEY_TO_GGML[quant_key], x_ptr, _KINDS[x_kind], qweight_ptr, out_ptr, _KINDS[out_kind], rows,
+                    in_features, out_features, k_slices, row_groups, blocks_per_wave, rows_per_lane, stream), runtime)
+
+
+def gguf_gemv_default_plan(quant_key: str, rows: int, in_features: int, out_features: int, *,
+                           library: ctypes.CDLL | None = None) -> dict[str, int]:
+    """The workgroup layout the library picks for a shape (host only)."""
+    plan = (ctypes.c_int32 * 5)()
+    fn = entry("hipengine_gfx950_gguf_gemv_default_plan", [I32, I64, I64, I64, ctypes.POINTER(ctypes.c_int32)], library)
+    check_launch(fn(QUANT_KEY_TO_GGML[quant_key], rows, in_features, out_features, plan), None)
+    return dict(zip(("batch_bucket", "rows_per_lane", "blocks_per_wave", "k_slices", "row_groups"), plan))
+
+
+def register_kernels(backend: str = "hip_gfx950", *, replace: bool = False) -> None:
+    for (quant, act, out), fn in FUSED.items():
+        for prefix in ("q8_1_fused_gemv", "q8_1_fused_prefill"):
+            register(KernelKey(backend, "linear", f"gguf_{quant}", f"{prefix}_{act}_{out}_out"), fn, replace=replace)
+    for quant, variant, fn in (
+        ("gguf_q4_k", "q8_1_dp4a_vdr_bf16_f32_out", gguf_q4_k_q8_1_dp4a_vdr_bf16_f32_out),
+        ("gguf_q4_k", "q8_1_dp4a_vdr_bf16_bf16_out", gguf_q4_k_q8_1_dp4a_vdr_bf16_bf16_out),
+        ("gguf_q6_k", "q8_1_dp4a_gemv_bf16_f32_out", gguf_q6_k_q8_1_dp4a_gemv_bf16_f32_out),
+        ("gguf_q6_k", "q8_1_dp4a_gemv_bf16_bf16_out", gguf_q6_k_q8_1_dp4a_gemv_bf16_bf16_out),
+        ("gguf_q8_0", "q8_1_dp4a_gemv_f32_f32_out", gguf_q8_0_dp4a_gemv_f32_f32_out),
+        ("gguf_q8_0", "q8_1_dp4a_gemv_bf16_bf16_out", gguf_q8_0_dp4a_gemv_bf16_bf16_out),
+    ):
+        register(KernelKey(backend, "linear", quant, variant), fn, replace=replace)

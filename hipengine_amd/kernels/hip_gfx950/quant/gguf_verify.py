@@ -1,0 +1,40 @@
+"""Verification exports: device-side block dequantization and the int32
+sub-block dots of the q8_1 kernels, for bit-exact comparison with a CPU oracle."""
+
+from __future__ import annotations
+
+import ctypes
+
+from hipengine_amd.core.hip import HipRuntime
+from hipengine_amd.kernels.hip_gfx950._launch import (
+    I32,
+    I64,
+    QUANT_KEY_TO_GGML,
+    VOID,
+    check_launch,
+    entry,
+    validate_pointers,
+)
+
+
+def gguf_dequantize_f32(quant_key: str, blocks_ptr: int, out_ptr: int, n_blocks: int, *, stream: int = 0,
+                        library: ctypes.CDLL | None = None, runtime: HipRuntime | None = None) -> None:
+    """``n_blocks`` raw blocks -> float32 (256 values per Q4_K/Q6_K block, 32 per Q8_0 block)."""
+    if n_blocks <= 0:
+        raise ValueError("n_blocks must be positive")
+    validate_pointers(blocks_ptr=blocks_ptr, out_ptr=out_ptr)
+    fn = entry("hipengine_gfx950_gguf_dequantize_f32", [I32, VOID, VOID, I64, VOID], library)
+    check_launch(fn(QUANT_KEY_TO_GGML[quant_key], blocks_ptr, out_ptr, n_blocks, stream), runtime)
+
+
+def gguf_q8_1_block_dots_i32(quant_key: str, xq_ptr: int, qweight_ptr: int, dots_ptr: int, qsums_ptr: int, rows: int,
+                             in_features: int, out_features: int, *, stream: int = 0,
+                             library: ctypes.CDLL | None = None, runtime: HipRuntime | None = None) -> None:
+    """int32 sub-block dots ``[rows, out_features, K/32]`` (Q6_K: ``K/16``) and, when
+    ``qsums_ptr`` is non-zero, the int32 q8 sums ``[rows, K/32]``."""
+    if rows <= 0 or out_features <= 0 or in_features <= 0 or in_features % 256:
+        raise ValueError("rows/out_features must be positive and in_features divisible by 256")
+    validate_pointers(xq_ptr=xq_ptr, qweight_ptr=qweight_ptr, dots_ptr=dots_ptr)
+    fn = entry("hipengine_gfx950_gguf_q8_1_block_dots_i32", [I32, VOID, VOID, VOID, VOID, I64, I64, I64, VOID], library)
+    check_launch(fn(QUANT_KEY_TO_GGML[quant_key], xq_ptr, qweight_ptr, dots_ptr, qsums_ptr or None, rows, in_features,
+                    out_features, stream), runtime)

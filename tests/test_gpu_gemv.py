@@ -1,0 +1,221 @@
+"""GPU parity of the q8_1 decode GEMV (Q4_K / Q6_K / Q8_0) through the C ABI.
+
+Parity definition (the reference CPU backend has no q8_1 path, so it is
+extended the way the reference's own q8_1 tests do,
+tests/test_gpu_gguf_k_mmq_prefill.py:534-540):
+  1. q8_1 activation bytes: identical to the oracle's;
+  2. unpacked weights / dequantized float32: identical bit patterns;
+  3. int32 sub-block dots: identical;
+  4. float32 outputs: max relative error <= 1e-3 (floor 1e-3*max|ref|) and
+     cosine >= 0.99999 against the reference CPU GEMV (dequantize -> float32
+     matmul) applied to the q8_1-dequantized activations;
+  5. bf16 output == bf16_round(float32 output) bit for bit;
+  6. reported, with a loose floor as in the reference: KL / top-1 of
+     softmax(out) against the unquantized-activation reference.
+"""
+
+from __future__ import annotations
+
+import numpy as np
+import pytest
+
+from oracle import c_oracle as C
+from oracle import gguf_oracle as O
+from hipengine_amd.kernels.hip_gfx950.quant import gguf_q8_1_gemv as G
+from hipengine_amd.kernels.hip_gfx950.quant import gguf_quantize as Q
+from hipengine_amd.kernels.hip_gfx950.quant import gguf_verify as V
+
+pytestmark = pytest.mark.gpu
+
+REL_TOL = 1e-3
+COS_MIN = 0.99999
+QT = {"gguf_q4_k": O.GGML_Q4_K, "gguf_q6_k": O.GGML_Q6_K, "gguf_q8_0": O.GGML_Q8_0}
+SHORT = {"gguf_q4_k": "q4_k", "gguf_q6_k": "q6_k", "gguf_q8_0": "q8_0"}
+CLOSED = {"gguf_q4_k": O.closed_form_q4_k, "gguf_q6_k": O.closed_form_q6_k, "gguf_q8_0": O.closed_form_q8_0}
+
+
+def _check_f32(got, xq, w, qt, x_unq=None):
+    ref = O.gguf_quant_gemv(O.dequantize_q8_1(xq), w, qt)
+    err, cos = O.max_rel_err(got, ref), O.cosine(got, ref)
+    assert err <= REL_TOL, f"max rel err {err}"
+    assert cos >= COS_MIN, f"cosine {cos}"
+    if x_unq is not None and got.shape[1] >= 16:
+        kl, top1 = O.softmax_kl_top1(O.gguf_quant_gemv(x_unq, w, qt), got)
+        assert kl <= 0.05 and top1 >= 0.75, (kl, top1)   # outer floor only; parity is the gate above
+
+
+def _run_fused(dev, quant, x, w, act="f32", out="f32"):
+    rows, k = x.shape
+    n = w.shape[0]
+    xin = x if act == "f32" else O.f32_to_bf16_bits(x)
+    dx, dw = dev.put(xin), dev.put(w)
+    dout = dev.empty(rows * n * (4 if out == "f32" else 2))
+    G.FUSED[(SHORT[quant], act, out)](dx.ptr, dw.ptr, dout.ptr, rows, k, n)
+    res = dev.get(dout, np.float32 if out == "f32" else np.uint16, (rows, n))
+    dev.free(dx, dw, dout)
+    return res
+
+
+@pytest.mark.parametrize("quant", ["gguf_q4_k", "gguf_q6_k", "gguf_q8_0"])
+def test_dequantize_bit_exact(dev, quant):
+    qt = QT[quant]
+    for w in (CLOSED[quant](37, 768), O.random_weight(qt, 64, 1024, seed=11)):
+        block, nbytes = {8: (32, 34), 12: (256, 144), 14: (256, 210)}[qt]
+        n_blocks = w.size // nbytes
+        dw = dev.put(w)
+        dout = dev.empty(n_blocks * block * 4)
+        V.gguf_dequantize_f32(quant, dw.ptr, dout.ptr, n_blocks)
+        got = dev.get(dout, np.float32, (w.shape[0], w.shape[1] // nbytes * block))
+        dev.free(dw, dout)
+        want = O.dequantize(w, qt)
+        assert np.array_equal(got.view(np.uint32), want.view(np.uint32))
+
+
+@pytest.mark.parametrize("kind", ["f32", "bf16"])
+def test_quantize_q8_1_bytes(dev, kind):
+    rng = np.random.default_rng(5)
+    x = rng.standard_normal((5, 1024)).astype(np.float32)
+    x[1, 32:64] = 0.0                       # a zero block
+    x[2, :32] = np.arange(-16, 16) / 8.0    # exact binary fractions
+    x[2, 31] = 127.0 / 8.0                  # amax such that x/d hits .5 ties
+    x[3] *= 1e-6
+    x[4] *= 3e4
+    xin = x if kind == "f32" else O.f32_to_bf16_bits(x)
+    xf = x if kind == "f32" else O.bf16_bits_to_f32(xin)
+    want = O.quantize_q8_1(xf)
+    dx = dev.put(xin)
+    dq = dev.empty(want.size)
+    (Q.gguf_q4_k_quantize_f32_q8_1 if kind == "f32" else Q.gguf_q4_k_quantize_bf16_q8_1)(dx.ptr, dq.ptr, 5, 1024)
+    got = dev.get(dq, np.uint8, want.shape)
+    dev.free(dx, dq)
+    assert np.array_equal(got, want)
+    assert np.array_equal(got, C.quantize_q8_1(xin, bf16=(kind == "bf16")))
+
+
+@pytest.mark.parametrize("quant", ["gguf_q4_k", "gguf_q6_k", "gguf_q8_0"])
+def test_block_dots_bit_exact(dev, quant):
+    qt = QT[quant]
+    rng = np.random.default_rng(7)
+    rows, k, n = 3, 1024, 40
+    x = rng.standard_normal((rows, k)).astype(np.float32)
+    xq = O.quantize_q8_1(x)
+    w = O.random_weight(qt, n, k, seed=3)
+    per = 16 if qt == O.GGML_Q6_K else 32
+    dxq, dw = dev.put(xq), dev.put(w)
+    ddots = dev.empty(rows * n * (k // per) * 4)
+    dqs = dev.empty(rows * (k // 32) * 4)
+    V.gguf_q8_1_block_dots_i32(quant, dxq.ptr, dw.ptr, ddots.ptr, dqs.ptr, rows, k, n)
+    dots = dev.get(ddots, np.int32, (rows, n, k // per))
+    qs = dev.get(dqs, np.int32, (rows, k // 32))
+    dev.free(dxq, dw, ddots, dqs)
+    ref = C.block_dots(xq, w, qt)
+    if qt == O.GGML_Q4_K:
+        assert np.array_equal(dots, ref[0]) and np.array_equal(qs, ref[1])
+    else:
+        assert np.array_equal(dots, ref)
+    assert np.array_equal(qs, O.q8_1_fields(xq)[2].astype(np.int32).sum(axis=-1))
+
+
+@pytest.mark.parametrize("quant", ["gguf_q4_k", "gguf_q6_k", "gguf_q8_0"])
+@pytest.mark.parametrize("rows", [1, 2, 3, 4, 8])
+def test_fused_gemv_closed_form_weights(dev, quant, rows):
+    """The reference's closed-form weights and its `(arange % 13 - 6) / 8` activations
+    (tests/test_gpu_gguf_q4_k_gemv.py:102-112)."""
+    k, n = 512, 37
+    x = ((np.arange(rows * k, dtype=np.float32).reshape(rows, k) % 13) - 6) / 8.0
+    w = CLOSED[quant](n, k)
+    got = _run_fused(dev, quant, x, w)
+    _check_f32(got, O.quantize_q8_1(x), w, QT[quant])
+
+
+@pytest.mark.parametrize("quant,k,n", [
+    ("gguf_q4_k", 5120, 1024), ("gguf_q4_k", 2048, 512), ("gguf_q4_k", 512, 2048), ("gguf_q4_k", 256, 16),
+    ("gguf_q6_k", 5120, 1000), ("gguf_q6_k", 17408, 160), ("gguf_q8_0", 5120, 640), ("gguf_q8_0", 768, 33),
+])
+@pytest.mark.parametrize("rows", [1, 5, 8])
+def test_fused_gemv_random_weights(dev, quant, k, n, rows):
+    rng = np.random.default_rng(1000 + k + n + rows)
+    x = rng.standard_normal((rows, k)).astype(np.float32)
+    w = O.random_weight(QT[quant], n, k, seed=k + n)
+    got = _run_fused(dev, quant, x, w)
+    _check_f32(got, O.quantize_q8_1(x), w, QT[quant], x_unq=x)
+
+
+@pytest.mark.parametrize("quant", ["gguf_q4_k", "gguf_q6_k", "gguf_q8_0"])
+def test_fused_gemv_bf16_in_out(dev, quant):
+    rng = np.random.default_rng(21)
+    rows, k, n = 2, 1024, 96
+    x = rng.standard_normal((rows, k)).astype(np.float32)
+    xb = O.f32_to_bf16_bits(x)
+    w = O.random_weight(QT[quant], n, k, seed=9)
+    f32 = _run_fused(dev, quant, x, w, act="bf16", out="f32")
+    _check_f32(f32, O.quantize_q8_1(O.bf16_bits_to_f32(xb)), w, QT[quant])
+    b16 = _run_fused(dev, quant, x, w, act="bf16", out="bf16")
+    assert np.array_equal(b16, O.f32_to_bf16_bits(f32))
+
+
+@pytest.mark.parametrize("quant,fn", [
+    ("gguf_q4_k", "gguf_q4_k_q8_1_dp4a_vdr_bf16_f32_out"),
+    ("gguf_q6_k", "gguf_q6_k_q8_1_dp4a_gemv_bf16_f32_out"),
+    ("gguf_q8_0", "gguf_q8_0_dp4a_gemv_f32_f32_out"),
+])
+def test_prequantized_gemv_matches_fused_bit_for_bit(dev, quant, fn):
+    """Sibling variants must agree exactly: same integer dots, same float32 order."""
+    rng = np.random.default_rng(33)
+    rows, k, n = 4, 2048, 80
+    x = rng.standard_normal((rows, k)).astype(np.float32)
+    w = O.random_weight(QT[quant], n, k, seed=4)
+    fused = _run_fused(dev, quant, x, w)
+    xq = O.quantize_q8_1(x)
+    dxq, dw = dev.put(xq), dev.put(w)
+    dout = dev.empty(rows * n * 4)
+    getattr(G, fn)(dxq.ptr, dw.ptr, dout.ptr, rows, k, n)
+    pre = dev.get(dout, np.float32, (rows, n))
+    dev.free(dxq, dw, dout)
+    assert np.array_equal(pre.view(np.uint32), fused.view(np.uint32))
+    _check_f32(pre, xq, w, QT[quant])
+
+
+def test_more_than_eight_rows_and_determinism(dev):
+    rng = np.random.default_rng(44)
+    rows, k, n = 19, 1024, 48
+    x = rng.standard_normal((rows, k)).astype(np.float32)
+    w = O.random_weight(O.GGML_Q4_K, n, k, seed=2)
+    a = _run_fused(dev, "gguf_q4_k", x, w)
+    b = _run_fused(dev, "gguf_q4_k", x, w)
+    assert np.array_equal(a.view(np.uint32), b.view(np.uint32))
+    _check_f32(a, O.quantize_q8_1(x), w, O.GGML_Q4_K)
+    # row invariance: a row computed alone equals the same row inside the batch
+    one = _run_fused(dev, "gguf_q4_k", x[7:8], w)
+    assert np.array_equal(one.view(np.uint32), a[7:8].view(np.uint32))
+
+
+def test_output_canaries_untouched(dev):
+    rng = np.random.default_rng(55)
+    rows, k, n = 3, 512, 21
+    x = rng.standard_normal((rows, k)).astype(np.float32)
+    w = O.random_weight(O.GGML_Q4_K, n, k, seed=6)
+    dx, dw = dev.put(x), dev.put(w)
+    pad = 64
+    dout = dev.empty((rows * n + 2 * pad) * 4, fill=0x5A)
+    G.FUSED[("q4_k", "f32", "f32")](dx.ptr, dw.ptr, dout.ptr + pad * 4, rows, k, n)
+    raw = dev.get(dout, np.uint32, (rows * n + 2 * pad,))
+    dev.free(dx, dw, dout)
+    assert np.all(raw[:pad] == 0x5A5A5A5A) and np.all(raw[-pad:] == 0x5A5A5A5A)
+
+
+def test_c_abi_rejects_bad_arguments(dev):
+    import ctypes
+    lib = dev.library
+    f = lib.hipengine_gguf_q4_k_q8_1_fused_gemv_f32_f32_out
+    f.argtypes = [ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p] + [ctypes.c_int64] * 4 + [ctypes.c_void_p]
+    f.restype = ctypes.c_int
+    buf = dev.empty(4096)
+    assert f(None, buf.ptr, buf.ptr, 1, 256, 1, 128, None) == 1
+    assert f(buf.ptr, buf.ptr, buf.ptr, 1, 255, 1, 128, None) == 1
+    assert f(buf.ptr, buf.ptr, buf.ptr, 0, 256, 1, 128, None) == 1
+    dev.free(buf)
+    with pytest.raises(ValueError, match="divisible"):
+        G.FUSED[("q4_k", "f32", "f32")](1, 1, 1, 1, 100, 8)
+    with pytest.raises(ValueError, match="threads"):
+        G.FUSED[("q4_k", "f32", "f32")](1, 1, 1, 1, 256, 8, threads=96)
