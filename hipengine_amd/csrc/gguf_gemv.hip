@@ -3,6 +3,8 @@
 // The kernel body lives in gguf_gemv.hpp.
 
 #include "gguf_gemv.hpp"
+#include "gguf_gemv_run.hpp"
+#include "gguf_gemv_stream.hpp"
 
 #include "../../include/hipengine_gfx950.h"
 
@@ -58,6 +60,163 @@ const Variant* find_variant(int qt, int b, int r, int cb) {
   return nullptr;
 }
 
+
+// ---- run form (whole rows per wave, contiguous block runs) -------------------
+
+template <int QT, int B, int G, int CB>
+__global__ void __launch_bounds__(512) gemv_run_kernel(GemvRunArgs a) {
+  extern __shared__ __align__(16) uint8_t smem[];
+  gemv_run_workgroup<QT, B, G, CB>(a, smem);
+}
+
+using RunKernelFn = void (*)(GemvRunArgs);
+
+struct RunVariant {
+  int b, g, cb;
+  RunKernelFn fn;
+};
+
+#define RUN_VARIANT(QT, B, G, CB) \
+  RunVariant { B, G, CB, gemv_run_kernel<QT, B, G, CB> }
+#define RUN_VARIANTS_FOR(QT)                                                                        \
+  RUN_VARIANT(QT, 1, 1, 1), RUN_VARIANT(QT, 1, 2, 1), RUN_VARIANT(QT, 1, 4, 1), RUN_VARIANT(QT, 1, 8, 1), \
+  RUN_VARIANT(QT, 1, 1, 5), RUN_VARIANT(QT, 1, 2, 5), RUN_VARIANT(QT, 1, 4, 5), RUN_VARIANT(QT, 1, 8, 5), \
+  RUN_VARIANT(QT, 2, 1, 1), RUN_VARIANT(QT, 2, 2, 1), RUN_VARIANT(QT, 2, 4, 1), RUN_VARIANT(QT, 2, 8, 1), \
+  RUN_VARIANT(QT, 2, 1, 5), RUN_VARIANT(QT, 2, 2, 5), RUN_VARIANT(QT, 2, 4, 5), RUN_VARIANT(QT, 2, 8, 5)
+
+const RunVariant kRunQ4K[] = {RUN_VARIANTS_FOR(GGML_Q4_K)};
+const RunVariant kRunQ6K[] = {RUN_VARIANTS_FOR(GGML_Q6_K)};
+const RunVariant kRunQ80[] = {RUN_VARIANTS_FOR(GGML_Q8_0)};
+constexpr int kRunVariants = 16;
+
+const RunVariant* find_run_variant(int qt, int b, int g, int cb) {
+  const RunVariant* table = qt == GGML_Q4_K ? kRunQ4K : qt == GGML_Q6_K ? kRunQ6K : qt == GGML_Q8_0 ? kRunQ80 : nullptr;
+  if (!table) return nullptr;
+  for (int i = 0; i < kRunVariants; ++i)
+    if (table[i].b == b && table[i].g == g && table[i].cb == cb) return &table[i];
+  return nullptr;
+}
+
+int gcd_int(int a, int b) { return b == 0 ? a : gcd_int(b, a % b); }
+
+struct RunPlan {
+  int b, g, cb, waves;
+  bool ok;
+};
+
+// The run form applies when a whole number of rows fills a whole number of
+// 16-block wave loads with at most 8 rows, the batch is 1 or 2 and the
+// quantized activations of the whole K fit in LDS.
+RunPlan default_run_plan(int qt, int rows, int64_t K, int64_t N) {
+  RunPlan p{};
+  const int nb = static_cast<int>(K / QK_K);
+  p.b = rows <= 1 ? 1 : 2;
+  p.g = 16 / gcd_int(nb, 16);
+  const int m = p.g * nb / 16;
+  p.cb = m >= 2 ? 5 : 1;
+  const int64_t runs = (N + p.g - 1) / p.g;
+  p.waves = 8;
+  while (p.waves > 1 && (runs + p.waves - 1) / p.waves < 512) p.waves >>= 1;
+  p.ok = rows <= 2 && p.g <= 8 && gemv_run_lds_bytes(qt, p.b, static_cast<int>(K)) <= 64 * 1024 &&
+         find_run_variant(qt, p.b, p.g, p.cb) != nullptr;
+  return p;
+}
+
+int launch_gemv_run(int qt, const void* x, int x_kind, const uint8_t* w, void* out, int out_kind, int rows, int64_t K,
+                    int64_t N, const RunPlan& p, hipStream_t stream) {
+  const RunVariant* v = find_run_variant(qt, p.b, p.g, p.cb);
+  const int nb = static_cast<int>(K / QK_K);
+  if (!v || p.waves < 1 || p.waves > 8 || (p.g * nb) % 16 != 0 || rows > p.b) {
+    return static_cast<int>(hipErrorInvalidValue);
+  }
+  const size_t lds = gemv_run_lds_bytes(qt, p.b, static_cast<int>(K));
+  if (lds > 64 * 1024) return static_cast<int>(hipErrorInvalidValue);
+  GemvRunArgs a;
+  a.x = x; a.w = w; a.out = out;
+  a.x_kind = x_kind; a.out_kind = out_kind;
+  a.rows = rows; a.K = static_cast<int>(K); a.N = static_cast<int>(N);
+  a.waves = p.waves;
+  const int64_t runs = (N + p.g - 1) / p.g;
+  const unsigned grid = static_cast<unsigned>((runs + p.waves - 1) / p.waves);
+  hipLaunchKernelGGL(v->fn, dim3(grid), dim3(p.waves * 64), lds, stream, a);
+  return static_cast<int>(hipGetLastError());
+}
+
+
+// ---- stream form (resident waves, ring of loads in flight) --------------------
+
+template <int QT, int B, int D>
+__global__ void __launch_bounds__(512) gemv_stream_kernel(GemvStreamArgs a) {
+  extern __shared__ __align__(16) uint8_t smem[];
+  gemv_stream_workgroup<QT, B, D>(a, smem);
+}
+
+using StreamKernelFn = void (*)(GemvStreamArgs);
+
+struct StreamVariant {
+  int qt, b, d;
+  StreamKernelFn fn;
+};
+
+#define STREAM_VARIANT(QT, B, D) \
+  StreamVariant { QT, B, D, gemv_stream_kernel<QT, B, D> }
+
+const StreamVariant kStream[] = {
+    STREAM_VARIANT(GGML_Q4_K, 1, 3), STREAM_VARIANT(GGML_Q4_K, 1, 5), STREAM_VARIANT(GGML_Q4_K, 2, 3),
+    STREAM_VARIANT(GGML_Q4_K, 2, 5), STREAM_VARIANT(GGML_Q6_K, 1, 3), STREAM_VARIANT(GGML_Q6_K, 1, 5),
+    STREAM_VARIANT(GGML_Q6_K, 2, 3), STREAM_VARIANT(GGML_Q6_K, 2, 5), STREAM_VARIANT(GGML_Q8_0, 1, 3),
+    STREAM_VARIANT(GGML_Q8_0, 1, 5), STREAM_VARIANT(GGML_Q8_0, 2, 3), STREAM_VARIANT(GGML_Q8_0, 2, 5),
+};
+
+const StreamVariant* find_stream_variant(int qt, int b, int d) {
+  for (const StreamVariant& v : kStream)
+    if (v.qt == qt && v.b == b && v.d == d) return &v;
+  return nullptr;
+}
+
+struct StreamPlan {
+  int b, d, waves, waves_total;
+  bool ok;
+};
+
+constexpr int kComputeUnits = 256;   // MI355X
+
+// The stream form applies to K >= 4096 (a 16-block load then spans at most two
+// rows), batch <= 2, when every resident wave gets at least a few loads.
+StreamPlan default_stream_plan(int qt, int rows, int64_t K, int64_t N) {
+  StreamPlan p{};
+  const int nb = static_cast<int>(K / QK_K);
+  p.b = rows <= 1 ? 1 : 2;
+  p.d = 3;
+  p.waves = 8;
+  const int64_t total_loads = N * nb / 16;
+  // 8 resident waves per CU once every wave gets ~8 loads or more, else 4 per CU
+  p.waves_total = total_loads >= 16384 ? kComputeUnits * 8 : kComputeUnits * 4;
+  p.ok = rows <= 2 && nb >= 16 && total_loads >= 4 * static_cast<int64_t>(p.waves_total) &&
+         N >= p.waves_total && gemv_run_lds_bytes(qt, p.b, static_cast<int>(K)) <= 64 * 1024 &&
+         find_stream_variant(qt, p.b, p.d) != nullptr;
+  return p;
+}
+
+int launch_gemv_stream(int qt, const void* x, int x_kind, const uint8_t* w, void* out, int out_kind, int rows,
+                       int64_t K, int64_t N, const StreamPlan& p, hipStream_t stream) {
+  const StreamVariant* v = find_stream_variant(qt, p.b, p.d);
+  const int nb = static_cast<int>(K / QK_K);
+  if (!v || nb < 16 || rows > p.b || p.waves < 1 || p.waves > 8 || p.waves_total < p.waves ||
+      (p.waves_total % p.waves) != 0 || p.waves_total > N) {
+    return static_cast<int>(hipErrorInvalidValue);
+  }
+  const size_t lds = gemv_run_lds_bytes(qt, p.b, static_cast<int>(K));
+  if (lds > 64 * 1024) return static_cast<int>(hipErrorInvalidValue);
+  GemvStreamArgs a;
+  a.x = x; a.w = w; a.out = out;
+  a.x_kind = x_kind; a.out_kind = out_kind;
+  a.rows = rows; a.K = static_cast<int>(K); a.N = static_cast<int>(N);
+  a.waves = p.waves; a.waves_total = p.waves_total;
+  hipLaunchKernelGGL(v->fn, dim3(p.waves_total / p.waves), dim3(p.waves * 64), lds, stream, a);
+  return static_cast<int>(hipGetLastError());
+}
+
 int batch_bucket(int rows) { return rows <= 1 ? 1 : rows <= 2 ? 2 : rows <= 4 ? 4 : 8; }
 
 struct Plan {
@@ -94,6 +253,24 @@ int launch_gemv(int qt, const void* x, int x_kind, const uint8_t* w, void* out, 
   const int64_t out_elem = out_kind == KIND_F32 ? 4 : 2;
   for (int64_t r0 = 0; r0 < rows; r0 += 8) {
     const int chunk = static_cast<int>(rows - r0 < 8 ? rows - r0 : 8);
+    if (!forced) {
+      const StreamPlan sp = default_stream_plan(qt, chunk, K, N);
+      if (sp.ok) {
+        const int rc = launch_gemv_stream(qt, static_cast<const uint8_t*>(x) + r0 * x_row_bytes, x_kind, w,
+                                          static_cast<uint8_t*>(out) + r0 * N * out_elem, out_kind, chunk, K, N,
+                                          sp, stream);
+        if (rc != static_cast<int>(hipSuccess)) return rc;
+        continue;
+      }
+      const RunPlan rp = default_run_plan(qt, chunk, K, N);
+      if (rp.ok) {
+        const int rc = launch_gemv_run(qt, static_cast<const uint8_t*>(x) + r0 * x_row_bytes, x_kind, w,
+                                       static_cast<uint8_t*>(out) + r0 * N * out_elem, out_kind, chunk, K, N, rp,
+                                       stream);
+        if (rc != static_cast<int>(hipSuccess)) return rc;
+        continue;
+      }
+    }
     Plan p = forced ? *forced : default_plan(qt, chunk, K, N);
     if (forced) p.b = batch_bucket(chunk);
     const Variant* v = find_variant(qt, p.b, p.r, p.cb);
@@ -190,4 +367,40 @@ extern "C" int hipengine_gfx950_gguf_gemv_default_plan(int32_t ggml_type, int64_
   const Plan p = default_plan(ggml_type, static_cast<int>(rows < 8 ? rows : 8), in_features, out_features);
   plan5[0] = p.b; plan5[1] = p.r; plan5[2] = p.cb; plan5[3] = p.ks; plan5[4] = p.nrg;
   return static_cast<int>(hipSuccess);
+}
+
+extern "C" int hipengine_gfx950_gguf_q8_1_fused_gemv_run_tuned(
+    int32_t ggml_type, const void* x, int32_t x_kind, const uint8_t* qweight, void* out, int32_t out_kind,
+    int64_t rows, int64_t in_features, int64_t out_features, int32_t rows_per_wave, int32_t loads_per_chunk,
+    int32_t waves, hipStream_t stream) {
+  if (!x || !qweight || !out || x_kind < KIND_F32 || x_kind > KIND_Q8_1 || out_kind < KIND_F32 ||
+      out_kind > KIND_F16 || rows <= 0 || rows > 2 || in_features <= 0 || (in_features % QK_K) != 0 ||
+      out_features <= 0) {
+    return static_cast<int>(hipErrorInvalidValue);
+  }
+  RunPlan p{};
+  p.b = rows <= 1 ? 1 : 2;
+  p.g = rows_per_wave;
+  p.cb = loads_per_chunk;
+  p.waves = waves;
+  return launch_gemv_run(ggml_type, x, x_kind, qweight, out, out_kind, static_cast<int>(rows), in_features,
+                         out_features, p, stream);
+}
+
+extern "C" int hipengine_gfx950_gguf_q8_1_fused_gemv_stream_tuned(
+    int32_t ggml_type, const void* x, int32_t x_kind, const uint8_t* qweight, void* out, int32_t out_kind,
+    int64_t rows, int64_t in_features, int64_t out_features, int32_t loads_in_flight, int32_t waves,
+    int32_t waves_total, hipStream_t stream) {
+  if (!x || !qweight || !out || x_kind < KIND_F32 || x_kind > KIND_Q8_1 || out_kind < KIND_F32 ||
+      out_kind > KIND_F16 || rows <= 0 || rows > 2 || in_features <= 0 || (in_features % QK_K) != 0 ||
+      out_features <= 0) {
+    return static_cast<int>(hipErrorInvalidValue);
+  }
+  StreamPlan p{};
+  p.b = rows <= 1 ? 1 : 2;
+  p.d = loads_in_flight;
+  p.waves = waves;
+  p.waves_total = waves_total;
+  return launch_gemv_stream(ggml_type, x, x_kind, qweight, out, out_kind, static_cast<int>(rows), in_features,
+                            out_features, p, stream);
 }

@@ -1,0 +1,417 @@
+// "Run" form of the q8_1 decode GEMV: every wave owns G whole consecutive rows
+// and streams them as ONE contiguous run of G*nb 256-value blocks.
+//
+// A wave-wide load covers 16 consecutive blocks (4 lanes per block), i.e. 2304
+// contiguous bytes of Q4_K: measured on MI355X this reads a 50 MB weight within
+// ~10% of a plain coalesced copy, where the row-strided layout of
+// gguf_gemv.hpp (16 different rows per load) is ~30% slower.  G is chosen so
+// that G*nb is a multiple of 16, which makes the run a whole number m of wave
+// loads; lane quad j of load i holds block 16*i + j of the run, which belongs
+// to row (16*i + j) / nb and K block (16*i + j) % nb.
+//
+// Consequences:
+//   * no K split and no cross-wave reduction: a row's m*16/G blocks all live in
+//     one wave; the only workgroup barrier is the one after activation staging;
+//   * activations for the whole K are quantized to q8_1 once per workgroup into
+//     LDS (a workgroup is several waves = several runs sharing them);
+//   * different lanes of a load need different K blocks, so the LDS image pads
+//     every block (272 or 288 bytes apart) to keep the 16-byte reads of a
+//     quarter wave on distinct banks;
+//   * each lane keeps G accumulators and adds its term to the one its block
+//     belongs to; rows are reduced across the wave with DPP at the end.
+//
+// The integer dots, the scale decode and the float32 combine are the functions
+// of gguf_gemv.hpp, so both kernels produce bit-identical sub-block dots.
+#pragma once
+
+#include "gguf_gemv.hpp"
+
+namespace hipengine_gfx950 {
+
+struct GemvRunArgs {
+  const void* x;
+  const uint8_t* w;
+  void* out;
+  int x_kind;
+  int out_kind;
+  int rows;     // batch rows, 1..B
+  int K;
+  int N;
+  int waves;    // waves (= runs) per workgroup
+};
+
+template <int QT>
+constexpr int run_q8_stride() {
+  return QT == GGML_Q6_K ? 288 : 272;
+}
+
+// Bytes of dynamic LDS: per batch row nb padded q8 blocks, nb*64 bytes of
+// scale records and, for Q6_K, nb*64 bytes of 16-wide q8 sums.
+inline size_t gemv_run_lds_bytes(int qt, int B, int K) {
+  const size_t nb = K / QK_K;
+  const size_t stride = qt == GGML_Q6_K ? 288 : 272;
+  return B * nb * (stride + 64 + (qt == GGML_Q6_K ? 64 : 0));
+}
+
+// q = clamp(roundf(v / d), -128, 127) evaluated through the reciprocal.  The
+// product v*inv is within 3e-5 of the exactly rounded quotient (|v/d| <= 127),
+// so truncating v*inv +- 0.5 gives roundf of the quotient unless the
+// fractional part is that close to one half; those lanes redo the IEEE
+// division.  Bit-exact with the direct evaluation.
+__device__ __forceinline__ int q8_round_div(float v, float d, float inv) {
+  const float t = v * inv;
+  const float f = fabsf(t) - floorf(fabsf(t));
+  int q = static_cast<int>(t + copysignf(0.5f, t));
+  if (__builtin_expect(fabsf(f - 0.5f) < 1.0e-4f, 0)) q = static_cast<int>(roundf(v / d));
+  return max(-128, min(127, q));
+}
+
+// Whole-K activation staging for the run kernel.
+//   q8   : [B][nb] blocks, Q8S bytes apart
+//   rec  : [B][nb][4] 16-byte records, one per lane q of a block:
+//            Q4_K {xd(2q), xd(2q+1), xd*qsum(2q), xd*qsum(2q+1)}
+//            Q8_0 {xd(2q), xd(2q+1), -, -}
+//            Q6_K {xd(4h), xd(4h+1), xd(4h+2), xd(4h+3)}, q = 2h+t
+//   s16  : Q6_K only, [B][nb][4] x {qsum16(4h+j, half t)} j = 0..3
+template <int QT, int B>
+__device__ __forceinline__ void gemv_run_stage(const GemvRunArgs& a, uint8_t* q8, float* rec, int* s16) {
+  constexpr int Q8S = run_q8_stride<QT>();
+  const int tid = threadIdx.x;
+  const int team = tid >> 3, e = tid & 7, nteams = blockDim.x >> 3;
+  const int nb = a.K / QK_K;
+  const int groups = nb * 8;
+#pragma unroll
+  for (int b = 0; b < B; ++b) {
+    for (int j = team; j < groups; j += nteams) {
+      uint32_t packed = 0;
+      float xd = 0.0f;
+      if (b < a.rows) {
+        if (a.x_kind == KIND_Q8_1) {
+          const uint8_t* blk = static_cast<const uint8_t*>(a.x) +
+                               (static_cast<int64_t>(b) * (a.K / 32) + j) * Q8_1_BYTES;
+          packed = *reinterpret_cast<const uint32_t*>(blk + 4 + 4 * e);
+          xd = f16_bits_to_float(*reinterpret_cast<const uint32_t*>(blk) & 0xFFFFu);
+        } else {
+          const int64_t k0 = static_cast<int64_t>(b) * a.K + j * 32 + e * 4;
+          float v0, v1, v2, v3;
+          if (a.x_kind == KIND_F32) {
+            const float4 v = *reinterpret_cast<const float4*>(static_cast<const float*>(a.x) + k0);
+            v0 = v.x; v1 = v.y; v2 = v.z; v3 = v.w;
+          } else {
+            const uint2 v = *reinterpret_cast<const uint2*>(static_cast<const uint16_t*>(a.x) + k0);
+            if (a.x_kind == KIND_BF16) {
+              v0 = bf16_bits_to_float(v.x & 0xFFFFu); v1 = bf16_bits_to_float(v.x >> 16);
+              v2 = bf16_bits_to_float(v.y & 0xFFFFu); v3 = bf16_bits_to_float(v.y >> 16);
+            } else {
+              v0 = f16_bits_to_float(v.x & 0xFFFFu); v1 = f16_bits_to_float(v.x >> 16);
+              v2 = f16_bits_to_float(v.y & 0xFFFFu); v3 = f16_bits_to_float(v.y >> 16);
+            }
+          }
+          const float amax = oct_max(fmaxf(fmaxf(fabsf(v0), fabsf(v1)), fmaxf(fabsf(v2), fabsf(v3))));
+          const float d = amax / 127.0f;
+          if (amax != 0.0f) {
+            const float inv = 1.0f / d;
+            const int q0 = q8_round_div(v0, d, inv), q1 = q8_round_div(v1, d, inv);
+            const int q2 = q8_round_div(v2, d, inv), q3 = q8_round_div(v3, d, inv);
+            packed = (q0 & 0xFF) | ((q1 & 0xFF) << 8) | ((q2 & 0xFF) << 16) | (static_cast<uint32_t>(q3 & 0xFF) << 24);
+          }
+          xd = static_cast<float>(static_cast<half_t>(d));
+        }
+      }
+      const int kb = j >> 3, sb = j & 7;
+      *reinterpret_cast<uint32_t*>(q8 + (b * nb + kb) * Q8S + sb * 32 + e * 4) = packed;
+      const int part = dot4(0x01010101u, packed, 0);
+      float* r = rec + (b * nb + kb) * 16;
+      if constexpr (QT == GGML_Q6_K) {
+        int h16 = part;
+        h16 += dpp_i<DPP_QUAD_XOR1>(h16);
+        h16 += dpp_i<DPP_QUAD_XOR2>(h16);
+        // group sb = 4h + jj, half t = e>>2 -> record of lane q = 2h+t, slot jj
+        const int h = sb >> 2, jj = sb & 3;
+        if ((e & 3) == 0) s16[(b * nb + kb) * 16 + (2 * h + (e >> 2)) * 4 + jj] = h16;
+        if (e == 0) {   // xd of group sb goes to both records (t = 0, 1) of half h
+          r[(2 * h) * 4 + jj] = xd;
+          r[(2 * h + 1) * 4 + jj] = xd;
+        }
+      } else {
+        const int total = oct_sum_i(part);
+        if (e == 0) {   // sub-block sb -> record of lane q = sb>>1, slot sb&1 (+2 for the xd*qsum term)
+          r[(sb >> 1) * 4 + (sb & 1)] = xd;
+          if constexpr (QT == GGML_Q4_K) r[(sb >> 1) * 4 + 2 + (sb & 1)] = xd * static_cast<float>(total);
+        }
+      }
+    }
+  }
+}
+
+
+// The same staging split in two so that a kernel can put the activation loads
+// in front of its weight loads: vmcnt counts loads in issue order, so waiting
+// for activations issued AFTER the weight ring would also wait for the ring.
+//   stage_fetch  : issue the loads of this thread's first S groups per batch row
+//   stage_commit : quantize them into LDS; groups beyond the first S per thread
+//                  are loaded and quantized here (large K only)
+template <int B, int S>
+struct StageRegs {
+  uint32_t raw[B][S][4];
+};
+
+template <int QT, int B, int S>
+__device__ __forceinline__ void gemv_run_stage_fetch(const GemvRunArgs& a, StageRegs<B, S>& sr) {
+  const int tid = threadIdx.x;
+  const int team = tid >> 3, e = tid & 7, nteams = blockDim.x >> 3;
+  const int groups = (a.K / QK_K) * 8;
+#pragma unroll
+  for (int b = 0; b < B; ++b) {
+#pragma unroll
+    for (int s = 0; s < S; ++s) {
+      const int j = team + s * nteams;
+      uint4 v = make_uint4(0u, 0u, 0u, 0u);
+      if (b < a.rows && j < groups) {
+        if (a.x_kind == KIND_F32) {
+          v = *reinterpret_cast<const uint4*>(static_cast<const float*>(a.x) + static_cast<int64_t>(b) * a.K + j * 32 + e * 4);
+        } else if (a.x_kind == KIND_Q8_1) {
+          const uint8_t* blk = static_cast<const uint8_t*>(a.x) + (static_cast<int64_t>(b) * (a.K / 32) + j) * Q8_1_BYTES;
+          v.x = *reinterpret_cast<const uint32_t*>(blk + 4 + 4 * e);
+          v.y = *reinterpret_cast<const uint32_t*>(blk);
+        } else {
+          const uint2 h = *reinterpret_cast<const uint2*>(static_cast<const uint16_t*>(a.x) + static_cast<int64_t>(b) * a.K + j * 32 + e * 4);
+          v.x = h.x; v.y = h.y;
+        }
+      }
+      sr.raw[b][s][0] = v.x; sr.raw[b][s][1] = v.y; sr.raw[b][s][2] = v.z; sr.raw[b][s][3] = v.w;
+    }
+  }
+}
+
+// Quantize one fetched group (4 values of one lane) and write it to the LDS image.
+template <int QT>
+__device__ __forceinline__ void gemv_run_stage_one(int x_kind, const uint32_t (&raw)[4], bool present, int j, int e,
+                                                   uint8_t* q8_row, float* rec_row, int* s16_row) {
+  constexpr int Q8S = run_q8_stride<QT>();
+  uint32_t packed = 0;
+  float xd = 0.0f;
+  if (present) {
+    if (x_kind == KIND_Q8_1) {
+      packed = raw[0];
+      xd = f16_bits_to_float(raw[1] & 0xFFFFu);
+    } else {
+      float v0, v1, v2, v3;
+      if (x_kind == KIND_F32) {
+        v0 = bits_to_float(raw[0]); v1 = bits_to_float(raw[1]); v2 = bits_to_float(raw[2]); v3 = bits_to_float(raw[3]);
+      } else if (x_kind == KIND_BF16) {
+        v0 = bf16_bits_to_float(raw[0] & 0xFFFFu); v1 = bf16_bits_to_float(raw[0] >> 16);
+        v2 = bf16_bits_to_float(raw[1] & 0xFFFFu); v3 = bf16_bits_to_float(raw[1] >> 16);
+      } else {
+        v0 = f16_bits_to_float(raw[0] & 0xFFFFu); v1 = f16_bits_to_float(raw[0] >> 16);
+        v2 = f16_bits_to_float(raw[1] & 0xFFFFu); v3 = f16_bits_to_float(raw[1] >> 16);
+      }
+      const float amax = oct_max(fmaxf(fmaxf(fabsf(v0), fabsf(v1)), fmaxf(fabsf(v2), fabsf(v3))));
+      const float d = amax / 127.0f;
+      if (amax != 0.0f) {
+        const float inv = 1.0f / d;
+        const int q0 = q8_round_div(v0, d, inv), q1 = q8_round_div(v1, d, inv);
+        const int q2 = q8_round_div(v2, d, inv), q3 = q8_round_div(v3, d, inv);
+        packed = (q0 & 0xFF) | ((q1 & 0xFF) << 8) | ((q2 & 0xFF) << 16) | (static_cast<uint32_t>(q3 & 0xFF) << 24);
+      }
+      xd = static_cast<float>(static_cast<half_t>(d));
+    }
+  }
+  const int kb = j >> 3, sb = j & 7;
+  *reinterpret_cast<uint32_t*>(q8_row + kb * Q8S + sb * 32 + e * 4) = packed;
+  const int part = dot4(0x01010101u, packed, 0);
+  float* r = rec_row + kb * 16;
+  if constexpr (QT == GGML_Q6_K) {
+    int h16 = part;
+    h16 += dpp_i<DPP_QUAD_XOR1>(h16);
+    h16 += dpp_i<DPP_QUAD_XOR2>(h16);
+    const int h = sb >> 2, jj = sb & 3;
+    if ((e & 3) == 0) s16_row[kb * 16 + (2 * h + (e >> 2)) * 4 + jj] = h16;
+    if (e == 0) {
+      r[(2 * h) * 4 + jj] = xd;
+      r[(2 * h + 1) * 4 + jj] = xd;
+    }
+  } else {
+    const int total = oct_sum_i(part);
+    if (e == 0) {
+      r[(sb >> 1) * 4 + (sb & 1)] = xd;
+      if constexpr (QT == GGML_Q4_K) r[(sb >> 1) * 4 + 2 + (sb & 1)] = xd * static_cast<float>(total);
+    }
+  }
+}
+
+template <int QT, int B, int S>
+__device__ __forceinline__ void gemv_run_stage_commit(const GemvRunArgs& a, const StageRegs<B, S>& sr, uint8_t* q8,
+                                                      float* rec, int* s16) {
+  constexpr int Q8S = run_q8_stride<QT>();
+  const int tid = threadIdx.x;
+  const int team = tid >> 3, e = tid & 7, nteams = blockDim.x >> 3;
+  const int nb = a.K / QK_K;
+  const int groups = nb * 8;
+#pragma unroll
+  for (int b = 0; b < B; ++b) {
+    uint8_t* q8_row = q8 + b * nb * Q8S;
+    float* rec_row = rec + b * nb * 16;
+    int* s16_row = s16 + b * nb * 16;
+#pragma unroll
+    for (int s = 0; s < S; ++s) {
+      const int j = team + s * nteams;
+      if (j < groups) gemv_run_stage_one<QT>(a.x_kind, sr.raw[b][s], b < a.rows, j, e, q8_row, rec_row, s16_row);
+    }
+    for (int j = team + S * nteams; j < groups; j += nteams) {   // large K: the rest, loaded here
+      uint32_t raw[4] = {0u, 0u, 0u, 0u};
+      if (b < a.rows) {
+        if (a.x_kind == KIND_F32) {
+          const uint4 v = *reinterpret_cast<const uint4*>(static_cast<const float*>(a.x) + static_cast<int64_t>(b) * a.K + j * 32 + e * 4);
+          raw[0] = v.x; raw[1] = v.y; raw[2] = v.z; raw[3] = v.w;
+        } else if (a.x_kind == KIND_Q8_1) {
+          const uint8_t* blk = static_cast<const uint8_t*>(a.x) + (static_cast<int64_t>(b) * (a.K / 32) + j) * Q8_1_BYTES;
+          raw[0] = *reinterpret_cast<const uint32_t*>(blk + 4 + 4 * e);
+          raw[1] = *reinterpret_cast<const uint32_t*>(blk);
+        } else {
+          const uint2 h = *reinterpret_cast<const uint2*>(static_cast<const uint16_t*>(a.x) + static_cast<int64_t>(b) * a.K + j * 32 + e * 4);
+          raw[0] = h.x; raw[1] = h.y;
+        }
+      }
+      gemv_run_stage_one<QT>(a.x_kind, raw, b < a.rows, j, e, q8_row, rec_row, s16_row);
+    }
+  }
+}
+
+// One lane's float32 contribution of one block to one batch row, run layout.
+template <int QT>
+__device__ __forceinline__ float gemv_run_block_term(const WeightRegs<GemvTraits<QT>::REGS>& r, const BlockScales<QT>& s,
+                                                     int q, const uint8_t* q8_blk, const float* rec_blk,
+                                                     const int* s16_blk) {
+  int dots[4];
+  if constexpr (QT == GGML_Q6_K) {
+    // gemv_block_dots expects the qsum16 of group g, half t at s16[g*2 + t]; the run
+    // records keep the four a lane needs together, so subtract them here instead.
+    const int h = q >> 1, t = q & 1;
+    const uint8_t* base = q8_blk + h * 128 + t * 16;
+    const uint4 x0 = *reinterpret_cast<const uint4*>(base);
+    const uint4 x1 = *reinterpret_cast<const uint4*>(base + 32);
+    const uint4 x2 = *reinterpret_cast<const uint4*>(base + 64);
+    const uint4 x3 = *reinterpret_cast<const uint4*>(base + 96);
+    const Q6KQuad u0 = q6k_unpack(r.v[0], r.v[4], r.v[8]);
+    const Q6KQuad u1 = q6k_unpack(r.v[1], r.v[5], r.v[9]);
+    const Q6KQuad u2 = q6k_unpack(r.v[2], r.v[6], r.v[10]);
+    const Q6KQuad u3 = q6k_unpack(r.v[3], r.v[7], r.v[11]);
+    int d0 = 0, d1 = 0, d2 = 0, d3 = 0;
+    d0 = dot4(u0.g0, x0.x, d0); d1 = dot4(u0.g1, x1.x, d1); d2 = dot4(u0.g2, x2.x, d2); d3 = dot4(u0.g3, x3.x, d3);
+    d0 = dot4(u1.g0, x0.y, d0); d1 = dot4(u1.g1, x1.y, d1); d2 = dot4(u1.g2, x2.y, d2); d3 = dot4(u1.g3, x3.y, d3);
+    d0 = dot4(u2.g0, x0.z, d0); d1 = dot4(u2.g1, x1.z, d1); d2 = dot4(u2.g2, x2.z, d2); d3 = dot4(u2.g3, x3.z, d3);
+    d0 = dot4(u3.g0, x0.w, d0); d1 = dot4(u3.g1, x1.w, d1); d2 = dot4(u3.g2, x2.w, d2); d3 = dot4(u3.g3, x3.w, d3);
+    const int4 sq = *reinterpret_cast<const int4*>(s16_blk + q * 4);
+    dots[0] = d0 - 32 * sq.x; dots[1] = d1 - 32 * sq.y; dots[2] = d2 - 32 * sq.z; dots[3] = d3 - 32 * sq.w;
+    const float4 xd = *reinterpret_cast<const float4*>(rec_blk + q * 4);
+    float v = s.f[0] * (xd.x * static_cast<float>(dots[0]));
+    v += s.f[1] * (xd.y * static_cast<float>(dots[1]));
+    v += s.f[2] * (xd.z * static_cast<float>(dots[2]));
+    v += s.f[3] * (xd.w * static_cast<float>(dots[3]));
+    return v;
+  } else {
+    gemv_block_dots<QT>(r, q, q8_blk, nullptr, dots);
+    const float4 rc = *reinterpret_cast<const float4*>(rec_blk + q * 4);
+    float v = s.f[0] * (rc.x * static_cast<float>(dots[0]));
+    v += s.f[1] * (rc.y * static_cast<float>(dots[1]));
+    if constexpr (QT == GGML_Q4_K) {
+      v -= s.m[0] * rc.z;
+      v -= s.m[1] * rc.w;
+    }
+    return v;
+  }
+}
+
+constexpr int DPP_ROW_MIRROR = 0x140;
+constexpr int DPP_ROW_BCAST15 = 0x142;
+constexpr int DPP_ROW_BCAST31 = 0x143;
+
+// Sum over the 64 lanes of a wave; the total is valid in lane 63.
+__device__ __forceinline__ float wave_sum_to_lane63(float v) {
+  v += dpp_f<DPP_QUAD_XOR1>(v);
+  v += dpp_f<DPP_QUAD_XOR2>(v);
+  v += dpp_f<DPP_ROW_HALF_MIRROR>(v);
+  v += dpp_f<DPP_ROW_MIRROR>(v);     // every lane of a row of 16 now holds the row total
+  v += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), DPP_ROW_BCAST15, 0xA, 0xF, false));
+  v += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), DPP_ROW_BCAST31, 0xC, 0xF, false));
+  return v;
+}
+
+template <int QT, int B, int G, int CB>
+__device__ __forceinline__ void gemv_run_workgroup(const GemvRunArgs& a, uint8_t* smem) {
+  using Regs = WeightRegs<GemvTraits<QT>::REGS>;
+  constexpr int Q8S = run_q8_stride<QT>();
+  constexpr int SUPER = GemvTraits<QT>::SUPER_BYTES;
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int q = lane & 3, j = lane >> 2;
+  const int nb = a.K / QK_K;
+  const int m = G * nb / 16;                                  // wave loads per run
+  const int64_t run = static_cast<int64_t>(blockIdx.x) * a.waves + wave;
+  const int64_t first_row = run * G;
+  const int64_t total_blocks = static_cast<int64_t>(a.N) * nb;
+  const int64_t run_block0 = first_row * nb;
+
+  uint8_t* q8 = smem;
+  float* rec = reinterpret_cast<float*>(q8 + B * nb * Q8S);
+  int* s16 = reinterpret_cast<int*>(rec + B * nb * 16);
+
+  float acc[G][B];
+#pragma unroll
+  for (int g = 0; g < G; ++g)
+#pragma unroll
+    for (int b = 0; b < B; ++b) acc[g][b] = 0.0f;
+
+  // position of this lane's block inside the run: K block kb and row r of load i
+  int kb = j % nb, r = j / nb;
+  const int step_r = 16 / nb, step_kb = 16 % nb;   // advance of (r, kb) per load
+
+  // activation loads first, then the weight loads, then the quantization: the wait
+  // for the activations must not include the (later issued) weight loads
+  constexpr int S = 3;
+  StageRegs<B, S> sr;
+  gemv_run_stage_fetch<QT, B, S>(a, sr);
+
+  for (int i0 = 0; i0 < m; i0 += CB) {
+    Regs wr[CB];
+#pragma unroll
+    for (int c = 0; c < CB; ++c) {
+      if (i0 + c < m) {
+        int64_t blk = run_block0 + static_cast<int64_t>(i0 + c) * 16 + j;
+        blk = blk < total_blocks ? blk : total_blocks - 1;   // runs past the last row re-read its last block
+        gemv_load_block<QT>(a.w + blk * SUPER, q, wr[c]);
+      }
+    }
+    if (i0 == 0) {
+      gemv_run_stage_commit<QT, B, S>(a, sr, q8, rec, s16);
+      __syncthreads();
+    }
+#pragma unroll
+    for (int c = 0; c < CB; ++c) {
+      if (i0 + c < m) {
+        const BlockScales<QT> s = gemv_block_scales<QT>(wr[c], q);
+#pragma unroll
+        for (int b = 0; b < B; ++b) {
+          const float term = gemv_run_block_term<QT>(wr[c], s, q, q8 + (b * nb + kb) * Q8S, rec + (b * nb + kb) * 16,
+                                                     s16 + (b * nb + kb) * 16);
+#pragma unroll
+          for (int g = 0; g < G; ++g) acc[g][b] += (r == g) ? term : 0.0f;
+        }
+        kb += step_kb;
+        r += step_r;
+        if (kb >= nb) { kb -= nb; r += 1; }
+      }
+    }
+  }
+
+#pragma unroll
+  for (int g = 0; g < G; ++g)
+#pragma unroll
+    for (int b = 0; b < B; ++b) {
+      const float v = wave_sum_to_lane63(acc[g][b]);
+      const int64_t row = first_row + g;
+      if (lane == 63 && row < a.N && b < a.rows) store_scalar(a.out, static_cast<int64_t>(b) * a.N + row, v, a.out_kind);
+    }
+}
+
+}  // namespace hipengine_gfx950

@@ -106,6 +106,31 @@ def gguf_q8_1_fused_gemv_tuned(quant_key: str, x_ptr: int, x_kind: str, qweight_
                     in_features, out_features, k_slices, row_groups, blocks_per_wave, rows_per_lane, stream), runtime)
 
 
+_RUN_TUNED_ARGS = [I32, VOID, I32, VOID, VOID, I32, I64, I64, I64, I32, I32, I32, VOID]
+
+
+def gguf_q8_1_fused_gemv_run_tuned(quant_key: str, x_ptr: int, x_kind: str, qweight_ptr: int, out_ptr: int,
+                                   out_kind: str, rows: int, in_features: int, out_features: int, *,
+                                   rows_per_wave: int, loads_per_chunk: int, waves: int, stream: int = 0,
+                                   library: ctypes.CDLL | None = None, runtime: HipRuntime | None = None) -> None:
+    """The run form of the fused GEMV with an explicit layout (tuning sweeps only)."""
+    validate_linear(rows, in_features, out_features)
+    fn = entry("hipengine_gfx950_gguf_q8_1_fused_gemv_run_tuned", _RUN_TUNED_ARGS, library)
+    check_launch(fn(QUANT_KEY_TO_GGML[quant_key], x_ptr, _KINDS[x_kind], qweight_ptr, out_ptr, _KINDS[out_kind], rows,
+                    in_features, out_features, rows_per_wave, loads_per_chunk, waves, stream), runtime)
+
+
+def gguf_q8_1_fused_gemv_stream_tuned(quant_key: str, x_ptr: int, x_kind: str, qweight_ptr: int, out_ptr: int,
+                                      out_kind: str, rows: int, in_features: int, out_features: int, *,
+                                      loads_in_flight: int, waves: int, waves_total: int, stream: int = 0,
+                                      library: ctypes.CDLL | None = None, runtime: HipRuntime | None = None) -> None:
+    """The stream form of the fused GEMV with an explicit layout (tuning sweeps only)."""
+    validate_linear(rows, in_features, out_features)
+    fn = entry("hipengine_gfx950_gguf_q8_1_fused_gemv_stream_tuned", _RUN_TUNED_ARGS, library)
+    check_launch(fn(QUANT_KEY_TO_GGML[quant_key], x_ptr, _KINDS[x_kind], qweight_ptr, out_ptr, _KINDS[out_kind], rows,
+                    in_features, out_features, loads_in_flight, waves, waves_total, stream), runtime)
+
+
 def gguf_gemv_default_plan(quant_key: str, rows: int, in_features: int, out_features: int, *,
                            library: ctypes.CDLL | None = None) -> dict[str, int]:
     """The workgroup layout the library picks for a shape (host only)."""

@@ -132,6 +132,26 @@ int hipengine_gfx950_gguf_q8_1_fused_gemv_tuned(int32_t ggml_type, const void* x
                                                 int32_t row_groups, int32_t blocks_per_wave, int32_t rows_per_lane,
                                                 hipengine_stream_t stream);
 
+/* The same for the "run" form of the kernel (a wave streams rows_per_wave whole
+ * rows as one contiguous run of blocks, loads_per_chunk 16-block loads at a
+ * time, `waves` waves per workgroup).  rows <= 2, rows_per_wave * (K/256) must
+ * be a multiple of 16.  New here. */
+int hipengine_gfx950_gguf_q8_1_fused_gemv_run_tuned(int32_t ggml_type, const void* x, int32_t x_kind,
+                                                    const uint8_t* qweight, void* out, int32_t out_kind,
+                                                    int64_t rows, int64_t in_features, int64_t out_features,
+                                                    int32_t rows_per_wave, int32_t loads_per_chunk, int32_t waves,
+                                                    hipengine_stream_t stream);
+
+/* The same for the "stream" form (waves_total resident waves, `waves` per
+ * workgroup, each owning a contiguous range of rows and keeping loads_in_flight
+ * 16-block loads in flight).  rows <= 2, in_features >= 4096,
+ * waves_total <= out_features.  New here. */
+int hipengine_gfx950_gguf_q8_1_fused_gemv_stream_tuned(int32_t ggml_type, const void* x, int32_t x_kind,
+                                                       const uint8_t* qweight, void* out, int32_t out_kind,
+                                                       int64_t rows, int64_t in_features, int64_t out_features,
+                                                       int32_t loads_in_flight, int32_t waves, int32_t waves_total,
+                                                       hipengine_stream_t stream);
+
 /* Host only: the layout the library picks for a shape, as
  * {batch_bucket, rows_per_lane, blocks_per_wave, k_slices, row_groups}.  New here. */
 int hipengine_gfx950_gguf_gemv_default_plan(int32_t ggml_type, int64_t rows, int64_t in_features,

@@ -1,0 +1,61 @@
+"""The C-ABI library loads and exports every function include/*.h declares.
+CPU only: nothing is launched."""
+
+from __future__ import annotations
+
+import ctypes
+import re
+import subprocess
+from pathlib import Path
+
+import pytest
+
+ROOT = Path(__file__).resolve().parents[1]
+HEADER = ROOT / "include" / "hipengine_gfx950.h"
+LIB = ROOT / "hipengine_amd" / "lib" / "libhipengine_gfx950.so"
+
+
+def declared_functions() -> list[str]:
+    text = subprocess.run(["gcc", "-E", "-P", str(HEADER)], check=True, capture_output=True, text=True).stdout
+    names = re.findall(r"\bint\s+(hipengine_[a-z0-9_]+)\s*\(", text)
+    assert len(names) >= 30
+    return sorted(set(names))
+
+
+@pytest.fixture(scope="module")
+def library() -> ctypes.CDLL:
+    if not LIB.exists():
+        from hipengine_amd.core.build import build_hip
+
+        build_hip(load=False)
+    return ctypes.CDLL(str(LIB))
+
+
+def test_header_compiles_as_c_and_cpp(tmp_path):
+    src = tmp_path / "t.c"
+    src.write_text(f'#include "{HEADER}"\nint main(void) {{ return 0; }}\n')
+    subprocess.run(["gcc", "-std=c11", "-Wall", "-Werror", "-fsyntax-only", str(src)], check=True)
+    subprocess.run(["g++", "-std=c++17", "-Wall", "-Werror", "-fsyntax-only", "-x", "c++", str(src)], check=True)
+
+
+def test_every_declared_function_is_exported(library):
+    missing = [n for n in declared_functions() if not hasattr(library, n)]
+    assert not missing, f"declared in the header but not exported: {missing}"
+
+
+def test_every_exported_entry_point_is_declared():
+    out = subprocess.run(["nm", "-D", "--defined-only", str(LIB)], check=True, capture_output=True, text=True).stdout
+    exported = {line.split()[-1] for line in out.splitlines() if " T " in line and "hipengine_" in line.split()[-1]
+                and not line.split()[-1].startswith("_Z")}
+    undeclared = sorted(exported - set(declared_functions()))
+    assert not undeclared, f"exported but not declared in the header: {undeclared}"
+
+
+def test_abi_version_and_host_only_entry_points(library):
+    assert library.hipengine_gfx950_abi_version() == 1
+    plan = (ctypes.c_int32 * 5)()
+    fn = library.hipengine_gfx950_gguf_gemv_default_plan
+    fn.argtypes = [ctypes.c_int32, ctypes.c_int64, ctypes.c_int64, ctypes.c_int64, ctypes.POINTER(ctypes.c_int32)]
+    assert fn(12, 1, 5120, 17408, plan) == 0 and plan[0] == 1
+    assert fn(12, 1, 100, 17408, plan) == 1          # hipErrorInvalidValue
+    assert fn(99, 1, 5120, 17408, plan) == 1

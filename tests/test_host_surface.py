@@ -1,0 +1,191 @@
+"""Host logic of the drop-in boundary: kernel registry semantics, quant plugin
+records, GGUF layout helpers and wrapper validation.  CPU only, no kernels run.
+
+The expectations restate hipEngine's own unit tests for these surfaces
+(tests/test_unit_kernel_registry.py:25-154, tests/test_unit_model_quant_and_imports.py:65-95,
+tests/test_unit_gguf_quant_layout.py:22-39, tests/test_gpu_gguf_q4_k_gemv.py:206-223).
+"""
+
+from __future__ import annotations
+
+import subprocess
+import sys
+from pathlib import Path
+
+import pytest
+
+from hipengine_amd import quant
+from hipengine_amd.kernels import registry as R
+from hipengine_amd.kernels.registry import KernelKey
+from hipengine_amd.quant import GGMLQuantizationType as T
+
+ROOT = Path(__file__).resolve().parents[1]
+
+
+@pytest.fixture()
+def clean_registry():
+    saved = R.snapshot_registry_for_tests()
+    R.clear_registry_for_tests()
+    yield
+    R.restore_registry_for_tests(saved)
+
+
+def test_kernel_key_validation_and_display():
+    with pytest.raises(ValueError):
+        KernelKey("", "linear", "fp16")
+    with pytest.raises(ValueError):
+        KernelKey("hip_gfx950", "linear", "")
+    assert "variant='v'" in KernelKey("b", "l", "q", "v").display()
+    assert KernelKey("a", "l", "q") < KernelKey("b", "l", "q")
+
+
+def test_registry_exact_duplicate_and_fallback_order(clean_registry):
+    def exact(): return "exact"
+    def novar(): return "novar"
+    def fp16(): return "fp16"
+    def cpu(): return "cpu"
+
+    R.register(KernelKey("cpu_reference", "linear", "fp16"), cpu)
+    assert R.resolve(backend="hip_gfx950", layer="linear", quant="gguf_q4_k", variant="v")() == "cpu"
+    R.register(KernelKey("hip_gfx950", "linear", "fp16"), fp16)
+    assert R.resolve(backend="hip_gfx950", layer="linear", quant="gguf_q4_k", variant="v")() == "fp16"
+    R.register(KernelKey("hip_gfx950", "linear", "gguf_q4_k"), novar)
+    assert R.resolve(backend="hip_gfx950", layer="linear", quant="gguf_q4_k", variant="v")() == "novar"
+    R.register(KernelKey("hip_gfx950", "linear", "gguf_q4_k", "v"), exact)
+    assert R.resolve(backend="hip_gfx950", layer="linear", quant="gguf_q4_k", variant="v")() == "exact"
+    with pytest.raises(R.DuplicateKernelError):
+        R.register(KernelKey("hip_gfx950", "linear", "gguf_q4_k", "v"), exact)
+    R.register(KernelKey("hip_gfx950", "linear", "gguf_q4_k", "v"), novar, replace=True)
+    assert R.resolve(backend="hip_gfx950", layer="linear", quant="gguf_q4_k", variant="v")() == "novar"
+    assert R.is_registered(KernelKey("hip_gfx950", "linear", "gguf_q4_k", "v"))
+    assert not R.is_registered(KernelKey("hip_gfx950", "linear", "gguf_q4_k", "other"))   # exact only
+    assert R.can_resolve(backend="hip_gfx950", layer="linear", quant="gguf_q4_k", variant="other")
+
+
+def test_registry_missing_error_generation_and_cache_invalidation(clean_registry):
+    g0 = R.generation()
+    with pytest.raises(R.MissingKernelError) as info:
+        R.resolve(backend="hip_gfx950", layer="linear", quant="gguf_q4_k", variant="v")
+    assert info.value.requested == KernelKey("hip_gfx950", "linear", "gguf_q4_k", "v")
+    assert [k.backend for k in info.value.attempted] == ["hip_gfx950"] * 4 + ["cpu_reference"] * 4
+    assert R.resolve(backend="x", layer="l", quant="q", missing="none") is None
+    def a(): return "a"
+    def b(): return "b"
+    R.register(KernelKey("hip_gfx950", "linear", "fp16"), a)
+    assert R.generation() > g0
+    assert R.resolve(backend="hip_gfx950", layer="linear", quant="gguf_q4_k")() == "a"      # memoized fallback
+    R.register(KernelKey("hip_gfx950", "linear", "gguf_q4_k"), b)
+    assert R.resolve(backend="hip_gfx950", layer="linear", quant="gguf_q4_k")() == "b"      # memo dropped
+    R.unregister(KernelKey("hip_gfx950", "linear", "gguf_q4_k"))
+    assert R.resolve(backend="hip_gfx950", layer="linear", quant="gguf_q4_k")() == "a"
+    snap = R.snapshot_registry_for_tests()
+    R.clear_registry_for_tests()
+    assert R.registered_keys() == ()
+    R.restore_registry_for_tests(snap)
+    assert R.registered_keys() == tuple(sorted(snap))
+
+
+def test_backend_registers_the_documented_keys(clean_registry):
+    from hipengine_amd.kernels import hip_gfx950
+
+    hip_gfx950.register_backend_kernels(replace=True)
+    keys = set(R.registered_keys())
+    for q in ("gguf_q4_k", "gguf_q6_k", "gguf_q8_0"):
+        for v in ("q8_1_fused_gemv_f32_f32_out", "q8_1_fused_gemv_bf16_bf16_out", "q8_1_fused_prefill_bf16_f32_out"):
+            assert KernelKey("hip_gfx950", "linear", q, v) in keys
+    assert KernelKey("hip_gfx950", "linear", "gguf_q4_k", "q8_1_dp4a_vdr_bf16_f32_out") in keys
+    assert KernelKey("hip_gfx950", "activation_quant", "q8_1_ds4", "bf16_kmajor") in keys
+    assert not any(k.backend == "cpu_reference" for k in keys)            # the package ships no CPU path
+    assert hip_gfx950.GGUF_CONSUMER_LAYERS >= {"linear", "moe_linear"}
+    fn = R.resolve(backend="hip_gfx950", layer="linear", quant="gguf_q4_k", variant="q8_1_fused_gemv_f32_f32_out")
+    assert fn.__name__ == "gguf_q4_k_q8_1_fused_gemv_f32_f32_out"
+
+
+def test_quant_plugin_records():
+    p = quant.resolve_quant("gguf_q4_k")
+    assert (p.weight_storage, p.activation_preprocess, p.compute_dtype, p.scale_granularity, p.calibration_artifact,
+            p.kernel_family) == ("gguf_block_q4_k", "none", "fp32_accum", "block256_subblock32_scale_min", "gguf",
+                                 "gguf_q4_k_gemv")
+    p6, p8 = quant.resolve_quant("gguf_q6_k"), quant.resolve_quant("gguf_q8_0")
+    assert (p6.weight_storage, p6.scale_granularity, p6.kernel_family) == ("gguf_block_q6_k", "block256_subblock16_scale", "gguf_k_gemv")
+    assert (p8.weight_storage, p8.scale_granularity, p8.kernel_family) == ("gguf_block_q8_0", "block32_scale", "gguf_k_gemv")
+    assert isinstance(p, quant.QuantPlugin)
+    with pytest.raises(quant.DuplicateQuantError):
+        quant.register_quant(quant.GGUFQ4KQuant())
+    with pytest.raises(quant.MissingQuantError, match="gguf_q4_k"):
+        quant.resolve_quant("nope")
+    with pytest.raises(ValueError):
+        quant.register_quant(quant.GGUFQ4KQuant(name=""))
+    assert [q.name for q in quant.registered_quants()] == sorted(q.name for q in quant.registered_quants())
+
+
+def test_gguf_layout_table_and_byte_shapes():
+    assert (quant.quant_layout(T.Q8_0).block_size, quant.quant_layout(T.Q8_0).type_size) == (32, 34)
+    assert (quant.quant_layout(T.Q4_K).block_size, quant.quant_layout(T.Q4_K).type_size) == (256, 144)
+    assert quant.quant_layout(T.Q5_K).type_size == 176
+    assert quant.quant_layout(T.Q6_K).type_size == 210
+    assert quant.quant_layout(T.BF16).type_size == 2
+    assert quant.quant_layout(12).name == "Q4_K" and quant.quant_layout(T.Q4_K).is_block_quantized
+    assert quant.nbytes_for_shape((3, 64), T.Q8_0) == 3 * 2 * 34
+    assert quant.nbytes_for_shape((17408, 5120), T.Q4_K) == 50_135_040
+    assert quant.nbytes_for_shape((5120, 17408), T.Q6_K) == 73_113_600
+    assert quant.quant_shape_to_byte_shape((3, 64), T.Q8_0) == (3, 68)
+    assert quant.quant_shape_from_byte_shape((3, 68), T.Q8_0) == (3, 64)
+    assert quant.quant_shape_to_byte_shape((2, 5), T.F32) == (2, 5)
+    with pytest.raises(ValueError, match="row size 63"):
+        quant.quant_shape_to_byte_shape((3, 63), T.Q8_0)
+    with pytest.raises(ValueError):
+        quant.nbytes_for_shape((3, 63), T.Q8_0)
+    with pytest.raises(ValueError):
+        quant.quant_shape_from_byte_shape((3, 67), T.Q8_0)
+    with pytest.raises(KeyError):
+        quant.quant_layout(999)
+    assert quant.GGUF_Q8_1_MMQ_DS4_BYTES == 144 and quant.GGUF_Q4_K_BLOCK_BYTES == 144 and quant.QK_K == 256
+
+
+def test_wrappers_validate_before_touching_the_library():
+    from hipengine_amd.kernels.hip_gfx950.quant import gguf_q8_1_gemv as G
+    from hipengine_amd.kernels.hip_gfx950.quant import gguf_quantize as Q
+
+    fn = G.FUSED[("q4_k", "bf16", "bf16")]
+    with pytest.raises(ValueError, match="divisible"):
+        fn(1, 1, 1, 1, 100, 8)
+    with pytest.raises(ValueError, match="threads"):
+        fn(1, 1, 1, 1, 256, 8, threads=96)
+    with pytest.raises(ValueError, match="rows"):
+        fn(1, 1, 1, 0, 256, 8)
+    with pytest.raises(ValueError, match="pointer"):
+        fn(0, 1, 1, 1, 256, 8)
+    with pytest.raises(ValueError, match="divisible"):
+        Q.gguf_q8_1_mmq_ds4_pack_bf16(1, 1, 1, 192)
+    assert Q.q8_1_workspace_nbytes(2, 5120) == 2 * 160 * 36
+    assert Q.ds4_workspace_nbytes(2048, 5120) == 2048 * 40 * 144
+
+
+def test_host_package_is_torch_free():
+    """Importing the package, the wrappers and bench.py's harness must not import torch."""
+    code = ("import sys; sys.path.insert(0, %r); import hipengine_amd, hipengine_amd.quant, "
+            "hipengine_amd.kernels.hip_gfx950 as b; b.register_backend_kernels(); "
+            "import hipengine_amd.core.hip, hipengine_amd.core.memory, hipengine_amd.core.build, hipengine_amd.synthetic; "
+            "assert 'torch' not in sys.modules, 'torch was imported'; "
+            "import hipengine_amd.core.hip as h; assert not h.is_default_runtime_loaded()") % str(ROOT)
+    subprocess.run([sys.executable, "-c", code], check=True)
+
+
+def test_product_package_never_imports_the_oracle():
+    for path in (ROOT / "hipengine_amd").rglob("*.py"):
+        text = path.read_text()
+        assert "import oracle" not in text and "from oracle" not in text, path
+
+
+def test_build_plan_is_stable_and_names_the_artifact():
+    from hipengine_amd.core import build
+
+    a = build.plan_hip_build(compiler_version="test")
+    b = build.plan_hip_build(compiler_version="test")
+    assert a.key == b.key and len(a.key) == 64
+    assert a.output.name == "libhipengine_gfx950.so"
+    assert {s.name for s in a.sources} >= {"gguf_gemv.hip", "gguf_quantize.hip", "gguf_verify.hip"}
+    assert "--offload-arch=gfx950" in a.flags and "-mcumode" not in a.flags
+    assert build.plan_hip_build(compiler_version="other").key != a.key
+    assert a.commands[-1][-1].endswith("libhipengine_gfx950.so")
