@@ -1,0 +1,248 @@
+// MMQ prefill GEMM on int8 MFMA for gfx950: raw Q4_K weights x DS4 q8_1
+// activations -> float32 / bf16, and raw Q6_K weights x D4S4 activations.
+//
+//   Q4_K: out[m,n] = sum_{32-wide sub-block j} (d*sc_j)[n] * xd_j[m] * dot_j[m,n] - (dmin*mn_j)[n] * xsum_j[m]
+//         (kernels/hip_gfx1100/quant/gguf_q4_k_q8_1_mmq_prefill.hip:265-276)
+//   Q6_K: out[m,n] = sum_{32-wide group g} xd_g[m] * (s0*dot0 + s1*dot1),  s = d*scale_i8, dots over 16 values
+//         (kernels/hip_gfx1100/quant/gguf_k_mmq_prefill.hip:652-667)
+//
+// Structure (256 threads = 4 waves, 128x128 output tile, each wave 64x64 as 2x2
+// MFMA tiles of 32x32):
+//   * per 256-value K block the workgroup copies the 128 raw weight blocks and
+//     the 128 activation rows into LDS with coalesced 16-byte loads and decodes
+//     the per-sub-block scale tables once;
+//   * a wave reads MFMA operands straight from those LDS images: the int8
+//     activation bytes as they are, the weight nibbles split in registers
+//     (Q6_K: 6-bit values rebuilt and centred in registers).  The MFMA K
+//     extent is one scale group: v_mfma_i32_32x32x32_i8 per Q4_K sub-block,
+//     v_mfma_i32_32x32x16_i8 per 16 Q6_K values, so every int32 result is an
+//     exact sub-block dot;
+//   * the accumulator input of each MFMA is the integer 0x4B400000, so the
+//     int32 result reinterpreted as float IS 12582912 + dot; one FMA with the
+//     per-column constants (sw, -12582912*sw) yields the correctly rounded
+//     sw*dot without an int->float conversion, a second FMA applies the
+//     per-row activation scale;
+//   * the Q4_K min term is rank-8 per block: sum_j mn_j[n]*xsum_j[m] is computed
+//     by one v_mfma_f32_32x32x8f16 (both operands are exact in fp16: xsum is
+//     stored as fp16, mn_j <= 63) and scaled by dmin[n] once per block.
+//
+// The float32 epilogue (2 VALU ops per output element per sub-block, 64 lanes
+// per CU-cycle) bounds this formulation at about a quarter of the int8 MFMA
+// peak: the MFMA pipe itself is mostly idle.
+
+#include "gguf_common.hpp"
+
+#include "../../include/hipengine_gfx950.h"
+
+namespace {
+
+using namespace hipengine_gfx950;
+
+typedef int v4i __attribute__((ext_vector_type(4)));
+typedef int v16i __attribute__((ext_vector_type(16)));
+typedef float v16f __attribute__((ext_vector_type(16)));
+typedef _Float16 v4h __attribute__((ext_vector_type(4)));
+
+constexpr int BM = 128, BN = 128, THREADS = 256;
+constexpr int W_STRIDE_Q4 = 144;            // raw block per row; 9 x 16 B is conflict free for b128 reads
+constexpr int A_STRIDE_DS4 = 304;           // 2 x 144 B padded to an odd number of 16-byte units
+constexpr uint32_t MAGIC_BITS = 0x4B400000u;   // float 12582912 = 1.5 * 2^23
+constexpr float MAGIC = 12582912.0f;
+
+struct MmqArgs {
+  const uint8_t* xq;
+  const uint8_t* w;
+  void* out;
+  int out_kind;
+  int M, K, N;
+};
+
+struct Q4Smem {
+  uint8_t wq[BN * W_STRIDE_Q4];
+  uint8_t xa[BM * A_STRIDE_DS4];
+  float sw[8][BN];       // d*sc per sub-block, column
+  float cw[8][BN];       // -MAGIC * sw
+  float xd[8][BM];       // activation scale per sub-block, row
+  float dmin[BN];
+  _Float16 mnh[BN][8];   // 6-bit mins as fp16
+  _Float16 xsh[BM][8];   // activation sums (already fp16 in the DS4 block)
+};
+
+__device__ __forceinline__ void store_tile(const MmqArgs& a, const float (&acc)[16], int m_base, int n_col) {
+  // lane holds column n_col and rows m_base + 8*(v/4) + v%4 (m_base already includes 4*(lane/32))
+  if (n_col >= a.N) return;
+#pragma unroll
+  for (int v = 0; v < 16; ++v) {
+    const int m = m_base + 8 * (v >> 2) + (v & 3);
+    if (m < a.M) store_scalar(a.out, static_cast<int64_t>(m) * a.N + n_col, acc[v], a.out_kind);
+  }
+}
+
+__global__ void __launch_bounds__(THREADS, 2) mmq_q4_k_ds4_kernel(MmqArgs a) {
+  extern __shared__ __align__(16) uint8_t smem_raw[];
+  Q4Smem& s = *reinterpret_cast<Q4Smem*>(smem_raw);
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int wm = wave & 1, wn = wave >> 1;
+  const int lc = lane & 31, g = lane >> 5;
+  const int m0 = blockIdx.x * BM, n0 = blockIdx.y * BN;
+  const int nb = a.K / QK_K;
+  const int64_t w_row_bytes = static_cast<int64_t>(nb) * Q4_K_BYTES;
+  const int64_t x_row_bytes = static_cast<int64_t>(a.K / 128) * DS4_BYTES;
+
+  float acc[2][2][16];   // [n tile][m tile][v]
+#pragma unroll
+  for (int i = 0; i < 2; ++i)
+#pragma unroll
+    for (int j = 0; j < 2; ++j)
+#pragma unroll
+      for (int v = 0; v < 16; ++v) acc[i][j][v] = 0.0f;
+
+  for (int kb = 0; kb < nb; ++kb) {
+    // ---- stage raw tiles --------------------------------------------------
+    for (int c = tid; c < BN * 9; c += THREADS) {
+      const int row = c / 9, part = c - row * 9;
+      const int n = min(n0 + row, a.N - 1);
+      const uint4 v = *reinterpret_cast<const uint4*>(a.w + n * w_row_bytes + static_cast<int64_t>(kb) * Q4_K_BYTES + part * 16);
+      *reinterpret_cast<uint4*>(s.wq + row * W_STRIDE_Q4 + part * 16) = v;
+    }
+    for (int c = tid; c < BM * 18; c += THREADS) {
+      const int row = c / 18, part = c - row * 18;
+      const int m = min(m0 + row, a.M - 1);
+      const uint4 v = *reinterpret_cast<const uint4*>(a.xq + m * x_row_bytes + static_cast<int64_t>(kb) * 2 * DS4_BYTES + part * 16);
+      *reinterpret_cast<uint4*>(s.xa + row * A_STRIDE_DS4 + part * 16) = v;
+    }
+    // ---- decode scale tables (from global again: no dependency on the tiles) ----
+    if (tid < BN) {
+      const int n = min(n0 + tid, a.N - 1);
+      const uint4 h = *reinterpret_cast<const uint4*>(a.w + n * w_row_bytes + static_cast<int64_t>(kb) * Q4_K_BYTES);
+      const Q4KScales u = q4k_unpack_scales(h.y, h.z, h.w);
+      const float d = f16_bits_to_float(h.x & 0xFFFFu);
+      s.dmin[tid] = f16_bits_to_float(h.x >> 16);
+#pragma unroll
+      for (int j = 0; j < 8; ++j) {
+        const uint32_t sc = ((j < 4 ? u.sc_lo : u.sc_hi) >> (8 * (j & 3))) & 0xFFu;
+        const uint32_t mn = ((j < 4 ? u.mn_lo : u.mn_hi) >> (8 * (j & 3))) & 0xFFu;
+        const float sw = d * static_cast<float>(sc);
+        s.sw[j][tid] = sw;
+        s.cw[j][tid] = -MAGIC * sw;
+        s.mnh[tid][j] = static_cast<_Float16>(static_cast<float>(mn));
+      }
+    } else {
+      const int r = tid - BN;
+      const int m = min(m0 + r, a.M - 1);
+      const uint8_t* xb = a.xq + m * x_row_bytes + static_cast<int64_t>(kb) * 2 * DS4_BYTES;
+      const uint4 h0 = *reinterpret_cast<const uint4*>(xb);
+      const uint4 h1 = *reinterpret_cast<const uint4*>(xb + DS4_BYTES);
+      const uint32_t hh[8] = {h0.x, h0.y, h0.z, h0.w, h1.x, h1.y, h1.z, h1.w};
+#pragma unroll
+      for (int j = 0; j < 8; ++j) {
+        s.xd[j][r] = f16_bits_to_float(hh[j] & 0xFFFFu);
+        s.xsh[r][j] = __builtin_bit_cast(_Float16, static_cast<uint16_t>(hh[j] >> 16));
+      }
+    }
+    __syncthreads();
+
+    // ---- int8 MFMA over the 8 sub-blocks ------------------------------------
+#pragma unroll
+    for (int sp = 0; sp < 4; ++sp) {
+      v4i wlo[2], whi[2];
+#pragma unroll
+      for (int nt = 0; nt < 2; ++nt) {
+        const int row = wn * 64 + nt * 32 + lc;
+        const uint4 qs = *reinterpret_cast<const uint4*>(s.wq + row * W_STRIDE_Q4 + 16 + sp * 32 + 16 * g);
+        wlo[nt] = v4i{static_cast<int>(q4k_low(qs.x)), static_cast<int>(q4k_low(qs.y)),
+                      static_cast<int>(q4k_low(qs.z)), static_cast<int>(q4k_low(qs.w))};
+        whi[nt] = v4i{static_cast<int>(q4k_high(qs.x)), static_cast<int>(q4k_high(qs.y)),
+                      static_cast<int>(q4k_high(qs.z)), static_cast<int>(q4k_high(qs.w))};
+      }
+#pragma unroll
+      for (int half = 0; half < 2; ++half) {
+        const int sb = 2 * sp + half;
+#pragma unroll
+        for (int mt = 0; mt < 2; ++mt) {
+          const int arow = wm * 64 + mt * 32 + lc;
+          const v4i xop = *reinterpret_cast<const v4i*>(s.xa + arow * A_STRIDE_DS4 + (sb >> 2) * DS4_BYTES + 16 +
+                                                        (sb & 3) * 32 + 16 * g);
+          float xdv[16];
+#pragma unroll
+          for (int j = 0; j < 4; ++j) {
+            const float4 t = *reinterpret_cast<const float4*>(&s.xd[sb][wm * 64 + mt * 32 + 8 * j + 4 * g]);
+            xdv[4 * j] = t.x; xdv[4 * j + 1] = t.y; xdv[4 * j + 2] = t.z; xdv[4 * j + 3] = t.w;
+          }
+#pragma unroll
+          for (int nt = 0; nt < 2; ++nt) {
+            const int col = wn * 64 + nt * 32 + lc;
+            const float sw = s.sw[sb][col], cw = s.cw[sb][col];
+            v16i c0;
+#pragma unroll
+            for (int v = 0; v < 16; ++v) c0[v] = static_cast<int>(MAGIC_BITS);
+            const v16i d = __builtin_amdgcn_mfma_i32_32x32x32_i8(xop, half ? whi[nt] : wlo[nt], c0, 0, 0, 0);
+#pragma unroll
+            for (int v = 0; v < 16; ++v) {
+              const float t = __builtin_fmaf(bits_to_float(static_cast<uint32_t>(d[v])), sw, cw);   // = sw * dot, rounded once
+              acc[nt][mt][v] = __builtin_fmaf(xdv[v], t, acc[nt][mt][v]);
+            }
+          }
+        }
+      }
+    }
+
+    // ---- min term: dmin[n] * sum_j mn_j[n] * xsum_j[m] on the fp16 MFMA -------
+#pragma unroll
+    for (int mt = 0; mt < 2; ++mt) {
+      const int arow = wm * 64 + mt * 32 + lc;
+      const v4h xs = *reinterpret_cast<const v4h*>(&s.xsh[arow][4 * g]);
+#pragma unroll
+      for (int nt = 0; nt < 2; ++nt) {
+        const int col = wn * 64 + nt * 32 + lc;
+        const v4h mn = *reinterpret_cast<const v4h*>(&s.mnh[col][4 * g]);
+        v16f z;
+#pragma unroll
+        for (int v = 0; v < 16; ++v) z[v] = 0.0f;
+        const v16f t = __builtin_amdgcn_mfma_f32_32x32x8f16(xs, mn, z, 0, 0, 0);
+        const float nd = -s.dmin[col];
+#pragma unroll
+        for (int v = 0; v < 16; ++v) acc[nt][mt][v] = __builtin_fmaf(nd, t[v], acc[nt][mt][v]);
+      }
+    }
+    __syncthreads();   // the next block overwrites the tiles
+  }
+
+#pragma unroll
+  for (int nt = 0; nt < 2; ++nt)
+#pragma unroll
+    for (int mt = 0; mt < 2; ++mt)
+      store_tile(a, acc[nt][mt], m0 + wm * 64 + mt * 32 + 4 * g, n0 + wn * 64 + nt * 32 + lc);
+}
+
+int launch_q4(const void* xq, const uint8_t* w, void* out, int out_kind, int64_t M, int64_t K, int64_t N,
+              hipStream_t stream) {
+  if (!xq || !w || !out || M <= 0 || M > (1 << 20) || K <= 0 || (K % QK_K) != 0 || N <= 0 || (N % 32) != 0 ||
+      N > (1 << 24)) {
+    return static_cast<int>(hipErrorInvalidValue);
+  }
+  MmqArgs a{static_cast<const uint8_t*>(xq), w, out, out_kind, static_cast<int>(M), static_cast<int>(K),
+            static_cast<int>(N)};
+  const dim3 grid(static_cast<unsigned>((M + BM - 1) / BM), static_cast<unsigned>((N + BN - 1) / BN));
+  static bool attr_set = false;
+  if (!attr_set) {
+    (void)hipFuncSetAttribute(reinterpret_cast<const void*>(mmq_q4_k_ds4_kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
+                              static_cast<int>(sizeof(Q4Smem)));
+    attr_set = true;
+  }
+  hipLaunchKernelGGL(mmq_q4_k_ds4_kernel, grid, dim3(THREADS), sizeof(Q4Smem), stream, a);
+  return static_cast<int>(hipGetLastError());
+}
+
+}  // namespace
+
+#define DEFINE_MMQ_Q4(SYMBOL, OKIND)                                                                        \
+  extern "C" int SYMBOL(const void* xq, const uint8_t* qweight, void* out, int64_t rows, int64_t in_features, \
+                        int64_t out_features, hipStream_t stream) {                                         \
+    return launch_q4(xq, qweight, out, OKIND, rows, in_features, out_features, stream);                     \
+  }
+
+DEFINE_MMQ_Q4(hipengine_gguf_q4_k_q8_1_mmq32_vdr_dense_bf16_f32_out, KIND_F32)
+DEFINE_MMQ_Q4(hipengine_gguf_q4_k_q8_1_mmq32_vdr_dense_bf16_bf16_out, KIND_BF16)
+DEFINE_MMQ_Q4(hipengine_gguf_q4_k_q8_1_mmq32_ctl_dense_bf16_f32_out, KIND_F32)
+DEFINE_MMQ_Q4(hipengine_gguf_q4_k_q8_1_mmq32_ctl_dense_bf16_bf16_out, KIND_BF16)

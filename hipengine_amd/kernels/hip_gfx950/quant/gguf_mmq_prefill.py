@@ -1,0 +1,61 @@
+"""MMQ prefill GEMM wrappers (int8 MFMA): raw Q4_K x DS4 q8_1 and raw Q6_K x D4S4 q8_1.
+
+Signature ``fn(xq_ptr, qweight_ptr, out_ptr, rows, hidden, out_features, *, stream,
+library, runtime)`` as in hipEngine's ``gguf_q4_k_q8_1_mmq_prefill.py`` /
+``gguf_k_mmq_prefill.py:349-397``; registry variants as in
+``tests/test_gpu_gguf_q4_k_q8_1_mmq_prefill.py:362-382`` and ``gguf_k_mmq_prefill.py:793-802``.
+"""
+
+from __future__ import annotations
+
+import ctypes
+
+from hipengine_amd.core.hip import HipRuntime
+from hipengine_amd.kernels.hip_gfx950._launch import I64, VOID, check_launch, entry, validate_pointers
+from hipengine_amd.kernels.registry import KernelKey, register
+
+_ARGS = [VOID, VOID, VOID, I64, I64, I64, VOID]
+
+
+def _validate(rows: int, hidden: int, out_features: int, out_multiple: int) -> None:
+    if rows <= 0 or rows > (1 << 20):
+        raise ValueError("rows must be in 1..2^20")
+    if hidden <= 0 or hidden % 256 != 0:
+        raise ValueError("hidden must be positive and divisible by the GGUF block size 256")
+    if out_features <= 0 or out_features % out_multiple != 0:
+        raise ValueError(f"out_features must be positive and divisible by {out_multiple}")
+
+
+def _make(name: str, symbol: str, out_multiple: int):
+    def wrapper(xq_ptr: int, qweight_ptr: int, out_ptr: int, rows: int, hidden: int, out_features: int, *,
+                stream: int = 0, library: ctypes.CDLL | None = None, runtime: HipRuntime | None = None) -> None:
+        _validate(rows, hidden, out_features, out_multiple)
+        validate_pointers(xq_ptr=xq_ptr, qweight_ptr=qweight_ptr, out_ptr=out_ptr)
+        check_launch(entry(symbol, _ARGS, library)(xq_ptr, qweight_ptr, out_ptr, rows, hidden, out_features, stream),
+                     runtime)
+
+    wrapper.__name__ = name
+    wrapper.__doc__ = f"MMQ prefill GEMM over pre-quantized q8_1 activations (C symbol ``{symbol}``)."
+    return wrapper
+
+
+gguf_q4_k_q8_1_mmq32_vdr_dense_bf16_f32_out = _make(
+    "gguf_q4_k_q8_1_mmq32_vdr_dense_bf16_f32_out", "hipengine_gguf_q4_k_q8_1_mmq32_vdr_dense_bf16_f32_out", 32)
+gguf_q4_k_q8_1_mmq32_vdr_dense_bf16_bf16_out = _make(
+    "gguf_q4_k_q8_1_mmq32_vdr_dense_bf16_bf16_out", "hipengine_gguf_q4_k_q8_1_mmq32_vdr_dense_bf16_bf16_out", 32)
+gguf_q4_k_q8_1_mmq32_ctl_dense_bf16_f32_out = _make(
+    "gguf_q4_k_q8_1_mmq32_ctl_dense_bf16_f32_out", "hipengine_gguf_q4_k_q8_1_mmq32_ctl_dense_bf16_f32_out", 32)
+gguf_q4_k_q8_1_mmq32_ctl_dense_bf16_bf16_out = _make(
+    "gguf_q4_k_q8_1_mmq32_ctl_dense_bf16_bf16_out", "hipengine_gguf_q4_k_q8_1_mmq32_ctl_dense_bf16_bf16_out", 32)
+
+_Q4 = (
+    ("mmq32_vdr_dense_bf16_f32_out", gguf_q4_k_q8_1_mmq32_vdr_dense_bf16_f32_out),
+    ("mmq32_vdr_dense_bf16_bf16_out", gguf_q4_k_q8_1_mmq32_vdr_dense_bf16_bf16_out),
+    ("mmq32_ctl_dense_bf16_f32_out", gguf_q4_k_q8_1_mmq32_ctl_dense_bf16_f32_out),
+    ("mmq32_ctl_dense_bf16_bf16_out", gguf_q4_k_q8_1_mmq32_ctl_dense_bf16_bf16_out),
+)
+
+
+def register_kernels(backend: str = "hip_gfx950", *, replace: bool = False) -> None:
+    for variant, fn in _Q4:
+        register(KernelKey(backend, "linear", "gguf_q4_k", variant), fn, replace=replace)

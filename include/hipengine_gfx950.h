@@ -158,6 +158,30 @@ int hipengine_gfx950_gguf_gemv_default_plan(int32_t ggml_type, int64_t rows, int
                                             int64_t out_features, int32_t* plan5);
 
 /* ------------------------------------------------------------------------
+ * MMQ prefill GEMM on int8 MFMA
+ *   out[m, n] = sum_k W[n, k] * x[m, k],  x pre-quantized to q8_1 (128-value blocks)
+ * rows <= 2^20, in_features % 256 == 0, out_features % 32 == 0.
+ * ------------------------------------------------------------------------ */
+
+/* Raw Q4_K weights x DS4 activations ([rows, in_features/128] 144-byte blocks):
+ * sum_j (d*sc_j)*xd_j*dot_j - (dmin*mn_j)*xsum_j per 32-wide sub-block.
+ * Replaces gguf_q4_k_q8_1_mmq_prefill.hip:421-454,516-519 (kernel :158-289); the
+ * ctl and vdr names are the same kernel here, as their results are identical by
+ * hipEngine's own contract (:20-27). */
+int hipengine_gguf_q4_k_q8_1_mmq32_vdr_dense_bf16_f32_out(const void* xq, const uint8_t* qweight, void* out,
+                                                          int64_t rows, int64_t in_features, int64_t out_features,
+                                                          hipengine_stream_t stream);
+int hipengine_gguf_q4_k_q8_1_mmq32_vdr_dense_bf16_bf16_out(const void* xq, const uint8_t* qweight, void* out,
+                                                           int64_t rows, int64_t in_features, int64_t out_features,
+                                                           hipengine_stream_t stream);
+int hipengine_gguf_q4_k_q8_1_mmq32_ctl_dense_bf16_f32_out(const void* xq, const uint8_t* qweight, void* out,
+                                                          int64_t rows, int64_t in_features, int64_t out_features,
+                                                          hipengine_stream_t stream);
+int hipengine_gguf_q4_k_q8_1_mmq32_ctl_dense_bf16_bf16_out(const void* xq, const uint8_t* qweight, void* out,
+                                                           int64_t rows, int64_t in_features, int64_t out_features,
+                                                           hipengine_stream_t stream);
+
+/* ------------------------------------------------------------------------
  * Verification exports: the integer unpack and the int32 sub-block dots the
  * production kernels compute, written out so that they can be compared bit for
  * bit with a CPU oracle.  New here.

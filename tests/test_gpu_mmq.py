@@ -1,0 +1,109 @@
+"""GPU parity of the activation packers (DS4, D4S4) and of the MMQ prefill GEMM
+(int8 MFMA) through the C ABI.
+
+Gates: packed activation bytes identical to the oracle's; float32 outputs within
+max relative error 1e-3 / cosine 0.99999 of (a) the MMQ formula evaluated in
+float64 and (b) the reference CPU GEMV (dequantize -> float32 matmul) applied to
+the dequantized q8 activations (the pattern of
+tests/test_gpu_gguf_k_mmq_prefill.py:528-541 in the hipEngine tree); bf16 output
+equals bf16_round(float32 output); ctl and vdr entry points bit-identical;
+repeated runs bit-identical.
+"""
+
+from __future__ import annotations
+
+import numpy as np
+import pytest
+
+from oracle import c_oracle as C
+from oracle import gguf_oracle as O
+from hipengine_amd.kernels.hip_gfx950.quant import gguf_mmq_prefill as M
+from hipengine_amd.kernels.hip_gfx950.quant import gguf_quantize as Q
+
+pytestmark = pytest.mark.gpu
+
+
+def _bf16_rows(seed, rows, k, scale=1.0, offset=0.0):
+    rng = np.random.default_rng(seed)
+    x = (rng.standard_normal((rows, k)) * scale + offset).astype(np.float32)
+    x[0, :32] = 0.0
+    if rows > 2:
+        x[2, 32:64] = np.arange(-16, 16) / 8.0
+        x[2, 63] = 127.0 / 8.0          # exact .5 ties: DS4 rounds to even, D4S4 away from zero
+    return O.f32_to_bf16_bits(x)
+
+
+@pytest.mark.parametrize("rows,k", [(1, 128), (5, 1024), (33, 5120)])
+def test_ds4_and_d4s4_pack_bytes(dev, rows, k):
+    xb = _bf16_rows(rows + k, rows, k)
+    dx = dev.put(xb)
+    for fn, nbytes, want in ((Q.gguf_q8_1_mmq_ds4_pack_bf16, 144, O.pack_q8_1_ds4(xb)),
+                             (Q.gguf_q8_1_d4s4_f32_quantize_bf16, 160, O.pack_q8_1_d4s4(xb))):
+        dq = dev.empty(rows * (k // 128) * nbytes)
+        fn(dx.ptr, dq.ptr, rows, k)
+        got = dev.get(dq, np.uint8, want.shape)
+        dev.free(dq)
+        assert np.array_equal(got, want)
+    assert np.array_equal(O.pack_q8_1_ds4(xb), C.pack_ds4(xb))
+    dev.free(dx)
+
+
+def _run_q4(dev, fn, ds4, w, rows, k, n, out_dtype=np.float32):
+    dxq, dw = dev.put(ds4), dev.put(w)
+    dout = dev.empty(rows * n * np.dtype(out_dtype).itemsize)
+    fn(dxq.ptr, dw.ptr, dout.ptr, rows, k, n)
+    got = dev.get(dout, out_dtype, (rows, n))
+    dev.free(dxq, dw, dout)
+    return got
+
+
+@pytest.mark.parametrize("rows,k,n", [(1, 256, 32), (7, 512, 64), (128, 1024, 128), (130, 768, 160), (300, 5120, 416)])
+def test_q4_k_mmq_matches_formula_and_cpu_reference(dev, rows, k, n):
+    xb = _bf16_rows(7 * rows + k + n, rows, k, scale=0.1, offset=0.002)
+    ds4 = O.pack_q8_1_ds4(xb)
+    w = O.random_weight(O.GGML_Q4_K, n, k, seed=k + n)
+    got = _run_q4(dev, M.gguf_q4_k_q8_1_mmq32_vdr_dense_bf16_f32_out, ds4, w, rows, k, n)
+    want = O.mmq_q4_k_ds4(ds4, w)                     # float64 evaluation of the MMQ formula
+    assert O.max_rel_err(got, want) <= 1e-3 and O.cosine(got, want) >= 0.99999
+    assert O.max_rel_err(got, C.mmq_q4_k_ds4(ds4, w)) <= 1e-3
+    # the reference CPU backend on the dequantized activations: equal up to the min-term
+    # convention (fp16 raw sum vs xd*sum(q8)), which the reference test bounds at rtol 2e-2
+    xd, _, qs = O.ds4_fields(ds4)
+    xdeq = (xd[..., None] * qs.astype(np.float32)).reshape(rows, k)
+    ref = O.gguf_quant_gemv(xdeq, w, O.GGML_Q4_K)
+    np.testing.assert_allclose(got, ref, rtol=2e-2, atol=1e-2 * (np.abs(ref).max() + 1))
+    assert O.cosine(got, ref) >= 0.9999
+
+
+def test_q4_k_mmq_closed_form_weights(dev):
+    rows, k, n = 40, 512, 96
+    xb = _bf16_rows(3, rows, k, scale=0.125)
+    ds4 = O.pack_q8_1_ds4(xb)
+    w = O.closed_form_q4_k(n, k)
+    got = _run_q4(dev, M.gguf_q4_k_q8_1_mmq32_vdr_dense_bf16_f32_out, ds4, w, rows, k, n)
+    want = O.mmq_q4_k_ds4(ds4, w)
+    assert O.max_rel_err(got, want) <= 1e-3 and O.cosine(got, want) >= 0.99999
+
+
+def test_q4_k_mmq_siblings_bf16_and_determinism(dev):
+    rows, k, n = 70, 1024, 96
+    xb = _bf16_rows(11, rows, k)
+    ds4 = O.pack_q8_1_ds4(xb)
+    w = O.random_weight(O.GGML_Q4_K, n, k, seed=5)
+    vdr = _run_q4(dev, M.gguf_q4_k_q8_1_mmq32_vdr_dense_bf16_f32_out, ds4, w, rows, k, n)
+    ctl = _run_q4(dev, M.gguf_q4_k_q8_1_mmq32_ctl_dense_bf16_f32_out, ds4, w, rows, k, n)
+    again = _run_q4(dev, M.gguf_q4_k_q8_1_mmq32_vdr_dense_bf16_f32_out, ds4, w, rows, k, n)
+    assert np.array_equal(vdr.view(np.uint32), ctl.view(np.uint32))
+    assert np.array_equal(vdr.view(np.uint32), again.view(np.uint32))
+    b16 = _run_q4(dev, M.gguf_q4_k_q8_1_mmq32_vdr_dense_bf16_bf16_out, ds4, w, rows, k, n, out_dtype=np.uint16)
+    assert np.array_equal(b16, O.f32_to_bf16_bits(vdr))
+
+
+def test_mmq_wrapper_rejects_bad_shapes(dev):
+    f = M.gguf_q4_k_q8_1_mmq32_vdr_dense_bf16_f32_out
+    with pytest.raises(ValueError, match="divisible"):
+        f(1, 1, 1, 4, 300, 32)
+    with pytest.raises(ValueError, match="divisible by 32"):
+        f(1, 1, 1, 4, 256, 40)
+    with pytest.raises(ValueError, match="rows"):
+        f(1, 1, 1, 0, 256, 32)
