@@ -44,8 +44,8 @@ typedef float v16f __attribute__((ext_vector_type(16)));
 typedef _Float16 v4h __attribute__((ext_vector_type(4)));
 
 constexpr int BM = 128, BN = 128, THREADS = 256;
-constexpr int W_STRIDE_Q4 = 144;            // raw block per row; 9 x 16 B is conflict free for b128 reads
-constexpr int A_STRIDE_DS4 = 304;           // 2 x 144 B padded to an odd number of 16-byte units
+constexpr int A_STRIDE = DS4_BYTES;         // 144 B = 9 x 16 B: conflict free for b128 reads
+constexpr int W_STRIDE = 80;                // 64 quant bytes per K step, padded to 5 x 16 B
 constexpr uint32_t MAGIC_BITS = 0x4B400000u;   // float 12582912 = 1.5 * 2^23
 constexpr float MAGIC = 12582912.0f;
 
@@ -57,15 +57,17 @@ struct MmqArgs {
   int M, K, N;
 };
 
+// One K step is 128 values: one DS4 activation block per row and half of a
+// Q4_K block (two nibble pairs = four 32-wide sub-blocks) per column.
 struct Q4Smem {
-  uint8_t wq[BN * W_STRIDE_Q4];
-  uint8_t xa[BM * A_STRIDE_DS4];
-  float sw[8][BN];       // d*sc per sub-block, column
-  float cw[8][BN];       // -MAGIC * sw
-  float xd[8][BM];       // activation scale per sub-block, row
+  uint8_t xa[BM * A_STRIDE];   // DS4 blocks of the step, as stored
+  uint8_t wq[BN * W_STRIDE];   // 64 nibble bytes per column
+  float sw[8][BN];             // d*sc per sub-block of the current Q4_K block, by column
+  float cw[8][BN];             // -MAGIC * sw
+  float xd[4][BM];             // activation scale per sub-block of the step, by row
   float dmin[BN];
-  _Float16 mnh[BN][8];   // 6-bit mins as fp16
-  _Float16 xsh[BM][8];   // activation sums (already fp16 in the DS4 block)
+  _Float16 mnh[BN][8];         // 6-bit mins as fp16
+  _Float16 xsh[BM][8];         // activation sums of the Q4_K block (fp16 in the DS4 block already)
 };
 
 __device__ __forceinline__ void store_tile(const MmqArgs& a, const float (&acc)[16], int m_base, int n_col) {
@@ -78,46 +80,56 @@ __device__ __forceinline__ void store_tile(const MmqArgs& a, const float (&acc)[
   }
 }
 
-__global__ void __launch_bounds__(THREADS, 2) mmq_q4_k_ds4_kernel(MmqArgs a) {
-  extern __shared__ __align__(16) uint8_t smem_raw[];
-  Q4Smem& s = *reinterpret_cast<Q4Smem*>(smem_raw);
-  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-  const int wm = wave & 1, wn = wave >> 1;
-  const int lc = lane & 31, g = lane >> 5;
-  const int m0 = blockIdx.x * BM, n0 = blockIdx.y * BN;
-  const int nb = a.K / QK_K;
-  const int64_t w_row_bytes = static_cast<int64_t>(nb) * Q4_K_BYTES;
-  const int64_t x_row_bytes = static_cast<int64_t>(a.K / 128) * DS4_BYTES;
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
 
-  float acc[2][2][16];   // [n tile][m tile][v]
-#pragma unroll
-  for (int i = 0; i < 2; ++i)
-#pragma unroll
-    for (int j = 0; j < 2; ++j)
-#pragma unroll
-      for (int v = 0; v < 16; ++v) acc[i][j][v] = 0.0f;
+// Registers of one K step in flight between global memory and LDS.
+struct Q4StepRegs {
+  u32x4 pa[5];   // activation tile chunks (128 rows x 9 chunks = 1152, 4.5 per thread)
+  u32x4 pw[2];   // weight nibble chunks (128 columns x 4 chunks = 512)
+  u32x4 ph;      // threads 0..127: Q4_K block header of column tid; 128..255: DS4 header of row tid-128
+};
 
-  for (int kb = 0; kb < nb; ++kb) {
-    // ---- stage raw tiles --------------------------------------------------
-    for (int c = tid; c < BN * 9; c += THREADS) {
-      const int row = c / 9, part = c - row * 9;
-      const int n = min(n0 + row, a.N - 1);
-      const uint4 v = *reinterpret_cast<const uint4*>(a.w + n * w_row_bytes + static_cast<int64_t>(kb) * Q4_K_BYTES + part * 16);
-      *reinterpret_cast<uint4*>(s.wq + row * W_STRIDE_Q4 + part * 16) = v;
-    }
-    for (int c = tid; c < BM * 18; c += THREADS) {
-      const int row = c / 18, part = c - row * 18;
-      const int m = min(m0 + row, a.M - 1);
-      const uint4 v = *reinterpret_cast<const uint4*>(a.xq + m * x_row_bytes + static_cast<int64_t>(kb) * 2 * DS4_BYTES + part * 16);
-      *reinterpret_cast<uint4*>(s.xa + row * A_STRIDE_DS4 + part * 16) = v;
-    }
-    // ---- decode scale tables (from global again: no dependency on the tiles) ----
-    if (tid < BN) {
-      const int n = min(n0 + tid, a.N - 1);
-      const uint4 h = *reinterpret_cast<const uint4*>(a.w + n * w_row_bytes + static_cast<int64_t>(kb) * Q4_K_BYTES);
-      const Q4KScales u = q4k_unpack_scales(h.y, h.z, h.w);
-      const float d = f16_bits_to_float(h.x & 0xFFFFu);
-      s.dmin[tid] = f16_bits_to_float(h.x >> 16);
+__device__ __forceinline__ void q4_step_load(const MmqArgs& a, int step, int m0, int n0, int64_t w_row_bytes,
+                                             int64_t x_row_bytes, int tid, Q4StepRegs& r) {
+  const int kb = step >> 1, h = step & 1;
+#pragma unroll
+  for (int i = 0; i < 5; ++i) {
+    const int c = min(tid + i * THREADS, BM * 9 - 1);
+    const int row = c / 9, part = c - row * 9;
+    const int m = min(m0 + row, a.M - 1);
+    r.pa[i] = *reinterpret_cast<const u32x4*>(a.xq + m * x_row_bytes + static_cast<int64_t>(step) * DS4_BYTES + part * 16);
+  }
+#pragma unroll
+  for (int i = 0; i < 2; ++i) {
+    const int c = tid + i * THREADS;
+    const int row = c >> 2, part = c & 3;
+    const int n = min(n0 + row, a.N - 1);
+    r.pw[i] = *reinterpret_cast<const u32x4*>(a.w + n * w_row_bytes + static_cast<int64_t>(kb) * Q4_K_BYTES + 16 + h * 64 +
+                                              part * 16);
+  }
+  const uint8_t* hp = tid < BN
+                          ? a.w + min(n0 + tid, a.N - 1) * w_row_bytes + static_cast<int64_t>(kb) * Q4_K_BYTES
+                          : a.xq + min(m0 + tid - BN, a.M - 1) * x_row_bytes + static_cast<int64_t>(step) * DS4_BYTES;
+  r.ph = *reinterpret_cast<const u32x4*>(hp);
+}
+
+__device__ __forceinline__ void q4_step_store(Q4Smem& s, int step, int tid, const Q4StepRegs& r) {
+  const int h = step & 1;
+#pragma unroll
+  for (int i = 0; i < 5; ++i) {
+    const int c = tid + i * THREADS;           // 144-byte rows are contiguous in LDS: offset c*16
+    if (c < BM * 9) *reinterpret_cast<u32x4*>(s.xa + c * 16) = r.pa[i];
+  }
+#pragma unroll
+  for (int i = 0; i < 2; ++i) {
+    const int c = tid + i * THREADS;
+    *reinterpret_cast<u32x4*>(s.wq + (c >> 2) * W_STRIDE + (c & 3) * 16) = r.pw[i];
+  }
+  if (tid < BN) {
+    if (h == 0) {
+      const Q4KScales u = q4k_unpack_scales(r.ph.y, r.ph.z, r.ph.w);
+      const float d = f16_bits_to_float(r.ph.x & 0xFFFFu);
+      s.dmin[tid] = f16_bits_to_float(r.ph.x >> 16);
 #pragma unroll
       for (int j = 0; j < 8; ++j) {
         const uint32_t sc = ((j < 4 ? u.sc_lo : u.sc_hi) >> (8 * (j & 3))) & 0xFFu;
@@ -127,29 +139,57 @@ __global__ void __launch_bounds__(THREADS, 2) mmq_q4_k_ds4_kernel(MmqArgs a) {
         s.cw[j][tid] = -MAGIC * sw;
         s.mnh[tid][j] = static_cast<_Float16>(static_cast<float>(mn));
       }
-    } else {
-      const int r = tid - BN;
-      const int m = min(m0 + r, a.M - 1);
-      const uint8_t* xb = a.xq + m * x_row_bytes + static_cast<int64_t>(kb) * 2 * DS4_BYTES;
-      const uint4 h0 = *reinterpret_cast<const uint4*>(xb);
-      const uint4 h1 = *reinterpret_cast<const uint4*>(xb + DS4_BYTES);
-      const uint32_t hh[8] = {h0.x, h0.y, h0.z, h0.w, h1.x, h1.y, h1.z, h1.w};
-#pragma unroll
-      for (int j = 0; j < 8; ++j) {
-        s.xd[j][r] = f16_bits_to_float(hh[j] & 0xFFFFu);
-        s.xsh[r][j] = __builtin_bit_cast(_Float16, static_cast<uint16_t>(hh[j] >> 16));
-      }
     }
-    __syncthreads();
-
-    // ---- int8 MFMA over the 8 sub-blocks ------------------------------------
+  } else {
+    const int row = tid - BN;
 #pragma unroll
-    for (int sp = 0; sp < 4; ++sp) {
+    for (int j = 0; j < 4; ++j) {
+      s.xd[j][row] = f16_bits_to_float(r.ph[j] & 0xFFFFu);
+      s.xsh[row][4 * h + j] = __builtin_bit_cast(_Float16, static_cast<uint16_t>(r.ph[j] >> 16));
+    }
+  }
+}
+
+template <bool PREFETCH>
+__global__ void __launch_bounds__(THREADS, (PREFETCH ? 2 : 3)) mmq_q4_k_ds4_kernel(MmqArgs a) {
+  extern __shared__ __align__(16) uint8_t smem_raw[];
+  Q4Smem& s = *reinterpret_cast<Q4Smem*>(smem_raw);
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int wm = wave & 1, wn = wave >> 1;
+  const int lc = lane & 31, g = lane >> 5;
+  const int m0 = blockIdx.x * BM, n0 = blockIdx.y * BN;
+  const int steps = a.K / 128;
+  const int64_t w_row_bytes = static_cast<int64_t>(a.K / QK_K) * Q4_K_BYTES;
+  const int64_t x_row_bytes = static_cast<int64_t>(steps) * DS4_BYTES;
+
+  float acc[2][2][16];   // [n tile][m tile][v]
+#pragma unroll
+  for (int i = 0; i < 2; ++i)
+#pragma unroll
+    for (int j = 0; j < 2; ++j)
+#pragma unroll
+      for (int v = 0; v < 16; ++v) acc[i][j][v] = 0.0f;
+
+  Q4StepRegs regs;
+  if (PREFETCH) q4_step_load(a, 0, m0, n0, w_row_bytes, x_row_bytes, tid, regs);
+
+  for (int step = 0; step < steps; ++step) {
+    const int h = step & 1;
+    if (!PREFETCH) q4_step_load(a, step, m0, n0, w_row_bytes, x_row_bytes, tid, regs);
+    q4_step_store(s, step, tid, regs);
+    __syncthreads();
+    // The loads of the next step are issued before this step is computed, so
+    // their latency hides behind the MFMA/FMA work.
+    if (PREFETCH && step + 1 < steps) q4_step_load(a, step + 1, m0, n0, w_row_bytes, x_row_bytes, tid, regs);
+
+    // ---- int8 MFMA over the 4 sub-blocks of the step --------------------------
+#pragma unroll
+    for (int sp = 0; sp < 2; ++sp) {
       v4i wlo[2], whi[2];
 #pragma unroll
       for (int nt = 0; nt < 2; ++nt) {
         const int row = wn * 64 + nt * 32 + lc;
-        const uint4 qs = *reinterpret_cast<const uint4*>(s.wq + row * W_STRIDE_Q4 + 16 + sp * 32 + 16 * g);
+        const u32x4 qs = *reinterpret_cast<const u32x4*>(s.wq + row * W_STRIDE + sp * 32 + 16 * g);
         wlo[nt] = v4i{static_cast<int>(q4k_low(qs.x)), static_cast<int>(q4k_low(qs.y)),
                       static_cast<int>(q4k_low(qs.z)), static_cast<int>(q4k_low(qs.w))};
         whi[nt] = v4i{static_cast<int>(q4k_high(qs.x)), static_cast<int>(q4k_high(qs.y)),
@@ -157,16 +197,16 @@ __global__ void __launch_bounds__(THREADS, 2) mmq_q4_k_ds4_kernel(MmqArgs a) {
       }
 #pragma unroll
       for (int half = 0; half < 2; ++half) {
-        const int sb = 2 * sp + half;
+        const int sl = 2 * sp + half;      // sub-block within the step
+        const int sb = 4 * h + sl;         // sub-block within the Q4_K block
 #pragma unroll
         for (int mt = 0; mt < 2; ++mt) {
           const int arow = wm * 64 + mt * 32 + lc;
-          const v4i xop = *reinterpret_cast<const v4i*>(s.xa + arow * A_STRIDE_DS4 + (sb >> 2) * DS4_BYTES + 16 +
-                                                        (sb & 3) * 32 + 16 * g);
+          const v4i xop = *reinterpret_cast<const v4i*>(s.xa + arow * A_STRIDE + 16 + sl * 32 + 16 * g);
           float xdv[16];
 #pragma unroll
           for (int j = 0; j < 4; ++j) {
-            const float4 t = *reinterpret_cast<const float4*>(&s.xd[sb][wm * 64 + mt * 32 + 8 * j + 4 * g]);
+            const float4 t = *reinterpret_cast<const float4*>(&s.xd[sl][wm * 64 + mt * 32 + 8 * j + 4 * g]);
             xdv[4 * j] = t.x; xdv[4 * j + 1] = t.y; xdv[4 * j + 2] = t.z; xdv[4 * j + 3] = t.w;
           }
 #pragma unroll
@@ -187,25 +227,27 @@ __global__ void __launch_bounds__(THREADS, 2) mmq_q4_k_ds4_kernel(MmqArgs a) {
       }
     }
 
-    // ---- min term: dmin[n] * sum_j mn_j[n] * xsum_j[m] on the fp16 MFMA -------
+    // ---- min term, once per Q4_K block: dmin[n] * sum_j mn_j[n] * xsum_j[m] on the fp16 MFMA
+    if (h == 1) {
 #pragma unroll
-    for (int mt = 0; mt < 2; ++mt) {
-      const int arow = wm * 64 + mt * 32 + lc;
-      const v4h xs = *reinterpret_cast<const v4h*>(&s.xsh[arow][4 * g]);
+      for (int mt = 0; mt < 2; ++mt) {
+        const int arow = wm * 64 + mt * 32 + lc;
+        const v4h xs = *reinterpret_cast<const v4h*>(&s.xsh[arow][4 * g]);
 #pragma unroll
-      for (int nt = 0; nt < 2; ++nt) {
-        const int col = wn * 64 + nt * 32 + lc;
-        const v4h mn = *reinterpret_cast<const v4h*>(&s.mnh[col][4 * g]);
-        v16f z;
+        for (int nt = 0; nt < 2; ++nt) {
+          const int col = wn * 64 + nt * 32 + lc;
+          const v4h mn = *reinterpret_cast<const v4h*>(&s.mnh[col][4 * g]);
+          v16f z;
 #pragma unroll
-        for (int v = 0; v < 16; ++v) z[v] = 0.0f;
-        const v16f t = __builtin_amdgcn_mfma_f32_32x32x8f16(xs, mn, z, 0, 0, 0);
-        const float nd = -s.dmin[col];
+          for (int v = 0; v < 16; ++v) z[v] = 0.0f;
+          const v16f t = __builtin_amdgcn_mfma_f32_32x32x8f16(xs, mn, z, 0, 0, 0);
+          const float nd = -s.dmin[col];
 #pragma unroll
-        for (int v = 0; v < 16; ++v) acc[nt][mt][v] = __builtin_fmaf(nd, t[v], acc[nt][mt][v]);
+          for (int v = 0; v < 16; ++v) acc[nt][mt][v] = __builtin_fmaf(nd, t[v], acc[nt][mt][v]);
+        }
       }
     }
-    __syncthreads();   // the next block overwrites the tiles
+    __syncthreads();   // the next step overwrites the tiles
   }
 
 #pragma unroll
@@ -216,30 +258,34 @@ __global__ void __launch_bounds__(THREADS, 2) mmq_q4_k_ds4_kernel(MmqArgs a) {
 }
 
 int launch_q4(const void* xq, const uint8_t* w, void* out, int out_kind, int64_t M, int64_t K, int64_t N,
-              hipStream_t stream) {
+              int variant, hipStream_t stream) {
   if (!xq || !w || !out || M <= 0 || M > (1 << 20) || K <= 0 || (K % QK_K) != 0 || N <= 0 || (N % 32) != 0 ||
-      N > (1 << 24)) {
+      N > (1 << 24) || out_kind < KIND_F32 || out_kind > KIND_F16) {
     return static_cast<int>(hipErrorInvalidValue);
   }
   MmqArgs a{static_cast<const uint8_t*>(xq), w, out, out_kind, static_cast<int>(M), static_cast<int>(K),
             static_cast<int>(N)};
   const dim3 grid(static_cast<unsigned>((M + BM - 1) / BM), static_cast<unsigned>((N + BN - 1) / BN));
-  static bool attr_set = false;
-  if (!attr_set) {
-    (void)hipFuncSetAttribute(reinterpret_cast<const void*>(mmq_q4_k_ds4_kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
-                              static_cast<int>(sizeof(Q4Smem)));
-    attr_set = true;
+  if (variant == 1) {
+    hipLaunchKernelGGL(mmq_q4_k_ds4_kernel<false>, grid, dim3(THREADS), sizeof(Q4Smem), stream, a);
+  } else {
+    hipLaunchKernelGGL(mmq_q4_k_ds4_kernel<true>, grid, dim3(THREADS), sizeof(Q4Smem), stream, a);
   }
-  hipLaunchKernelGGL(mmq_q4_k_ds4_kernel, grid, dim3(THREADS), sizeof(Q4Smem), stream, a);
   return static_cast<int>(hipGetLastError());
 }
 
 }  // namespace
 
+extern "C" int hipengine_gfx950_gguf_q4_k_mmq_tuned(const void* xq, const uint8_t* qweight, void* out, int out_kind,
+                                                   int64_t rows, int64_t in_features, int64_t out_features,
+                                                   int variant, hipStream_t stream) {
+  return launch_q4(xq, qweight, out, out_kind, rows, in_features, out_features, variant, stream);
+}
+
 #define DEFINE_MMQ_Q4(SYMBOL, OKIND)                                                                        \
   extern "C" int SYMBOL(const void* xq, const uint8_t* qweight, void* out, int64_t rows, int64_t in_features, \
                         int64_t out_features, hipStream_t stream) {                                         \
-    return launch_q4(xq, qweight, out, OKIND, rows, in_features, out_features, stream);                     \
+    return launch_q4(xq, qweight, out, OKIND, rows, in_features, out_features, 0, stream);                     \
   }
 
 DEFINE_MMQ_Q4(hipengine_gguf_q4_k_q8_1_mmq32_vdr_dense_bf16_f32_out, KIND_F32)

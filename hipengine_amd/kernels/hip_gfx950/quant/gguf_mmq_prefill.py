@@ -48,6 +48,18 @@ gguf_q4_k_q8_1_mmq32_ctl_dense_bf16_f32_out = _make(
 gguf_q4_k_q8_1_mmq32_ctl_dense_bf16_bf16_out = _make(
     "gguf_q4_k_q8_1_mmq32_ctl_dense_bf16_bf16_out", "hipengine_gguf_q4_k_q8_1_mmq32_ctl_dense_bf16_bf16_out", 32)
 
+
+def gguf_q4_k_q8_1_mmq_tuned(xq_ptr: int, qweight_ptr: int, out_ptr: int, rows: int, hidden: int, out_features: int, *,
+                             out_kind: int = 0, variant: int = 0, stream: int = 0,
+                             library: ctypes.CDLL | None = None, runtime: HipRuntime | None = None) -> None:
+    """Q4_K x DS4 MMQ with an explicit kernel form (``hipengine_gfx950_gguf_q4_k_mmq_tuned``)."""
+    _validate(rows, hidden, out_features, 32)
+    validate_pointers(xq_ptr=xq_ptr, qweight_ptr=qweight_ptr, out_ptr=out_ptr)
+    fn = entry("hipengine_gfx950_gguf_q4_k_mmq_tuned", [VOID, VOID, VOID, ctypes.c_int, I64, I64, I64, ctypes.c_int, VOID],
+               library)
+    check_launch(fn(xq_ptr, qweight_ptr, out_ptr, out_kind, rows, hidden, out_features, variant, stream), runtime)
+
+
 _Q4 = (
     ("mmq32_vdr_dense_bf16_f32_out", gguf_q4_k_q8_1_mmq32_vdr_dense_bf16_f32_out),
     ("mmq32_vdr_dense_bf16_bf16_out", gguf_q4_k_q8_1_mmq32_vdr_dense_bf16_bf16_out),

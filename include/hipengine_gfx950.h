@@ -181,6 +181,14 @@ int hipengine_gguf_q4_k_q8_1_mmq32_ctl_dense_bf16_bf16_out(const void* xq, const
                                                            int64_t rows, int64_t in_features, int64_t out_features,
                                                            hipengine_stream_t stream);
 
+/* The same Q4_K x DS4 GEMM with the kernel form chosen by the caller (benchmarks
+ * and tuning; no counterpart in hipEngine).  out_kind: 0 float32, 1 bf16, 2 fp16.
+ * variant 0: the next K step is prefetched into registers (what the named entry
+ * points run); variant 1: no prefetch, one more workgroup per CU. */
+int hipengine_gfx950_gguf_q4_k_mmq_tuned(const void* xq, const uint8_t* qweight, void* out, int out_kind,
+                                         int64_t rows, int64_t in_features, int64_t out_features, int variant,
+                                         hipengine_stream_t stream);
+
 /* ------------------------------------------------------------------------
  * Verification exports: the integer unpack and the int32 sub-block dots the
  * production kernels compute, written out so that they can be compared bit for
