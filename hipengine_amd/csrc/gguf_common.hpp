@@ -197,4 +197,26 @@ __device__ __forceinline__ uint32_t q6k_center(uint32_t u6x4) {
   return ((u6x4 | 0x80808080u) - 0x20202020u) ^ 0x80808080u;
 }
 
+// Loads from GGUF blocks, which are only 2-byte aligned (Q6_K 210 B, Q8_0 34 B).
+__device__ __forceinline__ uint4 load16(const uint8_t* p) {
+  uint4 v;
+  __builtin_memcpy(&v, __builtin_assume_aligned(p, 2), 16);
+  return v;
+}
+__device__ __forceinline__ uint2 load8(const uint8_t* p) {
+  uint2 v;
+  __builtin_memcpy(&v, __builtin_assume_aligned(p, 2), 8);
+  return v;
+}
+__device__ __forceinline__ uint32_t load4(const uint8_t* p) {
+  uint32_t v;
+  __builtin_memcpy(&v, __builtin_assume_aligned(p, 2), 4);
+  return v;
+}
+__device__ __forceinline__ uint32_t load2(const uint8_t* p) {
+  uint16_t v;
+  __builtin_memcpy(&v, __builtin_assume_aligned(p, 2), 2);
+  return v;
+}
+
 }  // namespace hipengine_gfx950

@@ -69,27 +69,6 @@ struct WeightRegs {
   uint32_t v[N];
 };
 
-__device__ __forceinline__ uint4 load16(const uint8_t* p) {
-  uint4 v;
-  __builtin_memcpy(&v, __builtin_assume_aligned(p, 2), 16);
-  return v;
-}
-__device__ __forceinline__ uint2 load8(const uint8_t* p) {
-  uint2 v;
-  __builtin_memcpy(&v, __builtin_assume_aligned(p, 2), 8);
-  return v;
-}
-__device__ __forceinline__ uint32_t load4(const uint8_t* p) {
-  uint32_t v;
-  __builtin_memcpy(&v, __builtin_assume_aligned(p, 2), 4);
-  return v;
-}
-__device__ __forceinline__ uint32_t load2(const uint8_t* p) {
-  uint16_t v;
-  __builtin_memcpy(&v, __builtin_assume_aligned(p, 2), 2);
-  return v;
-}
-
 // Lane q (0..3) of a quad loads its share of the 256-value block at `blk`.
 template <int QT>
 __device__ __forceinline__ void gemv_load_block(const uint8_t* blk, int q, WeightRegs<GemvTraits<QT>::REGS>& r) {

@@ -274,6 +274,184 @@ int launch_q4(const void* xq, const uint8_t* w, void* out, int out_kind, int64_t
   return static_cast<int>(hipGetLastError());
 }
 
+// --------------------------------------------------------------------------
+// Q6_K x D4S4.  One K step is 128 values: one D4S4 block per row and one half of
+// a Q6_K block per column (64 ql bytes, 32 qh bytes, 8 int8 scales).  The 6-bit
+// values are rebuilt and centred (u - 32) once per workgroup while the tile is
+// written to LDS, so the waves read plain int8 MFMA operands on both sides.
+// --------------------------------------------------------------------------
+constexpr int A6_STRIDE = 176;   // 160-byte D4S4 block padded to 11 x 16 B
+constexpr int W6_STRIDE = 144;   // 128 centred int8 values padded to 9 x 16 B
+
+struct Q6Smem {
+  uint8_t xa[BM * A6_STRIDE];
+  uint8_t w8[BN * W6_STRIDE];
+  float sw[8][BN];     // d * scale of the 8 16-value groups of the step, by column
+  float cw[8][BN];     // -MAGIC * sw (exact: d has 11 significant bits, the scale 8)
+  float xd[4][BM];     // activation scale per 32 values, by row
+};
+
+struct Q6StepRegs {
+  u32x4 pa[5];         // 128 rows x 10 chunks = 1280 = 5 per thread
+  u32x4 qla, qlb, qh;  // 16 bytes each of the column tid/2, byte offset 16*(tid&1)
+  uint2 sc;            // threads 0..127: the 8 scales of column tid
+  uint32_t d;          //                 and its fp16 d
+  u32x4 xd;            // threads 128..255: the four float scales of row tid-128
+};
+
+__device__ __forceinline__ void q6_step_load(const MmqArgs& a, int step, int m0, int n0, int64_t w_row_bytes,
+                                             int64_t x_row_bytes, int tid, Q6StepRegs& r) {
+  const int kb = step >> 1, hh = step & 1;
+#pragma unroll
+  for (int i = 0; i < 5; ++i) {
+    const int c = tid + i * THREADS;
+    const int row = c / 10, part = c - row * 10;
+    const int m = min(m0 + row, a.M - 1);
+    r.pa[i] = *reinterpret_cast<const u32x4*>(a.xq + m * x_row_bytes + static_cast<int64_t>(step) * D4S4_BYTES + part * 16);
+  }
+  {
+    const int n = min(n0 + (tid >> 1), a.N - 1);
+    const uint8_t* blk = a.w + n * w_row_bytes + static_cast<int64_t>(kb) * Q6_K_BYTES;
+    const int o = (tid & 1) * 16;
+    const uint4 x = load16(blk + 64 * hh + o), y = load16(blk + 64 * hh + 32 + o), z = load16(blk + 128 + 32 * hh + o);
+    r.qla = u32x4{x.x, x.y, x.z, x.w};
+    r.qlb = u32x4{y.x, y.y, y.z, y.w};
+    r.qh = u32x4{z.x, z.y, z.z, z.w};
+  }
+  if (tid < BN) {
+    const uint8_t* blk = a.w + min(n0 + tid, a.N - 1) * w_row_bytes + static_cast<int64_t>(kb) * Q6_K_BYTES;
+    r.sc = load8(blk + 192 + 8 * hh);
+    r.d = load2(blk + 208);
+  } else {
+    r.xd = *reinterpret_cast<const u32x4*>(a.xq + min(m0 + tid - BN, a.M - 1) * x_row_bytes +
+                                           static_cast<int64_t>(step) * D4S4_BYTES);
+  }
+}
+
+__device__ __forceinline__ void q6_step_store(Q6Smem& s, int tid, const Q6StepRegs& r) {
+#pragma unroll
+  for (int i = 0; i < 5; ++i) {
+    const int c = tid + i * THREADS;
+    const int row = c / 10, part = c - row * 10;
+    *reinterpret_cast<u32x4*>(s.xa + row * A6_STRIDE + part * 16) = r.pa[i];
+  }
+  {
+    u32x4 q0, q1, q2, q3;   // the four 32-value quarters of the half, bytes o..o+15 of each
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const Q6KQuad u = q6k_unpack(r.qla[i], r.qlb[i], r.qh[i]);
+      q0[i] = q6k_center(u.g0); q1[i] = q6k_center(u.g1); q2[i] = q6k_center(u.g2); q3[i] = q6k_center(u.g3);
+    }
+    uint8_t* dst = s.w8 + (tid >> 1) * W6_STRIDE + (tid & 1) * 16;
+    *reinterpret_cast<u32x4*>(dst) = q0;
+    *reinterpret_cast<u32x4*>(dst + 32) = q1;
+    *reinterpret_cast<u32x4*>(dst + 64) = q2;
+    *reinterpret_cast<u32x4*>(dst + 96) = q3;
+  }
+  if (tid < BN) {
+    const float d = f16_bits_to_float(r.d & 0xFFFFu);
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+      const uint32_t word = j < 4 ? r.sc.x : r.sc.y;
+      const int sc = static_cast<int>(static_cast<int8_t>((word >> (8 * (j & 3))) & 0xFFu));
+      const float sw = d * static_cast<float>(sc);
+      s.sw[j][tid] = sw;
+      s.cw[j][tid] = -MAGIC * sw;
+    }
+  } else {
+#pragma unroll
+    for (int j = 0; j < 4; ++j) s.xd[j][tid - BN] = bits_to_float(r.xd[j]);
+  }
+}
+
+__global__ void __launch_bounds__(THREADS, 2) mmq_q6_k_d4s4_kernel(MmqArgs a) {
+  extern __shared__ __align__(16) uint8_t smem_raw[];
+  Q6Smem& s = *reinterpret_cast<Q6Smem*>(smem_raw);
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int wm = wave & 1, wn = wave >> 1;
+  const int lc = lane & 31, g = lane >> 5;
+  const int m0 = blockIdx.x * BM, n0 = blockIdx.y * BN;
+  const int steps = a.K / 128;
+  const int64_t w_row_bytes = static_cast<int64_t>(a.K / QK_K) * Q6_K_BYTES;
+  const int64_t x_row_bytes = static_cast<int64_t>(steps) * D4S4_BYTES;
+
+  float acc[2][2][16];
+#pragma unroll
+  for (int i = 0; i < 2; ++i)
+#pragma unroll
+    for (int j = 0; j < 2; ++j)
+#pragma unroll
+      for (int v = 0; v < 16; ++v) acc[i][j][v] = 0.0f;
+
+  Q6StepRegs regs;
+  q6_step_load(a, 0, m0, n0, w_row_bytes, x_row_bytes, tid, regs);
+
+  for (int step = 0; step < steps; ++step) {
+    q6_step_store(s, tid, regs);
+    __syncthreads();
+    if (step + 1 < steps) q6_step_load(a, step + 1, m0, n0, w_row_bytes, x_row_bytes, tid, regs);
+
+#pragma unroll
+    for (int sl = 0; sl < 4; ++sl) {            // 32 activation values share one scale
+      long wop[2][2];                            // [n tile][16-value group]
+#pragma unroll
+      for (int nt = 0; nt < 2; ++nt)
+#pragma unroll
+        for (int t = 0; t < 2; ++t)
+          wop[nt][t] = *reinterpret_cast<const long*>(s.w8 + (wn * 64 + nt * 32 + lc) * W6_STRIDE + 32 * sl + 16 * t + 8 * g);
+#pragma unroll
+      for (int mt = 0; mt < 2; ++mt) {
+        const uint8_t* ap = s.xa + (wm * 64 + mt * 32 + lc) * A6_STRIDE + 32 + 32 * sl + 8 * g;
+        const long xop0 = *reinterpret_cast<const long*>(ap);
+        const long xop1 = *reinterpret_cast<const long*>(ap + 16);
+        float xdv[16];
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+          const float4 t = *reinterpret_cast<const float4*>(&s.xd[sl][wm * 64 + mt * 32 + 8 * j + 4 * g]);
+          xdv[4 * j] = t.x; xdv[4 * j + 1] = t.y; xdv[4 * j + 2] = t.z; xdv[4 * j + 3] = t.w;
+        }
+#pragma unroll
+        for (int nt = 0; nt < 2; ++nt) {
+          const int col = wn * 64 + nt * 32 + lc;
+          const float s0 = s.sw[2 * sl][col], c0 = s.cw[2 * sl][col];
+          const float s1 = s.sw[2 * sl + 1][col], c1 = s.cw[2 * sl + 1][col];
+          v16i ci;
+#pragma unroll
+          for (int v = 0; v < 16; ++v) ci[v] = static_cast<int>(MAGIC_BITS);
+          const v16i d0 = __builtin_amdgcn_mfma_i32_32x32x16_i8(xop0, wop[nt][0], ci, 0, 0, 0);
+          const v16i d1 = __builtin_amdgcn_mfma_i32_32x32x16_i8(xop1, wop[nt][1], ci, 0, 0, 0);
+#pragma unroll
+          for (int v = 0; v < 16; ++v) {
+            const float t0 = __builtin_fmaf(bits_to_float(static_cast<uint32_t>(d0[v])), s0, c0);   // s0 * dot0, rounded once
+            const float t1 = __builtin_fmaf(bits_to_float(static_cast<uint32_t>(d1[v])), s1, c1);
+            acc[nt][mt][v] = __builtin_fmaf(xdv[v], t0 + t1, acc[nt][mt][v]);
+          }
+        }
+      }
+    }
+    __syncthreads();
+  }
+
+#pragma unroll
+  for (int nt = 0; nt < 2; ++nt)
+#pragma unroll
+    for (int mt = 0; mt < 2; ++mt)
+      store_tile(a, acc[nt][mt], m0 + wm * 64 + mt * 32 + 4 * g, n0 + wn * 64 + nt * 32 + lc);
+}
+
+int launch_q6(const void* xq, const uint8_t* w, void* out, int out_kind, int64_t M, int64_t K, int64_t N,
+              hipStream_t stream) {
+  if (!xq || !w || !out || M <= 0 || M > (1 << 20) || K <= 0 || (K % QK_K) != 0 || N <= 0 || N > (1 << 24) ||
+      out_kind < KIND_F32 || out_kind > KIND_F16) {
+    return static_cast<int>(hipErrorInvalidValue);
+  }
+  MmqArgs a{static_cast<const uint8_t*>(xq), w, out, out_kind, static_cast<int>(M), static_cast<int>(K),
+            static_cast<int>(N)};
+  const dim3 grid(static_cast<unsigned>((M + BM - 1) / BM), static_cast<unsigned>((N + BN - 1) / BN));
+  hipLaunchKernelGGL(mmq_q6_k_d4s4_kernel, grid, dim3(THREADS), sizeof(Q6Smem), stream, a);
+  return static_cast<int>(hipGetLastError());
+}
+
 }  // namespace
 
 extern "C" int hipengine_gfx950_gguf_q4_k_mmq_tuned(const void* xq, const uint8_t* qweight, void* out, int out_kind,
@@ -292,3 +470,12 @@ DEFINE_MMQ_Q4(hipengine_gguf_q4_k_q8_1_mmq32_vdr_dense_bf16_f32_out, KIND_F32)
 DEFINE_MMQ_Q4(hipengine_gguf_q4_k_q8_1_mmq32_vdr_dense_bf16_bf16_out, KIND_BF16)
 DEFINE_MMQ_Q4(hipengine_gguf_q4_k_q8_1_mmq32_ctl_dense_bf16_f32_out, KIND_F32)
 DEFINE_MMQ_Q4(hipengine_gguf_q4_k_q8_1_mmq32_ctl_dense_bf16_bf16_out, KIND_BF16)
+
+#define DEFINE_MMQ_Q6(SYMBOL, OKIND)                                                                        \
+  extern "C" int SYMBOL(const void* xq, const uint8_t* qweight, void* out, int64_t rows, int64_t in_features, \
+                        int64_t out_features, hipStream_t stream) {                                         \
+    return launch_q6(xq, qweight, out, OKIND, rows, in_features, out_features, stream);                     \
+  }
+
+DEFINE_MMQ_Q6(hipengine_gguf_q6_k_mmq32_q8_1_d4s4_f32_bf16_f32_out, KIND_F32)
+DEFINE_MMQ_Q6(hipengine_gguf_q6_k_mmq32_q8_1_d4s4_f32_bf16_bf16_out, KIND_BF16)

@@ -69,7 +69,7 @@ def register_kernels(backend: str = "hip_gfx950", *, replace: bool = False) -> N
     for quant, variant, fn in (
         ("q8_1", "f32", gguf_q4_k_quantize_f32_q8_1),
         ("q8_1", "bf16", gguf_q4_k_quantize_bf16_q8_1),
-        ("q8_1_ds4", "bf16_kmajor", gguf_q8_1_mmq_ds4_pack_bf16),
-        ("q8_1_d4s4_f32", "bf16_kmajor", gguf_q8_1_d4s4_f32_quantize_bf16),
+        ("q8_1_ds4", "bf16", gguf_q8_1_mmq_ds4_pack_bf16),
+        ("q8_1_d4s4_f32", "bf16", gguf_q8_1_d4s4_f32_quantize_bf16),
     ):
         register(KernelKey(backend, "activation_quant", quant, variant), fn, replace=replace)

@@ -181,6 +181,19 @@ int hipengine_gguf_q4_k_q8_1_mmq32_ctl_dense_bf16_bf16_out(const void* xq, const
                                                            int64_t rows, int64_t in_features, int64_t out_features,
                                                            hipengine_stream_t stream);
 
+/* Raw Q6_K weights x D4S4 activations ([rows, in_features/128] 160-byte blocks
+ * {float d4[4]; float s4[4]; int8 qs[128]}): sum over 32-value groups of
+ * xd_g * (s0*dot0 + s1*dot1), s = d*scale_i8 per 16 values, dots of the centred
+ * 6-bit values.  Any out_features >= 1.
+ * Replaces gguf_k_mmq_prefill.hip:2588 (HIPENGINE_GGUF_K_MMQ_EXPORTS(gguf_q6_k, 6);
+ * kernel :519-685), Python side gguf_k_mmq_prefill.py:349-397. */
+int hipengine_gguf_q6_k_mmq32_q8_1_d4s4_f32_bf16_f32_out(const void* xq, const uint8_t* qweight, void* out,
+                                                         int64_t rows, int64_t in_features, int64_t out_features,
+                                                         hipengine_stream_t stream);
+int hipengine_gguf_q6_k_mmq32_q8_1_d4s4_f32_bf16_bf16_out(const void* xq, const uint8_t* qweight, void* out,
+                                                          int64_t rows, int64_t in_features, int64_t out_features,
+                                                          hipengine_stream_t stream);
+
 /* The same Q4_K x DS4 GEMM with the kernel form chosen by the caller (benchmarks
  * and tuning; no counterpart in hipEngine).  out_kind: 0 float32, 1 bf16, 2 fp16.
  * variant 0: the next K step is prefetched into registers (what the named entry

@@ -99,6 +99,48 @@ def test_q4_k_mmq_siblings_bf16_and_determinism(dev):
     assert np.array_equal(b16, O.f32_to_bf16_bits(vdr))
 
 
+def test_q4_k_mmq_kernel_forms_agree(dev):
+    rows, k, n = 150, 1536, 160
+    xb = _bf16_rows(21, rows, k)
+    ds4 = O.pack_q8_1_ds4(xb)
+    w = O.random_weight(O.GGML_Q4_K, n, k, seed=9)
+    import functools
+    a = _run_q4(dev, functools.partial(M.gguf_q4_k_q8_1_mmq_tuned, variant=0), ds4, w, rows, k, n)
+    b = _run_q4(dev, functools.partial(M.gguf_q4_k_q8_1_mmq_tuned, variant=1), ds4, w, rows, k, n)
+    assert np.array_equal(a.view(np.uint32), b.view(np.uint32))
+    assert O.max_rel_err(a, O.mmq_q4_k_ds4(ds4, w)) <= 1e-3
+
+
+@pytest.mark.parametrize("rows,k,n", [(1, 256, 1), (7, 512, 33), (128, 1024, 128), (130, 768, 160), (300, 5120, 200)])
+def test_q6_k_mmq_matches_formula_and_cpu_reference(dev, rows, k, n):
+    xb = _bf16_rows(5 * rows + k + n, rows, k, scale=0.1, offset=0.002)
+    d4 = O.pack_q8_1_d4s4(xb)
+    w = O.random_weight(O.GGML_Q6_K, n, k, seed=k + n + 1)
+    got = _run_q4(dev, M.gguf_q6_k_mmq32_q8_1_d4s4_f32_bf16_f32_out, d4, w, rows, k, n)
+    want = O.mmq_q6_k_d4s4(d4, w)                     # float64 evaluation of the MMQ formula
+    assert O.max_rel_err(got, want) <= 1e-3 and O.cosine(got, want) >= 0.99999
+    assert O.max_rel_err(got, C.mmq_q6_k_d4s4(d4, w)) <= 1e-3
+    # the reference CPU backend (dequantize -> float32 matmul) on the dequantized activations
+    xd, _, qs = O.d4s4_fields(d4)
+    xdeq = (xd[..., None] * qs.astype(np.float32)).reshape(rows, k)
+    ref = O.gguf_quant_gemv(xdeq, w, O.GGML_Q6_K)
+    assert O.max_rel_err(got, ref) <= 1e-3 and O.cosine(got, ref) >= 0.99999
+
+
+def test_q6_k_mmq_closed_form_bf16_and_determinism(dev):
+    rows, k, n = 70, 512, 96
+    xb = _bf16_rows(13, rows, k, scale=0.125)
+    d4 = O.pack_q8_1_d4s4(xb)
+    w = O.closed_form_q6_k(n, k)
+    f32 = _run_q4(dev, M.gguf_q6_k_mmq32_q8_1_d4s4_f32_bf16_f32_out, d4, w, rows, k, n)
+    again = _run_q4(dev, M.gguf_q6_k_mmq32_q8_1_d4s4_f32_bf16_f32_out, d4, w, rows, k, n)
+    want = O.mmq_q6_k_d4s4(d4, w)
+    assert O.max_rel_err(f32, want) <= 1e-3 and O.cosine(f32, want) >= 0.99999
+    assert np.array_equal(f32.view(np.uint32), again.view(np.uint32))
+    b16 = _run_q4(dev, M.gguf_q6_k_mmq32_q8_1_d4s4_f32_bf16_bf16_out, d4, w, rows, k, n, out_dtype=np.uint16)
+    assert np.array_equal(b16, O.f32_to_bf16_bits(f32))
+
+
 def test_mmq_wrapper_rejects_bad_shapes(dev):
     f = M.gguf_q4_k_q8_1_mmq32_vdr_dense_bf16_f32_out
     with pytest.raises(ValueError, match="divisible"):

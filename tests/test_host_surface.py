@@ -94,7 +94,7 @@ def test_backend_registers_the_documented_keys(clean_registry):
         for v in ("q8_1_fused_gemv_f32_f32_out", "q8_1_fused_gemv_bf16_bf16_out", "q8_1_fused_prefill_bf16_f32_out"):
             assert KernelKey("hip_gfx950", "linear", q, v) in keys
     assert KernelKey("hip_gfx950", "linear", "gguf_q4_k", "q8_1_dp4a_vdr_bf16_f32_out") in keys
-    assert KernelKey("hip_gfx950", "activation_quant", "q8_1_ds4", "bf16_kmajor") in keys
+    assert KernelKey("hip_gfx950", "activation_quant", "q8_1_ds4", "bf16") in keys
     assert not any(k.backend == "cpu_reference" for k in keys)            # the package ships no CPU path
     assert hip_gfx950.GGUF_CONSUMER_LAYERS >= {"linear", "moe_linear"}
     fn = R.resolve(backend="hip_gfx950", layer="linear", quant="gguf_q4_k", variant="q8_1_fused_gemv_f32_f32_out")
