@@ -331,8 +331,13 @@ inline size_t gemv_lds_bytes(int qt, int B, int R, int CB, int ks, int nrg) {
 
 // `w_row0` / `out` already point at the matrix this workgroup column works on;
 // `first_row` is the first output row of the workgroup.
-template <int QT, int B, int R, int CB>
-__device__ __forceinline__ void gemv_workgroup(const GemvArgs& a, const uint8_t* w, int first_row, uint8_t* smem) {
+// `emit(b, row, value)` receives each finished output once (batch row b, output
+// row `row` < N), from the thread that summed its K-slices.  A caller that runs
+// the body more than once in a kernel separates the calls with a barrier, as
+// the LDS staging area is reused.
+template <int QT, int B, int R, int CB, class Emit>
+__device__ __forceinline__ void gemv_workgroup_emit(const GemvArgs& a, const uint8_t* w, int first_row, uint8_t* smem,
+                                                    Emit emit) {
   using Regs = WeightRegs<GemvTraits<QT>::REGS>;
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int kslice = wave % a.ks, rowgrp = wave / a.ks;
@@ -409,9 +414,16 @@ __device__ __forceinline__ void gemv_workgroup(const GemvArgs& a, const uint8_t*
     if (row < a.N && b < a.rows) {
       float v = 0.0f;
       for (int s = 0; s < a.ks; ++s) v += red[(s * B + b) * rows_wg + rl];
-      store_scalar(a.out, static_cast<int64_t>(b) * a.N + row, v, a.out_kind);
+      emit(b, row, v);
     }
   }
+}
+
+template <int QT, int B, int R, int CB>
+__device__ __forceinline__ void gemv_workgroup(const GemvArgs& a, const uint8_t* w, int first_row, uint8_t* smem) {
+  gemv_workgroup_emit<QT, B, R, CB>(a, w, first_row, smem, [&](int b, int row, float v) {
+    store_scalar(a.out, static_cast<int64_t>(b) * a.N + row, v, a.out_kind);
+  });
 }
 
 }  // namespace hipengine_gfx950

@@ -6,31 +6,12 @@
 //   Q6_K: out[m,n] = sum_{32-wide group g} xd_g[m] * (s0*dot0 + s1*dot1),  s = d*scale_i8, dots over 16 values
 //         (kernels/hip_gfx1100/quant/gguf_k_mmq_prefill.hip:652-667)
 //
-// Structure (256 threads = 4 waves, 128x128 output tile, each wave 64x64 as 2x2
-// MFMA tiles of 32x32):
-//   * per 256-value K block the workgroup copies the 128 raw weight blocks and
-//     the 128 activation rows into LDS with coalesced 16-byte loads and decodes
-//     the per-sub-block scale tables once;
-//   * a wave reads MFMA operands straight from those LDS images: the int8
-//     activation bytes as they are, the weight nibbles split in registers
-//     (Q6_K: 6-bit values rebuilt and centred in registers).  The MFMA K
-//     extent is one scale group: v_mfma_i32_32x32x32_i8 per Q4_K sub-block,
-//     v_mfma_i32_32x32x16_i8 per 16 Q6_K values, so every int32 result is an
-//     exact sub-block dot;
-//   * the accumulator input of each MFMA is the integer 0x4B400000, so the
-//     int32 result reinterpreted as float IS 12582912 + dot; one FMA with the
-//     per-column constants (sw, -12582912*sw) yields the correctly rounded
-//     sw*dot without an int->float conversion, a second FMA applies the
-//     per-row activation scale;
-//   * the Q4_K min term is rank-8 per block: sum_j mn_j[n]*xsum_j[m] is computed
-//     by one v_mfma_f32_32x32x8f16 (both operands are exact in fp16: xsum is
-//     stored as fp16, mn_j <= 63) and scaled by dmin[n] once per block.
-//
-// The float32 epilogue (2 VALU ops per output element per sub-block, 64 lanes
-// per CU-cycle) bounds this formulation at about a quarter of the int8 MFMA
-// peak: the MFMA pipe itself is mostly idle.
+// Both run 256 threads = 4 waves on a 128x128 output tile, each wave 64x64 as
+// 2x2 MFMA tiles of 32x32, one 128-value K step at a time.  The Q4_K tile
+// engine is in gguf_mmq_q4k.hpp; the Q6_K kernel below follows the same plan
+// with v_mfma_i32_32x32x16_i8 per 16 values.
 
-#include "gguf_common.hpp"
+#include "gguf_mmq_q4k.hpp"
 
 #include "../../include/hipengine_gfx950.h"
 
@@ -38,16 +19,10 @@ namespace {
 
 using namespace hipengine_gfx950;
 
-typedef int v4i __attribute__((ext_vector_type(4)));
-typedef int v16i __attribute__((ext_vector_type(16)));
-typedef float v16f __attribute__((ext_vector_type(16)));
-typedef _Float16 v4h __attribute__((ext_vector_type(4)));
-
-constexpr int BM = 128, BN = 128, THREADS = 256;
-constexpr int A_STRIDE = DS4_BYTES;         // 144 B = 9 x 16 B: conflict free for b128 reads
-constexpr int W_STRIDE = 80;                // 64 quant bytes per K step, padded to 5 x 16 B
-constexpr uint32_t MAGIC_BITS = 0x4B400000u;   // float 12582912 = 1.5 * 2^23
-constexpr float MAGIC = 12582912.0f;
+using DenseQ4 = Q4Tile<2, 2, 2, 2>;
+constexpr int BM = DenseQ4::BM, BN = DenseQ4::BN, THREADS = DenseQ4::THREADS;
+constexpr uint32_t MAGIC_BITS = MMQ_MAGIC_BITS;
+constexpr float MAGIC = MMQ_MAGIC;
 
 struct MmqArgs {
   const uint8_t* xq;
@@ -55,19 +30,6 @@ struct MmqArgs {
   void* out;
   int out_kind;
   int M, K, N;
-};
-
-// One K step is 128 values: one DS4 activation block per row and half of a
-// Q4_K block (two nibble pairs = four 32-wide sub-blocks) per column.
-struct Q4Smem {
-  uint8_t xa[BM * A_STRIDE];   // DS4 blocks of the step, as stored
-  uint8_t wq[BN * W_STRIDE];   // 64 nibble bytes per column
-  float sw[8][BN];             // d*sc per sub-block of the current Q4_K block, by column
-  float cw[8][BN];             // -MAGIC * sw
-  float xd[4][BM];             // activation scale per sub-block of the step, by row
-  float dmin[BN];
-  _Float16 mnh[BN][8];         // 6-bit mins as fp16
-  _Float16 xsh[BM][8];         // activation sums of the Q4_K block (fp16 in the DS4 block already)
 };
 
 __device__ __forceinline__ void store_tile(const MmqArgs& a, const float (&acc)[16], int m_base, int n_col) {
@@ -80,181 +42,22 @@ __device__ __forceinline__ void store_tile(const MmqArgs& a, const float (&acc)[
   }
 }
 
-typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
-
-// Registers of one K step in flight between global memory and LDS.
-struct Q4StepRegs {
-  u32x4 pa[5];   // activation tile chunks (128 rows x 9 chunks = 1152, 4.5 per thread)
-  u32x4 pw[2];   // weight nibble chunks (128 columns x 4 chunks = 512)
-  u32x4 ph;      // threads 0..127: Q4_K block header of column tid; 128..255: DS4 header of row tid-128
-};
-
-__device__ __forceinline__ void q4_step_load(const MmqArgs& a, int step, int m0, int n0, int64_t w_row_bytes,
-                                             int64_t x_row_bytes, int tid, Q4StepRegs& r) {
-  const int kb = step >> 1, h = step & 1;
-#pragma unroll
-  for (int i = 0; i < 5; ++i) {
-    const int c = min(tid + i * THREADS, BM * 9 - 1);
-    const int row = c / 9, part = c - row * 9;
-    const int m = min(m0 + row, a.M - 1);
-    r.pa[i] = *reinterpret_cast<const u32x4*>(a.xq + m * x_row_bytes + static_cast<int64_t>(step) * DS4_BYTES + part * 16);
-  }
-#pragma unroll
-  for (int i = 0; i < 2; ++i) {
-    const int c = tid + i * THREADS;
-    const int row = c >> 2, part = c & 3;
-    const int n = min(n0 + row, a.N - 1);
-    r.pw[i] = *reinterpret_cast<const u32x4*>(a.w + n * w_row_bytes + static_cast<int64_t>(kb) * Q4_K_BYTES + 16 + h * 64 +
-                                              part * 16);
-  }
-  const uint8_t* hp = tid < BN
-                          ? a.w + min(n0 + tid, a.N - 1) * w_row_bytes + static_cast<int64_t>(kb) * Q4_K_BYTES
-                          : a.xq + min(m0 + tid - BN, a.M - 1) * x_row_bytes + static_cast<int64_t>(step) * DS4_BYTES;
-  r.ph = *reinterpret_cast<const u32x4*>(hp);
-}
-
-__device__ __forceinline__ void q4_step_store(Q4Smem& s, int step, int tid, const Q4StepRegs& r) {
-  const int h = step & 1;
-#pragma unroll
-  for (int i = 0; i < 5; ++i) {
-    const int c = tid + i * THREADS;           // 144-byte rows are contiguous in LDS: offset c*16
-    if (c < BM * 9) *reinterpret_cast<u32x4*>(s.xa + c * 16) = r.pa[i];
-  }
-#pragma unroll
-  for (int i = 0; i < 2; ++i) {
-    const int c = tid + i * THREADS;
-    *reinterpret_cast<u32x4*>(s.wq + (c >> 2) * W_STRIDE + (c & 3) * 16) = r.pw[i];
-  }
-  if (tid < BN) {
-    if (h == 0) {
-      const Q4KScales u = q4k_unpack_scales(r.ph.y, r.ph.z, r.ph.w);
-      const float d = f16_bits_to_float(r.ph.x & 0xFFFFu);
-      s.dmin[tid] = f16_bits_to_float(r.ph.x >> 16);
-#pragma unroll
-      for (int j = 0; j < 8; ++j) {
-        const uint32_t sc = ((j < 4 ? u.sc_lo : u.sc_hi) >> (8 * (j & 3))) & 0xFFu;
-        const uint32_t mn = ((j < 4 ? u.mn_lo : u.mn_hi) >> (8 * (j & 3))) & 0xFFu;
-        const float sw = d * static_cast<float>(sc);
-        s.sw[j][tid] = sw;
-        s.cw[j][tid] = -MAGIC * sw;
-        s.mnh[tid][j] = static_cast<_Float16>(static_cast<float>(mn));
-      }
-    }
-  } else {
-    const int row = tid - BN;
-#pragma unroll
-    for (int j = 0; j < 4; ++j) {
-      s.xd[j][row] = f16_bits_to_float(r.ph[j] & 0xFFFFu);
-      s.xsh[row][4 * h + j] = __builtin_bit_cast(_Float16, static_cast<uint16_t>(r.ph[j] >> 16));
-    }
-  }
-}
-
 template <bool PREFETCH>
 __global__ void __launch_bounds__(THREADS, (PREFETCH ? 2 : 3)) mmq_q4_k_ds4_kernel(MmqArgs a) {
   extern __shared__ __align__(16) uint8_t smem_raw[];
-  Q4Smem& s = *reinterpret_cast<Q4Smem*>(smem_raw);
-  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-  const int wm = wave & 1, wn = wave >> 1;
-  const int lc = lane & 31, g = lane >> 5;
+  DenseQ4::Smem& s = *reinterpret_cast<DenseQ4::Smem*>(smem_raw);
   const int m0 = blockIdx.x * BM, n0 = blockIdx.y * BN;
   const int steps = a.K / 128;
   const int64_t w_row_bytes = static_cast<int64_t>(a.K / QK_K) * Q4_K_BYTES;
   const int64_t x_row_bytes = static_cast<int64_t>(steps) * DS4_BYTES;
-
-  float acc[2][2][16];   // [n tile][m tile][v]
-#pragma unroll
-  for (int i = 0; i < 2; ++i)
-#pragma unroll
-    for (int j = 0; j < 2; ++j)
-#pragma unroll
-      for (int v = 0; v < 16; ++v) acc[i][j][v] = 0.0f;
-
-  Q4StepRegs regs;
-  if (PREFETCH) q4_step_load(a, 0, m0, n0, w_row_bytes, x_row_bytes, tid, regs);
-
-  for (int step = 0; step < steps; ++step) {
-    const int h = step & 1;
-    if (!PREFETCH) q4_step_load(a, step, m0, n0, w_row_bytes, x_row_bytes, tid, regs);
-    q4_step_store(s, step, tid, regs);
-    __syncthreads();
-    // The loads of the next step are issued before this step is computed, so
-    // their latency hides behind the MFMA/FMA work.
-    if (PREFETCH && step + 1 < steps) q4_step_load(a, step + 1, m0, n0, w_row_bytes, x_row_bytes, tid, regs);
-
-    // ---- int8 MFMA over the 4 sub-blocks of the step --------------------------
-#pragma unroll
-    for (int sp = 0; sp < 2; ++sp) {
-      v4i wlo[2], whi[2];
-#pragma unroll
-      for (int nt = 0; nt < 2; ++nt) {
-        const int row = wn * 64 + nt * 32 + lc;
-        const u32x4 qs = *reinterpret_cast<const u32x4*>(s.wq + row * W_STRIDE + sp * 32 + 16 * g);
-        wlo[nt] = v4i{static_cast<int>(q4k_low(qs.x)), static_cast<int>(q4k_low(qs.y)),
-                      static_cast<int>(q4k_low(qs.z)), static_cast<int>(q4k_low(qs.w))};
-        whi[nt] = v4i{static_cast<int>(q4k_high(qs.x)), static_cast<int>(q4k_high(qs.y)),
-                      static_cast<int>(q4k_high(qs.z)), static_cast<int>(q4k_high(qs.w))};
-      }
-#pragma unroll
-      for (int half = 0; half < 2; ++half) {
-        const int sl = 2 * sp + half;      // sub-block within the step
-        const int sb = 4 * h + sl;         // sub-block within the Q4_K block
-#pragma unroll
-        for (int mt = 0; mt < 2; ++mt) {
-          const int arow = wm * 64 + mt * 32 + lc;
-          const v4i xop = *reinterpret_cast<const v4i*>(s.xa + arow * A_STRIDE + 16 + sl * 32 + 16 * g);
-          float xdv[16];
-#pragma unroll
-          for (int j = 0; j < 4; ++j) {
-            const float4 t = *reinterpret_cast<const float4*>(&s.xd[sl][wm * 64 + mt * 32 + 8 * j + 4 * g]);
-            xdv[4 * j] = t.x; xdv[4 * j + 1] = t.y; xdv[4 * j + 2] = t.z; xdv[4 * j + 3] = t.w;
-          }
-#pragma unroll
-          for (int nt = 0; nt < 2; ++nt) {
-            const int col = wn * 64 + nt * 32 + lc;
-            const float sw = s.sw[sb][col], cw = s.cw[sb][col];
-            v16i c0;
-#pragma unroll
-            for (int v = 0; v < 16; ++v) c0[v] = static_cast<int>(MAGIC_BITS);
-            const v16i d = __builtin_amdgcn_mfma_i32_32x32x32_i8(xop, half ? whi[nt] : wlo[nt], c0, 0, 0, 0);
-#pragma unroll
-            for (int v = 0; v < 16; ++v) {
-              const float t = __builtin_fmaf(bits_to_float(static_cast<uint32_t>(d[v])), sw, cw);   // = sw * dot, rounded once
-              acc[nt][mt][v] = __builtin_fmaf(xdv[v], t, acc[nt][mt][v]);
-            }
-          }
-        }
-      }
-    }
-
-    // ---- min term, once per Q4_K block: dmin[n] * sum_j mn_j[n] * xsum_j[m] on the fp16 MFMA
-    if (h == 1) {
-#pragma unroll
-      for (int mt = 0; mt < 2; ++mt) {
-        const int arow = wm * 64 + mt * 32 + lc;
-        const v4h xs = *reinterpret_cast<const v4h*>(&s.xsh[arow][4 * g]);
-#pragma unroll
-        for (int nt = 0; nt < 2; ++nt) {
-          const int col = wn * 64 + nt * 32 + lc;
-          const v4h mn = *reinterpret_cast<const v4h*>(&s.mnh[col][4 * g]);
-          v16f z;
-#pragma unroll
-          for (int v = 0; v < 16; ++v) z[v] = 0.0f;
-          const v16f t = __builtin_amdgcn_mfma_f32_32x32x8f16(xs, mn, z, 0, 0, 0);
-          const float nd = -s.dmin[col];
-#pragma unroll
-          for (int v = 0; v < 16; ++v) acc[nt][mt][v] = __builtin_fmaf(nd, t[v], acc[nt][mt][v]);
-        }
-      }
-    }
-    __syncthreads();   // the next step overwrites the tiles
-  }
-
-#pragma unroll
-  for (int nt = 0; nt < 2; ++nt)
-#pragma unroll
-    for (int mt = 0; mt < 2; ++mt)
-      store_tile(a, acc[nt][mt], m0 + wm * 64 + mt * 32 + 4 * g, n0 + wn * 64 + nt * 32 + lc);
+  DenseQ4::run<PREFETCH>(
+      a.xq, x_row_bytes, a.w, w_row_bytes, steps, s,
+      [=](int row) { return static_cast<int64_t>(min(m0 + row, a.M - 1)); },
+      [=](int col) { return static_cast<int64_t>(min(n0 + col, a.N - 1)); },
+      [=](int row, int col, float v) {
+        const int m = m0 + row, n = n0 + col;
+        if (m < a.M && n < a.N) store_scalar(a.out, static_cast<int64_t>(m) * a.N + n, v, a.out_kind);
+      });
 }
 
 int launch_q4(const void* xq, const uint8_t* w, void* out, int out_kind, int64_t M, int64_t K, int64_t N,
@@ -267,9 +70,9 @@ int launch_q4(const void* xq, const uint8_t* w, void* out, int out_kind, int64_t
             static_cast<int>(N)};
   const dim3 grid(static_cast<unsigned>((M + BM - 1) / BM), static_cast<unsigned>((N + BN - 1) / BN));
   if (variant == 1) {
-    hipLaunchKernelGGL(mmq_q4_k_ds4_kernel<false>, grid, dim3(THREADS), sizeof(Q4Smem), stream, a);
+    hipLaunchKernelGGL(mmq_q4_k_ds4_kernel<false>, grid, dim3(THREADS), sizeof(DenseQ4::Smem), stream, a);
   } else {
-    hipLaunchKernelGGL(mmq_q4_k_ds4_kernel<true>, grid, dim3(THREADS), sizeof(Q4Smem), stream, a);
+    hipLaunchKernelGGL(mmq_q4_k_ds4_kernel<true>, grid, dim3(THREADS), sizeof(DenseQ4::Smem), stream, a);
   }
   return static_cast<int>(hipGetLastError());
 }

@@ -1,0 +1,261 @@
+// Tile engine of the Q4_K x DS4 MMQ GEMM on the gfx950 int8 MFMA, shared by the
+// dense prefill GEMM and the expert-grouped (MoE) GEMM.
+//
+//   out[m,n] = sum_{32-wide sub-block j} (d*sc_j)[n] * xd_j[m] * dot_j[m,n] - (dmin*mn_j)[n] * xsum_j[m]
+//   (kernels/hip_gfx1100/quant/gguf_q4_k_q8_1_mmq_prefill.hip:265-276)
+//
+// A workgroup of WM x WN waves computes a (32*MT*WM) x (32*NT*WN) output tile;
+// each wave owns MT x NT MFMA tiles of 32x32.  One K step is 128 values: one
+// DS4 activation block per row and half of a Q4_K block (two nibble pairs =
+// four 32-wide sub-blocks) per column.
+//   * The step's activation blocks and weight nibbles are copied to LDS with
+//     16-byte loads; with PREFETCH the loads of step s+1 are issued into
+//     registers before step s is computed.
+//   * A wave reads MFMA operands straight from those LDS images: the int8
+//     activation bytes as they are, the weight nibbles split in registers.
+//     v_mfma_i32_32x32x32_i8 spans exactly one sub-block, so every int32
+//     result is an exact sub-block dot.
+//   * The accumulator input of each MFMA is the integer 0x4B400000, so the
+//     int32 result reinterpreted as float IS 12582912 + dot; one FMA with the
+//     per-column constants (sw, -12582912*sw) yields the correctly rounded
+//     sw*dot without an int->float conversion (12582912*sw is exact: sw = d*sc
+//     has at most 17 significant bits), a second FMA applies the per-row
+//     activation scale.
+//   * The min term is rank-8 per Q4_K block: sum_j mn_j[n]*xsum_j[m] is one
+//     v_mfma_f32_32x32x8f16 (both operands are exact in fp16: xsum is stored as
+//     fp16, mn_j <= 63), scaled by dmin[n] once per block.
+//
+// The float32 epilogue (2 VALU ops per output element per sub-block, 64 lanes
+// per CU-cycle) bounds this formulation at about a quarter of the int8 MFMA
+// peak: the MFMA pipe itself is mostly idle.
+#pragma once
+
+#include "gguf_common.hpp"
+
+namespace hipengine_gfx950 {
+
+typedef int v4i __attribute__((ext_vector_type(4)));
+typedef int v16i __attribute__((ext_vector_type(16)));
+typedef float v16f __attribute__((ext_vector_type(16)));
+typedef _Float16 v4h __attribute__((ext_vector_type(4)));
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+
+constexpr uint32_t MMQ_MAGIC_BITS = 0x4B400000u;   // float 12582912 = 1.5 * 2^23
+constexpr float MMQ_MAGIC = 12582912.0f;
+
+template <int MT_, int NT_, int WM_, int WN_>
+struct Q4Tile {
+  static constexpr int MT = MT_, NT = NT_, WM = WM_, WN = WN_;
+  static constexpr int BM = 32 * MT * WM, BN = 32 * NT * WN, THREADS = 64 * WM * WN;
+  static constexpr int A_STRIDE = DS4_BYTES;   // 144 B = 9 x 16 B: conflict free for b128 reads
+  static constexpr int W_STRIDE = 80;          // 64 nibble bytes per K step, padded to 5 x 16 B
+  static constexpr int A_CHUNKS = BM * 9, W_CHUNKS = BN * 4, H_ITEMS = BN + BM;
+  static constexpr int A_PER = (A_CHUNKS + THREADS - 1) / THREADS;
+  static constexpr int W_PER = (W_CHUNKS + THREADS - 1) / THREADS;
+  static constexpr int H_PER = (H_ITEMS + THREADS - 1) / THREADS;
+
+  struct Smem {
+    uint8_t xa[BM * A_STRIDE];   // DS4 blocks of the step, as stored
+    uint8_t wq[BN * W_STRIDE];   // 64 nibble bytes per column
+    float sw[8][BN];             // d*sc per sub-block of the current Q4_K block, by column
+    float cw[8][BN];             // -MAGIC * sw
+    float xd[4][BM];             // activation scale per sub-block of the step, by row
+    float dmin[BN];
+    _Float16 mnh[BN][8];         // 6-bit mins as fp16
+    _Float16 xsh[BM][8];         // activation sums of the Q4_K block (fp16 in the DS4 block already)
+  };
+
+  // Registers of one K step in flight between global memory and LDS.
+  struct Regs {
+    u32x4 pa[A_PER];
+    u32x4 pw[W_PER];
+    u32x4 ph[H_PER];   // item < BN: Q4_K block header of that column; else DS4 header of row item-BN
+  };
+
+  // `row_of(r)` / `col_of(c)` give the activation row (in DS4 blocks of x_row_bytes
+  // per row from xq) and the weight row (of w_row_bytes from w) that tile row r /
+  // tile column c read; rows and columns outside the problem are mapped to any
+  // valid one by the caller (their results are not stored).
+  template <class RowOf, class ColOf>
+  static __device__ __forceinline__ void load(const uint8_t* xq, int64_t x_row_bytes, const uint8_t* w,
+                                              int64_t w_row_bytes, int step, int tid, RowOf row_of, ColOf col_of,
+                                              Regs& r) {
+    const int kb = step >> 1, h = step & 1;
+#pragma unroll
+    for (int i = 0; i < A_PER; ++i) {
+      const int c = min(tid + i * THREADS, A_CHUNKS - 1);
+      const int row = c / 9, part = c - row * 9;
+      r.pa[i] = *reinterpret_cast<const u32x4*>(xq + row_of(row) * x_row_bytes + static_cast<int64_t>(step) * DS4_BYTES +
+                                                part * 16);
+    }
+#pragma unroll
+    for (int i = 0; i < W_PER; ++i) {
+      const int c = min(tid + i * THREADS, W_CHUNKS - 1);
+      const int col = c >> 2, part = c & 3;
+      r.pw[i] = *reinterpret_cast<const u32x4*>(w + col_of(col) * w_row_bytes + static_cast<int64_t>(kb) * Q4_K_BYTES + 16 +
+                                                h * 64 + part * 16);
+    }
+#pragma unroll
+    for (int i = 0; i < H_PER; ++i) {
+      const int item = min(tid + i * THREADS, H_ITEMS - 1);
+      const uint8_t* hp = item < BN ? w + col_of(item) * w_row_bytes + static_cast<int64_t>(kb) * Q4_K_BYTES
+                                    : xq + row_of(item - BN) * x_row_bytes + static_cast<int64_t>(step) * DS4_BYTES;
+      r.ph[i] = *reinterpret_cast<const u32x4*>(hp);
+    }
+  }
+
+  static __device__ __forceinline__ void store(Smem& s, int step, int tid, const Regs& r) {
+    const int h = step & 1;
+#pragma unroll
+    for (int i = 0; i < A_PER; ++i) {
+      const int c = tid + i * THREADS;           // 144-byte rows are contiguous in LDS: offset c*16
+      if (c < A_CHUNKS) *reinterpret_cast<u32x4*>(s.xa + c * 16) = r.pa[i];
+    }
+#pragma unroll
+    for (int i = 0; i < W_PER; ++i) {
+      const int c = tid + i * THREADS;
+      if (c < W_CHUNKS) *reinterpret_cast<u32x4*>(s.wq + (c >> 2) * W_STRIDE + (c & 3) * 16) = r.pw[i];
+    }
+#pragma unroll
+    for (int i = 0; i < H_PER; ++i) {
+      const int item = tid + i * THREADS;
+      const u32x4 ph = r.ph[i];
+      if (item < BN) {
+        if (h == 0) {
+          const Q4KScales u = q4k_unpack_scales(ph.y, ph.z, ph.w);
+          const float d = f16_bits_to_float(ph.x & 0xFFFFu);
+          s.dmin[item] = f16_bits_to_float(ph.x >> 16);
+#pragma unroll
+          for (int j = 0; j < 8; ++j) {
+            const uint32_t sc = ((j < 4 ? u.sc_lo : u.sc_hi) >> (8 * (j & 3))) & 0xFFu;
+            const uint32_t mn = ((j < 4 ? u.mn_lo : u.mn_hi) >> (8 * (j & 3))) & 0xFFu;
+            const float sw = d * static_cast<float>(sc);
+            s.sw[j][item] = sw;
+            s.cw[j][item] = -MMQ_MAGIC * sw;
+            s.mnh[item][j] = static_cast<_Float16>(static_cast<float>(mn));
+          }
+        }
+      } else if (item < H_ITEMS) {
+        const int row = item - BN;
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+          s.xd[j][row] = f16_bits_to_float(ph[j] & 0xFFFFu);
+          s.xsh[row][4 * h + j] = __builtin_bit_cast(_Float16, static_cast<uint16_t>(ph[j] >> 16));
+        }
+      }
+    }
+  }
+
+  // One K step of MFMA work on the LDS images; acc is [NT][MT][16].
+  static __device__ __forceinline__ void compute(const Smem& s, int step, int wm, int wn, int lc, int g,
+                                                 float (&acc)[NT][MT][16]) {
+    const int h = step & 1;
+#pragma unroll
+    for (int sp = 0; sp < 2; ++sp) {
+      v4i wlo[NT], whi[NT];
+#pragma unroll
+      for (int nt = 0; nt < NT; ++nt) {
+        const int col = (wn * NT + nt) * 32 + lc;
+        const u32x4 qs = *reinterpret_cast<const u32x4*>(s.wq + col * W_STRIDE + sp * 32 + 16 * g);
+        wlo[nt] = v4i{static_cast<int>(q4k_low(qs.x)), static_cast<int>(q4k_low(qs.y)),
+                      static_cast<int>(q4k_low(qs.z)), static_cast<int>(q4k_low(qs.w))};
+        whi[nt] = v4i{static_cast<int>(q4k_high(qs.x)), static_cast<int>(q4k_high(qs.y)),
+                      static_cast<int>(q4k_high(qs.z)), static_cast<int>(q4k_high(qs.w))};
+      }
+#pragma unroll
+      for (int half = 0; half < 2; ++half) {
+        const int sl = 2 * sp + half;      // sub-block within the step
+        const int sb = 4 * h + sl;         // sub-block within the Q4_K block
+#pragma unroll
+        for (int mt = 0; mt < MT; ++mt) {
+          const int rbase = (wm * MT + mt) * 32;
+          const v4i xop = *reinterpret_cast<const v4i*>(s.xa + (rbase + lc) * A_STRIDE + 16 + sl * 32 + 16 * g);
+          float xdv[16];
+#pragma unroll
+          for (int j = 0; j < 4; ++j) {
+            const float4 t = *reinterpret_cast<const float4*>(&s.xd[sl][rbase + 8 * j + 4 * g]);
+            xdv[4 * j] = t.x; xdv[4 * j + 1] = t.y; xdv[4 * j + 2] = t.z; xdv[4 * j + 3] = t.w;
+          }
+#pragma unroll
+          for (int nt = 0; nt < NT; ++nt) {
+            const int col = (wn * NT + nt) * 32 + lc;
+            const float sw = s.sw[sb][col], cw = s.cw[sb][col];
+            v16i c0;
+#pragma unroll
+            for (int v = 0; v < 16; ++v) c0[v] = static_cast<int>(MMQ_MAGIC_BITS);
+            const v16i d = __builtin_amdgcn_mfma_i32_32x32x32_i8(xop, half ? whi[nt] : wlo[nt], c0, 0, 0, 0);
+#pragma unroll
+            for (int v = 0; v < 16; ++v) {
+              const float t = __builtin_fmaf(bits_to_float(static_cast<uint32_t>(d[v])), sw, cw);   // = sw * dot, rounded once
+              acc[nt][mt][v] = __builtin_fmaf(xdv[v], t, acc[nt][mt][v]);
+            }
+          }
+        }
+      }
+    }
+
+    // min term, once per Q4_K block: dmin[n] * sum_j mn_j[n] * xsum_j[m] on the fp16 MFMA
+    if (h == 1) {
+#pragma unroll
+      for (int mt = 0; mt < MT; ++mt) {
+        const int arow = (wm * MT + mt) * 32 + lc;
+        const v4h xs = *reinterpret_cast<const v4h*>(&s.xsh[arow][4 * g]);
+#pragma unroll
+        for (int nt = 0; nt < NT; ++nt) {
+          const int col = (wn * NT + nt) * 32 + lc;
+          const v4h mn = *reinterpret_cast<const v4h*>(&s.mnh[col][4 * g]);
+          v16f z;
+#pragma unroll
+          for (int v = 0; v < 16; ++v) z[v] = 0.0f;
+          const v16f t = __builtin_amdgcn_mfma_f32_32x32x8f16(xs, mn, z, 0, 0, 0);
+          const float nd = -s.dmin[col];
+#pragma unroll
+          for (int v = 0; v < 16; ++v) acc[nt][mt][v] = __builtin_fmaf(nd, t[v], acc[nt][mt][v]);
+        }
+      }
+    }
+  }
+
+  // The whole K loop of one output tile.  `emit(row, col, value)` receives every
+  // element of the tile (tile-relative coordinates) once.
+  template <bool PREFETCH, class RowOf, class ColOf, class Emit>
+  static __device__ __forceinline__ void run(const uint8_t* xq, int64_t x_row_bytes, const uint8_t* w,
+                                             int64_t w_row_bytes, int steps, Smem& s, RowOf row_of, ColOf col_of,
+                                             Emit emit) {
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int wm = wave % WM, wn = wave / WM;
+    const int lc = lane & 31, g = lane >> 5;
+
+    float acc[NT][MT][16];
+#pragma unroll
+    for (int i = 0; i < NT; ++i)
+#pragma unroll
+      for (int j = 0; j < MT; ++j)
+#pragma unroll
+        for (int v = 0; v < 16; ++v) acc[i][j][v] = 0.0f;
+
+    Regs regs;
+    if (PREFETCH) load(xq, x_row_bytes, w, w_row_bytes, 0, tid, row_of, col_of, regs);
+    for (int step = 0; step < steps; ++step) {
+      if (!PREFETCH) load(xq, x_row_bytes, w, w_row_bytes, step, tid, row_of, col_of, regs);
+      store(s, step, tid, regs);
+      __syncthreads();
+      // The loads of the next step are issued before this step is computed, so
+      // their latency hides behind the MFMA/FMA work.
+      if (PREFETCH && step + 1 < steps) load(xq, x_row_bytes, w, w_row_bytes, step + 1, tid, row_of, col_of, regs);
+      compute(s, step, wm, wn, lc, g, acc);
+      __syncthreads();   // the next step overwrites the tiles
+    }
+
+    // lane holds column lc of each n tile and rows 8*(v/4) + 4*g + v%4 of each m tile
+#pragma unroll
+    for (int nt = 0; nt < NT; ++nt)
+#pragma unroll
+      for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+        for (int v = 0; v < 16; ++v)
+          emit((wm * MT + mt) * 32 + 8 * (v >> 2) + 4 * g + (v & 3), (wn * NT + nt) * 32 + lc, acc[nt][mt][v]);
+  }
+};
+
+}  // namespace hipengine_gfx950

@@ -1,0 +1,604 @@
+// Expert-indexed (MoE) forms of the GGUF k-quant matmul for gfx950, and the
+// routing index they consume.
+//
+//   routing index  selected[L] (lane = token*top_k + slot) -> expert-major order:
+//                  expert_start[E+1], sorted_lanes, compact_to_source, sorted_weights,
+//                  active list; tile map of 32-row tiles per expert
+//                  (kernels/hip_gfx1100/moe/group_scatter.hip:62-141,328-389)
+//   decode         selected GEMV: out[lane] = W[selected[lane]] . x[lane / top_k]
+//                  (kernels/hip_gfx1100/quant/gguf_q4_k_gemv.hip:322-359), the fused
+//                  gate/up form silu(gate)*up (:666-737) and the routed down
+//                  projection summed over a token's experts; all on the q8_1
+//                  integer GEMV body of gguf_gemv.hpp
+//   prefill        expert-grouped Q4_K x DS4 MMQ over compact rows and the tile map
+//                  (kernels/hip_gfx1100/quant/gguf_q4_k_q8_1_selected_prefill.hip:1256-1670)
+//                  on the tile engine of gguf_mmq_q4k.hpp
+
+#include "gguf_gemv.hpp"
+#include "gguf_mmq_q4k.hpp"
+
+#include "../../include/hipengine_gfx950.h"
+
+namespace {
+
+using namespace hipengine_gfx950;
+
+constexpr int MAX_EXPERTS = 2048;
+
+// --------------------------------------------------------------------------
+// routing index
+// --------------------------------------------------------------------------
+
+__device__ __forceinline__ int wave_sum_i(int v) {
+#pragma unroll
+  for (int off = 32; off > 0; off >>= 1) v += __shfl_xor(v, off, 64);
+  return v;
+}
+
+// One workgroup per expert: counts[e] = number of lanes that selected e.
+__global__ void __launch_bounds__(256) moe_count_kernel(const int64_t* __restrict__ selected, int64_t* __restrict__ counts,
+                                                        int64_t lanes) {
+  __shared__ int part[4];
+  const int64_t e = blockIdx.x;
+  int c = 0;
+  for (int64_t i = threadIdx.x; i < lanes; i += 256) c += selected[i] == e;
+  c = wave_sum_i(c);
+  if ((threadIdx.x & 63) == 0) part[threadIdx.x >> 6] = c;
+  __syncthreads();
+  if (threadIdx.x == 0) counts[e] = part[0] + part[1] + part[2] + part[3];
+}
+
+// One workgroup: counts (in expert_start[0..E)) -> exclusive starts, total in
+// expert_start[E], ascending list of the experts that own at least one lane.
+__global__ void __launch_bounds__(256) moe_prefix_active_kernel(int64_t* __restrict__ expert_start,
+                                                                int64_t* __restrict__ active_experts,
+                                                                int64_t* __restrict__ active_count, int num_experts) {
+  __shared__ int cnt[MAX_EXPERTS];
+  __shared__ int act[MAX_EXPERTS];
+  __shared__ int totals[2];
+  for (int e = threadIdx.x; e < num_experts; e += 256) cnt[e] = static_cast<int>(expert_start[e]);
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    int offset = 0, active = 0;
+    for (int e = 0; e < num_experts; ++e) {
+      const int c = cnt[e];
+      cnt[e] = offset;
+      if (c > 0) { act[active++] = e; offset += c; }
+    }
+    totals[0] = offset; totals[1] = active;
+  }
+  __syncthreads();
+  for (int e = threadIdx.x; e < num_experts; e += 256) expert_start[e] = cnt[e];
+  if (active_experts)
+    for (int i = threadIdx.x; i < totals[1]; i += 256) active_experts[i] = act[i];
+  if (threadIdx.x == 0) {
+    expert_start[num_experts] = totals[0];
+    if (active_count) active_count[0] = totals[1];
+  }
+}
+
+// One workgroup per expert: writes its lanes in ascending lane order (wave
+// ballots keep the order) into [expert_start[e], expert_start[e+1]).
+__global__ void __launch_bounds__(256) moe_place_kernel(const int64_t* __restrict__ selected,
+                                                        const float* __restrict__ routing,
+                                                        const int64_t* __restrict__ expert_start,
+                                                        int64_t* __restrict__ sorted_lanes,
+                                                        int64_t* __restrict__ sorted_experts,
+                                                        int64_t* __restrict__ compact_to_source,
+                                                        float* __restrict__ sorted_weights, int64_t lanes,
+                                                        int64_t top_k) {
+  __shared__ int wave_cnt[4];
+  const int64_t e = blockIdx.x;
+  const int64_t base = expert_start[e];
+  const int count = static_cast<int>(expert_start[e + 1] - base);
+  if (count <= 0) return;
+  const int lane_id = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  int running = 0;
+  for (int64_t chunk = 0; chunk < lanes && running < count; chunk += 256) {
+    const int64_t lane = chunk + threadIdx.x;
+    const bool flag = lane < lanes && selected[lane] == e;
+    const unsigned long long ballot = __ballot(flag);
+    const int before = __popcll(ballot & ((1ull << lane_id) - 1ull));
+    if (lane_id == 0) wave_cnt[wave] = __popcll(ballot);
+    __syncthreads();
+    int offset = running, total = 0;
+#pragma unroll
+    for (int w = 0; w < 4; ++w) {
+      if (w < wave) offset += wave_cnt[w];
+      total += wave_cnt[w];
+    }
+    if (flag) {
+      const int64_t idx = base + offset + before;
+      sorted_lanes[idx] = lane;
+      if (sorted_experts) sorted_experts[idx] = e;
+      if (compact_to_source) compact_to_source[idx] = lane / top_k;
+      if (sorted_weights) sorted_weights[idx] = routing[lane];
+    }
+    running += total;
+    __syncthreads();
+  }
+}
+
+int launch_compact(const int64_t* selected, const float* routing, int64_t* expert_start, int64_t* active_experts,
+                   int64_t* active_count, int64_t* sorted_lanes, int64_t* sorted_experts, int64_t* compact_to_source,
+                   float* sorted_weights, int64_t lanes, int64_t num_experts, int64_t top_k, hipStream_t stream) {
+  if (!selected || !expert_start || !sorted_lanes || (sorted_weights && !routing) || lanes <= 0 || lanes > (1ll << 30) ||
+      num_experts <= 0 || num_experts > MAX_EXPERTS || top_k <= 0) {
+    return static_cast<int>(hipErrorInvalidValue);
+  }
+  hipLaunchKernelGGL(moe_count_kernel, dim3(static_cast<unsigned>(num_experts)), dim3(256), 0, stream, selected,
+                     expert_start, lanes);
+  hipLaunchKernelGGL(moe_prefix_active_kernel, dim3(1), dim3(256), 0, stream, expert_start, active_experts, active_count,
+                     static_cast<int>(num_experts));
+  hipLaunchKernelGGL(moe_place_kernel, dim3(static_cast<unsigned>(num_experts)), dim3(256), 0, stream, selected, routing,
+                     expert_start, sorted_lanes, sorted_experts, compact_to_source, sorted_weights, lanes, top_k);
+  return static_cast<int>(hipGetLastError());
+}
+
+// One workgroup: per-expert row counts rounded up to tile_rows, their prefix,
+// and the tile -> expert map (-1 where a tile belongs to no expert).
+__global__ void __launch_bounds__(256) moe_tile_map_kernel(const int64_t* __restrict__ expert_start_compact,
+                                                           int64_t* __restrict__ tile_expert_start,
+                                                           int64_t* __restrict__ tile_expert,
+                                                           int64_t* __restrict__ total_out, int num_experts,
+                                                           int64_t tile_capacity, int tile_rows) {
+  __shared__ int start[MAX_EXPERTS + 1];
+  for (int e = threadIdx.x; e < num_experts; e += 256) {
+    const int c = static_cast<int>(expert_start_compact[e + 1] - expert_start_compact[e]);
+    start[e] = (c + tile_rows - 1) / tile_rows * tile_rows;
+  }
+  for (int64_t i = threadIdx.x; i < tile_capacity; i += 256) tile_expert[i] = -1;
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    int offset = 0;
+    for (int e = 0; e < num_experts; ++e) {
+      const int p = start[e];
+      start[e] = offset;
+      offset += p;
+    }
+    start[num_experts] = offset;
+  }
+  __syncthreads();
+  for (int e = threadIdx.x; e <= num_experts; e += 256) tile_expert_start[e] = start[e];
+  if (threadIdx.x == 0) total_out[0] = start[num_experts];
+  for (int e = threadIdx.x; e < num_experts; e += 256) {
+    for (int t = start[e] / tile_rows; t < start[e + 1] / tile_rows; ++t)
+      if (tile_capacity <= 0 || t < tile_capacity) tile_expert[t] = e;
+  }
+}
+
+int launch_tile_map(const int64_t* expert_start_compact, int64_t* tile_expert_start, int64_t* tile_expert,
+                    int64_t* total_out, int64_t num_experts, int64_t tile_capacity, int tile_rows,
+                    hipStream_t stream) {
+  if (!expert_start_compact || !tile_expert_start || !tile_expert || !total_out || num_experts <= 0 ||
+      num_experts > MAX_EXPERTS || tile_rows <= 0) {
+    return static_cast<int>(hipErrorInvalidValue);
+  }
+  hipLaunchKernelGGL(moe_tile_map_kernel, dim3(1), dim3(256), 0, stream, expert_start_compact, tile_expert_start,
+                     tile_expert, total_out, static_cast<int>(num_experts), tile_capacity, tile_rows);
+  return static_cast<int>(hipGetLastError());
+}
+
+// lane_to_compact[lane] = position of the lane in the expert-major order, -1 if dropped.
+__global__ void moe_fill_i64_kernel(int64_t* p, int64_t n, int64_t v) {
+  const int64_t i = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x;
+  if (i < n) p[i] = v;
+}
+__global__ void moe_invert_kernel(const int64_t* __restrict__ sorted_lanes, int64_t* __restrict__ lane_to_compact,
+                                  int64_t compact_rows, int64_t lanes) {
+  const int64_t i = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x;
+  if (i < compact_rows) {
+    const int64_t lane = sorted_lanes[i];
+    if (lane >= 0 && lane < lanes) lane_to_compact[lane] = i;
+  }
+}
+
+// --------------------------------------------------------------------------
+// elementwise steps between the projections
+// --------------------------------------------------------------------------
+
+__device__ __forceinline__ float silu_mul(float gate, float up) {
+  const float sig = 1.0f / (1.0f + expf(-gate));
+  return gate * sig * up;
+}
+
+// gate_up [rows, 2*inter] (gate columns first) -> out [rows, inter] = silu(gate) * up
+__global__ void moe_silu_mul_kernel(const void* __restrict__ gate_up, void* __restrict__ out, int64_t rows,
+                                    int64_t inter, int in_kind, int out_kind) {
+  const int64_t i = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x;
+  if (i >= rows * inter) return;
+  const int64_t r = i / inter, c = i - r * inter;
+  const float g = load_scalar(gate_up, r * 2 * inter + c, in_kind);
+  const float u = load_scalar(gate_up, r * 2 * inter + inter + c, in_kind);
+  store_scalar(out, i, silu_mul(g, u), out_kind);
+}
+
+// out[t, h] = sum over the token's slots, in slot order, of routing[lane] * down[lane_to_compact[lane], h]
+__global__ void moe_weighted_gather_kernel(const void* __restrict__ down, const int64_t* __restrict__ lane_to_compact,
+                                           const float* __restrict__ routing, void* __restrict__ out, int64_t tokens,
+                                           int64_t top_k, int64_t hidden, int64_t compact_rows, int in_kind,
+                                           int out_kind) {
+  const int64_t t = blockIdx.y;
+  const int64_t h = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x;
+  if (t >= tokens || h >= hidden) return;
+  float acc = 0.0f;
+  for (int64_t s = 0; s < top_k; ++s) {
+    const int64_t lane = t * top_k + s;
+    const int64_t c = lane_to_compact[lane];
+    if (c < 0 || c >= compact_rows) continue;
+    acc += routing[lane] * load_scalar(down, c * hidden + h, in_kind);
+  }
+  store_scalar(out, t * hidden + h, acc, out_kind);
+}
+
+// --------------------------------------------------------------------------
+// decode: selected GEMV on the q8_1 integer GEMV body
+// --------------------------------------------------------------------------
+
+enum SelMode : int { SEL_SINGLE = 0, SEL_DUAL_SILU = 1, SEL_DOWN_SUM = 2 };
+
+struct SelArgs {
+  GemvArgs g;                 // x, w (first weight), out, kinds, K, N, ks, nrg; rows = 1
+  const uint8_t* w_b;         // second weight (dual)
+  const int64_t* selected;    // [lanes]
+  const float* routing;       // [lanes] (down sum)
+  int x_rows;                 // activation rows (tokens) for single/dual; tokens for down sum
+  int lanes;
+  int num_experts;
+  int top_k;
+  int round_mid;              // dual: round gate and up to the output type before silu (the fused device form)
+};
+
+__device__ __forceinline__ int64_t scalar_bytes(int kind) { return kind == KIND_F32 ? 4 : 2; }
+
+// Workgroup size cap: the CB weight blocks of a chunk have to fit the VGPR
+// budget the cap implies (128 registers at 1024 threads, 256 at 512).
+template <int QT, int CB>
+constexpr int sel_max_threads() {
+  return CB * GemvTraits<QT>::REGS <= 64 ? 1024 : 512;
+}
+
+template <int QT, int R, int CB, int MODE>
+__global__ void __launch_bounds__((sel_max_threads<QT, CB>())) selected_gemv_kernel(SelArgs s) {
+  extern __shared__ __align__(16) uint8_t smem[];
+  const int rows_wg = s.g.nrg * 16 * R;
+  const int first_row = blockIdx.x * rows_wg;
+  const int64_t row_bytes = static_cast<int64_t>(s.g.K / QK_K) * GemvTraits<QT>::SUPER_BYTES;
+  const int64_t expert_bytes = static_cast<int64_t>(s.g.N) * row_bytes;
+  GemvArgs a = s.g;
+  a.rows = 1;
+
+  if constexpr (MODE == SEL_DOWN_SUM) {
+    const int t = blockIdx.y;
+    float total = 0.0f;
+    int my_row = -1;
+    for (int slot = 0; slot < s.top_k; ++slot) {
+      const int lane = t * s.top_k + slot;
+      const int64_t e = s.selected[lane];
+      if (e < 0 || e >= s.num_experts) continue;          // uniform over the workgroup
+      const float wgt = s.routing[lane];
+      a.x = static_cast<const uint8_t*>(s.g.x) + static_cast<int64_t>(lane) * s.g.K * scalar_bytes(s.g.x_kind);
+      __syncthreads();
+      gemv_workgroup_emit<QT, 1, R, CB>(a, s.g.w + e * expert_bytes, first_row, smem, [&](int, int row, float v) {
+        total += wgt * v;
+        my_row = row;
+      });
+    }
+    if (my_row >= 0) store_scalar(s.g.out, static_cast<int64_t>(t) * s.g.N + my_row, total, s.g.out_kind);
+    // rows whose token selected no valid expert at all are written as zero
+    if (my_row < 0) {
+      bool any = false;
+      for (int slot = 0; slot < s.top_k; ++slot) {
+        const int64_t e = s.selected[t * s.top_k + slot];
+        any |= (e >= 0 && e < s.num_experts);
+      }
+      if (!any)
+        for (int r = threadIdx.x; r < rows_wg; r += blockDim.x)
+          if (first_row + r < s.g.N) store_scalar(s.g.out, static_cast<int64_t>(t) * s.g.N + first_row + r, 0.0f, s.g.out_kind);
+    }
+  } else {
+    const int lane = blockIdx.y;
+    const int64_t e = s.selected[lane];
+    if (e < 0 || e >= s.num_experts) return;
+    const int per = s.lanes / s.x_rows;
+    const int x_row = s.x_rows == 1 ? 0 : lane / per;
+    a.x = static_cast<const uint8_t*>(s.g.x) + static_cast<int64_t>(x_row) * s.g.K * scalar_bytes(s.g.x_kind);
+    a.out = static_cast<uint8_t*>(s.g.out) + static_cast<int64_t>(lane) * s.g.N * scalar_bytes(s.g.out_kind);
+    if constexpr (MODE == SEL_SINGLE) {
+      gemv_workgroup<QT, 1, R, CB>(a, s.g.w + e * expert_bytes, first_row, smem);
+    } else {
+      float gate = 0.0f;
+      gemv_workgroup_emit<QT, 1, R, CB>(a, s.g.w + e * expert_bytes, first_row, smem,
+                                       [&](int, int, float v) { gate = v; });
+      __syncthreads();
+      gemv_workgroup_emit<QT, 1, R, CB>(a, s.w_b + e * expert_bytes, first_row, smem, [&](int, int row, float up) {
+        float gv = gate, uv = up;
+        if (s.round_mid && a.out_kind == KIND_BF16) {
+          gv = bf16_bits_to_float(float_to_bf16_bits(gv));
+          uv = bf16_bits_to_float(float_to_bf16_bits(uv));
+        } else if (s.round_mid && a.out_kind == KIND_F16) {
+          gv = f16_bits_to_float(float_to_f16_bits(gv));
+          uv = f16_bits_to_float(float_to_f16_bits(uv));
+        }
+        store_scalar(a.out, row, silu_mul(gv, uv), a.out_kind);
+      });
+    }
+  }
+}
+
+using SelFn = void (*)(SelArgs);
+struct SelVariant {
+  int qt, cb, mode, max_threads;
+  SelFn fn;
+};
+#define SEL_VARIANTS(QT, CB)                                                                       \
+  SelVariant{QT, CB, SEL_SINGLE, sel_max_threads<QT, CB>(), selected_gemv_kernel<QT, 1, CB, SEL_SINGLE>},       \
+  SelVariant{QT, CB, SEL_DUAL_SILU, sel_max_threads<QT, CB>(), selected_gemv_kernel<QT, 1, CB, SEL_DUAL_SILU>}, \
+  SelVariant{QT, CB, SEL_DOWN_SUM, sel_max_threads<QT, CB>(), selected_gemv_kernel<QT, 1, CB, SEL_DOWN_SUM>}
+const SelVariant kSel[] = {
+    SEL_VARIANTS(GGML_Q4_K, 1), SEL_VARIANTS(GGML_Q4_K, 2), SEL_VARIANTS(GGML_Q4_K, 5),
+    SEL_VARIANTS(GGML_Q6_K, 1), SEL_VARIANTS(GGML_Q6_K, 2), SEL_VARIANTS(GGML_Q6_K, 5),
+};
+
+int launch_selected(int qt, int mode, const void* x, int x_kind, const int64_t* selected, const float* routing,
+                    const uint8_t* w_a, const uint8_t* w_b, void* out, int out_kind, int64_t x_rows, int64_t lanes,
+                    int64_t num_experts, int64_t top_k, int64_t K, int64_t N, int round_mid, hipStream_t stream) {
+  if (!x || !selected || !w_a || !out || x_rows <= 0 || lanes <= 0 || lanes > 65535 || num_experts <= 0 || K <= 0 ||
+      (K % QK_K) != 0 || K > (1 << 20) || N <= 0 || N > (1 << 24) || x_kind < KIND_F32 || x_kind > KIND_F16 ||
+      out_kind < KIND_F32 || out_kind > KIND_F16) {
+    return static_cast<int>(hipErrorInvalidValue);
+  }
+  if (mode == SEL_DUAL_SILU && !w_b) return static_cast<int>(hipErrorInvalidValue);
+  if (mode == SEL_DOWN_SUM && (!routing || top_k <= 0 || lanes != x_rows * top_k)) return static_cast<int>(hipErrorInvalidValue);
+  if (mode != SEL_DOWN_SUM && (lanes % x_rows) != 0) return static_cast<int>(hipErrorInvalidValue);
+  const int nb = static_cast<int>(K / QK_K);
+  const int ks = nb >= 4 ? 4 : nb;
+  const int per_wave = (nb + ks - 1) / ks;
+  const int cb = per_wave >= 5 ? 5 : per_wave >= 2 ? 2 : 1;
+  const int64_t groups = mode == SEL_DOWN_SUM ? x_rows : lanes;   // grid.y
+  const SelVariant* v = nullptr;
+  for (const SelVariant& c : kSel)
+    if (c.qt == qt && c.cb == cb && c.mode == mode) v = &c;
+  if (!v) return static_cast<int>(hipErrorInvalidValue);
+  int nrg = v->max_threads / 64 / ks;
+  while (nrg > 1 && (N + nrg * 16 - 1) / (nrg * 16) * groups < 512) nrg >>= 1;
+  const size_t lds = gemv_lds_bytes(qt, 1, 1, cb, ks, nrg);
+  if (lds > 64 * 1024) return static_cast<int>(hipErrorInvalidValue);
+  SelArgs s;
+  s.g.x = x; s.g.w = w_a; s.g.out = out; s.g.x_kind = x_kind; s.g.out_kind = out_kind; s.g.rows = 1;
+  s.g.K = static_cast<int>(K); s.g.N = static_cast<int>(N); s.g.ks = ks; s.g.nrg = nrg;
+  s.w_b = w_b; s.selected = selected; s.routing = routing;
+  s.x_rows = static_cast<int>(x_rows); s.lanes = static_cast<int>(lanes);
+  s.num_experts = static_cast<int>(num_experts); s.top_k = static_cast<int>(top_k); s.round_mid = round_mid;
+  const dim3 grid(static_cast<unsigned>((N + nrg * 16 - 1) / (nrg * 16)), static_cast<unsigned>(groups));
+  hipLaunchKernelGGL(v->fn, grid, dim3(ks * nrg * 64), lds, stream, s);
+  return static_cast<int>(hipGetLastError());
+}
+
+// --------------------------------------------------------------------------
+// prefill: expert-grouped Q4_K x DS4 MMQ over 32-row tiles
+// --------------------------------------------------------------------------
+
+using MoeQ4 = Q4Tile<1, 2, 1, 4>;   // 32 compact rows x 256 columns, four waves side by side
+
+struct MoeMmqArgs {
+  const uint8_t* xq;                 // DS4 blocks [source_rows, K/128]
+  const int64_t* compact_to_source;  // [compact_rows] or null (compact row i reads source row i)
+  const int64_t* expert_start_compact;
+  const int64_t* expert_start_tiles; // row starts rounded up to 32 per expert
+  const int64_t* tile_expert;        // [total_rows/32]
+  const uint8_t* w_a;
+  const uint8_t* w_b;
+  void* out;                         // [compact_rows, Na + Nb]
+  int out_kind;
+  int compact_rows, source_rows, K, Na, Nb, num_experts;
+  int64_t expert_stride_rows;
+  int tiles_a;
+};
+
+__global__ void __launch_bounds__(MoeQ4::THREADS, 2) moe_mmq_q4_k_kernel(MoeMmqArgs a) {
+  extern __shared__ __align__(16) uint8_t smem_raw[];
+  MoeQ4::Smem& s = *reinterpret_cast<MoeQ4::Smem*>(smem_raw);
+  int* src_row = reinterpret_cast<int*>(smem_raw + sizeof(MoeQ4::Smem));
+
+  const int tile_row = blockIdx.y;
+  const int64_t e = a.tile_expert[tile_row];
+  if (e < 0 || e >= a.num_experts) return;
+  const bool use_b = static_cast<int>(blockIdx.x) >= a.tiles_a;
+  const int n0 = (use_b ? blockIdx.x - a.tiles_a : blockIdx.x) * MoeQ4::BN;
+  const int local_n = use_b ? a.Nb : a.Na;
+  const int64_t compact_base = a.expert_start_compact[e];
+  const int64_t count = a.expert_start_compact[e + 1] - compact_base;
+  const int64_t row0 = static_cast<int64_t>(tile_row) * MoeQ4::BM - a.expert_start_tiles[e];
+  const int64_t remaining = count - row0;
+  if (row0 < 0 || remaining <= 0) return;
+  const int valid_rows = remaining >= MoeQ4::BM ? MoeQ4::BM : static_cast<int>(remaining);
+  const int64_t first_compact = compact_base + row0;
+  if (first_compact + valid_rows > a.compact_rows) return;
+
+  const int steps = a.K / 128;
+  const int64_t w_row_bytes = static_cast<int64_t>(a.K / QK_K) * Q4_K_BYTES;
+  const int64_t x_row_bytes = static_cast<int64_t>(steps) * DS4_BYTES;
+  const int64_t stride_rows = a.expert_stride_rows > 0 ? a.expert_stride_rows : local_n;
+  const uint8_t* w = (use_b ? a.w_b : a.w_a) + e * stride_rows * w_row_bytes;
+
+  if (threadIdx.x < MoeQ4::BM) {
+    const int64_t crow = first_compact + min(static_cast<int>(threadIdx.x), valid_rows - 1);
+    int64_t src = a.compact_to_source ? a.compact_to_source[crow] : crow;
+    src = src < 0 ? 0 : (src >= a.source_rows ? a.source_rows - 1 : src);
+    src_row[threadIdx.x] = static_cast<int>(src);
+  }
+  __syncthreads();
+
+  const int64_t out_stride = static_cast<int64_t>(a.Na) + a.Nb;
+  const int col_base = (use_b ? a.Na : 0) + n0;
+  MoeQ4::run<true>(
+      a.xq, x_row_bytes, w, w_row_bytes, steps, s,
+      [=](int row) { return static_cast<int64_t>(src_row[row]); },
+      [=](int col) { return static_cast<int64_t>(min(n0 + col, local_n - 1)); },
+      [=](int row, int col, float v) {
+        if (row < valid_rows && n0 + col < local_n)
+          store_scalar(a.out, (first_compact + row) * out_stride + col_base + col, v, a.out_kind);
+      });
+}
+
+int launch_moe_mmq(const void* xq, const int64_t* compact_to_source, const int64_t* expert_start_compact,
+                   const int64_t* expert_start_tiles, const int64_t* tile_expert, const uint8_t* w_a,
+                   const uint8_t* w_b, void* out, int out_kind, int64_t compact_rows, int64_t source_rows, int64_t K,
+                   int64_t Na, int64_t Nb, int64_t num_experts, int64_t total_rows, int64_t expert_stride_rows,
+                   hipStream_t stream) {
+  if (!xq || !expert_start_compact || !expert_start_tiles || !tile_expert || !w_a || !out || compact_rows <= 0 ||
+      compact_rows > (1 << 24) || source_rows <= 0 || source_rows > (1 << 24) || K <= 0 || (K % QK_K) != 0 ||
+      Na <= 0 || (Na % 32) != 0 || Nb < 0 || (Nb % 32) != 0 || (Nb > 0 && !w_b) || Na + Nb > (1 << 24) ||
+      num_experts <= 0 || total_rows <= 0 || (total_rows % 32) != 0 || total_rows / 32 > 65535 ||
+      expert_stride_rows < 0 || out_kind < KIND_F32 || out_kind > KIND_F16) {
+    return static_cast<int>(hipErrorInvalidValue);
+  }
+  MoeMmqArgs a;
+  a.xq = static_cast<const uint8_t*>(xq);
+  a.compact_to_source = compact_to_source;
+  a.expert_start_compact = expert_start_compact;
+  a.expert_start_tiles = expert_start_tiles;
+  a.tile_expert = tile_expert;
+  a.w_a = w_a; a.w_b = w_b; a.out = out; a.out_kind = out_kind;
+  a.compact_rows = static_cast<int>(compact_rows); a.source_rows = static_cast<int>(source_rows);
+  a.K = static_cast<int>(K); a.Na = static_cast<int>(Na); a.Nb = static_cast<int>(Nb);
+  a.num_experts = static_cast<int>(num_experts);
+  a.expert_stride_rows = expert_stride_rows;
+  a.tiles_a = static_cast<int>((Na + MoeQ4::BN - 1) / MoeQ4::BN);
+  const int tiles_b = static_cast<int>((Nb + MoeQ4::BN - 1) / MoeQ4::BN);
+  const dim3 grid(static_cast<unsigned>(a.tiles_a + tiles_b), static_cast<unsigned>(total_rows / 32));
+  hipLaunchKernelGGL(moe_mmq_q4_k_kernel, grid, dim3(MoeQ4::THREADS), sizeof(MoeQ4::Smem) + MoeQ4::BM * sizeof(int),
+                     stream, a);
+  return static_cast<int>(hipGetLastError());
+}
+
+}  // namespace
+
+// ---- routing index ------------------------------------------------------------
+
+extern "C" int hipengine_qwen35_moe_group_compact_active(const int64_t* selected_experts, const float* routing_weights,
+                                                         int64_t* expert_start, int64_t* active_experts,
+                                                         int64_t* active_count, int64_t* sorted_lanes,
+                                                         int64_t* sorted_experts, float* sorted_weights,
+                                                         int64_t total_lanes, int64_t num_experts, hipStream_t stream) {
+  return launch_compact(selected_experts, routing_weights, expert_start, active_experts, active_count, sorted_lanes,
+                        sorted_experts, nullptr, sorted_weights, total_lanes, num_experts, 1, stream);
+}
+
+extern "C" int hipengine_qwen35_moe_group_compact_active_source_rows(
+    const int64_t* selected_experts, const float* routing_weights, int64_t* expert_start, int64_t* active_experts,
+    int64_t* active_count, int64_t* sorted_lanes, int64_t* compact_to_source, float* sorted_weights,
+    int64_t total_lanes, int64_t num_experts, int64_t top_k, hipStream_t stream) {
+  return launch_compact(selected_experts, routing_weights, expert_start, active_experts, active_count, sorted_lanes,
+                        nullptr, compact_to_source, sorted_weights, total_lanes, num_experts, top_k, stream);
+}
+
+extern "C" int hipengine_qwen35_moe_mmq32_tile_map(const int64_t* expert_start_compact, int64_t* mmq_expert_start,
+                                                   int64_t* tile_expert, int64_t* mmq_total_out, int64_t num_experts,
+                                                   int64_t tile_capacity, hipStream_t stream) {
+  return launch_tile_map(expert_start_compact, mmq_expert_start, tile_expert, mmq_total_out, num_experts, tile_capacity,
+                         32, stream);
+}
+
+extern "C" int hipengine_gfx950_moe_lane_to_compact(const int64_t* sorted_lanes, int64_t* lane_to_compact,
+                                                    int64_t compact_rows, int64_t total_lanes, hipStream_t stream) {
+  if (!sorted_lanes || !lane_to_compact || compact_rows <= 0 || total_lanes <= 0) {
+    return static_cast<int>(hipErrorInvalidValue);
+  }
+  hipLaunchKernelGGL(moe_fill_i64_kernel, dim3(static_cast<unsigned>((total_lanes + 255) / 256)), dim3(256), 0, stream,
+                     lane_to_compact, total_lanes, static_cast<int64_t>(-1));
+  hipLaunchKernelGGL(moe_invert_kernel, dim3(static_cast<unsigned>((compact_rows + 255) / 256)), dim3(256), 0, stream,
+                     sorted_lanes, lane_to_compact, compact_rows, total_lanes);
+  return static_cast<int>(hipGetLastError());
+}
+
+// ---- elementwise steps ----------------------------------------------------------
+
+extern "C" int hipengine_gfx950_moe_silu_mul(const void* gate_up, void* out, int64_t rows, int64_t inter, int in_kind,
+                                             int out_kind, hipStream_t stream) {
+  if (!gate_up || !out || rows <= 0 || inter <= 0 || in_kind < KIND_F32 || in_kind > KIND_F16 || out_kind < KIND_F32 ||
+      out_kind > KIND_F16 || rows * inter > (1ll << 40)) {
+    return static_cast<int>(hipErrorInvalidValue);
+  }
+  hipLaunchKernelGGL(moe_silu_mul_kernel, dim3(static_cast<unsigned>((rows * inter + 255) / 256)), dim3(256), 0, stream,
+                     gate_up, out, rows, inter, in_kind, out_kind);
+  return static_cast<int>(hipGetLastError());
+}
+
+extern "C" int hipengine_gfx950_moe_weighted_gather_sum(const void* down, const int64_t* lane_to_compact,
+                                                        const float* routing_weights, void* out, int64_t tokens,
+                                                        int64_t top_k, int64_t hidden, int64_t compact_rows,
+                                                        int in_kind, int out_kind, hipStream_t stream) {
+  if (!down || !lane_to_compact || !routing_weights || !out || tokens <= 0 || tokens > 65535 || top_k <= 0 ||
+      hidden <= 0 || compact_rows <= 0 || in_kind < KIND_F32 || in_kind > KIND_F16 || out_kind < KIND_F32 ||
+      out_kind > KIND_F16) {
+    return static_cast<int>(hipErrorInvalidValue);
+  }
+  hipLaunchKernelGGL(moe_weighted_gather_kernel, dim3(static_cast<unsigned>((hidden + 255) / 256),
+                                                      static_cast<unsigned>(tokens)),
+                     dim3(256), 0, stream, down, lane_to_compact, routing_weights, out, tokens, top_k, hidden,
+                     compact_rows, in_kind, out_kind);
+  return static_cast<int>(hipGetLastError());
+}
+
+// ---- decode ---------------------------------------------------------------------
+
+extern "C" int hipengine_gguf_q4_k_selected_gemv_bf16_bf16_out(const uint16_t* x, const int64_t* selected,
+                                                               const uint8_t* qweight, uint16_t* out, int64_t x_rows,
+                                                               int64_t rows, int64_t num_experts, int64_t in_features,
+                                                               int64_t out_features, int64_t threads,
+                                                               hipStream_t stream) {
+  (void)threads;
+  return launch_selected(GGML_Q4_K, SEL_SINGLE, x, KIND_BF16, selected, nullptr, qweight, nullptr, out, KIND_BF16,
+                         x_rows, rows, num_experts, 1, in_features, out_features, 0, stream);
+}
+
+extern "C" int hipengine_gguf_q4_k_selected_dual_silu_gemv_bf16_bf16_out(
+    const uint16_t* x, const int64_t* selected, const uint8_t* qweight_a, const uint8_t* qweight_b, uint16_t* out,
+    int64_t x_rows, int64_t rows, int64_t num_experts, int64_t in_features, int64_t out_features, int64_t threads,
+    hipStream_t stream) {
+  (void)threads;
+  return launch_selected(GGML_Q4_K, SEL_DUAL_SILU, x, KIND_BF16, selected, nullptr, qweight_a, qweight_b, out,
+                         KIND_BF16, x_rows, rows, num_experts, 1, in_features, out_features, 1, stream);
+}
+
+extern "C" int hipengine_gfx950_gguf_selected_gemv(int32_t ggml_type, int32_t mode, const void* x, int32_t x_kind,
+                                                   const int64_t* selected, const float* routing_weights,
+                                                   const uint8_t* qweight_a, const uint8_t* qweight_b, void* out,
+                                                   int32_t out_kind, int64_t x_rows, int64_t lanes,
+                                                   int64_t num_experts, int64_t top_k, int64_t in_features,
+                                                   int64_t out_features, int32_t round_mid, hipStream_t stream) {
+  if (mode < SEL_SINGLE || mode > SEL_DOWN_SUM) return static_cast<int>(hipErrorInvalidValue);
+  return launch_selected(ggml_type, mode, x, x_kind, selected, routing_weights, qweight_a, qweight_b, out, out_kind,
+                         x_rows, lanes, num_experts, top_k, in_features, out_features, round_mid, stream);
+}
+
+// ---- prefill ----------------------------------------------------------------------
+
+extern "C" int hipengine_gguf_q4_k_selected_dual_q8_1_ds4_mmq32_prefill_compact32_bf16_bf16_out(
+    const void* x_q8, const int64_t* compact_to_source, const int64_t* expert_start_compact,
+    const int64_t* expert_start_mmq32, const int64_t* tile_expert, const uint8_t* qweight_a, const uint8_t* qweight_b,
+    uint16_t* out, int64_t compact_rows, int64_t in_features, int64_t out_features_a, int64_t out_features_b,
+    int64_t num_experts, int64_t mmq_total_rows, int64_t expert_stride_rows, hipStream_t stream) {
+  if (!compact_to_source) return static_cast<int>(hipErrorInvalidValue);
+  // As in hipEngine, the activation rows are addressed through compact_to_source only; the
+  // source row count is not part of this signature, so the clamp is the compact row count.
+  return launch_moe_mmq(x_q8, compact_to_source, expert_start_compact, expert_start_mmq32, tile_expert, qweight_a,
+                        qweight_b, out, KIND_BF16, compact_rows, compact_rows, in_features, out_features_a,
+                        out_features_b, num_experts, mmq_total_rows, expert_stride_rows, stream);
+}
+
+extern "C" int hipengine_gfx950_gguf_q4_k_grouped_mmq(const void* x_q8, const int64_t* compact_to_source,
+                                                      const int64_t* expert_start_compact,
+                                                      const int64_t* expert_start_mmq32, const int64_t* tile_expert,
+                                                      const uint8_t* qweight_a, const uint8_t* qweight_b, void* out,
+                                                      int32_t out_kind, int64_t compact_rows, int64_t source_rows,
+                                                      int64_t in_features, int64_t out_features_a,
+                                                      int64_t out_features_b, int64_t num_experts,
+                                                      int64_t mmq_total_rows, int64_t expert_stride_rows,
+                                                      hipStream_t stream) {
+  return launch_moe_mmq(x_q8, compact_to_source, expert_start_compact, expert_start_mmq32, tile_expert, qweight_a,
+                        qweight_b, out, out_kind, compact_rows, source_rows, in_features, out_features_a,
+                        out_features_b, num_experts, mmq_total_rows, expert_stride_rows, stream);
+}

@@ -1,0 +1,94 @@
+"""Routing index of the MoE path: expert-major compaction of the selected lanes
+and the 32-row tile map the grouped MMQ walks.
+
+Signatures follow hipEngine's ``kernels/hip_gfx1100/moe/group_scatter.py``
+(``qwen35_moe_group_compact_active`` :184-241, ``..._source_rows`` :243-308,
+``qwen35_moe_mmq32_tile_map`` :423-462); registry keys as in :746-806.
+All arguments are raw device pointers; int64 index arrays, float32 weights.
+"""
+
+from __future__ import annotations
+
+import ctypes
+
+from hipengine_amd.core.hip import HipRuntime
+from hipengine_amd.kernels.hip_gfx950._launch import I64, VOID, check_launch, entry, validate_pointers
+from hipengine_amd.kernels.registry import KernelKey, register
+
+MAX_EXPERTS = 2048
+
+
+def _check_num_experts(num_experts: int) -> None:
+    if num_experts <= 0 or num_experts > MAX_EXPERTS:
+        raise ValueError(f"num_experts must be in 1..{MAX_EXPERTS}")
+
+
+def qwen35_moe_group_compact_active(selected_experts_ptr: int, routing_weights_ptr: int, expert_start_ptr: int,
+                                    active_experts_ptr: int, active_count_ptr: int, sorted_lanes_ptr: int,
+                                    sorted_experts_ptr: int, sorted_weights_ptr: int, total_lanes: int,
+                                    num_experts: int, *, stream: int = 0, library: ctypes.CDLL | None = None,
+                                    runtime: HipRuntime | None = None) -> None:
+    """Expert-major compaction: starts, active list, lanes (ascending within an
+    expert), experts and weights in that order."""
+    _check_num_experts(num_experts)
+    if total_lanes <= 0:
+        raise ValueError("total_lanes must be positive")
+    validate_pointers(selected_experts_ptr=selected_experts_ptr, expert_start_ptr=expert_start_ptr,
+                      sorted_lanes_ptr=sorted_lanes_ptr)
+    fn = entry("hipengine_qwen35_moe_group_compact_active", [VOID] * 8 + [I64, I64, VOID], library)
+    check_launch(fn(selected_experts_ptr, routing_weights_ptr, expert_start_ptr, active_experts_ptr, active_count_ptr,
+                    sorted_lanes_ptr, sorted_experts_ptr, sorted_weights_ptr, total_lanes, num_experts, stream), runtime)
+
+
+def qwen35_moe_group_compact_active_source_rows(selected_experts_ptr: int, routing_weights_ptr: int,
+                                                expert_start_ptr: int, active_experts_ptr: int, active_count_ptr: int,
+                                                sorted_lanes_ptr: int, compact_to_source_ptr: int,
+                                                sorted_weights_ptr: int, total_lanes: int, num_experts: int,
+                                                top_k: int, *, parallel: bool = False, stream: int = 0,
+                                                library: ctypes.CDLL | None = None,
+                                                runtime: HipRuntime | None = None) -> None:
+    """The same with each compact row's source token (``lane // top_k``).
+    ``parallel`` is accepted for signature compatibility: there is one kernel form here."""
+    _check_num_experts(num_experts)
+    if total_lanes <= 0 or top_k <= 0:
+        raise ValueError("total_lanes and top_k must be positive")
+    validate_pointers(selected_experts_ptr=selected_experts_ptr, expert_start_ptr=expert_start_ptr,
+                      sorted_lanes_ptr=sorted_lanes_ptr)
+    fn = entry("hipengine_qwen35_moe_group_compact_active_source_rows", [VOID] * 8 + [I64, I64, I64, VOID], library)
+    check_launch(fn(selected_experts_ptr, routing_weights_ptr, expert_start_ptr, active_experts_ptr, active_count_ptr,
+                    sorted_lanes_ptr, compact_to_source_ptr, sorted_weights_ptr, total_lanes, num_experts, top_k,
+                    stream), runtime)
+
+
+def qwen35_moe_mmq32_tile_map(expert_start_compact_ptr: int, mmq_expert_start_ptr: int, tile_expert_ptr: int,
+                              mmq_total_ptr: int, num_experts: int, *, tile_capacity: int = 0, stream: int = 0,
+                              library: ctypes.CDLL | None = None, runtime: HipRuntime | None = None) -> None:
+    """Compact expert starts -> 32-row tile starts and the tile -> expert map."""
+    _check_num_experts(num_experts)
+    if tile_capacity < 0:
+        raise ValueError("tile_capacity must be non-negative")
+    validate_pointers(expert_start_compact_ptr=expert_start_compact_ptr, mmq_expert_start_ptr=mmq_expert_start_ptr,
+                      tile_expert_ptr=tile_expert_ptr, mmq_total_ptr=mmq_total_ptr)
+    fn = entry("hipengine_qwen35_moe_mmq32_tile_map", [VOID] * 4 + [I64, I64, VOID], library)
+    check_launch(fn(expert_start_compact_ptr, mmq_expert_start_ptr, tile_expert_ptr, mmq_total_ptr, num_experts,
+                    tile_capacity, stream), runtime)
+
+
+def moe_lane_to_compact(sorted_lanes_ptr: int, lane_to_compact_ptr: int, compact_rows: int, total_lanes: int, *,
+                        stream: int = 0, library: ctypes.CDLL | None = None,
+                        runtime: HipRuntime | None = None) -> None:
+    """Inverse of ``sorted_lanes`` (-1 for dropped lanes)."""
+    if compact_rows <= 0 or total_lanes <= 0:
+        raise ValueError("compact_rows and total_lanes must be positive")
+    validate_pointers(sorted_lanes_ptr=sorted_lanes_ptr, lane_to_compact_ptr=lane_to_compact_ptr)
+    fn = entry("hipengine_gfx950_moe_lane_to_compact", [VOID, VOID, I64, I64, VOID], library)
+    check_launch(fn(sorted_lanes_ptr, lane_to_compact_ptr, compact_rows, total_lanes, stream), runtime)
+
+
+def register_kernels(backend: str = "hip_gfx950", *, replace: bool = False) -> None:
+    register(KernelKey(backend, "moe_group_compact", "generic", "active_experts"), qwen35_moe_group_compact_active,
+             replace=replace)
+    register(KernelKey(backend, "moe_group_compact", "generic", "active_experts_source_rows"),
+             qwen35_moe_group_compact_active_source_rows, replace=replace)
+    register(KernelKey(backend, "moe_mmq_tile_map", "generic", "tile32"), qwen35_moe_mmq32_tile_map, replace=replace)
+    register(KernelKey(backend, "moe_lane_to_compact", "generic", "sorted_lanes"), moe_lane_to_compact, replace=replace)

@@ -203,6 +203,129 @@ int hipengine_gfx950_gguf_q4_k_mmq_tuned(const void* xq, const uint8_t* qweight,
                                          hipengine_stream_t stream);
 
 /* ------------------------------------------------------------------------
+ * MoE: routing index, expert-indexed decode GEMV, expert-grouped prefill MMQ
+ * Expert weights are [num_experts, out_features, row_bytes] raw blocks.
+ * A lane is one (token, slot) pair: lane = token * top_k + slot.
+ * num_experts <= 2048.
+ * ------------------------------------------------------------------------ */
+
+/* selected_experts[total_lanes] -> expert-major order.  expert_start[num_experts+1]
+ * (exclusive prefix of the per-expert lane counts), active_experts (ascending ids
+ * of experts with at least one lane; may be NULL) and active_count[1] (may be NULL),
+ * sorted_lanes[total_lanes] (ascending lane within an expert), sorted_experts (may
+ * be NULL), sorted_weights (may be NULL).  Expert ids outside [0, num_experts) are
+ * dropped.  Replaces moe/group_scatter.hip:760-797 (kernel :85-141). */
+int hipengine_qwen35_moe_group_compact_active(const int64_t* selected_experts, const float* routing_weights,
+                                              int64_t* expert_start, int64_t* active_experts, int64_t* active_count,
+                                              int64_t* sorted_lanes, int64_t* sorted_experts, float* sorted_weights,
+                                              int64_t total_lanes, int64_t num_experts, hipengine_stream_t stream);
+
+/* The same with compact_to_source[i] = sorted_lanes[i] / top_k instead of
+ * sorted_experts.  Replaces moe/group_scatter.hip:799-836. */
+int hipengine_qwen35_moe_group_compact_active_source_rows(const int64_t* selected_experts,
+                                                          const float* routing_weights, int64_t* expert_start,
+                                                          int64_t* active_experts, int64_t* active_count,
+                                                          int64_t* sorted_lanes, int64_t* compact_to_source,
+                                                          float* sorted_weights, int64_t total_lanes,
+                                                          int64_t num_experts, int64_t top_k,
+                                                          hipengine_stream_t stream);
+
+/* expert_start_compact[num_experts+1] -> mmq_expert_start[num_experts+1] (row
+ * starts with every expert's count rounded up to 32), tile_expert[tile] (expert
+ * of each 32-row tile; the first tile_capacity entries are preset to -1 when
+ * tile_capacity > 0 and tiles beyond it are not written), mmq_total_out[1].
+ * Replaces moe/group_scatter.hip:1023-1052 (kernel :328-389). */
+int hipengine_qwen35_moe_mmq32_tile_map(const int64_t* expert_start_compact, int64_t* mmq_expert_start,
+                                        int64_t* tile_expert, int64_t* mmq_total_out, int64_t num_experts,
+                                        int64_t tile_capacity, hipengine_stream_t stream);
+
+/* lane_to_compact[total_lanes]: position of each lane in sorted_lanes, -1 for a
+ * dropped lane.  New here (hipEngine scatters with atomics instead,
+ * moe/group_scatter.hip:391-417; this inverse keeps the weighted sum ordered). */
+int hipengine_gfx950_moe_lane_to_compact(const int64_t* sorted_lanes, int64_t* lane_to_compact, int64_t compact_rows,
+                                         int64_t total_lanes, hipengine_stream_t stream);
+
+/* gate_up[rows, 2*inter] (gate columns first) -> out[rows, inter] = gate*sigmoid(gate)*up.
+ * Kinds: 0 float32, 1 bf16, 2 fp16.  The step between the gate/up and the down
+ * projection (fused/paro_silu silu_mul_separate_out_bf16 in hipEngine). */
+int hipengine_gfx950_moe_silu_mul(const void* gate_up, void* out, int64_t rows, int64_t inter, int in_kind,
+                                  int out_kind, hipengine_stream_t stream);
+
+/* out[t, h] = sum over slots s = 0..top_k-1, in that order, of
+ * routing_weights[t*top_k+s] * down[lane_to_compact[t*top_k+s], h]; lanes mapped
+ * to -1 are skipped.  tokens <= 65535.  New here (see lane_to_compact). */
+int hipengine_gfx950_moe_weighted_gather_sum(const void* down, const int64_t* lane_to_compact,
+                                             const float* routing_weights, void* out, int64_t tokens, int64_t top_k,
+                                             int64_t hidden, int64_t compact_rows, int in_kind, int out_kind,
+                                             hipengine_stream_t stream);
+
+/* Decode: out[lane, :] = W[selected[lane]] . x[lane / (rows / x_rows), :] for
+ * rows lanes (<= 65535) over x_rows activation rows; lanes with an expert id
+ * outside [0, num_experts) are left unwritten.  Activations are quantized to
+ * q8_1 in the kernel.  `threads` is accepted and ignored.
+ * Replaces gguf_q4_k_gemv.hip selected GEMV export (kernel :322-359; Python
+ * gguf_q4_k_gemv.py:667-715,1403). */
+int hipengine_gguf_q4_k_selected_gemv_bf16_bf16_out(const uint16_t* x, const int64_t* selected,
+                                                    const uint8_t* qweight, uint16_t* out, int64_t x_rows,
+                                                    int64_t rows, int64_t num_experts, int64_t in_features,
+                                                    int64_t out_features, int64_t threads,
+                                                    hipengine_stream_t stream);
+
+/* Decode gate/up pair: out[lane, n] = silu(bf16(gate)) * bf16(up), gate and up
+ * rounded to bf16 before the activation as in gguf_q4_k_gemv.hip:732-736.
+ * Replaces gguf_q4_k_gemv.hip:2751-2767. */
+int hipengine_gguf_q4_k_selected_dual_silu_gemv_bf16_bf16_out(const uint16_t* x, const int64_t* selected,
+                                                              const uint8_t* qweight_a, const uint8_t* qweight_b,
+                                                              uint16_t* out, int64_t x_rows, int64_t rows,
+                                                              int64_t num_experts, int64_t in_features,
+                                                              int64_t out_features, int64_t threads,
+                                                              hipengine_stream_t stream);
+
+/* The decode kernels with every choice explicit.  ggml_type 12 (Q4_K) or 14 (Q6_K).
+ *   mode 0: out[lanes, N] = W_a[selected[lane]] . x[lane / (lanes/x_rows)]
+ *   mode 1: out[lanes, N] = silu(gate) * up with W_a = gate, W_b = up; round_mid != 0
+ *           rounds gate and up to the output type first
+ *   mode 2: x is [lanes, K] (one row per lane, lanes = x_rows * top_k); out[x_rows, N]
+ *           = sum over the token's slots, in slot order, of routing_weights[lane] *
+ *           (W_a[selected[lane]] . x[lane]); invalid experts are skipped
+ * Kinds: 0 float32, 1 bf16, 2 fp16.  New here. */
+int hipengine_gfx950_gguf_selected_gemv(int32_t ggml_type, int32_t mode, const void* x, int32_t x_kind,
+                                        const int64_t* selected, const float* routing_weights,
+                                        const uint8_t* qweight_a, const uint8_t* qweight_b, void* out,
+                                        int32_t out_kind, int64_t x_rows, int64_t lanes, int64_t num_experts,
+                                        int64_t top_k, int64_t in_features, int64_t out_features, int32_t round_mid,
+                                        hipengine_stream_t stream);
+
+/* Prefill: for every 32-row tile t with expert e = tile_expert[t] >= 0, the rows
+ * r = expert_start_compact[e] + (32*t - expert_start_mmq32[e]) + 0..31 that lie
+ * below expert_start_compact[e+1] get
+ *   out[r, 0:Na]     = W_a[e] . x[compact_to_source[r]]
+ *   out[r, Na:Na+Nb] = W_b[e] . x[compact_to_source[r]]
+ * with x_q8 the DS4 blocks of the source rows.  expert_stride_rows is the
+ * distance between experts in rows (0: the half's own width).  Na, Nb multiples
+ * of 32, mmq_total_rows a multiple of 32 with at most 65535 tiles.
+ * Replaces gguf_q4_k_q8_1_selected_prefill.hip:7426-7461 (body :1256-1670). */
+int hipengine_gguf_q4_k_selected_dual_q8_1_ds4_mmq32_prefill_compact32_bf16_bf16_out(
+    const void* x_q8, const int64_t* compact_to_source, const int64_t* expert_start_compact,
+    const int64_t* expert_start_mmq32, const int64_t* tile_expert, const uint8_t* qweight_a,
+    const uint8_t* qweight_b, uint16_t* out, int64_t compact_rows, int64_t in_features, int64_t out_features_a,
+    int64_t out_features_b, int64_t num_experts, int64_t mmq_total_rows, int64_t expert_stride_rows,
+    hipengine_stream_t stream);
+
+/* The same with the output kind explicit (0 float32, 1 bf16, 2 fp16), the source
+ * row count given (indices are clamped to it), compact_to_source optional (NULL:
+ * compact row r reads source row r) and the second weight optional
+ * (out_features_b = 0).  New here. */
+int hipengine_gfx950_gguf_q4_k_grouped_mmq(const void* x_q8, const int64_t* compact_to_source,
+                                           const int64_t* expert_start_compact, const int64_t* expert_start_mmq32,
+                                           const int64_t* tile_expert, const uint8_t* qweight_a,
+                                           const uint8_t* qweight_b, void* out, int32_t out_kind,
+                                           int64_t compact_rows, int64_t source_rows, int64_t in_features,
+                                           int64_t out_features_a, int64_t out_features_b, int64_t num_experts,
+                                           int64_t mmq_total_rows, int64_t expert_stride_rows,
+                                           hipengine_stream_t stream);
+
+/* ------------------------------------------------------------------------
  * Verification exports: the integer unpack and the int32 sub-block dots the
  * production kernels compute, written out so that they can be compared bit for
  * bit with a CPU oracle.  New here.

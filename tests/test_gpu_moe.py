@@ -1,0 +1,328 @@
+"""GPU parity of the MoE forms through the C ABI: routing index and tile map
+(integer, bit-exact against the oracle), the expert-indexed decode GEMV family
+and the expert-grouped Q4_K x DS4 MMQ (float32 within max relative error 1e-3 /
+cosine 0.99999 of the reference CPU arithmetic on the same quantized
+activations), and the whole selected-expert FFN against the reference CPU MoE
+(hipengine/kernels/cpu_reference/ops.py:624-678 as restated by the oracle).
+
+The full-chain comparison is against UNQUANTIZED activations, so its gate is the
+looser end-to-end one the reference uses for q8_1 paths (cosine, rtol 2e-2;
+tests/test_gpu_gguf_q4_k_q8_1_mmq_prefill.py:343-357); the per-stage tests
+carry the 1e-3 gate.
+"""
+
+from __future__ import annotations
+
+import numpy as np
+import pytest
+
+from oracle import gguf_oracle as O
+from hipengine_amd.kernels.hip_gfx950.moe import group_scatter as GS
+from hipengine_amd.kernels.hip_gfx950.quant import gguf_moe as M
+from hipengine_amd.kernels.hip_gfx950.quant import gguf_quantize as Q
+
+pytestmark = pytest.mark.gpu
+
+REL_TOL = 1e-3
+COS_MIN = 0.99999
+
+
+def _routing(seed, tokens, top_k, num_experts, bad=False):
+    rng = np.random.default_rng(seed)
+    sel = np.stack([rng.permutation(num_experts)[:top_k] for _ in range(tokens)]).astype(np.int64)
+    w = rng.random((tokens, top_k)).astype(np.float32)
+    w /= w.sum(axis=1, keepdims=True)
+    if bad and tokens > 2:
+        sel[1, 0] = -1
+        sel[2, top_k - 1] = num_experts + 3
+    return sel, w
+
+
+def _device_index(dev, sel, w, num_experts, tile_capacity=0):
+    """Runs compact_active_source_rows + mmq32_tile_map + lane_to_compact; returns host copies and device buffers."""
+    tokens, top_k = sel.shape
+    lanes = tokens * top_k
+    d = {
+        "sel": dev.put(sel), "w": dev.put(w),
+        "expert_start": dev.empty((num_experts + 1) * 8), "active": dev.empty(num_experts * 8, fill=0xFF),
+        "active_count": dev.empty(8), "sorted_lanes": dev.empty(lanes * 8, fill=0xFF),
+        "c2s": dev.empty(lanes * 8, fill=0xFF), "sorted_w": dev.empty(lanes * 4, fill=0),
+    }
+    GS.qwen35_moe_group_compact_active_source_rows(d["sel"].ptr, d["w"].ptr, d["expert_start"].ptr, d["active"].ptr,
+                                                   d["active_count"].ptr, d["sorted_lanes"].ptr, d["c2s"].ptr,
+                                                   d["sorted_w"].ptr, lanes, num_experts, top_k)
+    host = {
+        "expert_start": dev.get(d["expert_start"], np.int64, (num_experts + 1,)),
+        "active": dev.get(d["active"], np.int64, (num_experts,)),
+        "active_count": int(dev.get(d["active_count"], np.int64, (1,))[0]),
+        "sorted_lanes": dev.get(d["sorted_lanes"], np.int64, (lanes,)),
+        "c2s": dev.get(d["c2s"], np.int64, (lanes,)),
+        "sorted_w": dev.get(d["sorted_w"], np.float32, (lanes,)),
+    }
+    total = int(host["expert_start"][-1])
+    max_tiles = (lanes + 31) // 32 + num_experts
+    cap = tile_capacity or max_tiles
+    d["mmq_start"] = dev.empty((num_experts + 1) * 8)
+    d["tile_expert"] = dev.empty(cap * 8, fill=0x11)
+    d["mmq_total"] = dev.empty(8)
+    GS.qwen35_moe_mmq32_tile_map(d["expert_start"].ptr, d["mmq_start"].ptr, d["tile_expert"].ptr, d["mmq_total"].ptr,
+                                 num_experts, tile_capacity=cap)
+    host["mmq_start"] = dev.get(d["mmq_start"], np.int64, (num_experts + 1,))
+    host["tile_expert"] = dev.get(d["tile_expert"], np.int64, (cap,))
+    host["mmq_total"] = int(dev.get(d["mmq_total"], np.int64, (1,))[0])
+    d["l2c"] = dev.empty(lanes * 8, fill=0x22)
+    if total > 0:
+        GS.moe_lane_to_compact(d["sorted_lanes"].ptr, d["l2c"].ptr, total, lanes)
+        host["l2c"] = dev.get(d["l2c"], np.int64, (lanes,))
+    host["total"] = total
+    return host, d
+
+
+@pytest.mark.parametrize("tokens,top_k,experts,bad", [(1, 8, 256, False), (8, 8, 256, True), (300, 4, 64, True),
+                                                      (2048, 8, 256, False), (77, 2, 5, True)])
+def test_routing_index_and_tile_map_bit_exact(dev, tokens, top_k, experts, bad):
+    sel, w = _routing(tokens + experts, tokens, top_k, experts, bad)
+    host, d = _device_index(dev, sel, w, experts)
+    want = O.build_routing_index(sel, w, experts)
+    total = want["total"]
+    assert host["total"] == total
+    assert np.array_equal(host["expert_start"], want["expert_start"])
+    assert host["active_count"] == want["active_count"]
+    assert np.array_equal(host["active"][:want["active_count"]], want["active_experts"])
+    assert np.array_equal(host["sorted_lanes"][:total], want["sorted_lanes"])
+    assert np.array_equal(host["c2s"][:total], want["compact_to_source"])
+    assert np.array_equal(host["sorted_w"][:total].view(np.uint32), want["sorted_weights"].view(np.uint32))
+    tm = O.tile_map(want["expert_start"], experts, 32, tile_capacity=host["tile_expert"].size)
+    assert np.array_equal(host["mmq_start"], tm["tile_expert_start"])
+    assert host["mmq_total"] == tm["total"]
+    assert np.array_equal(host["tile_expert"], tm["tile_expert"])
+    inv = np.full(tokens * top_k, -1, dtype=np.int64)
+    inv[want["sorted_lanes"]] = np.arange(total)
+    assert np.array_equal(host["l2c"], inv)
+    dev.free(*d.values())
+
+
+def _experts(qt, num_experts, n, k, seed):
+    return O.stack_experts(O.random_weight(qt, n, k, seed=seed), num_experts, seed=seed % 7)
+
+
+def _ref_lane(x_row, w_e, qt):
+    """Reference CPU GEMV (dequantize -> float32 matmul) on the q8_1-dequantized activations."""
+    xq = O.quantize_q8_1(x_row[None, :])
+    return O.gguf_quant_gemv(O.dequantize_q8_1(xq), w_e, qt)[0]
+
+
+@pytest.mark.parametrize("quant,qt", [("gguf_q4_k", O.GGML_Q4_K), ("gguf_q6_k", O.GGML_Q6_K)])
+@pytest.mark.parametrize("tokens,top_k,experts,k,n", [(1, 8, 16, 2048, 512), (3, 4, 8, 512, 2048), (5, 2, 6, 1280, 80)])
+def test_selected_gemv_single(dev, quant, qt, tokens, top_k, experts, k, n):
+    sel, _ = _routing(k + n, tokens, top_k, experts)
+    if tokens > 1:
+        sel[1, 0] = -1                                   # an invalid lane stays unwritten
+    w = _experts(qt, experts, n, k, seed=3)
+    x = np.random.default_rng(9).standard_normal((tokens, k)).astype(np.float32)
+    lanes = tokens * top_k
+    dx, dsel, dw = dev.put(x), dev.put(sel), dev.put(w)
+    dout = dev.empty(lanes * n * 4, fill=0x7F)
+    M.gguf_selected_gemv(quant, M.SEL_SINGLE, dx.ptr, dsel.ptr, dw.ptr, dout.ptr, tokens, lanes, experts, k, n)
+    got = dev.get(dout, np.float32, (lanes, n))
+    dev.free(dx, dsel, dw, dout)
+    sentinel = np.frombuffer(b"\x7f\x7f\x7f\x7f", dtype=np.uint32)[0]
+    for lane in range(lanes):
+        e = int(sel.reshape(-1)[lane])
+        if e < 0:
+            assert np.all(got[lane].view(np.uint32) == sentinel)
+            continue
+        ref = _ref_lane(x[lane // top_k], w[e], qt)
+        assert O.max_rel_err(got[lane], ref) <= REL_TOL and O.cosine(got[lane], ref) >= COS_MIN
+
+
+def test_selected_gemv_bf16_entry_points(dev):
+    tokens, top_k, experts, k, n = 2, 8, 12, 2048, 512
+    sel, _ = _routing(4, tokens, top_k, experts)
+    wg, wu = _experts(O.GGML_Q4_K, experts, n, k, seed=5), _experts(O.GGML_Q4_K, experts, n, k, seed=6)
+    x = (np.random.default_rng(2).standard_normal((tokens, k)) * 0.5).astype(np.float32)
+    xb = O.f32_to_bf16_bits(x)
+    xf = O.bf16_bits_to_f32(xb)
+    lanes = tokens * top_k
+    dx, dsel, dg, du = dev.put(xb), dev.put(sel), dev.put(wg), dev.put(wu)
+    dout = dev.empty(lanes * n * 2)
+    M.gguf_q4_k_selected_gemv_bf16_bf16_out(dx.ptr, dsel.ptr, dg.ptr, dout.ptr, tokens, lanes, experts, k, n)
+    single = O.bf16_bits_to_f32(dev.get(dout, np.uint16, (lanes, n)))
+    M.gguf_q4_k_selected_dual_silu_gemv_bf16_bf16_out(dx.ptr, dsel.ptr, dg.ptr, du.ptr, dout.ptr, tokens, lanes,
+                                                      experts, k, n)
+    dual = O.bf16_bits_to_f32(dev.get(dout, np.uint16, (lanes, n)))
+    dev.free(dx, dsel, dg, du, dout)
+    for lane in range(lanes):
+        e = int(sel.reshape(-1)[lane])
+        g = _ref_lane(xf[lane // top_k], wg[e], O.GGML_Q4_K)
+        u = _ref_lane(xf[lane // top_k], wu[e], O.GGML_Q4_K)
+        # bf16 outputs: half a bf16 ulp (2^-9) on top of the float32 gate
+        assert O.max_rel_err(single[lane], g, floor_frac=1e-2) <= 6e-3
+        gb = O.bf16_bits_to_f32(O.f32_to_bf16_bits(g))
+        ub = O.bf16_bits_to_f32(O.f32_to_bf16_bits(u))
+        want = (O.silu(gb) * ub).astype(np.float32)
+        assert O.cosine(dual[lane], want) >= 0.9999
+        assert O.max_rel_err(dual[lane], want, floor_frac=2e-2) <= 2e-2
+
+
+@pytest.mark.parametrize("tokens", [1, 8])
+def test_decode_chain_matches_cpu_moe(dev, tokens):
+    """dual SiLU GEMV -> routed down sum (two launches) against the reference CPU MoE FFN."""
+    top_k, experts, hidden, inter = 8, 32, 2048, 512
+    sel, wts = _routing(tokens, tokens, top_k, experts)
+    wg = _experts(O.GGML_Q4_K, experts, inter, hidden, seed=1)
+    wu = _experts(O.GGML_Q4_K, experts, inter, hidden, seed=2)
+    wd = _experts(O.GGML_Q4_K, experts, hidden, inter, seed=3)
+    x = (np.random.default_rng(tokens).standard_normal((tokens, hidden)) * 0.3).astype(np.float32)
+    lanes = tokens * top_k
+    dx, dsel, dwt = dev.put(x), dev.put(sel), dev.put(wts)
+    dg, du, dd = dev.put(wg), dev.put(wu), dev.put(wd)
+    dmid, dout = dev.empty(lanes * inter * 4), dev.empty(tokens * hidden * 4)
+    M.gguf_selected_gemv("gguf_q4_k", M.SEL_DUAL_SILU, dx.ptr, dsel.ptr, dg.ptr, dmid.ptr, tokens, lanes, experts,
+                         hidden, inter, qweight_b_ptr=du.ptr)
+    M.gguf_selected_gemv("gguf_q4_k", M.SEL_DOWN_SUM, dmid.ptr, dsel.ptr, dd.ptr, dout.ptr, tokens, lanes, experts,
+                         inter, hidden, routing_weights_ptr=dwt.ptr, top_k=top_k)
+    mid = dev.get(dmid, np.float32, (lanes, inter))
+    got = dev.get(dout, np.float32, (tokens, hidden))
+    dev.free(dx, dsel, dwt, dg, du, dd, dmid, dout)
+    # stage gates: each stage against the reference arithmetic on the same quantized inputs
+    want = np.zeros((tokens, hidden), dtype=np.float32)
+    for lane in range(lanes):
+        t, e = lane // top_k, int(sel.reshape(-1)[lane])
+        g, u = _ref_lane(x[t], wg[e], O.GGML_Q4_K), _ref_lane(x[t], wu[e], O.GGML_Q4_K)
+        ref_mid = (O.silu(g) * u).astype(np.float32)
+        assert O.max_rel_err(mid[lane], ref_mid) <= REL_TOL and O.cosine(mid[lane], ref_mid) >= COS_MIN
+        want[t] += wts.reshape(-1)[lane] * _ref_lane(mid[lane], wd[e], O.GGML_Q4_K)
+    assert O.max_rel_err(got, want) <= REL_TOL and O.cosine(got, want) >= COS_MIN
+    # end to end against the reference CPU MoE on unquantized activations
+    ref = O.moe_selected_ffn(x, sel, wts, wg, wu, wd)
+    assert O.cosine(got, ref) >= 0.9995
+    np.testing.assert_allclose(got, ref, rtol=2e-2, atol=2e-2 * np.abs(ref).max())
+
+
+def _grouped(dev, host, d, ds4, w_a, w_b, rows_src, k, na, nb, experts, identity=False, out_dtype="f32"):
+    total = host["total"]
+    dxq, dwa = dev.put(ds4), dev.put(w_a)
+    dwb = dev.put(w_b) if w_b is not None else None
+    item = 4 if out_dtype == "f32" else 2
+    dout = dev.empty(total * (na + nb) * item, fill=0)
+    M.gguf_q4_k_grouped_mmq(dxq.ptr, d["expert_start"].ptr, d["mmq_start"].ptr, d["tile_expert"].ptr, dwa.ptr, dout.ptr,
+                            total, rows_src, k, na, experts, host["mmq_total"],
+                            compact_to_source_ptr=0 if identity else d["c2s"].ptr,
+                            qweight_b_ptr=dwb.ptr if dwb else 0, out_features_b=nb, out_dtype=out_dtype)
+    got = dev.get(dout, np.float32 if out_dtype == "f32" else np.uint16, (total, na + nb))
+    dev.free(dxq, dwa, dout, *([dwb] if dwb else []))
+    return got
+
+
+@pytest.mark.parametrize("tokens,top_k,experts,k,na,nb", [(40, 4, 8, 512, 96, 64), (150, 8, 16, 2048, 512, 512),
+                                                          (9, 2, 40, 768, 288, 0)])
+def test_grouped_mmq_matches_dense_formula_per_expert(dev, tokens, top_k, experts, k, na, nb):
+    sel, wts = _routing(tokens * 3 + k, tokens, top_k, experts, bad=tokens > 20)
+    host, d = _device_index(dev, sel, wts, experts)
+    x = (np.random.default_rng(k).standard_normal((tokens, k)) * 0.2).astype(np.float32)
+    ds4 = O.pack_q8_1_ds4(O.f32_to_bf16_bits(x))
+    w_a = _experts(O.GGML_Q4_K, experts, na, k, seed=11)
+    w_b = _experts(O.GGML_Q4_K, experts, nb, k, seed=12) if nb else None
+    got = _grouped(dev, host, d, ds4, w_a, w_b, tokens, k, na, nb, experts)
+    es = host["expert_start"]
+    for e in range(experts):
+        lo, hi = int(es[e]), int(es[e + 1])
+        if hi == lo:
+            continue
+        src = host["c2s"][lo:hi]
+        want_a = O.mmq_q4_k_ds4(ds4[src], w_a[e])
+        assert O.max_rel_err(got[lo:hi, :na], want_a) <= REL_TOL and O.cosine(got[lo:hi, :na], want_a) >= COS_MIN
+        if nb:
+            want_b = O.mmq_q4_k_ds4(ds4[src], w_b[e])
+            assert O.max_rel_err(got[lo:hi, na:], want_b) <= REL_TOL and O.cosine(got[lo:hi, na:], want_b) >= COS_MIN
+    dev.free(*d.values())
+
+
+def test_grouped_mmq_bf16_named_entry(dev):
+    tokens, top_k, experts, k, na, nb = 64, 4, 8, 1024, 128, 128
+    sel, wts = _routing(31, tokens, top_k, experts)
+    host, d = _device_index(dev, sel, wts, experts)
+    x = (np.random.default_rng(1).standard_normal((tokens, k)) * 0.2).astype(np.float32)
+    ds4 = O.pack_q8_1_ds4(O.f32_to_bf16_bits(x))
+    w_a, w_b = _experts(O.GGML_Q4_K, experts, na, k, seed=21), _experts(O.GGML_Q4_K, experts, nb, k, seed=22)
+    f32 = _grouped(dev, host, d, ds4, w_a, w_b, tokens, k, na, nb, experts)
+    total = host["total"]
+    dxq, dwa, dwb = dev.put(ds4), dev.put(w_a), dev.put(w_b)
+    dout = dev.empty(total * (na + nb) * 2, fill=0)
+    M.gguf_q4_k_selected_dual_q8_1_ds4_mmq32_prefill_compact32_bf16_bf16_out(
+        dxq.ptr, d["c2s"].ptr, d["expert_start"].ptr, d["mmq_start"].ptr, d["tile_expert"].ptr, dwa.ptr, dwb.ptr,
+        dout.ptr, total, k, na, nb, experts, host["mmq_total"])
+    b16 = dev.get(dout, np.uint16, (total, na + nb))
+    dev.free(dxq, dwa, dwb, dout, *d.values())
+    assert np.array_equal(b16, O.f32_to_bf16_bits(f32))
+
+
+def test_prefill_chain_matches_cpu_moe(dev):
+    """index -> DS4 pack -> grouped gate|up MMQ -> SiLU*up -> DS4 pack -> grouped down MMQ ->
+    ordered weighted gather, against the reference CPU MoE FFN on a token subsample."""
+    tokens, top_k, experts, hidden, inter = 256, 8, 32, 2048, 512
+    sel, wts = _routing(77, tokens, top_k, experts)
+    host, d = _device_index(dev, sel, wts, experts)
+    total, lanes = host["total"], tokens * top_k
+    wg = _experts(O.GGML_Q4_K, experts, inter, hidden, seed=1)
+    wu = _experts(O.GGML_Q4_K, experts, inter, hidden, seed=2)
+    wd = _experts(O.GGML_Q4_K, experts, hidden, inter, seed=3)
+    x = (np.random.default_rng(8).standard_normal((tokens, hidden)) * 0.3).astype(np.float32)
+    xb = O.f32_to_bf16_bits(x)
+    dxb, dg, du, dd = dev.put(xb), dev.put(wg), dev.put(wu), dev.put(wd)
+    dxq = dev.empty(tokens * (hidden // 128) * 144)
+    Q.gguf_q8_1_mmq_ds4_pack_bf16(dxb.ptr, dxq.ptr, tokens, hidden)
+    dgu = dev.empty(total * 2 * inter * 4)
+    M.gguf_q4_k_grouped_mmq(dxq.ptr, d["expert_start"].ptr, d["mmq_start"].ptr, d["tile_expert"].ptr, dg.ptr, dgu.ptr,
+                            total, tokens, hidden, inter, experts, host["mmq_total"], compact_to_source_ptr=d["c2s"].ptr,
+                            qweight_b_ptr=du.ptr, out_features_b=inter)
+    dmid = dev.empty(total * inter * 2)
+    M.moe_silu_mul(dgu.ptr, dmid.ptr, total, inter, in_dtype="f32", out_dtype="bf16")
+    dmq = dev.empty(total * (inter // 128) * 144)
+    Q.gguf_q8_1_mmq_ds4_pack_bf16(dmid.ptr, dmq.ptr, total, inter)
+    ddown = dev.empty(total * hidden * 4)
+    M.gguf_q4_k_grouped_mmq(dmq.ptr, d["expert_start"].ptr, d["mmq_start"].ptr, d["tile_expert"].ptr, dd.ptr, ddown.ptr,
+                            total, total, inter, hidden, experts, host["mmq_total"])
+    dout = dev.empty(tokens * hidden * 4)
+    M.moe_weighted_gather_sum(ddown.ptr, d["l2c"].ptr, d["w"].ptr, dout.ptr, tokens, top_k, hidden, total)
+    got = dev.get(dout, np.float32, (tokens, hidden))
+    gu = dev.get(dgu, np.float32, (total, 2 * inter))
+    mid_bits = dev.get(dmid, np.uint16, (total, inter))
+    mid = O.bf16_bits_to_f32(mid_bits)
+    down = dev.get(ddown, np.float32, (total, hidden))
+    dev.free(dxb, dg, du, dd, dxq, dgu, dmid, dmq, ddown, dout, *d.values())
+    # elementwise stage: bf16(silu(gate)*up) of the device's own gate|up
+    want_mid = O.bf16_bits_to_f32(O.f32_to_bf16_bits((O.silu(gu[:, :inter]) * gu[:, inter:]).astype(np.float32)))
+    assert O.max_rel_err(mid, want_mid, floor_frac=1e-2) <= 1e-2
+    # down stage: the MMQ formula on the device's own intermediate, expert by expert
+    mid_ds4 = O.pack_q8_1_ds4(mid_bits)
+    es = host["expert_start"]
+    for e in range(0, experts, 5):
+        lo, hi = int(es[e]), int(es[e + 1])
+        if hi > lo:
+            want_down = O.mmq_q4_k_ds4(mid_ds4[lo:hi], wd[e])
+            assert O.max_rel_err(down[lo:hi], want_down) <= REL_TOL and O.cosine(down[lo:hi], want_down) >= COS_MIN
+    # ordered weighted gather of the device's own down rows
+    want_out = np.zeros((tokens, hidden), dtype=np.float64)
+    for lane in range(lanes):
+        want_out[lane // top_k] += np.float64(wts.reshape(-1)[lane]) * down[host["l2c"][lane]]
+    assert O.max_rel_err(got, want_out.astype(np.float32), floor_frac=1e-3) <= 1e-4
+    # end to end on a token subsample (the CPU MoE is a Python loop over tokens x slots)
+    pick = np.arange(0, tokens, 16)
+    # (two q8_1 quantizations and a bf16 intermediate separate the two: ~0.4% noise per stage)
+    ref = O.moe_selected_ffn(O.bf16_bits_to_f32(xb)[pick], sel[pick], wts[pick], wg, wu, wd)
+    assert O.cosine(got[pick], ref) >= 0.999
+    np.testing.assert_allclose(got[pick], ref, rtol=2e-2, atol=5e-2 * np.abs(ref).max())
+    assert np.all(np.isfinite(got))
+
+
+def test_moe_wrappers_reject_bad_arguments(dev):
+    with pytest.raises(ValueError, match="num_experts"):
+        GS.qwen35_moe_mmq32_tile_map(1, 1, 1, 1, 0)
+    with pytest.raises(ValueError, match="multiple of x_rows"):
+        M.gguf_q4_k_selected_gemv_bf16_bf16_out(1, 1, 1, 1, 3, 8, 4, 256, 32)
+    with pytest.raises(ValueError, match="divisible"):
+        M.gguf_q4_k_selected_gemv_bf16_bf16_out(1, 1, 1, 1, 1, 8, 4, 200, 32)
+    with pytest.raises(ValueError, match="multiples of 32"):
+        M.gguf_q4_k_grouped_mmq(1, 1, 1, 1, 1, 1, 8, 8, 256, 40, 4, 32)
