@@ -1,7 +1,7 @@
 #!/usr/bin/env python3
 """Benchmark of the gfx950 GGUF k-quant matmul path on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-extra] [--no-cpu]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-extra] [--no-cpu] [--pmc-pass]
 
 One "step" is one pass of the hot path over one batch of synthetic input: the
 fused q8_1 decode GEMV of a Q4_K 17408x5120 weight at batch 1 (the shape the
@@ -12,6 +12,10 @@ region is bracketed by device synchronisations and, for the roofline figure,
 by HIP events recorded on the launch stream.
 
 Prints ONE JSON line.  `value` is algorithmic bytes per step / time per step.
+`extra` carries the other configurations of the path: decode GEMV shapes, the
+MMQ prefill GEMM (int8 TOPS), and the MoE decode / prefill chains.
+`--pmc-pass` launches only a 256 MiB calibration copy and the headline kernel,
+for hardware-counter runs (FETCH_SIZE / WRITE_SIZE) under rocprofv3 --pmc.
 The host side is torch-free (ctypes HIP binding).
 """
 
@@ -36,6 +40,19 @@ METRIC = "Q4_K decode GEMV GB/s (% HBM peak); MMQ prefill int8 TOPS (% MFMA peak
 GGML = {"q8_0": 8, "q4_k": 12, "q6_k": 14}
 BLOCK = {"q8_0": (32, 34), "q4_k": (256, 144), "q6_k": (256, 210)}
 MALL_BYTES = 256 << 20
+TRAFFIC_FILE = ROOT / "profiles" / "gemv_stream_q4k_17408x5120_b1_pmc.md"
+
+
+def measured_traffic() -> int | None:
+    """HBM bytes per launch of the headline kernel as derived from the committed
+    hardware-counter summary (a line `traffic_bytes_per_launch: N`), else None."""
+    try:
+        for line in TRAFFIC_FILE.read_text().splitlines():
+            if line.strip().startswith("traffic_bytes_per_launch:"):
+                return int(float(line.split(":", 1)[1].strip()))
+    except OSError:
+        pass
+    return None
 
 
 def gemv_bytes(quant: str, rows: int, k: int, n: int, act_bytes: int = 4) -> int:
@@ -93,6 +110,104 @@ class Harness:
                 "weight_host": w, "x_host": x}
 
 
+    def mmq_case(self, quant: str, m: int, k: int, n: int, steps: int, warmup: int):
+        """MMQ prefill GEMM on pre-packed activations: (seconds per launch, int8 ops per launch)."""
+        from hipengine_amd.kernels.hip_gfx950.quant import gguf_mmq_prefill as M
+        from hipengine_amd.kernels.hip_gfx950.quant import gguf_quantize as Q
+        from hipengine_amd.synthetic import synthetic_blocks
+
+        w = synthetic_blocks(GGML[quant], n, k, seed=3)
+        x = np.random.default_rng(4).standard_normal((m, k)).astype(np.float32)
+        xb = (x.view(np.uint32) >> 16).astype(np.uint16)
+        dw, dx = self.memory.to_device(w, runtime=self.rt), self.memory.to_device(xb, runtime=self.rt)
+        block_bytes = 144 if quant == "q4_k" else 160
+        dxq = self.memory.malloc(m * (k // 128) * block_bytes, runtime=self.rt)
+        dout = self.memory.malloc(m * n * 4, runtime=self.rt)
+        if quant == "q4_k":
+            Q.gguf_q8_1_mmq_ds4_pack_bf16(dx.ptr, dxq.ptr, m, k)
+            fn = M.gguf_q4_k_q8_1_mmq32_vdr_dense_bf16_f32_out
+        else:
+            Q.gguf_q8_1_d4s4_f32_quantize_bf16(dx.ptr, dxq.ptr, m, k)
+            fn = M.gguf_q6_k_mmq32_q8_1_d4s4_f32_bf16_f32_out
+        _, ev = self.time_launches(lambda i: fn(dxq.ptr, dw.ptr, dout.ptr, m, k, n), steps, warmup)
+        for buf in (dw, dx, dxq, dout):
+            self.memory.free(buf)
+        return ev, 2.0 * m * n * k
+
+    def moe_case(self, tokens: int, steps: int, warmup: int, experts: int = 256, top_k: int = 8, hidden: int = 2048,
+                 inter: int = 512):
+        """Selected-expert FFN (Q4_K gate/up/down): the two-launch decode chain for
+        tokens <= 8, the grouped-MMQ prefill chain (index, pack, gate|up, SiLU, pack,
+        down, ordered gather) above.  Returns seconds per chain and the bytes of
+        distinct expert weights it touches."""
+        from hipengine_amd.kernels.hip_gfx950.moe import group_scatter as GS
+        from hipengine_amd.kernels.hip_gfx950.quant import gguf_moe as M
+        from hipengine_amd.kernels.hip_gfx950.quant import gguf_quantize as Q
+        from hipengine_amd.synthetic import synthetic_blocks
+
+        rt, mem = self.rt, self.memory
+        rng = np.random.default_rng(tokens)
+        wg = synthetic_blocks(GGML["q4_k"], experts * inter, hidden, seed=5)
+        wu = synthetic_blocks(GGML["q4_k"], experts * inter, hidden, seed=6)
+        wd = synthetic_blocks(GGML["q4_k"], experts * hidden, inter, seed=7)
+        sel = np.stack([rng.permutation(experts)[:top_k] for _ in range(tokens)]).astype(np.int64)
+        wts = rng.random((tokens, top_k)).astype(np.float32)
+        wts /= wts.sum(axis=1, keepdims=True)
+        x = (rng.standard_normal((tokens, hidden)) * 0.3).astype(np.float32)
+        lanes = tokens * top_k
+        bufs = {"wg": mem.to_device(wg, runtime=rt), "wu": mem.to_device(wu, runtime=rt), "wd": mem.to_device(wd, runtime=rt),
+                "sel": mem.to_device(sel, runtime=rt), "wts": mem.to_device(wts, runtime=rt),
+                "out": mem.malloc(tokens * hidden * 4, runtime=rt)}
+        b = bufs
+        per_expert = (2 * inter * (hidden // 256) + hidden * (inter // 256)) * 144
+        touched = len(np.unique(sel)) * per_expert
+        if tokens <= 8:
+            b["x"] = mem.to_device(x, runtime=rt)
+            b["mid"] = mem.malloc(lanes * inter * 4, runtime=rt)
+
+            def chain(_i):
+                M.gguf_selected_gemv("gguf_q4_k", M.SEL_DUAL_SILU, b["x"].ptr, b["sel"].ptr, b["wg"].ptr, b["mid"].ptr,
+                                     tokens, lanes, experts, hidden, inter, qweight_b_ptr=b["wu"].ptr)
+                M.gguf_selected_gemv("gguf_q4_k", M.SEL_DOWN_SUM, b["mid"].ptr, b["sel"].ptr, b["wd"].ptr, b["out"].ptr,
+                                     tokens, lanes, experts, inter, hidden, routing_weights_ptr=b["wts"].ptr,
+                                     top_k=top_k)
+        else:
+            xb = (x.view(np.uint32) >> 16).astype(np.uint16)
+            cap = lanes // 32 + experts
+            b["x"] = mem.to_device(xb, runtime=rt)
+            for name, nbytes in (("es", (experts + 1) * 8), ("act", experts * 8), ("actn", 8), ("sl", lanes * 8),
+                                 ("c2s", lanes * 8), ("sw", lanes * 4), ("ms", (experts + 1) * 8), ("te", cap * 8),
+                                 ("mt", 8), ("l2c", lanes * 8), ("xq", tokens * (hidden // 128) * 144),
+                                 ("gu", lanes * 2 * inter * 4), ("mid", lanes * inter * 2),
+                                 ("mq", lanes * (inter // 128) * 144), ("down", lanes * hidden * 4)):
+                b[name] = mem.malloc(nbytes, runtime=rt)
+            mmq_rows = cap * 32     # upper bound known on the host; unused tiles are marked -1
+
+            def chain(_i):
+                GS.qwen35_moe_group_compact_active_source_rows(b["sel"].ptr, b["wts"].ptr, b["es"].ptr, b["act"].ptr,
+                                                               b["actn"].ptr, b["sl"].ptr, b["c2s"].ptr, b["sw"].ptr,
+                                                               lanes, experts, top_k)
+                GS.qwen35_moe_mmq32_tile_map(b["es"].ptr, b["ms"].ptr, b["te"].ptr, b["mt"].ptr, experts,
+                                             tile_capacity=cap)
+                GS.moe_lane_to_compact(b["sl"].ptr, b["l2c"].ptr, lanes, lanes)
+                Q.gguf_q8_1_mmq_ds4_pack_bf16(b["x"].ptr, b["xq"].ptr, tokens, hidden)
+                M.gguf_q4_k_grouped_mmq(b["xq"].ptr, b["es"].ptr, b["ms"].ptr, b["te"].ptr, b["wg"].ptr, b["gu"].ptr,
+                                        lanes, tokens, hidden, inter, experts, mmq_rows,
+                                        compact_to_source_ptr=b["c2s"].ptr, qweight_b_ptr=b["wu"].ptr,
+                                        out_features_b=inter)
+                M.moe_silu_mul(b["gu"].ptr, b["mid"].ptr, lanes, inter, in_dtype="f32", out_dtype="bf16")
+                Q.gguf_q8_1_mmq_ds4_pack_bf16(b["mid"].ptr, b["mq"].ptr, lanes, inter)
+                M.gguf_q4_k_grouped_mmq(b["mq"].ptr, b["es"].ptr, b["ms"].ptr, b["te"].ptr, b["wd"].ptr, b["down"].ptr,
+                                        lanes, lanes, inter, hidden, experts, mmq_rows)
+                M.moe_weighted_gather_sum(b["down"].ptr, b["l2c"].ptr, b["wts"].ptr, b["out"].ptr, tokens, top_k, hidden,
+                                          lanes)
+        _, ev = self.time_launches(chain, steps, warmup)
+        for buf in bufs.values():
+            mem.free(buf)
+        ops = 2.0 * lanes * (2 * inter * hidden + hidden * inter)
+        return ev, touched, ops
+
+
 def cpu_baseline(w: np.ndarray, x: np.ndarray, nbytes: int) -> dict:
     """The reference CPU backend path (dequantize the whole weight to float32, then a
     float32 matmul; hipengine/kernels/cpu_reference/ops.py:466-484) as restated by
@@ -119,12 +234,26 @@ def main() -> None:
     ap.add_argument("--warmup", type=int, default=50)
     ap.add_argument("--no-extra", action="store_true", help="skip the secondary shapes")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--pmc-pass", action="store_true",
+                    help="hardware-counter pass: a 256 MiB calibration copy, then the headline kernel only")
     args = ap.parse_args()
     if args.gpus != 1:
         raise SystemExit("bench.py measures one GPU: this path is single-GPU (run with --gpus 1)")
 
     h = Harness()
     k, n = 5120, 17408
+    if args.pmc_pass:
+        from hipengine_amd.kernels.hip_gfx950.quant.gguf_verify import copy_bytes
+
+        nbytes = 256 << 20
+        src, dst = h.memory.malloc(nbytes, runtime=h.rt), h.memory.malloc(nbytes, runtime=h.rt)
+        h.rt.memset(src.ptr, 1, nbytes)
+        for _ in range(3):
+            copy_bytes(src.ptr, dst.ptr, nbytes)
+        h.rt.device_synchronize()
+        case = h.gemv_case("q4_k", 1, k, n, max(22, min(args.steps, 44)), 0)
+        print(json.dumps({"pmc_pass": True, "copy_bytes": nbytes, "gemv_bytes": case["bytes"], "copies": case["copies"]}))
+        return
     main_case = h.gemv_case("q4_k", 1, k, n, args.steps, args.warmup)
     gbs = main_case["bytes"] / main_case["wall_s"] / 1e9
     achieved = main_case["bytes"] / main_case["event_s"] / 1e9
@@ -142,6 +271,22 @@ def main() -> None:
             extra[name] = {"us": round(c["event_s"] * 1e6, 2), "GB/s": round(c["bytes"] / c["event_s"] / 1e9, 1),
                            "frac_hbm": round(c["bytes"] / c["event_s"] / 1e9 / HBM_PEAK_GBS, 4), "copies": c["copies"]}
 
+        msteps = max(5, args.steps // 50)
+        for name, (quant, m, kk, nn) in {
+            "mmq_q4_k_17408x5120_m512": ("q4_k", 512, 5120, 17408),
+            "mmq_q4_k_17408x5120_m2048": ("q4_k", 2048, 5120, 17408),
+            "mmq_q4_k_17408x5120_m8192": ("q4_k", 8192, 5120, 17408),
+            "mmq_q6_k_5120x17408_m2048": ("q6_k", 2048, 17408, 5120),
+        }.items():
+            sec, ops = h.mmq_case(quant, m, kk, nn, msteps, 2)
+            extra[name] = {"us": round(sec * 1e6, 1), "int8_TOPS": round(ops / sec / 1e12, 1),
+                           "frac_int8_peak": round(ops / sec / 1e12 / INT8_PEAK_TOPS, 4)}
+        for tokens in (1, 8, 2048):
+            sec, touched, ops = h.moe_case(tokens, max(10, args.steps // 10) if tokens <= 8 else msteps, 3)
+            extra[f"moe_q4_k_e256_k8_h2048_i512_t{tokens}"] = {
+                "us": round(sec * 1e6, 1), "expert_GB/s": round(touched / sec / 1e9, 1),
+                "int8_TOPS": round(ops / sec / 1e12, 2), "launches": 2 if tokens <= 8 else 12}
+
     result = {
         "metric": METRIC,
         "value": round(gbs, 2),
@@ -158,7 +303,7 @@ def main() -> None:
         "config": {"workload": "Q4_K 17408x5120 decode GEMV, batch 1, f32 activations quantized to q8_1 in-kernel",
                    "weight_copies_rotated": main_case["copies"], "bytes_per_step": main_case["bytes"]},
         "roofline": {"bound": "hbm", "achieved": round(achieved, 2), "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                     "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": None,
+                     "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": measured_traffic(),
                      "kernel_us": round(main_case["event_s"] * 1e6, 3)},
         "cpu_baseline": None if args.no_cpu else cpu_baseline(main_case["weight_host"], main_case["x_host"],
                                                                main_case["bytes"]),

@@ -124,7 +124,23 @@ __global__ void __launch_bounds__(64) block_dots_kernel(const uint8_t* __restric
   }
 }
 
+// Plain 16-byte-per-lane copy: the known-size kernel that hardware counter
+// readings (HBM fetch / write sizes) are calibrated against.
+__global__ void __launch_bounds__(256) copy_kernel(const uint4* __restrict__ src, uint4* __restrict__ dst, int64_t n16) {
+  const int64_t stride = static_cast<int64_t>(gridDim.x) * blockDim.x;
+  for (int64_t i = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x; i < n16; i += stride) dst[i] = src[i];
+}
+
 }  // namespace
+
+extern "C" int hipengine_gfx950_copy_bytes(const void* src, void* dst, int64_t bytes, hipStream_t stream) {
+  if (!src || !dst || bytes <= 0 || (bytes % 16) != 0) return static_cast<int>(hipErrorInvalidValue);
+  const int64_t n16 = bytes / 16;
+  const int64_t want = (n16 + 255) / 256;
+  hipLaunchKernelGGL(copy_kernel, dim3(static_cast<unsigned>(want < 16384 ? want : 16384)), dim3(256), 0, stream,
+                     static_cast<const uint4*>(src), static_cast<uint4*>(dst), n16);
+  return static_cast<int>(hipGetLastError());
+}
 
 extern "C" int hipengine_gfx950_gguf_dequantize_f32(int32_t ggml_type, const uint8_t* blocks, float* out,
                                                     int64_t n_blocks, hipStream_t stream) {

@@ -38,3 +38,13 @@ def gguf_q8_1_block_dots_i32(quant_key: str, xq_ptr: int, qweight_ptr: int, dots
     fn = entry("hipengine_gfx950_gguf_q8_1_block_dots_i32", [I32, VOID, VOID, VOID, VOID, I64, I64, I64, VOID], library)
     check_launch(fn(QUANT_KEY_TO_GGML[quant_key], xq_ptr, qweight_ptr, dots_ptr, qsums_ptr or None, rows, in_features,
                     out_features, stream), runtime)
+
+
+def copy_bytes(src_ptr: int, dst_ptr: int, nbytes: int, *, stream: int = 0, library: ctypes.CDLL | None = None,
+               runtime: HipRuntime | None = None) -> None:
+    """Plain device copy kernel of a known size (calibration of HBM byte counters)."""
+    if nbytes <= 0 or nbytes % 16:
+        raise ValueError("nbytes must be a positive multiple of 16")
+    validate_pointers(src_ptr=src_ptr, dst_ptr=dst_ptr)
+    fn = entry("hipengine_gfx950_copy_bytes", [VOID, VOID, I64, VOID], library)
+    check_launch(fn(src_ptr, dst_ptr, nbytes, stream), runtime)

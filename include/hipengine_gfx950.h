@@ -343,6 +343,10 @@ int hipengine_gfx950_gguf_q8_1_block_dots_i32(int32_t ggml_type, const void* xq,
                                               int32_t* dots, int32_t* qsums, int64_t rows, int64_t in_features,
                                               int64_t out_features, hipengine_stream_t stream);
 
+/* dst[0:bytes] = src[0:bytes] with a plain 16-byte-per-lane kernel (bytes % 16 == 0):
+ * the known-size launch that HBM counter readings are calibrated against. */
+int hipengine_gfx950_copy_bytes(const void* src, void* dst, int64_t bytes, hipengine_stream_t stream);
+
 #ifdef __cplusplus
 }
 #endif
