@@ -5,6 +5,7 @@
 #include "gguf_gemv.hpp"
 #include "gguf_gemv_run.hpp"
 #include "gguf_gemv_stream.hpp"
+#include "gguf_gemv_mfma.hpp"
 
 #include "../../include/hipengine_gfx950.h"
 
@@ -97,6 +98,61 @@ const RunVariant* find_run_variant(int qt, int b, int g, int cb) {
   return nullptr;
 }
 
+// ---- tile form (Q4_K on the int8 MFMA, every load of the matrix in flight at once) ----
+
+template <int B, int BPW>
+constexpr int mfma_stage_regs() {
+  return B == 1 ? 5 : B == 2 ? 3 : B == 4 ? 2 : 1;
+}
+
+template <int B, int BPW>
+__global__ void __launch_bounds__(256, 2) gemv_mfma_q4k_kernel(GemvMfmaArgs a) {
+  extern __shared__ __align__(16) uint8_t smem[];
+  gemv_mfma_q4k_workgroup<B, BPW, mfma_stage_regs<B, BPW>()>(a, smem);
+}
+
+using MfmaKernelFn = void (*)(GemvMfmaArgs);
+struct MfmaVariant {
+  int b, bpw;
+  MfmaKernelFn fn;
+};
+#define MFMA_VARIANTS(B)                                                                             \
+  MfmaVariant{B, 1, gemv_mfma_q4k_kernel<B, 1>}, MfmaVariant{B, 2, gemv_mfma_q4k_kernel<B, 2>},       \
+  MfmaVariant{B, 3, gemv_mfma_q4k_kernel<B, 3>}, MfmaVariant{B, 4, gemv_mfma_q4k_kernel<B, 4>},       \
+  MfmaVariant{B, 5, gemv_mfma_q4k_kernel<B, 5>}
+const MfmaVariant kMfma[] = {MFMA_VARIANTS(1), MFMA_VARIANTS(2), MFMA_VARIANTS(4), MFMA_VARIANTS(8)};
+
+struct MfmaPlan {
+  int b, bpw, waves;
+  bool ok;
+};
+
+// Applies to Q4_K with at most 20 blocks per row (4 waves x 5 blocks).
+MfmaPlan default_mfma_plan(int qt, int rows, int64_t K, int64_t N) {
+  MfmaPlan p{};
+  const int nb = static_cast<int>(K / QK_K);
+  p.b = rows <= 1 ? 1 : rows <= 2 ? 2 : rows <= 4 ? 4 : 8;
+  p.bpw = (nb + 3) / 4;
+  p.waves = p.bpw > 0 ? (nb + p.bpw - 1) / p.bpw : 0;
+  p.ok = qt == GGML_Q4_K && rows <= 8 && nb >= 1 && p.bpw <= 5 && N >= 1 &&
+         gemv_mfma_lds_bytes(p.b, static_cast<int>(K), p.waves) <= 64 * 1024;
+  return p;
+}
+
+int launch_gemv_mfma(const void* x, int x_kind, const uint8_t* w, void* out, int out_kind, int rows, int64_t K,
+                     int64_t N, const MfmaPlan& p, hipStream_t stream) {
+  const int nb = static_cast<int>(K / QK_K);
+  const MfmaVariant* v = nullptr;
+  for (const MfmaVariant& c : kMfma)
+    if (c.b == p.b && c.bpw == p.bpw) v = &c;
+  if (!v || rows > p.b || p.waves < 1 || p.waves > 4 || p.waves * p.bpw < nb) return static_cast<int>(hipErrorInvalidValue);
+  const size_t lds = gemv_mfma_lds_bytes(p.b, static_cast<int>(K), p.waves);
+  if (lds > 64 * 1024) return static_cast<int>(hipErrorInvalidValue);
+  GemvMfmaArgs a{x, w, out, x_kind, out_kind, rows, static_cast<int>(K), static_cast<int>(N), p.waves};
+  hipLaunchKernelGGL(v->fn, dim3(static_cast<unsigned>((N + 31) / 32)), dim3(p.waves * 64), lds, stream, a);
+  return static_cast<int>(hipGetLastError());
+}
+
 int gcd_int(int a, int b) { return b == 0 ? a : gcd_int(b, a % b); }
 
 struct RunPlan {
@@ -145,27 +201,39 @@ int launch_gemv_run(int qt, const void* x, int x_kind, const uint8_t* w, void* o
 
 // ---- stream form (resident waves, ring of loads in flight) --------------------
 
-template <int QT, int B, int D>
+template <int QT, int B, int D, bool REFILL>
 __global__ void __launch_bounds__(512) gemv_stream_kernel(GemvStreamArgs a) {
   extern __shared__ __align__(16) uint8_t smem[];
-  gemv_stream_workgroup<QT, B, D>(a, smem);
+  gemv_stream_workgroup<QT, B, D, REFILL>(a, smem);
 }
 
 using StreamKernelFn = void (*)(GemvStreamArgs);
 
+// d > 0: ring of d loads, refilled as they are consumed.  d < 0: all of a wave's
+// loads (at most -d) are issued up front and none later.
 struct StreamVariant {
   int qt, b, d;
   StreamKernelFn fn;
 };
 
 #define STREAM_VARIANT(QT, B, D) \
-  StreamVariant { QT, B, D, gemv_stream_kernel<QT, B, D> }
+  StreamVariant { QT, B, D, gemv_stream_kernel<QT, B, D, true> }
+#define STREAM_UPFRONT(QT, B, D) \
+  StreamVariant { QT, B, -D, gemv_stream_kernel<QT, B, D, false> }
 
 const StreamVariant kStream[] = {
     STREAM_VARIANT(GGML_Q4_K, 1, 3), STREAM_VARIANT(GGML_Q4_K, 1, 5), STREAM_VARIANT(GGML_Q4_K, 2, 3),
     STREAM_VARIANT(GGML_Q4_K, 2, 5), STREAM_VARIANT(GGML_Q6_K, 1, 3), STREAM_VARIANT(GGML_Q6_K, 1, 5),
     STREAM_VARIANT(GGML_Q6_K, 2, 3), STREAM_VARIANT(GGML_Q6_K, 2, 5), STREAM_VARIANT(GGML_Q8_0, 1, 3),
     STREAM_VARIANT(GGML_Q8_0, 1, 5), STREAM_VARIANT(GGML_Q8_0, 2, 3), STREAM_VARIANT(GGML_Q8_0, 2, 5),
+    STREAM_VARIANT(GGML_Q4_K, 4, 3), STREAM_VARIANT(GGML_Q4_K, 8, 3), STREAM_VARIANT(GGML_Q6_K, 4, 3),
+    STREAM_VARIANT(GGML_Q6_K, 8, 3), STREAM_VARIANT(GGML_Q8_0, 4, 3), STREAM_VARIANT(GGML_Q8_0, 8, 3),
+    STREAM_UPFRONT(GGML_Q4_K, 1, 6), STREAM_UPFRONT(GGML_Q4_K, 1, 8), STREAM_UPFRONT(GGML_Q4_K, 1, 12),
+    STREAM_UPFRONT(GGML_Q4_K, 2, 6), STREAM_UPFRONT(GGML_Q4_K, 2, 8), STREAM_UPFRONT(GGML_Q4_K, 2, 12),
+    STREAM_UPFRONT(GGML_Q6_K, 1, 6), STREAM_UPFRONT(GGML_Q6_K, 1, 8), STREAM_UPFRONT(GGML_Q6_K, 1, 12),
+    STREAM_UPFRONT(GGML_Q6_K, 2, 6), STREAM_UPFRONT(GGML_Q6_K, 2, 8), STREAM_UPFRONT(GGML_Q6_K, 2, 12),
+    STREAM_UPFRONT(GGML_Q8_0, 1, 6), STREAM_UPFRONT(GGML_Q8_0, 1, 8), STREAM_UPFRONT(GGML_Q8_0, 1, 12),
+    STREAM_UPFRONT(GGML_Q8_0, 2, 6), STREAM_UPFRONT(GGML_Q8_0, 2, 8), STREAM_UPFRONT(GGML_Q8_0, 2, 12),
 };
 
 const StreamVariant* find_stream_variant(int qt, int b, int d) {
@@ -174,10 +242,18 @@ const StreamVariant* find_stream_variant(int qt, int b, int d) {
   return nullptr;
 }
 
+int batch_bucket(int rows) { return rows <= 1 ? 1 : rows <= 2 ? 2 : rows <= 4 ? 4 : 8; }
+
 struct StreamPlan {
   int b, d, waves, waves_total;
   bool ok;
 };
+
+// Most 16-block loads any wave has: rows are split as evenly as possible.
+int64_t stream_max_loads(int64_t N, int nb, int waves_total) {
+  const int64_t rows = (N + waves_total - 1) / waves_total;
+  return (rows * nb + 15) / 16;
+}
 
 constexpr int kComputeUnits = 256;   // MI355X
 
@@ -186,13 +262,13 @@ constexpr int kComputeUnits = 256;   // MI355X
 StreamPlan default_stream_plan(int qt, int rows, int64_t K, int64_t N) {
   StreamPlan p{};
   const int nb = static_cast<int>(K / QK_K);
-  p.b = rows <= 1 ? 1 : 2;
+  p.b = batch_bucket(rows);
   p.d = 3;
   p.waves = 8;
   const int64_t total_loads = N * nb / 16;
   // 8 resident waves per CU once every wave gets ~8 loads or more, else 4 per CU
   p.waves_total = total_loads >= 16384 ? kComputeUnits * 8 : kComputeUnits * 4;
-  p.ok = rows <= 2 && nb >= 16 && total_loads >= 4 * static_cast<int64_t>(p.waves_total) &&
+  p.ok = rows <= 8 && nb >= 16 && total_loads >= 4 * static_cast<int64_t>(p.waves_total) &&
          N >= p.waves_total && gemv_run_lds_bytes(qt, p.b, static_cast<int>(K)) <= 64 * 1024 &&
          find_stream_variant(qt, p.b, p.d) != nullptr;
   return p;
@@ -203,7 +279,8 @@ int launch_gemv_stream(int qt, const void* x, int x_kind, const uint8_t* w, void
   const StreamVariant* v = find_stream_variant(qt, p.b, p.d);
   const int nb = static_cast<int>(K / QK_K);
   if (!v || nb < 16 || rows > p.b || p.waves < 1 || p.waves > 8 || p.waves_total < p.waves ||
-      (p.waves_total % p.waves) != 0 || p.waves_total > N) {
+      (p.waves_total % p.waves) != 0 || p.waves_total > N ||
+      (p.d < 0 && stream_max_loads(N, nb, p.waves_total) > -p.d)) {
     return static_cast<int>(hipErrorInvalidValue);
   }
   const size_t lds = gemv_run_lds_bytes(qt, p.b, static_cast<int>(K));
@@ -216,8 +293,6 @@ int launch_gemv_stream(int qt, const void* x, int x_kind, const uint8_t* w, void
   hipLaunchKernelGGL(v->fn, dim3(p.waves_total / p.waves), dim3(p.waves * 64), lds, stream, a);
   return static_cast<int>(hipGetLastError());
 }
-
-int batch_bucket(int rows) { return rows <= 1 ? 1 : rows <= 2 ? 2 : rows <= 4 ? 4 : 8; }
 
 struct Plan {
   int b, r, cb, ks, nrg;
@@ -392,15 +467,32 @@ extern "C" int hipengine_gfx950_gguf_q8_1_fused_gemv_stream_tuned(
     int64_t rows, int64_t in_features, int64_t out_features, int32_t loads_in_flight, int32_t waves,
     int32_t waves_total, hipStream_t stream) {
   if (!x || !qweight || !out || x_kind < KIND_F32 || x_kind > KIND_Q8_1 || out_kind < KIND_F32 ||
-      out_kind > KIND_F16 || rows <= 0 || rows > 2 || in_features <= 0 || (in_features % QK_K) != 0 ||
+      out_kind > KIND_F16 || rows <= 0 || rows > 8 || in_features <= 0 || (in_features % QK_K) != 0 ||
       out_features <= 0) {
     return static_cast<int>(hipErrorInvalidValue);
   }
   StreamPlan p{};
-  p.b = rows <= 1 ? 1 : 2;
+  p.b = batch_bucket(static_cast<int>(rows));
   p.d = loads_in_flight;
   p.waves = waves;
   p.waves_total = waves_total;
   return launch_gemv_stream(ggml_type, x, x_kind, qweight, out, out_kind, static_cast<int>(rows), in_features,
                             out_features, p, stream);
+}
+
+extern "C" int hipengine_gfx950_gguf_q4_k_q8_1_fused_gemv_tile_tuned(const void* x, int32_t x_kind,
+                                                                    const uint8_t* qweight, void* out,
+                                                                    int32_t out_kind, int64_t rows,
+                                                                    int64_t in_features, int64_t out_features,
+                                                                    int32_t blocks_per_wave, hipStream_t stream) {
+  if (!x || !qweight || !out || x_kind < KIND_F32 || x_kind > KIND_Q8_1 || out_kind < KIND_F32 ||
+      out_kind > KIND_F16 || rows <= 0 || rows > 8 || in_features <= 0 || (in_features % QK_K) != 0 ||
+      out_features <= 0 || blocks_per_wave < 1 || blocks_per_wave > 5) {
+    return static_cast<int>(hipErrorInvalidValue);
+  }
+  MfmaPlan p = default_mfma_plan(GGML_Q4_K, static_cast<int>(rows), in_features, out_features);
+  p.bpw = blocks_per_wave;
+  p.waves = static_cast<int>((in_features / QK_K + p.bpw - 1) / p.bpw);
+  return launch_gemv_mfma(x, x_kind, qweight, out, out_kind, static_cast<int>(rows), in_features, out_features, p,
+                          stream);
 }

@@ -196,6 +196,45 @@ def test_more_than_eight_rows_and_determinism(dev):
     assert O.max_rel_err(one, a[7:8]) <= 1e-4
 
 
+@pytest.mark.parametrize("rows,k,n,bpw", [(1, 5120, 96, 5), (2, 2048, 70, 2), (4, 1024, 33, 1), (8, 3072, 64, 3),
+                                          (3, 1280, 40, 5), (8, 512, 200, 1)])
+def test_tile_form_q4_k(dev, rows, k, n, bpw):
+    """The int8 MFMA ("tile") form of the fused Q4_K GEMV, K split over up to four waves."""
+    rng = np.random.default_rng(77 + rows + k)
+    x = rng.standard_normal((rows, k)).astype(np.float32)
+    x[0, :32] = 0.0
+    w = O.random_weight(O.GGML_Q4_K, n, k, seed=k + n)
+    if (k // 256 + bpw - 1) // bpw > 4:
+        pytest.skip("more than four K slices")
+    dx, dw = dev.put(x), dev.put(w)
+    dout = dev.empty(rows * n * 4)
+    G.gguf_q4_k_q8_1_fused_gemv_tile_tuned(dx.ptr, "f32", dw.ptr, dout.ptr, "f32", rows, k, n, blocks_per_wave=bpw)
+    got = dev.get(dout, np.float32, (rows, n))
+    dev.free(dx, dw, dout)
+    _check_f32(got, O.quantize_q8_1(x), w, O.GGML_Q4_K)
+
+
+@pytest.mark.parametrize("quant,d,waves_total", [("gguf_q4_k", -12, 64), ("gguf_q4_k", -6, 128), ("gguf_q6_k", -8, 64),
+                                                ("gguf_q8_0", -8, 64), ("gguf_q4_k", 5, 64)])
+def test_stream_form_up_front_and_ring(dev, quant, d, waves_total):
+    """Stream form with all of a wave's loads issued up front (d < 0) and with a ring (d > 0):
+    same bits as the library's default choice for the shape."""
+    rng = np.random.default_rng(5 + waves_total)
+    rows, k, n = 2, 5120, 256
+    x = rng.standard_normal((rows, k)).astype(np.float32)
+    w = O.random_weight(QT[quant], n, k, seed=3)
+    dx, dw = dev.put(x), dev.put(w)
+    dout = dev.empty(rows * n * 4)
+    G.gguf_q8_1_fused_gemv_stream_tuned(quant, dx.ptr, "f32", dw.ptr, dout.ptr, "f32", rows, k, n, loads_in_flight=d,
+                                        waves=4, waves_total=waves_total)
+    got = dev.get(dout, np.float32, (rows, n))
+    dev.free(dx, dw, dout)
+    _check_f32(got, O.quantize_q8_1(x), w, QT[quant])
+    with pytest.raises(Exception):      # a wave with more loads than the up-front depth is refused
+        G.gguf_q8_1_fused_gemv_stream_tuned(quant, 1, "f32", 1, 1, "f32", rows, k, 4096, loads_in_flight=-6, waves=4,
+                                            waves_total=64)
+
+
 def test_output_canaries_untouched(dev):
     rng = np.random.default_rng(55)
     rows, k, n = 3, 512, 21

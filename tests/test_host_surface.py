@@ -95,6 +95,14 @@ def test_backend_registers_the_documented_keys(clean_registry):
             assert KernelKey("hip_gfx950", "linear", q, v) in keys
     assert KernelKey("hip_gfx950", "linear", "gguf_q4_k", "q8_1_dp4a_vdr_bf16_f32_out") in keys
     assert KernelKey("hip_gfx950", "activation_quant", "q8_1_ds4", "bf16") in keys
+    for key in (KernelKey("hip_gfx950", "linear", "gguf_q4_k", "mmq32_vdr_dense_bf16_f32_out"),
+                KernelKey("hip_gfx950", "linear", "gguf_q6_k", "mmq32_q8_1_d4s4_f32_bf16_f32_out"),
+                KernelKey("hip_gfx950", "linear", "gguf_q4_k", "selected_gemv_bf16_bf16_out"),
+                KernelKey("hip_gfx950", "moe_linear", "gguf_q4_k",
+                          "selected_dual_q8_1_ds4_mmq32_prefill_compact32_bf16_bf16_out"),
+                KernelKey("hip_gfx950", "moe_group_compact", "generic", "active_experts_source_rows"),
+                KernelKey("hip_gfx950", "moe_mmq_tile_map", "generic", "tile32")):
+        assert key in keys
     assert not any(k.backend == "cpu_reference" for k in keys)            # the package ships no CPU path
     assert hip_gfx950.GGUF_CONSUMER_LAYERS >= {"linear", "moe_linear"}
     fn = R.resolve(backend="hip_gfx950", layer="linear", quant="gguf_q4_k", variant="q8_1_fused_gemv_f32_f32_out")
@@ -189,3 +197,30 @@ def test_build_plan_is_stable_and_names_the_artifact():
     assert "--offload-arch=gfx950" in a.flags and "-mcumode" not in a.flags
     assert build.plan_hip_build(compiler_version="other").key != a.key
     assert a.commands[-1][-1].endswith("libhipengine_gfx950.so")
+
+
+def test_moe_wrappers_validate_before_touching_the_device():
+    """Argument errors are raised on the host, before any library call (hipEngine's wrappers do the same)."""
+    from hipengine_amd.kernels.hip_gfx950.moe import group_scatter as GS
+    from hipengine_amd.kernels.hip_gfx950.quant import gguf_moe as M
+
+    with pytest.raises(ValueError, match="num_experts"):
+        GS.qwen35_moe_mmq32_tile_map(1, 1, 1, 1, 0)
+    with pytest.raises(ValueError, match="num_experts"):
+        GS.qwen35_moe_group_compact_active_source_rows(1, 1, 1, 1, 1, 1, 1, 1, 8, 4096, 8)
+    with pytest.raises(ValueError, match="tile_capacity"):
+        GS.qwen35_moe_mmq32_tile_map(1, 1, 1, 1, 8, tile_capacity=-1)
+    with pytest.raises(ValueError, match="multiple of x_rows"):
+        M.gguf_q4_k_selected_gemv_bf16_bf16_out(1, 1, 1, 1, 3, 8, 4, 256, 32)
+    with pytest.raises(ValueError, match="divisible"):
+        M.gguf_q4_k_selected_gemv_bf16_bf16_out(1, 1, 1, 1, 1, 8, 4, 200, 32)
+    with pytest.raises(ValueError, match="non-null"):
+        M.gguf_q4_k_selected_gemv_bf16_bf16_out(0, 1, 1, 1, 1, 8, 4, 256, 32)
+    with pytest.raises(ValueError, match="x_rows \\* top_k"):
+        M.gguf_selected_gemv("gguf_q4_k", M.SEL_DOWN_SUM, 1, 1, 1, 1, 2, 9, 4, 256, 32, routing_weights_ptr=1, top_k=4)
+    with pytest.raises(ValueError, match="gguf_q4_k or gguf_q6_k"):
+        M.gguf_selected_gemv("gguf_q8_0", M.SEL_SINGLE, 1, 1, 1, 1, 1, 8, 4, 256, 32)
+    with pytest.raises(ValueError, match="multiples of 32"):
+        M.gguf_q4_k_grouped_mmq(1, 1, 1, 1, 1, 1, 8, 8, 256, 40, 4, 32)
+    with pytest.raises(ValueError, match="multiple of 32"):
+        M.gguf_q4_k_grouped_mmq(1, 1, 1, 1, 1, 1, 8, 8, 256, 64, 4, 40)
