@@ -178,7 +178,7 @@ class Harness:
             for name, nbytes in (("es", (experts + 1) * 8), ("act", experts * 8), ("actn", 8), ("sl", lanes * 8),
                                  ("c2s", lanes * 8), ("sw", lanes * 4), ("ms", (experts + 1) * 8), ("te", cap * 8),
                                  ("mt", 8), ("l2c", lanes * 8), ("xq", tokens * (hidden // 128) * 144),
-                                 ("gu", lanes * 2 * inter * 4), ("mid", lanes * inter * 2),
+                                 ("gu", lanes * 2 * inter * 4),
                                  ("mq", lanes * (inter // 128) * 144), ("down", lanes * hidden * 4)):
                 b[name] = mem.malloc(nbytes, runtime=rt)
             mmq_rows = cap * 32     # upper bound known on the host; unused tiles are marked -1
@@ -195,8 +195,7 @@ class Harness:
                                         lanes, tokens, hidden, inter, experts, mmq_rows,
                                         compact_to_source_ptr=b["c2s"].ptr, qweight_b_ptr=b["wu"].ptr,
                                         out_features_b=inter)
-                M.moe_silu_mul(b["gu"].ptr, b["mid"].ptr, lanes, inter, in_dtype="f32", out_dtype="bf16")
-                Q.gguf_q8_1_mmq_ds4_pack_bf16(b["mid"].ptr, b["mq"].ptr, lanes, inter)
+                M.moe_silu_mul_ds4_pack(b["gu"].ptr, b["mq"].ptr, lanes, inter, in_dtype="f32")
                 M.gguf_q4_k_grouped_mmq(b["mq"].ptr, b["es"].ptr, b["ms"].ptr, b["te"].ptr, b["wd"].ptr, b["down"].ptr,
                                         lanes, lanes, inter, hidden, experts, mmq_rows)
                 M.moe_weighted_gather_sum(b["down"].ptr, b["l2c"].ptr, b["wts"].ptr, b["out"].ptr, tokens, top_k, hidden,
@@ -263,6 +262,8 @@ def main() -> None:
         steps = max(20, args.steps // 5)
         for name, (quant, rows, kk, nn) in {
             "q4_k_17408x5120_b2": ("q4_k", 2, 5120, 17408),
+            "q4_k_17408x5120_b4": ("q4_k", 4, 5120, 17408),
+            "q4_k_17408x5120_b8": ("q4_k", 8, 5120, 17408),
             "q8_0_5120x5120_b1": ("q8_0", 1, 5120, 5120),
             "q6_k_5120x17408_b1": ("q6_k", 1, 17408, 5120),
             "q6_k_151936x5120_b1": ("q6_k", 1, 5120, 151936),
@@ -270,6 +271,21 @@ def main() -> None:
             c = h.gemv_case(quant, rows, kk, nn, steps, max(5, args.warmup // 5))
             extra[name] = {"us": round(c["event_s"] * 1e6, 2), "GB/s": round(c["bytes"] / c["event_s"] / 1e9, 1),
                            "frac_hbm": round(c["bytes"] / c["event_s"] / 1e9 / HBM_PEAK_GBS, 4), "copies": c["copies"]}
+
+        # One dense 27B-shape decoder layer at batch 1 (q, k, o, gate, up in Q4_K; v, down in Q6_K),
+        # every matmul with its own rotating weights: bytes / sum of kernel times, and the
+        # decode rate a 64-layer stack of these matmuls alone would allow.
+        layer = (("q4_k", 5120, 5120), ("q4_k", 5120, 1024), ("q4_k", 5120, 5120), ("q4_k", 5120, 17408),
+                 ("q4_k", 5120, 17408), ("q6_k", 5120, 1024), ("q6_k", 17408, 5120))
+        lbytes, lsec = 0, 0.0
+        for quant, kk, nn in layer:
+            c = h.gemv_case(quant, 1, kk, nn, steps, max(5, args.warmup // 5))
+            lbytes += c["bytes"]
+            lsec += c["event_s"]
+        extra["layer_sweep_27b_b1"] = {"bytes_per_layer": lbytes, "us_per_layer": round(lsec * 1e6, 1),
+                                       "GB/s": round(lbytes / lsec / 1e9, 1),
+                                       "frac_hbm": round(lbytes / lsec / 1e9 / HBM_PEAK_GBS, 4),
+                                       "tok_per_s_64_layers_matmuls_only": round(1.0 / (64 * lsec), 1)}
 
         msteps = max(5, args.steps // 50)
         for name, (quant, m, kk, nn) in {
@@ -285,7 +301,7 @@ def main() -> None:
             sec, touched, ops = h.moe_case(tokens, max(10, args.steps // 10) if tokens <= 8 else msteps, 3)
             extra[f"moe_q4_k_e256_k8_h2048_i512_t{tokens}"] = {
                 "us": round(sec * 1e6, 1), "expert_GB/s": round(touched / sec / 1e9, 1),
-                "int8_TOPS": round(ops / sec / 1e12, 2), "launches": 2 if tokens <= 8 else 12}
+                "int8_TOPS": round(ops / sec / 1e12, 2), "launches": 2 if tokens <= 8 else 10}
 
     result = {
         "metric": METRIC,

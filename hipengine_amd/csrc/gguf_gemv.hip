@@ -226,6 +226,8 @@ const StreamVariant kStream[] = {
     STREAM_VARIANT(GGML_Q4_K, 2, 5), STREAM_VARIANT(GGML_Q6_K, 1, 3), STREAM_VARIANT(GGML_Q6_K, 1, 5),
     STREAM_VARIANT(GGML_Q6_K, 2, 3), STREAM_VARIANT(GGML_Q6_K, 2, 5), STREAM_VARIANT(GGML_Q8_0, 1, 3),
     STREAM_VARIANT(GGML_Q8_0, 1, 5), STREAM_VARIANT(GGML_Q8_0, 2, 3), STREAM_VARIANT(GGML_Q8_0, 2, 5),
+    STREAM_VARIANT(GGML_Q4_K, 1, 4), STREAM_VARIANT(GGML_Q4_K, 1, 6), STREAM_VARIANT(GGML_Q4_K, 2, 4),
+    STREAM_VARIANT(GGML_Q4_K, 2, 6), STREAM_VARIANT(GGML_Q6_K, 1, 4), STREAM_VARIANT(GGML_Q8_0, 1, 4),
     STREAM_VARIANT(GGML_Q4_K, 4, 3), STREAM_VARIANT(GGML_Q4_K, 8, 3), STREAM_VARIANT(GGML_Q6_K, 4, 3),
     STREAM_VARIANT(GGML_Q6_K, 8, 3), STREAM_VARIANT(GGML_Q8_0, 4, 3), STREAM_VARIANT(GGML_Q8_0, 8, 3),
     STREAM_UPFRONT(GGML_Q4_K, 1, 6), STREAM_UPFRONT(GGML_Q4_K, 1, 8), STREAM_UPFRONT(GGML_Q4_K, 1, 12),
@@ -266,9 +268,9 @@ StreamPlan default_stream_plan(int qt, int rows, int64_t K, int64_t N) {
   p.d = 3;
   p.waves = 8;
   const int64_t total_loads = N * nb / 16;
-  // 8 resident waves per CU once every wave gets ~8 loads or more, else 4 per CU
-  p.waves_total = total_loads >= 16384 ? kComputeUnits * 8 : kComputeUnits * 4;
-  p.ok = rows <= 8 && nb >= 16 && total_loads >= 4 * static_cast<int64_t>(p.waves_total) &&
+  // 8 resident waves per CU once every wave gets 3 loads or more, else 4 per CU
+  p.waves_total = total_loads >= 6144 ? kComputeUnits * 8 : kComputeUnits * 4;
+  p.ok = rows <= 8 && nb >= 16 && total_loads >= 3 * static_cast<int64_t>(p.waves_total) &&
          N >= p.waves_total && gemv_run_lds_bytes(qt, p.b, static_cast<int>(K)) <= 64 * 1024 &&
          find_stream_variant(qt, p.b, p.d) != nullptr;
   return p;

@@ -22,14 +22,13 @@
 //     loads are issued before the weight loads, because the memory counter
 //     retires in order);
 //   * per sub-block: A = int8 activations of batch row (lane % 32) from LDS
-//     (zero for rows >= batch), B = unpacked nibbles, accumulator input
-//     0x4B400000 so that the int32 result read as float is 12582912 + dot.
+//     (zero for rows >= batch), B = unpacked nibbles, zero accumulator input.
 //     The result tile has the batch row in the register index: lane (n, g)
 //     register v holds batch row 4*g + v of output row n for v < 4, so a batch
 //     of 1..4 costs VB = 1..4 epilogue chains per sub-block and lanes g = 1
 //     carry batch rows 4..7;
-//   * epilogue per used register: t = fma(U, d*sc, -12582912*d*sc) = d*sc*dot
-//     (one rounding), acc = fma(xd, t, acc), acc = fma(-dmin*mn, xd*qsum, acc)
+//   * epilogue per used register: t = (d*sc) * float(dot), acc = fma(xd, t, acc),
+//     acc = fma(-dmin*mn, xd*qsum, acc)
 //     (the arithmetic of gguf_q4_k_gemv.hip:893-904);
 //   * K slices are summed through LDS in slice order.
 #pragma once
@@ -64,8 +63,6 @@ template <int B, int BPW, int S>
 __device__ __forceinline__ void gemv_mfma_q4k_workgroup(const GemvMfmaArgs& a, uint8_t* smem) {
   constexpr int Q8S = run_q8_stride<GGML_Q4_K>();
   constexpr int VB = B < 4 ? B : 4;                 // result registers in use per lane
-  constexpr uint32_t MAGIC_BITS = 0x4B400000u;
-  constexpr float MAGIC = 12582912.0f;
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int n = lane & 31, g = lane >> 5;
   const int nb = a.K / QK_K;
@@ -132,19 +129,18 @@ __device__ __forceinline__ void gemv_mfma_q4k_workgroup(const GemvMfmaArgs& a, u
         const gm_v4i xop = *reinterpret_cast<const gm_v4i*>(a_base + a_mul * (kbc * Q8S + sb * 32));
         gm_v16i c0;
 #pragma unroll
-        for (int v = 0; v < 16; ++v) c0[v] = static_cast<int>(MAGIC_BITS);
+        for (int v = 0; v < 16; ++v) c0[v] = 0;
         const gm_v16i dots = __builtin_amdgcn_mfma_i32_32x32x32_i8(xop, wop, c0, 0, 0, 0);
         const uint32_t sc = ((sb < 4 ? u.sc_lo : u.sc_hi) >> (8 * (sb & 3))) & 0xFFu;
         const uint32_t mn = ((sb < 4 ? u.mn_lo : u.mn_hi) >> (8 * (sb & 3))) & 0xFFu;
         const float sw = d * static_cast<float>(sc);
-        const float cw = -MAGIC * sw;
         const float mw = -(dmin * static_cast<float>(mn));
 #pragma unroll
         for (int v = 0; v < VB; ++v) {
           // record of batch row 4*g + v: {xd(2j), xd(2j+1), xd*qsum(2j), xd*qsum(2j+1)} at [kb*16 + j*4]
           const float* r = rec_g + min(v, B - 1 - min(4 * g, B - 1)) * nb * 16 + kbc * 16 + j * 4;
           const float xd = r[half], xs = r[2 + half];
-          const float t = __builtin_fmaf(bits_to_float(static_cast<uint32_t>(dots[v])), sw, cw);
+          const float t = sw * static_cast<float>(dots[v]);      // d*sc*dot, one rounding (|dot| < 2^24)
           acc[v] = __builtin_fmaf(xd, t, acc[v]);
           acc[v] = __builtin_fmaf(mw, xs, acc[v]);
         }

@@ -29,34 +29,23 @@ constexpr int MAX_EXPERTS = 2048;
 // routing index
 // --------------------------------------------------------------------------
 
-__device__ __forceinline__ int wave_sum_i(int v) {
-#pragma unroll
-  for (int off = 32; off > 0; off >>= 1) v += __shfl_xor(v, off, 64);
-  return v;
-}
-
-// One workgroup per expert: counts[e] = number of lanes that selected e.
-__global__ void __launch_bounds__(256) moe_count_kernel(const int64_t* __restrict__ selected, int64_t* __restrict__ counts,
-                                                        int64_t lanes) {
-  __shared__ int part[4];
-  const int64_t e = blockIdx.x;
-  int c = 0;
-  for (int64_t i = threadIdx.x; i < lanes; i += 256) c += selected[i] == e;
-  c = wave_sum_i(c);
-  if ((threadIdx.x & 63) == 0) part[threadIdx.x >> 6] = c;
-  __syncthreads();
-  if (threadIdx.x == 0) counts[e] = part[0] + part[1] + part[2] + part[3];
-}
-
-// One workgroup: counts (in expert_start[0..E)) -> exclusive starts, total in
-// expert_start[E], ascending list of the experts that own at least one lane.
-__global__ void __launch_bounds__(256) moe_prefix_active_kernel(int64_t* __restrict__ expert_start,
+// One workgroup: histogram of the selected experts in LDS (integer atomics, so the
+// result does not depend on order), exclusive prefix -> expert_start[0..E],
+// ascending list of the experts that own at least one lane.
+__global__ void __launch_bounds__(1024) moe_count_prefix_kernel(const int64_t* __restrict__ selected,
+                                                                int64_t* __restrict__ expert_start,
                                                                 int64_t* __restrict__ active_experts,
-                                                                int64_t* __restrict__ active_count, int num_experts) {
+                                                                int64_t* __restrict__ active_count, int64_t lanes,
+                                                                int num_experts) {
   __shared__ int cnt[MAX_EXPERTS];
   __shared__ int act[MAX_EXPERTS];
   __shared__ int totals[2];
-  for (int e = threadIdx.x; e < num_experts; e += 256) cnt[e] = static_cast<int>(expert_start[e]);
+  for (int e = threadIdx.x; e < num_experts; e += 1024) cnt[e] = 0;
+  __syncthreads();
+  for (int64_t i = threadIdx.x; i < lanes; i += 1024) {
+    const int64_t e = selected[i];
+    if (e >= 0 && e < num_experts) atomicAdd(&cnt[e], 1);
+  }
   __syncthreads();
   if (threadIdx.x == 0) {
     int offset = 0, active = 0;
@@ -68,9 +57,9 @@ __global__ void __launch_bounds__(256) moe_prefix_active_kernel(int64_t* __restr
     totals[0] = offset; totals[1] = active;
   }
   __syncthreads();
-  for (int e = threadIdx.x; e < num_experts; e += 256) expert_start[e] = cnt[e];
+  for (int e = threadIdx.x; e < num_experts; e += 1024) expert_start[e] = cnt[e];
   if (active_experts)
-    for (int i = threadIdx.x; i < totals[1]; i += 256) active_experts[i] = act[i];
+    for (int i = threadIdx.x; i < totals[1]; i += 1024) active_experts[i] = act[i];
   if (threadIdx.x == 0) {
     expert_start[num_experts] = totals[0];
     if (active_count) active_count[0] = totals[1];
@@ -79,33 +68,34 @@ __global__ void __launch_bounds__(256) moe_prefix_active_kernel(int64_t* __restr
 
 // One workgroup per expert: writes its lanes in ascending lane order (wave
 // ballots keep the order) into [expert_start[e], expert_start[e+1]).
-__global__ void __launch_bounds__(256) moe_place_kernel(const int64_t* __restrict__ selected,
-                                                        const float* __restrict__ routing,
-                                                        const int64_t* __restrict__ expert_start,
-                                                        int64_t* __restrict__ sorted_lanes,
-                                                        int64_t* __restrict__ sorted_experts,
-                                                        int64_t* __restrict__ compact_to_source,
-                                                        float* __restrict__ sorted_weights, int64_t lanes,
-                                                        int64_t top_k) {
-  __shared__ int wave_cnt[4];
+__global__ void __launch_bounds__(1024) moe_place_kernel(const int64_t* __restrict__ selected,
+                                                         const float* __restrict__ routing,
+                                                         const int64_t* __restrict__ expert_start,
+                                                         int64_t* __restrict__ sorted_lanes,
+                                                         int64_t* __restrict__ sorted_experts,
+                                                         int64_t* __restrict__ compact_to_source,
+                                                         float* __restrict__ sorted_weights, int64_t lanes,
+                                                         int64_t top_k) {
+  __shared__ int wave_cnt[2][16];
   const int64_t e = blockIdx.x;
   const int64_t base = expert_start[e];
   const int count = static_cast<int>(expert_start[e + 1] - base);
   if (count <= 0) return;
   const int lane_id = threadIdx.x & 63, wave = threadIdx.x >> 6;
-  int running = 0;
-  for (int64_t chunk = 0; chunk < lanes && running < count; chunk += 256) {
+  int running = 0, buf = 0;
+  for (int64_t chunk = 0; chunk < lanes && running < count; chunk += 1024, buf ^= 1) {
     const int64_t lane = chunk + threadIdx.x;
     const bool flag = lane < lanes && selected[lane] == e;
     const unsigned long long ballot = __ballot(flag);
     const int before = __popcll(ballot & ((1ull << lane_id) - 1ull));
-    if (lane_id == 0) wave_cnt[wave] = __popcll(ballot);
-    __syncthreads();
+    if (lane_id == 0) wave_cnt[buf][wave] = __popcll(ballot);
+    __syncthreads();      // one barrier per chunk: the count buffers alternate
     int offset = running, total = 0;
 #pragma unroll
-    for (int w = 0; w < 4; ++w) {
-      if (w < wave) offset += wave_cnt[w];
-      total += wave_cnt[w];
+    for (int w = 0; w < 16; ++w) {
+      const int c = wave_cnt[buf][w];
+      if (w < wave) offset += c;
+      total += c;
     }
     if (flag) {
       const int64_t idx = base + offset + before;
@@ -115,7 +105,6 @@ __global__ void __launch_bounds__(256) moe_place_kernel(const int64_t* __restric
       if (sorted_weights) sorted_weights[idx] = routing[lane];
     }
     running += total;
-    __syncthreads();
   }
 }
 
@@ -126,11 +115,9 @@ int launch_compact(const int64_t* selected, const float* routing, int64_t* exper
       num_experts <= 0 || num_experts > MAX_EXPERTS || top_k <= 0) {
     return static_cast<int>(hipErrorInvalidValue);
   }
-  hipLaunchKernelGGL(moe_count_kernel, dim3(static_cast<unsigned>(num_experts)), dim3(256), 0, stream, selected,
-                     expert_start, lanes);
-  hipLaunchKernelGGL(moe_prefix_active_kernel, dim3(1), dim3(256), 0, stream, expert_start, active_experts, active_count,
-                     static_cast<int>(num_experts));
-  hipLaunchKernelGGL(moe_place_kernel, dim3(static_cast<unsigned>(num_experts)), dim3(256), 0, stream, selected, routing,
+  hipLaunchKernelGGL(moe_count_prefix_kernel, dim3(1), dim3(1024), 0, stream, selected, expert_start, active_experts,
+                     active_count, lanes, static_cast<int>(num_experts));
+  hipLaunchKernelGGL(moe_place_kernel, dim3(static_cast<unsigned>(num_experts)), dim3(1024), 0, stream, selected, routing,
                      expert_start, sorted_lanes, sorted_experts, compact_to_source, sorted_weights, lanes, top_k);
   return static_cast<int>(hipGetLastError());
 }

@@ -60,6 +60,27 @@ __global__ void __launch_bounds__(256) quantize_q8_1_kernel(const void* __restri
 
 constexpr float kFp16Max = 65504.0f;
 
+// One lane's share (4 of 32 values) of a DS4 group: ties-to-even, clamp +-127, fp16 scale and sum.
+__device__ __forceinline__ void ds4_pack_group(const float (&v)[4], float amax, int64_t g, int e, uint8_t* out) {
+  const int64_t blk_idx = g >> 2;
+  const int grp = static_cast<int>(g & 3);
+  const float sum = fminf(kFp16Max, fmaxf(-kFp16Max, oct_tree_sum32(v[0], v[1], v[2], v[3])));
+  const float scale = fminf(kFp16Max, amax / 127.0f);
+  uint32_t packed = 0;
+  if (scale > 0.0f) {
+    packed = pack_i8x4(static_cast<int>(fminf(127.0f, fmaxf(-127.0f, rintf(v[0] / scale)))),
+                       static_cast<int>(fminf(127.0f, fmaxf(-127.0f, rintf(v[1] / scale)))),
+                       static_cast<int>(fminf(127.0f, fmaxf(-127.0f, rintf(v[2] / scale)))),
+                       static_cast<int>(fminf(127.0f, fmaxf(-127.0f, rintf(v[3] / scale)))));
+  }
+  uint8_t* blk = out + blk_idx * DS4_BYTES;
+  *reinterpret_cast<uint32_t*>(blk + 16 + grp * 32 + 4 * e) = packed;
+  if (e == 0) {
+    *reinterpret_cast<uint32_t*>(blk + 4 * grp) =
+        static_cast<uint32_t>(float_to_f16_bits(scale)) | (static_cast<uint32_t>(float_to_f16_bits(sum)) << 16);
+  }
+}
+
 // DS4 (ties-to-even, clamp +-127, fp16 scale and sum) or D4S4 (ties away,
 // clamp -128..127, float32 scale and sum).  One group of 8 lanes per 32 values;
 // a 128-value block is four consecutive groups.
@@ -95,22 +116,30 @@ __global__ void __launch_bounds__(256) pack_mmq_kernel(const uint16_t* __restric
       *reinterpret_cast<float*>(blk + 16 + 4 * grp) = s;
     }
   } else {
-    const float sum = fminf(kFp16Max, fmaxf(-kFp16Max, oct_tree_sum32(v[0], v[1], v[2], v[3])));
-    const float scale = fminf(kFp16Max, amax / 127.0f);
-    uint32_t packed = 0;
-    if (scale > 0.0f) {
-      packed = pack_i8x4(static_cast<int>(fminf(127.0f, fmaxf(-127.0f, rintf(v[0] / scale)))),
-                         static_cast<int>(fminf(127.0f, fmaxf(-127.0f, rintf(v[1] / scale)))),
-                         static_cast<int>(fminf(127.0f, fmaxf(-127.0f, rintf(v[2] / scale)))),
-                         static_cast<int>(fminf(127.0f, fmaxf(-127.0f, rintf(v[3] / scale)))));
-    }
-    uint8_t* blk = out + blk_idx * DS4_BYTES;
-    *reinterpret_cast<uint32_t*>(blk + 16 + grp * 32 + 4 * e) = packed;
-    if (e == 0) {
-      *reinterpret_cast<uint32_t*>(blk + 4 * grp) =
-          static_cast<uint32_t>(float_to_f16_bits(scale)) | (static_cast<uint32_t>(float_to_f16_bits(sum)) << 16);
-    }
+    ds4_pack_group(v, amax, g, e, out);
   }
+}
+
+// gate_up [rows, 2*inter] (gate columns first) -> DS4 blocks of bf16_round(silu(gate) * up):
+// the bytes the two-step path (SiLU*up to bf16, then the DS4 pack) produces.
+__global__ void __launch_bounds__(256) silu_mul_ds4_pack_kernel(const void* __restrict__ gate_up, int in_kind,
+                                                                uint8_t* __restrict__ out, int64_t total_groups,
+                                                                int64_t inter) {
+  const int64_t g = static_cast<int64_t>(blockIdx.x) * 32 + (threadIdx.x >> 3);
+  const int e = threadIdx.x & 7;
+  if (g >= total_groups) return;
+  const int64_t flat = g * 32 + e * 4;
+  const int64_t row = flat / inter, col = flat - row * inter;
+  float gate[4], up[4], v[4];
+  load4_values(gate_up, in_kind, row * 2 * inter + col, gate);
+  load4_values(gate_up, in_kind, row * 2 * inter + inter + col, up);
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    const float sig = 1.0f / (1.0f + expf(-gate[i]));
+    v[i] = bf16_bits_to_float(float_to_bf16_bits(gate[i] * sig * up[i]));
+  }
+  const float amax = oct_max(fmaxf(fmaxf(fabsf(v[0]), fabsf(v[1])), fmaxf(fabsf(v[2]), fabsf(v[3]))));
+  ds4_pack_group(v, amax, g, e, out);
 }
 
 int launch_q8_1(const void* x, int kind, void* xq, int64_t rows, int64_t in_features, hipStream_t stream) {
@@ -160,4 +189,17 @@ extern "C" int hipengine_gguf_q8_1_mmq_ds4_pack_bf16(const void* x, void* out, i
 extern "C" int hipengine_gguf_q8_1_d4s4_f32_quantize_bf16(const void* x, void* out, int64_t rows, int64_t hidden,
                                                           hipStream_t stream) {
   return launch_pack<true>(x, out, rows, hidden, stream);
+}
+
+extern "C" int hipengine_gfx950_moe_silu_mul_ds4_pack(const void* gate_up, int in_kind, void* out, int64_t rows,
+                                                      int64_t inter, hipStream_t stream) {
+  if (!gate_up || !out || rows <= 0 || inter <= 0 || (inter % 128) != 0 || in_kind < KIND_F32 || in_kind > KIND_F16) {
+    return static_cast<int>(hipErrorInvalidValue);
+  }
+  const int64_t groups = rows * (inter / 32);
+  const int64_t grid = (groups + 31) / 32;
+  if (grid > 0x7FFFFFFF) return static_cast<int>(hipErrorInvalidValue);
+  hipLaunchKernelGGL(silu_mul_ds4_pack_kernel, dim3(static_cast<unsigned>(grid)), dim3(256), 0, stream, gate_up,
+                     in_kind, static_cast<uint8_t*>(out), groups, inter);
+  return static_cast<int>(hipGetLastError());
 }

@@ -156,6 +156,17 @@ def moe_silu_mul(gate_up_ptr: int, out_ptr: int, rows: int, inter: int, *, in_dt
     check_launch(fn(gate_up_ptr, out_ptr, rows, inter, _KIND[in_dtype], _KIND[out_dtype], stream), runtime)
 
 
+def moe_silu_mul_ds4_pack(gate_up_ptr: int, out_ptr: int, rows: int, inter: int, *, in_dtype: str = "f32",
+                          stream: int = 0, library: ctypes.CDLL | None = None,
+                          runtime: HipRuntime | None = None) -> None:
+    """``silu(gate) * up`` rounded to bf16 and packed to DS4 blocks ``[rows, inter/128]`` in one launch."""
+    if rows <= 0 or inter <= 0 or inter % 128 != 0:
+        raise ValueError("rows must be positive and inter a positive multiple of 128")
+    validate_pointers(gate_up_ptr=gate_up_ptr, out_ptr=out_ptr)
+    fn = entry("hipengine_gfx950_moe_silu_mul_ds4_pack", [VOID, ctypes.c_int, VOID, I64, I64, VOID], library)
+    check_launch(fn(gate_up_ptr, _KIND[in_dtype], out_ptr, rows, inter, stream), runtime)
+
+
 def moe_weighted_gather_sum(down_ptr: int, lane_to_compact_ptr: int, routing_weights_ptr: int, out_ptr: int,
                             tokens: int, top_k: int, hidden: int, compact_rows: int, *, in_dtype: str = "f32",
                             out_dtype: str = "f32", stream: int = 0, library: ctypes.CDLL | None = None,

@@ -259,6 +259,14 @@ int hipengine_gfx950_moe_lane_to_compact(const int64_t* sorted_lanes, int64_t* l
 int hipengine_gfx950_moe_silu_mul(const void* gate_up, void* out, int64_t rows, int64_t inter, int in_kind,
                                   int out_kind, hipengine_stream_t stream);
 
+/* gate_up[rows, 2*inter] -> DS4 blocks [rows, inter/128] of bf16(gate*sigmoid(gate)*up):
+ * byte for byte what hipengine_gfx950_moe_silu_mul (bf16 out) followed by
+ * hipengine_gguf_q8_1_mmq_ds4_pack_bf16 writes, in one launch.  inter % 128 == 0.
+ * (hipEngine fuses the same pair in its ds4_f32 pack_dual_silu kernels,
+ * gguf_q4_k_q8_1_selected_prefill.py:77-84.) */
+int hipengine_gfx950_moe_silu_mul_ds4_pack(const void* gate_up, int in_kind, void* out, int64_t rows, int64_t inter,
+                                           hipengine_stream_t stream);
+
 /* out[t, h] = sum over slots s = 0..top_k-1, in that order, of
  * routing_weights[t*top_k+s] * down[lane_to_compact[t*top_k+s], h]; lanes mapped
  * to -1 are skipped.  tokens <= 65535.  New here (see lane_to_compact). */

@@ -281,6 +281,9 @@ def test_prefill_chain_matches_cpu_moe(dev):
     M.moe_silu_mul(dgu.ptr, dmid.ptr, total, inter, in_dtype="f32", out_dtype="bf16")
     dmq = dev.empty(total * (inter // 128) * 144)
     Q.gguf_q8_1_mmq_ds4_pack_bf16(dmid.ptr, dmq.ptr, total, inter)
+    two_step = dev.get(dmq, np.uint8, (total, inter // 128, 144)).copy()
+    M.moe_silu_mul_ds4_pack(dgu.ptr, dmq.ptr, total, inter, in_dtype="f32")     # the same bytes in one launch
+    assert np.array_equal(dev.get(dmq, np.uint8, (total, inter // 128, 144)), two_step)
     ddown = dev.empty(total * hidden * 4)
     M.gguf_q4_k_grouped_mmq(dmq.ptr, d["expert_start"].ptr, d["mmq_start"].ptr, d["tile_expert"].ptr, dd.ptr, ddown.ptr,
                             total, total, inter, hidden, experts, host["mmq_total"])
