@@ -258,22 +258,34 @@ __device__ __forceinline__ void gemv_run_stage_commit(const GemvRunArgs& a, cons
       const int j = team + s * nteams;
       if (j < groups) gemv_run_stage_one<QT>(a.x_kind, sr.raw[b][s], b < a.rows, j, e, q8_row, rec_row, s16_row);
     }
-    for (int j = team + S * nteams; j < groups; j += nteams) {   // large K: the rest, loaded here
-      uint32_t raw[4] = {0u, 0u, 0u, 0u};
-      if (b < a.rows) {
-        if (a.x_kind == KIND_F32) {
-          const uint4 v = *reinterpret_cast<const uint4*>(static_cast<const float*>(a.x) + static_cast<int64_t>(b) * a.K + j * 32 + e * 4);
-          raw[0] = v.x; raw[1] = v.y; raw[2] = v.z; raw[3] = v.w;
-        } else if (a.x_kind == KIND_Q8_1) {
-          const uint8_t* blk = static_cast<const uint8_t*>(a.x) + (static_cast<int64_t>(b) * (a.K / 32) + j) * Q8_1_BYTES;
-          raw[0] = *reinterpret_cast<const uint32_t*>(blk + 4 + 4 * e);
-          raw[1] = *reinterpret_cast<const uint32_t*>(blk);
-        } else {
-          const uint2 h = *reinterpret_cast<const uint2*>(static_cast<const uint16_t*>(a.x) + static_cast<int64_t>(b) * a.K + j * 32 + e * 4);
-          raw[0] = h.x; raw[1] = h.y;
+    // large K: the rest is loaded here, four groups per thread at a time so that the
+    // load latency is paid once per four groups and not once per group
+    constexpr int P = 4;
+    for (int j0 = team + S * nteams; j0 < groups; j0 += P * nteams) {
+      uint32_t raw[P][4];
+#pragma unroll
+      for (int p = 0; p < P; ++p) {
+        const int j = j0 + p * nteams;
+        raw[p][0] = raw[p][1] = raw[p][2] = raw[p][3] = 0u;
+        if (b < a.rows && j < groups) {
+          if (a.x_kind == KIND_F32) {
+            const uint4 v = *reinterpret_cast<const uint4*>(static_cast<const float*>(a.x) + static_cast<int64_t>(b) * a.K + j * 32 + e * 4);
+            raw[p][0] = v.x; raw[p][1] = v.y; raw[p][2] = v.z; raw[p][3] = v.w;
+          } else if (a.x_kind == KIND_Q8_1) {
+            const uint8_t* blk = static_cast<const uint8_t*>(a.x) + (static_cast<int64_t>(b) * (a.K / 32) + j) * Q8_1_BYTES;
+            raw[p][0] = *reinterpret_cast<const uint32_t*>(blk + 4 + 4 * e);
+            raw[p][1] = *reinterpret_cast<const uint32_t*>(blk);
+          } else {
+            const uint2 h = *reinterpret_cast<const uint2*>(static_cast<const uint16_t*>(a.x) + static_cast<int64_t>(b) * a.K + j * 32 + e * 4);
+            raw[p][0] = h.x; raw[p][1] = h.y;
+          }
         }
       }
-      gemv_run_stage_one<QT>(a.x_kind, raw, b < a.rows, j, e, q8_row, rec_row, s16_row);
+#pragma unroll
+      for (int p = 0; p < P; ++p) {
+        const int j = j0 + p * nteams;
+        if (j < groups) gemv_run_stage_one<QT>(a.x_kind, raw[p], b < a.rows, j, e, q8_row, rec_row, s16_row);
+      }
     }
   }
 }
