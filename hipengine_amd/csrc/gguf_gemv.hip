@@ -203,47 +203,52 @@ int launch_gemv_run(int qt, const void* x, int x_kind, const uint8_t* w, void* o
 
 // ---- stream form (resident waves, ring of loads in flight) --------------------
 
-template <int QT, int B, int D, bool REFILL>
-__global__ void __launch_bounds__(512) gemv_stream_kernel(GemvStreamArgs a) {
+// Batch 1 kernels fit 170 registers and may run 12 waves per workgroup, which lets the
+// planner pick a wave count that divides the rows evenly.
+template <int B>
+constexpr int stream_max_threads() {
+  return B == 1 ? 768 : 512;
+}
+
+template <int QT, int B, int D, int S>
+__global__ void __launch_bounds__((stream_max_threads<B>())) gemv_stream_kernel(GemvStreamArgs a) {
   extern __shared__ __align__(16) uint8_t smem[];
-  gemv_stream_workgroup<QT, B, D, REFILL>(a, smem);
+  gemv_stream_workgroup<QT, B, D, S>(a, smem);
 }
 
 using StreamKernelFn = void (*)(GemvStreamArgs);
 
-// d > 0: ring of d loads, refilled as they are consumed.  d < 0: all of a wave's
-// loads (at most -d) are issued up front and none later.
+// `long_k`: the instantiation that fetches nine activation groups per thread up front
+// (batch 1 only); the other fetches three (batch 1, 2) or one (batch 4, 8).
 struct StreamVariant {
   int qt, b, d;
+  bool long_k;
   StreamKernelFn fn;
 };
 
 #define STREAM_VARIANT(QT, B, D) \
-  StreamVariant { QT, B, D, gemv_stream_kernel<QT, B, D, true> }
-#define STREAM_UPFRONT(QT, B, D) \
-  StreamVariant { QT, B, -D, gemv_stream_kernel<QT, B, D, false> }
+  StreamVariant { QT, B, D, false, gemv_stream_kernel<QT, B, D, (B <= 2 ? 3 : 1)> }
+#define STREAM_VARIANT_LONG_K(QT, D) \
+  StreamVariant { QT, 1, D, true, gemv_stream_kernel<QT, 1, D, 9> }
 
 const StreamVariant kStream[] = {
     STREAM_VARIANT(GGML_Q4_K, 1, 3), STREAM_VARIANT(GGML_Q4_K, 1, 5), STREAM_VARIANT(GGML_Q4_K, 2, 3),
     STREAM_VARIANT(GGML_Q4_K, 2, 5), STREAM_VARIANT(GGML_Q6_K, 1, 3), STREAM_VARIANT(GGML_Q6_K, 1, 5),
     STREAM_VARIANT(GGML_Q6_K, 2, 3), STREAM_VARIANT(GGML_Q6_K, 2, 5), STREAM_VARIANT(GGML_Q8_0, 1, 3),
     STREAM_VARIANT(GGML_Q8_0, 1, 5), STREAM_VARIANT(GGML_Q8_0, 2, 3), STREAM_VARIANT(GGML_Q8_0, 2, 5),
-    STREAM_VARIANT(GGML_Q4_K, 1, 4), STREAM_VARIANT(GGML_Q4_K, 1, 6), STREAM_VARIANT(GGML_Q4_K, 2, 4),
-    STREAM_VARIANT(GGML_Q4_K, 2, 6), STREAM_VARIANT(GGML_Q6_K, 1, 4), STREAM_VARIANT(GGML_Q8_0, 1, 4),
+    STREAM_VARIANT_LONG_K(GGML_Q4_K, 3), STREAM_VARIANT_LONG_K(GGML_Q6_K, 3), STREAM_VARIANT_LONG_K(GGML_Q8_0, 3),
     STREAM_VARIANT(GGML_Q4_K, 4, 3), STREAM_VARIANT(GGML_Q4_K, 8, 3), STREAM_VARIANT(GGML_Q6_K, 4, 3),
     STREAM_VARIANT(GGML_Q6_K, 8, 3), STREAM_VARIANT(GGML_Q8_0, 4, 3), STREAM_VARIANT(GGML_Q8_0, 8, 3),
-    STREAM_UPFRONT(GGML_Q4_K, 1, 6), STREAM_UPFRONT(GGML_Q4_K, 1, 8), STREAM_UPFRONT(GGML_Q4_K, 1, 12),
-    STREAM_UPFRONT(GGML_Q4_K, 2, 6), STREAM_UPFRONT(GGML_Q4_K, 2, 8), STREAM_UPFRONT(GGML_Q4_K, 2, 12),
-    STREAM_UPFRONT(GGML_Q6_K, 1, 6), STREAM_UPFRONT(GGML_Q6_K, 1, 8), STREAM_UPFRONT(GGML_Q6_K, 1, 12),
-    STREAM_UPFRONT(GGML_Q6_K, 2, 6), STREAM_UPFRONT(GGML_Q6_K, 2, 8), STREAM_UPFRONT(GGML_Q6_K, 2, 12),
-    STREAM_UPFRONT(GGML_Q8_0, 1, 6), STREAM_UPFRONT(GGML_Q8_0, 1, 8), STREAM_UPFRONT(GGML_Q8_0, 1, 12),
-    STREAM_UPFRONT(GGML_Q8_0, 2, 6), STREAM_UPFRONT(GGML_Q8_0, 2, 8), STREAM_UPFRONT(GGML_Q8_0, 2, 12),
 };
 
-const StreamVariant* find_stream_variant(int qt, int b, int d) {
-  for (const StreamVariant& v : kStream)
-    if (v.qt == qt && v.b == b && v.d == d) return &v;
-  return nullptr;
+const StreamVariant* find_stream_variant(int qt, int b, int d, bool long_k = false) {
+  const StreamVariant* fallback = nullptr;
+  for (const StreamVariant& v : kStream) {
+    if (v.qt != qt || v.b != b || v.d != d) continue;
+    if (v.long_k == long_k) return &v;
+    if (!v.long_k) fallback = &v;
+  }
+  return fallback;
 }
 
 int batch_bucket(int rows) { return rows <= 1 ? 1 : rows <= 2 ? 2 : rows <= 4 ? 4 : 8; }
@@ -252,12 +257,6 @@ struct StreamPlan {
   int b, d, waves, waves_total;
   bool ok;
 };
-
-// Most 16-block loads any wave has: rows are split as evenly as possible.
-int64_t stream_max_loads(int64_t N, int nb, int waves_total) {
-  const int64_t rows = (N + waves_total - 1) / waves_total;
-  return (rows * nb + 15) / 16;
-}
 
 constexpr int kComputeUnits = 256;   // MI355X
 
@@ -272,6 +271,17 @@ StreamPlan default_stream_plan(int qt, int rows, int64_t K, int64_t N) {
   const int64_t total_loads = N * nb / 16;
   // 8 resident waves per CU once every wave gets 3 loads or more, else 4 per CU
   p.waves_total = total_loads >= 6144 ? kComputeUnits * 8 : kComputeUnits * 4;
+  if (p.b == 1 && total_loads >= 6144) {
+    // whole rows per wave: 8, 10 or 12 waves per CU, whichever splits the rows most
+    // evenly (N = 5120: 2.5 rows per wave at 8, exactly 2 at 10)
+    double best = 1e9;
+    for (int w = 8; w <= 12; w += 2) {
+      const int64_t wt = static_cast<int64_t>(kComputeUnits) * w;
+      if (wt > N) break;
+      const double imbalance = static_cast<double>((N + wt - 1) / wt) * wt / static_cast<double>(N);
+      if (imbalance < best - 0.1) { best = imbalance; p.waves = w; p.waves_total = static_cast<int>(wt); }
+    }
+  }
   p.ok = rows <= 8 && nb >= 16 && total_loads >= 3 * static_cast<int64_t>(p.waves_total) &&
          N >= p.waves_total && gemv_run_lds_bytes(qt, p.b, static_cast<int>(K)) <= 64 * 1024 &&
          find_stream_variant(qt, p.b, p.d) != nullptr;
@@ -280,11 +290,11 @@ StreamPlan default_stream_plan(int qt, int rows, int64_t K, int64_t N) {
 
 int launch_gemv_stream(int qt, const void* x, int x_kind, const uint8_t* w, void* out, int out_kind, int rows,
                        int64_t K, int64_t N, const StreamPlan& p, hipStream_t stream) {
-  const StreamVariant* v = find_stream_variant(qt, p.b, p.d);
   const int nb = static_cast<int>(K / QK_K);
-  if (!v || nb < 16 || rows > p.b || p.waves < 1 || p.waves > 8 || p.waves_total < p.waves ||
-      (p.waves_total % p.waves) != 0 || p.waves_total > N ||
-      (p.d < 0 && stream_max_loads(N, nb, p.waves_total) > -p.d)) {
+  // more than three activation groups per thread: take the instantiation that fetches nine up front
+  const StreamVariant* v = find_stream_variant(qt, p.b, p.d, p.waves > 0 && nb > 3 * p.waves);
+  if (!v || nb < 16 || rows > p.b || p.waves < 1 || p.waves > (p.b == 1 ? 12 : 8) || p.waves_total < p.waves ||
+      (p.waves_total % p.waves) != 0 || p.waves_total > N) {
     return static_cast<int>(hipErrorInvalidValue);
   }
   const size_t lds = gemv_run_lds_bytes(qt, p.b, static_cast<int>(K));

@@ -39,10 +39,7 @@ struct GemvStreamArgs {
   int waves_total;  // waves in the whole grid (grid * waves)
 };
 
-// REFILL = false: the wave has at most D loads in all (checked by the launcher),
-// every one of them is issued before the activations are staged and none is
-// issued later, so the whole matrix is in flight from the first microsecond.
-template <int QT, int B, int D, bool REFILL = true>
+template <int QT, int B, int D, int S>
 __device__ __forceinline__ void gemv_stream_workgroup(const GemvStreamArgs& a, uint8_t* smem) {
   using Regs = WeightRegs<GemvTraits<QT>::REGS>;
   constexpr int Q8S = run_q8_stride<QT>();
@@ -65,7 +62,9 @@ __device__ __forceinline__ void gemv_stream_workgroup(const GemvStreamArgs& a, u
   int* s16 = reinterpret_cast<int*>(rec + B * nb * 16);
 
   // Activation loads go first (see gemv_run_stage_fetch), then the weight ring.
-  constexpr int S = B <= 2 ? 3 : 1;   // activation groups fetched ahead of the weight ring, per batch row
+  // S activation groups per thread have their loads issued ahead of the weight ring,
+  // per batch row.  Loads issued after the ring queue behind it (the memory counter
+  // retires in order), so a long K wants them all up front: nine cover K = 17408.
   const GemvRunArgs ra{a.x, a.w, a.out, a.x_kind, a.out_kind, a.rows, a.K, a.N, a.waves};
   StageRegs<B, S> sr;
   gemv_run_stage_fetch<QT, B, S>(ra, sr);
@@ -106,7 +105,7 @@ __device__ __forceinline__ void gemv_stream_workgroup(const GemvStreamArgs& a, u
     }
   };
 
-  for (int i0 = 0; i0 < (REFILL ? nloads : 1); i0 += D) {
+  for (int i0 = 0; i0 < nloads; i0 += D) {
 #pragma unroll
     for (int c = 0; c < D; ++c) {
       const int i = i0 + c;
@@ -120,7 +119,7 @@ __device__ __forceinline__ void gemv_stream_workgroup(const GemvStreamArgs& a, u
         acc_cur[b] += (lrow == row_lo) ? term : 0.0f;
         acc_next[b] += (lrow == row_lo) ? 0.0f : term;
       }
-      if (REFILL) issue(i + D, ring[c]);
+      issue(i + D, ring[c]);
       // advance the lane to load i+1
       kb += step_kb; lrow += step_r;
       if (kb >= nb) { kb -= nb; lrow += 1; }
