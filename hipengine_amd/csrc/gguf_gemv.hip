@@ -210,10 +210,10 @@ constexpr int stream_max_threads() {
   return B == 1 ? 768 : 512;
 }
 
-template <int QT, int B, int D, int S>
+template <int QT, int B, int D, int S, int XK = -1>
 __global__ void __launch_bounds__((stream_max_threads<B>())) gemv_stream_kernel(GemvStreamArgs a) {
   extern __shared__ __align__(16) uint8_t smem[];
-  gemv_stream_workgroup<QT, B, D, S>(a, smem);
+  gemv_stream_workgroup<QT, B, D, S, XK>(a, smem);
 }
 
 using StreamKernelFn = void (*)(GemvStreamArgs);
@@ -224,19 +224,23 @@ struct StreamVariant {
   int qt, b, d;
   bool long_k;
   StreamKernelFn fn;
+  StreamKernelFn by_kind[4];   // instantiations with the activation kind fixed (null: use fn)
 };
 
 #define STREAM_VARIANT(QT, B, D) \
-  StreamVariant { QT, B, D, false, gemv_stream_kernel<QT, B, D, (B <= 2 ? 3 : 1)> }
-#define STREAM_VARIANT_LONG_K(QT, D) \
-  StreamVariant { QT, 1, D, true, gemv_stream_kernel<QT, 1, D, 9> }
+  StreamVariant { QT, B, D, false, gemv_stream_kernel<QT, B, D, (B <= 2 ? 3 : 1)>, {nullptr, nullptr, nullptr, nullptr} }
+#define STREAM_VARIANT_BY_KIND(QT, B, D, S, LONG_K)                                                      \
+  StreamVariant { QT, B, D, LONG_K, gemv_stream_kernel<QT, B, D, S>,                                      \
+                  {gemv_stream_kernel<QT, B, D, S, KIND_F32>, gemv_stream_kernel<QT, B, D, S, KIND_BF16>, \
+                   gemv_stream_kernel<QT, B, D, S, KIND_F16>, gemv_stream_kernel<QT, B, D, S, KIND_Q8_1>} }
 
 const StreamVariant kStream[] = {
-    STREAM_VARIANT(GGML_Q4_K, 1, 3), STREAM_VARIANT(GGML_Q4_K, 1, 5), STREAM_VARIANT(GGML_Q4_K, 2, 3),
-    STREAM_VARIANT(GGML_Q4_K, 2, 5), STREAM_VARIANT(GGML_Q6_K, 1, 3), STREAM_VARIANT(GGML_Q6_K, 1, 5),
-    STREAM_VARIANT(GGML_Q6_K, 2, 3), STREAM_VARIANT(GGML_Q6_K, 2, 5), STREAM_VARIANT(GGML_Q8_0, 1, 3),
+    STREAM_VARIANT_BY_KIND(GGML_Q4_K, 1, 3, 3, false), STREAM_VARIANT(GGML_Q4_K, 1, 5), STREAM_VARIANT(GGML_Q4_K, 2, 3),
+    STREAM_VARIANT(GGML_Q4_K, 2, 5), STREAM_VARIANT_BY_KIND(GGML_Q6_K, 1, 3, 3, false), STREAM_VARIANT(GGML_Q6_K, 1, 5),
+    STREAM_VARIANT(GGML_Q6_K, 2, 3), STREAM_VARIANT(GGML_Q6_K, 2, 5), STREAM_VARIANT_BY_KIND(GGML_Q8_0, 1, 3, 3, false),
     STREAM_VARIANT(GGML_Q8_0, 1, 5), STREAM_VARIANT(GGML_Q8_0, 2, 3), STREAM_VARIANT(GGML_Q8_0, 2, 5),
-    STREAM_VARIANT_LONG_K(GGML_Q4_K, 3), STREAM_VARIANT_LONG_K(GGML_Q6_K, 3), STREAM_VARIANT_LONG_K(GGML_Q8_0, 3),
+    STREAM_VARIANT_BY_KIND(GGML_Q4_K, 1, 3, 9, true), STREAM_VARIANT_BY_KIND(GGML_Q6_K, 1, 3, 9, true),
+    STREAM_VARIANT_BY_KIND(GGML_Q8_0, 1, 3, 9, true),
     STREAM_VARIANT(GGML_Q4_K, 4, 3), STREAM_VARIANT(GGML_Q4_K, 8, 3), STREAM_VARIANT(GGML_Q6_K, 4, 3),
     STREAM_VARIANT(GGML_Q6_K, 8, 3), STREAM_VARIANT(GGML_Q8_0, 4, 3), STREAM_VARIANT(GGML_Q8_0, 8, 3),
 };
@@ -304,7 +308,9 @@ int launch_gemv_stream(int qt, const void* x, int x_kind, const uint8_t* w, void
   a.x_kind = x_kind; a.out_kind = out_kind;
   a.rows = rows; a.K = static_cast<int>(K); a.N = static_cast<int>(N);
   a.waves = p.waves; a.waves_total = p.waves_total;
-  hipLaunchKernelGGL(v->fn, dim3(p.waves_total / p.waves), dim3(p.waves * 64), lds, stream, a);
+  a.base_rows = static_cast<int>(N / p.waves_total);
+  const StreamKernelFn fn = (x_kind >= KIND_F32 && x_kind <= KIND_Q8_1 && v->by_kind[x_kind]) ? v->by_kind[x_kind] : v->fn;
+  hipLaunchKernelGGL(fn, dim3(p.waves_total / p.waves), dim3(p.waves * 64), lds, stream, a);
   return static_cast<int>(hipGetLastError());
 }
 

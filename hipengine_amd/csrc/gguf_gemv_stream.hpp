@@ -37,9 +37,14 @@ struct GemvStreamArgs {
   int N;
   int waves;        // waves per workgroup
   int waves_total;  // waves in the whole grid (grid * waves)
+  int base_rows;    // N / waves_total (computed on the host: an integer division is ~40 instructions here)
 };
 
-template <int QT, int B, int D, int S>
+// XK >= 0 fixes the activation kind at compile time (the staging code of the other
+// kinds is then not generated: a decode kernel runs its prologue once per launch
+// with a cold instruction cache, so prologue code size is launch latency), XK < 0
+// reads it from the arguments.
+template <int QT, int B, int D, int S, int XK = -1>
 __device__ __forceinline__ void gemv_stream_workgroup(const GemvStreamArgs& a, uint8_t* smem) {
   using Regs = WeightRegs<GemvTraits<QT>::REGS>;
   constexpr int Q8S = run_q8_stride<QT>();
@@ -50,7 +55,7 @@ __device__ __forceinline__ void gemv_stream_workgroup(const GemvStreamArgs& a, u
 
   // rows [r0, r0 + nrows) of this wave: N split as evenly as possible
   const int gw = blockIdx.x * a.waves + wave;
-  const int base_rows = a.N / a.waves_total, extra = a.N % a.waves_total;
+  const int base_rows = a.base_rows, extra = a.N - a.base_rows * a.waves_total;
   const int r0 = gw * base_rows + min(gw, extra);
   const int nrows = base_rows + (gw < extra ? 1 : 0);
   const int run_blocks = nrows * nb;
@@ -65,7 +70,7 @@ __device__ __forceinline__ void gemv_stream_workgroup(const GemvStreamArgs& a, u
   // S activation groups per thread have their loads issued ahead of the weight ring,
   // per batch row.  Loads issued after the ring queue behind it (the memory counter
   // retires in order), so a long K wants them all up front: nine cover K = 17408.
-  const GemvRunArgs ra{a.x, a.w, a.out, a.x_kind, a.out_kind, a.rows, a.K, a.N, a.waves};
+  const GemvRunArgs ra{a.x, a.w, a.out, XK >= 0 ? XK : a.x_kind, a.out_kind, a.rows, a.K, a.N, a.waves};
   StageRegs<B, S> sr;
   gemv_run_stage_fetch<QT, B, S>(ra, sr);
 

@@ -166,6 +166,10 @@ def test_prequantized_gemv_matches_fused_bit_for_bit(dev, quant, fn):
     rng = np.random.default_rng(33)
     rows, k, n = 4, 2048, 80
     x = rng.standard_normal((rows, k)).astype(np.float32)
+    x[1, 64:96] *= np.float32(1e-36)         # scale in the denormal range
+    x[2, :32] = np.arange(-16, 16) / 8.0     # exact .5 ties
+    x[2, 31] = 127.0 / 8.0
+    x[3, 128:160] *= np.float32(3e4)
     w = O.random_weight(QT[quant], n, k, seed=4)
     fused = _run_fused(dev, quant, x, w)
     xq = O.quantize_q8_1(x)
