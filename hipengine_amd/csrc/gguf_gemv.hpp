@@ -335,9 +335,15 @@ inline size_t gemv_lds_bytes(int qt, int B, int R, int CB, int ks, int nrg) {
 // row `row` < N), from the thread that summed its K-slices.  A caller that runs
 // the body more than once in a kernel separates the calls with a barrier, as
 // the LDS staging area is reused.
-template <int QT, int B, int R, int CB, class Emit>
+//
+// DUAL (R == 2, B == 1): the lane's two rows are the SAME row index of two matrices
+// `w` and `w2` (a gate/up pair), so one pass with one staging of the activations
+// yields both; the workgroup then owns nrg*16 output rows and `emit` receives the
+// matrix (0 or 1) in place of the batch row.
+template <int QT, int B, int R, int CB, bool DUAL = false, class Emit>
 __device__ __forceinline__ void gemv_workgroup_emit(const GemvArgs& a, const uint8_t* w, int first_row, uint8_t* smem,
-                                                    Emit emit) {
+                                                    Emit emit, const uint8_t* w2 = nullptr) {
+  static_assert(!DUAL || (R == 2 && B == 1), "the dual form pairs two matrices at batch 1");
   using Regs = WeightRegs<GemvTraits<QT>::REGS>;
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int kslice = wave % a.ks, rowgrp = wave / a.ks;
@@ -359,8 +365,9 @@ __device__ __forceinline__ void gemv_workgroup_emit(const GemvArgs& a, const uin
   const uint8_t* wrow[R];
 #pragma unroll
   for (int r = 0; r < R; ++r) {
-    const int row = min(first_row + rowgrp * 16 * R + 16 * r + rg, a.N - 1);
-    wrow[r] = w + static_cast<int64_t>(row) * row_bytes;
+    const int row = DUAL ? min(first_row + rowgrp * 16 + rg, a.N - 1)
+                         : min(first_row + rowgrp * 16 * R + 16 * r + rg, a.N - 1);
+    wrow[r] = ((DUAL && r == 1) ? w2 : w) + static_cast<int64_t>(row) * row_bytes;
   }
 
   float acc[R][B];
@@ -410,18 +417,19 @@ __device__ __forceinline__ void gemv_workgroup_emit(const GemvArgs& a, const uin
   __syncthreads();
   for (int idx = tid; idx < rows_wg * B; idx += blockDim.x) {
     const int b = idx / rows_wg, rl = idx - b * rows_wg;
-    const int row = first_row + rl;
+    const int which = (rl >> 4) & 1;                                  // DUAL: 16 rows of w, then 16 of w2, per row group
+    const int row = DUAL ? first_row + (rl >> 5) * 16 + (rl & 15) : first_row + rl;
     if (row < a.N && b < a.rows) {
       float v = 0.0f;
       for (int s = 0; s < a.ks; ++s) v += red[(s * B + b) * rows_wg + rl];
-      emit(b, row, v);
+      emit(DUAL ? which : b, row, v);
     }
   }
 }
 
 template <int QT, int B, int R, int CB>
 __device__ __forceinline__ void gemv_workgroup(const GemvArgs& a, const uint8_t* w, int first_row, uint8_t* smem) {
-  gemv_workgroup_emit<QT, B, R, CB>(a, w, first_row, smem, [&](int b, int row, float v) {
+  gemv_workgroup_emit<QT, B, R, CB, false>(a, w, first_row, smem, [&](int b, int row, float v) {
     store_scalar(a.out, static_cast<int64_t>(b) * a.N + row, v, a.out_kind);
   });
 }

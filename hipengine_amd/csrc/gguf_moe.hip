@@ -234,82 +234,135 @@ struct SelArgs {
   int num_experts;
   int top_k;
   int round_mid;              // dual: round gate and up to the output type before silu (the fused device form)
+  int pair_offset;            // dual: byte offset in LDS of the [2][rows] gate/up exchange buffer
 };
 
 __device__ __forceinline__ int64_t scalar_bytes(int kind) { return kind == KIND_F32 ? 4 : 2; }
 
 // Workgroup size cap: the CB weight blocks of a chunk have to fit the VGPR
 // budget the cap implies (128 registers at 1024 threads, 256 at 512).
-template <int QT, int CB>
+template <int QT, int BLOCKS>
 constexpr int sel_max_threads() {
-  return CB * GemvTraits<QT>::REGS <= 64 ? 1024 : 512;
+  return BLOCKS * GemvTraits<QT>::REGS <= 48 ? 1024 : 512;
 }
 
 template <int QT, int R, int CB, int MODE>
-__global__ void __launch_bounds__((sel_max_threads<QT, CB>())) selected_gemv_kernel(SelArgs s) {
+__global__ void __launch_bounds__((sel_max_threads<QT, R * CB>())) selected_gemv_kernel(SelArgs s) {
   extern __shared__ __align__(16) uint8_t smem[];
-  const int rows_wg = s.g.nrg * 16 * R;
-  const int first_row = blockIdx.x * rows_wg;
   const int64_t row_bytes = static_cast<int64_t>(s.g.K / QK_K) * GemvTraits<QT>::SUPER_BYTES;
   const int64_t expert_bytes = static_cast<int64_t>(s.g.N) * row_bytes;
   GemvArgs a = s.g;
   a.rows = 1;
-
-  if constexpr (MODE == SEL_DOWN_SUM) {
-    const int t = blockIdx.y;
-    float total = 0.0f;
-    int my_row = -1;
-    for (int slot = 0; slot < s.top_k; ++slot) {
-      const int lane = t * s.top_k + slot;
-      const int64_t e = s.selected[lane];
-      if (e < 0 || e >= s.num_experts) continue;          // uniform over the workgroup
-      const float wgt = s.routing[lane];
-      a.x = static_cast<const uint8_t*>(s.g.x) + static_cast<int64_t>(lane) * s.g.K * scalar_bytes(s.g.x_kind);
-      __syncthreads();
-      gemv_workgroup_emit<QT, 1, R, CB>(a, s.g.w + e * expert_bytes, first_row, smem, [&](int, int row, float v) {
-        total += wgt * v;
-        my_row = row;
-      });
-    }
-    if (my_row >= 0) store_scalar(s.g.out, static_cast<int64_t>(t) * s.g.N + my_row, total, s.g.out_kind);
-    // rows whose token selected no valid expert at all are written as zero
-    if (my_row < 0) {
-      bool any = false;
-      for (int slot = 0; slot < s.top_k; ++slot) {
-        const int64_t e = s.selected[t * s.top_k + slot];
-        any |= (e >= 0 && e < s.num_experts);
-      }
-      if (!any)
-        for (int r = threadIdx.x; r < rows_wg; r += blockDim.x)
-          if (first_row + r < s.g.N) store_scalar(s.g.out, static_cast<int64_t>(t) * s.g.N + first_row + r, 0.0f, s.g.out_kind);
-    }
+  const int lane = blockIdx.y;
+  const int64_t e = s.selected[lane];
+  if (e < 0 || e >= s.num_experts) return;
+  const int per = s.lanes / s.x_rows;
+  const int x_row = s.x_rows == 1 ? 0 : lane / per;
+  a.x = static_cast<const uint8_t*>(s.g.x) + static_cast<int64_t>(x_row) * s.g.K * scalar_bytes(s.g.x_kind);
+  a.out = static_cast<uint8_t*>(s.g.out) + static_cast<int64_t>(lane) * s.g.N * scalar_bytes(s.g.out_kind);
+  if constexpr (MODE == SEL_SINGLE) {
+    gemv_workgroup<QT, 1, R, CB>(a, s.g.w + e * expert_bytes, blockIdx.x * s.g.nrg * 16 * R, smem);
   } else {
-    const int lane = blockIdx.y;
-    const int64_t e = s.selected[lane];
-    if (e < 0 || e >= s.num_experts) return;
-    const int per = s.lanes / s.x_rows;
-    const int x_row = s.x_rows == 1 ? 0 : lane / per;
-    a.x = static_cast<const uint8_t*>(s.g.x) + static_cast<int64_t>(x_row) * s.g.K * scalar_bytes(s.g.x_kind);
-    a.out = static_cast<uint8_t*>(s.g.out) + static_cast<int64_t>(lane) * s.g.N * scalar_bytes(s.g.out_kind);
-    if constexpr (MODE == SEL_SINGLE) {
-      gemv_workgroup<QT, 1, R, CB>(a, s.g.w + e * expert_bytes, first_row, smem);
-    } else {
-      float gate = 0.0f;
-      gemv_workgroup_emit<QT, 1, R, CB>(a, s.g.w + e * expert_bytes, first_row, smem,
-                                       [&](int, int, float v) { gate = v; });
-      __syncthreads();
-      gemv_workgroup_emit<QT, 1, R, CB>(a, s.w_b + e * expert_bytes, first_row, smem, [&](int, int row, float up) {
-        float gv = gate, uv = up;
-        if (s.round_mid && a.out_kind == KIND_BF16) {
-          gv = bf16_bits_to_float(float_to_bf16_bits(gv));
-          uv = bf16_bits_to_float(float_to_bf16_bits(uv));
-        } else if (s.round_mid && a.out_kind == KIND_F16) {
-          gv = f16_bits_to_float(float_to_f16_bits(gv));
-          uv = f16_bits_to_float(float_to_f16_bits(uv));
-        }
-        store_scalar(a.out, row, silu_mul(gv, uv), a.out_kind);
-      });
+    // gate and up rows of the same index in one pass: one staging of the activations,
+    // all weight loads of both matrices in flight together
+    static_assert(R == 2, "the gate/up form pairs two matrices");
+    const int rows_out = s.g.nrg * 16;
+    const int first_row = blockIdx.x * rows_out;
+    float* pair = reinterpret_cast<float*>(smem + s.pair_offset);      // [2][rows_out]
+    gemv_workgroup_emit<QT, 1, 2, CB, true>(
+        a, s.g.w + e * expert_bytes, first_row, smem,
+        [&](int which, int row, float v) { pair[which * rows_out + (row - first_row)] = v; }, s.w_b + e * expert_bytes);
+    __syncthreads();
+    const int i = threadIdx.x;
+    if (i < rows_out && first_row + i < s.g.N) {
+      float gv = pair[i], uv = pair[rows_out + i];
+      if (s.round_mid && a.out_kind == KIND_BF16) {
+        gv = bf16_bits_to_float(float_to_bf16_bits(gv));
+        uv = bf16_bits_to_float(float_to_bf16_bits(uv));
+      } else if (s.round_mid && a.out_kind == KIND_F16) {
+        gv = f16_bits_to_float(float_to_f16_bits(gv));
+        uv = f16_bits_to_float(float_to_f16_bits(uv));
+      }
+      store_scalar(a.out, first_row + i, silu_mul(gv, uv), a.out_kind);
     }
+  }
+}
+
+// Routed down projection of one token: out[t, row] = sum over slots s, in slot order, of
+// routing[t*top_k + s] * (W[selected[t*top_k + s]] . x[t*top_k + s]).
+// One workgroup per (16 output rows, token); its waves are (slot, K slice) pairs, so the
+// weight blocks of all the token's experts are in flight together and the activations
+// of all slots (top_k consecutive rows of x) are quantized in one pass per K chunk.
+template <int QT, int TK, int RG>
+__global__ void __launch_bounds__(1024) selected_down_sum_kernel(SelArgs s) {
+  extern __shared__ __align__(16) uint8_t smem[];
+  using Regs = WeightRegs<GemvTraits<QT>::REGS>;
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int ks = s.g.ks;                       // K slices per slot; waves = TK * ks
+  const int slot = wave / ks, kslice = wave - slot * ks;
+  const int q = lane & 3, rg = lane >> 2;
+  const int t = blockIdx.y;
+  const int first_row = blockIdx.x * 16 * RG;  // RG groups of 16 rows share one staging of the activations
+  const int nb = s.g.K / QK_K;
+  const int chunk_elems = ks * QK_K, chunk_sb = ks * 8;
+  const int64_t row_bytes = static_cast<int64_t>(nb) * GemvTraits<QT>::SUPER_BYTES;
+  const int64_t expert_bytes = static_cast<int64_t>(s.g.N) * row_bytes;
+
+  uint8_t* q8 = smem;
+  float* xd = reinterpret_cast<float*>(q8 + TK * chunk_elems);
+  float* xs = xd + TK * chunk_sb;
+  int* s16 = reinterpret_cast<int*>(xs);
+  float* red = (QT == GGML_Q4_K) ? xs + TK * chunk_sb
+             : (QT == GGML_Q6_K) ? reinterpret_cast<float*>(s16 + TK * chunk_sb * 2)
+                                 : xs;                                  // [TK][ks][16 * RG]
+  GemvArgs a = s.g;
+  a.rows = s.top_k;
+  a.x = static_cast<const uint8_t*>(s.g.x) + static_cast<int64_t>(t) * s.top_k * s.g.K * scalar_bytes(s.g.x_kind);
+  ActTile tile{q8, xd, xs, s16, chunk_elems, chunk_sb};
+
+  const int64_t e = slot < s.top_k ? s.selected[t * s.top_k + slot] : -1;
+  const bool valid = e >= 0 && e < s.num_experts;
+  const uint8_t* wexp = s.g.w + (valid ? e : 0) * expert_bytes;
+
+  float acc[RG];
+#pragma unroll
+  for (int g = 0; g < RG; ++g) acc[g] = 0.0f;
+  for (int kc = 0; kc < nb; kc += ks) {
+    Regs wr[RG];
+    const int kb = kc + kslice;
+    const bool live = valid && kb < nb;
+#pragma unroll
+    for (int g = 0; g < RG; ++g) {
+      const int row = min(first_row + 16 * g + rg, s.g.N - 1);
+      gemv_load_block<QT>(wexp + static_cast<int64_t>(row) * row_bytes +
+                              static_cast<int64_t>(min(kb, nb - 1)) * GemvTraits<QT>::SUPER_BYTES, q, wr[g]);
+    }
+    if (kc > 0) __syncthreads();
+    gemv_stage_activations<QT, TK>(a, kc, ks, q8, xd, xs, s16, chunk_elems, chunk_sb);
+    __syncthreads();
+#pragma unroll
+    for (int g = 0; g < RG; ++g) {
+      const BlockScales<QT> sc = gemv_block_scales<QT>(wr[g], q);
+      const float term = gemv_block_term<QT>(wr[g], sc, q, tile, slot, kslice);
+      acc[g] += live ? term : 0.0f;
+    }
+  }
+#pragma unroll
+  for (int g = 0; g < RG; ++g) {
+    const float v = quad_sum(acc[g]);
+    if (q == 0) red[(slot * ks + kslice) * 16 * RG + 16 * g + rg] = v;
+  }
+  __syncthreads();
+  if (tid < 16 * RG && first_row + tid < s.g.N) {
+    float total = 0.0f;
+    for (int sl = 0; sl < s.top_k; ++sl) {
+      const int64_t es = s.selected[t * s.top_k + sl];
+      if (es < 0 || es >= s.num_experts) continue;
+      float dot = 0.0f;
+      for (int k = 0; k < ks; ++k) dot += red[(sl * ks + k) * 16 * RG + tid];
+      total += s.routing[t * s.top_k + sl] * dot;
+    }
+    store_scalar(s.g.out, static_cast<int64_t>(t) * s.g.N + first_row + tid, total, s.g.out_kind);
   }
 }
 
@@ -318,10 +371,9 @@ struct SelVariant {
   int qt, cb, mode, max_threads;
   SelFn fn;
 };
-#define SEL_VARIANTS(QT, CB)                                                                       \
-  SelVariant{QT, CB, SEL_SINGLE, sel_max_threads<QT, CB>(), selected_gemv_kernel<QT, 1, CB, SEL_SINGLE>},       \
-  SelVariant{QT, CB, SEL_DUAL_SILU, sel_max_threads<QT, CB>(), selected_gemv_kernel<QT, 1, CB, SEL_DUAL_SILU>}, \
-  SelVariant{QT, CB, SEL_DOWN_SUM, sel_max_threads<QT, CB>(), selected_gemv_kernel<QT, 1, CB, SEL_DOWN_SUM>}
+#define SEL_VARIANTS(QT, CB)                                                                                   \
+  SelVariant{QT, CB, SEL_SINGLE, sel_max_threads<QT, CB>(), selected_gemv_kernel<QT, 1, CB, SEL_SINGLE>},         \
+  SelVariant{QT, CB, SEL_DUAL_SILU, sel_max_threads<QT, 2 * CB>(), selected_gemv_kernel<QT, 2, CB, SEL_DUAL_SILU>}
 const SelVariant kSel[] = {
     SEL_VARIANTS(GGML_Q4_K, 1), SEL_VARIANTS(GGML_Q4_K, 2), SEL_VARIANTS(GGML_Q4_K, 5),
     SEL_VARIANTS(GGML_Q6_K, 1), SEL_VARIANTS(GGML_Q6_K, 2), SEL_VARIANTS(GGML_Q6_K, 5),
@@ -332,32 +384,71 @@ int launch_selected(int qt, int mode, const void* x, int x_kind, const int64_t* 
                     int64_t num_experts, int64_t top_k, int64_t K, int64_t N, int round_mid, hipStream_t stream) {
   if (!x || !selected || !w_a || !out || x_rows <= 0 || lanes <= 0 || lanes > 65535 || num_experts <= 0 || K <= 0 ||
       (K % QK_K) != 0 || K > (1 << 20) || N <= 0 || N > (1 << 24) || x_kind < KIND_F32 || x_kind > KIND_F16 ||
-      out_kind < KIND_F32 || out_kind > KIND_F16) {
+      out_kind < KIND_F32 || out_kind > KIND_F16 || (qt != GGML_Q4_K && qt != GGML_Q6_K)) {
     return static_cast<int>(hipErrorInvalidValue);
   }
   if (mode == SEL_DUAL_SILU && !w_b) return static_cast<int>(hipErrorInvalidValue);
-  if (mode == SEL_DOWN_SUM && (!routing || top_k <= 0 || lanes != x_rows * top_k)) return static_cast<int>(hipErrorInvalidValue);
+  if (mode == SEL_DOWN_SUM && (!routing || top_k <= 0 || top_k > 8 || lanes != x_rows * top_k)) {
+    return static_cast<int>(hipErrorInvalidValue);
+  }
   if (mode != SEL_DOWN_SUM && (lanes % x_rows) != 0) return static_cast<int>(hipErrorInvalidValue);
   const int nb = static_cast<int>(K / QK_K);
-  const int ks = nb >= 4 ? 4 : nb;
-  const int per_wave = (nb + ks - 1) / ks;
-  const int cb = per_wave >= 5 ? 5 : per_wave >= 2 ? 2 : 1;
-  const int64_t groups = mode == SEL_DOWN_SUM ? x_rows : lanes;   // grid.y
+  SelArgs s;
+  s.g.x = x; s.g.w = w_a; s.g.out = out; s.g.x_kind = x_kind; s.g.out_kind = out_kind; s.g.rows = 1;
+  s.g.K = static_cast<int>(K); s.g.N = static_cast<int>(N);
+  s.w_b = w_b; s.selected = selected; s.routing = routing;
+  s.x_rows = static_cast<int>(x_rows); s.lanes = static_cast<int>(lanes);
+  s.num_experts = static_cast<int>(num_experts); s.top_k = static_cast<int>(top_k); s.round_mid = round_mid;
+  s.pair_offset = 0;
+
+  if (mode == SEL_DOWN_SUM) {
+    // waves = 8 slots x ks K slices <= 16; one or two groups of 16 rows per workgroup, one as
+    // long as the grid stays above ~2 workgroups per CU
+    const int ks = nb >= 2 ? 2 : 1;
+    int rgn = 2;
+    while (rgn > 1 && (N + 16 * rgn - 1) / (16 * rgn) * x_rows < 512) rgn >>= 1;
+    s.g.ks = ks; s.g.nrg = rgn;
+    const size_t lds = gemv_lds_bytes(qt, 8, 1, 1, ks, 1) + static_cast<size_t>(8) * ks * 16 * rgn * 4;
+    if (lds > 64 * 1024) return static_cast<int>(hipErrorInvalidValue);
+    const dim3 grid(static_cast<unsigned>((N + 16 * rgn - 1) / (16 * rgn)), static_cast<unsigned>(x_rows));
+    const dim3 block(8 * ks * 64);
+#define LAUNCH_DOWN(QT, RGN) hipLaunchKernelGGL((selected_down_sum_kernel<QT, 8, RGN>), grid, block, lds, stream, s)
+    if (qt == GGML_Q4_K) {
+      if (rgn == 2) LAUNCH_DOWN(GGML_Q4_K, 2); else LAUNCH_DOWN(GGML_Q4_K, 1);
+    } else {
+      if (rgn == 2) LAUNCH_DOWN(GGML_Q6_K, 2); else LAUNCH_DOWN(GGML_Q6_K, 1);
+    }
+#undef LAUNCH_DOWN
+    return static_cast<int>(hipGetLastError());
+  }
+
+  // all of a row's blocks in flight at once when they fit 8 K slices, else chunks
+  int ks, cb;
+  if (nb <= 8) { ks = nb; cb = 1; }
+  else if (nb <= 16) { ks = 8; cb = 2; }
+  else { ks = 4; cb = 5; }
+  // many lanes: half the K slices, twice the rows per workgroup (the staging of the
+  // activations is per workgroup, so a grid far above the CU count only repeats it)
+  if (nb == 8 && lanes * ((N + 31) / 32) > 768) { ks = 4; cb = 2; }
   const SelVariant* v = nullptr;
   for (const SelVariant& c : kSel)
     if (c.qt == qt && c.cb == cb && c.mode == mode) v = &c;
   if (!v) return static_cast<int>(hipErrorInvalidValue);
+  const int r = mode == SEL_DUAL_SILU ? 2 : 1;
   int nrg = v->max_threads / 64 / ks;
-  while (nrg > 1 && (N + nrg * 16 - 1) / (nrg * 16) * groups < 512) nrg >>= 1;
-  const size_t lds = gemv_lds_bytes(qt, 1, 1, cb, ks, nrg);
+  if (nrg < 1) return static_cast<int>(hipErrorInvalidValue);
+  const int rows_out_per_group = mode == SEL_DUAL_SILU ? 16 : 16 * r;
+  while (nrg > 1 && (N + nrg * rows_out_per_group - 1) / (nrg * rows_out_per_group) * lanes < 512) nrg >>= 1;
+  s.g.ks = ks; s.g.nrg = nrg;
+  size_t lds = gemv_lds_bytes(qt, 1, r, cb, ks, nrg);
+  if (mode == SEL_DUAL_SILU) {
+    lds = (lds + 15) & ~static_cast<size_t>(15);
+    s.pair_offset = static_cast<int>(lds);
+    lds += 2 * nrg * 16 * 4;
+  }
   if (lds > 64 * 1024) return static_cast<int>(hipErrorInvalidValue);
-  SelArgs s;
-  s.g.x = x; s.g.w = w_a; s.g.out = out; s.g.x_kind = x_kind; s.g.out_kind = out_kind; s.g.rows = 1;
-  s.g.K = static_cast<int>(K); s.g.N = static_cast<int>(N); s.g.ks = ks; s.g.nrg = nrg;
-  s.w_b = w_b; s.selected = selected; s.routing = routing;
-  s.x_rows = static_cast<int>(x_rows); s.lanes = static_cast<int>(lanes);
-  s.num_experts = static_cast<int>(num_experts); s.top_k = static_cast<int>(top_k); s.round_mid = round_mid;
-  const dim3 grid(static_cast<unsigned>((N + nrg * 16 - 1) / (nrg * 16)), static_cast<unsigned>(groups));
+  const int rows_out = nrg * rows_out_per_group;
+  const dim3 grid(static_cast<unsigned>((N + rows_out - 1) / rows_out), static_cast<unsigned>(lanes));
   hipLaunchKernelGGL(v->fn, grid, dim3(ks * nrg * 64), lds, stream, s);
   return static_cast<int>(hipGetLastError());
 }

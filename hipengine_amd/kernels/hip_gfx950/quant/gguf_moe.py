@@ -80,6 +80,8 @@ def gguf_selected_gemv(quant: str, mode: int, x_ptr: int, selected_ptr: int, qwe
     if mode == SEL_DOWN_SUM:
         if lanes != x_rows * top_k:
             raise ValueError("lanes must equal x_rows * top_k for the routed down sum")
+        if top_k > 8:
+            raise ValueError("the routed down sum handles at most 8 experts per token")
         _validate_selected(x_rows, lanes, num_experts, in_features, out_features, 128)
         validate_pointers(routing_weights_ptr=routing_weights_ptr)
     else:

@@ -303,7 +303,7 @@ int hipengine_gguf_q4_k_selected_dual_silu_gemv_bf16_bf16_out(const uint16_t* x,
  *           rounds gate and up to the output type first
  *   mode 2: x is [lanes, K] (one row per lane, lanes = x_rows * top_k); out[x_rows, N]
  *           = sum over the token's slots, in slot order, of routing_weights[lane] *
- *           (W_a[selected[lane]] . x[lane]); invalid experts are skipped
+ *           (W_a[selected[lane]] . x[lane]); invalid experts are skipped; top_k <= 8
  * Kinds: 0 float32, 1 bf16, 2 fp16.  New here. */
 int hipengine_gfx950_gguf_selected_gemv(int32_t ggml_type, int32_t mode, const void* x, int32_t x_kind,
                                         const int64_t* selected, const float* routing_weights,
