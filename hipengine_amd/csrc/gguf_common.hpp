@@ -101,11 +101,15 @@ __device__ __forceinline__ float quad_sum(float v) {
 }
 
 // All eight lanes of an aligned group of 8 receive the group maximum.
+// Maximum over an aligned group of 8 lanes of a NON-NEGATIVE float: the bit patterns of
+// non-negative floats order like unsigned integers, and the integer maximum takes its DPP
+// operand directly (one instruction per stage, no NaN canonicalization).
 __device__ __forceinline__ float oct_max(float v) {
-  v = fmaxf(v, dpp_f<DPP_QUAD_XOR1>(v));
-  v = fmaxf(v, dpp_f<DPP_QUAD_XOR2>(v));
-  v = fmaxf(v, dpp_f<DPP_ROW_HALF_MIRROR>(v));
-  return v;
+  uint32_t u = float_to_bits(v);
+  u = max(u, static_cast<uint32_t>(dpp_i<DPP_QUAD_XOR1>(static_cast<int>(u))));
+  u = max(u, static_cast<uint32_t>(dpp_i<DPP_QUAD_XOR2>(static_cast<int>(u))));
+  u = max(u, static_cast<uint32_t>(dpp_i<DPP_ROW_HALF_MIRROR>(static_cast<int>(u))));
+  return bits_to_float(u);
 }
 
 __device__ __forceinline__ int oct_sum_i(int v) {

@@ -6,6 +6,7 @@
 #include "gguf_gemv_run.hpp"
 #include "gguf_gemv_stream.hpp"
 #include "gguf_gemv_mfma.hpp"
+#include "gguf_gemv_slab.hpp"
 
 #include "../../include/hipengine_gfx950.h"
 
@@ -150,6 +151,71 @@ int launch_gemv_mfma(const void* x, int x_kind, const uint8_t* w, void* out, int
   if (lds > 64 * 1024) return static_cast<int>(hipErrorInvalidValue);
   GemvMfmaArgs a{x, w, out, x_kind, out_kind, rows, static_cast<int>(K), static_cast<int>(N), p.waves};
   hipLaunchKernelGGL(v->fn, dim3(static_cast<unsigned>((N + 31) / 32)), dim3(p.waves * 64), lds, stream, a);
+  return static_cast<int>(hipGetLastError());
+}
+
+// ---- slab form (Q4_K on the int8 MFMA, one workgroup per CU, waves split K) ----
+
+// BPW = 1: up to 16 waves (K <= 4096); BPW = 2: up to 12 waves (K <= 6144), whose 64
+// operand registers want the 170-register budget of a 768-thread bound.
+template <int B, int BPW, int XK>
+__global__ void __launch_bounds__(BPW == 1 ? 1024 : 768) gemv_slab_q4k_kernel(GemvSlabArgs a) {
+  extern __shared__ __align__(16) uint8_t smem[];
+  gemv_slab_q4k_workgroup<B, BPW, XK>(a, smem);
+}
+
+using SlabKernelFn = void (*)(GemvSlabArgs);
+struct SlabVariant {
+  int b, bpw;
+  SlabKernelFn by_kind[4];
+  bool lds_raised[4];
+};
+#define SLAB_VARIANT(B, BPW)                                                                            \
+  SlabVariant { B, BPW, {gemv_slab_q4k_kernel<B, BPW, KIND_F32>, gemv_slab_q4k_kernel<B, BPW, KIND_BF16>, \
+                         gemv_slab_q4k_kernel<B, BPW, KIND_F16>, gemv_slab_q4k_kernel<B, BPW, KIND_Q8_1>}, \
+                {false, false, false, false} }
+SlabVariant kSlab[] = {SLAB_VARIANT(1, 1), SLAB_VARIANT(1, 2), SLAB_VARIANT(2, 1), SLAB_VARIANT(2, 2),
+                       SLAB_VARIANT(4, 1), SLAB_VARIANT(4, 2), SLAB_VARIANT(8, 1), SLAB_VARIANT(8, 2)};
+
+struct SlabPlan {
+  int b, bpw, waves, rows_wg;
+  bool ok;
+};
+
+SlabPlan default_slab_plan(int qt, int rows, int64_t K, int64_t N) {
+  SlabPlan p{};
+  const int nb = static_cast<int>(K / QK_K);
+  p.b = rows <= 1 ? 1 : rows <= 2 ? 2 : rows <= 4 ? 4 : 8;
+  p.bpw = nb <= 16 ? 1 : 2;
+  p.waves = (nb + p.bpw - 1) / p.bpw;
+  const int64_t per_cu = (N + 255) / 256;
+  p.rows_wg = static_cast<int>(per_cu < 1 ? 1 : per_cu > SLAB_MAX_ROWS ? SLAB_MAX_ROWS : per_cu);
+  p.ok = qt == GGML_Q4_K && rows >= 1 && rows <= 8 && nb >= 4 && p.waves <= (p.bpw == 1 ? 16 : 12) &&
+         gemv_slab_lds_bytes(p.b, p.bpw, p.waves) <= 160 * 1024;
+  return p;
+}
+
+int launch_gemv_slab(const void* x, int x_kind, const uint8_t* w, void* out, int out_kind, int rows, int64_t K,
+                     int64_t N, const SlabPlan& p, hipStream_t stream) {
+  const int nb = static_cast<int>(K / QK_K);
+  SlabVariant* v = nullptr;
+  for (SlabVariant& c : kSlab)
+    if (c.b == p.b && c.bpw == p.bpw) v = &c;
+  if (!v || rows > p.b || x_kind < KIND_F32 || x_kind > KIND_Q8_1 || p.rows_wg < 1 || p.rows_wg > SLAB_MAX_ROWS ||
+      p.waves != (nb + p.bpw - 1) / p.bpw || p.waves > (p.bpw == 1 ? 16 : 12) || K > (1 << 20) || N > (1 << 30)) {
+    return static_cast<int>(hipErrorInvalidValue);
+  }
+  const size_t lds = gemv_slab_lds_bytes(p.b, p.bpw, p.waves);
+  if (lds > 160 * 1024) return static_cast<int>(hipErrorInvalidValue);
+  if (lds > 64 * 1024 && !v->lds_raised[x_kind]) {
+    const hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(v->by_kind[x_kind]),
+                                             hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
+    if (e != hipSuccess) return static_cast<int>(e);
+    v->lds_raised[x_kind] = true;
+  }
+  GemvSlabArgs a{x, w, out, x_kind, out_kind, rows, static_cast<int>(K), static_cast<int>(N), p.rows_wg, p.waves};
+  const unsigned grid = static_cast<unsigned>((N + p.rows_wg - 1) / p.rows_wg);
+  hipLaunchKernelGGL(v->by_kind[x_kind], dim3(grid), dim3(p.waves * 64), lds, stream, a);
   return static_cast<int>(hipGetLastError());
 }
 
@@ -349,6 +415,16 @@ int launch_gemv(int qt, const void* x, int x_kind, const uint8_t* w, void* out, 
   for (int64_t r0 = 0; r0 < rows; r0 += 8) {
     const int chunk = static_cast<int>(rows - r0 < 8 ? rows - r0 : 8);
     if (!forced) {
+      // Q4_K, K <= 6144: the int8 MFMA slab form wins for batches of 3 and more, and at any
+      // batch when a slab is a single 32-row step (N <= 8192); measured on MI355X
+      const SlabPlan sl = default_slab_plan(qt, chunk, K, N);
+      if (sl.ok && (chunk >= 3 || sl.rows_wg <= 32)) {
+        const int rc = launch_gemv_slab(static_cast<const uint8_t*>(x) + r0 * x_row_bytes, x_kind, w,
+                                        static_cast<uint8_t*>(out) + r0 * N * out_elem, out_kind, chunk, K, N, sl,
+                                        stream);
+        if (rc != static_cast<int>(hipSuccess)) return rc;
+        continue;
+      }
       const StreamPlan sp = default_stream_plan(qt, chunk, K, N);
       if (sp.ok) {
         const int rc = launch_gemv_stream(qt, static_cast<const uint8_t*>(x) + r0 * x_row_bytes, x_kind, w,
@@ -514,5 +590,22 @@ extern "C" int hipengine_gfx950_gguf_q4_k_q8_1_fused_gemv_tile_tuned(const void*
   p.bpw = blocks_per_wave;
   p.waves = static_cast<int>((in_features / QK_K + p.bpw - 1) / p.bpw);
   return launch_gemv_mfma(x, x_kind, qweight, out, out_kind, static_cast<int>(rows), in_features, out_features, p,
+                          stream);
+}
+
+extern "C" int hipengine_gfx950_gguf_q4_k_q8_1_fused_gemv_slab_tuned(const void* x, int32_t x_kind,
+                                                                    const uint8_t* qweight, void* out,
+                                                                    int32_t out_kind, int64_t rows,
+                                                                    int64_t in_features, int64_t out_features,
+                                                                    int32_t rows_per_workgroup, hipStream_t stream) {
+  if (!x || !qweight || !out || x_kind < KIND_F32 || x_kind > KIND_Q8_1 || out_kind < KIND_F32 ||
+      out_kind > KIND_F16 || rows <= 0 || rows > 8 || in_features <= 0 || (in_features % QK_K) != 0 ||
+      out_features <= 0) {
+    return static_cast<int>(hipErrorInvalidValue);
+  }
+  SlabPlan p = default_slab_plan(GGML_Q4_K, static_cast<int>(rows), in_features, out_features);
+  if (!p.ok) return static_cast<int>(hipErrorInvalidValue);
+  if (rows_per_workgroup > 0) p.rows_wg = rows_per_workgroup;
+  return launch_gemv_slab(x, x_kind, qweight, out, out_kind, static_cast<int>(rows), in_features, out_features, p,
                           stream);
 }

@@ -75,6 +75,57 @@ __device__ __forceinline__ float div_by_127(float a) {
   return __builtin_fmaf(__builtin_fmaf(-q, 127.0f, a), c, q);
 }
 
+// One lane's share of a 32-value activation group (8 lanes x 4 values): quantize the
+// fetched values to q8_1 (or take them from a q8_1 block) -> 4 packed int8 and the
+// group's scale, rounded to half as the q8_1 block stores it.
+__device__ __forceinline__ void q8_quantize4(int x_kind, const uint32_t (&raw)[4], bool present, uint32_t& packed,
+                                             float& xd) {
+  packed = 0;
+  xd = 0.0f;
+  if (!present) return;
+  if (x_kind == KIND_Q8_1) {
+    packed = raw[0];
+    xd = f16_bits_to_float(raw[1] & 0xFFFFu);
+    return;
+  }
+  float v0, v1, v2, v3;
+  if (x_kind == KIND_F32) {
+    v0 = bits_to_float(raw[0]); v1 = bits_to_float(raw[1]); v2 = bits_to_float(raw[2]); v3 = bits_to_float(raw[3]);
+  } else if (x_kind == KIND_BF16) {
+    v0 = bf16_bits_to_float(raw[0] & 0xFFFFu); v1 = bf16_bits_to_float(raw[0] >> 16);
+    v2 = bf16_bits_to_float(raw[1] & 0xFFFFu); v3 = bf16_bits_to_float(raw[1] >> 16);
+  } else {
+    v0 = f16_bits_to_float(raw[0] & 0xFFFFu); v1 = f16_bits_to_float(raw[0] >> 16);
+    v2 = f16_bits_to_float(raw[1] & 0xFFFFu); v3 = f16_bits_to_float(raw[1] >> 16);
+  }
+  const float amax = oct_max(fmaxf(fmaxf(fabsf(v0), fabsf(v1)), fmaxf(fabsf(v2), fabsf(v3))));
+  const float d = div_by_127(amax);
+  if (amax != 0.0f) {
+    // Fast path: t = v * rcp(d) is within 3e-5 of the quotient (|v/d| <= 127, reciprocal good
+    // to 1 ulp).  t + 1.5*2^23 rounds t to the nearest integer r and leaves r's two's
+    // complement in the low mantissa bits; unless t is within 1e-4 of a tie, r equals
+    // roundf(v/d).  Near ties, and scales in the denormal range where the reciprocal
+    // overflows, redo the lane's four values with the IEEE division.
+    constexpr float MAGIC = 12582912.0f;
+    const float inv = __builtin_amdgcn_rcpf(d);
+    const float t0 = v0 * inv, t1 = v1 * inv, t2 = v2 * inv, t3 = v3 * inv;
+    const float m0 = t0 + MAGIC, m1 = t1 + MAGIC, m2 = t2 + MAGIC, m3 = t3 + MAGIC;
+    const float e0 = fabsf(t0 - (m0 - MAGIC)), e1 = fabsf(t1 - (m1 - MAGIC));
+    const float e2 = fabsf(t2 - (m2 - MAGIC)), e3 = fabsf(t3 - (m3 - MAGIC));
+    const bool near_tie = __builtin_fmaxf(__builtin_fmaxf(e0, e1), __builtin_fmaxf(e2, e3)) > 0.4999f;
+    packed = __builtin_amdgcn_perm(float_to_bits(m1), float_to_bits(m0), 0x0c0c0400u) |
+             __builtin_amdgcn_perm(float_to_bits(m3), float_to_bits(m2), 0x04000c0cu);
+    if (__builtin_expect(near_tie || d < 1.0e-30f, 0)) {
+      const int q0 = max(-128, min(127, static_cast<int>(roundf(v0 / d))));
+      const int q1 = max(-128, min(127, static_cast<int>(roundf(v1 / d))));
+      const int q2 = max(-128, min(127, static_cast<int>(roundf(v2 / d))));
+      const int q3 = max(-128, min(127, static_cast<int>(roundf(v3 / d))));
+      packed = (q0 & 0xFF) | ((q1 & 0xFF) << 8) | ((q2 & 0xFF) << 16) | (static_cast<uint32_t>(q3 & 0xFF) << 24);
+    }
+  }
+  xd = static_cast<float>(static_cast<half_t>(d));
+}
+
 // Whole-K activation staging for the run kernel.
 //   q8   : [B][nb] blocks, Q8S bytes apart
 //   rec  : [B][nb][4] 16-byte records, one per lane q of a block:
@@ -199,37 +250,9 @@ template <int QT>
 __device__ __forceinline__ void gemv_run_stage_one(int x_kind, const uint32_t (&raw)[4], bool present, int j, int e,
                                                    uint8_t* q8_row, float* rec_row, int* s16_row) {
   constexpr int Q8S = run_q8_stride<QT>();
-  uint32_t packed = 0;
-  float xd = 0.0f;
-  if (present) {
-    if (x_kind == KIND_Q8_1) {
-      packed = raw[0];
-      xd = f16_bits_to_float(raw[1] & 0xFFFFu);
-    } else {
-      float v0, v1, v2, v3;
-      if (x_kind == KIND_F32) {
-        v0 = bits_to_float(raw[0]); v1 = bits_to_float(raw[1]); v2 = bits_to_float(raw[2]); v3 = bits_to_float(raw[3]);
-      } else if (x_kind == KIND_BF16) {
-        v0 = bf16_bits_to_float(raw[0] & 0xFFFFu); v1 = bf16_bits_to_float(raw[0] >> 16);
-        v2 = bf16_bits_to_float(raw[1] & 0xFFFFu); v3 = bf16_bits_to_float(raw[1] >> 16);
-      } else {
-        v0 = f16_bits_to_float(raw[0] & 0xFFFFu); v1 = f16_bits_to_float(raw[0] >> 16);
-        v2 = f16_bits_to_float(raw[1] & 0xFFFFu); v3 = f16_bits_to_float(raw[1] >> 16);
-      }
-      const float amax = oct_max(fmaxf(fmaxf(fabsf(v0), fabsf(v1)), fmaxf(fabsf(v2), fabsf(v3))));
-      const float d = div_by_127(amax);
-      if (amax != 0.0f) {
-        // hardware reciprocal (1 ulp): v*inv stays within 2e-5 of the quotient; scales in the
-        // denormal range, where the reciprocal overflows, take the exact division
-        const float inv = __builtin_amdgcn_rcpf(d);
-        const bool exact = d < 1.0e-30f;
-        const int q0 = q8_round_div(v0, d, inv, exact), q1 = q8_round_div(v1, d, inv, exact);
-        const int q2 = q8_round_div(v2, d, inv, exact), q3 = q8_round_div(v3, d, inv, exact);
-        packed = (q0 & 0xFF) | ((q1 & 0xFF) << 8) | ((q2 & 0xFF) << 16) | (static_cast<uint32_t>(q3 & 0xFF) << 24);
-      }
-      xd = static_cast<float>(static_cast<half_t>(d));
-    }
-  }
+  uint32_t packed;
+  float xd;
+  q8_quantize4(x_kind, raw, present, packed, xd);
   const int kb = j >> 3, sb = j & 7;
   *reinterpret_cast<uint32_t*>(q8_row + kb * Q8S + sb * 32 + e * 4) = packed;
   const int part = dot4(0x01010101u, packed, 0);

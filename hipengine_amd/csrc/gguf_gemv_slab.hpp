@@ -1,0 +1,299 @@
+// "Slab" form of the q8_1 decode GEMV for Q4_K weights, batch 1..8, on the int8
+// MFMA: one workgroup per CU owns a slab of consecutive output rows, its waves
+// split K, and nothing in the kernel waits for another wave until the final sum.
+//
+// Why: with v_dot4 a batch of 8 costs eight times the VALU work of batch 1 and
+// the kernel stops being bound by HBM.  v_mfma_i32_32x32x32_i8 takes 32 weight
+// rows x 32 values against up to 32 activation rows in one instruction, so the
+// batch rides along and the VALU only splits nibbles and applies scales.
+//
+// Work decomposition
+//   * workgroup b owns rows [b*R, b*R + R), R = ceil(N / 256) <= 96, in steps of 32;
+//   * wave w owns the K blocks [w*BPW, w*BPW + BPW) of every row, BPW in {1, 2}
+//     (K = 5120: 10 waves x 2 blocks).  It quantizes ONLY its own K slice of the
+//     activations (B x BPW x 256 values) into wave-private LDS: no workgroup
+//     barrier before the final sum;
+//   * per step the wave reads its 32 x (BPW*144) byte piece of the weight with
+//     loads that are contiguous along each row (lane c takes 16-byte chunk c of
+//     the piece: BPW*9 chunks per row), writes the registers to wave-private LDS
+//     in that natural order and reads them back in MFMA operand order: lane
+//     (n = l % 32, g = l / 32) takes bytes [16 + 32j + 16g, +16) of row n, the
+//     values 16g..16g+15 of sub-blocks 2j (low nibbles) and 2j+1 (high nibbles).
+//     Loading in operand order directly would make every lane of a load touch a
+//     different row (2880 bytes apart), which the texture addresser serializes;
+//     The loads are unconditional: rows past the slab and chunks past the piece are
+//     clamped to valid addresses and their bytes land in rows whose results are
+//     dropped (or in a dump slot), which keeps the issue code free of branches;
+//   * the loads of step t+1 are issued into step t's registers as soon as those are in
+//     LDS and fly while step t is computed;
+//   * A = int8 activations of batch row (l % 32) (zero for rows >= batch), B = the
+//     nibbles, zero accumulator input.  Lane (n, g) register v < 4 of the result
+//     is batch row 4g + v of output row n; per sub-block and batch row
+//     t = (d*sc) * float(dot), acc = fma(xd, t, acc), acc = fma(-dmin*mn, xd*qsum, acc)
+//     (the arithmetic of gguf_q4_k_gemv.hip:893-904);
+//   * K slices are summed through LDS in slice order.
+//
+// LDS row pitch: 144 bytes (BPW = 1) or 304 (BPW = 2), i.e. 4 x an odd number of
+// dwords, which puts the 16-byte operand reads of 16 consecutive rows on
+// distinct banks.
+#pragma once
+
+#include "gguf_gemv_run.hpp"
+
+namespace hipengine_gfx950 {
+
+typedef int sl_v4i __attribute__((ext_vector_type(4)));
+typedef int sl_v16i __attribute__((ext_vector_type(16)));
+typedef uint32_t sl_u32x4 __attribute__((ext_vector_type(4)));
+typedef float sl_f4 __attribute__((ext_vector_type(4)));
+
+struct GemvSlabArgs {
+  const void* x;
+  const uint8_t* w;
+  void* out;
+  int x_kind;
+  int out_kind;
+  int rows;      // batch rows, 1..B
+  int K;
+  int N;
+  int rows_wg;   // output rows per workgroup, 1..96
+  int waves;     // waves per workgroup = ceil(nb / BPW)
+};
+
+constexpr int SLAB_MAX_ROWS = 96;
+
+template <int BPW>
+constexpr int slab_row_pitch() { return BPW == 1 ? 144 : 304; }
+
+// Per wave: the weight piece of a step (reused for the partial sums after the last
+// step), a 16-byte dump slot, the scale records and the int8 activations.
+constexpr int slab_wave_bytes(int B, int BPW) {
+  return 32 * (BPW == 1 ? 144 : 304) + 16 + BPW * 8 * 16 * 4 + B * (BPW * 256 + 16);
+}
+
+inline size_t gemv_slab_lds_bytes(int b, int bpw, int waves) {
+  return static_cast<size_t>(waves) * slab_wave_bytes(b, bpw);
+}
+
+template <int B, int BPW, int XK>
+__device__ __forceinline__ void gemv_slab_q4k_workgroup(const GemvSlabArgs& a, uint8_t* smem) {
+  constexpr int VB = B < 4 ? B : 4;                  // result registers in use per lane
+  constexpr int PITCH = slab_row_pitch<BPW>();
+  constexpr int XQ_PITCH = BPW * 256 + 16;           // int8 activations, one batch row
+  constexpr int WQ_BYTES = 32 * PITCH;
+  constexpr int DUMP = WQ_BYTES;
+  constexpr int REC = WQ_BYTES + 16;
+  constexpr int XQ = REC + BPW * 8 * 16 * 4;
+  constexpr int WAVE_BYTES = slab_wave_bytes(B, BPW);
+  constexpr int NL = (32 * BPW * 9 + 63) / 64;       // 16-byte loads per lane and step
+  constexpr int MAX_STEPS = SLAB_MAX_ROWS / 32;
+  static_assert(B * SLAB_MAX_ROWS * 4 <= WQ_BYTES, "partial sums must fit the weight piece");
+  const int x_kind = XK >= 0 ? XK : a.x_kind;
+
+  const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int n = lane & 31, g = lane >> 5;
+  const int nb = a.K / QK_K;
+  const int kb0 = wave * BPW;
+  const int blocks_w = min(BPW, nb - kb0);           // >= 1: waves = ceil(nb / BPW)
+  const int r0 = static_cast<int>(blockIdx.x) * a.rows_wg;
+  const int rows_wg = min(a.rows_wg, a.N - r0);
+  const int steps = (rows_wg + 31) >> 5;
+  const int row_bytes = nb * Q4_K_BYTES;
+  const uint8_t* wbase = a.w + static_cast<int64_t>(r0) * row_bytes + kb0 * Q4_K_BYTES;
+
+  uint8_t* wq = smem + wave * WAVE_BYTES;
+  float* rec = reinterpret_cast<float*>(wq + REC);   // [BPW*8 sub-blocks][xd[8], xd*qsum[8]]
+  uint8_t* xq = wq + XQ;
+
+  // ---- activation loads of this wave's K slice (8 lanes per 32-value group, 4 values per lane)
+  const int team = lane >> 3, e = lane & 7;
+  uint32_t raw[B][BPW][4];
+#pragma unroll
+  for (int b = 0; b < B; ++b) {
+#pragma unroll
+    for (int s = 0; s < BPW; ++s) {
+      // clamped, unconditional: rows >= a.rows and blocks past the slice are quantized but not used
+      const int bb = min(b, a.rows - 1);
+      const int j = (kb0 + min(s, blocks_w - 1)) * 8 + team;
+      uint4 v = make_uint4(0u, 0u, 0u, 0u);
+      if (x_kind == KIND_F32) {
+        v = *reinterpret_cast<const uint4*>(static_cast<const float*>(a.x) + static_cast<int64_t>(bb) * a.K + j * 32 + e * 4);
+      } else if (x_kind == KIND_Q8_1) {
+        const uint8_t* blk = static_cast<const uint8_t*>(a.x) + (static_cast<int64_t>(bb) * (a.K / 32) + j) * Q8_1_BYTES;
+        v.x = *reinterpret_cast<const uint32_t*>(blk + 4 + 4 * e);
+        v.y = *reinterpret_cast<const uint32_t*>(blk);
+      } else {
+        const uint2 h = *reinterpret_cast<const uint2*>(static_cast<const uint16_t*>(a.x) + static_cast<int64_t>(bb) * a.K + j * 32 + e * 4);
+        v.x = h.x; v.y = h.y;
+      }
+      raw[b][s][0] = v.x; raw[b][s][1] = v.y; raw[b][s][2] = v.z; raw[b][s][3] = v.w;
+    }
+  }
+
+  // ---- chunk c = i*64 + lane of a step's piece: row c / cpr, 16-byte column c % cpr
+  const int cpr = blocks_w * 9;
+  const int row_inc = (BPW == 2 && cpr == 18) ? 3 : 7, col_inc = (BPW == 2 && cpr == 18) ? 10 : 1;   // 64 = row_inc*cpr + col_inc
+  // The positions are walked again from (row0, col0) wherever they are needed (four
+  // operations per chunk) instead of being kept in NL registers.
+  const int row0 = (BPW == 2 && cpr == 18) ? lane / 18 : lane / 9;
+  const int col0 = lane - row0 * cpr;
+  auto walk = [&](auto&& visit) {
+    int row = row0, col = col0;
+#pragma unroll
+    for (int i = 0; i < NL; ++i) {
+      visit(i, row, col * 16);
+      row += row_inc; col += col_inc;
+      if (col >= cpr) { col -= cpr; row += 1; }
+    }
+  };
+
+  sl_u32x4 buf[NL];
+  // Buffer loads: a descriptor over this wave's K slice of the slab (the hardware returns
+  // zeros past its end), a 32-bit lane offset and a scalar step offset: no 64-bit
+  // address arithmetic per load.
+  const __amdgpu_buffer_rsrc_t wrsrc = __builtin_amdgcn_make_buffer_rsrc(
+      const_cast<uint8_t*>(wbase), 0, (rows_wg - 1) * row_bytes + blocks_w * Q4_K_BYTES, 0x00020000);
+  auto issue = [&](int t, sl_u32x4 (&dst)[NL]) {
+    const int last = rows_wg - 32 * t - 1;           // >= 0 for t < steps
+    walk([&](int i, int row, int col16) {
+      dst[i] = __builtin_amdgcn_raw_buffer_load_b128(wrsrc, min(row, last) * row_bytes + col16, t * 32 * row_bytes, 0);
+    });
+  };
+  // batch 8 holds 64 registers of fetched activations: its first weight loads wait until half of
+  // them are quantized (they are not needed before the staging is done)
+  if constexpr (B < 8) issue(0, buf);
+
+  // ---- quantize the slice into LDS
+#pragma unroll
+  for (int b = 0; b < B; ++b) {
+    if constexpr (B >= 8) {
+      if (b == B / 2) issue(0, buf);
+    }
+#pragma unroll
+    for (int s = 0; s < BPW; ++s) {
+      uint32_t packed;
+      float xd;
+      q8_quantize4(x_kind, raw[b][s], true, packed, xd);
+      const bool used = b < a.rows && s < blocks_w;
+      packed = used ? packed : 0u;
+      xd = used ? xd : 0.0f;
+      *reinterpret_cast<uint32_t*>(xq + b * XQ_PITCH + s * 256 + team * 32 + e * 4) = packed;
+      const int total = oct_sum_i(dot4(0x01010101u, packed, 0));
+      if (e == 0) {
+        rec[(s * 8 + team) * 16 + b] = xd;
+        rec[(s * 8 + team) * 16 + 8 + b] = xd * static_cast<float>(total);
+      }
+    }
+  }
+  __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+  __builtin_amdgcn_wave_barrier();
+  __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+
+  // partial sums of the steps done so far, filed with selects (the step loop is a real loop)
+  float done[MAX_STEPS][VB];
+#pragma unroll
+  for (int t = 0; t < MAX_STEPS; ++t)
+#pragma unroll
+    for (int v = 0; v < VB; ++v) done[t][v] = 0.0f;
+
+  const uint8_t* wlane = wq + n * PITCH;
+  const uint8_t* alane = xq + min(n, B - 1) * XQ_PITCH + 16 * g;   // A operand row: batch row n (zeros for n >= B)
+  const sl_f4* rec4 = reinterpret_cast<const sl_f4*>(rec);
+
+  auto to_lds = [&](const sl_u32x4 (&src)[NL]) {
+    walk([&](int i, int row, int col16) {
+      *reinterpret_cast<sl_u32x4*>(wq + (row < 32 ? row * PITCH + col16 : DUMP)) = src[i];
+    });
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+  };
+
+  auto compute = [&](int t) {
+    float acc[VB];
+#pragma unroll
+    for (int v = 0; v < VB; ++v) acc[v] = 0.0f;
+#pragma unroll
+    for (int s = 0; s < BPW; ++s) {
+      if (s < blocks_w) {
+        const sl_u32x4 hd = *reinterpret_cast<const sl_u32x4*>(wlane + s * Q4_K_BYTES);
+        const Q4KScales u = q4k_unpack_scales(hd.y, hd.z, hd.w);
+        const float d = f16_bits_to_float(hd.x & 0xFFFFu);
+        const float dmin = f16_bits_to_float(hd.x >> 16);
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+          const sl_u32x4 qs = *reinterpret_cast<const sl_u32x4*>(wlane + s * Q4_K_BYTES + 16 + 32 * j + 16 * g);
+#pragma unroll
+          for (int half = 0; half < 2; ++half) {
+            const int sb = 2 * j + half;
+            const sl_v4i wop = half == 0
+                ? sl_v4i{static_cast<int>(q4k_low(qs.x)), static_cast<int>(q4k_low(qs.y)),
+                         static_cast<int>(q4k_low(qs.z)), static_cast<int>(q4k_low(qs.w))}
+                : sl_v4i{static_cast<int>(q4k_high(qs.x)), static_cast<int>(q4k_high(qs.y)),
+                         static_cast<int>(q4k_high(qs.z)), static_cast<int>(q4k_high(qs.w))};
+            sl_v4i xop = sl_v4i{0, 0, 0, 0};
+            xop = *reinterpret_cast<const sl_v4i*>(alane + s * 256 + sb * 32);
+            sl_v16i c0;
+#pragma unroll
+            for (int v = 0; v < 16; ++v) c0[v] = 0;
+            const sl_v16i dots = __builtin_amdgcn_mfma_i32_32x32x32_i8(xop, wop, c0, 0, 0, 0);
+            const uint32_t sc = ((sb < 4 ? u.sc_lo : u.sc_hi) >> (8 * (sb & 3))) & 0xFFu;
+            const uint32_t mn = ((sb < 4 ? u.mn_lo : u.mn_hi) >> (8 * (sb & 3))) & 0xFFu;
+            const float sw = d * static_cast<float>(sc);
+            const float mw = -(dmin * static_cast<float>(mn));
+            // scales of batch rows 4g..4g+VB-1: read only what the batch uses
+            float xd[VB], xs[VB];
+            if constexpr (VB == 4) {
+              const sl_f4 d4 = rec4[(s * 8 + sb) * 4 + g], s4 = rec4[(s * 8 + sb) * 4 + 2 + g];
+#pragma unroll
+              for (int v = 0; v < 4; ++v) { xd[v] = d4[v]; xs[v] = s4[v]; }
+            } else {
+#pragma unroll
+              for (int v = 0; v < VB; ++v) { xd[v] = rec[(s * 8 + sb) * 16 + v]; xs[v] = rec[(s * 8 + sb) * 16 + 8 + v]; }
+            }
+#pragma unroll
+            for (int v = 0; v < VB; ++v) {
+              const float tv = sw * static_cast<float>(dots[v]);   // |dot| < 2^24: one rounding
+              acc[v] = __builtin_fmaf(xd[v], tv, acc[v]);
+              acc[v] = __builtin_fmaf(mw, xs[v], acc[v]);
+            }
+          }
+        }
+      }
+    }
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+#pragma unroll
+    for (int u = 0; u < MAX_STEPS; ++u)
+#pragma unroll
+      for (int v = 0; v < VB; ++v) done[u][v] = (u == t) ? acc[v] : done[u][v];
+  };
+
+#pragma unroll 1
+  for (int t = 0; t < steps; ++t) {
+    to_lds(buf);
+    if (t + 1 < steps) issue(t + 1, buf);
+    compute(t);
+  }
+
+  // ---- K-slice reduction: each wave's partial sums [batch row][SLAB_MAX_ROWS] replace its weight piece
+  float* red = reinterpret_cast<float*>(wq);
+#pragma unroll
+  for (int t = 0; t < MAX_STEPS; ++t) {
+#pragma unroll
+    for (int v = 0; v < VB; ++v) {
+      const int m = 4 * g + v, rl = 32 * t + n;
+      if (m < B && rl < rows_wg) red[m * SLAB_MAX_ROWS + rl] = done[t][v];
+    }
+  }
+  __syncthreads();
+  for (int idx = tid; idx < a.rows * rows_wg; idx += blockDim.x) {
+    const int m = idx / rows_wg, rl = idx - m * rows_wg;
+    float v = 0.0f;
+    for (int s = 0; s < a.waves; ++s)
+      v += reinterpret_cast<const float*>(smem + s * WAVE_BYTES)[m * SLAB_MAX_ROWS + rl];
+    store_scalar(a.out, static_cast<int64_t>(m) * a.N + r0 + rl, v, a.out_kind);
+  }
+}
+
+}  // namespace hipengine_gfx950

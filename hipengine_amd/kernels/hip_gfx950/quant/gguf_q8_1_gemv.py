@@ -143,6 +143,20 @@ def gguf_q4_k_q8_1_fused_gemv_tile_tuned(x_ptr: int, x_kind: str, qweight_ptr: i
                     blocks_per_wave, stream), runtime)
 
 
+def gguf_q4_k_q8_1_fused_gemv_slab_tuned(x_ptr: int, x_kind: str, qweight_ptr: int, out_ptr: int, out_kind: str,
+                                         rows: int, in_features: int, out_features: int, *,
+                                         rows_per_workgroup: int = 0, stream: int = 0,
+                                         library: ctypes.CDLL | None = None,
+                                         runtime: HipRuntime | None = None) -> None:
+    """The slab (int8 MFMA, K split over the waves of one workgroup per CU) form of the fused Q4_K GEMV with an
+    explicit slab height; 0 takes the planner's (tuning sweeps only)."""
+    validate_linear(rows, in_features, out_features)
+    fn = entry("hipengine_gfx950_gguf_q4_k_q8_1_fused_gemv_slab_tuned",
+               [VOID, I32, VOID, VOID, I32, I64, I64, I64, I32, VOID], library)
+    check_launch(fn(x_ptr, _KINDS[x_kind], qweight_ptr, out_ptr, _KINDS[out_kind], rows, in_features, out_features,
+                    rows_per_workgroup, stream), runtime)
+
+
 def gguf_gemv_default_plan(quant_key: str, rows: int, in_features: int, out_features: int, *,
                            library: ctypes.CDLL | None = None) -> dict[str, int]:
     """The workgroup layout the library picks for a shape (host only)."""

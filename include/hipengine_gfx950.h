@@ -160,6 +160,15 @@ int hipengine_gfx950_gguf_q4_k_q8_1_fused_gemv_tile_tuned(const void* x, int32_t
                                                           int64_t in_features, int64_t out_features,
                                                           int32_t blocks_per_wave, hipengine_stream_t stream);
 
+/* The "slab" form for Q4_K: one workgroup per CU owns rows_per_workgroup (<= 96;
+ * 0 = ceil(out_features / 256)) consecutive output rows, its waves split K in
+ * slices of one or two 256-value blocks and run on the int8 MFMA.  rows <= 8,
+ * 1024 <= in_features <= 6144.  New here. */
+int hipengine_gfx950_gguf_q4_k_q8_1_fused_gemv_slab_tuned(const void* x, int32_t x_kind, const uint8_t* qweight,
+                                                          void* out, int32_t out_kind, int64_t rows,
+                                                          int64_t in_features, int64_t out_features,
+                                                          int32_t rows_per_workgroup, hipengine_stream_t stream);
+
 /* Host only: the layout the library picks for a shape, as
  * {batch_bucket, rows_per_lane, blocks_per_wave, k_slices, row_groups}.  New here. */
 int hipengine_gfx950_gguf_gemv_default_plan(int32_t ggml_type, int64_t rows, int64_t in_features,

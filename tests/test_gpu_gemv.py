@@ -218,6 +218,28 @@ def test_tile_form_q4_k(dev, rows, k, n, bpw):
     _check_f32(got, O.quantize_q8_1(x), w, O.GGML_Q4_K)
 
 
+@pytest.mark.parametrize("rows,k,n,rpw,kind", [(1, 5120, 300, 0, "f32"), (8, 5120, 1000, 68, "f32"),
+                                               (4, 2048, 257, 33, "bf16"), (2, 4096, 96, 96, "fp16"),
+                                               (5, 4352, 64, 7, "f32"), (8, 1024, 40, 0, "bf16"),
+                                               (3, 6144, 130, 65, "f32")])
+def test_slab_form_q4_k(dev, rows, k, n, rpw, kind):
+    """The slab form of the fused Q4_K GEMV: K split over the waves of a workgroup (one or two blocks per wave,
+    odd block counts included), slabs of up to three 32-row steps with ragged last steps and a ragged last slab."""
+    rng = np.random.default_rng(91 + rows + k)
+    x = rng.standard_normal((rows, k)).astype(np.float32)
+    x[0, :32] = 0.0
+    if kind != "f32":
+        x = O.bf16_bits_to_f32(O.f32_to_bf16_bits(x)) if kind == "bf16" else x.astype(np.float16).astype(np.float32)
+    w = O.random_weight(O.GGML_Q4_K, n, k, seed=k + n)
+    xin = x if kind == "f32" else (O.f32_to_bf16_bits(x) if kind == "bf16" else x.astype(np.float16))
+    dx, dw = dev.put(xin), dev.put(w)
+    dout = dev.empty(rows * n * 4)
+    G.gguf_q4_k_q8_1_fused_gemv_slab_tuned(dx.ptr, kind, dw.ptr, dout.ptr, "f32", rows, k, n, rows_per_workgroup=rpw)
+    got = dev.get(dout, np.float32, (rows, n))
+    dev.free(dx, dw, dout)
+    _check_f32(got, O.quantize_q8_1(x), w, O.GGML_Q4_K)
+
+
 @pytest.mark.parametrize("quant,d,waves,waves_total", [("gguf_q4_k", 3, 4, 64), ("gguf_q4_k", 5, 10, 120),
                                                       ("gguf_q6_k", 3, 12, 96), ("gguf_q8_0", 5, 8, 64)])
 def test_stream_form_explicit_layouts(dev, quant, d, waves, waves_total):
