@@ -126,6 +126,60 @@ __device__ __forceinline__ void q8_quantize4(int x_kind, const uint32_t (&raw)[4
   xd = static_cast<float>(static_cast<half_t>(d));
 }
 
+// The same for a group held by 4 lanes, 8 values per lane: half the per-group overhead
+// (scale, reciprocal, reductions) per value.  raw: 8 floats, or 8 halves/bf16 in raw[0..3],
+// or for q8_1 input the lane's 8 quants in raw[0..1] and the block's {d, s} halves in raw[2].
+__device__ __forceinline__ void q8_quantize8(int x_kind, const uint32_t (&raw)[8], bool present, uint32_t (&packed)[2],
+                                             float& xd) {
+  packed[0] = 0; packed[1] = 0;
+  xd = 0.0f;
+  if (!present) return;
+  if (x_kind == KIND_Q8_1) {
+    packed[0] = raw[0]; packed[1] = raw[1];
+    xd = f16_bits_to_float(raw[2] & 0xFFFFu);
+    return;
+  }
+  float v[8];
+#pragma unroll
+  for (int i = 0; i < 8; ++i) {
+    if (x_kind == KIND_F32) v[i] = bits_to_float(raw[i]);
+    else if (x_kind == KIND_BF16) v[i] = bf16_bits_to_float((raw[i >> 1] >> (16 * (i & 1))) & 0xFFFFu);
+    else v[i] = f16_bits_to_float((raw[i >> 1] >> (16 * (i & 1))) & 0xFFFFu);
+  }
+  float m = fmaxf(fmaxf(fmaxf(fabsf(v[0]), fabsf(v[1])), fmaxf(fabsf(v[2]), fabsf(v[3]))),
+                  fmaxf(fmaxf(fabsf(v[4]), fabsf(v[5])), fmaxf(fabsf(v[6]), fabsf(v[7]))));
+  uint32_t u = float_to_bits(m);                       // non-negative: integer order = float order
+  u = max(u, static_cast<uint32_t>(dpp_i<DPP_QUAD_XOR1>(static_cast<int>(u))));
+  u = max(u, static_cast<uint32_t>(dpp_i<DPP_QUAD_XOR2>(static_cast<int>(u))));
+  const float amax = bits_to_float(u);
+  const float d = div_by_127(amax);
+  if (amax != 0.0f) {
+    constexpr float MAGIC = 12582912.0f;               // see q8_quantize4
+    const float inv = __builtin_amdgcn_rcpf(d);
+    float mg[8], worst = 0.0f;
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+      const float t = v[i] * inv;
+      mg[i] = t + MAGIC;
+      worst = __builtin_fmaxf(worst, fabsf(t - (mg[i] - MAGIC)));
+    }
+    packed[0] = __builtin_amdgcn_perm(float_to_bits(mg[1]), float_to_bits(mg[0]), 0x0c0c0400u) |
+                __builtin_amdgcn_perm(float_to_bits(mg[3]), float_to_bits(mg[2]), 0x04000c0cu);
+    packed[1] = __builtin_amdgcn_perm(float_to_bits(mg[5]), float_to_bits(mg[4]), 0x0c0c0400u) |
+                __builtin_amdgcn_perm(float_to_bits(mg[7]), float_to_bits(mg[6]), 0x04000c0cu);
+    if (__builtin_expect(worst > 0.4999f || d < 1.0e-30f, 0)) {
+      uint32_t p[2] = {0u, 0u};
+#pragma unroll
+      for (int i = 0; i < 8; ++i) {
+        const int q = max(-128, min(127, static_cast<int>(roundf(v[i] / d))));
+        p[i >> 2] |= static_cast<uint32_t>(q & 0xFF) << (8 * (i & 3));
+      }
+      packed[0] = p[0]; packed[1] = p[1];
+    }
+  }
+  xd = static_cast<float>(static_cast<half_t>(d));
+}
+
 // Whole-K activation staging for the run kernel.
 //   q8   : [B][nb] blocks, Q8S bytes apart
 //   rec  : [B][nb][4] 16-byte records, one per lane q of a block:

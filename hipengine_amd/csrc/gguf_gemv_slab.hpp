@@ -87,6 +87,8 @@ __device__ __forceinline__ void gemv_slab_q4k_workgroup(const GemvSlabArgs& a, u
   constexpr int WAVE_BYTES = slab_wave_bytes(B, BPW);
   constexpr int NL = (32 * BPW * 9 + 63) / 64;       // 16-byte loads per lane and step
   constexpr int MAX_STEPS = SLAB_MAX_ROWS / 32;
+  constexpr int EARLY_TAIL_ROWS = 7;                 // a last step of at most this many rows is done first
+  constexpr int NLT = (EARLY_TAIL_ROWS * BPW * 9 + 63) / 64;
   static_assert(B * SLAB_MAX_ROWS * 4 <= WQ_BYTES, "partial sums must fit the weight piece");
   const int x_kind = XK >= 0 ? XK : a.x_kind;
 
@@ -105,28 +107,33 @@ __device__ __forceinline__ void gemv_slab_q4k_workgroup(const GemvSlabArgs& a, u
   float* rec = reinterpret_cast<float*>(wq + REC);   // [BPW*8 sub-blocks][xd[8], xd*qsum[8]]
   uint8_t* xq = wq + XQ;
 
-  // ---- activation loads of this wave's K slice (8 lanes per 32-value group, 4 values per lane)
-  const int team = lane >> 3, e = lane & 7;
-  uint32_t raw[B][BPW][4];
+  // ---- activation loads of this wave's K slice: 4 lanes per 32-value group, 8 values per lane,
+  // 16 groups per pass.  Group p*16 + quad is batch row gid / (BPW*8), sub-block gid % (BPW*8).
+  constexpr int PASSES = (B * BPW * 8 + 15) / 16;
+  const int quad = lane >> 2, e = lane & 3;
+  uint32_t raw[PASSES][8];
 #pragma unroll
-  for (int b = 0; b < B; ++b) {
+  for (int p = 0; p < PASSES; ++p) {
+    const int gid = p * 16 + quad;
+    // clamped, unconditional: rows >= a.rows and blocks past the slice are quantized but not used
+    const int bb = min(gid / (BPW * 8), a.rows - 1);
+    const int rem = gid % (BPW * 8);
+    const int j = (kb0 + min(rem >> 3, blocks_w - 1)) * 8 + (rem & 7);
 #pragma unroll
-    for (int s = 0; s < BPW; ++s) {
-      // clamped, unconditional: rows >= a.rows and blocks past the slice are quantized but not used
-      const int bb = min(b, a.rows - 1);
-      const int j = (kb0 + min(s, blocks_w - 1)) * 8 + team;
-      uint4 v = make_uint4(0u, 0u, 0u, 0u);
-      if (x_kind == KIND_F32) {
-        v = *reinterpret_cast<const uint4*>(static_cast<const float*>(a.x) + static_cast<int64_t>(bb) * a.K + j * 32 + e * 4);
-      } else if (x_kind == KIND_Q8_1) {
-        const uint8_t* blk = static_cast<const uint8_t*>(a.x) + (static_cast<int64_t>(bb) * (a.K / 32) + j) * Q8_1_BYTES;
-        v.x = *reinterpret_cast<const uint32_t*>(blk + 4 + 4 * e);
-        v.y = *reinterpret_cast<const uint32_t*>(blk);
-      } else {
-        const uint2 h = *reinterpret_cast<const uint2*>(static_cast<const uint16_t*>(a.x) + static_cast<int64_t>(bb) * a.K + j * 32 + e * 4);
-        v.x = h.x; v.y = h.y;
-      }
-      raw[b][s][0] = v.x; raw[b][s][1] = v.y; raw[b][s][2] = v.z; raw[b][s][3] = v.w;
+    for (int i = 0; i < 8; ++i) raw[p][i] = 0u;
+    if (x_kind == KIND_F32) {
+      const uint4* src = reinterpret_cast<const uint4*>(static_cast<const float*>(a.x) + static_cast<int64_t>(bb) * a.K + j * 32 + e * 8);
+      const uint4 lo = src[0], hi = src[1];
+      raw[p][0] = lo.x; raw[p][1] = lo.y; raw[p][2] = lo.z; raw[p][3] = lo.w;
+      raw[p][4] = hi.x; raw[p][5] = hi.y; raw[p][6] = hi.z; raw[p][7] = hi.w;
+    } else if (x_kind == KIND_Q8_1) {
+      const uint8_t* blk = static_cast<const uint8_t*>(a.x) + (static_cast<int64_t>(bb) * (a.K / 32) + j) * Q8_1_BYTES;
+      raw[p][0] = *reinterpret_cast<const uint32_t*>(blk + 4 + 8 * e);
+      raw[p][1] = *reinterpret_cast<const uint32_t*>(blk + 8 + 8 * e);
+      raw[p][2] = *reinterpret_cast<const uint32_t*>(blk);
+    } else {
+      const uint4 h = *reinterpret_cast<const uint4*>(static_cast<const uint16_t*>(a.x) + static_cast<int64_t>(bb) * a.K + j * 32 + e * 8);
+      raw[p][0] = h.x; raw[p][1] = h.y; raw[p][2] = h.z; raw[p][3] = h.w;
     }
   }
 
@@ -159,29 +166,46 @@ __device__ __forceinline__ void gemv_slab_q4k_workgroup(const GemvSlabArgs& a, u
       dst[i] = __builtin_amdgcn_raw_buffer_load_b128(wrsrc, min(row, last) * row_bytes + col16, t * 32 * row_bytes, 0);
     });
   };
+  // A short last step (N = 17408: 68 rows per slab = 32 + 32 + 4) is loaded up front into its own
+  // few registers and computed first, while the first full step is still on its way; done
+  // last, it would cost a whole step of MFMA and scale work with nothing left to overlap.
+  const int tail_rows = rows_wg & 31;
+  const bool early_tail = steps > 1 && tail_rows >= 1 && tail_rows <= EARLY_TAIL_ROWS;
+  sl_u32x4 tbuf[NLT];
+  if (early_tail) {
+    walk([&](int i, int row, int col16) {
+      if (i < NLT)
+        tbuf[i] = __builtin_amdgcn_raw_buffer_load_b128(wrsrc, min(row, tail_rows - 1) * row_bytes + col16,
+                                                        (steps - 1) * 32 * row_bytes, 0);
+    });
+  }
   // batch 8 holds 64 registers of fetched activations: its first weight loads wait until half of
   // them are quantized (they are not needed before the staging is done)
   if constexpr (B < 8) issue(0, buf);
 
   // ---- quantize the slice into LDS
 #pragma unroll
-  for (int b = 0; b < B; ++b) {
+  for (int p = 0; p < PASSES; ++p) {
     if constexpr (B >= 8) {
-      if (b == B / 2) issue(0, buf);
+      if (p == PASSES / 2) issue(0, buf);
     }
-#pragma unroll
-    for (int s = 0; s < BPW; ++s) {
-      uint32_t packed;
-      float xd;
-      q8_quantize4(x_kind, raw[b][s], true, packed, xd);
-      const bool used = b < a.rows && s < blocks_w;
-      packed = used ? packed : 0u;
-      xd = used ? xd : 0.0f;
-      *reinterpret_cast<uint32_t*>(xq + b * XQ_PITCH + s * 256 + team * 32 + e * 4) = packed;
-      const int total = oct_sum_i(dot4(0x01010101u, packed, 0));
+    const int gid = p * 16 + quad;
+    const int b = gid / (BPW * 8), rem = gid % (BPW * 8);
+    uint32_t packed[2];
+    float xd;
+    q8_quantize8(x_kind, raw[p], true, packed, xd);
+    const bool used = b < a.rows && (rem >> 3) < blocks_w;
+    packed[0] = used ? packed[0] : 0u;
+    packed[1] = used ? packed[1] : 0u;
+    xd = used ? xd : 0.0f;
+    int total = dot4(0x01010101u, packed[1], dot4(0x01010101u, packed[0], 0));
+    total += dpp_i<DPP_QUAD_XOR1>(total);
+    total += dpp_i<DPP_QUAD_XOR2>(total);
+    if (b < B) {
+      *reinterpret_cast<uint2*>(xq + b * XQ_PITCH + rem * 32 + e * 8) = make_uint2(packed[0], packed[1]);
       if (e == 0) {
-        rec[(s * 8 + team) * 16 + b] = xd;
-        rec[(s * 8 + team) * 16 + 8 + b] = xd * static_cast<float>(total);
+        rec[rem * 16 + b] = xd;
+        rec[rem * 16 + 8 + b] = xd * static_cast<float>(total);
       }
     }
   }
@@ -269,11 +293,21 @@ __device__ __forceinline__ void gemv_slab_q4k_workgroup(const GemvSlabArgs& a, u
       for (int v = 0; v < VB; ++v) done[u][v] = (u == t) ? acc[v] : done[u][v];
   };
 
+  const int full_steps = early_tail ? steps - 1 : steps;
 #pragma unroll 1
-  for (int t = 0; t < steps; ++t) {
-    to_lds(buf);
-    if (t + 1 < steps) issue(t + 1, buf);
-    compute(t);
+  for (int t = early_tail ? -1 : 0; t < full_steps; ++t) {
+    if (t < 0) {
+      walk([&](int i, int row, int col16) {
+        if (i < NLT) *reinterpret_cast<sl_u32x4*>(wq + row * PITCH + col16) = tbuf[i];   // rows 0..7
+      });
+      __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+      __builtin_amdgcn_wave_barrier();
+      __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+    } else {
+      to_lds(buf);
+      if (t + 1 < full_steps) issue(t + 1, buf);
+    }
+    compute(t < 0 ? steps - 1 : t);
   }
 
   // ---- K-slice reduction: each wave's partial sums [batch row][SLAB_MAX_ROWS] replace its weight piece
