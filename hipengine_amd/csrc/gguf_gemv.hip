@@ -5,7 +5,6 @@
 #include "gguf_gemv.hpp"
 #include "gguf_gemv_run.hpp"
 #include "gguf_gemv_stream.hpp"
-#include "gguf_gemv_mfma.hpp"
 #include "gguf_gemv_slab.hpp"
 
 #include "../../include/hipengine_gfx950.h"
@@ -99,61 +98,6 @@ const RunVariant* find_run_variant(int qt, int b, int g, int cb) {
   return nullptr;
 }
 
-// ---- tile form (Q4_K on the int8 MFMA, every load of the matrix in flight at once) ----
-
-template <int B, int BPW>
-constexpr int mfma_stage_regs() {
-  return B == 1 ? 5 : B == 2 ? 3 : B == 4 ? 2 : 1;
-}
-
-template <int B, int BPW>
-__global__ void __launch_bounds__(256, 2) gemv_mfma_q4k_kernel(GemvMfmaArgs a) {
-  extern __shared__ __align__(16) uint8_t smem[];
-  gemv_mfma_q4k_workgroup<B, BPW, mfma_stage_regs<B, BPW>()>(a, smem);
-}
-
-using MfmaKernelFn = void (*)(GemvMfmaArgs);
-struct MfmaVariant {
-  int b, bpw;
-  MfmaKernelFn fn;
-};
-#define MFMA_VARIANTS(B)                                                                             \
-  MfmaVariant{B, 1, gemv_mfma_q4k_kernel<B, 1>}, MfmaVariant{B, 2, gemv_mfma_q4k_kernel<B, 2>},       \
-  MfmaVariant{B, 3, gemv_mfma_q4k_kernel<B, 3>}, MfmaVariant{B, 4, gemv_mfma_q4k_kernel<B, 4>},       \
-  MfmaVariant{B, 5, gemv_mfma_q4k_kernel<B, 5>}
-const MfmaVariant kMfma[] = {MFMA_VARIANTS(1), MFMA_VARIANTS(2), MFMA_VARIANTS(4), MFMA_VARIANTS(8)};
-
-struct MfmaPlan {
-  int b, bpw, waves;
-  bool ok;
-};
-
-// Applies to Q4_K with at most 20 blocks per row (4 waves x 5 blocks).
-MfmaPlan default_mfma_plan(int qt, int rows, int64_t K, int64_t N) {
-  MfmaPlan p{};
-  const int nb = static_cast<int>(K / QK_K);
-  p.b = rows <= 1 ? 1 : rows <= 2 ? 2 : rows <= 4 ? 4 : 8;
-  p.bpw = (nb + 3) / 4;
-  p.waves = p.bpw > 0 ? (nb + p.bpw - 1) / p.bpw : 0;
-  p.ok = qt == GGML_Q4_K && rows <= 8 && nb >= 1 && p.bpw <= 5 && N >= 1 &&
-         gemv_mfma_lds_bytes(p.b, static_cast<int>(K), p.waves) <= 64 * 1024;
-  return p;
-}
-
-int launch_gemv_mfma(const void* x, int x_kind, const uint8_t* w, void* out, int out_kind, int rows, int64_t K,
-                     int64_t N, const MfmaPlan& p, hipStream_t stream) {
-  const int nb = static_cast<int>(K / QK_K);
-  const MfmaVariant* v = nullptr;
-  for (const MfmaVariant& c : kMfma)
-    if (c.b == p.b && c.bpw == p.bpw) v = &c;
-  if (!v || rows > p.b || p.waves < 1 || p.waves > 4 || p.waves * p.bpw < nb) return static_cast<int>(hipErrorInvalidValue);
-  const size_t lds = gemv_mfma_lds_bytes(p.b, static_cast<int>(K), p.waves);
-  if (lds > 64 * 1024) return static_cast<int>(hipErrorInvalidValue);
-  GemvMfmaArgs a{x, w, out, x_kind, out_kind, rows, static_cast<int>(K), static_cast<int>(N), p.waves};
-  hipLaunchKernelGGL(v->fn, dim3(static_cast<unsigned>((N + 31) / 32)), dim3(p.waves * 64), lds, stream, a);
-  return static_cast<int>(hipGetLastError());
-}
-
 // ---- slab form (Q4_K on the int8 MFMA, one workgroup per CU, waves split K) ----
 
 // BPW = 1: up to 16 waves (K <= 4096); BPW = 2: up to 12 waves (K <= 6144), whose 64
@@ -236,10 +180,10 @@ RunPlan default_run_plan(int qt, int rows, int64_t K, int64_t N) {
   p.g = 16 / gcd_int(nb, 16);
   const int m = p.g * nb / 16;
   p.cb = m >= 2 ? 5 : 1;
-  // Every workgroup quantizes the whole activation row (nb*64 lane tasks), so the
-  // workgroup is sized for at most ~3 of them per thread rather than for a large
+  // Every workgroup quantizes the whole activation row (nb*32 lane tasks of 8 values), so
+  // the workgroup is sized for at most ~2 of them per thread rather than for a large
   // grid: 13.5 -> 6.7 us at K=5120, N=1024 with 8 waves instead of 1.
-  const int want = (nb * 64 + 191) / 192;
+  const int want = (nb * 32 + 127) / 128;
   p.waves = want >= 5 ? 8 : want >= 3 ? 4 : 2;
   p.ok = rows <= 2 && p.g <= 8 && gemv_run_lds_bytes(qt, p.b, static_cast<int>(K)) <= 64 * 1024 &&
          find_run_variant(qt, p.b, p.g, p.cb) != nullptr;
@@ -284,8 +228,8 @@ __global__ void __launch_bounds__((stream_max_threads<B>())) gemv_stream_kernel(
 
 using StreamKernelFn = void (*)(GemvStreamArgs);
 
-// `long_k`: the instantiation that fetches nine activation groups per thread up front
-// (batch 1 only); the other fetches three (batch 1, 2) or one (batch 4, 8).
+// `long_k`: the instantiation that fetches five activation groups (of 8 values) per thread
+// up front (batch 1 only); the other fetches two (batch 1, 2) or one (batch 4, 8).
 struct StreamVariant {
   int qt, b, d;
   bool long_k;
@@ -294,19 +238,19 @@ struct StreamVariant {
 };
 
 #define STREAM_VARIANT(QT, B, D) \
-  StreamVariant { QT, B, D, false, gemv_stream_kernel<QT, B, D, (B <= 2 ? 3 : 1)>, {nullptr, nullptr, nullptr, nullptr} }
+  StreamVariant { QT, B, D, false, gemv_stream_kernel<QT, B, D, (B <= 2 ? 2 : 1)>, {nullptr, nullptr, nullptr, nullptr} }
 #define STREAM_VARIANT_BY_KIND(QT, B, D, S, LONG_K)                                                      \
   StreamVariant { QT, B, D, LONG_K, gemv_stream_kernel<QT, B, D, S>,                                      \
                   {gemv_stream_kernel<QT, B, D, S, KIND_F32>, gemv_stream_kernel<QT, B, D, S, KIND_BF16>, \
                    gemv_stream_kernel<QT, B, D, S, KIND_F16>, gemv_stream_kernel<QT, B, D, S, KIND_Q8_1>} }
 
 const StreamVariant kStream[] = {
-    STREAM_VARIANT_BY_KIND(GGML_Q4_K, 1, 3, 3, false), STREAM_VARIANT(GGML_Q4_K, 1, 5), STREAM_VARIANT(GGML_Q4_K, 2, 3),
-    STREAM_VARIANT(GGML_Q4_K, 2, 5), STREAM_VARIANT_BY_KIND(GGML_Q6_K, 1, 3, 3, false), STREAM_VARIANT(GGML_Q6_K, 1, 5),
-    STREAM_VARIANT(GGML_Q6_K, 2, 3), STREAM_VARIANT(GGML_Q6_K, 2, 5), STREAM_VARIANT_BY_KIND(GGML_Q8_0, 1, 3, 3, false),
+    STREAM_VARIANT_BY_KIND(GGML_Q4_K, 1, 3, 2, false), STREAM_VARIANT(GGML_Q4_K, 1, 5), STREAM_VARIANT(GGML_Q4_K, 2, 3),
+    STREAM_VARIANT(GGML_Q4_K, 2, 5), STREAM_VARIANT_BY_KIND(GGML_Q6_K, 1, 3, 2, false), STREAM_VARIANT(GGML_Q6_K, 1, 5),
+    STREAM_VARIANT(GGML_Q6_K, 2, 3), STREAM_VARIANT(GGML_Q6_K, 2, 5), STREAM_VARIANT_BY_KIND(GGML_Q8_0, 1, 3, 2, false),
     STREAM_VARIANT(GGML_Q8_0, 1, 5), STREAM_VARIANT(GGML_Q8_0, 2, 3), STREAM_VARIANT(GGML_Q8_0, 2, 5),
-    STREAM_VARIANT_BY_KIND(GGML_Q4_K, 1, 3, 9, true), STREAM_VARIANT_BY_KIND(GGML_Q6_K, 1, 3, 9, true),
-    STREAM_VARIANT_BY_KIND(GGML_Q8_0, 1, 3, 9, true),
+    STREAM_VARIANT_BY_KIND(GGML_Q4_K, 1, 3, 5, true), STREAM_VARIANT_BY_KIND(GGML_Q6_K, 1, 3, 5, true),
+    STREAM_VARIANT_BY_KIND(GGML_Q8_0, 1, 3, 5, true),
     STREAM_VARIANT(GGML_Q4_K, 4, 3), STREAM_VARIANT(GGML_Q4_K, 8, 3), STREAM_VARIANT(GGML_Q6_K, 4, 3),
     STREAM_VARIANT(GGML_Q6_K, 8, 3), STREAM_VARIANT(GGML_Q8_0, 4, 3), STREAM_VARIANT(GGML_Q8_0, 8, 3),
 };
@@ -361,8 +305,9 @@ StreamPlan default_stream_plan(int qt, int rows, int64_t K, int64_t N) {
 int launch_gemv_stream(int qt, const void* x, int x_kind, const uint8_t* w, void* out, int out_kind, int rows,
                        int64_t K, int64_t N, const StreamPlan& p, hipStream_t stream) {
   const int nb = static_cast<int>(K / QK_K);
-  // more than three activation groups per thread: take the instantiation that fetches nine up front
-  const StreamVariant* v = find_stream_variant(qt, p.b, p.d, p.waves > 0 && nb > 3 * p.waves);
+  // more than two activation groups per thread (16 teams of 4 lanes per wave): take the
+  // instantiation that fetches five up front
+  const StreamVariant* v = find_stream_variant(qt, p.b, p.d, p.waves > 0 && nb > 4 * p.waves);
   if (!v || nb < 16 || rows > p.b || p.waves < 1 || p.waves > (p.b == 1 ? 12 : 8) || p.waves_total < p.waves ||
       (p.waves_total % p.waves) != 0 || p.waves_total > N) {
     return static_cast<int>(hipErrorInvalidValue);
@@ -574,23 +519,6 @@ extern "C" int hipengine_gfx950_gguf_q8_1_fused_gemv_stream_tuned(
   p.waves_total = waves_total;
   return launch_gemv_stream(ggml_type, x, x_kind, qweight, out, out_kind, static_cast<int>(rows), in_features,
                             out_features, p, stream);
-}
-
-extern "C" int hipengine_gfx950_gguf_q4_k_q8_1_fused_gemv_tile_tuned(const void* x, int32_t x_kind,
-                                                                    const uint8_t* qweight, void* out,
-                                                                    int32_t out_kind, int64_t rows,
-                                                                    int64_t in_features, int64_t out_features,
-                                                                    int32_t blocks_per_wave, hipStream_t stream) {
-  if (!x || !qweight || !out || x_kind < KIND_F32 || x_kind > KIND_Q8_1 || out_kind < KIND_F32 ||
-      out_kind > KIND_F16 || rows <= 0 || rows > 8 || in_features <= 0 || (in_features % QK_K) != 0 ||
-      out_features <= 0 || blocks_per_wave < 1 || blocks_per_wave > 5) {
-    return static_cast<int>(hipErrorInvalidValue);
-  }
-  MfmaPlan p = default_mfma_plan(GGML_Q4_K, static_cast<int>(rows), in_features, out_features);
-  p.bpw = blocks_per_wave;
-  p.waves = static_cast<int>((in_features / QK_K + p.bpw - 1) / p.bpw);
-  return launch_gemv_mfma(x, x_kind, qweight, out, out_kind, static_cast<int>(rows), in_features, out_features, p,
-                          stream);
 }
 
 extern "C" int hipengine_gfx950_gguf_q4_k_q8_1_fused_gemv_slab_tuned(const void* x, int32_t x_kind,

@@ -53,19 +53,6 @@ inline size_t gemv_run_lds_bytes(int qt, int B, int K) {
   return B * nb * (stride + 64 + (qt == GGML_Q6_K ? 64 : 0));
 }
 
-// q = clamp(roundf(v / d), -128, 127) evaluated through the reciprocal.  The
-// product v*inv is within 3e-5 of the exactly rounded quotient (|v/d| <= 127),
-// so truncating v*inv +- 0.5 gives roundf of the quotient unless the
-// fractional part is that close to one half; those lanes redo the IEEE
-// division.  Bit-exact with the direct evaluation.
-__device__ __forceinline__ int q8_round_div(float v, float d, float inv, bool exact) {
-  const float t = v * inv;
-  const float f = fabsf(t) - floorf(fabsf(t));
-  int q = static_cast<int>(t + copysignf(0.5f, t));
-  if (__builtin_expect(exact || fabsf(f - 0.5f) < 1.0e-4f, 0)) q = static_cast<int>(roundf(v / d));
-  return max(-128, min(127, q));
-}
-
 // amax / 127.0f, correctly rounded, in three operations: q = a*c, r = fma(-q, 127, a),
 // q' = fma(r, c, q) with c = RN(1/127).  Equal to the IEEE quotient for every finite
 // non-negative float (checked exhaustively on the host over all 2^31 - 2^23 values).
@@ -75,60 +62,18 @@ __device__ __forceinline__ float div_by_127(float a) {
   return __builtin_fmaf(__builtin_fmaf(-q, 127.0f, a), c, q);
 }
 
-// One lane's share of a 32-value activation group (8 lanes x 4 values): quantize the
-// fetched values to q8_1 (or take them from a q8_1 block) -> 4 packed int8 and the
-// group's scale, rounded to half as the q8_1 block stores it.
-__device__ __forceinline__ void q8_quantize4(int x_kind, const uint32_t (&raw)[4], bool present, uint32_t& packed,
-                                             float& xd) {
-  packed = 0;
-  xd = 0.0f;
-  if (!present) return;
-  if (x_kind == KIND_Q8_1) {
-    packed = raw[0];
-    xd = f16_bits_to_float(raw[1] & 0xFFFFu);
-    return;
-  }
-  float v0, v1, v2, v3;
-  if (x_kind == KIND_F32) {
-    v0 = bits_to_float(raw[0]); v1 = bits_to_float(raw[1]); v2 = bits_to_float(raw[2]); v3 = bits_to_float(raw[3]);
-  } else if (x_kind == KIND_BF16) {
-    v0 = bf16_bits_to_float(raw[0] & 0xFFFFu); v1 = bf16_bits_to_float(raw[0] >> 16);
-    v2 = bf16_bits_to_float(raw[1] & 0xFFFFu); v3 = bf16_bits_to_float(raw[1] >> 16);
-  } else {
-    v0 = f16_bits_to_float(raw[0] & 0xFFFFu); v1 = f16_bits_to_float(raw[0] >> 16);
-    v2 = f16_bits_to_float(raw[1] & 0xFFFFu); v3 = f16_bits_to_float(raw[1] >> 16);
-  }
-  const float amax = oct_max(fmaxf(fmaxf(fabsf(v0), fabsf(v1)), fmaxf(fabsf(v2), fabsf(v3))));
-  const float d = div_by_127(amax);
-  if (amax != 0.0f) {
-    // Fast path: t = v * rcp(d) is within 3e-5 of the quotient (|v/d| <= 127, reciprocal good
-    // to 1 ulp).  t + 1.5*2^23 rounds t to the nearest integer r and leaves r's two's
-    // complement in the low mantissa bits; unless t is within 1e-4 of a tie, r equals
-    // roundf(v/d).  Near ties, and scales in the denormal range where the reciprocal
-    // overflows, redo the lane's four values with the IEEE division.
-    constexpr float MAGIC = 12582912.0f;
-    const float inv = __builtin_amdgcn_rcpf(d);
-    const float t0 = v0 * inv, t1 = v1 * inv, t2 = v2 * inv, t3 = v3 * inv;
-    const float m0 = t0 + MAGIC, m1 = t1 + MAGIC, m2 = t2 + MAGIC, m3 = t3 + MAGIC;
-    const float e0 = fabsf(t0 - (m0 - MAGIC)), e1 = fabsf(t1 - (m1 - MAGIC));
-    const float e2 = fabsf(t2 - (m2 - MAGIC)), e3 = fabsf(t3 - (m3 - MAGIC));
-    const bool near_tie = __builtin_fmaxf(__builtin_fmaxf(e0, e1), __builtin_fmaxf(e2, e3)) > 0.4999f;
-    packed = __builtin_amdgcn_perm(float_to_bits(m1), float_to_bits(m0), 0x0c0c0400u) |
-             __builtin_amdgcn_perm(float_to_bits(m3), float_to_bits(m2), 0x04000c0cu);
-    if (__builtin_expect(near_tie || d < 1.0e-30f, 0)) {
-      const int q0 = max(-128, min(127, static_cast<int>(roundf(v0 / d))));
-      const int q1 = max(-128, min(127, static_cast<int>(roundf(v1 / d))));
-      const int q2 = max(-128, min(127, static_cast<int>(roundf(v2 / d))));
-      const int q3 = max(-128, min(127, static_cast<int>(roundf(v3 / d))));
-      packed = (q0 & 0xFF) | ((q1 & 0xFF) << 8) | ((q2 & 0xFF) << 16) | (static_cast<uint32_t>(q3 & 0xFF) << 24);
-    }
-  }
-  xd = static_cast<float>(static_cast<half_t>(d));
-}
-
-// The same for a group held by 4 lanes, 8 values per lane: half the per-group overhead
-// (scale, reciprocal, reductions) per value.  raw: 8 floats, or 8 halves/bf16 in raw[0..3],
-// or for q8_1 input the lane's 8 quants in raw[0..1] and the block's {d, s} halves in raw[2].
+// One lane's share of a 32-value activation group (4 lanes x 8 values): quantize the
+// fetched values to q8_1 (or take them from a q8_1 block) -> 8 packed int8 and the
+// group's scale, rounded to half as the q8_1 block stores it.  raw: 8 floats, or 8
+// halves/bf16 in raw[0..3], or for q8_1 input the lane's 8 quants in raw[0..1] and the
+// block's {d, s} halves in raw[2].
+//
+// q = clamp(roundf(v / d), -128, 127) goes through the reciprocal: t = v * rcp(d) is within
+// 3e-5 of the quotient (|v/d| <= 127, reciprocal good to 1 ulp).  t + 1.5*2^23 rounds t to
+// the nearest integer r and leaves r's two's complement in the low mantissa bits; unless t
+// is within 1e-4 of a tie, r equals roundf(v/d).  Near ties, and scales in the denormal
+// range where the reciprocal overflows, redo the lane's values with the IEEE division.
+// Bit-exact with the direct evaluation.
 __device__ __forceinline__ void q8_quantize8(int x_kind, const uint32_t (&raw)[8], bool present, uint32_t (&packed)[2],
                                              float& xd) {
   packed[0] = 0; packed[1] = 0;
@@ -154,7 +99,7 @@ __device__ __forceinline__ void q8_quantize8(int x_kind, const uint32_t (&raw)[8
   const float amax = bits_to_float(u);
   const float d = div_by_127(amax);
   if (amax != 0.0f) {
-    constexpr float MAGIC = 12582912.0f;               // see q8_quantize4
+    constexpr float MAGIC = 12582912.0f;
     const float inv = __builtin_amdgcn_rcpf(d);
     float mg[8], worst = 0.0f;
 #pragma unroll
@@ -180,150 +125,91 @@ __device__ __forceinline__ void q8_quantize8(int x_kind, const uint32_t (&raw)[8
   xd = static_cast<float>(static_cast<half_t>(d));
 }
 
-// Whole-K activation staging for the run kernel.
+// Whole-K activation staging for the run and stream kernels: teams of 4 lanes take one
+// 32-value group each, 8 values per lane.
 //   q8   : [B][nb] blocks, Q8S bytes apart
 //   rec  : [B][nb][4] 16-byte records, one per lane q of a block:
 //            Q4_K {xd(2q), xd(2q+1), xd*qsum(2q), xd*qsum(2q+1)}
 //            Q8_0 {xd(2q), xd(2q+1), -, -}
 //            Q6_K {xd(4h), xd(4h+1), xd(4h+2), xd(4h+3)}, q = 2h+t
 //   s16  : Q6_K only, [B][nb][4] x {qsum16(4h+j, half t)} j = 0..3
-template <int QT, int B>
-__device__ __forceinline__ void gemv_run_stage(const GemvRunArgs& a, uint8_t* q8, float* rec, int* s16) {
-  constexpr int Q8S = run_q8_stride<QT>();
-  const int tid = threadIdx.x;
-  const int team = tid >> 3, e = tid & 7, nteams = blockDim.x >> 3;
-  const int nb = a.K / QK_K;
-  const int groups = nb * 8;
-#pragma unroll
-  for (int b = 0; b < B; ++b) {
-    for (int j = team; j < groups; j += nteams) {
-      uint32_t packed = 0;
-      float xd = 0.0f;
-      if (b < a.rows) {
-        if (a.x_kind == KIND_Q8_1) {
-          const uint8_t* blk = static_cast<const uint8_t*>(a.x) +
-                               (static_cast<int64_t>(b) * (a.K / 32) + j) * Q8_1_BYTES;
-          packed = *reinterpret_cast<const uint32_t*>(blk + 4 + 4 * e);
-          xd = f16_bits_to_float(*reinterpret_cast<const uint32_t*>(blk) & 0xFFFFu);
-        } else {
-          const int64_t k0 = static_cast<int64_t>(b) * a.K + j * 32 + e * 4;
-          float v0, v1, v2, v3;
-          if (a.x_kind == KIND_F32) {
-            const float4 v = *reinterpret_cast<const float4*>(static_cast<const float*>(a.x) + k0);
-            v0 = v.x; v1 = v.y; v2 = v.z; v3 = v.w;
-          } else {
-            const uint2 v = *reinterpret_cast<const uint2*>(static_cast<const uint16_t*>(a.x) + k0);
-            if (a.x_kind == KIND_BF16) {
-              v0 = bf16_bits_to_float(v.x & 0xFFFFu); v1 = bf16_bits_to_float(v.x >> 16);
-              v2 = bf16_bits_to_float(v.y & 0xFFFFu); v3 = bf16_bits_to_float(v.y >> 16);
-            } else {
-              v0 = f16_bits_to_float(v.x & 0xFFFFu); v1 = f16_bits_to_float(v.x >> 16);
-              v2 = f16_bits_to_float(v.y & 0xFFFFu); v3 = f16_bits_to_float(v.y >> 16);
-            }
-          }
-          const float amax = oct_max(fmaxf(fmaxf(fabsf(v0), fabsf(v1)), fmaxf(fabsf(v2), fabsf(v3))));
-          const float d = div_by_127(amax);
-          if (amax != 0.0f) {
-            const float inv = __builtin_amdgcn_rcpf(d);
-            const bool exact = d < 1.0e-30f;
-            const int q0 = q8_round_div(v0, d, inv, exact), q1 = q8_round_div(v1, d, inv, exact);
-            const int q2 = q8_round_div(v2, d, inv, exact), q3 = q8_round_div(v3, d, inv, exact);
-            packed = (q0 & 0xFF) | ((q1 & 0xFF) << 8) | ((q2 & 0xFF) << 16) | (static_cast<uint32_t>(q3 & 0xFF) << 24);
-          }
-          xd = static_cast<float>(static_cast<half_t>(d));
-        }
-      }
-      const int kb = j >> 3, sb = j & 7;
-      *reinterpret_cast<uint32_t*>(q8 + (b * nb + kb) * Q8S + sb * 32 + e * 4) = packed;
-      const int part = dot4(0x01010101u, packed, 0);
-      float* r = rec + (b * nb + kb) * 16;
-      if constexpr (QT == GGML_Q6_K) {
-        int h16 = part;
-        h16 += dpp_i<DPP_QUAD_XOR1>(h16);
-        h16 += dpp_i<DPP_QUAD_XOR2>(h16);
-        // group sb = 4h + jj, half t = e>>2 -> record of lane q = 2h+t, slot jj
-        const int h = sb >> 2, jj = sb & 3;
-        if ((e & 3) == 0) s16[(b * nb + kb) * 16 + (2 * h + (e >> 2)) * 4 + jj] = h16;
-        if (e == 0) {   // xd of group sb goes to both records (t = 0, 1) of half h
-          r[(2 * h) * 4 + jj] = xd;
-          r[(2 * h + 1) * 4 + jj] = xd;
-        }
-      } else {
-        const int total = oct_sum_i(part);
-        if (e == 0) {   // sub-block sb -> record of lane q = sb>>1, slot sb&1 (+2 for the xd*qsum term)
-          r[(sb >> 1) * 4 + (sb & 1)] = xd;
-          if constexpr (QT == GGML_Q4_K) r[(sb >> 1) * 4 + 2 + (sb & 1)] = xd * static_cast<float>(total);
-        }
-      }
-    }
-  }
-}
-
-
-// The same staging split in two so that a kernel can put the activation loads
-// in front of its weight loads: vmcnt counts loads in issue order, so waiting
-// for activations issued AFTER the weight ring would also wait for the ring.
+//
+// Split in two so that a kernel can put the activation loads in front of its weight
+// loads: vmcnt counts loads in issue order, so waiting for activations issued AFTER
+// the weight ring would also wait for the ring.
 //   stage_fetch  : issue the loads of this thread's first S groups per batch row
 //   stage_commit : quantize them into LDS; groups beyond the first S per thread
 //                  are loaded and quantized here (large K only)
 template <int B, int S>
 struct StageRegs {
-  uint32_t raw[B][S][4];
+  uint32_t raw[B][S][8];
 };
+
+// The lane's 8 values of group j of one batch row (or its share of a q8_1 block).
+__device__ __forceinline__ void gemv_run_fetch8(const GemvRunArgs& a, int b, int j, int e, uint32_t (&raw)[8]) {
+#pragma unroll
+  for (int i = 0; i < 8; ++i) raw[i] = 0u;
+  if (a.x_kind == KIND_F32) {
+    const uint4* src = reinterpret_cast<const uint4*>(static_cast<const float*>(a.x) + static_cast<int64_t>(b) * a.K + j * 32 + e * 8);
+    const uint4 lo = src[0], hi = src[1];
+    raw[0] = lo.x; raw[1] = lo.y; raw[2] = lo.z; raw[3] = lo.w;
+    raw[4] = hi.x; raw[5] = hi.y; raw[6] = hi.z; raw[7] = hi.w;
+  } else if (a.x_kind == KIND_Q8_1) {
+    const uint8_t* blk = static_cast<const uint8_t*>(a.x) + (static_cast<int64_t>(b) * (a.K / 32) + j) * Q8_1_BYTES;
+    raw[0] = *reinterpret_cast<const uint32_t*>(blk + 4 + 8 * e);
+    raw[1] = *reinterpret_cast<const uint32_t*>(blk + 8 + 8 * e);
+    raw[2] = *reinterpret_cast<const uint32_t*>(blk);
+  } else {
+    const uint4 h = *reinterpret_cast<const uint4*>(static_cast<const uint16_t*>(a.x) + static_cast<int64_t>(b) * a.K + j * 32 + e * 8);
+    raw[0] = h.x; raw[1] = h.y; raw[2] = h.z; raw[3] = h.w;
+  }
+}
 
 template <int QT, int B, int S>
 __device__ __forceinline__ void gemv_run_stage_fetch(const GemvRunArgs& a, StageRegs<B, S>& sr) {
   const int tid = threadIdx.x;
-  const int team = tid >> 3, e = tid & 7, nteams = blockDim.x >> 3;
+  const int team = tid >> 2, e = tid & 3, nteams = blockDim.x >> 2;
   const int groups = (a.K / QK_K) * 8;
 #pragma unroll
   for (int b = 0; b < B; ++b) {
 #pragma unroll
     for (int s = 0; s < S; ++s) {
       const int j = team + s * nteams;
-      uint4 v = make_uint4(0u, 0u, 0u, 0u);
       if (b < a.rows && j < groups) {
-        if (a.x_kind == KIND_F32) {
-          v = *reinterpret_cast<const uint4*>(static_cast<const float*>(a.x) + static_cast<int64_t>(b) * a.K + j * 32 + e * 4);
-        } else if (a.x_kind == KIND_Q8_1) {
-          const uint8_t* blk = static_cast<const uint8_t*>(a.x) + (static_cast<int64_t>(b) * (a.K / 32) + j) * Q8_1_BYTES;
-          v.x = *reinterpret_cast<const uint32_t*>(blk + 4 + 4 * e);
-          v.y = *reinterpret_cast<const uint32_t*>(blk);
-        } else {
-          const uint2 h = *reinterpret_cast<const uint2*>(static_cast<const uint16_t*>(a.x) + static_cast<int64_t>(b) * a.K + j * 32 + e * 4);
-          v.x = h.x; v.y = h.y;
-        }
+        gemv_run_fetch8(a, b, j, e, sr.raw[b][s]);
+      } else {
+#pragma unroll
+        for (int i = 0; i < 8; ++i) sr.raw[b][s][i] = 0u;
       }
-      sr.raw[b][s][0] = v.x; sr.raw[b][s][1] = v.y; sr.raw[b][s][2] = v.z; sr.raw[b][s][3] = v.w;
     }
   }
 }
 
-// Quantize one fetched group (4 values of one lane) and write it to the LDS image.
+// Quantize one fetched group (8 values of one lane) and write it to the LDS image.
 template <int QT>
-__device__ __forceinline__ void gemv_run_stage_one(int x_kind, const uint32_t (&raw)[4], bool present, int j, int e,
+__device__ __forceinline__ void gemv_run_stage_one(int x_kind, const uint32_t (&raw)[8], bool present, int j, int e,
                                                    uint8_t* q8_row, float* rec_row, int* s16_row) {
   constexpr int Q8S = run_q8_stride<QT>();
-  uint32_t packed;
+  uint32_t packed[2];
   float xd;
-  q8_quantize4(x_kind, raw, present, packed, xd);
+  q8_quantize8(x_kind, raw, present, packed, xd);
   const int kb = j >> 3, sb = j & 7;
-  *reinterpret_cast<uint32_t*>(q8_row + kb * Q8S + sb * 32 + e * 4) = packed;
-  const int part = dot4(0x01010101u, packed, 0);
+  *reinterpret_cast<uint2*>(q8_row + kb * Q8S + sb * 32 + e * 8) = make_uint2(packed[0], packed[1]);
+  const int part = dot4(0x01010101u, packed[1], dot4(0x01010101u, packed[0], 0));
   float* r = rec_row + kb * 16;
   if constexpr (QT == GGML_Q6_K) {
-    int h16 = part;
-    h16 += dpp_i<DPP_QUAD_XOR1>(h16);
-    h16 += dpp_i<DPP_QUAD_XOR2>(h16);
+    const int h16 = part + dpp_i<DPP_QUAD_XOR1>(part);   // lanes 0,1: values 0..15; lanes 2,3: values 16..31
+    // group sb = 4h + jj, half t = e>>1 -> record of lane q = 2h+t, slot jj
     const int h = sb >> 2, jj = sb & 3;
-    if ((e & 3) == 0) s16_row[kb * 16 + (2 * h + (e >> 2)) * 4 + jj] = h16;
-    if (e == 0) {
+    if ((e & 1) == 0) s16_row[kb * 16 + (2 * h + (e >> 1)) * 4 + jj] = h16;
+    if (e == 0) {   // xd of group sb goes to both records (t = 0, 1) of half h
       r[(2 * h) * 4 + jj] = xd;
       r[(2 * h + 1) * 4 + jj] = xd;
     }
   } else {
-    const int total = oct_sum_i(part);
-    if (e == 0) {
+    int total = part + dpp_i<DPP_QUAD_XOR1>(part);
+    total += dpp_i<DPP_QUAD_XOR2>(total);
+    if (e == 0) {   // sub-block sb -> record of lane q = sb>>1, slot sb&1 (+2 for the xd*qsum term)
       r[(sb >> 1) * 4 + (sb & 1)] = xd;
       if constexpr (QT == GGML_Q4_K) r[(sb >> 1) * 4 + 2 + (sb & 1)] = xd * static_cast<float>(total);
     }
@@ -335,7 +221,7 @@ __device__ __forceinline__ void gemv_run_stage_commit(const GemvRunArgs& a, cons
                                                       float* rec, int* s16) {
   constexpr int Q8S = run_q8_stride<QT>();
   const int tid = threadIdx.x;
-  const int team = tid >> 3, e = tid & 7, nteams = blockDim.x >> 3;
+  const int team = tid >> 2, e = tid & 3, nteams = blockDim.x >> 2;
   const int nb = a.K / QK_K;
   const int groups = nb * 8;
 #pragma unroll
@@ -348,27 +234,19 @@ __device__ __forceinline__ void gemv_run_stage_commit(const GemvRunArgs& a, cons
       const int j = team + s * nteams;
       if (j < groups) gemv_run_stage_one<QT>(a.x_kind, sr.raw[b][s], b < a.rows, j, e, q8_row, rec_row, s16_row);
     }
-    // large K: the rest is loaded here, four groups per thread at a time so that the
-    // load latency is paid once per four groups and not once per group
-    constexpr int P = 4;
+    // large K: the rest is loaded here, two groups per thread at a time so that the
+    // load latency is paid once per two groups and not once per group
+    constexpr int P = 2;
     for (int j0 = team + S * nteams; j0 < groups; j0 += P * nteams) {
-      uint32_t raw[P][4];
+      uint32_t raw[P][8];
 #pragma unroll
       for (int p = 0; p < P; ++p) {
         const int j = j0 + p * nteams;
-        raw[p][0] = raw[p][1] = raw[p][2] = raw[p][3] = 0u;
         if (b < a.rows && j < groups) {
-          if (a.x_kind == KIND_F32) {
-            const uint4 v = *reinterpret_cast<const uint4*>(static_cast<const float*>(a.x) + static_cast<int64_t>(b) * a.K + j * 32 + e * 4);
-            raw[p][0] = v.x; raw[p][1] = v.y; raw[p][2] = v.z; raw[p][3] = v.w;
-          } else if (a.x_kind == KIND_Q8_1) {
-            const uint8_t* blk = static_cast<const uint8_t*>(a.x) + (static_cast<int64_t>(b) * (a.K / 32) + j) * Q8_1_BYTES;
-            raw[p][0] = *reinterpret_cast<const uint32_t*>(blk + 4 + 4 * e);
-            raw[p][1] = *reinterpret_cast<const uint32_t*>(blk);
-          } else {
-            const uint2 h = *reinterpret_cast<const uint2*>(static_cast<const uint16_t*>(a.x) + static_cast<int64_t>(b) * a.K + j * 32 + e * 4);
-            raw[p][0] = h.x; raw[p][1] = h.y;
-          }
+          gemv_run_fetch8(a, b, j, e, raw[p]);
+        } else {
+#pragma unroll
+          for (int i = 0; i < 8; ++i) raw[p][i] = 0u;
         }
       }
 #pragma unroll
@@ -470,7 +348,7 @@ __device__ __forceinline__ void gemv_run_workgroup(const GemvRunArgs& a, uint8_t
 
   // activation loads first, then the weight loads, then the quantization: the wait
   // for the activations must not include the (later issued) weight loads
-  constexpr int S = 3;
+  constexpr int S = 2;
   StageRegs<B, S> sr;
   gemv_run_stage_fetch<QT, B, S>(a, sr);
 

@@ -69,7 +69,7 @@ __device__ __forceinline__ void gemv_stream_workgroup(const GemvStreamArgs& a, u
   // Activation loads go first (see gemv_run_stage_fetch), then the weight ring.
   // S activation groups per thread have their loads issued ahead of the weight ring,
   // per batch row.  Loads issued after the ring queue behind it (the memory counter
-  // retires in order), so a long K wants them all up front: nine cover K = 17408.
+  // retires in order), so a long K wants them all up front: five cover K = 17408.
   const GemvRunArgs ra{a.x, a.w, a.out, XK >= 0 ? XK : a.x_kind, a.out_kind, a.rows, a.K, a.N, a.waves};
   StageRegs<B, S> sr;
   gemv_run_stage_fetch<QT, B, S>(ra, sr);

@@ -131,18 +131,6 @@ def gguf_q8_1_fused_gemv_stream_tuned(quant_key: str, x_ptr: int, x_kind: str, q
                     in_features, out_features, loads_in_flight, waves, waves_total, stream), runtime)
 
 
-def gguf_q4_k_q8_1_fused_gemv_tile_tuned(x_ptr: int, x_kind: str, qweight_ptr: int, out_ptr: int, out_kind: str,
-                                         rows: int, in_features: int, out_features: int, *, blocks_per_wave: int,
-                                         stream: int = 0, library: ctypes.CDLL | None = None,
-                                         runtime: HipRuntime | None = None) -> None:
-    """The tile (int8 MFMA) form of the fused Q4_K GEMV with an explicit K split (tuning sweeps only)."""
-    validate_linear(rows, in_features, out_features)
-    fn = entry("hipengine_gfx950_gguf_q4_k_q8_1_fused_gemv_tile_tuned",
-               [VOID, I32, VOID, VOID, I32, I64, I64, I64, I32, VOID], library)
-    check_launch(fn(x_ptr, _KINDS[x_kind], qweight_ptr, out_ptr, _KINDS[out_kind], rows, in_features, out_features,
-                    blocks_per_wave, stream), runtime)
-
-
 def gguf_q4_k_q8_1_fused_gemv_slab_tuned(x_ptr: int, x_kind: str, qweight_ptr: int, out_ptr: int, out_kind: str,
                                          rows: int, in_features: int, out_features: int, *,
                                          rows_per_workgroup: int = 0, stream: int = 0,

@@ -152,14 +152,6 @@ int hipengine_gfx950_gguf_q8_1_fused_gemv_stream_tuned(int32_t ggml_type, const 
                                                        int32_t loads_in_flight, int32_t waves, int32_t waves_total,
                                                        hipengine_stream_t stream);
 
-/* The "tile" form for Q4_K: 32 output rows per workgroup on the int8 MFMA, K split
- * over ceil((K/256) / blocks_per_wave) <= 4 waves, every weight load issued up
- * front.  rows <= 8, blocks_per_wave 1..5.  New here. */
-int hipengine_gfx950_gguf_q4_k_q8_1_fused_gemv_tile_tuned(const void* x, int32_t x_kind, const uint8_t* qweight,
-                                                          void* out, int32_t out_kind, int64_t rows,
-                                                          int64_t in_features, int64_t out_features,
-                                                          int32_t blocks_per_wave, hipengine_stream_t stream);
-
 /* The "slab" form for Q4_K: one workgroup per CU owns rows_per_workgroup (<= 96;
  * 0 = ceil(out_features / 256)) consecutive output rows, its waves split K in
  * slices of one or two 256-value blocks and run on the int8 MFMA.  rows <= 8,

@@ -200,24 +200,6 @@ def test_more_than_eight_rows_and_determinism(dev):
     assert O.max_rel_err(one, a[7:8]) <= 1e-4
 
 
-@pytest.mark.parametrize("rows,k,n,bpw", [(1, 5120, 96, 5), (2, 2048, 70, 2), (4, 1024, 33, 1), (8, 3072, 64, 3),
-                                          (3, 1280, 40, 5), (8, 512, 200, 1)])
-def test_tile_form_q4_k(dev, rows, k, n, bpw):
-    """The int8 MFMA ("tile") form of the fused Q4_K GEMV, K split over up to four waves."""
-    rng = np.random.default_rng(77 + rows + k)
-    x = rng.standard_normal((rows, k)).astype(np.float32)
-    x[0, :32] = 0.0
-    w = O.random_weight(O.GGML_Q4_K, n, k, seed=k + n)
-    if (k // 256 + bpw - 1) // bpw > 4:
-        pytest.skip("more than four K slices")
-    dx, dw = dev.put(x), dev.put(w)
-    dout = dev.empty(rows * n * 4)
-    G.gguf_q4_k_q8_1_fused_gemv_tile_tuned(dx.ptr, "f32", dw.ptr, dout.ptr, "f32", rows, k, n, blocks_per_wave=bpw)
-    got = dev.get(dout, np.float32, (rows, n))
-    dev.free(dx, dw, dout)
-    _check_f32(got, O.quantize_q8_1(x), w, O.GGML_Q4_K)
-
-
 @pytest.mark.parametrize("rows,k,n,rpw,kind", [(1, 5120, 300, 0, "f32"), (8, 5120, 1000, 68, "f32"),
                                                (4, 2048, 257, 33, "bf16"), (2, 4096, 96, 96, "fp16"),
                                                (5, 4352, 64, 7, "f32"), (8, 1024, 40, 0, "bf16"),
