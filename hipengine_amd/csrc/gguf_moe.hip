@@ -551,6 +551,63 @@ int launch_moe_mmq(const void* xq, const int64_t* compact_to_source, const int64
   return static_cast<int>(hipGetLastError());
 }
 
+
+// ---- router: top-k experts of a row of logits and the softmax of their logits --------
+//
+// One wave per token.  Lane l keeps the logits of experts l, l+64, ... (up to 16 of them,
+// so num_experts <= 1024) in registers.  top_k times: every lane's best remaining
+// (value, index), a butterfly maximum over the wave that prefers the lower index on
+// equal values, and the owner retires its entry.  The winners' logits sit in lanes
+// 0..top_k-1 at the end, where the softmax over them is taken
+// (max = the first winner, denominator floored at 1e-20: router.hip:628-715).
+constexpr int ROUTER_MAX_PER_LANE = 16;
+constexpr float ROUTER_LOWEST = -3.4028234663852886e38f;
+
+__global__ void __launch_bounds__(256) router_select_kernel(const float* __restrict__ logits,
+                                                            int64_t* __restrict__ selected,
+                                                            float* __restrict__ routing, int64_t tokens,
+                                                            int64_t logits_stride, int num_experts, int top_k) {
+  const int lane = threadIdx.x & 63;
+  const int64_t token = static_cast<int64_t>(blockIdx.x) * (blockDim.x >> 6) + (threadIdx.x >> 6);
+  if (token >= tokens) return;
+  const float* row = logits + token * logits_stride;
+  float vals[ROUTER_MAX_PER_LANE];
+#pragma unroll
+  for (int i = 0; i < ROUTER_MAX_PER_LANE; ++i) {
+    const int ex = lane + 64 * i;
+    vals[i] = ex < num_experts ? row[ex] : ROUTER_LOWEST;
+  }
+  float mine = 0.0f;    // lane p < top_k: logit of the p-th winner
+  for (int pos = 0; pos < top_k; ++pos) {
+    float best = ROUTER_LOWEST;
+    int best_i = -1;
+#pragma unroll
+    for (int i = 0; i < ROUTER_MAX_PER_LANE; ++i) {
+      const int ex = lane + 64 * i;
+      if (ex < num_experts && vals[i] > best) { best = vals[i]; best_i = ex; }   // strict: lowest index of equals
+    }
+    // (a retired expert holds ROUTER_LOWEST, which the strict comparison never picks)
+#pragma unroll
+    for (int off = 1; off < 64; off <<= 1) {
+      const float ov = __shfl_xor(best, off);
+      const int oi = __shfl_xor(best_i, off);
+      const bool take = oi >= 0 && (best_i < 0 || ov > best || (ov == best && oi < best_i));
+      best = take ? ov : best;
+      best_i = take ? oi : best_i;
+    }
+    if (lane == pos) mine = best;
+    if (lane == 0) selected[token * top_k + pos] = best_i;
+#pragma unroll
+    for (int i = 0; i < ROUTER_MAX_PER_LANE; ++i)
+      if (lane + 64 * i == best_i) vals[i] = ROUTER_LOWEST;
+  }
+  const float top = __shfl(mine, 0);
+  const float ev = lane < top_k ? expf(mine - top) : 0.0f;
+  float denom = 0.0f;
+  for (int p = 0; p < top_k; ++p) denom += __shfl(ev, p);   // in position order, as the reference sums
+  denom = fmaxf(denom, 1.0e-20f);
+  if (lane < top_k) routing[token * top_k + lane] = ev / denom;
+}
 }  // namespace
 
 // ---- routing index ------------------------------------------------------------
@@ -679,4 +736,20 @@ extern "C" int hipengine_gfx950_gguf_q4_k_grouped_mmq(const void* x_q8, const in
   return launch_moe_mmq(x_q8, compact_to_source, expert_start_compact, expert_start_mmq32, tile_expert, qweight_a,
                         qweight_b, out, out_kind, compact_rows, source_rows, in_features, out_features_a,
                         out_features_b, num_experts, mmq_total_rows, expert_stride_rows, stream);
+}
+
+extern "C" int hipengine_qwen35_router_select(const float* logits, int64_t* selected, float* routing, int64_t tokens,
+                                              int64_t logits_stride, int64_t num_experts, int64_t top_k,
+                                              int64_t threads, hipStream_t stream) {
+  if (!logits || !selected || !routing || tokens <= 0 || logits_stride <= 0 || num_experts <= 0 || top_k <= 0 ||
+      top_k > 16 || top_k > num_experts || num_experts > logits_stride ||
+      !(threads == 64 || threads == 128 || threads == 256 || threads == 512) ||
+      num_experts > 64 * ROUTER_MAX_PER_LANE) {
+    return static_cast<int>(hipErrorInvalidValue);
+  }
+  const int waves = 4;   // tokens per workgroup; `threads` is accepted and ignored
+  const unsigned grid = static_cast<unsigned>((tokens + waves - 1) / waves);
+  hipLaunchKernelGGL(router_select_kernel, dim3(grid), dim3(waves * 64), 0, stream, logits, selected, routing, tokens,
+                     logits_stride, static_cast<int>(num_experts), static_cast<int>(top_k));
+  return static_cast<int>(hipGetLastError());
 }

@@ -24,7 +24,7 @@ def register_backend_kernels(replace: bool = False) -> None:
     global _registered
     if _registered and not replace:
         return
-    from hipengine_amd.kernels.hip_gfx950.moe import group_scatter
+    from hipengine_amd.kernels.hip_gfx950.moe import group_scatter, router
     from hipengine_amd.kernels.hip_gfx950.quant import gguf_mmq_prefill, gguf_moe, gguf_q8_1_gemv, gguf_quantize
 
     gguf_quantize.register_kernels(BACKEND, replace=True)
@@ -32,4 +32,5 @@ def register_backend_kernels(replace: bool = False) -> None:
     gguf_mmq_prefill.register_kernels(BACKEND, replace=True)
     gguf_moe.register_kernels(BACKEND, replace=True)
     group_scatter.register_kernels(BACKEND, replace=True)
+    router.register_kernels(BACKEND, replace=True)
     _registered = True

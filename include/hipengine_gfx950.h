@@ -218,6 +218,17 @@ int hipengine_gfx950_gguf_q4_k_mmq_tuned(const void* xq, const uint8_t* qweight,
  * num_experts <= 2048.
  * ------------------------------------------------------------------------ */
 
+/* Router: for each of `tokens` rows of float32 logits (row pitch logits_stride), the top_k
+ * experts by logit, highest first (equal logits: lowest index), as int64 into
+ * selected[tokens*top_k], and the softmax over those top_k logits into
+ * routing[tokens*top_k].  top_k <= 16, num_experts <= 1024; `threads` in {64,128,256,512}
+ * is accepted and ignored.
+ * Replaces hipengine_qwen35_router_select (kernels/hip_gfx1100/moe/router.hip:1284-1311,
+ * device function :628-715). */
+int hipengine_qwen35_router_select(const float* logits, int64_t* selected, float* routing, int64_t tokens,
+                                   int64_t logits_stride, int64_t num_experts, int64_t top_k, int64_t threads,
+                                   hipengine_stream_t stream);
+
 /* selected_experts[total_lanes] -> expert-major order.  expert_start[num_experts+1]
  * (exclusive prefix of the per-expert lane counts), active_experts (ascending ids
  * of experts with at least one lane; may be NULL) and active_count[1] (may be NULL),

@@ -18,6 +18,7 @@ import pytest
 
 from oracle import gguf_oracle as O
 from hipengine_amd.kernels.hip_gfx950.moe import group_scatter as GS
+from hipengine_amd.kernels.hip_gfx950.moe import router as RT
 from hipengine_amd.kernels.hip_gfx950.quant import gguf_moe as M
 from hipengine_amd.kernels.hip_gfx950.quant import gguf_quantize as Q
 
@@ -76,6 +77,29 @@ def _device_index(dev, sel, w, num_experts, tile_capacity=0):
         host["l2c"] = dev.get(d["l2c"], np.int64, (lanes,))
     host["total"] = total
     return host, d
+
+
+@pytest.mark.parametrize("tokens,experts,top_k,stride", [(1, 256, 8, 256), (7, 256, 8, 257), (33, 60, 4, 64),
+                                                        (5, 1024, 16, 1024), (3, 8, 8, 8), (2048, 256, 8, 256)])
+def test_router_select(dev, tokens, experts, top_k, stride):
+    """Top-k experts bit-exact (order included, equal logits to the lowest index) and the softmax over the
+    selected logits within 2 ulp-ish of the oracle (expf differs between libm and the device)."""
+    rng = np.random.default_rng(17 + tokens + experts)
+    logits = rng.standard_normal((tokens, stride)).astype(np.float32)
+    logits[:, experts:] = 1.0e9                     # padding columns must not be read as experts
+    logits[0, : min(experts, 6)] = 0.75             # equal logits
+    if tokens > 1:
+        logits[1, :experts] = -2.5                  # a whole row of equal logits
+    dl = dev.put(logits)
+    dsel, dw = dev.empty(tokens * top_k * 8, fill=0xFF), dev.empty(tokens * top_k * 4, fill=0xFF)
+    RT.qwen35_router_select(dl.ptr, dsel.ptr, dw.ptr, tokens, stride, experts, top_k)
+    sel = dev.get(dsel, np.int64, (tokens, top_k))
+    w = dev.get(dw, np.float32, (tokens, top_k))
+    dev.free(dl, dsel, dw)
+    want_sel, want_w = O.router_topk_softmax(logits[:, :experts], top_k)
+    assert np.array_equal(sel, want_sel)
+    assert np.allclose(w, want_w, rtol=2e-6, atol=1e-9)
+    assert np.allclose(w.sum(axis=1), 1.0, atol=1e-6)
 
 
 @pytest.mark.parametrize("tokens,top_k,experts,bad", [(1, 8, 256, False), (8, 8, 256, True), (300, 4, 64, True),

@@ -101,7 +101,8 @@ def test_backend_registers_the_documented_keys(clean_registry):
                 KernelKey("hip_gfx950", "moe_linear", "gguf_q4_k",
                           "selected_dual_q8_1_ds4_mmq32_prefill_compact32_bf16_bf16_out"),
                 KernelKey("hip_gfx950", "moe_group_compact", "generic", "active_experts_source_rows"),
-                KernelKey("hip_gfx950", "moe_mmq_tile_map", "generic", "tile32")):
+                KernelKey("hip_gfx950", "moe_mmq_tile_map", "generic", "tile32"),
+                KernelKey("hip_gfx950", "router_select", "fp32")):
         assert key in keys
     assert not any(k.backend == "cpu_reference" for k in keys)            # the package ships no CPU path
     assert hip_gfx950.GGUF_CONSUMER_LAYERS >= {"linear", "moe_linear"}
@@ -210,6 +211,15 @@ def test_moe_wrappers_validate_before_touching_the_device():
         GS.qwen35_moe_group_compact_active_source_rows(1, 1, 1, 1, 1, 1, 1, 1, 8, 4096, 8)
     with pytest.raises(ValueError, match="tile_capacity"):
         GS.qwen35_moe_mmq32_tile_map(1, 1, 1, 1, 8, tile_capacity=-1)
+    from hipengine_amd.kernels.hip_gfx950.moe import router as RT
+    with pytest.raises(ValueError, match="top_k must be <= 16"):
+        RT.qwen35_router_select(1, 1, 1, 4, 256, 256, 17)
+    with pytest.raises(ValueError, match="top_k must be <= num_experts"):
+        RT.qwen35_router_select(1, 1, 1, 4, 256, 4, 8)
+    with pytest.raises(ValueError, match="num_experts must be <= logits_stride"):
+        RT.qwen35_router_select(1, 1, 1, 4, 128, 256, 8)
+    with pytest.raises(ValueError, match="threads"):
+        RT.qwen35_router_select(1, 1, 1, 4, 256, 256, 8, threads=100)
     with pytest.raises(ValueError, match="multiple of x_rows"):
         M.gguf_q4_k_selected_gemv_bf16_bf16_out(1, 1, 1, 1, 3, 8, 4, 256, 32)
     with pytest.raises(ValueError, match="divisible"):
