@@ -272,20 +272,21 @@ def main() -> None:
             extra[name] = {"us": round(c["event_s"] * 1e6, 2), "GB/s": round(c["bytes"] / c["event_s"] / 1e9, 1),
                            "frac_hbm": round(c["bytes"] / c["event_s"] / 1e9 / HBM_PEAK_GBS, 4), "copies": c["copies"]}
 
-        # One dense 27B-shape decoder layer at batch 1 (q, k, o, gate, up in Q4_K; v, down in Q6_K),
+        # One dense 27B-shape decoder layer at batch 1 and 8 (q, k, o, gate, up in Q4_K; v, down in Q6_K),
         # every matmul with its own rotating weights: bytes / sum of kernel times, and the
         # decode rate a 64-layer stack of these matmuls alone would allow.
         layer = (("q4_k", 5120, 5120), ("q4_k", 5120, 1024), ("q4_k", 5120, 5120), ("q4_k", 5120, 17408),
                  ("q4_k", 5120, 17408), ("q6_k", 5120, 1024), ("q6_k", 17408, 5120))
-        lbytes, lsec = 0, 0.0
-        for quant, kk, nn in layer:
-            c = h.gemv_case(quant, 1, kk, nn, steps, max(5, args.warmup // 5))
-            lbytes += c["bytes"]
-            lsec += c["event_s"]
-        extra["layer_sweep_27b_b1"] = {"bytes_per_layer": lbytes, "us_per_layer": round(lsec * 1e6, 1),
-                                       "GB/s": round(lbytes / lsec / 1e9, 1),
-                                       "frac_hbm": round(lbytes / lsec / 1e9 / HBM_PEAK_GBS, 4),
-                                       "tok_per_s_64_layers_matmuls_only": round(1.0 / (64 * lsec), 1)}
+        for batch in (1, 8):
+            lbytes, lsec = 0, 0.0
+            for quant, kk, nn in layer:
+                c = h.gemv_case(quant, batch, kk, nn, steps, max(5, args.warmup // 5))
+                lbytes += c["bytes"]
+                lsec += c["event_s"]
+            extra[f"layer_sweep_27b_b{batch}"] = {
+                "bytes_per_layer": lbytes, "us_per_layer": round(lsec * 1e6, 1),
+                "GB/s": round(lbytes / lsec / 1e9, 1), "frac_hbm": round(lbytes / lsec / 1e9 / HBM_PEAK_GBS, 4),
+                "tok_per_s_64_layers_matmuls_only": round(batch / (64 * lsec), 1)}
 
         msteps = max(5, args.steps // 50)
         for name, (quant, m, kk, nn) in {

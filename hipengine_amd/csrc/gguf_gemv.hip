@@ -273,6 +273,7 @@ struct StreamPlan {
 };
 
 constexpr int kComputeUnits = 256;   // MI355X
+constexpr size_t kMaxLds = 160 * 1024;   // LDS of one CU
 
 // The stream form applies to K >= 4096 (a 16-block load then spans at most two
 // rows), batch <= 2, when every resident wave gets at least a few loads.
@@ -297,7 +298,7 @@ StreamPlan default_stream_plan(int qt, int rows, int64_t K, int64_t N) {
     }
   }
   p.ok = rows <= 8 && nb >= 16 && total_loads >= 3 * static_cast<int64_t>(p.waves_total) &&
-         N >= p.waves_total && gemv_run_lds_bytes(qt, p.b, static_cast<int>(K)) <= 64 * 1024 &&
+         N >= p.waves_total && gemv_run_lds_bytes(qt, p.b, static_cast<int>(K)) <= kMaxLds &&
          find_stream_variant(qt, p.b, p.d) != nullptr;
   return p;
 }
@@ -313,14 +314,27 @@ int launch_gemv_stream(int qt, const void* x, int x_kind, const uint8_t* w, void
     return static_cast<int>(hipErrorInvalidValue);
   }
   const size_t lds = gemv_run_lds_bytes(qt, p.b, static_cast<int>(K));
-  if (lds > 64 * 1024) return static_cast<int>(hipErrorInvalidValue);
+  if (lds > kMaxLds) return static_cast<int>(hipErrorInvalidValue);
+  const StreamKernelFn fn = (x_kind >= KIND_F32 && x_kind <= KIND_Q8_1 && v->by_kind[x_kind]) ? v->by_kind[x_kind] : v->fn;
+  if (lds > 64 * 1024) {
+    // above the default dynamic limit: raise it for this kernel, once (no stream work)
+    static const void* raised[64];
+    static int n_raised = 0;
+    bool done = false;
+    for (int i = 0; i < n_raised; ++i) done = done || raised[i] == reinterpret_cast<const void*>(fn);
+    if (!done) {
+      const hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(fn),
+                                               hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(kMaxLds));
+      if (e != hipSuccess) return static_cast<int>(e);
+      if (n_raised < 64) raised[n_raised++] = reinterpret_cast<const void*>(fn);
+    }
+  }
   GemvStreamArgs a;
   a.x = x; a.w = w; a.out = out;
   a.x_kind = x_kind; a.out_kind = out_kind;
   a.rows = rows; a.K = static_cast<int>(K); a.N = static_cast<int>(N);
   a.waves = p.waves; a.waves_total = p.waves_total;
   a.base_rows = static_cast<int>(N / p.waves_total);
-  const StreamKernelFn fn = (x_kind >= KIND_F32 && x_kind <= KIND_Q8_1 && v->by_kind[x_kind]) ? v->by_kind[x_kind] : v->fn;
   hipLaunchKernelGGL(fn, dim3(p.waves_total / p.waves), dim3(p.waves * 64), lds, stream, a);
   return static_cast<int>(hipGetLastError());
 }
@@ -357,8 +371,15 @@ int launch_gemv(int qt, const void* x, int x_kind, const uint8_t* w, void* out, 
   }
   const int64_t x_row_bytes = x_kind == KIND_Q8_1 ? K / 32 * Q8_1_BYTES : K * (x_kind == KIND_F32 ? 4 : 2);
   const int64_t out_elem = out_kind == KIND_F32 ? 4 : 2;
-  for (int64_t r0 = 0; r0 < rows; r0 += 8) {
-    const int chunk = static_cast<int>(rows - r0 < 8 ? rows - r0 : 8);
+  for (int64_t r0 = 0; r0 < rows;) {
+    int chunk = static_cast<int>(rows - r0 < 8 ? rows - r0 : 8);
+    // a batch of 5..8 whose quantized activations do not fit the LDS of the stream form
+    // (Q6_K, K = 17408) goes as two batches of at most 4, which do
+    if (!forced && chunk > 4 && !default_slab_plan(qt, chunk, K, N).ok && !default_stream_plan(qt, chunk, K, N).ok &&
+        default_stream_plan(qt, 4, K, N).ok) {
+      chunk = 4;
+    }
+    const int64_t next_r0 = r0 + chunk;
     if (!forced) {
       // Q4_K, K <= 6144: the int8 MFMA slab form wins for batches of 3 and more, and at any
       // batch when a slab is a single 32-row step (N <= 8192); measured on MI355X
@@ -368,6 +389,7 @@ int launch_gemv(int qt, const void* x, int x_kind, const uint8_t* w, void* out, 
                                         static_cast<uint8_t*>(out) + r0 * N * out_elem, out_kind, chunk, K, N, sl,
                                         stream);
         if (rc != static_cast<int>(hipSuccess)) return rc;
+        r0 = next_r0;
         continue;
       }
       const StreamPlan sp = default_stream_plan(qt, chunk, K, N);
@@ -376,6 +398,7 @@ int launch_gemv(int qt, const void* x, int x_kind, const uint8_t* w, void* out, 
                                           static_cast<uint8_t*>(out) + r0 * N * out_elem, out_kind, chunk, K, N,
                                           sp, stream);
         if (rc != static_cast<int>(hipSuccess)) return rc;
+        r0 = next_r0;
         continue;
       }
       const RunPlan rp = default_run_plan(qt, chunk, K, N);
@@ -384,6 +407,7 @@ int launch_gemv(int qt, const void* x, int x_kind, const uint8_t* w, void* out, 
                                        static_cast<uint8_t*>(out) + r0 * N * out_elem, out_kind, chunk, K, N, rp,
                                        stream);
         if (rc != static_cast<int>(hipSuccess)) return rc;
+        r0 = next_r0;
         continue;
       }
     }
@@ -411,6 +435,7 @@ int launch_gemv(int qt, const void* x, int x_kind, const uint8_t* w, void* out, 
     hipLaunchKernelGGL(v->fn, dim3(grid), dim3(p.ks * p.nrg * 64), lds, stream, a);
     const hipError_t err = hipGetLastError();
     if (err != hipSuccess) return static_cast<int>(err);
+    r0 = next_r0;
   }
   return static_cast<int>(hipSuccess);
 }
