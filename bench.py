@@ -110,6 +110,46 @@ class Harness:
                 "weight_host": w, "x_host": x}
 
 
+    def ffn_case(self, rows: int, steps: int, warmup: int, seed: int = 7):
+        """Dense 27B FFN at decode: gate/up pair with SiLU fused (one launch) and the down projection with the
+        residual add fused (one launch), against the unfused sequence (3 GEMVs; its SiLU and add kernels are
+        not timed).  Returns (fused seconds, unfused GEMV seconds, weight bytes)."""
+        from hipengine_amd.kernels.hip_gfx950.quant import gguf_q8_1_gemv as G
+        from hipengine_amd.synthetic import synthetic_blocks
+
+        h_, f_ = 5120, 17408
+        wg, wd = synthetic_blocks(GGML["q4_k"], f_, h_, seed=seed), synthetic_blocks(GGML["q6_k"], h_, f_, seed=seed + 1)
+        copies = 4   # 2 x 50 MB + 73 MB per copy: 694 MB rotating
+        g = [self.memory.to_device(wg, runtime=self.rt) for _ in range(copies)]
+        u = [self.memory.to_device(wg, runtime=self.rt) for _ in range(copies)]
+        d = [self.memory.to_device(wd, runtime=self.rt) for _ in range(copies)]
+        rng = np.random.default_rng(seed)
+        dx = self.memory.to_device(rng.standard_normal((rows, h_)).astype(np.float32), runtime=self.rt)
+        dres = self.memory.to_device(rng.standard_normal((rows, h_)).astype(np.float32), runtime=self.rt)
+        dmid = self.memory.malloc(rows * f_ * 4, runtime=self.rt)
+        dmid2 = self.memory.malloc(rows * f_ * 4, runtime=self.rt)
+        dout = self.memory.malloc(rows * h_ * 4, runtime=self.rt)
+
+        def fused(i):
+            c = i % copies
+            G.gguf_pair_silu_gemv("gguf_q4_k", dx.ptr, "f32", g[c].ptr, u[c].ptr, dmid.ptr, "f32", rows, h_, f_,
+                                  round_mid=False)
+            G.gguf_gemv_residual("gguf_q6_k", dmid.ptr, "f32", d[c].ptr, dres.ptr, dout.ptr, "f32", rows, f_, h_)
+
+        q4, q6 = G.FUSED[("q4_k", "f32", "f32")], G.FUSED[("q6_k", "f32", "f32")]
+
+        def unfused(i):
+            c = i % copies
+            q4(dx.ptr, g[c].ptr, dmid.ptr, rows, h_, f_)
+            q4(dx.ptr, u[c].ptr, dmid2.ptr, rows, h_, f_)
+            q6(dmid.ptr, d[c].ptr, dout.ptr, rows, f_, h_)
+
+        _, ev_f = self.time_launches(fused, steps, warmup)
+        _, ev_u = self.time_launches(unfused, steps, warmup)
+        for buf in (*g, *u, *d, dx, dres, dmid, dmid2, dout):
+            self.memory.free(buf)
+        return ev_f, ev_u, 2 * wg.nbytes + wd.nbytes
+
     def mmq_case(self, quant: str, m: int, k: int, n: int, steps: int, warmup: int):
         """MMQ prefill GEMM on pre-packed activations: (seconds per launch, int8 ops per launch)."""
         from hipengine_amd.kernels.hip_gfx950.quant import gguf_mmq_prefill as M
@@ -287,6 +327,12 @@ def main() -> None:
                 "bytes_per_layer": lbytes, "us_per_layer": round(lsec * 1e6, 1),
                 "GB/s": round(lbytes / lsec / 1e9, 1), "frac_hbm": round(lbytes / lsec / 1e9 / HBM_PEAK_GBS, 4),
                 "tok_per_s_64_layers_matmuls_only": round(batch / (64 * lsec), 1)}
+
+        ev_f, ev_u, wbytes = h.ffn_case(1, steps, max(5, args.warmup // 5))
+        extra["ffn_27b_b1_fused_pair_silu_and_down_residual"] = {
+            "us": round(ev_f * 1e6, 1), "launches": 2, "GB/s": round(wbytes / ev_f / 1e9, 1),
+            "frac_hbm": round(wbytes / ev_f / 1e9 / HBM_PEAK_GBS, 4),
+            "unfused_3_gemv_us": round(ev_u * 1e6, 1)}
 
         msteps = max(5, args.steps // 50)
         for name, (quant, m, kk, nn) in {

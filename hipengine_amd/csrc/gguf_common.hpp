@@ -77,6 +77,13 @@ __device__ __forceinline__ float load_scalar(const void* x, int64_t idx, int kin
 
 // ---- wave64 cross-lane helpers (DPP; no LDS) -----------------------------
 
+// Round-trip through the output type (what a separate kernel reading the stored value would see).
+__device__ __forceinline__ float round_to_kind(float v, int kind) {
+  if (kind == KIND_BF16) return bf16_bits_to_float(float_to_bf16_bits(v));
+  if (kind == KIND_F16) return f16_bits_to_float(float_to_f16_bits(v));
+  return v;
+}
+
 template <int CTRL>
 __device__ __forceinline__ float dpp_f(float v) {
   return __builtin_bit_cast(float, __builtin_amdgcn_mov_dpp(__builtin_bit_cast(int, v), CTRL, 0xF, 0xF, true));

@@ -140,7 +140,7 @@ SlabPlan default_slab_plan(int qt, int rows, int64_t K, int64_t N) {
 }
 
 int launch_gemv_slab(const void* x, int x_kind, const uint8_t* w, void* out, int out_kind, int rows, int64_t K,
-                     int64_t N, const SlabPlan& p, hipStream_t stream) {
+                     int64_t N, const SlabPlan& p, hipStream_t stream, const void* residual = nullptr) {
   const int nb = static_cast<int>(K / QK_K);
   SlabVariant* v = nullptr;
   for (SlabVariant& c : kSlab)
@@ -157,7 +157,7 @@ int launch_gemv_slab(const void* x, int x_kind, const uint8_t* w, void* out, int
     if (e != hipSuccess) return static_cast<int>(e);
     v->lds_raised[x_kind] = true;
   }
-  GemvSlabArgs a{x, w, out, x_kind, out_kind, rows, static_cast<int>(K), static_cast<int>(N), p.rows_wg, p.waves};
+  GemvSlabArgs a{x, w, out, x_kind, out_kind, rows, static_cast<int>(K), static_cast<int>(N), p.rows_wg, p.waves, residual};
   const unsigned grid = static_cast<unsigned>((N + p.rows_wg - 1) / p.rows_wg);
   hipLaunchKernelGGL(v->by_kind[x_kind], dim3(grid), dim3(p.waves * 64), lds, stream, a);
   return static_cast<int>(hipGetLastError());
@@ -220,45 +220,53 @@ constexpr int stream_max_threads() {
   return B == 1 ? 768 : 512;
 }
 
-template <int QT, int B, int D, int S, int XK = -1>
+template <int QT, int B, int D, int S, int XK = -1, int FUSE = FUSE_NONE>
 __global__ void __launch_bounds__((stream_max_threads<B>())) gemv_stream_kernel(GemvStreamArgs a) {
   extern __shared__ __align__(16) uint8_t smem[];
-  gemv_stream_workgroup<QT, B, D, S, XK>(a, smem);
+  gemv_stream_workgroup<QT, B, D, S, XK, FUSE>(a, smem);
 }
 
 using StreamKernelFn = void (*)(GemvStreamArgs);
 
 // `long_k`: the instantiation that fetches five activation groups (of 8 values) per thread
 // up front (batch 1 only); the other fetches two (batch 1, 2) or one (batch 4, 8).
+// `fuse`: plain projection, gate/up pair with SiLU, or projection plus residual.
 struct StreamVariant {
   int qt, b, d;
   bool long_k;
+  int fuse;
   StreamKernelFn fn;
   StreamKernelFn by_kind[4];   // instantiations with the activation kind fixed (null: use fn)
 };
 
 #define STREAM_VARIANT(QT, B, D) \
-  StreamVariant { QT, B, D, false, gemv_stream_kernel<QT, B, D, (B <= 2 ? 2 : 1)>, {nullptr, nullptr, nullptr, nullptr} }
+  StreamVariant { QT, B, D, false, FUSE_NONE, gemv_stream_kernel<QT, B, D, (B <= 2 ? 2 : 1)>, {nullptr, nullptr, nullptr, nullptr} }
 #define STREAM_VARIANT_BY_KIND(QT, B, D, S, LONG_K)                                                      \
-  StreamVariant { QT, B, D, LONG_K, gemv_stream_kernel<QT, B, D, S>,                                      \
+  StreamVariant { QT, B, D, LONG_K, FUSE_NONE, gemv_stream_kernel<QT, B, D, S>,                           \
                   {gemv_stream_kernel<QT, B, D, S, KIND_F32>, gemv_stream_kernel<QT, B, D, S, KIND_BF16>, \
                    gemv_stream_kernel<QT, B, D, S, KIND_F16>, gemv_stream_kernel<QT, B, D, S, KIND_Q8_1>} }
+#define STREAM_VARIANT_FUSED(QT, B, S, LONG_K, FUSE) \
+  StreamVariant { QT, B, 3, LONG_K, FUSE, gemv_stream_kernel<QT, B, 3, S, -1, FUSE>, {nullptr, nullptr, nullptr, nullptr} }
 
 const StreamVariant kStream[] = {
-    STREAM_VARIANT_BY_KIND(GGML_Q4_K, 1, 3, 2, false), STREAM_VARIANT(GGML_Q4_K, 1, 5), STREAM_VARIANT(GGML_Q4_K, 2, 3),
-    STREAM_VARIANT(GGML_Q4_K, 2, 5), STREAM_VARIANT_BY_KIND(GGML_Q6_K, 1, 3, 2, false), STREAM_VARIANT(GGML_Q6_K, 1, 5),
-    STREAM_VARIANT(GGML_Q6_K, 2, 3), STREAM_VARIANT(GGML_Q6_K, 2, 5), STREAM_VARIANT_BY_KIND(GGML_Q8_0, 1, 3, 2, false),
-    STREAM_VARIANT(GGML_Q8_0, 1, 5), STREAM_VARIANT(GGML_Q8_0, 2, 3), STREAM_VARIANT(GGML_Q8_0, 2, 5),
+    STREAM_VARIANT_BY_KIND(GGML_Q4_K, 1, 3, 2, false), STREAM_VARIANT(GGML_Q4_K, 2, 3),
+    STREAM_VARIANT_BY_KIND(GGML_Q6_K, 1, 3, 2, false), STREAM_VARIANT(GGML_Q6_K, 2, 3),
+    STREAM_VARIANT_BY_KIND(GGML_Q8_0, 1, 3, 2, false), STREAM_VARIANT(GGML_Q8_0, 2, 3),
     STREAM_VARIANT_BY_KIND(GGML_Q4_K, 1, 3, 5, true), STREAM_VARIANT_BY_KIND(GGML_Q6_K, 1, 3, 5, true),
     STREAM_VARIANT_BY_KIND(GGML_Q8_0, 1, 3, 5, true),
     STREAM_VARIANT(GGML_Q4_K, 4, 3), STREAM_VARIANT(GGML_Q4_K, 8, 3), STREAM_VARIANT(GGML_Q6_K, 4, 3),
     STREAM_VARIANT(GGML_Q6_K, 8, 3), STREAM_VARIANT(GGML_Q8_0, 4, 3), STREAM_VARIANT(GGML_Q8_0, 8, 3),
+    // gate/up pair with SiLU (Q4_K) and projection + residual (Q4_K, Q6_K), batch 1 and 2
+    STREAM_VARIANT_FUSED(GGML_Q4_K, 1, 2, false, FUSE_PAIR), STREAM_VARIANT_FUSED(GGML_Q4_K, 2, 2, false, FUSE_PAIR),
+    STREAM_VARIANT_FUSED(GGML_Q4_K, 1, 2, false, FUSE_RESIDUAL), STREAM_VARIANT_FUSED(GGML_Q4_K, 2, 2, false, FUSE_RESIDUAL),
+    STREAM_VARIANT_FUSED(GGML_Q6_K, 1, 2, false, FUSE_RESIDUAL), STREAM_VARIANT_FUSED(GGML_Q6_K, 2, 2, false, FUSE_RESIDUAL),
+    STREAM_VARIANT_FUSED(GGML_Q4_K, 1, 5, true, FUSE_RESIDUAL), STREAM_VARIANT_FUSED(GGML_Q6_K, 1, 5, true, FUSE_RESIDUAL),
 };
 
-const StreamVariant* find_stream_variant(int qt, int b, int d, bool long_k = false) {
+const StreamVariant* find_stream_variant(int qt, int b, int d, bool long_k = false, int fuse = FUSE_NONE) {
   const StreamVariant* fallback = nullptr;
   for (const StreamVariant& v : kStream) {
-    if (v.qt != qt || v.b != b || v.d != d) continue;
+    if (v.qt != qt || v.b != b || v.d != d || v.fuse != fuse) continue;
     if (v.long_k == long_k) return &v;
     if (!v.long_k) fallback = &v;
   }
@@ -303,17 +311,31 @@ StreamPlan default_stream_plan(int qt, int rows, int64_t K, int64_t N) {
   return p;
 }
 
+struct StreamFusion {
+  int fuse = FUSE_NONE;
+  const uint8_t* w_up = nullptr;
+  const void* residual = nullptr;
+  int round_mid = 0;
+};
+
 int launch_gemv_stream(int qt, const void* x, int x_kind, const uint8_t* w, void* out, int out_kind, int rows,
-                       int64_t K, int64_t N, const StreamPlan& p, hipStream_t stream) {
+                       int64_t K, int64_t N, const StreamPlan& p, hipStream_t stream,
+                       const StreamFusion& fusion = StreamFusion()) {
   const int nb = static_cast<int>(K / QK_K);
   // more than two activation groups per thread (16 teams of 4 lanes per wave): take the
   // instantiation that fetches five up front
-  const StreamVariant* v = find_stream_variant(qt, p.b, p.d, p.waves > 0 && nb > 4 * p.waves);
+  const StreamVariant* v = find_stream_variant(qt, p.b, p.d, p.waves > 0 && nb > 4 * p.waves, fusion.fuse);
   if (!v || nb < 16 || rows > p.b || p.waves < 1 || p.waves > (p.b == 1 ? 12 : 8) || p.waves_total < p.waves ||
       (p.waves_total % p.waves) != 0 || p.waves_total > N) {
     return static_cast<int>(hipErrorInvalidValue);
   }
-  const size_t lds = gemv_run_lds_bytes(qt, p.b, static_cast<int>(K));
+  size_t lds = gemv_run_lds_bytes(qt, p.b, static_cast<int>(K));
+  if (fusion.fuse == FUSE_PAIR) {
+    // gate results wait per wave; a wave may hold at most STREAM_PAIR_MAX_ROWS rows
+    if (!fusion.w_up || (N + p.waves_total - 1) / p.waves_total > STREAM_PAIR_MAX_ROWS) return static_cast<int>(hipErrorInvalidValue);
+    lds += static_cast<size_t>(p.waves) * p.b * STREAM_PAIR_MAX_ROWS * sizeof(float);
+  }
+  if (fusion.fuse == FUSE_RESIDUAL && !fusion.residual) return static_cast<int>(hipErrorInvalidValue);
   if (lds > kMaxLds) return static_cast<int>(hipErrorInvalidValue);
   const StreamKernelFn fn = (x_kind >= KIND_F32 && x_kind <= KIND_Q8_1 && v->by_kind[x_kind]) ? v->by_kind[x_kind] : v->fn;
   if (lds > 64 * 1024) {
@@ -335,6 +357,7 @@ int launch_gemv_stream(int qt, const void* x, int x_kind, const uint8_t* w, void
   a.rows = rows; a.K = static_cast<int>(K); a.N = static_cast<int>(N);
   a.waves = p.waves; a.waves_total = p.waves_total;
   a.base_rows = static_cast<int>(N / p.waves_total);
+  a.w_up = fusion.w_up; a.residual = fusion.residual; a.round_mid = fusion.round_mid;
   hipLaunchKernelGGL(fn, dim3(p.waves_total / p.waves), dim3(p.waves * 64), lds, stream, a);
   return static_cast<int>(hipGetLastError());
 }
@@ -561,4 +584,46 @@ extern "C" int hipengine_gfx950_gguf_q4_k_q8_1_fused_gemv_slab_tuned(const void*
   if (rows_per_workgroup > 0) p.rows_wg = rows_per_workgroup;
   return launch_gemv_slab(x, x_kind, qweight, out, out_kind, static_cast<int>(rows), in_features, out_features, p,
                           stream);
+}
+
+// ---- fused epilogues: gate/up pair with SiLU, projection + residual -------------------
+
+extern "C" int hipengine_gfx950_gguf_pair_silu_gemv(int32_t ggml_type, const void* x, int32_t x_kind,
+                                                    const uint8_t* qweight_gate, const uint8_t* qweight_up, void* out,
+                                                    int32_t out_kind, int64_t rows, int64_t in_features,
+                                                    int64_t out_features, int32_t round_mid, hipStream_t stream) {
+  if (!x || !qweight_gate || !qweight_up || !out || x_kind < KIND_F32 || x_kind > KIND_Q8_1 || out_kind < KIND_F32 ||
+      out_kind > KIND_F16 || rows <= 0 || rows > 2 || in_features <= 0 || (in_features % QK_K) != 0 ||
+      out_features <= 0) {
+    return static_cast<int>(hipErrorInvalidValue);
+  }
+  const StreamPlan sp = default_stream_plan(ggml_type, static_cast<int>(rows), in_features, out_features);
+  if (!sp.ok) return static_cast<int>(hipErrorInvalidValue);
+  StreamFusion f;
+  f.fuse = FUSE_PAIR; f.w_up = qweight_up; f.round_mid = round_mid;
+  return launch_gemv_stream(ggml_type, x, x_kind, qweight_gate, out, out_kind, static_cast<int>(rows), in_features,
+                            out_features, sp, stream, f);
+}
+
+extern "C" int hipengine_gfx950_gguf_gemv_residual(int32_t ggml_type, const void* x, int32_t x_kind,
+                                                   const uint8_t* qweight, const void* residual, void* out,
+                                                   int32_t out_kind, int64_t rows, int64_t in_features,
+                                                   int64_t out_features, hipStream_t stream) {
+  if (!x || !qweight || !residual || !out || x_kind < KIND_F32 || x_kind > KIND_Q8_1 || out_kind < KIND_F32 ||
+      out_kind > KIND_F16 || rows <= 0 || rows > 8 || in_features <= 0 || (in_features % QK_K) != 0 ||
+      out_features <= 0) {
+    return static_cast<int>(hipErrorInvalidValue);
+  }
+  const SlabPlan sl = default_slab_plan(ggml_type, static_cast<int>(rows), in_features, out_features);
+  if (sl.ok && (rows >= 3 || sl.rows_wg <= 32)) {
+    return launch_gemv_slab(x, x_kind, qweight, out, out_kind, static_cast<int>(rows), in_features, out_features, sl,
+                            stream, residual);
+  }
+  if (rows > 2) return static_cast<int>(hipErrorInvalidValue);
+  const StreamPlan sp = default_stream_plan(ggml_type, static_cast<int>(rows), in_features, out_features);
+  if (!sp.ok) return static_cast<int>(hipErrorInvalidValue);
+  StreamFusion f;
+  f.fuse = FUSE_RESIDUAL; f.residual = residual;
+  return launch_gemv_stream(ggml_type, x, x_kind, qweight, out, out_kind, static_cast<int>(rows), in_features,
+                            out_features, sp, stream, f);
 }

@@ -58,6 +58,7 @@ struct GemvSlabArgs {
   int N;
   int rows_wg;   // output rows per workgroup, 1..96
   int waves;     // waves per workgroup = ceil(nb / BPW)
+  const void* residual;   // null, or [rows, N] of the output type: out = round(projection) + residual
 };
 
 constexpr int SLAB_MAX_ROWS = 96;
@@ -326,7 +327,9 @@ __device__ __forceinline__ void gemv_slab_q4k_workgroup(const GemvSlabArgs& a, u
     float v = 0.0f;
     for (int s = 0; s < a.waves; ++s)
       v += reinterpret_cast<const float*>(smem + s * WAVE_BYTES)[m * SLAB_MAX_ROWS + rl];
-    store_scalar(a.out, static_cast<int64_t>(m) * a.N + r0 + rl, v, a.out_kind);
+    const int64_t oi = static_cast<int64_t>(m) * a.N + r0 + rl;
+    if (a.residual) v = round_to_kind(v, a.out_kind) + load_scalar(a.residual, oi, a.out_kind);
+    store_scalar(a.out, oi, v, a.out_kind);
   }
 }
 

@@ -38,13 +38,27 @@ struct GemvStreamArgs {
   int waves;        // waves per workgroup
   int waves_total;  // waves in the whole grid (grid * waves)
   int base_rows;    // N / waves_total (computed on the host: an integer division is ~40 instructions here)
+  const uint8_t* w_up;      // FUSE_PAIR: the second matrix (w is the gate); out = silu(gate.x) * (up.x)
+  const void* residual;     // FUSE_RESIDUAL: [rows, N] of the output type, added to the projection
+  int round_mid;            // FUSE_PAIR: round gate and up to the output type before the SiLU
 };
+
+enum StreamFuse { FUSE_NONE = 0, FUSE_PAIR = 1, FUSE_RESIDUAL = 2 };
+constexpr int STREAM_PAIR_MAX_ROWS = 16;   // rows per wave the pair form can hold back (gate results wait for up)
 
 // XK >= 0 fixes the activation kind at compile time (the staging code of the other
 // kinds is then not generated: a decode kernel runs its prologue once per launch
 // with a cold instruction cache, so prologue code size is launch latency), XK < 0
 // reads it from the arguments.
-template <int QT, int B, int D, int S, int XK = -1>
+//
+// FUSE selects the epilogue:
+//   FUSE_PAIR      the wave walks its rows of the gate matrix and then the same rows of the up
+//                  matrix as one run of 2*nrows rows; gate results wait in LDS (written and read
+//                  by lane 63 only) and the stored value is silu(gate) * up, with gate and up
+//                  rounded to the output type first when round_mid is set
+//                  (gguf_q4_k_gemv.hip:652-657);
+//   FUSE_RESIDUAL  out = round(projection) + residual in the output type (gguf_q4_k_gemv.hip:1669-1678).
+template <int QT, int B, int D, int S, int XK = -1, int FUSE = FUSE_NONE>
 __device__ __forceinline__ void gemv_stream_workgroup(const GemvStreamArgs& a, uint8_t* smem) {
   using Regs = WeightRegs<GemvTraits<QT>::REGS>;
   constexpr int Q8S = run_q8_stride<QT>();
@@ -58,13 +72,17 @@ __device__ __forceinline__ void gemv_stream_workgroup(const GemvStreamArgs& a, u
   const int base_rows = a.base_rows, extra = a.N - a.base_rows * a.waves_total;
   const int r0 = gw * base_rows + min(gw, extra);
   const int nrows = base_rows + (gw < extra ? 1 : 0);
-  const int run_blocks = nrows * nb;
+  const int mat_blocks = nrows * nb;                                   // blocks of this wave in one matrix
+  const int run_blocks = FUSE == FUSE_PAIR ? 2 * mat_blocks : mat_blocks;
   const int nloads = (run_blocks + 15) >> 4;
   const uint8_t* wbase = a.w + static_cast<int64_t>(r0) * nb * SUPER;
+  const uint8_t* wbase_up = FUSE == FUSE_PAIR ? a.w_up + static_cast<int64_t>(r0) * nb * SUPER : nullptr;
 
   uint8_t* q8 = smem;
   float* rec = reinterpret_cast<float*>(q8 + B * nb * Q8S);
   int* s16 = reinterpret_cast<int*>(rec + B * nb * 16);
+  // pair form: gate results of this wave, [B][STREAM_PAIR_MAX_ROWS], behind the activation image
+  float* gate_hold = reinterpret_cast<float*>(s16 + (QT == GGML_Q6_K ? B * nb * 16 : 0)) + wave * B * STREAM_PAIR_MAX_ROWS;
 
   // Activation loads go first (see gemv_run_stage_fetch), then the weight ring.
   // S activation groups per thread have their loads issued ahead of the weight ring,
@@ -81,7 +99,12 @@ __device__ __forceinline__ void gemv_stream_workgroup(const GemvStreamArgs& a, u
   const int last_blk = max(run_blocks - 1, 0);
   auto issue = [&](int i, Regs& dst) {
     const int blk = min(i * 16 + j, last_blk);
-    gemv_load_block<QT>(wbase + static_cast<int64_t>(blk) * SUPER, q, dst);
+    if constexpr (FUSE == FUSE_PAIR) {
+      const bool up = blk >= mat_blocks;
+      gemv_load_block<QT>((up ? wbase_up : wbase) + static_cast<int64_t>(up ? blk - mat_blocks : blk) * SUPER, q, dst);
+    } else {
+      gemv_load_block<QT>(wbase + static_cast<int64_t>(blk) * SUPER, q, dst);
+    }
   };
 #pragma unroll
   for (int c = 0; c < D; ++c) issue(c, ring[c]);
@@ -89,6 +112,7 @@ __device__ __forceinline__ void gemv_stream_workgroup(const GemvStreamArgs& a, u
   gemv_run_stage_commit<QT, B, S>(ra, sr, q8, rec, s16);
   __syncthreads();
 
+  const int total_rows = FUSE == FUSE_PAIR ? 2 * nrows : nrows;
   float acc_cur[B], acc_next[B];
 #pragma unroll
   for (int b = 0; b < B; ++b) { acc_cur[b] = 0.0f; acc_next[b] = 0.0f; }
@@ -102,9 +126,24 @@ __device__ __forceinline__ void gemv_stream_workgroup(const GemvStreamArgs& a, u
   auto flush = [&](int row_rel) {
 #pragma unroll
     for (int b = 0; b < B; ++b) {
-      const float v = wave_sum_to_lane63(acc_cur[b]);
-      if (lane == 63 && b < a.rows)
-        store_scalar(a.out, static_cast<int64_t>(b) * a.N + r0 + row_rel, v, a.out_kind);
+      float v = wave_sum_to_lane63(acc_cur[b]);
+      if (lane == 63 && b < a.rows) {
+        if constexpr (FUSE == FUSE_PAIR) {
+          if (row_rel < nrows) {
+            gate_hold[b * STREAM_PAIR_MAX_ROWS + row_rel] = v;
+          } else {
+            float gate = gate_hold[b * STREAM_PAIR_MAX_ROWS + row_rel - nrows];
+            if (a.round_mid) { gate = round_to_kind(gate, a.out_kind); v = round_to_kind(v, a.out_kind); }
+            const float sig = 1.0f / (1.0f + expf(-gate));
+            store_scalar(a.out, static_cast<int64_t>(b) * a.N + r0 + row_rel - nrows, gate * sig * v, a.out_kind);
+          }
+        } else if constexpr (FUSE == FUSE_RESIDUAL) {
+          const int64_t idx = static_cast<int64_t>(b) * a.N + r0 + row_rel;
+          store_scalar(a.out, idx, round_to_kind(v, a.out_kind) + load_scalar(a.residual, idx, a.out_kind), a.out_kind);
+        } else {
+          store_scalar(a.out, static_cast<int64_t>(b) * a.N + r0 + row_rel, v, a.out_kind);
+        }
+      }
       acc_cur[b] = acc_next[b];
       acc_next[b] = 0.0f;
     }
@@ -133,12 +172,12 @@ __device__ __forceinline__ void gemv_stream_workgroup(const GemvStreamArgs& a, u
       int new_lo = row_lo + step_r;
       if (pos_lo >= nb) { pos_lo -= nb; new_lo += 1; }
       if (new_lo > row_lo) {
-        if (row_lo < nrows) flush(row_lo);
+        if (row_lo < total_rows) flush(row_lo);
         row_lo = new_lo;
       }
     }
   }
-  if (row_lo < nrows) flush(row_lo);
+  if (row_lo < total_rows) flush(row_lo);
 }
 
 }  // namespace hipengine_gfx950

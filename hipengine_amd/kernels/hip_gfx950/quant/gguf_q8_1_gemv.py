@@ -131,6 +131,81 @@ def gguf_q8_1_fused_gemv_stream_tuned(quant_key: str, x_ptr: int, x_kind: str, q
                     in_features, out_features, loads_in_flight, waves, waves_total, stream), runtime)
 
 
+class FusedFormUnavailable(ValueError):
+    """The shape is outside the fused kernel's range; run the unfused sequence instead (hipEngine's
+    ``launch_gguf_linear_pair_silu`` / ``launch_gguf_linear_residual`` return False in that case:
+    ``runtime/qwen35_gguf_layer_ffn.py:519-538,619-630``)."""
+
+
+def gguf_pair_silu_gemv(quant_key: str, x_ptr: int, x_kind: str, qweight_gate_ptr: int, qweight_up_ptr: int,
+                        out_ptr: int, out_kind: str, rows: int, in_features: int, out_features: int, *,
+                        round_mid: bool = True, stream: int = 0, library: ctypes.CDLL | None = None,
+                        runtime: HipRuntime | None = None) -> None:
+    """Dense FFN gate/up pair in one pass with SiLU*up fused: ``out = silu(gate x) * (up x)``.
+    ``round_mid`` rounds gate and up to the output type first, as the unfused GEMV, GEMV, silu_mul sequence
+    does through its stored intermediates.  Raises :class:`FusedFormUnavailable` outside Q4_K / rows <= 2 /
+    stream-form shapes."""
+    validate_linear(rows, in_features, out_features)
+    validate_pointers(x_ptr=x_ptr, qweight_gate_ptr=qweight_gate_ptr, qweight_up_ptr=qweight_up_ptr, out_ptr=out_ptr)
+    if quant_key != "gguf_q4_k" or rows > 2 or in_features < 4096:
+        raise FusedFormUnavailable("pair_silu: Q4_K, rows <= 2, in_features >= 4096 only")
+    fn = entry("hipengine_gfx950_gguf_pair_silu_gemv",
+               [I32, VOID, I32, VOID, VOID, VOID, I32, I64, I64, I64, I32, VOID], library)
+    code = fn(QUANT_KEY_TO_GGML[quant_key], x_ptr, _KINDS[x_kind], qweight_gate_ptr, qweight_up_ptr, out_ptr,
+              _KINDS[out_kind], rows, in_features, out_features, int(bool(round_mid)), stream)
+    if code == 1:
+        raise FusedFormUnavailable("pair_silu: out_features too small for the fused kernel")
+    check_launch(code, runtime)
+
+
+def gguf_gemv_residual(quant_key: str, x_ptr: int, x_kind: str, qweight_ptr: int, residual_ptr: int, out_ptr: int,
+                       out_kind: str, rows: int, in_features: int, out_features: int, *, stream: int = 0,
+                       library: ctypes.CDLL | None = None, runtime: HipRuntime | None = None) -> None:
+    """Projection with the residual add fused: ``out = round(W x) + residual`` in the output type
+    (``residual_ptr`` may equal ``out_ptr``).  Raises :class:`FusedFormUnavailable` outside the fused range."""
+    validate_linear(rows, in_features, out_features)
+    validate_pointers(x_ptr=x_ptr, qweight_ptr=qweight_ptr, residual_ptr=residual_ptr, out_ptr=out_ptr)
+    if quant_key not in ("gguf_q4_k", "gguf_q6_k") or rows > 8:
+        raise FusedFormUnavailable("gemv_residual: Q4_K / Q6_K, rows <= 8 only")
+    fn = entry("hipengine_gfx950_gguf_gemv_residual",
+               [I32, VOID, I32, VOID, VOID, VOID, I32, I64, I64, I64, VOID], library)
+    code = fn(QUANT_KEY_TO_GGML[quant_key], x_ptr, _KINDS[x_kind], qweight_ptr, residual_ptr, out_ptr,
+              _KINDS[out_kind], rows, in_features, out_features, stream)
+    if code == 1:
+        raise FusedFormUnavailable("gemv_residual: shape outside the fused kernels' range")
+    check_launch(code, runtime)
+
+
+def _make_pair_silu(act: str, out: str):
+    def wrapper(x_ptr: int, qweight_gate_ptr: int, qweight_up_ptr: int, out_ptr: int, rows: int, in_features: int,
+                out_features: int, *, stream: int = 0, library: ctypes.CDLL | None = None,
+                runtime: HipRuntime | None = None) -> None:
+        gguf_pair_silu_gemv("gguf_q4_k", x_ptr, act, qweight_gate_ptr, qweight_up_ptr, out_ptr, out, rows, in_features,
+                            out_features, round_mid=True, stream=stream, library=library, runtime=runtime)
+
+    wrapper.__name__ = f"gguf_q4_k_dual_silu_gemv_{act}_{out}_out"
+    wrapper.__doc__ = f"Q4_K gate/up pair with SiLU fused, {act} activations, {out} output (dual+SiLU operand order)."
+    return wrapper
+
+
+def _make_residual(quant: str, act: str, out: str):
+    def wrapper(x_ptr: int, qweight_ptr: int, residual_ptr: int, out_ptr: int, rows: int, in_features: int,
+                out_features: int, *, stream: int = 0, library: ctypes.CDLL | None = None,
+                runtime: HipRuntime | None = None) -> None:
+        gguf_gemv_residual(f"gguf_{quant}", x_ptr, act, qweight_ptr, residual_ptr, out_ptr, out, rows, in_features,
+                           out_features, stream=stream, library=library, runtime=runtime)
+
+    wrapper.__name__ = f"gguf_{quant}_gemv_{act}_residual_{out}_out"
+    wrapper.__doc__ = (f"{quant.upper()} projection + residual, {act} activations, {out} residual and output "
+                       "(operand order of hipEngine's pack8_gemv_bf16_residual_bf16_out).")
+    return wrapper
+
+
+PAIR_SILU = {(act, out): _make_pair_silu(act, out) for act, out in (("bf16", "bf16"), ("f32", "f32"))}
+RESIDUAL = {(quant, act, out): _make_residual(quant, act, out)
+            for quant in ("q4_k", "q6_k") for act, out in (("bf16", "bf16"), ("f32", "f32"))}
+
+
 def gguf_q4_k_q8_1_fused_gemv_slab_tuned(x_ptr: int, x_kind: str, qweight_ptr: int, out_ptr: int, out_kind: str,
                                          rows: int, in_features: int, out_features: int, *,
                                          rows_per_workgroup: int = 0, stream: int = 0,
@@ -155,6 +230,10 @@ def gguf_gemv_default_plan(quant_key: str, rows: int, in_features: int, out_feat
 
 
 def register_kernels(backend: str = "hip_gfx950", *, replace: bool = False) -> None:
+    for (act, out), fn in PAIR_SILU.items():
+        register(KernelKey(backend, "linear", "gguf_q4_k", f"dual_silu_gemv_{act}_{out}_out"), fn, replace=replace)
+    for (quant, act, out), fn in RESIDUAL.items():
+        register(KernelKey(backend, "linear", f"gguf_{quant}", f"gemv_{act}_residual_{out}_out"), fn, replace=replace)
     for (quant, act, out), fn in FUSED.items():
         for prefix in ("q8_1_fused_gemv", "q8_1_fused_prefill"):
             register(KernelKey(backend, "linear", f"gguf_{quant}", f"{prefix}_{act}_{out}_out"), fn, replace=replace)

@@ -144,13 +144,36 @@ int hipengine_gfx950_gguf_q8_1_fused_gemv_run_tuned(int32_t ggml_type, const voi
 
 /* The same for the "stream" form (waves_total resident waves, `waves` per
  * workgroup, each owning a contiguous range of rows and keeping loads_in_flight
- * 16-block loads in flight).  rows <= 2, in_features >= 4096,
+ * 16-block loads in flight; the library builds loads_in_flight = 3 only, deeper
+ * rings measured slower).  rows <= 8, in_features >= 4096,
  * waves_total <= out_features.  New here. */
 int hipengine_gfx950_gguf_q8_1_fused_gemv_stream_tuned(int32_t ggml_type, const void* x, int32_t x_kind,
                                                        const uint8_t* qweight, void* out, int32_t out_kind,
                                                        int64_t rows, int64_t in_features, int64_t out_features,
                                                        int32_t loads_in_flight, int32_t waves, int32_t waves_total,
                                                        hipengine_stream_t stream);
+
+/* Gate/up pair of a dense FFN with SiLU*up fused: out[r, n] = silu(gate_n . x_r) * (up_n . x_r), one pass
+ * over both matrices, q8_1 quantization of x fused.  round_mid != 0 rounds gate and up to the output type
+ * before the SiLU, which reproduces the unfused sequence GEMV, GEMV, silu_mul on stored values
+ * (arithmetic of gguf_q4_k_gemv.hip:652-657; hipEngine fuses this for its pack8 layout only,
+ * hipengine_gguf_q4_k_pack8_dual_silu_gemv_bf16_bf16_out, and launch_gguf_linear_pair_silu
+ * (runtime/qwen35_gguf_layer_ffn.py:519-538) falls back to the unfused sequence when no fused kernel
+ * applies; so must a caller here when this returns 1).  Q4_K, rows <= 2, in_features >= 4096 and
+ * out_features large enough for the stream form (a 27B FFN is).  New here. */
+int hipengine_gfx950_gguf_pair_silu_gemv(int32_t ggml_type, const void* x, int32_t x_kind, const uint8_t* qweight_gate,
+                                         const uint8_t* qweight_up, void* out, int32_t out_kind, int64_t rows,
+                                         int64_t in_features, int64_t out_features, int32_t round_mid,
+                                         hipengine_stream_t stream);
+
+/* Projection with the residual add fused: out = round_to_out_type(W x) + residual, residual [rows, N] of the
+ * output type (may be the same buffer as out) - the epilogue of
+ * hipengine_gguf_q4_k_pack8_gemv_bf16_residual_bf16_out (gguf_q4_k_gemv.hip:1669-1678, :3080-3110) on the raw
+ * layout.  Q4_K in the slab form's range (any rows <= 8), Q4_K / Q6_K in the stream form's range (rows <= 2);
+ * returns 1 otherwise, and the caller runs the GEMV and the add separately.  New here. */
+int hipengine_gfx950_gguf_gemv_residual(int32_t ggml_type, const void* x, int32_t x_kind, const uint8_t* qweight,
+                                        const void* residual, void* out, int32_t out_kind, int64_t rows,
+                                        int64_t in_features, int64_t out_features, hipengine_stream_t stream);
 
 /* The "slab" form for Q4_K: one workgroup per CU owns rows_per_workgroup (<= 96;
  * 0 = ceil(out_features / 256)) consecutive output rows, its waves split K in

@@ -222,10 +222,10 @@ def test_slab_form_q4_k(dev, rows, k, n, rpw, kind):
     _check_f32(got, O.quantize_q8_1(x), w, O.GGML_Q4_K)
 
 
-@pytest.mark.parametrize("quant,d,waves,waves_total", [("gguf_q4_k", 3, 4, 64), ("gguf_q4_k", 5, 10, 120),
-                                                      ("gguf_q6_k", 3, 12, 96), ("gguf_q8_0", 5, 8, 64)])
+@pytest.mark.parametrize("quant,d,waves,waves_total", [("gguf_q4_k", 3, 4, 64), ("gguf_q4_k", 3, 10, 120),
+                                                      ("gguf_q6_k", 3, 12, 96), ("gguf_q8_0", 3, 8, 64)])
 def test_stream_form_explicit_layouts(dev, quant, d, waves, waves_total):
-    """Stream form with explicit ring depth and wave counts (up to 12 waves per workgroup at batch 1)."""
+    """Stream form with explicit wave counts (up to 12 waves per workgroup at batch 1); the ring depth built is 3."""
     rng = np.random.default_rng(5 + waves_total)
     rows, k, n = 1, 5120, 256
     x = rng.standard_normal((rows, k)).astype(np.float32)
@@ -268,3 +268,68 @@ def test_c_abi_rejects_bad_arguments(dev):
         G.FUSED[("q4_k", "f32", "f32")](1, 1, 1, 1, 100, 8)
     with pytest.raises(ValueError, match="threads"):
         G.FUSED[("q4_k", "f32", "f32")](1, 1, 1, 1, 256, 8, threads=96)
+
+
+@pytest.mark.parametrize("rows,kind,round_mid", [(1, "bf16", True), (2, "bf16", True), (1, "f32", False)])
+def test_pair_silu_gemv(dev, rows, kind, round_mid):
+    """Gate/up pair with SiLU fused (stream form, both matrices in one pass) against the unfused composition of
+    the oracle's GEMV and SiLU*up on the same q8_1 activations; bf16 intermediates rounded as the unfused
+    sequence stores them."""
+    k, n = 4096, 4096
+    rng = np.random.default_rng(5 + rows)
+    x = rng.standard_normal((rows, k)).astype(np.float32)
+    if kind == "bf16":
+        x = O.bf16_bits_to_f32(O.f32_to_bf16_bits(x))
+    wg = O.random_weight(O.GGML_Q4_K, n, k, seed=11)
+    wu = O.random_weight(O.GGML_Q4_K, n, k, seed=12)
+    xin = x if kind == "f32" else O.f32_to_bf16_bits(x)
+    dx, dg, du = dev.put(xin), dev.put(wg), dev.put(wu)
+    esz = 4 if kind == "f32" else 2
+    dout = dev.empty(rows * n * esz)
+    G.gguf_pair_silu_gemv("gguf_q4_k", dx.ptr, kind, dg.ptr, du.ptr, dout.ptr, kind, rows, k, n, round_mid=round_mid)
+    got = dev.get(dout, np.float32 if kind == "f32" else np.uint16, (rows, n))
+    dev.free(dx, dg, du, dout)
+    xdq = O.dequantize_q8_1(O.quantize_q8_1(x))
+    gate = O.gguf_quant_gemv(xdq, wg, O.GGML_Q4_K)
+    up = O.gguf_quant_gemv(xdq, wu, O.GGML_Q4_K)
+    if round_mid and kind == "bf16":
+        gate = O.bf16_bits_to_f32(O.f32_to_bf16_bits(gate))
+        up = O.bf16_bits_to_f32(O.f32_to_bf16_bits(up))
+    want = (O.silu(gate) * up).astype(np.float32)
+    if kind == "bf16":
+        got = O.bf16_bits_to_f32(got)
+        # one bf16 ulp of slack on top of the float32 gate: a gate or up value within float32 noise of a bf16
+        # rounding boundary may round the other way
+        assert O.cosine(got, want) >= 0.9999
+        assert np.max(np.abs(got - want)) <= 2.0 ** -6 * max(1.0, float(np.max(np.abs(want))))
+    else:
+        assert O.max_rel_err(got, want) <= 1e-3 and O.cosine(got, want) >= 0.99999
+
+
+@pytest.mark.parametrize("quant,rows,k,n,kind", [("gguf_q6_k", 1, 17408, 5120, "bf16"), ("gguf_q4_k", 2, 4096, 4096, "bf16"),
+                                                 ("gguf_q4_k", 5, 5120, 1000, "bf16"), ("gguf_q4_k", 1, 5120, 17408, "f32")])
+def test_gemv_residual(dev, quant, rows, k, n, kind):
+    """Projection + residual fused (stream and slab forms): out = round(W x) + residual in the output type,
+    bit for bit from the unfused kernel's own output."""
+    rng = np.random.default_rng(31 + rows + n)
+    x = rng.standard_normal((rows, k)).astype(np.float32)
+    res = rng.standard_normal((rows, n)).astype(np.float32)
+    w = O.random_weight(QT[quant], n, k, seed=n)
+    if kind == "bf16":
+        xin, rin, esz = O.f32_to_bf16_bits(x), O.f32_to_bf16_bits(res), 2
+    else:
+        xin, rin, esz = x, res, 4
+    dx, dw, dr = dev.put(xin), dev.put(w), dev.put(rin)
+    dplain, dout = dev.empty(rows * n * esz), dev.empty(rows * n * esz)
+    G.FUSED[(quant[5:], kind, kind)](dx.ptr, dw.ptr, dplain.ptr, rows, k, n)
+    G.gguf_gemv_residual(quant, dx.ptr, kind, dw.ptr, dr.ptr, dout.ptr, kind, rows, k, n)
+    if kind == "bf16":
+        plain = O.bf16_bits_to_f32(dev.get(dplain, np.uint16, (rows, n)))
+        got = dev.get(dout, np.uint16, (rows, n))
+        want = O.f32_to_bf16_bits(plain + O.bf16_bits_to_f32(rin))
+        assert np.array_equal(got, want)
+    else:
+        plain = dev.get(dplain, np.float32, (rows, n))
+        got = dev.get(dout, np.float32, (rows, n))
+        assert np.array_equal(got.view(np.uint32), (plain + res).astype(np.float32).view(np.uint32))
+    dev.free(dx, dw, dr, dplain, dout)
