@@ -24,6 +24,7 @@ using half_t = _Float16;
 
 constexpr int QK_K = 256;
 constexpr int Q4_K_BYTES = 144;
+constexpr int Q5_K_BYTES = 176;
 constexpr int Q6_K_BYTES = 210;
 constexpr int Q8_0_BYTES = 34;
 constexpr int Q8_1_BYTES = 36;
@@ -33,6 +34,7 @@ constexpr int D4S4_BYTES = 160;
 // GGML type ids (hipengine/quant/gguf.py:23-57)
 constexpr int GGML_Q8_0 = 8;
 constexpr int GGML_Q4_K = 12;
+constexpr int GGML_Q5_K = 13;
 constexpr int GGML_Q6_K = 14;
 
 // Element types at the C boundary.

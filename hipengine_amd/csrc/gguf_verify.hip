@@ -4,6 +4,7 @@
 // (gguf_common.hpp unpack, gemv_load_block / gemv_block_dots).
 
 #include "gguf_gemv.hpp"
+#include "gguf_dequant.hpp"
 
 #include "../../include/hipengine_gfx950.h"
 
@@ -11,74 +12,16 @@ namespace {
 
 using namespace hipengine_gfx950;
 
-__device__ __forceinline__ float byte_f(uint32_t w, int i) { return static_cast<float>((w >> (8 * i)) & 0xFFu); }
-
-// One thread per qs dword: 32 threads per Q4_K block.
-__global__ void __launch_bounds__(256) dequant_q4_k_kernel(const uint8_t* __restrict__ blocks, float* __restrict__ out,
-                                                           int64_t n_blocks) {
+// One unit of a block per thread (gguf_dequant.hpp).
+template <int QT>
+__global__ void __launch_bounds__(256) dequant_kernel(const uint8_t* __restrict__ blocks, float* __restrict__ out,
+                                                      int64_t n_blocks) {
+  using T = DequantTraits<QT>;
   const int64_t t = static_cast<int64_t>(blockIdx.x) * 256 + threadIdx.x;
-  const int64_t b = t >> 5;
+  const int64_t b = t / T::UNITS;
   if (b >= n_blocks) return;
-  const int i = static_cast<int>(t & 31);
-  const uint8_t* blk = blocks + b * Q4_K_BYTES;
-  const uint4 h = load16(blk);
-  const uint32_t qs = load4(blk + 16 + 4 * i);
-  const Q4KScales s = q4k_unpack_scales(h.y, h.z, h.w);
-  const float d = f16_bits_to_float(h.x & 0xFFFFu), dmin = f16_bits_to_float(h.x >> 16);
-  const int pair = i >> 3, lane0 = (i & 7) * 4;
-  const float sa = d * static_cast<float>(q4k_scale_of(s, 2 * pair));
-  const float sb = d * static_cast<float>(q4k_scale_of(s, 2 * pair + 1));
-  const float ma = dmin * static_cast<float>(q4k_min_of(s, 2 * pair));
-  const float mb = dmin * static_cast<float>(q4k_min_of(s, 2 * pair + 1));
-  const uint32_t lo = q4k_low(qs), hi = q4k_high(qs);
-  float* o = out + b * QK_K;
-#pragma unroll
-  for (int j = 0; j < 4; ++j) {
-    o[(2 * pair) * 32 + lane0 + j] = sa * byte_f(lo, j) - ma;
-    o[(2 * pair + 1) * 32 + lane0 + j] = sb * byte_f(hi, j) - mb;
-  }
-}
-
-// One thread per (half, lane dword): 16 threads per Q6_K block.
-__global__ void __launch_bounds__(256) dequant_q6_k_kernel(const uint8_t* __restrict__ blocks, float* __restrict__ out,
-                                                           int64_t n_blocks) {
-  const int64_t t = static_cast<int64_t>(blockIdx.x) * 256 + threadIdx.x;
-  const int64_t b = t >> 4;
-  if (b >= n_blocks) return;
-  const int h = static_cast<int>(t >> 3) & 1, i = static_cast<int>(t & 7);
-  const uint8_t* blk = blocks + b * Q6_K_BYTES;
-  const Q6KQuad u = q6k_unpack(load4(blk + 64 * h + 4 * i), load4(blk + 64 * h + 32 + 4 * i),
-                               load4(blk + 128 + 32 * h + 4 * i));
-  const uint32_t g[4] = {q6k_center(u.g0), q6k_center(u.g1), q6k_center(u.g2), q6k_center(u.g3)};
-  const float d = f16_bits_to_float(load2(blk + 208));
-  const int8_t* sc = reinterpret_cast<const int8_t*>(blk + 192);
-  float* o = out + b * QK_K;
-#pragma unroll
-  for (int j = 0; j < 4; ++j) {
-    const int grp = 4 * h + j;
-    const float step = d * static_cast<float>(sc[grp * 2 + (i >> 2)]);
-#pragma unroll
-    for (int e = 0; e < 4; ++e) {
-      const int q = static_cast<int8_t>((g[j] >> (8 * e)) & 0xFFu);
-      o[grp * 32 + 4 * i + e] = step * static_cast<float>(q);
-    }
-  }
-}
-
-// One thread per quant dword: 8 threads per Q8_0 block.
-__global__ void __launch_bounds__(256) dequant_q8_0_kernel(const uint8_t* __restrict__ blocks, float* __restrict__ out,
-                                                           int64_t n_blocks) {
-  const int64_t t = static_cast<int64_t>(blockIdx.x) * 256 + threadIdx.x;
-  const int64_t b = t >> 3;
-  if (b >= n_blocks) return;
-  const int i = static_cast<int>(t & 7);
-  const uint8_t* blk = blocks + b * Q8_0_BYTES;
-  const float d = f16_bits_to_float(load2(blk));
-  const uint32_t w = (load2(blk + 2 + 4 * i)) | (load2(blk + 4 + 4 * i) << 16);
-#pragma unroll
-  for (int e = 0; e < 4; ++e) {
-    out[b * 32 + 4 * i + e] = static_cast<float>(static_cast<int8_t>((w >> (8 * e)) & 0xFFu)) * d;
-  }
+  float* o = out + b * T::VALUES;
+  dequant_unit<QT>(blocks + b * T::BYTES, static_cast<int>(t - b * T::UNITS), [=](int k, float v) { o[k] = v; });
 }
 
 // One wave per (16 weight rows, one 256-value K block); grid (ceil(N/16), K/256, rows).
@@ -145,14 +88,16 @@ extern "C" int hipengine_gfx950_copy_bytes(const void* src, void* dst, int64_t b
 extern "C" int hipengine_gfx950_gguf_dequantize_f32(int32_t ggml_type, const uint8_t* blocks, float* out,
                                                     int64_t n_blocks, hipStream_t stream) {
   if (!blocks || !out || n_blocks <= 0) return static_cast<int>(hipErrorInvalidValue);
-  const int per_block = ggml_type == GGML_Q4_K ? 32 : ggml_type == GGML_Q6_K ? 16 : ggml_type == GGML_Q8_0 ? 8 : 0;
+  const int per_block = ggml_type == GGML_Q4_K || ggml_type == GGML_Q5_K ? 32
+                        : ggml_type == GGML_Q6_K ? 16 : ggml_type == GGML_Q8_0 ? 8 : 0;
   if (!per_block) return static_cast<int>(hipErrorInvalidValue);
   const int64_t grid = (n_blocks * per_block + 255) / 256;
   if (grid > 0x7FFFFFFF) return static_cast<int>(hipErrorInvalidValue);
   const dim3 g(static_cast<unsigned>(grid)), b(256);
-  if (ggml_type == GGML_Q4_K) hipLaunchKernelGGL(dequant_q4_k_kernel, g, b, 0, stream, blocks, out, n_blocks);
-  else if (ggml_type == GGML_Q6_K) hipLaunchKernelGGL(dequant_q6_k_kernel, g, b, 0, stream, blocks, out, n_blocks);
-  else hipLaunchKernelGGL(dequant_q8_0_kernel, g, b, 0, stream, blocks, out, n_blocks);
+  if (ggml_type == GGML_Q4_K) hipLaunchKernelGGL(dequant_kernel<GGML_Q4_K>, g, b, 0, stream, blocks, out, n_blocks);
+  else if (ggml_type == GGML_Q5_K) hipLaunchKernelGGL(dequant_kernel<GGML_Q5_K>, g, b, 0, stream, blocks, out, n_blocks);
+  else if (ggml_type == GGML_Q6_K) hipLaunchKernelGGL(dequant_kernel<GGML_Q6_K>, g, b, 0, stream, blocks, out, n_blocks);
+  else hipLaunchKernelGGL(dequant_kernel<GGML_Q8_0>, g, b, 0, stream, blocks, out, n_blocks);
   return static_cast<int>(hipGetLastError());
 }
 

@@ -14,7 +14,7 @@ BACKEND = "hip_gfx950"
 TARGET_ARCH = "gfx950"
 WAVEFRONT_SIZE = 64
 
-GGUF_CONSUMER_LAYERS: frozenset[str] = frozenset({"linear", "moe_linear", "activation_quant"})
+GGUF_CONSUMER_LAYERS: frozenset[str] = frozenset({"linear", "moe_linear", "activation_quant", "embedding"})
 
 _registered = False
 
@@ -25,7 +25,13 @@ def register_backend_kernels(replace: bool = False) -> None:
     if _registered and not replace:
         return
     from hipengine_amd.kernels.hip_gfx950.moe import group_scatter, router
-    from hipengine_amd.kernels.hip_gfx950.quant import gguf_mmq_prefill, gguf_moe, gguf_q8_1_gemv, gguf_quantize
+    from hipengine_amd.kernels.hip_gfx950.quant import (
+        gguf_embedding,
+        gguf_mmq_prefill,
+        gguf_moe,
+        gguf_q8_1_gemv,
+        gguf_quantize,
+    )
 
     gguf_quantize.register_kernels(BACKEND, replace=True)
     gguf_q8_1_gemv.register_kernels(BACKEND, replace=True)
@@ -33,4 +39,5 @@ def register_backend_kernels(replace: bool = False) -> None:
     gguf_moe.register_kernels(BACKEND, replace=True)
     group_scatter.register_kernels(BACKEND, replace=True)
     router.register_kernels(BACKEND, replace=True)
+    gguf_embedding.register_kernels(BACKEND, replace=True)
     _registered = True

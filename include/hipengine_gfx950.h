@@ -241,6 +241,24 @@ int hipengine_gfx950_gguf_q4_k_mmq_tuned(const void* xq, const uint8_t* qweight,
  * num_experts <= 2048.
  * ------------------------------------------------------------------------ */
 
+/* Token embedding lookup over raw GGUF rows: out[r, 0..hidden_size) = bf16(dequantize(row token_ids[r] of
+ * qweight)), qweight [vocab_size, hidden_size / block * block_bytes].  A row whose token id is outside
+ * [0, vocab_size) is left untouched.  hidden_size % 256 == 0 (Q8_0: % 32); `threads` is accepted and ignored.
+ * Replace hipengine_gguf_{q4_k,q5_k,q6_k,q8_0}_embedding_bf16_out
+ * (kernels/hip_gfx1100/quant/gguf_q6_k_embedding.hip:240-350). */
+int hipengine_gguf_q4_k_embedding_bf16_out(const int64_t* token_ids, const uint8_t* qweight, uint16_t* out,
+                                           int64_t rows, int64_t hidden_size, int64_t vocab_size, int64_t threads,
+                                           hipengine_stream_t stream);
+int hipengine_gguf_q5_k_embedding_bf16_out(const int64_t* token_ids, const uint8_t* qweight, uint16_t* out,
+                                           int64_t rows, int64_t hidden_size, int64_t vocab_size, int64_t threads,
+                                           hipengine_stream_t stream);
+int hipengine_gguf_q6_k_embedding_bf16_out(const int64_t* token_ids, const uint8_t* qweight, uint16_t* out,
+                                           int64_t rows, int64_t hidden_size, int64_t vocab_size, int64_t threads,
+                                           hipengine_stream_t stream);
+int hipengine_gguf_q8_0_embedding_bf16_out(const int64_t* token_ids, const uint8_t* qweight, uint16_t* out,
+                                           int64_t rows, int64_t hidden_size, int64_t vocab_size, int64_t threads,
+                                           hipengine_stream_t stream);
+
 /* Router: for each of `tokens` rows of float32 logits (row pitch logits_stride), the top_k
  * experts by logit, highest first (equal logits: lowest index), as int64 into
  * selected[tokens*top_k], and the softmax over those top_k logits into

@@ -33,6 +33,9 @@ moe_selected_ffn             committed golden of the reference
                              moe_ffn_selected_gguf_q4_k.json, copied as data
                              to tests/golden/); independent dense recompute
 moe_ffn_block                same golden file (``expected_block``)
+embedding_lookup             definition: dequantize(qweight[ids]); error cases of the reference
+dequant_q5_k                 block builder inverse (reference generator restated),
+                             scalar per-element loop, qh = 0 equals Q4_K
 quantize_q8_1                float64 brute force, invariants (|q|<=127,
                              q[argmax]=+-127, zero block), tie cases built
                              from exact binary fractions
@@ -72,11 +75,13 @@ FP16_MAX = np.float32(65504.0)
 
 GGML_Q8_0 = 8
 GGML_Q4_K = 12
+GGML_Q5_K = 13
 GGML_Q6_K = 14
 
 _BLOCK_GEOMETRY = {
     GGML_Q8_0: (32, Q8_0_BLOCK_BYTES),
     GGML_Q4_K: (QK_K, Q4_K_BLOCK_BYTES),
+    GGML_Q5_K: (QK_K, Q5_K_BLOCK_BYTES),
     GGML_Q6_K: (QK_K, Q6_K_BLOCK_BYTES),
 }
 
@@ -175,6 +180,35 @@ def dequant_q4_k(blocks: np.ndarray) -> np.ndarray:
     return (scale * q - offset).reshape(-1, QK_K)
 
 
+def q5_k_quants(blocks: np.ndarray) -> np.ndarray:
+    """[n,176] block bytes -> unsigned 5-bit values [n,8,32] in element order.
+
+    ``{half d; half dmin; u8 scales[12]; u8 qh[32]; u8 qs[128]}``: the low four bits as in
+    Q4_K (byte ``j`` of 32-byte group ``g`` of ``qs``: element ``64g+j`` low nibble,
+    ``64g+32+j`` high nibble); bit 4 of the value of sub-block ``s``, lane ``l`` is bit
+    ``s`` of ``qh[l]`` (gguf.py:646-662, gguf_q6_k_embedding.hip q5_k_weight)."""
+    n = blocks.shape[0]
+    qs = blocks[:, 48:176].reshape(n, 4, 32)
+    qh = blocks[:, 16:48]
+    out = np.empty((n, 8, 32), dtype=np.uint8)
+    out[:, 0::2] = qs & 0x0F
+    out[:, 1::2] = qs >> 4
+    for sb in range(8):
+        out[:, sb] |= ((qh >> sb) & 1) << 4
+    return out
+
+
+def dequant_q5_k(blocks: np.ndarray) -> np.ndarray:
+    """``(d*sc)*q - (dmin*mn)`` in float32 with 5-bit ``q`` (gguf.py:646-662)."""
+    d = _fp16_field(blocks, 0)
+    dmin = _fp16_field(blocks, 2)
+    sc, mn = q4_k_scale_min(blocks[:, 4:16])
+    scale = (d[:, None] * sc.astype(np.float32))[:, :, None]
+    offset = (dmin[:, None] * mn.astype(np.float32))[:, :, None]
+    q = q5_k_quants(blocks).astype(np.float32)
+    return (scale * q - offset).reshape(-1, QK_K)
+
+
 def q6_k_quants(blocks: np.ndarray) -> np.ndarray:
     """[n,210] block bytes -> signed 6-bit values [n,8,32] (already ``-32``).
 
@@ -211,7 +245,7 @@ def dequant_q8_0(blocks: np.ndarray) -> np.ndarray:
     return q * d[:, None]
 
 
-_DEQUANT = {GGML_Q8_0: dequant_q8_0, GGML_Q4_K: dequant_q4_k, GGML_Q6_K: dequant_q6_k}
+_DEQUANT = {GGML_Q8_0: dequant_q8_0, GGML_Q4_K: dequant_q4_k, GGML_Q5_K: dequant_q5_k, GGML_Q6_K: dequant_q6_k}
 
 
 def dequantize(data, qtype: int) -> np.ndarray:
@@ -254,6 +288,20 @@ def gguf_quant_gemv_chunked(x, qweight, qtype: int, chunk_rows: int = 8192) -> n
         hi = min(qw.shape[0], lo + chunk_rows)
         out[:, lo:hi] = gguf_quant_gemv(xa, qw[lo:hi], qtype)
     return out
+
+
+def embedding_lookup(token_ids, qweight, qtype: int) -> np.ndarray:
+    """Rows ``token_ids`` of a quantized table, dequantized to float32
+    (``_gguf_k_embedding``, kernels/cpu_reference/ops.py:511-524)."""
+    ids = np.asarray(token_ids, dtype=np.int64)
+    qw = np.asarray(qweight)
+    if ids.ndim != 1:
+        raise ValueError("token_ids must have shape [rows]")
+    if qw.ndim != 2:
+        raise ValueError("qweight must have GGUF byte shape [vocab_size, bytes_per_row]")
+    if np.any(ids < 0) or np.any(ids >= qw.shape[0]):
+        raise ValueError("token_ids contain out-of-range token IDs")
+    return dequantize(qw[ids], qtype).astype(np.float32)
 
 
 def silu(v: np.ndarray) -> np.ndarray:
@@ -691,6 +739,42 @@ def closed_form_q4_k(out_features: int, in_features: int) -> np.ndarray:
     blk[..., 4:16] = pack_q4_k_scale_min(sc.reshape(-1, 8), mn.reshape(-1, 8)).reshape(out_features, nb, 12)
     blk[..., 16:] = (q[..., 0, :] | (q[..., 1, :] << 4)).reshape(out_features, nb, 128)
     return blk.reshape(out_features, nb * Q4_K_BLOCK_BYTES)
+
+
+def pack_q5_k_blocks(q5: np.ndarray, sc: np.ndarray, mn: np.ndarray, d: np.ndarray, dmin: np.ndarray) -> np.ndarray:
+    """Inverse of :func:`q5_k_quants` + header: ``q5`` [n,8,32] in 0..31, ``sc``/``mn`` [n,8] 6-bit,
+    ``d``/``dmin`` [n] -> [n,176] block bytes (builder of tests/_gguf_synthetic_weights.py:81-108)."""
+    q5 = np.asarray(q5, dtype=np.uint8)
+    n = q5.shape[0]
+    blk = np.empty((n, Q5_K_BLOCK_BYTES), dtype=np.uint8)
+    blk[:, 0:2] = _f16_bytes(d)
+    blk[:, 2:4] = _f16_bytes(dmin)
+    blk[:, 4:16] = pack_q4_k_scale_min(sc, mn)
+    qh = np.zeros((n, 32), dtype=np.uint8)
+    for sb in range(8):
+        qh |= ((q5[:, sb] >> 4) & 1) << sb
+    blk[:, 16:48] = qh
+    lo = q5 & 0x0F
+    blk[:, 48:176] = (lo[:, 0::2] | (lo[:, 1::2] << 4)).reshape(n, 128)
+    return blk
+
+
+def closed_form_q5_k(out_features: int, in_features: int) -> np.ndarray:
+    """Closed-form Q5_K weight of the reference tests, vectorized.  Block (o, b): ``d``, ``dmin``,
+    ``sc_j``, ``mn_j`` as in :func:`closed_form_q4_k`, ``q_k = (k+13o+17b)%32``
+    (tests/_gguf_synthetic_weights.py:81-121)."""
+    if in_features % QK_K:
+        raise ValueError("in_features must be a multiple of 256")
+    nb = in_features // QK_K
+    o = np.repeat(np.arange(out_features, dtype=np.int64), nb)
+    b = np.tile(np.arange(nb, dtype=np.int64), out_features)
+    j = np.arange(8, dtype=np.int64)
+    k = np.arange(QK_K, dtype=np.int64)
+    sc = ((3 * j + (o + b)[:, None]) % 63 + 1).astype(np.uint8)
+    mn = ((5 * j + (2 * o + b)[:, None]) % 17).astype(np.uint8)
+    q = ((k + (13 * o + 17 * b)[:, None]) % 32).astype(np.uint8).reshape(-1, 8, 32)
+    blk = pack_q5_k_blocks(q, sc, mn, 0.015625 * (1 + o % 5), 0.0078125 * (1 + b % 3))
+    return blk.reshape(out_features, nb * Q5_K_BLOCK_BYTES)
 
 
 def pack_q6_k_blocks(q_signed: np.ndarray, scales_i8: np.ndarray, d: np.ndarray) -> np.ndarray:

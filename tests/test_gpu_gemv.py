@@ -56,11 +56,23 @@ def _run_fused(dev, quant, x, w, act="f32", out="f32"):
     return res
 
 
-@pytest.mark.parametrize("quant", ["gguf_q4_k", "gguf_q6_k", "gguf_q8_0"])
+def _random_q5_k(n, k, seed):
+    rng = np.random.default_rng(seed)
+    nblk = n * (k // 256)
+    blk = O.pack_q5_k_blocks(rng.integers(0, 32, size=(nblk, 8, 32), dtype=np.uint8),
+                             rng.integers(0, 64, size=(nblk, 8), dtype=np.uint8),
+                             rng.integers(0, 64, size=(nblk, 8), dtype=np.uint8),
+                             (rng.random(nblk) * 0.05).astype(np.float32), (rng.random(nblk) * 0.02).astype(np.float32))
+    return blk.reshape(n, -1)
+
+
+@pytest.mark.parametrize("quant", ["gguf_q4_k", "gguf_q5_k", "gguf_q6_k", "gguf_q8_0"])
 def test_dequantize_bit_exact(dev, quant):
-    qt = QT[quant]
-    for w in (CLOSED[quant](37, 768), O.random_weight(qt, 64, 1024, seed=11)):
-        block, nbytes = {8: (32, 34), 12: (256, 144), 14: (256, 210)}[qt]
+    qt = {"gguf_q5_k": O.GGML_Q5_K, **QT}[quant]
+    cases = ((O.closed_form_q5_k(37, 768), _random_q5_k(64, 1024, 11)) if quant == "gguf_q5_k"
+             else (CLOSED[quant](37, 768), O.random_weight(qt, 64, 1024, seed=11)))
+    for w in cases:
+        block, nbytes = {8: (32, 34), 12: (256, 144), 13: (256, 176), 14: (256, 210)}[qt]
         n_blocks = w.size // nbytes
         dw = dev.put(w)
         dout = dev.empty(n_blocks * block * 4)
@@ -69,6 +81,25 @@ def test_dequantize_bit_exact(dev, quant):
         dev.free(dw, dout)
         want = O.dequantize(w, qt)
         assert np.array_equal(got.view(np.uint32), want.view(np.uint32))
+
+
+@pytest.mark.parametrize("quant", ["gguf_q4_k", "gguf_q5_k", "gguf_q6_k", "gguf_q8_0"])
+def test_embedding_lookup_bit_exact(dev, quant):
+    """bf16(dequantize(row token)) bit for bit; rows with an out-of-range token id stay untouched."""
+    from hipengine_amd.kernels.hip_gfx950.quant import gguf_embedding as E
+    qt = {"gguf_q5_k": O.GGML_Q5_K, **QT}[quant]
+    vocab, hidden = 301, 1280
+    w = _random_q5_k(vocab, hidden, 3) if quant == "gguf_q5_k" else O.random_weight(qt, vocab, hidden, seed=4)
+    ids = np.array([0, 300, 17, 17, -1, 301, 128, 5], dtype=np.int64)
+    did, dw = dev.put(ids), dev.put(w)
+    dout = dev.empty(ids.size * hidden * 2, fill=0xAB)
+    E.EMBEDDING[quant](did.ptr, dw.ptr, dout.ptr, ids.size, hidden, vocab)
+    got = dev.get(dout, np.uint16, (ids.size, hidden))
+    dev.free(did, dw, dout)
+    ok = (ids >= 0) & (ids < vocab)
+    want = O.f32_to_bf16_bits(O.embedding_lookup(ids[ok], w, qt))
+    assert np.array_equal(got[ok], want)
+    assert np.all(got[~ok] == 0xABAB)
 
 
 @pytest.mark.parametrize("kind", ["f32", "bf16"])

@@ -102,7 +102,11 @@ def test_backend_registers_the_documented_keys(clean_registry):
                           "selected_dual_q8_1_ds4_mmq32_prefill_compact32_bf16_bf16_out"),
                 KernelKey("hip_gfx950", "moe_group_compact", "generic", "active_experts_source_rows"),
                 KernelKey("hip_gfx950", "moe_mmq_tile_map", "generic", "tile32"),
-                KernelKey("hip_gfx950", "router_select", "fp32")):
+                KernelKey("hip_gfx950", "router_select", "fp32"),
+                KernelKey("hip_gfx950", "embedding", "gguf_q5_k", "lookup_bf16_out"),
+                KernelKey("hip_gfx950", "embedding", "gguf_q6_k", "lookup_bf16_out"),
+                KernelKey("hip_gfx950", "linear", "gguf_q4_k", "dual_silu_gemv_bf16_bf16_out"),
+                KernelKey("hip_gfx950", "linear", "gguf_q6_k", "gemv_bf16_residual_bf16_out")):
         assert key in keys
     assert not any(k.backend == "cpu_reference" for k in keys)            # the package ships no CPU path
     assert hip_gfx950.GGUF_CONSUMER_LAYERS >= {"linear", "moe_linear"}

@@ -419,3 +419,65 @@ def test_routing_index_invariants():
     assert tm["total"] == int(((counts + 31) // 32 * 32).sum())
     for tile, ex in enumerate(tm["tile_expert"]):
         assert tm["tile_expert_start"][ex] <= tile * 32 < tm["tile_expert_start"][ex + 1]
+
+
+def test_q5_k_dequant_against_the_block_builder_a_scalar_loop_and_q4_k():
+    """Q5_K: (i) values packed by the reference's block builder come back exactly, and the closed-form
+    generator equals its element formula d*sc*q - dmin*mn; (ii) a per-element scalar loop that follows
+    the device lookup formula (qs nibble | bit sb of qh[lane] << 4) agrees; (iii) with qh = 0 a Q5_K block
+    dequantizes like the Q4_K block with the same header and nibbles."""
+    rng = np.random.default_rng(55)
+    n = 6
+    q5 = rng.integers(0, 32, size=(n, 8, 32), dtype=np.uint8)
+    sc = rng.integers(0, 64, size=(n, 8), dtype=np.uint8)
+    mn = rng.integers(0, 64, size=(n, 8), dtype=np.uint8)
+    d = rng.random(n).astype(np.float16).astype(np.float32) * 0.05
+    dmin = rng.random(n).astype(np.float16).astype(np.float32) * 0.02
+    blk = O.pack_q5_k_blocks(q5, sc, mn, d, dmin)
+    assert blk.shape == (n, 176)
+    assert np.array_equal(O.q5_k_quants(blk), q5)
+    d16, m16 = d.astype(np.float16).astype(np.float32), dmin.astype(np.float16).astype(np.float32)
+    want = ((d16[:, None] * sc.astype(np.float32))[:, :, None] * q5.astype(np.float32)
+            - (m16[:, None] * mn.astype(np.float32))[:, :, None]).reshape(n, 256)
+    got = O.dequant_q5_k(blk)
+    assert np.array_equal(got.view(np.uint32), want.astype(np.float32).view(np.uint32))
+    # (ii) scalar loop over one block
+    b0 = blk[0]
+    scales = b0[4:16]
+    def sc_of(s):
+        return (scales[s] & 63) if s < 4 else ((scales[8 + s - 4] & 0x0F) | ((scales[s - 4] >> 2) & 0x30))
+    def mn_of(s):
+        return (scales[4 + s] & 63) if s < 4 else ((scales[8 + s - 4] >> 4) | ((scales[4 + s - 4] >> 2) & 0x30))
+    for k in range(256):
+        s, lane = k >> 5, k & 31
+        packed = b0[48 + (s >> 1) * 32 + lane]
+        ql = (packed >> 4) if (s & 1) else (packed & 0x0F)
+        q = int(ql) | (((int(b0[16 + lane]) >> s) & 1) << 4)
+        v = np.float32(d16[0]) * np.float32(sc_of(s)) * np.float32(q) - np.float32(m16[0]) * np.float32(mn_of(s))
+        assert np.float32(v) == got[0, k]
+    # (iii) qh = 0 -> Q4_K
+    blk0 = blk.copy()
+    blk0[:, 16:48] = 0
+    q4 = np.concatenate([blk0[:, :16], blk0[:, 48:]], axis=1)
+    assert np.array_equal(O.dequant_q5_k(blk0), O.dequant_q4_k(q4))
+    # closed-form generator of the reference tests
+    w = O.closed_form_q5_k(3, 512)
+    deq = O.dequantize(w, O.GGML_Q5_K)
+    for o in range(3):
+        for b in range(2):
+            dd, mm = np.float32(0.015625 * (1 + o % 5)), np.float32(0.0078125 * (1 + b % 3))
+            for k in (0, 31, 32, 100, 255):
+                j = k >> 5
+                q = (k + 13 * o + 17 * b) % 32
+                want1 = dd * np.float32((3 * j + o + b) % 63 + 1) * np.float32(q) - mm * np.float32((5 * j + 2 * o + b) % 17)
+                assert deq[o, b * 256 + k] == np.float32(want1)
+
+
+def test_embedding_lookup_definition_and_errors():
+    w = O.closed_form_q4_k(9, 512)
+    ids = np.array([3, 0, 8, 3], dtype=np.int64)
+    assert np.array_equal(O.embedding_lookup(ids, w, O.GGML_Q4_K), O.dequantize(w, O.GGML_Q4_K)[ids])
+    with pytest.raises(ValueError, match="out-of-range"):
+        O.embedding_lookup(np.array([9]), w, O.GGML_Q4_K)
+    with pytest.raises(ValueError, match="shape"):
+        O.embedding_lookup(np.array([[1]]), w, O.GGML_Q4_K)
