@@ -259,6 +259,15 @@ int hipengine_gguf_q8_0_embedding_bf16_out(const int64_t* token_ids, const uint8
                                            int64_t rows, int64_t hidden_size, int64_t vocab_size, int64_t threads,
                                            hipengine_stream_t stream);
 
+/* Row-wise arg-max of float32 logits [rows, vocab_size] (greedy decode after the lm_head GEMV): the highest
+ * value's index (lowest index among equal values) as int32 into out_indices[rows], the value into out_values
+ * when that is not null.  block_values / block_indices are caller-owned scratch of
+ * rows * ceil(vocab_size / (threads * 4)) entries; threads in {128, 256, 512}.
+ * Replaces hipengine_argmax_f32_rows_i32 (kernels/hip_gfx1100/linear/lm_head.hip:746-793). */
+int hipengine_argmax_f32_rows_i32(const float* logits, float* block_values, int32_t* block_indices,
+                                  int32_t* out_indices, float* out_values, int64_t rows, int64_t vocab_size,
+                                  int64_t threads, hipengine_stream_t stream);
+
 /* Router: for each of `tokens` rows of float32 logits (row pitch logits_stride), the top_k
  * experts by logit, highest first (equal logits: lowest index), as int64 into
  * selected[tokens*top_k], and the softmax over those top_k logits into

@@ -33,6 +33,7 @@ moe_selected_ffn             committed golden of the reference
                              moe_ffn_selected_gguf_q4_k.json, copied as data
                              to tests/golden/); independent dense recompute
 moe_ffn_block                same golden file (``expected_block``)
+argmax_rows                  brute-force loop with the reference's pair comparison, ties
 embedding_lookup             definition: dequantize(qweight[ids]); error cases of the reference
 dequant_q5_k                 block builder inverse (reference generator restated),
                              scalar per-element loop, qh = 0 equals Q4_K
@@ -302,6 +303,14 @@ def embedding_lookup(token_ids, qweight, qtype: int) -> np.ndarray:
     if np.any(ids < 0) or np.any(ids >= qw.shape[0]):
         raise ValueError("token_ids contain out-of-range token IDs")
     return dequantize(qw[ids], qtype).astype(np.float32)
+
+
+def argmax_rows(logits) -> tuple[np.ndarray, np.ndarray]:
+    """Row-wise (index, value) of the maximum, lowest index among equal values
+    (``better_pair_i32``, kernels/hip_gfx1100/linear/lm_head.hip:188-190)."""
+    lg = np.asarray(logits, dtype=np.float32)
+    idx = np.argmax(lg, axis=-1).astype(np.int32)          # first occurrence = lowest index
+    return idx, np.take_along_axis(lg, idx[:, None].astype(np.int64), axis=-1)[:, 0]
 
 
 def silu(v: np.ndarray) -> np.ndarray:

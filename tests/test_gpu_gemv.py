@@ -364,3 +364,26 @@ def test_gemv_residual(dev, quant, rows, k, n, kind):
         got = dev.get(dout, np.float32, (rows, n))
         assert np.array_equal(got.view(np.uint32), (plain + res).astype(np.float32).view(np.uint32))
     dev.free(dx, dw, dr, dplain, dout)
+
+
+@pytest.mark.parametrize("rows,vocab,threads", [(1, 151936, 256), (8, 151936, 512), (3, 1000, 128), (5, 129, 256)])
+def test_argmax_rows(dev, rows, vocab, threads):
+    """Row-wise arg-max over the caller-owned two-stage scratch; equal values go to the lowest index."""
+    from hipengine_amd.kernels.hip_gfx950.linear import lm_head as L
+    rng = np.random.default_rng(rows + vocab)
+    lg = rng.standard_normal((rows, vocab)).astype(np.float32)
+    lg[0, [vocab - 1, vocab // 2, 5]] = 7.5
+    if rows > 1:
+        lg[1, :] = 0.25
+    n = L.argmax_scratch_entries(rows, vocab, threads)
+    dl = dev.put(lg)
+    dbv, dbi = dev.empty(n * 4, fill=0xFF), dev.empty(n * 4, fill=0xFF)
+    doi, dov = dev.empty(rows * 4, fill=0xFF), dev.empty(rows * 4, fill=0xFF)
+    L.argmax_f32_rows_i32(dl.ptr, dbv.ptr, dbi.ptr, doi.ptr, dov.ptr, rows, vocab, threads=threads)
+    idx, val = dev.get(doi, np.int32, (rows,)), dev.get(dov, np.float32, (rows,))
+    L.argmax_f32_rows_i32(dl.ptr, dbv.ptr, dbi.ptr, doi.ptr, None, rows, vocab, threads=threads)
+    idx2 = dev.get(doi, np.int32, (rows,))
+    dev.free(dl, dbv, dbi, doi, dov)
+    want_idx, want_val = O.argmax_rows(lg)
+    assert np.array_equal(idx, want_idx) and np.array_equal(idx2, want_idx)
+    assert np.array_equal(val.view(np.uint32), want_val.view(np.uint32))

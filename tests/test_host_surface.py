@@ -103,6 +103,7 @@ def test_backend_registers_the_documented_keys(clean_registry):
                 KernelKey("hip_gfx950", "moe_group_compact", "generic", "active_experts_source_rows"),
                 KernelKey("hip_gfx950", "moe_mmq_tile_map", "generic", "tile32"),
                 KernelKey("hip_gfx950", "router_select", "fp32"),
+                KernelKey("hip_gfx950", "argmax", "f32", "rows_i32"),
                 KernelKey("hip_gfx950", "embedding", "gguf_q5_k", "lookup_bf16_out"),
                 KernelKey("hip_gfx950", "embedding", "gguf_q6_k", "lookup_bf16_out"),
                 KernelKey("hip_gfx950", "linear", "gguf_q4_k", "dual_silu_gemv_bf16_bf16_out"),

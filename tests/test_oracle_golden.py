@@ -481,3 +481,18 @@ def test_embedding_lookup_definition_and_errors():
         O.embedding_lookup(np.array([9]), w, O.GGML_Q4_K)
     with pytest.raises(ValueError, match="shape"):
         O.embedding_lookup(np.array([[1]]), w, O.GGML_Q4_K)
+
+
+def test_argmax_rows_brute_force_with_ties():
+    rng = np.random.default_rng(8)
+    lg = rng.standard_normal((5, 97)).astype(np.float32)
+    lg[1, [7, 40, 90]] = 9.0
+    lg[2, :] = -1.5
+    idx, val = O.argmax_rows(lg)
+    for r in range(5):
+        bv, bi = np.float32(-3.4028234663852886e38), 2**31 - 1
+        for i in range(97):
+            if lg[r, i] > bv or (lg[r, i] == bv and i < bi):
+                bv, bi = lg[r, i], i
+        assert idx[r] == bi and val[r] == bv
+    assert idx[1] == 7 and idx[2] == 0
