@@ -150,6 +150,70 @@ class Harness:
             self.memory.free(buf)
         return ev_f, ev_u, 2 * wg.nbytes + wd.nbytes
 
+    def layer_graph_case(self, rows: int, steps: int, warmup: int, layers: int = 4, seed: int = 11):
+        """The matmuls of `layers` dense 27B-shape decoder layers (q, k, v, o + residual, gate/up pair with SiLU,
+        down + residual: 6 launches and 210.5 MB per layer, distinct weights per layer so that the working set
+        exceeds the Infinity Cache) launched eagerly and replayed as ONE HIP graph.
+        Returns (eager seconds per layer, graph seconds per layer, weight bytes per layer)."""
+        from hipengine_amd.kernels.hip_gfx950.quant import gguf_q8_1_gemv as G
+        from hipengine_amd.synthetic import synthetic_blocks
+
+        h_, kv, f_ = 5120, 1024, 17408
+        host = {"q": synthetic_blocks(GGML["q4_k"], h_, h_, seed=seed), "k": synthetic_blocks(GGML["q4_k"], kv, h_, seed=seed + 1),
+                "v": synthetic_blocks(GGML["q6_k"], kv, h_, seed=seed + 2), "o": synthetic_blocks(GGML["q4_k"], h_, h_, seed=seed + 3),
+                "g": synthetic_blocks(GGML["q4_k"], f_, h_, seed=seed + 4), "d": synthetic_blocks(GGML["q6_k"], h_, f_, seed=seed + 5)}
+        wbytes = host["q"].nbytes + host["k"].nbytes + host["v"].nbytes + host["o"].nbytes + 2 * host["g"].nbytes + host["d"].nbytes
+        dev_w = [{name: self.memory.to_device(w, runtime=self.rt) for name, w in host.items()} for _ in range(layers)]
+        up_w = [self.memory.to_device(host["g"], runtime=self.rt) for _ in range(layers)]
+        rng = np.random.default_rng(seed)
+        x = self.memory.to_device(rng.standard_normal((rows, h_)).astype(np.float32), runtime=self.rt)
+        bq, bo, bh = (self.memory.malloc(rows * h_ * 4, runtime=self.rt) for _ in range(3))
+        bk, bv = (self.memory.malloc(rows * kv * 4, runtime=self.rt) for _ in range(2))
+        bmid = self.memory.malloc(rows * f_ * 4, runtime=self.rt)
+        q4, q6 = G.FUSED[("q4_k", "f32", "f32")], G.FUSED[("q6_k", "f32", "f32")]
+
+        def chain(stream):
+            for l in range(layers):
+                w = dev_w[l]
+                q4(x.ptr, w["q"].ptr, bq.ptr, rows, h_, h_, stream=stream)
+                q4(x.ptr, w["k"].ptr, bk.ptr, rows, h_, kv, stream=stream)
+                q6(x.ptr, w["v"].ptr, bv.ptr, rows, h_, kv, stream=stream)
+                G.gguf_gemv_residual("gguf_q4_k", bq.ptr, "f32", w["o"].ptr, x.ptr, bo.ptr, "f32", rows, h_, h_, stream=stream)
+                G.gguf_pair_silu_gemv("gguf_q4_k", bo.ptr, "f32", w["g"].ptr, up_w[l].ptr, bmid.ptr, "f32", rows, h_, f_,
+                                      round_mid=False, stream=stream)
+                G.gguf_gemv_residual("gguf_q6_k", bmid.ptr, "f32", w["d"].ptr, bo.ptr, bh.ptr, "f32", rows, f_, h_, stream=stream)
+
+        stream = self.rt.stream_create()
+        chain(stream)
+        self.rt.stream_synchronize(stream)
+        self.rt.stream_begin_capture(stream)
+        chain(stream)
+        graph = self.rt.stream_end_capture(stream)
+        graph_exec = self.rt.graph_instantiate(graph)
+
+        def timed(fn):
+            for _ in range(warmup):
+                fn()
+            self.rt.stream_synchronize(stream)
+            self.rt.event_record(self.ev0, stream)
+            for _ in range(steps):
+                fn()
+            self.rt.event_record(self.ev1, stream)
+            self.rt.stream_synchronize(stream)
+            return self.rt.event_elapsed_time_ms(self.ev0, self.ev1) * 1e-3 / steps / layers
+
+        eager = timed(lambda: chain(stream))
+        replay = timed(lambda: self.rt.graph_launch(graph_exec, stream))
+        self.rt.graph_exec_destroy(graph_exec)
+        self.rt.graph_destroy(graph)
+        self.rt.stream_destroy(stream)
+        for d in dev_w:
+            for buf in d.values():
+                self.memory.free(buf)
+        for buf in (*up_w, x, bq, bo, bh, bk, bv, bmid):
+            self.memory.free(buf)
+        return eager, replay, wbytes
+
     def mmq_case(self, quant: str, m: int, k: int, n: int, steps: int, warmup: int):
         """MMQ prefill GEMM on pre-packed activations: (seconds per launch, int8 ops per launch)."""
         from hipengine_amd.kernels.hip_gfx950.quant import gguf_mmq_prefill as M
@@ -333,6 +397,12 @@ def main() -> None:
             "us": round(ev_f * 1e6, 1), "launches": 2, "GB/s": round(wbytes / ev_f / 1e9, 1),
             "frac_hbm": round(wbytes / ev_f / 1e9 / HBM_PEAK_GBS, 4),
             "unfused_3_gemv_us": round(ev_u * 1e6, 1)}
+
+        eager, replay, lbytes = h.layer_graph_case(1, max(10, steps // 4), 3)
+        extra["layer_27b_b1_fused_6_launches"] = {
+            "eager_us_per_layer": round(eager * 1e6, 1), "hip_graph_us_per_layer": round(replay * 1e6, 1),
+            "GB/s_graph": round(lbytes / replay / 1e9, 1), "frac_hbm_graph": round(lbytes / replay / 1e9 / HBM_PEAK_GBS, 4),
+            "tok_per_s_64_layers_matmuls_only_graph": round(1.0 / (64 * replay), 1)}
 
         msteps = max(5, args.steps // 50)
         for name, (quant, m, kk, nn) in {
