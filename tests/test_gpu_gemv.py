@@ -387,3 +387,28 @@ def test_argmax_rows(dev, rows, vocab, threads):
     want_idx, want_val = O.argmax_rows(lg)
     assert np.array_equal(idx, want_idx) and np.array_equal(idx2, want_idx)
     assert np.array_equal(val.view(np.uint32), want_val.view(np.uint32))
+
+
+def test_gemv_from_a_gguf_file(dev, tmp_path):
+    """File to kernel: tensors written into a GGUF container, read back through the reader's memory maps, uploaded
+    unchanged and multiplied - the raw block layout of the file IS the kernels' weight layout."""
+    from hipengine_amd.loading import gguf as GG
+    from hipengine_amd.quant.gguf import GGMLQuantizationType as T
+    k, n = 1024, 96
+    w4 = O.random_weight(O.GGML_Q4_K, n, k, seed=21)
+    w6 = O.random_weight(O.GGML_Q6_K, n, k, seed=22)
+    path = GG.write_gguf(tmp_path / "tiny.gguf", {"general.architecture": "test"},
+                         [("a.weight", T.Q4_K, (n, k), w4), ("b.weight", T.Q6_K, (n, k), w6)])
+    reader = GG.GGUFReader(path)
+    x = np.random.default_rng(3).standard_normal((2, k)).astype(np.float32)
+    dx = dev.put(x)
+    for name, quant, w in (("a.weight", "gguf_q4_k", w4), ("b.weight", "gguf_q6_k", w6)):
+        info = reader.tensor_info(name)
+        assert info.shape == (n, k) and info.byte_shape == w.shape
+        dw = reader.to_device(name, runtime=dev.runtime)
+        dout = dev.empty(2 * n * 4)
+        G.FUSED[(SHORT[quant], "f32", "f32")](dx.ptr, dw.ptr, dout.ptr, 2, k, n)
+        got = dev.get(dout, np.float32, (2, n))
+        dev.free(dw, dout)
+        _check_f32(got, O.quantize_q8_1(x), w, QT[quant])
+    dev.free(dx)

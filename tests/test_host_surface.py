@@ -239,3 +239,72 @@ def test_moe_wrappers_validate_before_touching_the_device():
         M.gguf_q4_k_grouped_mmq(1, 1, 1, 1, 1, 1, 8, 8, 256, 40, 4, 32)
     with pytest.raises(ValueError, match="multiple of 32"):
         M.gguf_q4_k_grouped_mmq(1, 1, 1, 1, 1, 1, 8, 8, 256, 64, 4, 40)
+
+
+def test_gguf_container_round_trip_and_errors(tmp_path):
+    """GGUF intake: a container written with the synthetic writer comes back with the same metadata, logical and
+    byte shapes and payload bytes (raw block rows as the kernels take them); malformed files raise as hipEngine's
+    scanner does (hipengine/loading/gguf.py:185-268)."""
+    import struct
+
+    import numpy as np
+
+    from hipengine_amd.loading import gguf as GG
+    from hipengine_amd.quant.gguf import GGMLQuantizationType as T
+
+    rng = np.random.default_rng(0)
+    q4 = rng.integers(0, 256, size=(6, 512 // 256 * 144), dtype=np.uint8)
+    q6 = rng.integers(0, 256, size=(2, 3, 256 // 256 * 210), dtype=np.uint8)      # [experts, rows, bytes]
+    f32 = rng.standard_normal((5,)).astype(np.float32)
+    bf16 = rng.integers(0, 65536, size=(4, 8), dtype=np.uint16)
+    meta = {"general.architecture": "qwen35", "general.file_type": 15, "qwen35.block_count": 2,
+            "tokenizer.ggml.tokens": ["a", "bc", ""], "qwen35.rope.freq_base": 1000000.0, "flag": True,
+            "qwen35.dims": [1, 2, 3], "big": 2**40, "neg": -7}
+    path = GG.write_gguf(tmp_path / "m.gguf", meta, [
+        ("blk.0.ffn_gate.weight", T.Q4_K, (6, 512), q4), ("blk.0.ffn_down_exps.weight", T.Q6_K, (2, 3, 256), q6),
+        ("output_norm.weight", T.F32, (5,), f32), ("token_embd.weight", T.BF16, (4, 8), bf16)], alignment=64)
+    reader = GG.GGUFReader(path)
+    info = reader.info
+    assert info.version == 3 and info.alignment == 64 and info.tensor_count == 4
+    assert info.architecture == "qwen35" and info.file_type == 15
+    assert info.metadata["tokenizer.ggml.tokens"] == ["a", "bc", ""] and info.metadata["flag"] is True
+    assert info.metadata["qwen35.dims"] == [1, 2, 3] and info.metadata["big"] == 2**40 and info.metadata["neg"] == -7
+    assert info.tensor_data_offset % 64 == 0
+    t = reader.tensor_info("blk.0.ffn_gate.weight")
+    assert t.shape == (6, 512) and t.ggml_shape == (512, 6) and t.byte_shape == (6, 288) and t.nbytes == 6 * 288
+    assert t.ggml_type == 12 and t.ggml_type_name == "Q4_K" and t.n_elements == 6 * 512 and t.data_offset % 64 == 0
+    assert np.array_equal(reader.tensor_data("blk.0.ffn_gate.weight"), q4)
+    e = reader.tensor_info("blk.0.ffn_down_exps.weight")
+    assert e.shape == (2, 3, 256) and e.byte_shape == (2, 3, 210)
+    assert np.array_equal(reader.tensor_data("blk.0.ffn_down_exps.weight"), q6)
+    assert np.array_equal(reader.tensor_data("output_norm.weight"), f32)
+    assert reader.tensor_data("token_embd.weight").dtype == np.uint16
+    assert np.array_equal(reader.tensor_data("token_embd.weight"), bf16)
+    assert info.total_tensor_nbytes == q4.nbytes + q6.nbytes + f32.nbytes + bf16.nbytes
+    assert info.names_with_prefix("blk.0.") == ("blk.0.ffn_gate.weight", "blk.0.ffn_down_exps.weight")
+    assert [x.name for x in info.require(["output_norm.weight", "token_embd.weight"])] == ["output_norm.weight", "token_embd.weight"]
+    with pytest.raises(GG.MissingGGUFTensorError, match="missing required GGUF tensors: nope"):
+        info.require(["output_norm.weight", "nope"])
+    with pytest.raises(GG.MissingGGUFTensorError):
+        reader.tensor_info("absent")
+
+    raw = path.read_bytes()
+    bad = tmp_path / "bad.gguf"
+    bad.write_bytes(b"GGUX" + raw[4:])
+    with pytest.raises(GG.GGUFFormatError, match="magic"):
+        GG.scan_gguf(bad)
+    bad.write_bytes(raw[:4] + struct.pack("<I", 9) + raw[8:])
+    with pytest.raises(GG.GGUFFormatError, match="unsupported GGUF version 9"):
+        GG.scan_gguf(bad)
+    bad.write_bytes(raw[: info.tensor_data_offset + 100])          # payload cut short
+    with pytest.raises(GG.GGUFFormatError, match="falls outside file size"):
+        GG.scan_gguf(bad)
+    bad.write_bytes(raw[:40])                                        # header cut short
+    with pytest.raises(EOFError):
+        GG.scan_gguf(bad)
+    with pytest.raises(ValueError, match="stored bytes"):
+        GG.write_gguf(tmp_path / "x.gguf", {}, [("w", T.Q4_K, (6, 512), q4[:5])])
+    v2 = GG.write_gguf(tmp_path / "v2.gguf", {"general.architecture": "x"}, [("w", T.Q8_0, (3, 64), np.zeros((3, 68), np.uint8))],
+                       version=2)
+    assert GG.scan_gguf(v2).version == 2 and GG.scan_gguf(v2).alignment == 32
+    assert GG.scan_gguf(v2).tensor("w").byte_shape == (3, 68)
