@@ -49,12 +49,13 @@ struct Variant {
   GEMV_VARIANT(QT, 8, 2, 1), GEMV_VARIANT(QT, 8, 2, 2), GEMV_VARIANT(QT, 8, 2, 5)
 
 const Variant kQ4K[] = {GEMV_VARIANTS_FOR(GGML_Q4_K)};
+const Variant kQ5K[] = {GEMV_VARIANTS_FOR(GGML_Q5_K)};
 const Variant kQ6K[] = {GEMV_VARIANTS_FOR(GGML_Q6_K)};
 const Variant kQ80[] = {GEMV_VARIANTS_FOR(GGML_Q8_0)};
 constexpr int kVariants = 24;
 
 const Variant* find_variant(int qt, int b, int r, int cb) {
-  const Variant* table = qt == GGML_Q4_K ? kQ4K : qt == GGML_Q6_K ? kQ6K : qt == GGML_Q8_0 ? kQ80 : nullptr;
+  const Variant* table = qt == GGML_Q4_K ? kQ4K : qt == GGML_Q5_K ? kQ5K : qt == GGML_Q6_K ? kQ6K : qt == GGML_Q8_0 ? kQ80 : nullptr;
   if (!table) return nullptr;
   for (int i = 0; i < kVariants; ++i)
     if (table[i].b == b && table[i].r == r && table[i].cb == cb) return &table[i];
@@ -485,6 +486,7 @@ int launch_gemv(int qt, const void* x, int x_kind, const uint8_t* w, void* out, 
   DEFINE_FUSED(QNAME, QT, fp16, KIND_F16, fp16, KIND_F16)
 
 DEFINE_FUSED_ALL(q4_k, GGML_Q4_K)
+DEFINE_FUSED_ALL(q5_k, GGML_Q5_K)
 DEFINE_FUSED_ALL(q6_k, GGML_Q6_K)
 DEFINE_FUSED_ALL(q8_0, GGML_Q8_0)
 

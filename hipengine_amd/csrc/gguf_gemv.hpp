@@ -6,6 +6,7 @@
 // evaluated as int32 sub-block dots of the packed weight integers with int8
 // activations (v_dot4_i32_i8), combined in float32 with the block scales:
 //   Q4_K: xd*(d*sc*dot - dmin*mn*qsum)   (gguf_q4_k_gemv.hip:893-904)
+//   Q5_K: the same with 5-bit quants       (gguf_k_gemv.hip:115-137)
 //   Q6_K: xd*d*sc16*(dot_u - 32*qsum16)  (gguf_k_gemv.hip:233-246)
 //   Q8_0: wd*xd*dot                      (gguf_q8_0_dp4a_gemv.hip:122-129)
 //
@@ -45,6 +46,9 @@ struct GemvArgs {
   int nrg;              // row groups per workgroup
 };
 
+// Q4_K and Q5_K share the header (d, dmin, 6-bit scales and mins) and the min term.
+constexpr bool gemv_has_mins(int qt) { return qt == GGML_Q4_K || qt == GGML_Q5_K; }
+
 template <int QT>
 struct GemvTraits;
 
@@ -52,6 +56,11 @@ template <>
 struct GemvTraits<GGML_Q4_K> {
   static constexpr int SUPER_BYTES = Q4_K_BYTES;  // bytes per 256 values
   static constexpr int REGS = 12;
+};
+template <>
+struct GemvTraits<GGML_Q5_K> {
+  static constexpr int SUPER_BYTES = Q5_K_BYTES;
+  static constexpr int REGS = 20;   // header 4, low nibbles 8, high bits qh[32] 8
 };
 template <>
 struct GemvTraits<GGML_Q6_K> {
@@ -79,6 +88,16 @@ __device__ __forceinline__ void gemv_load_block(const uint8_t* blk, int q, Weigh
     r.v[0] = h.x; r.v[1] = h.y; r.v[2] = h.z; r.v[3] = h.w;
     r.v[4] = a.x; r.v[5] = a.y; r.v[6] = a.z; r.v[7] = a.w;
     r.v[8] = b.x; r.v[9] = b.y; r.v[10] = b.z; r.v[11] = b.w;
+  } else if constexpr (QT == GGML_Q5_K) {
+    const uint4 h = load16(blk);                    // d, dmin, scales[12]
+    const uint4 a = load16(blk + 48 + q * 32);      // low nibbles, values 0..15 of sub-blocks 2q / 2q+1
+    const uint4 b = load16(blk + 64 + q * 32);      // values 16..31
+    const uint4 c = load16(blk + 16), d = load16(blk + 32);   // qh[32]: bit s of qh[l] = bit 4 of sub-block s, lane l
+    r.v[0] = h.x; r.v[1] = h.y; r.v[2] = h.z; r.v[3] = h.w;
+    r.v[4] = a.x; r.v[5] = a.y; r.v[6] = a.z; r.v[7] = a.w;
+    r.v[8] = b.x; r.v[9] = b.y; r.v[10] = b.z; r.v[11] = b.w;
+    r.v[12] = c.x; r.v[13] = c.y; r.v[14] = c.z; r.v[15] = c.w;
+    r.v[16] = d.x; r.v[17] = d.y; r.v[18] = d.z; r.v[19] = d.w;
   } else if constexpr (QT == GGML_Q6_K) {
     const int h = q >> 1, t = q & 1;
     const uint4 a = load16(blk + 64 * h + 16 * t);          // ql, first 32-byte group of the half
@@ -131,6 +150,19 @@ __device__ __forceinline__ void gemv_block_dots(const WeightRegs<GemvTraits<QT>:
     da = dot4(q4k_low(r.v[9]), a1.y, da);  db = dot4(q4k_high(r.v[9]), b1.y, db);
     da = dot4(q4k_low(r.v[10]), a1.z, da); db = dot4(q4k_high(r.v[10]), b1.z, db);
     da = dot4(q4k_low(r.v[11]), a1.w, da); db = dot4(q4k_high(r.v[11]), b1.w, db);
+    dots[0] = da; dots[1] = db; dots[2] = 0; dots[3] = 0;
+  } else if constexpr (QT == GGML_Q5_K) {
+    const uint4* xp = reinterpret_cast<const uint4*>(q8_blk + q * 64);
+    const uint4 a0 = xp[0], a1 = xp[1], b0 = xp[2], b1 = xp[3];
+    const uint32_t xa[8] = {a0.x, a0.y, a0.z, a0.w, a1.x, a1.y, a1.z, a1.w};
+    const uint32_t xb[8] = {b0.x, b0.y, b0.z, b0.w, b1.x, b1.y, b1.z, b1.w};
+    int da = 0, db = 0;
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+      const uint32_t qh = r.v[12 + i] >> (2 * q);               // bit 0: sub-block 2q, bit 1: sub-block 2q+1
+      da = dot4(q4k_low(r.v[4 + i]) | ((qh & 0x01010101u) << 4), xa[i], da);
+      db = dot4(q4k_high(r.v[4 + i]) | (((qh >> 1) & 0x01010101u) << 4), xb[i], db);
+    }
     dots[0] = da; dots[1] = db; dots[2] = 0; dots[3] = 0;
   } else if constexpr (QT == GGML_Q6_K) {
     const int h = q >> 1, t = q & 1;
@@ -185,7 +217,7 @@ struct BlockScales {
 template <int QT>
 __device__ __forceinline__ BlockScales<QT> gemv_block_scales(const WeightRegs<GemvTraits<QT>::REGS>& r, int q) {
   BlockScales<QT> s;
-  if constexpr (QT == GGML_Q4_K) {
+  if constexpr (gemv_has_mins(QT)) {
     const Q4KScales u = q4k_unpack_scales(r.v[1], r.v[2], r.v[3]);
     const float d = f16_bits_to_float(r.v[0] & 0xFFFFu), dmin = f16_bits_to_float(r.v[0] >> 16);
     // sub-blocks 2q and 2q+1 sit in bytes 2(q&1), 2(q&1)+1 of the low (q<2) or high word
@@ -222,7 +254,7 @@ __device__ __forceinline__ float gemv_block_term(const WeightRegs<GemvTraits<QT>
   const int sb0 = b * t.chunk_sb + blk_local * 8;
   int dots[4];
   gemv_block_dots<QT>(r, q, q8_blk, QT == GGML_Q6_K ? t.s16 + sb0 * 2 : nullptr, dots);
-  if constexpr (QT == GGML_Q4_K) {
+  if constexpr (gemv_has_mins(QT)) {
     const float2 xd = *reinterpret_cast<const float2*>(t.xd + sb0 + 2 * q);
     const float2 xs = *reinterpret_cast<const float2*>(t.xs + sb0 + 2 * q);
     float v = s.f[0] * (xd.x * static_cast<float>(dots[0]));
@@ -310,7 +342,7 @@ __device__ __forceinline__ void gemv_stage_activations(const GemvArgs& a, int kc
         const int total = oct_sum_i(part);
         if (e == 0) {
           xd_out[b * chunk_sb + j] = xd;
-          if constexpr (QT == GGML_Q4_K) xs_out[b * chunk_sb + j] = xd * static_cast<float>(total);
+          if constexpr (gemv_has_mins(QT)) xs_out[b * chunk_sb + j] = xd * static_cast<float>(total);
         }
       }
     }
@@ -323,7 +355,7 @@ inline size_t gemv_lds_bytes(int qt, int B, int R, int CB, int ks, int nrg) {
   const size_t chunk_sb = chunk_elems / 32;
   size_t bytes = B * chunk_elems;                       // q8
   bytes += B * chunk_sb * 4;                            // xd
-  if (qt == GGML_Q4_K) bytes += B * chunk_sb * 4;       // xs
+  if (gemv_has_mins(qt)) bytes += B * chunk_sb * 4;     // xs
   if (qt == GGML_Q6_K) bytes += B * chunk_sb * 8;       // s16
   bytes += static_cast<size_t>(ks) * nrg * 16 * R * B * 4;  // K-slice reduction
   return bytes;
@@ -358,7 +390,7 @@ __device__ __forceinline__ void gemv_workgroup_emit(const GemvArgs& a, const uin
   float* xd = reinterpret_cast<float*>(q8 + B * chunk_elems);
   float* xs = xd + B * chunk_sb;
   int* s16 = reinterpret_cast<int*>(xs);
-  float* red = (QT == GGML_Q4_K) ? xs + B * chunk_sb
+  float* red = gemv_has_mins(QT) ? xs + B * chunk_sb
              : (QT == GGML_Q6_K) ? reinterpret_cast<float*>(s16 + B * chunk_sb * 2)
                                  : xs;
 

@@ -115,6 +115,8 @@ extern "C" int hipengine_gfx950_gguf_q8_1_block_dots_i32(int32_t ggml_type, cons
   const int K = static_cast<int>(in_features), N = static_cast<int>(out_features);
   if (ggml_type == GGML_Q4_K) {
     hipLaunchKernelGGL(block_dots_kernel<GGML_Q4_K>, g, dim3(64), 0, stream, x, qweight, dots, qsums, K, N);
+  } else if (ggml_type == GGML_Q5_K) {
+    hipLaunchKernelGGL(block_dots_kernel<GGML_Q5_K>, g, dim3(64), 0, stream, x, qweight, dots, qsums, K, N);
   } else if (ggml_type == GGML_Q6_K) {
     hipLaunchKernelGGL(block_dots_kernel<GGML_Q6_K>, g, dim3(64), 0, stream, x, qweight, dots, qsums, K, N);
   } else if (ggml_type == GGML_Q8_0) {

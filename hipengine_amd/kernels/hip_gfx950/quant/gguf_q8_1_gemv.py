@@ -35,7 +35,7 @@ from hipengine_amd.kernels.registry import KernelKey, register
 
 _FUSED_ARGS = [VOID, VOID, VOID, I64, I64, I64, I64, VOID]
 _Q8_1_ARGS = [VOID, VOID, VOID, I64, I64, I64, VOID]
-_QUANTS = ("q4_k", "q6_k", "q8_0")
+_QUANTS = ("q4_k", "q5_k", "q6_k", "q8_0")
 _FUSED_DTYPES = (("f32", "f32"), ("bf16", "f32"), ("bf16", "bf16"), ("bf16", "fp16"), ("fp16", "f32"), ("fp16", "fp16"))
 _KINDS = {"f32": KIND_F32, "bf16": KIND_BF16, "fp16": KIND_F16, "q8_1": KIND_Q8_1}
 

@@ -75,8 +75,9 @@ int hipengine_gguf_q8_1_d4s4_f32_quantize_bf16(const void* x, void* out, int64_t
 
 /* ------------------------------------------------------------------------
  * Decode GEMV, batch 1..8 per launch (more rows are split into launches of 8)
- *   out[r, n] = sum_k W[n, k] * x[r, k],  W raw Q4_K / Q6_K / Q8_0 blocks
- * in_features % 256 == 0 for all three weight types.
+ *   out[r, n] = sum_k W[n, k] * x[r, k],  W raw Q4_K / Q5_K / Q6_K / Q8_0 blocks
+ * in_features % 256 == 0 for all weight types.  Q5_K (arithmetic of gguf_k_gemv.hip:115-137 on q8_1
+ * activations) runs the row-strided form only.
  * ------------------------------------------------------------------------ */
 
 /* Fused: x is [rows, in_features] float32 / bf16 / fp16; the q8_1 quantization
@@ -97,6 +98,7 @@ int hipengine_gguf_q8_1_d4s4_f32_quantize_bf16(const void* x, void* out, int64_t
   HIPENGINE_GFX950_DECLARE_FUSED(q, fp16, f32) \
   HIPENGINE_GFX950_DECLARE_FUSED(q, fp16, fp16)
 HIPENGINE_GFX950_DECLARE_FUSED_ALL(q4_k)
+HIPENGINE_GFX950_DECLARE_FUSED_ALL(q5_k)
 HIPENGINE_GFX950_DECLARE_FUSED_ALL(q6_k)
 HIPENGINE_GFX950_DECLARE_FUSED_ALL(q8_0)
 

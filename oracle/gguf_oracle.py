@@ -532,6 +532,17 @@ def block_dots_q4_k(qs_i8: np.ndarray, qweight: np.ndarray) -> tuple[np.ndarray,
     return dots, a.sum(axis=-1, dtype=np.int32)
 
 
+def block_dots_q5_k(qs_i8: np.ndarray, qweight: np.ndarray) -> tuple[np.ndarray, np.ndarray]:
+    """Per 32-wide sub-block ``dot[r,n,j] = sum q5*q8`` and ``qsum[r,j] = sum q8`` as int32
+    (Q5_K through the Q4_K q8_1 formula with 5-bit quants, gguf_k_gemv.hip:115-137)."""
+    n = qweight.shape[0]
+    blocks, _ = _as_blocks(qweight, Q5_K_BLOCK_BYTES)
+    q5 = q5_k_quants(blocks).reshape(n, -1, 32).astype(np.int32)
+    a = qs_i8.astype(np.int32)
+    dots = np.einsum("rjk,njk->rnj", a, q5, optimize=True).astype(np.int32)
+    return dots, a.sum(axis=-1, dtype=np.int32)
+
+
 def block_dots_q6_k(qs_i8: np.ndarray, qweight: np.ndarray) -> np.ndarray:
     """Per 16-wide sub-block: ``dot = sum u6*q8 - 32*sum q8 = sum (u6-32)*q8``
     as int32 ``[rows, N, K/16]`` (gguf_k_gemv.hip:233-246)."""

@@ -412,3 +412,25 @@ def test_gemv_from_a_gguf_file(dev, tmp_path):
         dev.free(dw, dout)
         _check_f32(got, O.quantize_q8_1(x), w, QT[quant])
     dev.free(dx)
+
+
+@pytest.mark.parametrize("rows,k,n", [(1, 5120, 300), (2, 1024, 77), (5, 2048, 64), (8, 512, 33)])
+def test_q5_k_fused_gemv_and_block_dots(dev, rows, k, n):
+    """Q5_K (row-strided form): int32 sub-block dots bit-exact, float32 output within the parity gate of the
+    reference CPU GEMV on the q8_1-dequantized activations; closed-form weights of the reference tests too."""
+    rng = np.random.default_rng(rows + k + n)
+    x = rng.standard_normal((rows, k)).astype(np.float32)
+    xq = O.quantize_q8_1(x)
+    for w in (_random_q5_k(n, k, 9), O.closed_form_q5_k(n, k)):
+        dx, dxq, dw = dev.put(x), dev.put(xq), dev.put(w)
+        dout = dev.empty(rows * n * 4)
+        ddots, dqs = dev.empty(rows * n * (k // 32) * 4), dev.empty(rows * (k // 32) * 4)
+        G.FUSED[("q5_k", "f32", "f32")](dx.ptr, dw.ptr, dout.ptr, rows, k, n)
+        V.gguf_q8_1_block_dots_i32("gguf_q5_k", dxq.ptr, dw.ptr, ddots.ptr, dqs.ptr, rows, k, n)
+        got = dev.get(dout, np.float32, (rows, n))
+        dots = dev.get(ddots, np.int32, (rows, n, k // 32))
+        dev.free(dx, dxq, dw, dout, ddots, dqs)
+        want_dots, _ = O.block_dots_q5_k(O.q8_1_fields(xq)[2], w)
+        assert np.array_equal(dots, want_dots)
+        ref = O.gguf_quant_gemv(O.dequantize_q8_1(xq), w, O.GGML_Q5_K)
+        assert O.max_rel_err(got, ref) <= REL_TOL and O.cosine(got, ref) >= COS_MIN

@@ -496,3 +496,20 @@ def test_argmax_rows_brute_force_with_ties():
                 bv, bi = lg[r, i], i
         assert idx[r] == bi and val[r] == bv
     assert idx[1] == 7 and idx[2] == 0
+
+
+def test_q5_k_block_dots_against_int64_brute_force():
+    rng = np.random.default_rng(77)
+    n, k, rows = 3, 512, 2
+    nblk = n * (k // 256)
+    w = O.pack_q5_k_blocks(rng.integers(0, 32, size=(nblk, 8, 32), dtype=np.uint8), rng.integers(0, 64, size=(nblk, 8), dtype=np.uint8),
+                           rng.integers(0, 64, size=(nblk, 8), dtype=np.uint8), np.full(nblk, 0.01, np.float32),
+                           np.full(nblk, 0.005, np.float32)).reshape(n, -1)
+    qs = rng.integers(-128, 128, size=(rows, k // 32, 32), dtype=np.int8)
+    dots, qsum = O.block_dots_q5_k(qs, w)
+    deq = O.q5_k_quants(w.reshape(-1, 176)).reshape(n, k).astype(np.int64)
+    for r in range(rows):
+        for row in range(n):
+            for j in range(k // 32):
+                assert dots[r, row, j] == int(np.dot(qs[r, j].astype(np.int64), deq[row, j * 32:(j + 1) * 32]))
+        assert np.array_equal(qsum[r], qs[r].astype(np.int64).sum(axis=-1))
