@@ -123,20 +123,23 @@ SlabVariant kSlab[] = {SLAB_VARIANT(1, 1), SLAB_VARIANT(1, 2), SLAB_VARIANT(2, 1
                        SLAB_VARIANT(4, 1), SLAB_VARIANT(4, 2), SLAB_VARIANT(8, 1), SLAB_VARIANT(8, 2)};
 
 struct SlabPlan {
-  int b, bpw, waves, rows_wg;
+  int b, bpw, waves, two_block_waves, rows_wg;
   bool ok;
 };
 
+// K <= 4096: one block per wave (up to 16 waves).  4352 <= K <= 6144: 12 waves, the first nb - 12 of them
+// with two blocks, so that every SIMD gets three waves and (at K = 5120) five blocks.
 SlabPlan default_slab_plan(int qt, int rows, int64_t K, int64_t N) {
   SlabPlan p{};
   const int nb = static_cast<int>(K / QK_K);
   p.b = rows <= 1 ? 1 : rows <= 2 ? 2 : rows <= 4 ? 4 : 8;
   p.bpw = nb <= 16 ? 1 : 2;
-  p.waves = (nb + p.bpw - 1) / p.bpw;
+  p.waves = p.bpw == 1 ? nb : 12;
+  p.two_block_waves = p.bpw == 1 ? 0 : nb - 12;
   const int64_t per_cu = (N + 255) / 256;
   p.rows_wg = static_cast<int>(per_cu < 1 ? 1 : per_cu > SLAB_MAX_ROWS ? SLAB_MAX_ROWS : per_cu);
-  p.ok = qt == GGML_Q4_K && rows >= 1 && rows <= 8 && nb >= 4 && p.waves <= (p.bpw == 1 ? 16 : 12) &&
-         gemv_slab_lds_bytes(p.b, p.bpw, p.waves) <= 160 * 1024;
+  p.ok = qt == GGML_Q4_K && rows >= 1 && rows <= 8 && nb >= 4 && nb <= 24 &&
+         gemv_slab_lds_bytes(p.b, p.waves, p.two_block_waves) <= 160 * 1024;
   return p;
 }
 
@@ -147,10 +150,12 @@ int launch_gemv_slab(const void* x, int x_kind, const uint8_t* w, void* out, int
   for (SlabVariant& c : kSlab)
     if (c.b == p.b && c.bpw == p.bpw) v = &c;
   if (!v || rows > p.b || x_kind < KIND_F32 || x_kind > KIND_Q8_1 || p.rows_wg < 1 || p.rows_wg > SLAB_MAX_ROWS ||
-      p.waves != (nb + p.bpw - 1) / p.bpw || p.waves > (p.bpw == 1 ? 16 : 12) || K > (1 << 20) || N > (1 << 30)) {
+      p.waves < 1 || p.waves > (p.bpw == 1 ? 16 : 12) || p.two_block_waves < 0 || p.two_block_waves > p.waves ||
+      (p.bpw == 1 && p.two_block_waves != 0) || p.waves + p.two_block_waves != nb || K > (1 << 20) ||
+      N > (1 << 30)) {
     return static_cast<int>(hipErrorInvalidValue);
   }
-  const size_t lds = gemv_slab_lds_bytes(p.b, p.bpw, p.waves);
+  const size_t lds = gemv_slab_lds_bytes(p.b, p.waves, p.two_block_waves);
   if (lds > 160 * 1024) return static_cast<int>(hipErrorInvalidValue);
   if (lds > 64 * 1024 && !v->lds_raised[x_kind]) {
     const hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(v->by_kind[x_kind]),
@@ -158,7 +163,8 @@ int launch_gemv_slab(const void* x, int x_kind, const uint8_t* w, void* out, int
     if (e != hipSuccess) return static_cast<int>(e);
     v->lds_raised[x_kind] = true;
   }
-  GemvSlabArgs a{x, w, out, x_kind, out_kind, rows, static_cast<int>(K), static_cast<int>(N), p.rows_wg, p.waves, residual};
+  GemvSlabArgs a{x, w, out, x_kind, out_kind, rows, static_cast<int>(K), static_cast<int>(N), p.rows_wg, p.waves,
+                 p.two_block_waves, residual};
   const unsigned grid = static_cast<unsigned>((N + p.rows_wg - 1) / p.rows_wg);
   hipLaunchKernelGGL(v->by_kind[x_kind], dim3(grid), dim3(p.waves * 64), lds, stream, a);
   return static_cast<int>(hipGetLastError());

@@ -234,26 +234,39 @@ __device__ __forceinline__ void gemv_run_stage_commit(const GemvRunArgs& a, cons
       const int j = team + s * nteams;
       if (j < groups) gemv_run_stage_one<QT>(a.x_kind, sr.raw[b][s], b < a.rows, j, e, q8_row, rec_row, s16_row);
     }
-    // large K: the rest is loaded here, two groups per thread at a time so that the
-    // load latency is paid once per two groups and not once per group
-    constexpr int P = 2;
-    for (int j0 = team + S * nteams; j0 < groups; j0 += P * nteams) {
+  }
+  // large K or batch: the rest - (batch row, group) items past the first S groups per row - is loaded here, P
+  // items per thread at a time across the batch rows, so that a load latency is paid once per P items
+  // and not once per item per row
+  const int rest = groups - S * nteams;              // groups per row still to do (may be <= 0)
+  if (rest > 0) {
+    constexpr int P = B >= 4 ? 8 : 2;
+    const int per_row = (rest + nteams - 1) / nteams;  // items of this team per batch row
+    const int items = per_row * B;
+    int b0 = 0, r0 = 0;                               // batch row and per-row index of item i0 (no division)
+    for (int i0 = 0; i0 < items; i0 += P) {
       uint32_t raw[P][8];
+      int b = b0, r = r0;
 #pragma unroll
       for (int p = 0; p < P; ++p) {
-        const int j = j0 + p * nteams;
-        if (b < a.rows && j < groups) {
+        const int j = team + (S + r) * nteams;
+        if (b < a.rows && j < groups) {               // b >= B only past the last item; then b >= a.rows too
           gemv_run_fetch8(a, b, j, e, raw[p]);
         } else {
 #pragma unroll
           for (int i = 0; i < 8; ++i) raw[p][i] = 0u;
         }
+        if (++r == per_row) { r = 0; ++b; }
       }
+      b = b0; r = r0;
 #pragma unroll
       for (int p = 0; p < P; ++p) {
-        const int j = j0 + p * nteams;
-        if (j < groups) gemv_run_stage_one<QT>(a.x_kind, raw[p], b < a.rows, j, e, q8_row, rec_row, s16_row);
+        const int j = team + (S + r) * nteams;
+        if (b < B && j < groups)
+          gemv_run_stage_one<QT>(a.x_kind, raw[p], b < a.rows, j, e, q8 + b * nb * Q8S, rec + b * nb * 16, s16 + b * nb * 16);
+        if (++r == per_row) { r = 0; ++b; }
       }
+      b0 = b; r0 = r;
     }
   }
 }

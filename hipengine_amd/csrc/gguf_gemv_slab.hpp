@@ -9,8 +9,9 @@
 //
 // Work decomposition
 //   * workgroup b owns rows [b*R, b*R + R), R = ceil(N / 256) <= 96, in steps of 32;
-//   * wave w owns the K blocks [w*BPW, w*BPW + BPW) of every row, BPW in {1, 2}
-//     (K = 5120: 10 waves x 2 blocks).  It quantizes ONLY its own K slice of the
+//   * wave w owns one or two consecutive K blocks of every row: the first `two_block_waves`
+//     waves two, the others one (K = 5120: 12 waves = 8 x 2 + 4 x 1 blocks, which gives every
+//     SIMD three waves and five blocks; 10 waves x 2 blocks would load two SIMDs with six).  It quantizes ONLY its own K slice of the
 //     activations (B x BPW x 256 values) into wave-private LDS: no workgroup
 //     barrier before the final sum;
 //   * per step the wave reads its 32 x (BPW*144) byte piece of the weight with
@@ -57,7 +58,8 @@ struct GemvSlabArgs {
   int K;
   int N;
   int rows_wg;   // output rows per workgroup, 1..96
-  int waves;     // waves per workgroup = ceil(nb / BPW)
+  int waves;     // waves per workgroup
+  int two_block_waves;   // waves 0..two_block_waves-1 own two K blocks each, the rest one
   const void* residual;   // null, or [rows, N] of the output type: out = round(projection) + residual
 };
 
@@ -66,63 +68,72 @@ constexpr int SLAB_MAX_ROWS = 96;
 template <int BPW>
 constexpr int slab_row_pitch() { return BPW == 1 ? 144 : 304; }
 
-// Per wave: the weight piece of a step (reused for the partial sums after the last
-// step), a 16-byte dump slot, the scale records and the int8 activations.
-constexpr int slab_wave_bytes(int B, int BPW) {
-  return 32 * (BPW == 1 ? 144 : 304) + 16 + BPW * 8 * 16 * 4 + B * (BPW * 256 + 16);
+// Per wave of `blocks` (1 or 2) K blocks: the weight piece of a step (reused for the partial sums
+// after the last step), a 16-byte dump slot, the scale records and the int8 activations.
+constexpr int slab_pitch(int blocks) { return blocks == 1 ? 144 : 304; }
+constexpr int slab_wave_bytes(int B, int blocks) {
+  return 32 * slab_pitch(blocks) + 16 + blocks * 8 * 16 * 4 + B * (blocks * 256 + 16);
 }
 
-inline size_t gemv_slab_lds_bytes(int b, int bpw, int waves) {
-  return static_cast<size_t>(waves) * slab_wave_bytes(b, bpw);
+inline size_t gemv_slab_lds_bytes(int b, int waves, int two_block_waves) {
+  return static_cast<size_t>(two_block_waves) * slab_wave_bytes(b, 2) +
+         static_cast<size_t>(waves - two_block_waves) * slab_wave_bytes(b, 1);
 }
 
 template <int B, int BPW, int XK>
 __device__ __forceinline__ void gemv_slab_q4k_workgroup(const GemvSlabArgs& a, uint8_t* smem) {
   constexpr int VB = B < 4 ? B : 4;                  // result registers in use per lane
-  constexpr int PITCH = slab_row_pitch<BPW>();
-  constexpr int XQ_PITCH = BPW * 256 + 16;           // int8 activations, one batch row
-  constexpr int WQ_BYTES = 32 * PITCH;
-  constexpr int DUMP = WQ_BYTES;
-  constexpr int REC = WQ_BYTES + 16;
-  constexpr int XQ = REC + BPW * 8 * 16 * 4;
-  constexpr int WAVE_BYTES = slab_wave_bytes(B, BPW);
   constexpr int NL = (32 * BPW * 9 + 63) / 64;       // 16-byte loads per lane and step
   constexpr int MAX_STEPS = SLAB_MAX_ROWS / 32;
   constexpr int EARLY_TAIL_ROWS = 7;                 // a last step of at most this many rows is done first
   constexpr int NLT = (EARLY_TAIL_ROWS * BPW * 9 + 63) / 64;
-  static_assert(B * SLAB_MAX_ROWS * 4 <= WQ_BYTES, "partial sums must fit the weight piece");
+  static_assert(B * SLAB_MAX_ROWS * 4 <= 32 * slab_pitch(1), "partial sums must fit the weight piece");
   const int x_kind = XK >= 0 ? XK : a.x_kind;
 
   const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int n = lane & 31, g = lane >> 5;
   const int nb = a.K / QK_K;
-  const int kb0 = wave * BPW;
-  const int blocks_w = min(BPW, nb - kb0);           // >= 1: waves = ceil(nb / BPW)
+  const int t2 = BPW == 2 ? a.two_block_waves : 0;
+  const int blocks_w = wave < t2 ? 2 : 1;
+  const int kb0 = wave < t2 ? 2 * wave : t2 + wave;
+  // LDS layout of this wave (sizes depend on its block count)
+  const int PITCH = slab_pitch(blocks_w);
+  const int XQ_PITCH = blocks_w * 256 + 16;            // int8 activations, one batch row
+  const int DUMP = 32 * PITCH;
+  const int REC = DUMP + 16;
+  const int XQ = REC + blocks_w * 8 * 16 * 4;
+  const int wave_off = wave < t2 ? wave * slab_wave_bytes(B, 2)
+                                 : t2 * slab_wave_bytes(B, 2) + (wave - t2) * slab_wave_bytes(B, 1);
   const int r0 = static_cast<int>(blockIdx.x) * a.rows_wg;
   const int rows_wg = min(a.rows_wg, a.N - r0);
   const int steps = (rows_wg + 31) >> 5;
   const int row_bytes = nb * Q4_K_BYTES;
   const uint8_t* wbase = a.w + static_cast<int64_t>(r0) * row_bytes + kb0 * Q4_K_BYTES;
 
-  uint8_t* wq = smem + wave * WAVE_BYTES;
+  uint8_t* wq = smem + wave_off;
   float* rec = reinterpret_cast<float*>(wq + REC);   // [BPW*8 sub-blocks][xd[8], xd*qsum[8]]
   uint8_t* xq = wq + XQ;
 
   // ---- activation loads of this wave's K slice: 4 lanes per 32-value group, 8 values per lane,
-  // 16 groups per pass.  Group p*16 + quad is batch row gid / (BPW*8), sub-block gid % (BPW*8).
+  // 16 groups per pass.  Group p*16 + quad is batch row gid / (blocks_w*8), sub-block gid % (blocks_w*8);
+  // a one-block wave is done after half the passes of a two-block wave.
   constexpr int PASSES = (B * BPW * 8 + 15) / 16;
+  const int gshift = blocks_w == 2 ? 4 : 3;
+  const int passes = (B * blocks_w * 8 + 15) >> 4;
   const int quad = lane >> 2, e = lane & 3;
   uint32_t raw[PASSES][8];
 #pragma unroll
   for (int p = 0; p < PASSES; ++p) {
     const int gid = p * 16 + quad;
     // clamped, unconditional: rows >= a.rows and blocks past the slice are quantized but not used
-    const int bb = min(gid / (BPW * 8), a.rows - 1);
-    const int rem = gid % (BPW * 8);
-    const int j = (kb0 + min(rem >> 3, blocks_w - 1)) * 8 + (rem & 7);
+    const int bb = min(gid >> gshift, a.rows - 1);
+    const int rem = gid & ((1 << gshift) - 1);
+    const int j = (kb0 + (rem >> 3)) * 8 + (rem & 7);
 #pragma unroll
     for (int i = 0; i < 8; ++i) raw[p][i] = 0u;
-    if (x_kind == KIND_F32) {
+    if (p >= passes) {
+      // nothing left for this wave
+    } else if (x_kind == KIND_F32) {
       const uint4* src = reinterpret_cast<const uint4*>(static_cast<const float*>(a.x) + static_cast<int64_t>(bb) * a.K + j * 32 + e * 8);
       const uint4 lo = src[0], hi = src[1];
       raw[p][0] = lo.x; raw[p][1] = lo.y; raw[p][2] = lo.z; raw[p][3] = lo.w;
@@ -190,12 +201,13 @@ __device__ __forceinline__ void gemv_slab_q4k_workgroup(const GemvSlabArgs& a, u
     if constexpr (B >= 8) {
       if (p == PASSES / 2) issue(0, buf);
     }
+    if (p >= passes) continue;
     const int gid = p * 16 + quad;
-    const int b = gid / (BPW * 8), rem = gid % (BPW * 8);
+    const int b = gid >> gshift, rem = gid & ((1 << gshift) - 1);
     uint32_t packed[2];
     float xd;
     q8_quantize8(x_kind, raw[p], true, packed, xd);
-    const bool used = b < a.rows && (rem >> 3) < blocks_w;
+    const bool used = b < a.rows;
     packed[0] = used ? packed[0] : 0u;
     packed[1] = used ? packed[1] : 0u;
     xd = used ? xd : 0.0f;
@@ -325,8 +337,10 @@ __device__ __forceinline__ void gemv_slab_q4k_workgroup(const GemvSlabArgs& a, u
   for (int idx = tid; idx < a.rows * rows_wg; idx += blockDim.x) {
     const int m = idx / rows_wg, rl = idx - m * rows_wg;
     float v = 0.0f;
-    for (int s = 0; s < a.waves; ++s)
-      v += reinterpret_cast<const float*>(smem + s * WAVE_BYTES)[m * SLAB_MAX_ROWS + rl];
+    for (int s = 0; s < a.waves; ++s) {
+      const int off = s < t2 ? s * slab_wave_bytes(B, 2) : t2 * slab_wave_bytes(B, 2) + (s - t2) * slab_wave_bytes(B, 1);
+      v += reinterpret_cast<const float*>(smem + off)[m * SLAB_MAX_ROWS + rl];
+    }
     const int64_t oi = static_cast<int64_t>(m) * a.N + r0 + rl;
     if (a.residual) v = round_to_kind(v, a.out_kind) + load_scalar(a.residual, oi, a.out_kind);
     store_scalar(a.out, oi, v, a.out_kind);
