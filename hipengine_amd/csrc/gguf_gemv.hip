@@ -6,6 +6,7 @@
 #include "gguf_gemv_run.hpp"
 #include "gguf_gemv_stream.hpp"
 #include "gguf_gemv_slab.hpp"
+#include "gguf_gemv_pslab.hpp"
 
 #include "../../include/hipengine_gfx950.h"
 
@@ -99,6 +100,8 @@ const RunVariant* find_run_variant(int qt, int b, int g, int cb) {
   return nullptr;
 }
 
+constexpr size_t kMaxLds = 160 * 1024;   // LDS of one CU
+
 // ---- slab form (Q4_K on the int8 MFMA, one workgroup per CU, waves split K) ----
 
 // BPW = 1: up to 16 waves (K <= 4096); BPW = 2: up to 12 waves (K <= 6144), whose 64
@@ -167,6 +170,114 @@ int launch_gemv_slab(const void* x, int x_kind, const uint8_t* w, void* out, int
                  p.two_block_waves, residual};
   const unsigned grid = static_cast<unsigned>((N + p.rows_wg - 1) / p.rows_wg);
   hipLaunchKernelGGL(v->by_kind[x_kind], dim3(grid), dim3(p.waves * 64), lds, stream, a);
+  return static_cast<int>(hipGetLastError());
+}
+
+// ---- phased slab form (Q6_K / Q8_0 on the int8 MFMA, batch 3..8, any K) ----
+
+template <int QT, int B, bool PHASED, int XK>
+__global__ void __launch_bounds__(768) gemv_pslab_kernel(GemvPslabArgs a) {
+  extern __shared__ __align__(16) uint8_t smem[];
+  gemv_pslab_workgroup<QT, B, PHASED, XK>(a, smem);
+}
+
+using PslabKernelFn = void (*)(GemvPslabArgs);
+struct PslabVariant {
+  int qt, b;
+  bool phased;
+  PslabKernelFn by_kind[4];
+  bool lds_raised[4];
+};
+#define PSLAB_VARIANT(QT, B, P)                                                                              \
+  PslabVariant { QT, B, P, {gemv_pslab_kernel<QT, B, P, KIND_F32>, gemv_pslab_kernel<QT, B, P, KIND_BF16>,   \
+                            gemv_pslab_kernel<QT, B, P, KIND_F16>, gemv_pslab_kernel<QT, B, P, KIND_Q8_1>}, \
+                 {false, false, false, false} }
+PslabVariant kPslab[] = {PSLAB_VARIANT(GGML_Q6_K, 4, false), PSLAB_VARIANT(GGML_Q6_K, 4, true),
+                         PSLAB_VARIANT(GGML_Q6_K, 8, false), PSLAB_VARIANT(GGML_Q6_K, 8, true),
+                         PSLAB_VARIANT(GGML_Q8_0, 4, false), PSLAB_VARIANT(GGML_Q8_0, 4, true),
+                         PSLAB_VARIANT(GGML_Q8_0, 8, false), PSLAB_VARIANT(GGML_Q8_0, 8, true)};
+
+struct PslabPlan {
+  int b, waves, bpw_log2, phases, grid;
+  bool ok;
+};
+
+size_t pslab_lds_bytes(int qt, int b, int waves, int bpw) {
+  return static_cast<size_t>(waves) *
+         (qt == GGML_Q6_K ? pslab_wave_bytes<GGML_Q6_K>(b, bpw) : pslab_wave_bytes<GGML_Q8_0>(b, bpw));
+}
+
+int pslab_grid(int64_t N, int phases) {
+  // one phase: a workgroup per CU walks its share of the rows group by group; several phases: a
+  // workgroup has one group of at most 96 rows
+  const int64_t groups = (N + PSLAB_GROUP_ROWS - 1) / PSLAB_GROUP_ROWS;
+  const int64_t per_cu = N < 256 ? N : 256;
+  return static_cast<int>(phases == 1 ? per_cu : (groups > per_cu ? groups : per_cu));
+}
+
+// Waves and blocks per wave: the split of K/256 blocks over W <= 12 waves x bpw in {1, 2, 4} x phases
+// that wastes the fewest block slots, preferring a single phase (activations quantized once) and more
+// waves.
+PslabPlan default_pslab_plan(int qt, int rows, int64_t K, int64_t N, const void* w) {
+  PslabPlan p{};
+  const int nb = static_cast<int>(K / QK_K);
+  const int64_t row_bytes = static_cast<int64_t>(nb) * (qt == GGML_Q6_K ? Q6_K_BYTES : 8 * Q8_0_BYTES);
+  if ((qt != GGML_Q6_K && qt != GGML_Q8_0) || rows < 1 || rows > 8 || nb < 8 || (nb & 1) != 0 ||
+      (reinterpret_cast<uintptr_t>(w) & 3u) != 0 || N < 1 || N * row_bytes > 0xFFFF0000ll) {
+    return p;
+  }
+  p.b = rows <= 4 ? 4 : 8;
+  float best = -1.0f;
+  for (int waves = 12; waves >= 6; --waves) {
+    for (int bl2 = 0; bl2 <= 2; ++bl2) {
+      const int bpw = 1 << bl2;
+      if (waves * bpw > nb || pslab_lds_bytes(qt, p.b, waves, bpw) > kMaxLds) continue;
+      const int phases = (nb + waves * bpw - 1) / (waves * bpw);
+      const float score = static_cast<float>(nb) / static_cast<float>(waves * bpw * phases) -
+                          0.02f * static_cast<float>(12 - waves) + (phases == 1 ? 0.05f : 0.0f) - 0.001f * bl2;
+      if (score > best) {
+        best = score;
+        p.waves = waves; p.bpw_log2 = bl2; p.phases = phases;
+      }
+    }
+  }
+  if (best < 0.0f) return p;
+  p.grid = pslab_grid(N, p.phases);
+  p.ok = true;
+  return p;
+}
+
+int launch_gemv_pslab(int qt, const void* x, int x_kind, const uint8_t* w, void* out, int out_kind, int rows,
+                      int64_t K, int64_t N, const PslabPlan& p, hipStream_t stream, const void* residual = nullptr) {
+  const int nb = static_cast<int>(K / QK_K);
+  const int bpw = 1 << p.bpw_log2;
+  const int64_t row_bytes = static_cast<int64_t>(nb) * (qt == GGML_Q6_K ? Q6_K_BYTES : 8 * Q8_0_BYTES);
+  PslabVariant* v = nullptr;
+  for (PslabVariant& c : kPslab)
+    if (c.qt == qt && c.b == p.b && c.phased == (p.phases > 1)) v = &c;
+  if (!v || rows < 1 || rows > p.b || x_kind < KIND_F32 || x_kind > KIND_Q8_1 || p.waves < 1 || p.waves > 12 ||
+      p.bpw_log2 < 0 || p.bpw_log2 > 2 || p.waves * bpw > nb || (nb & 1) != 0 ||
+      p.phases != (nb + p.waves * bpw - 1) / (p.waves * bpw) || p.grid < 1 ||
+      (p.phases > 1 && static_cast<int64_t>(p.grid) * PSLAB_GROUP_ROWS < N) ||
+      (reinterpret_cast<uintptr_t>(w) & 3u) != 0 || N * row_bytes > 0xFFFF0000ll) {
+    return static_cast<int>(hipErrorInvalidValue);
+  }
+  const size_t lds = pslab_lds_bytes(qt, p.b, p.waves, bpw);
+  if (lds > kMaxLds) return static_cast<int>(hipErrorInvalidValue);
+  if (lds > 64 * 1024 && !v->lds_raised[x_kind]) {
+    const hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(v->by_kind[x_kind]),
+                                             hipFuncAttributeMaxDynamicSharedMemorySize, kMaxLds);
+    if (e != hipSuccess) return static_cast<int>(e);
+    v->lds_raised[x_kind] = true;
+  }
+  GemvPslabArgs a{};
+  a.x = x; a.w = w; a.out = out; a.residual = residual;
+  a.x_kind = x_kind; a.out_kind = out_kind; a.rows = rows;
+  a.K = static_cast<int>(K); a.N = static_cast<int>(N);
+  a.waves = p.waves; a.bpw_log2 = p.bpw_log2; a.phases = p.phases;
+  a.base_rows = static_cast<int>(N / p.grid);
+  a.w_bytes = static_cast<uint32_t>((N * row_bytes + 3) & ~3ll);
+  hipLaunchKernelGGL(v->by_kind[x_kind], dim3(static_cast<unsigned>(p.grid)), dim3(p.waves * 64), lds, stream, a);
   return static_cast<int>(hipGetLastError());
 }
 
@@ -288,7 +399,6 @@ struct StreamPlan {
 };
 
 constexpr int kComputeUnits = 256;   // MI355X
-constexpr size_t kMaxLds = 160 * 1024;   // LDS of one CU
 
 // The stream form applies to K >= 4096 (a 16-block load then spans at most two
 // rows), batch <= 2, when every resident wave gets at least a few loads.
@@ -405,8 +515,8 @@ int launch_gemv(int qt, const void* x, int x_kind, const uint8_t* w, void* out, 
     int chunk = static_cast<int>(rows - r0 < 8 ? rows - r0 : 8);
     // a batch of 5..8 whose quantized activations do not fit the LDS of the stream form
     // (Q6_K, K = 17408) goes as two batches of at most 4, which do
-    if (!forced && chunk > 4 && !default_slab_plan(qt, chunk, K, N).ok && !default_stream_plan(qt, chunk, K, N).ok &&
-        default_stream_plan(qt, 4, K, N).ok) {
+    if (!forced && chunk > 4 && !default_slab_plan(qt, chunk, K, N).ok && !default_pslab_plan(qt, chunk, K, N, w).ok &&
+        !default_stream_plan(qt, chunk, K, N).ok && default_stream_plan(qt, 4, K, N).ok) {
       chunk = 4;
     }
     const int64_t next_r0 = r0 + chunk;
@@ -421,6 +531,19 @@ int launch_gemv(int qt, const void* x, int x_kind, const uint8_t* w, void* out, 
         if (rc != static_cast<int>(hipSuccess)) return rc;
         r0 = next_r0;
         continue;
+      }
+      // Q6_K batch 5..8, Q8_0 batch 3..8: the phased slab form on the int8 MFMA (measured on MI355X: at
+      // batch 3..4 the Q6_K stream form is as fast or faster)
+      if (chunk >= 5 || (qt == GGML_Q8_0 && chunk >= 3)) {
+        const PslabPlan pp = default_pslab_plan(qt, chunk, K, N, w);
+        if (pp.ok) {
+          const int rc = launch_gemv_pslab(qt, static_cast<const uint8_t*>(x) + r0 * x_row_bytes, x_kind, w,
+                                           static_cast<uint8_t*>(out) + r0 * N * out_elem, out_kind, chunk, K, N, pp,
+                                           stream);
+          if (rc != static_cast<int>(hipSuccess)) return rc;
+          r0 = next_r0;
+          continue;
+        }
       }
       const StreamPlan sp = default_stream_plan(qt, chunk, K, N);
       if (sp.ok) {
@@ -592,6 +715,32 @@ extern "C" int hipengine_gfx950_gguf_q4_k_q8_1_fused_gemv_slab_tuned(const void*
   if (rows_per_workgroup > 0) p.rows_wg = rows_per_workgroup;
   return launch_gemv_slab(x, x_kind, qweight, out, out_kind, static_cast<int>(rows), in_features, out_features, p,
                           stream);
+}
+
+extern "C" int hipengine_gfx950_gguf_q8_1_fused_gemv_pslab_tuned(int32_t ggml_type, const void* x, int32_t x_kind,
+                                                                const uint8_t* qweight, void* out, int32_t out_kind,
+                                                                int64_t rows, int64_t in_features,
+                                                                int64_t out_features, int32_t waves,
+                                                                int32_t blocks_per_wave, int32_t workgroups,
+                                                                hipStream_t stream) {
+  if (!x || !qweight || !out || x_kind < KIND_F32 || x_kind > KIND_Q8_1 || out_kind < KIND_F32 ||
+      out_kind > KIND_F16 || rows <= 0 || rows > 8 || in_features <= 0 || (in_features % QK_K) != 0 ||
+      out_features <= 0) {
+    return static_cast<int>(hipErrorInvalidValue);
+  }
+  PslabPlan p = default_pslab_plan(ggml_type, static_cast<int>(rows), in_features, out_features, qweight);
+  if (!p.ok) return static_cast<int>(hipErrorInvalidValue);
+  if (waves > 0 || blocks_per_wave > 0) {
+    const int nb = static_cast<int>(in_features / QK_K);
+    if (waves > 0) p.waves = waves;
+    if (blocks_per_wave > 0) p.bpw_log2 = blocks_per_wave == 1 ? 0 : blocks_per_wave == 2 ? 1 : blocks_per_wave == 4 ? 2 : -1;
+    if (p.bpw_log2 < 0 || p.waves > 12) return static_cast<int>(hipErrorInvalidValue);
+    p.phases = (nb + p.waves * (1 << p.bpw_log2) - 1) / (p.waves * (1 << p.bpw_log2));
+    p.grid = pslab_grid(out_features, p.phases);
+  }
+  if (workgroups > 0) p.grid = workgroups;
+  return launch_gemv_pslab(ggml_type, x, x_kind, qweight, out, out_kind, static_cast<int>(rows), in_features,
+                           out_features, p, stream);
 }
 
 // ---- fused epilogues: gate/up pair with SiLU, projection + residual -------------------

@@ -220,6 +220,21 @@ def gguf_q4_k_q8_1_fused_gemv_slab_tuned(x_ptr: int, x_kind: str, qweight_ptr: i
                     rows_per_workgroup, stream), runtime)
 
 
+def gguf_q8_1_fused_gemv_pslab_tuned(quant_key: str, x_ptr: int, x_kind: str, qweight_ptr: int, out_ptr: int,
+                                     out_kind: str, rows: int, in_features: int, out_features: int, *,
+                                     waves: int = 0, blocks_per_wave: int = 0, workgroups: int = 0, stream: int = 0,
+                                     library: ctypes.CDLL | None = None,
+                                     runtime: HipRuntime | None = None) -> None:
+    """The phased slab (int8 MFMA, K blocks dealt to the waves phase by phase) form of the fused Q6_K / Q8_0
+    GEMV with an explicit wave count, blocks per wave and phase (1, 2 or 4) and grid; 0 takes the
+    planner's (tuning sweeps and tests only)."""
+    validate_linear(rows, in_features, out_features)
+    fn = entry("hipengine_gfx950_gguf_q8_1_fused_gemv_pslab_tuned",
+               [I32, VOID, I32, VOID, VOID, I32, I64, I64, I64, I32, I32, I32, VOID], library)
+    check_launch(fn(QUANT_KEY_TO_GGML[quant_key], x_ptr, _KINDS[x_kind], qweight_ptr, out_ptr, _KINDS[out_kind], rows,
+                    in_features, out_features, waves, blocks_per_wave, workgroups, stream), runtime)
+
+
 def gguf_gemv_default_plan(quant_key: str, rows: int, in_features: int, out_features: int, *,
                            library: ctypes.CDLL | None = None) -> dict[str, int]:
     """The workgroup layout the library picks for a shape (host only)."""

@@ -253,6 +253,45 @@ def test_slab_form_q4_k(dev, rows, k, n, rpw, kind):
     _check_f32(got, O.quantize_q8_1(x), w, O.GGML_Q4_K)
 
 
+@pytest.mark.parametrize("quant,rows,k,n,waves,bpw,wgs,kind", [
+    ("gguf_q6_k", 8, 5120, 300, 0, 0, 0, "f32"),      # planner: one phase, 10 waves x 2 blocks, 1-2 rows per workgroup
+    ("gguf_q6_k", 8, 17408, 200, 0, 0, 0, "f32"),     # planner: phased (activations re-quantized per phase)
+    ("gguf_q6_k", 4, 2048, 257, 8, 1, 3, "bf16"),     # three 32-row steps with a ragged last one
+    ("gguf_q6_k", 5, 4096, 700, 6, 1, 8, "f32"),      # three phases, 87-88 rows per workgroup
+    ("gguf_q6_k", 3, 3072, 130, 6, 2, 1, "fp16"),     # one workgroup, two row groups (96 + 34)
+    ("gguf_q6_k", 8, 8192, 64, 8, 4, 2, "f32"),       # four blocks per wave
+    ("gguf_q6_k", 8, 10240, 100, 10, 2, 0, "q8_1"),   # two phases of two blocks per wave, pre-quantized activations
+    ("gguf_q6_k", 4, 5632, 50, 8, 1, 0, "f32"),       # last phase: two waves without a block
+    ("gguf_q8_0", 8, 5120, 300, 0, 0, 0, "f32"),
+    ("gguf_q8_0", 4, 4096, 100, 0, 0, 0, "bf16"),
+    ("gguf_q8_0", 6, 17408, 97, 0, 0, 0, "f32"),
+    ("gguf_q8_0", 3, 2048, 200, 8, 1, 2, "q8_1"),
+])
+def test_pslab_form(dev, quant, rows, k, n, waves, bpw, wgs, kind):
+    """The phased slab form (Q6_K / Q8_0 on the int8 MFMA): planner layouts and explicit ones - one and several
+    phases, 1/2/4 blocks per wave, several row groups per workgroup, ragged steps, the last row of the tensor."""
+    rng = np.random.default_rng(17 + rows + k + n)
+    x = rng.standard_normal((rows, k)).astype(np.float32)
+    x[0, :32] = 0.0
+    if kind == "bf16":
+        x = O.bf16_bits_to_f32(O.f32_to_bf16_bits(x))
+    elif kind == "fp16":
+        x = x.astype(np.float16).astype(np.float32)
+    w = O.random_weight(QT[quant], n, k, seed=k + n)
+    xq = O.quantize_q8_1(x)
+    xin = {"f32": x, "bf16": O.f32_to_bf16_bits(x), "fp16": x.astype(np.float16), "q8_1": xq}[kind]
+    dx, dw = dev.put(xin), dev.put(w)
+    dout = dev.empty(rows * n * 4)
+    G.gguf_q8_1_fused_gemv_pslab_tuned(quant, dx.ptr, kind, dw.ptr, dout.ptr, "f32", rows, k, n, waves=waves,
+                                       blocks_per_wave=bpw, workgroups=wgs)
+    got = dev.get(dout, np.float32, (rows, n))
+    dev.free(dx, dw, dout)
+    _check_f32(got, xq, w, QT[quant])
+    # against the float64 evaluation of the kernel's own formula, which isolates float32 summation order
+    exact = (O.gemv_q8_1_q6_k if quant == "gguf_q6_k" else O.gemv_q8_1_q8_0)(xq, w)
+    assert O.max_rel_err(got, exact) <= 1e-4
+
+
 @pytest.mark.parametrize("quant,d,waves,waves_total", [("gguf_q4_k", 3, 4, 64), ("gguf_q4_k", 3, 10, 120),
                                                       ("gguf_q6_k", 3, 12, 96), ("gguf_q8_0", 3, 8, 64)])
 def test_stream_form_explicit_layouts(dev, quant, d, waves, waves_total):
