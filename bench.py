@@ -368,9 +368,9 @@ def main() -> None:
             "q4_k_17408x5120_b2": ("q4_k", 2, 5120, 17408),
             "q4_k_17408x5120_b4": ("q4_k", 4, 5120, 17408),
             "q4_k_17408x5120_b8": ("q4_k", 8, 5120, 17408),
-            "q8_0_5120x5120_b1": ("q8_0", 1, 5120, 5120),
-            "q6_k_5120x17408_b1": ("q6_k", 1, 17408, 5120),
-            "q6_k_151936x5120_b1": ("q6_k", 1, 5120, 151936),
+            **{f"q8_0_5120x5120_b{b}": ("q8_0", b, 5120, 5120) for b in (1, 2, 4, 8)},
+            **{f"q6_k_5120x17408_b{b}": ("q6_k", b, 17408, 5120) for b in (1, 2, 4, 8)},
+            **{f"q6_k_151936x5120_b{b}": ("q6_k", b, 5120, 151936) for b in (1, 2, 4, 8)},
         }.items():
             c = h.gemv_case(quant, rows, kk, nn, steps, max(5, args.warmup // 5))
             extra[name] = {"us": round(c["event_s"] * 1e6, 2), "GB/s": round(c["bytes"] / c["event_s"] / 1e9, 1),

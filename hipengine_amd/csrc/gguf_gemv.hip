@@ -532,9 +532,9 @@ int launch_gemv(int qt, const void* x, int x_kind, const uint8_t* w, void* out, 
         r0 = next_r0;
         continue;
       }
-      // Q6_K batch 5..8, Q8_0 batch 3..8: the phased slab form on the int8 MFMA (measured on MI355X: at
-      // batch 3..4 the Q6_K stream form is as fast or faster)
-      if (chunk >= 5 || (qt == GGML_Q8_0 && chunk >= 3)) {
+      // Q6_K / Q8_0, batch 3..8: the phased slab form on the int8 MFMA (measured on MI355X: at batch
+      // 3..4 the Q6_K stream form is still ahead on a matrix as tall as an lm_head)
+      if (chunk >= 5 || (chunk >= 3 && (qt == GGML_Q8_0 || N < 32768))) {
         const PslabPlan pp = default_pslab_plan(qt, chunk, K, N, w);
         if (pp.ok) {
           const int rc = launch_gemv_pslab(qt, static_cast<const uint8_t*>(x) + r0 * x_row_bytes, x_kind, w,
@@ -776,7 +776,12 @@ extern "C" int hipengine_gfx950_gguf_gemv_residual(int32_t ggml_type, const void
     return launch_gemv_slab(x, x_kind, qweight, out, out_kind, static_cast<int>(rows), in_features, out_features, sl,
                             stream, residual);
   }
-  if (rows > 2) return static_cast<int>(hipErrorInvalidValue);
+  if (rows > 2) {
+    const PslabPlan pp = default_pslab_plan(ggml_type, static_cast<int>(rows), in_features, out_features, qweight);
+    if (!pp.ok) return static_cast<int>(hipErrorInvalidValue);
+    return launch_gemv_pslab(ggml_type, x, x_kind, qweight, out, out_kind, static_cast<int>(rows), in_features,
+                             out_features, pp, stream, residual);
+  }
   const StreamPlan sp = default_stream_plan(ggml_type, static_cast<int>(rows), in_features, out_features);
   if (!sp.ok) return static_cast<int>(hipErrorInvalidValue);
   StreamFusion f;

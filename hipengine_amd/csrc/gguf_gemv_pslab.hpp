@@ -258,67 +258,108 @@ __device__ __forceinline__ void gemv_pslab_workgroup(const GemvPslabArgs& a, uin
 #pragma unroll
       for (int v = 0; v < 16; ++v) zero16[v] = 0;
       const float d = f16_bits_to_float(load2(wl + 208));
-#pragma unroll
-      for (int h = 0; h < 2; ++h) {
-        uint2 qa[2], qb[2], qh[2];
+      // Software pipeline over the eight 32-value groups: the LDS reads of group k+1 (and of the second
+      // half's weights) are in flight while the MFMAs and the scale arithmetic of group k run.
+      // (The phased kernels hold the staging registers as well and read each group's operands when it is due.)
+      constexpr bool PIPE = !PHASED;
+      struct Wq { uint2 qa[2], qb[2], qh[2]; };
+      struct Act { uint2 xv[2]; ps_v4i cs[2]; ps_f4 xd; };
+      auto load_w = [&](int h) {
+        Wq w;
 #pragma unroll
         for (int l = 0; l < 2; ++l) {
-          qa[l] = load8(wl + 64 * h + 16 * l + 8 * g);
-          qb[l] = load8(wl + 64 * h + 32 + 16 * l + 8 * g);
-          qh[l] = load8(wl + 128 + 32 * h + 16 * l + 8 * g);
+          w.qa[l] = load8(wl + 64 * h + 16 * l + 8 * g);
+          w.qb[l] = load8(wl + 64 * h + 32 + 16 * l + 8 * g);
+          w.qh[l] = load8(wl + 128 + 32 * h + 16 * l + 8 * g);
         }
+        return w;
+      };
+      auto load_act = [&](int j32) {
+        Act t;
 #pragma unroll
-        for (int q = 0; q < 4; ++q) {
-          const int j32 = 4 * h + q;                         // 32-value group of the block
-          int dots[2][VB];
-#pragma unroll
-          for (int l = 0; l < 2; ++l) {
-            const int grp = 2 * j32 + l;                     // 16-value group: scale index
-            const Q6KQuad ux = q6k_unpack(qa[l].x, qb[l].x, qh[l].x);
-            const Q6KQuad uy = q6k_unpack(qa[l].y, qb[l].y, qh[l].y);
-            const uint32_t wx = q == 0 ? ux.g0 : q == 1 ? ux.g1 : q == 2 ? ux.g2 : ux.g3;
-            const uint32_t wy = q == 0 ? uy.g0 : q == 1 ? uy.g1 : q == 2 ? uy.g2 : uy.g3;
-            const long wop = static_cast<long>(static_cast<uint64_t>(wx) | (static_cast<uint64_t>(wy) << 32));
-            const uint2 xv = *reinterpret_cast<const uint2*>(xl + 16 * grp + 8 * g);
-            const long xop = static_cast<long>(static_cast<uint64_t>(xv.x) | (static_cast<uint64_t>(xv.y) << 32));
-            const ps_v4i cs = *reinterpret_cast<const ps_v4i*>(s16 + grp * 8 + 4 * g);   // -32 * qsum16 of rows 4g..4g+3
-            const ps_v16i r = __builtin_amdgcn_mfma_i32_32x32x16_i8(xop, wop, zero16, 0, 0, 0);
-#pragma unroll
-            for (int v = 0; v < VB; ++v) dots[l][v] = r[v] + cs[v];   // signed dot: sum x*(u - 32)
-          }
-          const ps_f4 xd4 = *reinterpret_cast<const ps_f4*>(xdp + j32 * 8 + 4 * g);   // xd of batch rows 4g..4g+3
-          const uint32_t sw = j32 < 2 ? scw.x : j32 < 4 ? scw.y : j32 < 6 ? scw.z : scw.w;
-          const int sc0 = static_cast<int>(sw << (16 - 16 * (j32 & 1) + 8)) >> 24;   // int8 scale of group 2*j32
-          const int sc1 = static_cast<int>(sw << (16 - 16 * (j32 & 1))) >> 24;       // int8 scale of group 2*j32+1
-#pragma unroll
-          for (int v = 0; v < VB; ++v) {
-            // |dot| <= 16*127*32 < 2^23 and |sc| <= 128: 24-bit multiplies, exact sum
-            const int iv = __mul24(dots[0][v], sc0) + __mul24(dots[1][v], sc1);
-            acc[v] = __builtin_fmaf(xd4[v], static_cast<float>(iv), acc[v]);
-          }
+        for (int l = 0; l < 2; ++l) {
+          t.xv[l] = *reinterpret_cast<const uint2*>(xl + 16 * (2 * j32 + l) + 8 * g);
+          t.cs[l] = *reinterpret_cast<const ps_v4i*>(s16 + (2 * j32 + l) * 8 + 4 * g);   // -32 * qsum16 of rows 4g..4g+3
         }
+        t.xd = *reinterpret_cast<const ps_f4*>(xdp + j32 * 8 + 4 * g);                   // xd of rows 4g..4g+3
+        return t;
+      };
+      Wq wq[2];
+      wq[0] = load_w(0);
+      Act act = load_act(0);
+#pragma unroll
+      for (int j32 = 0; j32 < 8; ++j32) {                   // 32-value group of the block
+        const int h = j32 >> 2, q = j32 & 3;
+        Act act_next = act;
+        if constexpr (PIPE) {
+          if (j32 + 1 < 8) act_next = load_act(j32 + 1);
+          if (j32 == 1) wq[1] = load_w(1);
+        }
+        int dots[2][VB];
+#pragma unroll
+        for (int l = 0; l < 2; ++l) {                       // 16-value group 2*j32 + l: scale index
+          const Q6KQuad ux = q6k_unpack(wq[h].qa[l].x, wq[h].qb[l].x, wq[h].qh[l].x);
+          const Q6KQuad uy = q6k_unpack(wq[h].qa[l].y, wq[h].qb[l].y, wq[h].qh[l].y);
+          const uint32_t wx = q == 0 ? ux.g0 : q == 1 ? ux.g1 : q == 2 ? ux.g2 : ux.g3;
+          const uint32_t wy = q == 0 ? uy.g0 : q == 1 ? uy.g1 : q == 2 ? uy.g2 : uy.g3;
+          const long wop = static_cast<long>(static_cast<uint64_t>(wx) | (static_cast<uint64_t>(wy) << 32));
+          const long xop = static_cast<long>(static_cast<uint64_t>(act.xv[l].x) | (static_cast<uint64_t>(act.xv[l].y) << 32));
+          const ps_v16i r = __builtin_amdgcn_mfma_i32_32x32x16_i8(xop, wop, zero16, 0, 0, 0);
+#pragma unroll
+          for (int v = 0; v < VB; ++v) dots[l][v] = r[v] + act.cs[l][v];   // signed dot: sum x*(u - 32)
+        }
+        const uint32_t sw = j32 < 2 ? scw.x : j32 < 4 ? scw.y : j32 < 6 ? scw.z : scw.w;
+        const int sc0 = static_cast<int>(sw << (16 - 16 * (j32 & 1) + 8)) >> 24;   // int8 scale of group 2*j32
+        const int sc1 = static_cast<int>(sw << (16 - 16 * (j32 & 1))) >> 24;       // int8 scale of group 2*j32+1
+#pragma unroll
+        for (int v = 0; v < VB; ++v) {
+          // |dot| <= 16*127*32 < 2^23 and |sc| <= 128: 24-bit multiplies, exact sum
+          const int iv = __mul24(dots[0][v], sc0) + __mul24(dots[1][v], sc1);
+          acc[v] = __builtin_fmaf(act.xd[v], static_cast<float>(iv), acc[v]);
+        }
+        if constexpr (!PIPE) {
+          if (j32 + 1 < 8) act_next = load_act(j32 + 1);
+          if (j32 == 3) wq[1] = load_w(1);
+        }
+        act = act_next;
       }
 #pragma unroll
       for (int v = 0; v < VB; ++v) acc[v] *= d;
     } else {
       const uint8_t* wl = stage + n * PITCH;
+      constexpr bool PIPE = !PHASED;   // as above: operands of block i+1 in flight during block i
+      struct Ops { uint4 wv; uint32_t dw; ps_v4i xop; ps_f4 xd; };
+      auto load_ops = [&](int i) {
+        Ops t;
+        t.wv = load16(wl + Q8_0_BYTES * i + 2 + 16 * g);
+        t.dw = load2(wl + Q8_0_BYTES * i);
+        t.xop = *reinterpret_cast<const ps_v4i*>(xl + 32 * i + 16 * g);
+        t.xd = *reinterpret_cast<const ps_f4*>(xdp + i * 8 + 4 * g);
+        return t;
+      };
+      ps_v16i zero16;
+#pragma unroll
+      for (int v = 0; v < 16; ++v) zero16[v] = 0;
+      Ops ops = load_ops(0);
 #pragma unroll
       for (int i = 0; i < 8; ++i) {
-        const uint4 wv = load16(wl + Q8_0_BYTES * i + 2 + 16 * g);
-        const float dw = f16_bits_to_float(load2(wl + Q8_0_BYTES * i));
-        const ps_v4i wop = ps_v4i{static_cast<int>(wv.x), static_cast<int>(wv.y), static_cast<int>(wv.z), static_cast<int>(wv.w)};
-        const ps_v4i xop = *reinterpret_cast<const ps_v4i*>(xl + 32 * i + 16 * g);
-        ps_v16i c;
-#pragma unroll
-        for (int v = 0; v < 16; ++v) c[v] = 0;
-        const ps_v16i r = __builtin_amdgcn_mfma_i32_32x32x32_i8(xop, wop, c, 0, 0, 0);
-        const ps_f4 xd4 = *reinterpret_cast<const ps_f4*>(xdp + i * 8 + 4 * g);
+        Ops ops_next = ops;
+        if constexpr (PIPE) {
+          if (i + 1 < 8) ops_next = load_ops(i + 1);
+        }
+        const float dw = f16_bits_to_float(ops.dw);
+        const ps_v4i wop = ps_v4i{static_cast<int>(ops.wv.x), static_cast<int>(ops.wv.y), static_cast<int>(ops.wv.z),
+                                  static_cast<int>(ops.wv.w)};
+        const ps_v16i r = __builtin_amdgcn_mfma_i32_32x32x32_i8(ops.xop, wop, zero16, 0, 0, 0);
 #pragma unroll
         for (int v = 0; v < VB; ++v) {
           const float tv = dw * static_cast<float>(r[v]);    // |dot| < 2^24: one rounding
-          acc[v] = __builtin_fmaf(xd4[v], tv, acc[v]);
+          acc[v] = __builtin_fmaf(ops.xd[v], tv, acc[v]);
         }
-        if (i & 1) __builtin_amdgcn_sched_barrier(0);   // at most two 16-register results in flight
+        if constexpr (!PIPE) {
+          if (i + 1 < 8) ops_next = load_ops(i + 1);
+        }
+        ops = ops_next;
       }
     }
     __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");

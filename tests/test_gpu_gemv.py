@@ -377,9 +377,10 @@ def test_pair_silu_gemv(dev, rows, kind, round_mid):
 
 
 @pytest.mark.parametrize("quant,rows,k,n,kind", [("gguf_q6_k", 1, 17408, 5120, "bf16"), ("gguf_q4_k", 2, 4096, 4096, "bf16"),
-                                                 ("gguf_q4_k", 5, 5120, 1000, "bf16"), ("gguf_q4_k", 1, 5120, 17408, "f32")])
+                                                 ("gguf_q4_k", 5, 5120, 1000, "bf16"), ("gguf_q4_k", 1, 5120, 17408, "f32"),
+                                                 ("gguf_q6_k", 8, 17408, 700, "bf16"), ("gguf_q6_k", 3, 5120, 300, "f32")])
 def test_gemv_residual(dev, quant, rows, k, n, kind):
-    """Projection + residual fused (stream and slab forms): out = round(W x) + residual in the output type,
+    """Projection + residual fused (stream, slab and phased slab forms): out = round(W x) + residual in the output type,
     bit for bit from the unfused kernel's own output."""
     rng = np.random.default_rng(31 + rows + n)
     x = rng.standard_normal((rows, k)).astype(np.float32)
