@@ -124,7 +124,7 @@ __device__ __forceinline__ void gemv_pslab_workgroup(const GemvPslabArgs& a, uin
   // ---- quantize the activations of owned blocks j0 .. j0+bpw-1 into xq / rec: 4 lanes per 32-value
   // group, 8 values per lane, 16 groups per pass; group id = (batch row, slot, sub-block)
   auto stage_x = [&](int j0) {
-    constexpr int PCH = PHASED ? 2 : 8;                 // passes whose loads are in flight together
+    constexpr int PCH = PHASED ? (QT == GGML_Q6_K ? 4 : 2) : 8;                 // passes whose loads are in flight together
     // inside the main loop the lane's positions are recomputed on every call: hoisted out of the
     // loop they would stay in registers across the MFMA code, which has none to spare
     int lane_here = lane;
