@@ -173,7 +173,7 @@ int launch_gemv_slab(const void* x, int x_kind, const uint8_t* w, void* out, int
   return static_cast<int>(hipGetLastError());
 }
 
-// ---- phased slab form (Q6_K / Q8_0 on the int8 MFMA, batch 3..8, any K) ----
+// ---- phased slab form (Q6_K / Q8_0, and Q4_K rows too long for the slab form, on the int8 MFMA; batch 3..8) ----
 
 template <int QT, int B, bool PHASED, int XK>
 __global__ void __launch_bounds__(768) gemv_pslab_kernel(GemvPslabArgs a) {
@@ -192,7 +192,9 @@ struct PslabVariant {
   PslabVariant { QT, B, P, {gemv_pslab_kernel<QT, B, P, KIND_F32>, gemv_pslab_kernel<QT, B, P, KIND_BF16>,   \
                             gemv_pslab_kernel<QT, B, P, KIND_F16>, gemv_pslab_kernel<QT, B, P, KIND_Q8_1>}, \
                  {false, false, false, false} }
-PslabVariant kPslab[] = {PSLAB_VARIANT(GGML_Q6_K, 4, false), PSLAB_VARIANT(GGML_Q6_K, 4, true),
+PslabVariant kPslab[] = {PSLAB_VARIANT(GGML_Q4_K, 4, false), PSLAB_VARIANT(GGML_Q4_K, 4, true),
+                         PSLAB_VARIANT(GGML_Q4_K, 8, false), PSLAB_VARIANT(GGML_Q4_K, 8, true),
+                         PSLAB_VARIANT(GGML_Q6_K, 4, false), PSLAB_VARIANT(GGML_Q6_K, 4, true),
                          PSLAB_VARIANT(GGML_Q6_K, 8, false), PSLAB_VARIANT(GGML_Q6_K, 8, true),
                          PSLAB_VARIANT(GGML_Q8_0, 4, false), PSLAB_VARIANT(GGML_Q8_0, 4, true),
                          PSLAB_VARIANT(GGML_Q8_0, 8, false), PSLAB_VARIANT(GGML_Q8_0, 8, true)};
@@ -203,8 +205,13 @@ struct PslabPlan {
 };
 
 size_t pslab_lds_bytes(int qt, int b, int waves, int bpw) {
-  return static_cast<size_t>(waves) *
-         (qt == GGML_Q6_K ? pslab_wave_bytes<GGML_Q6_K>(b, bpw) : pslab_wave_bytes<GGML_Q8_0>(b, bpw));
+  return static_cast<size_t>(waves) * (qt == GGML_Q6_K   ? pslab_wave_bytes<GGML_Q6_K>(b, bpw)
+                                       : qt == GGML_Q4_K ? pslab_wave_bytes<GGML_Q4_K>(b, bpw)
+                                                         : pslab_wave_bytes<GGML_Q8_0>(b, bpw));
+}
+
+int64_t pslab_row_bytes(int qt, int nb) {
+  return static_cast<int64_t>(nb) * (qt == GGML_Q6_K ? Q6_K_BYTES : qt == GGML_Q4_K ? Q4_K_BYTES : 8 * Q8_0_BYTES);
 }
 
 int pslab_grid(int64_t N, int phases) {
@@ -221,8 +228,8 @@ int pslab_grid(int64_t N, int phases) {
 PslabPlan default_pslab_plan(int qt, int rows, int64_t K, int64_t N, const void* w) {
   PslabPlan p{};
   const int nb = static_cast<int>(K / QK_K);
-  const int64_t row_bytes = static_cast<int64_t>(nb) * (qt == GGML_Q6_K ? Q6_K_BYTES : 8 * Q8_0_BYTES);
-  if ((qt != GGML_Q6_K && qt != GGML_Q8_0) || rows < 1 || rows > 8 || nb < 8 || (nb & 1) != 0 ||
+  const int64_t row_bytes = pslab_row_bytes(qt, nb);
+  if ((qt != GGML_Q4_K && qt != GGML_Q6_K && qt != GGML_Q8_0) || rows < 1 || rows > 8 || nb < 8 || (nb & 1) != 0 ||
       (reinterpret_cast<uintptr_t>(w) & 3u) != 0 || N < 1 || N * row_bytes > 0xFFFF0000ll) {
     return p;
   }
@@ -251,7 +258,7 @@ int launch_gemv_pslab(int qt, const void* x, int x_kind, const uint8_t* w, void*
                       int64_t K, int64_t N, const PslabPlan& p, hipStream_t stream, const void* residual = nullptr) {
   const int nb = static_cast<int>(K / QK_K);
   const int bpw = 1 << p.bpw_log2;
-  const int64_t row_bytes = static_cast<int64_t>(nb) * (qt == GGML_Q6_K ? Q6_K_BYTES : 8 * Q8_0_BYTES);
+  const int64_t row_bytes = pslab_row_bytes(qt, nb);
   PslabVariant* v = nullptr;
   for (PslabVariant& c : kPslab)
     if (c.qt == qt && c.b == p.b && c.phased == (p.phases > 1)) v = &c;
@@ -532,9 +539,9 @@ int launch_gemv(int qt, const void* x, int x_kind, const uint8_t* w, void* out, 
         r0 = next_r0;
         continue;
       }
-      // Q6_K / Q8_0, batch 3..8: the phased slab form on the int8 MFMA (measured on MI355X: at batch
-      // 3..4 the Q6_K stream form is still ahead on a matrix as tall as an lm_head)
-      if (chunk >= 5 || (chunk >= 3 && (qt == GGML_Q8_0 || N < 32768))) {
+      // Q6_K / Q8_0 (and Q4_K with K > 6144), batch 3..8: the phased slab form on the int8 MFMA (measured on
+      // MI355X: at batch 3..4 the Q6_K stream form is still ahead on a matrix as tall as an lm_head)
+      if (chunk >= 5 || (chunk >= 3 && (qt != GGML_Q6_K || N < 32768))) {
         const PslabPlan pp = default_pslab_plan(qt, chunk, K, N, w);
         if (pp.ok) {
           const int rc = launch_gemv_pslab(qt, static_cast<const uint8_t*>(x) + r0 * x_row_bytes, x_kind, w,

@@ -1,5 +1,5 @@
-// "Phased slab" form of the q8_1 decode GEMV for Q6_K and Q8_0 weights, batch 3..8,
-// on the int8 MFMA, for any K that is a multiple of 512.
+// "Phased slab" form of the q8_1 decode GEMV for Q6_K and Q8_0 weights (and Q4_K rows too
+// long for the slab form), batch 3..8, on the int8 MFMA, for any K that is a multiple of 512.
 //
 // Why: the v_dot4 forms do the weight unpacking once but the dot products once per
 // batch row, so at batch 8 they are bound by VALU issue (a 5120x17408 Q6_K matrix takes
@@ -71,6 +71,13 @@ struct PslabTraits<GGML_Q6_K> {
   static constexpr int REC_SLOT = 256 + 512;    // xd[8][8] floats, -32*qsum16[16][8] ints
 };
 template <>
+struct PslabTraits<GGML_Q4_K> {
+  static constexpr int BLK = Q4_K_BYTES;        // 144: 16-byte aligned rows, 9 chunks
+  static constexpr int CPR = 9;
+  static constexpr int PITCH = 144;             // 4 x 9 dwords
+  static constexpr int REC_SLOT = 256 + 256;    // xd[8][8] floats, xd*qsum32[8][8] floats
+};
+template <>
 struct PslabTraits<GGML_Q8_0> {
   static constexpr int BLK = 8 * Q8_0_BYTES;    // 272
   static constexpr int CPR = 17;
@@ -124,7 +131,7 @@ __device__ __forceinline__ void gemv_pslab_workgroup(const GemvPslabArgs& a, uin
   // ---- quantize the activations of owned blocks j0 .. j0+bpw-1 into xq / rec: 4 lanes per 32-value
   // group, 8 values per lane, 16 groups per pass; group id = (batch row, slot, sub-block)
   auto stage_x = [&](int j0) {
-    constexpr int PCH = PHASED ? (QT == GGML_Q6_K ? 4 : 2) : 8;                 // passes whose loads are in flight together
+    constexpr int PCH = PHASED ? (QT == GGML_Q8_0 ? 2 : 4) : 8;                 // passes whose loads are in flight together
     // inside the main loop the lane's positions are recomputed on every call: hoisted out of the
     // loop they would stay in registers across the MFMA code, which has none to spare
     int lane_here = lane;
@@ -181,6 +188,11 @@ __device__ __forceinline__ void gemv_pslab_workgroup(const GemvPslabArgs& a, uin
           part += dpp_i<DPP_QUAD_XOR1>(part);                // lanes 0,1: values 0..15; lanes 2,3: values 16..31
           int* s16 = reinterpret_cast<int*>(rec + slot * T::REC_SLOT + 256);
           if ((e & 1) == 0) s16[(2 * sub + (e >> 1)) * 8 + b] = -32 * part;
+        } else if constexpr (QT == GGML_Q4_K) {
+          int total = dot4(0x01010101u, packed[1], dot4(0x01010101u, packed[0], 0));
+          total += dpp_i<DPP_QUAD_XOR1>(total);
+          total += dpp_i<DPP_QUAD_XOR2>(total);
+          if (e == 0) xdp[64 + sub * 8 + b] = xd * static_cast<float>(total);
         }
       }
     }
@@ -325,6 +337,44 @@ __device__ __forceinline__ void gemv_pslab_workgroup(const GemvPslabArgs& a, uin
       }
 #pragma unroll
       for (int v = 0; v < VB; ++v) acc[v] *= d;
+    } else if constexpr (QT == GGML_Q4_K) {
+      // v_mfma_i32_32x32x32_i8 per 32-value sub-block; t = (d*sc) * float(dot), acc = fma(xd, t, acc),
+      // acc = fma(-dmin*mn, xd*qsum, acc) (the arithmetic of gguf_q4_k_gemv.hip:893-904)
+      const uint8_t* wl = stage + n * PITCH;
+      const ps_u32x4 hd = *reinterpret_cast<const ps_u32x4*>(wl);
+      const Q4KScales u = q4k_unpack_scales(hd.y, hd.z, hd.w);
+      const float d = f16_bits_to_float(hd.x & 0xFFFFu);
+      const float dmin = f16_bits_to_float(hd.x >> 16);
+      ps_v16i zero16;
+#pragma unroll
+      for (int v = 0; v < 16; ++v) zero16[v] = 0;
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        const ps_u32x4 qs = *reinterpret_cast<const ps_u32x4*>(wl + 16 + 32 * j + 16 * g);
+#pragma unroll
+        for (int half = 0; half < 2; ++half) {
+          const int sb = 2 * j + half;
+          const ps_v4i wop = half == 0
+              ? ps_v4i{static_cast<int>(q4k_low(qs.x)), static_cast<int>(q4k_low(qs.y)),
+                       static_cast<int>(q4k_low(qs.z)), static_cast<int>(q4k_low(qs.w))}
+              : ps_v4i{static_cast<int>(q4k_high(qs.x)), static_cast<int>(q4k_high(qs.y)),
+                       static_cast<int>(q4k_high(qs.z)), static_cast<int>(q4k_high(qs.w))};
+          const ps_v4i xop = *reinterpret_cast<const ps_v4i*>(xl + sb * 32 + 16 * g);
+          const ps_v16i r = __builtin_amdgcn_mfma_i32_32x32x32_i8(xop, wop, zero16, 0, 0, 0);
+          const ps_f4 xd4 = *reinterpret_cast<const ps_f4*>(xdp + sb * 8 + 4 * g);
+          const ps_f4 xs4 = *reinterpret_cast<const ps_f4*>(xdp + 64 + sb * 8 + 4 * g);
+          const uint32_t sc = ((sb < 4 ? u.sc_lo : u.sc_hi) >> (8 * (sb & 3))) & 0xFFu;
+          const uint32_t mn = ((sb < 4 ? u.mn_lo : u.mn_hi) >> (8 * (sb & 3))) & 0xFFu;
+          const float sw = d * static_cast<float>(sc);
+          const float mw = -(dmin * static_cast<float>(mn));
+#pragma unroll
+          for (int v = 0; v < VB; ++v) {
+            const float tv = sw * static_cast<float>(r[v]);   // |dot| < 2^24: one rounding
+            acc[v] = __builtin_fmaf(xd4[v], tv, acc[v]);
+            acc[v] = __builtin_fmaf(mw, xs4[v], acc[v]);
+          }
+        }
+      }
     } else {
       const uint8_t* wl = stage + n * PITCH;
       constexpr bool PIPE = !PHASED;   // as above: operands of block i+1 in flight during block i

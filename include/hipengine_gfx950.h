@@ -186,12 +186,13 @@ int hipengine_gfx950_gguf_q4_k_q8_1_fused_gemv_slab_tuned(const void* x, int32_t
                                                           int64_t in_features, int64_t out_features,
                                                           int32_t rows_per_workgroup, hipengine_stream_t stream);
 
-/* The phased slab form of the fused Q6_K / Q8_0 GEMV with an explicit layout
+/* The phased slab form of the fused Q4_K / Q6_K / Q8_0 GEMV with an explicit layout
  * (0 = the planner's choice): `waves` <= 12 waves per workgroup split K by
  * 256-value blocks, `blocks_per_wave` (1, 2 or 4) per wave and phase, on the
  * int8 MFMA; `workgroups` share the output rows.  rows <= 8, in_features a
  * multiple of 512 and >= 2048, weights 4-byte aligned and < 4 GiB.  The default
- * dispatch uses this form for batches of 3 to 8.  New here. */
+ * dispatch uses this form for batches of 3 to 8 (Q4_K: where in_features > 6144,
+ * below that its slab form).  New here. */
 int hipengine_gfx950_gguf_q8_1_fused_gemv_pslab_tuned(int32_t ggml_type, const void* x, int32_t x_kind,
                                                       const uint8_t* qweight, void* out, int32_t out_kind,
                                                       int64_t rows, int64_t in_features, int64_t out_features,

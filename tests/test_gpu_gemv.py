@@ -262,6 +262,9 @@ def test_slab_form_q4_k(dev, rows, k, n, rpw, kind):
     ("gguf_q6_k", 8, 8192, 64, 8, 4, 2, "f32"),       # four blocks per wave
     ("gguf_q6_k", 8, 10240, 100, 10, 2, 0, "q8_1"),   # two phases of two blocks per wave, pre-quantized activations
     ("gguf_q6_k", 4, 5632, 50, 8, 1, 0, "f32"),       # last phase: two waves without a block
+    ("gguf_q4_k", 8, 17408, 200, 0, 0, 0, "f32"),     # Q4_K rows too long for the slab form: phased
+    ("gguf_q4_k", 4, 5120, 131, 0, 0, 2, "bf16"),     # one phase, 65-66 rows per workgroup
+    ("gguf_q4_k", 5, 8192, 97, 8, 2, 0, "q8_1"),      # two phases of two blocks
     ("gguf_q8_0", 8, 5120, 300, 0, 0, 0, "f32"),
     ("gguf_q8_0", 4, 4096, 100, 0, 0, 0, "bf16"),
     ("gguf_q8_0", 6, 17408, 97, 0, 0, 0, "f32"),
@@ -288,7 +291,7 @@ def test_pslab_form(dev, quant, rows, k, n, waves, bpw, wgs, kind):
     dev.free(dx, dw, dout)
     _check_f32(got, xq, w, QT[quant])
     # against the float64 evaluation of the kernel's own formula, which isolates float32 summation order
-    exact = (O.gemv_q8_1_q6_k if quant == "gguf_q6_k" else O.gemv_q8_1_q8_0)(xq, w)
+    exact = {"gguf_q4_k": O.gemv_q8_1_q4_k, "gguf_q6_k": O.gemv_q8_1_q6_k, "gguf_q8_0": O.gemv_q8_1_q8_0}[quant](xq, w)
     assert O.max_rel_err(got, exact) <= 1e-4
 
 
