@@ -192,7 +192,9 @@ struct PslabVariant {
   PslabVariant { QT, B, P, {gemv_pslab_kernel<QT, B, P, KIND_F32>, gemv_pslab_kernel<QT, B, P, KIND_BF16>,   \
                             gemv_pslab_kernel<QT, B, P, KIND_F16>, gemv_pslab_kernel<QT, B, P, KIND_Q8_1>}, \
                  {false, false, false, false} }
-PslabVariant kPslab[] = {PSLAB_VARIANT(GGML_Q4_K, 4, false), PSLAB_VARIANT(GGML_Q4_K, 4, true),
+PslabVariant kPslab[] = {PSLAB_VARIANT(GGML_Q5_K, 4, false), PSLAB_VARIANT(GGML_Q5_K, 4, true),
+                         PSLAB_VARIANT(GGML_Q5_K, 8, false), PSLAB_VARIANT(GGML_Q5_K, 8, true),
+                         PSLAB_VARIANT(GGML_Q4_K, 4, false), PSLAB_VARIANT(GGML_Q4_K, 4, true),
                          PSLAB_VARIANT(GGML_Q4_K, 8, false), PSLAB_VARIANT(GGML_Q4_K, 8, true),
                          PSLAB_VARIANT(GGML_Q6_K, 4, false), PSLAB_VARIANT(GGML_Q6_K, 4, true),
                          PSLAB_VARIANT(GGML_Q6_K, 8, false), PSLAB_VARIANT(GGML_Q6_K, 8, true),
@@ -207,11 +209,15 @@ struct PslabPlan {
 size_t pslab_lds_bytes(int qt, int b, int waves, int bpw) {
   return static_cast<size_t>(waves) * (qt == GGML_Q6_K   ? pslab_wave_bytes<GGML_Q6_K>(b, bpw)
                                        : qt == GGML_Q4_K ? pslab_wave_bytes<GGML_Q4_K>(b, bpw)
+                                       : qt == GGML_Q5_K ? pslab_wave_bytes<GGML_Q5_K>(b, bpw)
                                                          : pslab_wave_bytes<GGML_Q8_0>(b, bpw));
 }
 
 int64_t pslab_row_bytes(int qt, int nb) {
-  return static_cast<int64_t>(nb) * (qt == GGML_Q6_K ? Q6_K_BYTES : qt == GGML_Q4_K ? Q4_K_BYTES : 8 * Q8_0_BYTES);
+  return static_cast<int64_t>(nb) * (qt == GGML_Q6_K   ? Q6_K_BYTES
+                                     : qt == GGML_Q4_K ? Q4_K_BYTES
+                                     : qt == GGML_Q5_K ? Q5_K_BYTES
+                                                       : 8 * Q8_0_BYTES);
 }
 
 int pslab_grid(int64_t N, int phases) {
@@ -229,7 +235,7 @@ PslabPlan default_pslab_plan(int qt, int rows, int64_t K, int64_t N, const void*
   PslabPlan p{};
   const int nb = static_cast<int>(K / QK_K);
   const int64_t row_bytes = pslab_row_bytes(qt, nb);
-  if ((qt != GGML_Q4_K && qt != GGML_Q6_K && qt != GGML_Q8_0) || rows < 1 || rows > 8 || nb < 8 || (nb & 1) != 0 ||
+  if ((qt != GGML_Q4_K && qt != GGML_Q5_K && qt != GGML_Q6_K && qt != GGML_Q8_0) || rows < 1 || rows > 8 || nb < 8 || (nb & 1) != 0 ||
       (reinterpret_cast<uintptr_t>(w) & 3u) != 0 || N < 1 || N * row_bytes > 0xFFFF0000ll) {
     return p;
   }

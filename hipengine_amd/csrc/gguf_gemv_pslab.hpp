@@ -1,5 +1,5 @@
-// "Phased slab" form of the q8_1 decode GEMV for Q6_K and Q8_0 weights (and Q4_K rows too
-// long for the slab form), batch 3..8, on the int8 MFMA, for any K that is a multiple of 512.
+// "Phased slab" form of the q8_1 decode GEMV for Q5_K, Q6_K and Q8_0 weights (and Q4_K rows
+// too long for the slab form), batch 3..8, on the int8 MFMA, for any K that is a multiple of 512.
 //
 // Why: the v_dot4 forms do the weight unpacking once but the dot products once per
 // batch row, so at batch 8 they are bound by VALU issue (a 5120x17408 Q6_K matrix takes
@@ -76,6 +76,13 @@ struct PslabTraits<GGML_Q4_K> {
   static constexpr int CPR = 9;
   static constexpr int PITCH = 144;             // 4 x 9 dwords
   static constexpr int REC_SLOT = 256 + 256;    // xd[8][8] floats, xd*qsum32[8][8] floats
+};
+template <>
+struct PslabTraits<GGML_Q5_K> {
+  static constexpr int BLK = Q5_K_BYTES;        // 176: 16-byte aligned rows, 11 chunks
+  static constexpr int CPR = 11;
+  static constexpr int PITCH = 176;             // 4 x 11 dwords
+  static constexpr int REC_SLOT = 256 + 256;    // as Q4_K
 };
 template <>
 struct PslabTraits<GGML_Q8_0> {
@@ -188,7 +195,7 @@ __device__ __forceinline__ void gemv_pslab_workgroup(const GemvPslabArgs& a, uin
           part += dpp_i<DPP_QUAD_XOR1>(part);                // lanes 0,1: values 0..15; lanes 2,3: values 16..31
           int* s16 = reinterpret_cast<int*>(rec + slot * T::REC_SLOT + 256);
           if ((e & 1) == 0) s16[(2 * sub + (e >> 1)) * 8 + b] = -32 * part;
-        } else if constexpr (QT == GGML_Q4_K) {
+        } else if constexpr (QT == GGML_Q4_K || QT == GGML_Q5_K) {
           int total = dot4(0x01010101u, packed[1], dot4(0x01010101u, packed[0], 0));
           total += dpp_i<DPP_QUAD_XOR1>(total);
           total += dpp_i<DPP_QUAD_XOR2>(total);
@@ -337,10 +344,14 @@ __device__ __forceinline__ void gemv_pslab_workgroup(const GemvPslabArgs& a, uin
       }
 #pragma unroll
       for (int v = 0; v < VB; ++v) acc[v] *= d;
-    } else if constexpr (QT == GGML_Q4_K) {
+    } else if constexpr (QT == GGML_Q4_K || QT == GGML_Q5_K) {
       // v_mfma_i32_32x32x32_i8 per 32-value sub-block; t = (d*sc) * float(dot), acc = fma(xd, t, acc),
-      // acc = fma(-dmin*mn, xd*qsum, acc) (the arithmetic of gguf_q4_k_gemv.hip:893-904)
+      // acc = fma(-dmin*mn, xd*qsum, acc) (the arithmetic of gguf_q4_k_gemv.hip:893-904).  Q5_K: the same
+      // with bit 4 of sub-block s, value l taken from bit s of qh[l] (gguf_k_gemv.hip:115-137).
+      constexpr int QS = QT == GGML_Q5_K ? 48 : 16;      // offset of the nibbles
       const uint8_t* wl = stage + n * PITCH;
+      ps_u32x4 qh = ps_u32x4{0u, 0u, 0u, 0u};
+      if constexpr (QT == GGML_Q5_K) qh = *reinterpret_cast<const ps_u32x4*>(wl + 16 + 16 * g);   // qh[16g .. 16g+15]
       const ps_u32x4 hd = *reinterpret_cast<const ps_u32x4*>(wl);
       const Q4KScales u = q4k_unpack_scales(hd.y, hd.z, hd.w);
       const float d = f16_bits_to_float(hd.x & 0xFFFFu);
@@ -350,15 +361,17 @@ __device__ __forceinline__ void gemv_pslab_workgroup(const GemvPslabArgs& a, uin
       for (int v = 0; v < 16; ++v) zero16[v] = 0;
 #pragma unroll
       for (int j = 0; j < 4; ++j) {
-        const ps_u32x4 qs = *reinterpret_cast<const ps_u32x4*>(wl + 16 + 32 * j + 16 * g);
+        const ps_u32x4 qs = *reinterpret_cast<const ps_u32x4*>(wl + QS + 32 * j + 16 * g);
 #pragma unroll
         for (int half = 0; half < 2; ++half) {
           const int sb = 2 * j + half;
-          const ps_v4i wop = half == 0
-              ? ps_v4i{static_cast<int>(q4k_low(qs.x)), static_cast<int>(q4k_low(qs.y)),
-                       static_cast<int>(q4k_low(qs.z)), static_cast<int>(q4k_low(qs.w))}
-              : ps_v4i{static_cast<int>(q4k_high(qs.x)), static_cast<int>(q4k_high(qs.y)),
-                       static_cast<int>(q4k_high(qs.z)), static_cast<int>(q4k_high(qs.w))};
+          ps_v4i wop;
+#pragma unroll
+          for (int c = 0; c < 4; ++c) {
+            uint32_t wv = half == 0 ? q4k_low(qs[c]) : q4k_high(qs[c]);
+            if constexpr (QT == GGML_Q5_K) wv |= ((qh[c] >> sb) & 0x01010101u) << 4;
+            wop[c] = static_cast<int>(wv);
+          }
           const ps_v4i xop = *reinterpret_cast<const ps_v4i*>(xl + sb * 32 + 16 * g);
           const ps_v16i r = __builtin_amdgcn_mfma_i32_32x32x32_i8(xop, wop, zero16, 0, 0, 0);
           const ps_f4 xd4 = *reinterpret_cast<const ps_f4*>(xdp + sb * 8 + 4 * g);

@@ -225,7 +225,7 @@ def gguf_q8_1_fused_gemv_pslab_tuned(quant_key: str, x_ptr: int, x_kind: str, qw
                                      waves: int = 0, blocks_per_wave: int = 0, workgroups: int = 0, stream: int = 0,
                                      library: ctypes.CDLL | None = None,
                                      runtime: HipRuntime | None = None) -> None:
-    """The phased slab (int8 MFMA, K blocks dealt to the waves phase by phase) form of the fused Q4_K / Q6_K / Q8_0
+    """The phased slab (int8 MFMA, K blocks dealt to the waves phase by phase) form of the fused Q4_K / Q5_K / Q6_K / Q8_0
     GEMV with an explicit wave count, blocks per wave and phase (1, 2 or 4) and grid; 0 takes the
     planner's (tuning sweeps and tests only)."""
     validate_linear(rows, in_features, out_features)

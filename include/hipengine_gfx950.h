@@ -186,7 +186,7 @@ int hipengine_gfx950_gguf_q4_k_q8_1_fused_gemv_slab_tuned(const void* x, int32_t
                                                           int64_t in_features, int64_t out_features,
                                                           int32_t rows_per_workgroup, hipengine_stream_t stream);
 
-/* The phased slab form of the fused Q4_K / Q6_K / Q8_0 GEMV with an explicit layout
+/* The phased slab form of the fused Q4_K / Q5_K / Q6_K / Q8_0 GEMV with an explicit layout
  * (0 = the planner's choice): `waves` <= 12 waves per workgroup split K by
  * 256-value blocks, `blocks_per_wave` (1, 2 or 4) per wave and phase, on the
  * int8 MFMA; `workgroups` share the output rows.  rows <= 8, in_features a

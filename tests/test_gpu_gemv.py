@@ -295,6 +295,29 @@ def test_pslab_form(dev, quant, rows, k, n, waves, bpw, wgs, kind):
     assert O.max_rel_err(got, exact) <= 1e-4
 
 
+@pytest.mark.parametrize("rows,k,n,waves,bpw,wgs", [(8, 5120, 300, 0, 0, 0), (4, 17408, 100, 0, 0, 0), (5, 2048, 130, 8, 1, 1)])
+def test_pslab_form_q5_k(dev, rows, k, n, waves, bpw, wgs):
+    """Q5_K in the phased slab form (one phase, several phases, two row groups); the default dispatch takes the same
+    form from batch 3 and must give the same bits."""
+    rng = np.random.default_rng(23 + rows + k)
+    x = rng.standard_normal((rows, k)).astype(np.float32)
+    w = _random_q5_k(n, k, seed=k + n)
+    xq = O.quantize_q8_1(x)
+    dx, dw = dev.put(x), dev.put(w)
+    dout, ddef = dev.empty(rows * n * 4), dev.empty(rows * n * 4)
+    G.gguf_q8_1_fused_gemv_pslab_tuned("gguf_q5_k", dx.ptr, "f32", dw.ptr, dout.ptr, "f32", rows, k, n, waves=waves,
+                                       blocks_per_wave=bpw, workgroups=wgs)
+    G.FUSED[("q5_k", "f32", "f32")](dx.ptr, dw.ptr, ddef.ptr, rows, k, n)
+    got = dev.get(dout, np.float32, (rows, n))
+    default = dev.get(ddef, np.float32, (rows, n))
+    dev.free(dx, dw, dout, ddef)
+    _check_f32(got, xq, w, O.GGML_Q5_K)
+    if waves == 0:
+        assert np.array_equal(got.view(np.uint32), default.view(np.uint32))
+    else:
+        _check_f32(default, xq, w, O.GGML_Q5_K)
+
+
 @pytest.mark.parametrize("quant,d,waves,waves_total", [("gguf_q4_k", 3, 4, 64), ("gguf_q4_k", 3, 10, 120),
                                                       ("gguf_q6_k", 3, 12, 96), ("gguf_q8_0", 3, 8, 64)])
 def test_stream_form_explicit_layouts(dev, quant, d, waves, waves_total):
