@@ -383,6 +383,8 @@ const StreamVariant kStream[] = {
     STREAM_VARIANT_BY_KIND(GGML_Q4_K, 1, 3, 2, false), STREAM_VARIANT(GGML_Q4_K, 2, 3),
     STREAM_VARIANT_BY_KIND(GGML_Q6_K, 1, 3, 2, false), STREAM_VARIANT(GGML_Q6_K, 2, 3),
     STREAM_VARIANT_BY_KIND(GGML_Q8_0, 1, 3, 2, false), STREAM_VARIANT(GGML_Q8_0, 2, 3),
+    STREAM_VARIANT_BY_KIND(GGML_Q5_K, 1, 3, 2, false), STREAM_VARIANT(GGML_Q5_K, 2, 3),
+    STREAM_VARIANT_BY_KIND(GGML_Q5_K, 1, 3, 5, true),
     STREAM_VARIANT_BY_KIND(GGML_Q4_K, 1, 3, 5, true), STREAM_VARIANT_BY_KIND(GGML_Q6_K, 1, 3, 5, true),
     STREAM_VARIANT_BY_KIND(GGML_Q8_0, 1, 3, 5, true),
     STREAM_VARIANT(GGML_Q4_K, 4, 3), STREAM_VARIANT(GGML_Q4_K, 8, 3), STREAM_VARIANT(GGML_Q6_K, 4, 3),

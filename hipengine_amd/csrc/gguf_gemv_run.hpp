@@ -211,7 +211,7 @@ __device__ __forceinline__ void gemv_run_stage_one(int x_kind, const uint32_t (&
     total += dpp_i<DPP_QUAD_XOR2>(total);
     if (e == 0) {   // sub-block sb -> record of lane q = sb>>1, slot sb&1 (+2 for the xd*qsum term)
       r[(sb >> 1) * 4 + (sb & 1)] = xd;
-      if constexpr (QT == GGML_Q4_K) r[(sb >> 1) * 4 + 2 + (sb & 1)] = xd * static_cast<float>(total);
+      if constexpr (gemv_has_mins(QT)) r[(sb >> 1) * 4 + 2 + (sb & 1)] = xd * static_cast<float>(total);
     }
   }
 }
@@ -308,7 +308,7 @@ __device__ __forceinline__ float gemv_run_block_term(const WeightRegs<GemvTraits
     const float4 rc = *reinterpret_cast<const float4*>(rec_blk + q * 4);
     float v = s.f[0] * (rc.x * static_cast<float>(dots[0]));
     v += s.f[1] * (rc.y * static_cast<float>(dots[1]));
-    if constexpr (QT == GGML_Q4_K) {
+    if constexpr (gemv_has_mins(QT)) {
       v -= s.m[0] * rc.z;
       v -= s.m[1] * rc.w;
     }

@@ -480,9 +480,10 @@ def test_gemv_from_a_gguf_file(dev, tmp_path):
     dev.free(dx)
 
 
-@pytest.mark.parametrize("rows,k,n", [(1, 5120, 300), (2, 1024, 77), (5, 2048, 64), (8, 512, 33)])
+@pytest.mark.parametrize("rows,k,n", [(1, 5120, 300), (2, 1024, 77), (5, 2048, 64), (8, 512, 33), (1, 5120, 2560),
+                                      (2, 5120, 4096), (1, 17408, 1100)])
 def test_q5_k_fused_gemv_and_block_dots(dev, rows, k, n):
-    """Q5_K (row-strided form): int32 sub-block dots bit-exact, float32 output within the parity gate of the
+    """Q5_K (row-strided, stream and phased slab forms by shape): int32 sub-block dots bit-exact, float32 output within the parity gate of the
     reference CPU GEMV on the q8_1-dequantized activations; closed-form weights of the reference tests too."""
     rng = np.random.default_rng(rows + k + n)
     x = rng.standard_normal((rows, k)).astype(np.float32)
