@@ -519,6 +519,31 @@ Plan default_plan(int qt, int rows, int64_t K, int64_t N) {
   return p;
 }
 
+// The kernel form a batch of `chunk` <= 8 rows takes, and the rows of it that go in one launch.
+enum GemvForm { FORM_ROW_STRIDED = 0, FORM_RUN = 1, FORM_STREAM = 2, FORM_SLAB = 3, FORM_PSLAB = 4 };
+
+GemvForm pick_form(int qt, int& chunk, int64_t K, int64_t N, const void* w) {
+  const SlabPlan sl = default_slab_plan(qt, chunk, K, N);
+  const PslabPlan pp = default_pslab_plan(qt, chunk, K, N, w);
+  // a batch of 5..8 whose quantized activations do not fit the LDS of any form that takes it whole
+  // goes as two batches of at most 4, which do
+  if (chunk > 4 && !sl.ok && !pp.ok && !default_stream_plan(qt, chunk, K, N).ok &&
+      default_stream_plan(qt, 4, K, N).ok) {
+    chunk = 4;
+  }
+  // Q4_K, K <= 6144: the int8 MFMA slab form wins for batches of 3 and more, and at any
+  // batch when a slab is a single 32-row step (N <= 8192); measured on MI355X
+  if (sl.ok && (chunk >= 3 || sl.rows_wg <= 32)) return FORM_SLAB;
+  // the other types (and Q4_K with K > 6144), batch 3..8: the phased slab form on the int8 MFMA (measured
+  // on MI355X: at batch 3..4 the Q6_K stream form is still ahead on a matrix as tall as an lm_head)
+  if ((chunk >= 5 || (chunk >= 3 && (qt != GGML_Q6_K || N < 32768))) && default_pslab_plan(qt, chunk, K, N, w).ok) {
+    return FORM_PSLAB;
+  }
+  if (default_stream_plan(qt, chunk, K, N).ok) return FORM_STREAM;
+  if (default_run_plan(qt, chunk, K, N).ok) return FORM_RUN;
+  return FORM_ROW_STRIDED;
+}
+
 int launch_gemv(int qt, const void* x, int x_kind, const uint8_t* w, void* out, int out_kind, int64_t rows, int64_t K,
                 int64_t N, const Plan* forced, hipStream_t stream) {
   if (!x || !w || !out || rows <= 0 || K <= 0 || N <= 0 || (K % QK_K) != 0 || K > (1 << 24) || N > (1 << 30)) {
@@ -528,56 +553,26 @@ int launch_gemv(int qt, const void* x, int x_kind, const uint8_t* w, void* out, 
   const int64_t out_elem = out_kind == KIND_F32 ? 4 : 2;
   for (int64_t r0 = 0; r0 < rows;) {
     int chunk = static_cast<int>(rows - r0 < 8 ? rows - r0 : 8);
-    // a batch of 5..8 whose quantized activations do not fit the LDS of the stream form
-    // (Q6_K, K = 17408) goes as two batches of at most 4, which do
-    if (!forced && chunk > 4 && !default_slab_plan(qt, chunk, K, N).ok && !default_pslab_plan(qt, chunk, K, N, w).ok &&
-        !default_stream_plan(qt, chunk, K, N).ok && default_stream_plan(qt, 4, K, N).ok) {
-      chunk = 4;
-    }
+    const GemvForm form = forced ? FORM_ROW_STRIDED : pick_form(qt, chunk, K, N, w);
     const int64_t next_r0 = r0 + chunk;
-    if (!forced) {
-      // Q4_K, K <= 6144: the int8 MFMA slab form wins for batches of 3 and more, and at any
-      // batch when a slab is a single 32-row step (N <= 8192); measured on MI355X
-      const SlabPlan sl = default_slab_plan(qt, chunk, K, N);
-      if (sl.ok && (chunk >= 3 || sl.rows_wg <= 32)) {
-        const int rc = launch_gemv_slab(static_cast<const uint8_t*>(x) + r0 * x_row_bytes, x_kind, w,
-                                        static_cast<uint8_t*>(out) + r0 * N * out_elem, out_kind, chunk, K, N, sl,
-                                        stream);
-        if (rc != static_cast<int>(hipSuccess)) return rc;
-        r0 = next_r0;
-        continue;
+    const void* xr = static_cast<const uint8_t*>(x) + r0 * x_row_bytes;
+    void* outr = static_cast<uint8_t*>(out) + r0 * N * out_elem;
+    if (form != FORM_ROW_STRIDED) {
+      int rc;
+      if (form == FORM_SLAB) {
+        rc = launch_gemv_slab(xr, x_kind, w, outr, out_kind, chunk, K, N, default_slab_plan(qt, chunk, K, N), stream);
+      } else if (form == FORM_PSLAB) {
+        rc = launch_gemv_pslab(qt, xr, x_kind, w, outr, out_kind, chunk, K, N, default_pslab_plan(qt, chunk, K, N, w),
+                               stream);
+      } else if (form == FORM_STREAM) {
+        rc = launch_gemv_stream(qt, xr, x_kind, w, outr, out_kind, chunk, K, N, default_stream_plan(qt, chunk, K, N),
+                                stream);
+      } else {
+        rc = launch_gemv_run(qt, xr, x_kind, w, outr, out_kind, chunk, K, N, default_run_plan(qt, chunk, K, N), stream);
       }
-      // Q6_K / Q8_0 (and Q4_K with K > 6144), batch 3..8: the phased slab form on the int8 MFMA (measured on
-      // MI355X: at batch 3..4 the Q6_K stream form is still ahead on a matrix as tall as an lm_head)
-      if (chunk >= 5 || (chunk >= 3 && (qt != GGML_Q6_K || N < 32768))) {
-        const PslabPlan pp = default_pslab_plan(qt, chunk, K, N, w);
-        if (pp.ok) {
-          const int rc = launch_gemv_pslab(qt, static_cast<const uint8_t*>(x) + r0 * x_row_bytes, x_kind, w,
-                                           static_cast<uint8_t*>(out) + r0 * N * out_elem, out_kind, chunk, K, N, pp,
-                                           stream);
-          if (rc != static_cast<int>(hipSuccess)) return rc;
-          r0 = next_r0;
-          continue;
-        }
-      }
-      const StreamPlan sp = default_stream_plan(qt, chunk, K, N);
-      if (sp.ok) {
-        const int rc = launch_gemv_stream(qt, static_cast<const uint8_t*>(x) + r0 * x_row_bytes, x_kind, w,
-                                          static_cast<uint8_t*>(out) + r0 * N * out_elem, out_kind, chunk, K, N,
-                                          sp, stream);
-        if (rc != static_cast<int>(hipSuccess)) return rc;
-        r0 = next_r0;
-        continue;
-      }
-      const RunPlan rp = default_run_plan(qt, chunk, K, N);
-      if (rp.ok) {
-        const int rc = launch_gemv_run(qt, static_cast<const uint8_t*>(x) + r0 * x_row_bytes, x_kind, w,
-                                       static_cast<uint8_t*>(out) + r0 * N * out_elem, out_kind, chunk, K, N, rp,
-                                       stream);
-        if (rc != static_cast<int>(hipSuccess)) return rc;
-        r0 = next_r0;
-        continue;
-      }
+      if (rc != static_cast<int>(hipSuccess)) return rc;
+      r0 = next_r0;
+      continue;
     }
     Plan p = forced ? *forced : default_plan(qt, chunk, K, N);
     if (forced) p.b = batch_bucket(chunk);
@@ -676,6 +671,18 @@ extern "C" int hipengine_gfx950_gguf_gemv_default_plan(int32_t ggml_type, int64_
   }
   const Plan p = default_plan(ggml_type, static_cast<int>(rows < 8 ? rows : 8), in_features, out_features);
   plan5[0] = p.b; plan5[1] = p.r; plan5[2] = p.cb; plan5[3] = p.ks; plan5[4] = p.nrg;
+  return static_cast<int>(hipSuccess);
+}
+
+extern "C" int hipengine_gfx950_gguf_gemv_default_form(int32_t ggml_type, int64_t rows, int64_t in_features,
+                                                       int64_t out_features, int32_t* form2) {
+  if (!form2 || rows <= 0 || in_features <= 0 || (in_features % QK_K) != 0 || out_features <= 0 ||
+      !find_variant(ggml_type, 1, 1, 1)) {
+    return static_cast<int>(hipErrorInvalidValue);
+  }
+  int chunk = static_cast<int>(rows < 8 ? rows : 8);
+  form2[0] = static_cast<int32_t>(pick_form(ggml_type, chunk, in_features, out_features, nullptr));
+  form2[1] = chunk;
   return static_cast<int>(hipSuccess);
 }
 

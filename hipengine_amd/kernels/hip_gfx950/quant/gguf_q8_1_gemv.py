@@ -244,6 +244,18 @@ def gguf_gemv_default_plan(quant_key: str, rows: int, in_features: int, out_feat
     return dict(zip(("batch_bucket", "rows_per_lane", "blocks_per_wave", "k_slices", "row_groups"), plan))
 
 
+GEMV_FORMS = ("row_strided", "run", "stream", "slab", "phased_slab")
+
+
+def gguf_gemv_default_form(quant_key: str, rows: int, in_features: int, out_features: int, *,
+                           library: ctypes.CDLL | None = None) -> tuple[str, int]:
+    """The kernel form the default dispatch takes for a shape and the batch rows of its first launch (host only)."""
+    form = (ctypes.c_int32 * 2)()
+    fn = entry("hipengine_gfx950_gguf_gemv_default_form", [I32, I64, I64, I64, ctypes.POINTER(ctypes.c_int32)], library)
+    check_launch(fn(QUANT_KEY_TO_GGML[quant_key], rows, in_features, out_features, form), None)
+    return GEMV_FORMS[form[0]], int(form[1])
+
+
 def register_kernels(backend: str = "hip_gfx950", *, replace: bool = False) -> None:
     for (act, out), fn in PAIR_SILU.items():
         register(KernelKey(backend, "linear", "gguf_q4_k", f"dual_silu_gemv_{act}_{out}_out"), fn, replace=replace)

@@ -204,6 +204,13 @@ int hipengine_gfx950_gguf_q8_1_fused_gemv_pslab_tuned(int32_t ggml_type, const v
 int hipengine_gfx950_gguf_gemv_default_plan(int32_t ggml_type, int64_t rows, int64_t in_features,
                                             int64_t out_features, int32_t* plan5);
 
+/* Host only: the kernel form the default dispatch takes for the first launch of a
+ * batch, as {form, rows in that launch}: form 0 row-strided, 1 run, 2 stream,
+ * 3 slab (Q4_K on the int8 MFMA), 4 phased slab (int8 MFMA).  Weights are assumed
+ * 4-byte aligned.  New here. */
+int hipengine_gfx950_gguf_gemv_default_form(int32_t ggml_type, int64_t rows, int64_t in_features,
+                                            int64_t out_features, int32_t* form2);
+
 /* ------------------------------------------------------------------------
  * MMQ prefill GEMM on int8 MFMA
  *   out[m, n] = sum_k W[n, k] * x[m, k],  x pre-quantized to q8_1 (128-value blocks)
