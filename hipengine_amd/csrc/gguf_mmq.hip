@@ -43,7 +43,7 @@ __device__ __forceinline__ void store_tile(const MmqArgs& a, const float (&acc)[
 }
 
 template <bool PREFETCH>
-__global__ void __launch_bounds__(THREADS, (PREFETCH ? 2 : 3)) mmq_q4_k_ds4_kernel(MmqArgs a) {
+__global__ void __launch_bounds__(THREADS, 2) mmq_q4_k_ds4_kernel(MmqArgs a) {
   extern __shared__ __align__(16) uint8_t smem_raw[];
   DenseQ4::Smem& s = *reinterpret_cast<DenseQ4::Smem*>(smem_raw);
   const int m0 = blockIdx.x * BM, n0 = blockIdx.y * BN;
@@ -194,6 +194,9 @@ __global__ void __launch_bounds__(THREADS, 2) mmq_q6_k_d4s4_kernel(MmqArgs a) {
     __syncthreads();
     if (step + 1 < steps) q6_step_load(a, step + 1, m0, n0, w_row_bytes, x_row_bytes, tid, regs);
 
+    v16i ci;
+#pragma unroll
+    for (int v = 0; v < 16; ++v) ci[v] = static_cast<int>(MAGIC_BITS);
 #pragma unroll
     for (int sl = 0; sl < 4; ++sl) {            // 32 activation values share one scale
       long wop[2][2];                            // [n tile][16-value group]
@@ -202,34 +205,45 @@ __global__ void __launch_bounds__(THREADS, 2) mmq_q6_k_d4s4_kernel(MmqArgs a) {
 #pragma unroll
         for (int t = 0; t < 2; ++t)
           wop[nt][t] = *reinterpret_cast<const long*>(s.w8 + (wn * 64 + nt * 32 + lc) * W6_STRIDE + 32 * sl + 16 * t + 8 * g);
+      long xop[2][2];                            // [m tile][16-value group]
 #pragma unroll
       for (int mt = 0; mt < 2; ++mt) {
         const uint8_t* ap = s.xa + (wm * 64 + mt * 32 + lc) * A6_STRIDE + 32 + 32 * sl + 8 * g;
-        const long xop0 = *reinterpret_cast<const long*>(ap);
-        const long xop1 = *reinterpret_cast<const long*>(ap + 16);
+        xop[mt][0] = *reinterpret_cast<const long*>(ap);
+        xop[mt][1] = *reinterpret_cast<const long*>(ap + 16);
+      }
+      // Software pipeline over the four (m tile, n tile) pairs: the two MFMAs of pair i+1 are issued before
+      // the scale arithmetic of pair i.
+      struct Dots { v16i d0, d1; };
+      auto issue = [&](int i) {
+        const int mt = i >> 1, nt = i & 1;
+        Dots r;
+        r.d0 = __builtin_amdgcn_mfma_i32_32x32x16_i8(xop[mt][0], wop[nt][0], ci, 0, 0, 0);
+        r.d1 = __builtin_amdgcn_mfma_i32_32x32x16_i8(xop[mt][1], wop[nt][1], ci, 0, 0, 0);
+        return r;
+      };
+      Dots cur = issue(0);
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        const int mt = i >> 1, nt = i & 1;
+        Dots next = cur;
+        if (i + 1 < 4) next = issue(i + 1);
         float xdv[16];
 #pragma unroll
         for (int j = 0; j < 4; ++j) {
           const float4 t = *reinterpret_cast<const float4*>(&s.xd[sl][wm * 64 + mt * 32 + 8 * j + 4 * g]);
           xdv[4 * j] = t.x; xdv[4 * j + 1] = t.y; xdv[4 * j + 2] = t.z; xdv[4 * j + 3] = t.w;
         }
+        const int col = wn * 64 + nt * 32 + lc;
+        const float s0 = s.sw[2 * sl][col], c0 = s.cw[2 * sl][col];
+        const float s1 = s.sw[2 * sl + 1][col], c1 = s.cw[2 * sl + 1][col];
 #pragma unroll
-        for (int nt = 0; nt < 2; ++nt) {
-          const int col = wn * 64 + nt * 32 + lc;
-          const float s0 = s.sw[2 * sl][col], c0 = s.cw[2 * sl][col];
-          const float s1 = s.sw[2 * sl + 1][col], c1 = s.cw[2 * sl + 1][col];
-          v16i ci;
-#pragma unroll
-          for (int v = 0; v < 16; ++v) ci[v] = static_cast<int>(MAGIC_BITS);
-          const v16i d0 = __builtin_amdgcn_mfma_i32_32x32x16_i8(xop0, wop[nt][0], ci, 0, 0, 0);
-          const v16i d1 = __builtin_amdgcn_mfma_i32_32x32x16_i8(xop1, wop[nt][1], ci, 0, 0, 0);
-#pragma unroll
-          for (int v = 0; v < 16; ++v) {
-            const float t0 = __builtin_fmaf(bits_to_float(static_cast<uint32_t>(d0[v])), s0, c0);   // s0 * dot0, rounded once
-            const float t1 = __builtin_fmaf(bits_to_float(static_cast<uint32_t>(d1[v])), s1, c1);
-            acc[nt][mt][v] = __builtin_fmaf(xdv[v], t0 + t1, acc[nt][mt][v]);
-          }
+        for (int v = 0; v < 16; ++v) {
+          const float t0 = __builtin_fmaf(bits_to_float(static_cast<uint32_t>(cur.d0[v])), s0, c0);   // s0 * dot0, rounded once
+          const float t1 = __builtin_fmaf(bits_to_float(static_cast<uint32_t>(cur.d1[v])), s1, c1);
+          acc[nt][mt][v] = __builtin_fmaf(xdv[v], t0 + t1, acc[nt][mt][v]);
         }
+        cur = next;
       }
     }
     __syncthreads();

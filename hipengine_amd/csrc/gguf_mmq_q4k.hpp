@@ -150,6 +150,9 @@ struct Q4Tile {
   static __device__ __forceinline__ void compute(const Smem& s, int step, int wm, int wn, int lc, int g,
                                                  float (&acc)[NT][MT][16]) {
     const int h = step & 1;
+    v16i c0;
+#pragma unroll
+    for (int v = 0; v < 16; ++v) c0[v] = static_cast<int>(MMQ_MAGIC_BITS);
 #pragma unroll
     for (int sp = 0; sp < 2; ++sp) {
       v4i wlo[NT], whi[NT];
@@ -162,34 +165,56 @@ struct Q4Tile {
         whi[nt] = v4i{static_cast<int>(q4k_high(qs.x)), static_cast<int>(q4k_high(qs.y)),
                       static_cast<int>(q4k_high(qs.z)), static_cast<int>(q4k_high(qs.w))};
       }
+      // The 2*MT*NT MFMAs of this nibble pair, software-pipelined: the MFMA of tile i+1 is issued
+      // before the 32 scale FMAs of tile i, so the matrix pipe works while the VALU does.
+      constexpr int TILES = 2 * MT * NT;          // tile i: half = i / (MT*NT), mt = (i / NT) % MT, nt = i % NT
+      v4i xop[2][MT];
 #pragma unroll
-      for (int half = 0; half < 2; ++half) {
-        const int sl = 2 * sp + half;      // sub-block within the step
-        const int sb = 4 * h + sl;         // sub-block within the Q4_K block
+      for (int half = 0; half < 2; ++half)
 #pragma unroll
-        for (int mt = 0; mt < MT; ++mt) {
-          const int rbase = (wm * MT + mt) * 32;
-          const v4i xop = *reinterpret_cast<const v4i*>(s.xa + (rbase + lc) * A_STRIDE + 16 + sl * 32 + 16 * g);
-          float xdv[16];
+        for (int mt = 0; mt < MT; ++mt)
+          xop[half][mt] = *reinterpret_cast<const v4i*>(s.xa + ((wm * MT + mt) * 32 + lc) * A_STRIDE + 16 +
+                                                        (2 * sp + half) * 32 + 16 * g);
+      auto issue = [&](int i) {
+        const int half = i / (MT * NT), mt = (i / NT) % MT, nt = i % NT;
+        return __builtin_amdgcn_mfma_i32_32x32x32_i8(xop[half][mt], half ? whi[nt] : wlo[nt], c0, 0, 0, 0);
+      };
+      // per (half, mt) pair: the activation scales of the lane's 16 rows and the column constants of its NT tiles
+      // (reading them a pair ahead costs 20 registers and measured no faster)
+      struct PairOps { float xdv[16]; float sw[NT], cw[NT]; };
+      auto load_pair = [&](int pr) {
+        const int half = pr / MT, mt = pr % MT;
+        const int sl = 2 * sp + half, sb = 4 * h + sl;
+        const int rbase = (wm * MT + mt) * 32;
+        PairOps o;
 #pragma unroll
-          for (int j = 0; j < 4; ++j) {
-            const float4 t = *reinterpret_cast<const float4*>(&s.xd[sl][rbase + 8 * j + 4 * g]);
-            xdv[4 * j] = t.x; xdv[4 * j + 1] = t.y; xdv[4 * j + 2] = t.z; xdv[4 * j + 3] = t.w;
+        for (int j = 0; j < 4; ++j) {
+          const float4 t = *reinterpret_cast<const float4*>(&s.xd[sl][rbase + 8 * j + 4 * g]);
+          o.xdv[4 * j] = t.x; o.xdv[4 * j + 1] = t.y; o.xdv[4 * j + 2] = t.z; o.xdv[4 * j + 3] = t.w;
+        }
+#pragma unroll
+        for (int nt = 0; nt < NT; ++nt) {
+          const int col = (wn * NT + nt) * 32 + lc;
+          o.sw[nt] = s.sw[sb][col]; o.cw[nt] = s.cw[sb][col];
+        }
+        return o;
+      };
+      v16i dcur = issue(0);
+#pragma unroll
+      for (int pr = 0; pr < 2 * MT; ++pr) {
+        const int mt = pr % MT;
+        const PairOps ops = load_pair(pr);
+#pragma unroll
+        for (int nt = 0; nt < NT; ++nt) {
+          const int i = pr * NT + nt;
+          v16i dnext = dcur;
+          if (i + 1 < TILES) dnext = issue(i + 1);
+#pragma unroll
+          for (int v = 0; v < 16; ++v) {
+            const float t = __builtin_fmaf(bits_to_float(static_cast<uint32_t>(dcur[v])), ops.sw[nt], ops.cw[nt]);   // = sw * dot, rounded once
+            acc[nt][mt][v] = __builtin_fmaf(ops.xdv[v], t, acc[nt][mt][v]);
           }
-#pragma unroll
-          for (int nt = 0; nt < NT; ++nt) {
-            const int col = (wn * NT + nt) * 32 + lc;
-            const float sw = s.sw[sb][col], cw = s.cw[sb][col];
-            v16i c0;
-#pragma unroll
-            for (int v = 0; v < 16; ++v) c0[v] = static_cast<int>(MMQ_MAGIC_BITS);
-            const v16i d = __builtin_amdgcn_mfma_i32_32x32x32_i8(xop, half ? whi[nt] : wlo[nt], c0, 0, 0, 0);
-#pragma unroll
-            for (int v = 0; v < 16; ++v) {
-              const float t = __builtin_fmaf(bits_to_float(static_cast<uint32_t>(d[v])), sw, cw);   // = sw * dot, rounded once
-              acc[nt][mt][v] = __builtin_fmaf(xdv[v], t, acc[nt][mt][v]);
-            }
-          }
+          dcur = dnext;
         }
       }
     }
