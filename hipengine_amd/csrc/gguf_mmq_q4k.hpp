@@ -57,8 +57,8 @@ struct Q4Tile {
   struct Smem {
     uint8_t xa[BM * A_STRIDE];   // DS4 blocks of the step, as stored
     uint8_t wq[BN * W_STRIDE];   // 64 nibble bytes per column
-    float sw[8][BN];             // d*sc per sub-block of the current Q4_K block, by column
-    float cw[8][BN];             // -MAGIC * sw
+    float sw[4][BN];             // d*sc of the four sub-blocks of the current K step, by column
+    float cw[4][BN];             // -MAGIC * sw
     float xd[4][BM];             // activation scale per sub-block of the step, by row
     float dmin[BN];
     _Float16 mnh[BN][8];         // 6-bit mins as fp16
@@ -121,17 +121,20 @@ struct Q4Tile {
       const int item = tid + i * THREADS;
       const u32x4 ph = r.ph[i];
       if (item < BN) {
+        const Q4KScales u = q4k_unpack_scales(ph.y, ph.z, ph.w);
+        const float d = f16_bits_to_float(ph.x & 0xFFFFu);
+        const uint32_t scw = h == 0 ? u.sc_lo : u.sc_hi;         // the step's four sub-blocks
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+          const float sw = d * static_cast<float>((scw >> (8 * j)) & 0xFFu);
+          s.sw[j][item] = sw;
+          s.cw[j][item] = -MMQ_MAGIC * sw;
+        }
         if (h == 0) {
-          const Q4KScales u = q4k_unpack_scales(ph.y, ph.z, ph.w);
-          const float d = f16_bits_to_float(ph.x & 0xFFFFu);
           s.dmin[item] = f16_bits_to_float(ph.x >> 16);
 #pragma unroll
           for (int j = 0; j < 8; ++j) {
-            const uint32_t sc = ((j < 4 ? u.sc_lo : u.sc_hi) >> (8 * (j & 3))) & 0xFFu;
             const uint32_t mn = ((j < 4 ? u.mn_lo : u.mn_hi) >> (8 * (j & 3))) & 0xFFu;
-            const float sw = d * static_cast<float>(sc);
-            s.sw[j][item] = sw;
-            s.cw[j][item] = -MMQ_MAGIC * sw;
             s.mnh[item][j] = static_cast<_Float16>(static_cast<float>(mn));
           }
         }
@@ -184,7 +187,7 @@ struct Q4Tile {
       struct PairOps { float xdv[16]; float sw[NT], cw[NT]; };
       auto load_pair = [&](int pr) {
         const int half = pr / MT, mt = pr % MT;
-        const int sl = 2 * sp + half, sb = 4 * h + sl;
+        const int sl = 2 * sp + half;
         const int rbase = (wm * MT + mt) * 32;
         PairOps o;
 #pragma unroll
@@ -195,7 +198,7 @@ struct Q4Tile {
 #pragma unroll
         for (int nt = 0; nt < NT; ++nt) {
           const int col = (wn * NT + nt) * 32 + lc;
-          o.sw[nt] = s.sw[sb][col]; o.cw[nt] = s.cw[sb][col];
+          o.sw[nt] = s.sw[sl][col]; o.cw[nt] = s.cw[sl][col];
         }
         return o;
       };
