@@ -42,19 +42,55 @@ __global__ void __launch_bounds__(1024) moe_count_prefix_kernel(const int64_t* _
   __shared__ int totals[2];
   for (int e = threadIdx.x; e < num_experts; e += 1024) cnt[e] = 0;
   __syncthreads();
-  for (int64_t i = threadIdx.x; i < lanes; i += 1024) {
-    const int64_t e = selected[i];
-    if (e >= 0 && e < num_experts) atomicAdd(&cnt[e], 1);
+  // eight loads in flight per thread: the loop is otherwise a chain of global-memory round trips
+  for (int64_t i0 = threadIdx.x; i0 < lanes; i0 += 8 * 1024) {
+    int64_t e[8];
+#pragma unroll
+    for (int u = 0; u < 8; ++u) {
+      const int64_t i = i0 + u * 1024;
+      e[u] = i < lanes ? selected[i] : -1;
+    }
+#pragma unroll
+    for (int u = 0; u < 8; ++u)
+      if (e[u] >= 0 && e[u] < num_experts) atomicAdd(&cnt[static_cast<int>(e[u])], 1);
   }
   __syncthreads();
-  if (threadIdx.x == 0) {
-    int offset = 0, active = 0;
-    for (int e = 0; e < num_experts; ++e) {
-      const int c = cnt[e];
-      cnt[e] = offset;
-      if (c > 0) { act[active++] = e; offset += c; }
+  {
+    // exclusive prefix of the counts and rank among the non-empty experts, over the whole workgroup:
+    // PER consecutive experts per thread, a shuffle scan per wave, the wave totals through LDS
+    // (a single thread walking 256 counters in LDS costs ~10 us of read latency)
+    constexpr int PER = MAX_EXPERTS / 1024;
+    __shared__ int wsum[16], wnz[16];
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    int c[PER], sum = 0, nz = 0;
+#pragma unroll
+    for (int k = 0; k < PER; ++k) {
+      const int e = tid * PER + k;
+      c[k] = e < num_experts ? cnt[e] : 0;
+      sum += c[k];
+      nz += c[k] > 0 ? 1 : 0;
     }
-    totals[0] = offset; totals[1] = active;
+    int isum = sum, inz = nz;
+#pragma unroll
+    for (int off = 1; off < 64; off <<= 1) {
+      const int t = __shfl_up(isum, off), u = __shfl_up(inz, off);
+      if (lane >= off) { isum += t; inz += u; }
+    }
+    if (lane == 63) { wsum[wave] = isum; wnz[wave] = inz; }
+    __syncthreads();
+    int base = 0, base_nz = 0;
+    for (int w = 0; w < wave; ++w) { base += wsum[w]; base_nz += wnz[w]; }
+    int offset = base + isum - sum, rank = base_nz + inz - nz;
+#pragma unroll
+    for (int k = 0; k < PER; ++k) {
+      const int e = tid * PER + k;
+      if (e < num_experts) {
+        cnt[e] = offset;
+        if (c[k] > 0) act[rank++] = e;
+        offset += c[k];
+      }
+    }
+    if (tid == 1023) { totals[0] = base + isum; totals[1] = base_nz + inz; }
   }
   __syncthreads();
   for (int e = threadIdx.x; e < num_experts; e += 1024) expert_start[e] = cnt[e];
@@ -83,9 +119,12 @@ __global__ void __launch_bounds__(1024) moe_place_kernel(const int64_t* __restri
   if (count <= 0) return;
   const int lane_id = threadIdx.x & 63, wave = threadIdx.x >> 6;
   int running = 0, buf = 0;
+  // the selection of the next chunk is loaded before this chunk's barrier
+  int64_t sel_next = threadIdx.x < lanes ? selected[threadIdx.x] : -1;
   for (int64_t chunk = 0; chunk < lanes && running < count; chunk += 1024, buf ^= 1) {
     const int64_t lane = chunk + threadIdx.x;
-    const bool flag = lane < lanes && selected[lane] == e;
+    const bool flag = lane < lanes && sel_next == e;
+    sel_next = lane + 1024 < lanes ? selected[lane + 1024] : -1;
     const unsigned long long ballot = __ballot(flag);
     const int before = __popcll(ballot & ((1ull << lane_id) - 1ull));
     if (lane_id == 0) wave_cnt[buf][wave] = __popcll(ballot);
@@ -136,14 +175,34 @@ __global__ void __launch_bounds__(256) moe_tile_map_kernel(const int64_t* __rest
   }
   for (int64_t i = threadIdx.x; i < tile_capacity; i += 256) tile_expert[i] = -1;
   __syncthreads();
-  if (threadIdx.x == 0) {
-    int offset = 0;
-    for (int e = 0; e < num_experts; ++e) {
-      const int p = start[e];
-      start[e] = offset;
-      offset += p;
+  {
+    constexpr int PER = MAX_EXPERTS / 256;   // consecutive experts per thread
+    __shared__ int wsum[4];
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    int c[PER], sum = 0;
+#pragma unroll
+    for (int k = 0; k < PER; ++k) {
+      const int e = tid * PER + k;
+      c[k] = e < num_experts ? start[e] : 0;
+      sum += c[k];
     }
-    start[num_experts] = offset;
+    int isum = sum;
+#pragma unroll
+    for (int off = 1; off < 64; off <<= 1) {
+      const int t = __shfl_up(isum, off);
+      if (lane >= off) isum += t;
+    }
+    if (lane == 63) wsum[wave] = isum;
+    __syncthreads();
+    int base = 0;
+    for (int w = 0; w < wave; ++w) base += wsum[w];
+    int offset = base + isum - sum;
+#pragma unroll
+    for (int k = 0; k < PER; ++k) {
+      const int e = tid * PER + k;
+      if (e < num_experts) { start[e] = offset; offset += c[k]; }
+    }
+    if (tid == 255) start[num_experts] = base + isum;
   }
   __syncthreads();
   for (int e = threadIdx.x; e <= num_experts; e += 256) tile_expert_start[e] = start[e];
