@@ -74,3 +74,13 @@ def test_abi_version_and_host_only_entry_points(library):
                      "q4_long_b8": (4, 8), "q5_b2": (2, 2), "short_k": picks["short_k"], "odd_blocks_b8": (2, 8)}
     assert picks["short_k"][0] in (0, 1)
     assert ff(12, 1, 100, 64, form) == 1
+    # argument checks come before any HIP call: null pointers and bad sizes are refused on a host without a GPU
+    ps = library.hipengine_gfx950_gguf_q8_1_fused_gemv_pslab_tuned
+    ps.argtypes = [ctypes.c_int32, ctypes.c_void_p, ctypes.c_int32, ctypes.c_void_p, ctypes.c_void_p, ctypes.c_int32,
+                   ctypes.c_int64, ctypes.c_int64, ctypes.c_int64, ctypes.c_int32, ctypes.c_int32, ctypes.c_int32,
+                   ctypes.c_void_p]
+    assert ps(14, None, 0, None, None, 0, 8, 5120, 5120, 0, 0, 0, None) == 1
+    assert ps(14, 16, 0, 16, 16, 0, 9, 5120, 5120, 0, 0, 0, None) == 1        # more than 8 batch rows
+    assert ps(14, 16, 0, 16, 16, 0, 8, 256 * 17, 5120, 0, 0, 0, None) == 1    # odd block count: not this form
+    assert ps(14, 16, 0, 18, 16, 0, 8, 5120, 5120, 0, 0, 0, None) == 1        # weights not 4-byte aligned
+    assert ps(14, 16, 0, 16, 16, 0, 8, 5120, 5120, 13, 1, 0, None) == 1       # more than 12 waves
