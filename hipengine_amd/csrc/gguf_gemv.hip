@@ -236,7 +236,7 @@ PslabPlan default_pslab_plan(int qt, int rows, int64_t K, int64_t N, const void*
   const int nb = static_cast<int>(K / QK_K);
   const int64_t row_bytes = pslab_row_bytes(qt, nb);
   if ((qt != GGML_Q4_K && qt != GGML_Q5_K && qt != GGML_Q6_K && qt != GGML_Q8_0) || rows < 1 || rows > 8 || nb < 8 || (nb & 1) != 0 ||
-      (reinterpret_cast<uintptr_t>(w) & 3u) != 0 || N < 1 || N * row_bytes > 0xFFFF0000ll) {
+      (reinterpret_cast<uintptr_t>(w) & 3u) != 0 || N < 1 || row_bytes >= (1 << 24) || N * row_bytes > 0xFFFF0000ll) {
     return p;
   }
   p.b = rows <= 4 ? 4 : 8;
@@ -272,7 +272,7 @@ int launch_gemv_pslab(int qt, const void* x, int x_kind, const uint8_t* w, void*
       p.bpw_log2 < 0 || p.bpw_log2 > 2 || p.waves * bpw > nb || (nb & 1) != 0 ||
       p.phases != (nb + p.waves * bpw - 1) / (p.waves * bpw) || p.grid < 1 ||
       (p.phases > 1 && static_cast<int64_t>(p.grid) * PSLAB_GROUP_ROWS < N) ||
-      (reinterpret_cast<uintptr_t>(w) & 3u) != 0 || N * row_bytes > 0xFFFF0000ll) {
+      (reinterpret_cast<uintptr_t>(w) & 3u) != 0 || row_bytes >= (1 << 24) || N * row_bytes > 0xFFFF0000ll) {
     return static_cast<int>(hipErrorInvalidValue);
   }
   const size_t lds = pslab_lds_bytes(qt, p.b, p.waves, bpw);
