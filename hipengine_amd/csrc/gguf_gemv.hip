@@ -147,7 +147,8 @@ SlabPlan default_slab_plan(int qt, int rows, int64_t K, int64_t N) {
 }
 
 int launch_gemv_slab(const void* x, int x_kind, const uint8_t* w, void* out, int out_kind, int rows, int64_t K,
-                     int64_t N, const SlabPlan& p, hipStream_t stream, const void* residual = nullptr) {
+                     int64_t N, const SlabPlan& p, hipStream_t stream, const void* residual = nullptr,
+                     const void* gate = nullptr) {
   const int nb = static_cast<int>(K / QK_K);
   SlabVariant* v = nullptr;
   for (SlabVariant& c : kSlab)
@@ -167,7 +168,7 @@ int launch_gemv_slab(const void* x, int x_kind, const uint8_t* w, void* out, int
     v->lds_raised[x_kind] = true;
   }
   GemvSlabArgs a{x, w, out, x_kind, out_kind, rows, static_cast<int>(K), static_cast<int>(N), p.rows_wg, p.waves,
-                 p.two_block_waves, residual};
+                 p.two_block_waves, residual, gate};
   const unsigned grid = static_cast<unsigned>((N + p.rows_wg - 1) / p.rows_wg);
   hipLaunchKernelGGL(v->by_kind[x_kind], dim3(grid), dim3(p.waves * 64), lds, stream, a);
   return static_cast<int>(hipGetLastError());
@@ -261,7 +262,8 @@ PslabPlan default_pslab_plan(int qt, int rows, int64_t K, int64_t N, const void*
 }
 
 int launch_gemv_pslab(int qt, const void* x, int x_kind, const uint8_t* w, void* out, int out_kind, int rows,
-                      int64_t K, int64_t N, const PslabPlan& p, hipStream_t stream, const void* residual = nullptr) {
+                      int64_t K, int64_t N, const PslabPlan& p, hipStream_t stream, const void* residual = nullptr,
+                      const void* gate = nullptr) {
   const int nb = static_cast<int>(K / QK_K);
   const int bpw = 1 << p.bpw_log2;
   const int64_t row_bytes = pslab_row_bytes(qt, nb);
@@ -284,7 +286,7 @@ int launch_gemv_pslab(int qt, const void* x, int x_kind, const uint8_t* w, void*
     v->lds_raised[x_kind] = true;
   }
   GemvPslabArgs a{};
-  a.x = x; a.w = w; a.out = out; a.residual = residual;
+  a.x = x; a.w = w; a.out = out; a.residual = residual; a.gate = gate;
   a.x_kind = x_kind; a.out_kind = out_kind; a.rows = rows;
   a.K = static_cast<int>(K); a.N = static_cast<int>(N);
   a.waves = p.waves; a.bpw_log2 = p.bpw_log2; a.phases = p.phases;
@@ -772,9 +774,30 @@ extern "C" int hipengine_gfx950_gguf_pair_silu_gemv(int32_t ggml_type, const voi
                                                     int32_t out_kind, int64_t rows, int64_t in_features,
                                                     int64_t out_features, int32_t round_mid, hipStream_t stream) {
   if (!x || !qweight_gate || !qweight_up || !out || x_kind < KIND_F32 || x_kind > KIND_Q8_1 || out_kind < KIND_F32 ||
-      out_kind > KIND_F16 || rows <= 0 || rows > 2 || in_features <= 0 || (in_features % QK_K) != 0 ||
+      out_kind > KIND_F16 || rows <= 0 || rows > 8 || in_features <= 0 || (in_features % QK_K) != 0 ||
       out_features <= 0) {
     return static_cast<int>(hipErrorInvalidValue);
+  }
+  if (rows > 2) {
+    // batch 3..8, on the MFMA forms: the gate projection goes to `out` (rounded to the output type by the
+    // store), the up projection's epilogue reads it back: out = silu(gate) * round(up).  That is the
+    // round_mid arithmetic, so a 16-bit output without round_mid is not taken.
+    if (!round_mid && out_kind != KIND_F32) return static_cast<int>(hipErrorInvalidValue);
+    const int r = static_cast<int>(rows);
+    const SlabPlan sl = default_slab_plan(ggml_type, r, in_features, out_features);
+    if (sl.ok) {
+      const int rc = launch_gemv_slab(x, x_kind, qweight_gate, out, out_kind, r, in_features, out_features, sl, stream);
+      if (rc != static_cast<int>(hipSuccess)) return rc;
+      return launch_gemv_slab(x, x_kind, qweight_up, out, out_kind, r, in_features, out_features, sl, stream, nullptr, out);
+    }
+    const PslabPlan pg = default_pslab_plan(ggml_type, r, in_features, out_features, qweight_gate);
+    const PslabPlan pu = default_pslab_plan(ggml_type, r, in_features, out_features, qweight_up);
+    if (!pg.ok || !pu.ok) return static_cast<int>(hipErrorInvalidValue);
+    const int rc = launch_gemv_pslab(ggml_type, x, x_kind, qweight_gate, out, out_kind, r, in_features, out_features, pg,
+                                     stream);
+    if (rc != static_cast<int>(hipSuccess)) return rc;
+    return launch_gemv_pslab(ggml_type, x, x_kind, qweight_up, out, out_kind, r, in_features, out_features, pu, stream,
+                             nullptr, out);
   }
   const StreamPlan sp = default_stream_plan(ggml_type, static_cast<int>(rows), in_features, out_features);
   if (!sp.ok) return static_cast<int>(hipErrorInvalidValue);

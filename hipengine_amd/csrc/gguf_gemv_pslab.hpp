@@ -47,6 +47,7 @@ struct GemvPslabArgs {
   const uint8_t* w;
   void* out;
   const void* residual;   // null, or [rows, N] of the output type: out = round(projection) + residual
+  const void* gate;       // null, or [rows, N] of the output type (may be `out` itself): out = silu(gate) * round(projection)
   int x_kind;
   int out_kind;
   int rows;        // batch rows, 1..B
@@ -502,6 +503,11 @@ __device__ __forceinline__ void gemv_pslab_workgroup(const GemvPslabArgs& a, uin
       for (int s = 0; s < W; ++s) v += reinterpret_cast<const float*>(smem + s * wave_bytes)[m * PSLAB_GROUP_ROWS + rl];
       const int64_t oi = static_cast<int64_t>(m) * a.N + r_begin + g0 + rl;
       if (a.residual) v = round_to_kind(v, a.out_kind) + load_scalar(a.residual, oi, a.out_kind);
+      if (a.gate) {   // the up half of a gate/up pair: the gate projection is already stored, rounded
+        const float gt = load_scalar(a.gate, oi, a.out_kind);
+        const float sig = 1.0f / (1.0f + expf(-gt));
+        v = gt * sig * round_to_kind(v, a.out_kind);
+      }
       store_scalar(a.out, oi, v, a.out_kind);
     }
     __syncthreads();

@@ -61,6 +61,7 @@ struct GemvSlabArgs {
   int waves;     // waves per workgroup
   int two_block_waves;   // waves 0..two_block_waves-1 own two K blocks each, the rest one
   const void* residual;   // null, or [rows, N] of the output type: out = round(projection) + residual
+  const void* gate;       // null, or [rows, N] of the output type (may be `out` itself): out = silu(gate) * round(projection)
 };
 
 constexpr int SLAB_MAX_ROWS = 96;
@@ -343,6 +344,11 @@ __device__ __forceinline__ void gemv_slab_q4k_workgroup(const GemvSlabArgs& a, u
     }
     const int64_t oi = static_cast<int64_t>(m) * a.N + r0 + rl;
     if (a.residual) v = round_to_kind(v, a.out_kind) + load_scalar(a.residual, oi, a.out_kind);
+    if (a.gate) {   // the up half of a gate/up pair: the gate projection is already stored, rounded (gguf_q4_k_gemv.hip:652-657)
+      const float gt = load_scalar(a.gate, oi, a.out_kind);
+      const float sig = 1.0f / (1.0f + expf(-gt));
+      v = gt * sig * round_to_kind(v, a.out_kind);
+    }
     store_scalar(a.out, oi, v, a.out_kind);
   }
 }

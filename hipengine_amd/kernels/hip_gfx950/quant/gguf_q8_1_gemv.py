@@ -143,18 +143,22 @@ def gguf_pair_silu_gemv(quant_key: str, x_ptr: int, x_kind: str, qweight_gate_pt
                         runtime: HipRuntime | None = None) -> None:
     """Dense FFN gate/up pair in one pass with SiLU*up fused: ``out = silu(gate x) * (up x)``.
     ``round_mid`` rounds gate and up to the output type first, as the unfused GEMV, GEMV, silu_mul sequence
-    does through its stored intermediates.  Raises :class:`FusedFormUnavailable` outside Q4_K / rows <= 2 /
-    stream-form shapes."""
+    does through its stored intermediates.  Rows 1-2: one launch (Q4_K, stream form).  Rows 3-8: two launches on
+    the MFMA forms, the gate projection stored to ``out`` and read back by the up projection's epilogue (any
+    type; 16-bit outputs need ``round_mid``, which is what storing the gate does).  Raises
+    :class:`FusedFormUnavailable` outside those ranges."""
     validate_linear(rows, in_features, out_features)
     validate_pointers(x_ptr=x_ptr, qweight_gate_ptr=qweight_gate_ptr, qweight_up_ptr=qweight_up_ptr, out_ptr=out_ptr)
-    if quant_key != "gguf_q4_k" or rows > 2 or in_features < 4096:
-        raise FusedFormUnavailable("pair_silu: Q4_K, rows <= 2, in_features >= 4096 only")
+    if rows > 8 or (rows <= 2 and (quant_key != "gguf_q4_k" or in_features < 4096)):
+        raise FusedFormUnavailable("pair_silu: rows <= 2 need Q4_K and in_features >= 4096; rows <= 8")
+    if rows > 2 and not round_mid and out_kind != "f32":
+        raise FusedFormUnavailable("pair_silu: rows 3-8 with a 16-bit output round the gate (round_mid)")
     fn = entry("hipengine_gfx950_gguf_pair_silu_gemv",
                [I32, VOID, I32, VOID, VOID, VOID, I32, I64, I64, I64, I32, VOID], library)
     code = fn(QUANT_KEY_TO_GGML[quant_key], x_ptr, _KINDS[x_kind], qweight_gate_ptr, qweight_up_ptr, out_ptr,
               _KINDS[out_kind], rows, in_features, out_features, int(bool(round_mid)), stream)
     if code == 1:
-        raise FusedFormUnavailable("pair_silu: out_features too small for the fused kernel")
+        raise FusedFormUnavailable("pair_silu: shape outside the fused kernels' range")
     check_launch(code, runtime)
 
 

@@ -161,8 +161,11 @@ int hipengine_gfx950_gguf_q8_1_fused_gemv_stream_tuned(int32_t ggml_type, const 
  * (arithmetic of gguf_q4_k_gemv.hip:652-657; hipEngine fuses this for its pack8 layout only,
  * hipengine_gguf_q4_k_pack8_dual_silu_gemv_bf16_bf16_out, and launch_gguf_linear_pair_silu
  * (runtime/qwen35_gguf_layer_ffn.py:519-538) falls back to the unfused sequence when no fused kernel
- * applies; so must a caller here when this returns 1).  Q4_K, rows <= 2, in_features >= 4096 and
- * out_features large enough for the stream form (a 27B FFN is).  New here. */
+ * applies; so must a caller here when this returns 1).  rows <= 2: Q4_K, in_features >= 4096 and
+ * out_features large enough for the stream form (a 27B FFN is), one launch.  rows 3..8: any of the four
+ * types, two launches on the int8 MFMA forms - the gate projection is stored to `out` and the up
+ * projection's epilogue reads it back, which is the round_mid arithmetic: a 16-bit out_kind needs
+ * round_mid != 0.  New here. */
 int hipengine_gfx950_gguf_pair_silu_gemv(int32_t ggml_type, const void* x, int32_t x_kind, const uint8_t* qweight_gate,
                                          const uint8_t* qweight_up, void* out, int32_t out_kind, int64_t rows,
                                          int64_t in_features, int64_t out_features, int32_t round_mid,

@@ -402,6 +402,43 @@ def test_pair_silu_gemv(dev, rows, kind, round_mid):
         assert O.max_rel_err(got, want) <= 1e-3 and O.cosine(got, want) >= 0.99999
 
 
+@pytest.mark.parametrize("quant,rows,k,n,kind,round_mid", [
+    ("gguf_q4_k", 8, 5120, 600, "bf16", True),      # slab form, gate stored then read by the up launch
+    ("gguf_q4_k", 4, 5120, 300, "f32", False),
+    ("gguf_q6_k", 5, 5120, 300, "bf16", True),      # phased slab, one phase
+    ("gguf_q4_k", 8, 17408, 200, "f32", False),     # phased slab, several phases
+])
+def test_pair_silu_gemv_batch_3_to_8(dev, quant, rows, k, n, kind, round_mid):
+    """Gate/up pair at batch 3..8: two launches on the MFMA forms, out = silu(stored gate) * round(up), against
+    the unfused kernels' own gate and up outputs."""
+    rng = np.random.default_rng(15 + rows + n)
+    x = rng.standard_normal((rows, k)).astype(np.float32)
+    if kind == "bf16":
+        x = O.bf16_bits_to_f32(O.f32_to_bf16_bits(x))
+    wg = O.random_weight(QT[quant], n, k, seed=21)
+    wu = O.random_weight(QT[quant], n, k, seed=22)
+    xin = x if kind == "f32" else O.f32_to_bf16_bits(x)
+    dx, dg, du = dev.put(xin), dev.put(wg), dev.put(wu)
+    esz = 4 if kind == "f32" else 2
+    dout, dgate, dup = dev.empty(rows * n * esz), dev.empty(rows * n * esz), dev.empty(rows * n * esz)
+    G.gguf_pair_silu_gemv(quant, dx.ptr, kind, dg.ptr, du.ptr, dout.ptr, kind, rows, k, n, round_mid=round_mid)
+    G.FUSED[(quant[5:], kind, kind)](dx.ptr, dg.ptr, dgate.ptr, rows, k, n)
+    G.FUSED[(quant[5:], kind, kind)](dx.ptr, du.ptr, dup.ptr, rows, k, n)
+    dt = np.float32 if kind == "f32" else np.uint16
+    got, gate, up = (dev.get(b, dt, (rows, n)) for b in (dout, dgate, dup))
+    dev.free(dx, dg, du, dout, dgate, dup)
+    if kind == "bf16":
+        got, gate, up = (O.bf16_bits_to_f32(a) for a in (got, gate, up))
+    want = (O.silu(gate) * up).astype(np.float32)
+    # the device's expf and the final rounding to the output type are the only differences
+    tol = 2.0 ** -7 if kind == "bf16" else 1e-5
+    assert np.max(np.abs(got - want)) <= tol * max(1.0, float(np.max(np.abs(want))))
+    assert O.cosine(got, want) >= 0.99999
+    if kind != "f32":
+        with pytest.raises(G.FusedFormUnavailable):
+            G.gguf_pair_silu_gemv(quant, 16, kind, 16, 16, 16, kind, rows, k, n, round_mid=False)
+
+
 @pytest.mark.parametrize("quant,rows,k,n,kind", [("gguf_q6_k", 1, 17408, 5120, "bf16"), ("gguf_q4_k", 2, 4096, 4096, "bf16"),
                                                  ("gguf_q4_k", 5, 5120, 1000, "bf16"), ("gguf_q4_k", 1, 5120, 17408, "f32"),
                                                  ("gguf_q6_k", 8, 17408, 700, "bf16"), ("gguf_q6_k", 3, 5120, 300, "f32")])
