@@ -422,6 +422,12 @@ def main() -> None:
             "frac_hbm": round(wbytes / ev_f / 1e9 / HBM_PEAK_GBS, 4),
             "unfused_3_gemv_us": round(ev_u * 1e6, 1)}
 
+        ev_f, ev_u, wbytes = h.ffn_case(8, steps, max(5, args.warmup // 5))
+        extra["ffn_27b_b8_pair_silu_and_down_residual"] = {
+            "us": round(ev_f * 1e6, 1), "launches": 3, "GB/s": round(wbytes / ev_f / 1e9, 1),
+            "frac_hbm": round(wbytes / ev_f / 1e9 / HBM_PEAK_GBS, 4),
+            "unfused_3_gemv_us": round(ev_u * 1e6, 1)}
+
         eager, replay, lbytes = h.layer_graph_case(1, max(10, steps // 4), 3)
         extra["layer_27b_b1_fused_6_launches"] = {
             "eager_us_per_layer": round(eager * 1e6, 1), "hip_graph_us_per_layer": round(replay * 1e6, 1),
