@@ -229,8 +229,8 @@ int pslab_grid(int64_t N, int phases) {
   return static_cast<int>(phases == 1 ? per_cu : (groups > per_cu ? groups : per_cu));
 }
 
-// Waves and blocks per wave: the split of K/256 blocks over W <= 12 waves x bpw in {1, 2, 4} x phases
-// that wastes the fewest block slots, preferring a single phase (activations quantized once) and more
+// Waves and blocks per wave: the split of K/256 blocks over W <= 12 waves x bpw in {1, 2, 4} slots x phases
+// that loads the four SIMDs most evenly, preferring a single phase (activations quantized once) and more
 // waves.
 PslabPlan default_pslab_plan(int qt, int rows, int64_t K, int64_t N, const void* w) {
   PslabPlan p{};
@@ -245,9 +245,14 @@ PslabPlan default_pslab_plan(int qt, int rows, int64_t K, int64_t N, const void*
   for (int waves = 12; waves >= 6; --waves) {
     for (int bl2 = 0; bl2 <= 2; ++bl2) {
       const int bpw = 1 << bl2;
-      if (waves * bpw > nb || pslab_lds_bytes(qt, p.b, waves, bpw) > kMaxLds) continue;
+      if (waves > nb || pslab_lds_bytes(qt, p.b, waves, bpw) > kMaxLds) continue;
       const int phases = (nb + waves * bpw - 1) / (waves * bpw);
-      const float score = static_cast<float>(nb) / static_cast<float>(waves * bpw * phases) -
+      // wave w owns blocks w, w + waves, ...: the SIMD (w % 4) with the most blocks sets the pace
+      int simd_blocks[4] = {0, 0, 0, 0};
+      for (int w = 0; w < waves; ++w) simd_blocks[w & 3] += (nb - w + waves - 1) / waves;
+      int worst = 0;
+      for (int v : simd_blocks) worst = v > worst ? v : worst;
+      const float score = static_cast<float>(nb) / static_cast<float>(4 * worst) -
                           0.02f * static_cast<float>(12 - waves) + (phases == 1 ? 0.05f : 0.0f) - 0.001f * bl2;
       if (score > best) {
         best = score;
@@ -271,7 +276,7 @@ int launch_gemv_pslab(int qt, const void* x, int x_kind, const uint8_t* w, void*
   for (PslabVariant& c : kPslab)
     if (c.qt == qt && c.b == p.b && c.phased == (p.phases > 1)) v = &c;
   if (!v || rows < 1 || rows > p.b || x_kind < KIND_F32 || x_kind > KIND_Q8_1 || p.waves < 1 || p.waves > 12 ||
-      p.bpw_log2 < 0 || p.bpw_log2 > 2 || p.waves * bpw > nb || (nb & 1) != 0 ||
+      p.bpw_log2 < 0 || p.bpw_log2 > 2 || p.waves > nb || (nb & 1) != 0 ||
       p.phases != (nb + p.waves * bpw - 1) / (p.waves * bpw) || p.grid < 1 ||
       (p.phases > 1 && static_cast<int64_t>(p.grid) * PSLAB_GROUP_ROWS < N) ||
       (reinterpret_cast<uintptr_t>(w) & 3u) != 0 || row_bytes >= (1 << 24) || N * row_bytes > 0xFFFF0000ll) {

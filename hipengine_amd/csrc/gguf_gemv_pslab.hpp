@@ -10,7 +10,7 @@
 //   * a workgroup owns a contiguous range of output rows and walks it in groups of up
 //     to 96 rows = 3 steps of 32;
 //   * its W waves split K by 256-value blocks: wave w owns blocks
-//     (p*W + w)*bpw + s, s < bpw, of every phase p.  With one phase (W*bpw >= K/256) the
+//     (p*bpw + s)*W + w, s < bpw, of every phase p.  With one phase (W*bpw >= K/256) the
 //     wave quantizes its K slice of the activations once into wave-private LDS and keeps
 //     it for all row groups; with several phases a workgroup has a single row group and
 //     the wave re-quantizes its bpw blocks at the start of each phase (the whole
@@ -126,9 +126,12 @@ __device__ __forceinline__ void gemv_pslab_workgroup(const GemvPslabArgs& a, uin
   if (nrows <= 0) return;   // uniform over the workgroup
 
   // blocks of this wave: owned block j is block kb_of(j); nown of them are inside K
-  auto kb_of = [&](int j) { return ((j >> bl2) * W + wave) * bpw + (j & (bpw - 1)); };
+  // (slot s of phase p is block (p*bpw + s)*W + wave: the waves take the blocks of a phase round robin, so
+  // 20 blocks over 12 waves x 2 slots give eight waves two blocks and four waves one - five per SIMD - and
+  // the blocks a wave owns are a prefix of its slots)
+  auto kb_of = [&](int j) { return j * W + wave; };
   int nown = 0;
-  for (int p = 0; p < a.phases; ++p) nown += max(0, min(bpw, nb - (p * W + wave) * bpw));
+  for (int j = 0; j < (a.phases << bl2); ++j) nown += kb_of(j) < nb ? 1 : 0;
 
   const int wave_bytes = pslab_wave_bytes<QT>(B, bpw);
   const int XQ_PITCH = bpw * 256 + 16;
