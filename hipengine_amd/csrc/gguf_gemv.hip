@@ -444,7 +444,10 @@ StreamPlan default_stream_plan(int qt, int rows, int64_t K, int64_t N) {
       if (imbalance < best - 0.1) { best = imbalance; p.waves = w; p.waves_total = static_cast<int>(wt); }
     }
   }
-  p.ok = rows <= 8 && nb >= 16 && total_loads >= 3 * static_cast<int64_t>(p.waves_total) &&
+  // every wave should get the ring's three loads; Q4_K at batch 1 still beats the slab form with two
+  // (5120 x 5120 on 10 waves per CU: 6.7 us against 7.8)
+  const int min_loads = (qt == GGML_Q4_K && p.b == 1) ? 2 : 3;
+  p.ok = rows <= 8 && nb >= 16 && total_loads >= min_loads * static_cast<int64_t>(p.waves_total) &&
          N >= p.waves_total && gemv_run_lds_bytes(qt, p.b, static_cast<int>(K)) <= kMaxLds &&
          find_stream_variant(qt, p.b, p.d) != nullptr;
   return p;
@@ -529,6 +532,16 @@ Plan default_plan(int qt, int rows, int64_t K, int64_t N) {
 // The kernel form a batch of `chunk` <= 8 rows takes, and the rows of it that go in one launch.
 enum GemvForm { FORM_ROW_STRIDED = 0, FORM_RUN = 1, FORM_STREAM = 2, FORM_SLAB = 3, FORM_PSLAB = 4 };
 
+// Q4_K, K <= 6144: the int8 MFMA slab form wins for batches of 3 and more; at batch 2 when a slab is a single
+// 32-row step (N <= 8192); at batch 1 only below 4096 rows (above, the stream form is ~1 us faster) or where
+// the stream form does not apply.  Measured on MI355X.
+bool slab_preferred(int qt, int chunk, int64_t K, int64_t N, const SlabPlan& sl) {
+  if (!sl.ok) return false;
+  if (chunk >= 3) return true;
+  if (chunk == 2) return sl.rows_wg <= 32;
+  return sl.rows_wg < 16 || (sl.rows_wg <= 32 && !default_stream_plan(qt, chunk, K, N).ok);
+}
+
 GemvForm pick_form(int qt, int& chunk, int64_t K, int64_t N, const void* w) {
   const SlabPlan sl = default_slab_plan(qt, chunk, K, N);
   const PslabPlan pp = default_pslab_plan(qt, chunk, K, N, w);
@@ -538,9 +551,7 @@ GemvForm pick_form(int qt, int& chunk, int64_t K, int64_t N, const void* w) {
       default_stream_plan(qt, 4, K, N).ok) {
     chunk = 4;
   }
-  // Q4_K, K <= 6144: the int8 MFMA slab form wins for batches of 3 and more, and at any
-  // batch when a slab is a single 32-row step (N <= 8192); measured on MI355X
-  if (sl.ok && (chunk >= 3 || sl.rows_wg <= 32)) return FORM_SLAB;
+  if (slab_preferred(qt, chunk, K, N, sl)) return FORM_SLAB;
   // the other types (and Q4_K with K > 6144), batch 3..8: the phased slab form on the int8 MFMA (measured
   // on MI355X: at batch 3..4 the Q6_K stream form is still ahead on a matrix as tall as an lm_head)
   if ((chunk >= 5 || (chunk >= 3 && (qt != GGML_Q6_K || N < 32768))) && default_pslab_plan(qt, chunk, K, N, w).ok) {
@@ -822,7 +833,7 @@ extern "C" int hipengine_gfx950_gguf_gemv_residual(int32_t ggml_type, const void
     return static_cast<int>(hipErrorInvalidValue);
   }
   const SlabPlan sl = default_slab_plan(ggml_type, static_cast<int>(rows), in_features, out_features);
-  if (sl.ok && (rows >= 3 || sl.rows_wg <= 32)) {
+  if (slab_preferred(ggml_type, static_cast<int>(rows), in_features, out_features, sl)) {
     return launch_gemv_slab(x, x_kind, qweight, out, out_kind, static_cast<int>(rows), in_features, out_features, sl,
                             stream, residual);
   }

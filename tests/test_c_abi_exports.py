@@ -66,12 +66,13 @@ def test_abi_version_and_host_only_entry_points(library):
     for name, (qt, rows, k, n) in {"c1": (12, 1, 5120, 17408), "c1_b8": (12, 8, 5120, 17408), "down_b1": (14, 1, 17408, 5120),
                                    "down_b8": (14, 8, 17408, 5120), "head_b4": (14, 4, 5120, 151936), "o_b4": (8, 4, 5120, 5120),
                                    "q4_long_b8": (12, 8, 17408, 5120), "q5_b2": (13, 2, 5120, 4096), "short_k": (12, 1, 512, 64),
-                                   "odd_blocks_b8": (14, 8, 256 * 17, 5120)}.items():
+                                   "odd_blocks_b8": (14, 8, 256 * 17, 5120), "o_q4_b1": (12, 1, 5120, 5120), "o_q4_b2": (12, 2, 5120, 5120),
+                                   "k_q4_b1": (12, 1, 5120, 1024)}.items():
         assert ff(qt, rows, k, n, form) == 0
         picks[name] = (form[0], form[1])
     # 0 row-strided, 1 run, 2 stream, 3 slab, 4 phased slab; second field: batch rows of the first launch
     assert picks == {"c1": (2, 1), "c1_b8": (3, 8), "down_b1": (2, 1), "down_b8": (4, 8), "head_b4": (2, 4), "o_b4": (4, 4),
-                     "q4_long_b8": (4, 8), "q5_b2": (2, 2), "short_k": picks["short_k"], "odd_blocks_b8": (2, 8)}
+                     "q4_long_b8": (4, 8), "q5_b2": (2, 2), "short_k": picks["short_k"], "odd_blocks_b8": (2, 8), "o_q4_b1": (2, 1), "o_q4_b2": (3, 2), "k_q4_b1": (3, 1)}
     assert picks["short_k"][0] in (0, 1)
     assert ff(12, 1, 100, 64, form) == 1
     # argument checks come before any HIP call: null pointers and bad sizes are refused on a host without a GPU
