@@ -1,7 +1,7 @@
 #!/usr/bin/env python3
 """Benchmark of the gfx950 GGUF k-quant matmul path on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-extra] [--no-cpu] [--pmc-pass]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-extra] [--no-cpu] [--pmc-pass [--pmc-shape quant,rows,K,N]]
 
 One "step" is one pass of the hot path over one batch of synthetic input: the
 fused q8_1 decode GEMV of a Q4_K 17408x5120 weight at batch 1 (the shape the
@@ -355,6 +355,9 @@ def main() -> None:
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--pmc-pass", action="store_true",
                     help="hardware-counter pass: a 256 MiB calibration copy, then the headline kernel only")
+    ap.add_argument("--pmc-shape", default="",
+                    help="with --pmc-pass: launch this GEMV case instead of the headline one, as quant,rows,K,N "
+                         "(e.g. q6_k,8,5120,151936)")
     args = ap.parse_args()
     if args.gpus != 1:
         raise SystemExit("bench.py measures one GPU: this path is single-GPU (run with --gpus 1)")
@@ -370,7 +373,11 @@ def main() -> None:
         for _ in range(3):
             copy_bytes(src.ptr, dst.ptr, nbytes)
         h.rt.device_synchronize()
-        case = h.gemv_case("q4_k", 1, k, n, max(22, min(args.steps, 44)), 0)
+        if args.pmc_shape:
+            pq, pr, pk, pn = args.pmc_shape.split(",")
+            case = h.gemv_case(pq, int(pr), int(pk), int(pn), 16, 0)
+        else:
+            case = h.gemv_case("q4_k", 1, k, n, max(22, min(args.steps, 44)), 0)
         print(json.dumps({"pmc_pass": True, "copy_bytes": nbytes, "gemv_bytes": case["bytes"], "copies": case["copies"]}))
         return
     main_case = h.gemv_case("q4_k", 1, k, n, args.steps, args.warmup, spread=True)
