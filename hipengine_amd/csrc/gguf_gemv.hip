@@ -552,9 +552,8 @@ GemvForm pick_form(int qt, int& chunk, int64_t K, int64_t N, const void* w) {
     chunk = 4;
   }
   if (slab_preferred(qt, chunk, K, N, sl)) return FORM_SLAB;
-  // the other types (and Q4_K with K > 6144), batch 3..8: the phased slab form on the int8 MFMA (measured
-  // on MI355X: at batch 3..4 the Q6_K stream form is still ahead on a matrix as tall as an lm_head)
-  if ((chunk >= 5 || (chunk >= 3 && (qt != GGML_Q6_K || N < 32768))) && default_pslab_plan(qt, chunk, K, N, w).ok) {
+  // the other types (and Q4_K with K > 6144), batch 3..8: the phased slab form on the int8 MFMA
+  if (chunk >= 3 && default_pslab_plan(qt, chunk, K, N, w).ok) {
     return FORM_PSLAB;
   }
   if (default_stream_plan(qt, chunk, K, N).ok) return FORM_STREAM;

@@ -20,9 +20,8 @@
 //     wave-private LDS and reads them back in MFMA operand order (lane (n, g) = row n,
 //     k half g).  The loads of the next unit are issued before the current one is
 //     computed.  Q6_K blocks are 210 bytes, so a block starts 0 or 2 bytes past a
-//     4-byte boundary: the loads start at the boundary (never straddling the end of the
-//     tensor; the buffer descriptor returns zeros past it) and the LDS reads add the
-//     2 bytes back, which makes them 2-byte aligned;
+//     4-byte boundary: the buffer loads start at the block (2-byte aligned loads run at
+//     full rate) so that its LDS image, and every LDS read of it, is 16-byte aligned;
 //   * Q6_K: v_mfma_i32_32x32x16_i8 per 16-value group with B = the unsigned 6-bit values;
 //     adding -32 * sum(q8 of the group) of the batch row gives the signed dot of
 //     gguf_k_gemv.hip:233-246 (a shared all-zero accumulator input: a per-instruction
@@ -217,6 +216,12 @@ __device__ __forceinline__ void gemv_pslab_workgroup(const GemvPslabArgs& a, uin
   // load and its LDS addresses by an immediate.
   const int r4 = lane / CPR, col16 = (lane - r4 * CPR) * 16;
   const bool loader = r4 < RPI;
+  // Q6_K: a 210-byte block is 13 chunks and 2 bytes (the fp16 d).  The loads start at the block itself
+  // (2-byte aligned buffer loads run at full rate; a 16-byte LDS read that is not 4-byte aligned takes a
+  // cycle per lane), and the 14th chunk is the block's last 16 bytes, [194, 210), so that no load leaves
+  // the row: its top half word, d, is stored as the first word of LDS chunk 13.
+  const bool tail13 = QT == GGML_Q6_K && col16 == 13 * 16;
+  const int goff = tail13 ? BLK - 16 : col16;
   const __amdgpu_buffer_rsrc_t wrsrc = __builtin_amdgcn_make_buffer_rsrc(const_cast<uint8_t*>(a.w), 0, a.w_bytes, 0x00020000);
   ps_u32x4 buf[NL];
   // unit (owned block j, step t) of the row group that starts at row g0 and has grows rows.  The whole
@@ -226,7 +231,7 @@ __device__ __forceinline__ void gemv_pslab_workgroup(const GemvPslabArgs& a, uin
   auto issue = [&](int j, int t, int g0, int grows) {
     const int last = min(grows - 32 * t - 1, 31);           // >= 0
     const uint32_t base = static_cast<uint32_t>(r_begin + g0 + 32 * t) * static_cast<uint32_t>(row_bytes) +
-                          (static_cast<uint32_t>(kb_of(j) * BLK) & ~3u) + static_cast<uint32_t>(col16);
+                          static_cast<uint32_t>(kb_of(j) * BLK) + static_cast<uint32_t>(goff);
     if (loader) {
       if (last == 31) {
         uint32_t off = base + static_cast<uint32_t>(__mul24(r4, row_bytes));
@@ -250,6 +255,7 @@ __device__ __forceinline__ void gemv_pslab_workgroup(const GemvPslabArgs& a, uin
       uint8_t* dst = stage + r4 * PITCH + col16;
 #pragma unroll
       for (int i = 0; i < NL; ++i) {
+        if constexpr (QT == GGML_Q6_K) buf[i].x = tail13 ? buf[i].w >> 16 : buf[i].x;
         if ((i + 1) * RPI <= 32 || i * RPI + r4 < 32) *reinterpret_cast<ps_u32x4*>(dst + i * RPI * PITCH) = buf[i];
       }
     }
@@ -274,7 +280,7 @@ __device__ __forceinline__ void gemv_pslab_workgroup(const GemvPslabArgs& a, uin
 #pragma unroll
     for (int v = 0; v < VB; ++v) acc[v] = 0.0f;
     if constexpr (QT == GGML_Q6_K) {
-      const uint8_t* wl = stage + n * PITCH + ((kb * BLK) & 2);
+      const uint8_t* wl = stage + n * PITCH;
       const int* s16 = reinterpret_cast<const int*>(rec + slot * T::REC_SLOT + 256);
       const uint4 scw = load16(wl + 192);
       ps_v16i zero16;
