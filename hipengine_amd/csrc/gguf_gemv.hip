@@ -383,19 +383,23 @@ struct StreamVariant {
   StreamVariant { QT, B, D, LONG_K, FUSE_NONE, gemv_stream_kernel<QT, B, D, S>,                           \
                   {gemv_stream_kernel<QT, B, D, S, KIND_F32>, gemv_stream_kernel<QT, B, D, S, KIND_BF16>, \
                    gemv_stream_kernel<QT, B, D, S, KIND_F16>, gemv_stream_kernel<QT, B, D, S, KIND_Q8_1>} }
-#define STREAM_VARIANT_FUSED_D(QT, B, D, S, LONG_K, FUSE) \
-  StreamVariant { QT, B, D, LONG_K, FUSE, gemv_stream_kernel<QT, B, D, S, -1, FUSE>, {nullptr, nullptr, nullptr, nullptr} }
+// fused epilogues: float32 and bf16 activations get instantiations of their own, the other kinds the generic one
+#define STREAM_VARIANT_FUSED_D(QT, B, D, S, LONG_K, FUSE)                                                        \
+  StreamVariant { QT, B, D, LONG_K, FUSE, gemv_stream_kernel<QT, B, D, S, -1, FUSE>,                              \
+                  {gemv_stream_kernel<QT, B, D, S, KIND_F32, FUSE>, gemv_stream_kernel<QT, B, D, S, KIND_BF16, FUSE>, \
+                   nullptr, nullptr} }
 #define STREAM_VARIANT_FUSED(QT, B, S, LONG_K, FUSE) STREAM_VARIANT_FUSED_D(QT, B, 3, S, LONG_K, FUSE)
 
 const StreamVariant kStream[] = {
-    STREAM_VARIANT_BY_KIND(GGML_Q4_K, 1, 3, 2, false), STREAM_VARIANT(GGML_Q4_K, 2, 3),
+    STREAM_VARIANT_BY_KIND(GGML_Q4_K, 1, 3, 2, false), STREAM_VARIANT_BY_KIND(GGML_Q4_K, 2, 3, 2, false),
     STREAM_VARIANT_BY_KIND(GGML_Q4_K, 1, 2, 2, false),
-    STREAM_VARIANT_BY_KIND(GGML_Q6_K, 1, 3, 2, false), STREAM_VARIANT(GGML_Q6_K, 2, 3),
-    STREAM_VARIANT_BY_KIND(GGML_Q8_0, 1, 3, 2, false), STREAM_VARIANT(GGML_Q8_0, 2, 3),
-    STREAM_VARIANT_BY_KIND(GGML_Q5_K, 1, 3, 2, false), STREAM_VARIANT(GGML_Q5_K, 2, 3),
+    STREAM_VARIANT_BY_KIND(GGML_Q6_K, 1, 3, 2, false), STREAM_VARIANT_BY_KIND(GGML_Q6_K, 2, 3, 2, false),
+    STREAM_VARIANT_BY_KIND(GGML_Q8_0, 1, 3, 2, false), STREAM_VARIANT_BY_KIND(GGML_Q8_0, 2, 3, 2, false),
+    STREAM_VARIANT_BY_KIND(GGML_Q5_K, 1, 3, 2, false), STREAM_VARIANT_BY_KIND(GGML_Q5_K, 2, 3, 2, false),
     STREAM_VARIANT_BY_KIND(GGML_Q5_K, 1, 3, 5, true),
     STREAM_VARIANT_BY_KIND(GGML_Q4_K, 1, 3, 5, true), STREAM_VARIANT_BY_KIND(GGML_Q6_K, 1, 3, 5, true),
     STREAM_VARIANT_BY_KIND(GGML_Q8_0, 1, 3, 5, true),
+    STREAM_VARIANT_BY_KIND(GGML_Q4_K, 2, 3, 5, true), STREAM_VARIANT_BY_KIND(GGML_Q6_K, 2, 3, 5, true),
     STREAM_VARIANT(GGML_Q4_K, 4, 3), STREAM_VARIANT(GGML_Q4_K, 8, 3), STREAM_VARIANT(GGML_Q6_K, 4, 3),
     STREAM_VARIANT(GGML_Q6_K, 8, 3), STREAM_VARIANT(GGML_Q8_0, 4, 3), STREAM_VARIANT(GGML_Q8_0, 8, 3),
     // gate/up pair with SiLU (Q4_K) and projection + residual (Q4_K, Q6_K), batch 1 and 2
