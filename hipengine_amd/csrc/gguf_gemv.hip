@@ -66,9 +66,12 @@ const Variant* find_variant(int qt, int b, int r, int cb) {
 
 // ---- run form (whole rows per wave, contiguous block runs) -------------------
 
-template <int QT, int B, int G, int CB>
+// XK >= 0 fixes the activation kind at compile time (less prologue code to fetch cold), XK < 0 reads it
+// from the arguments.
+template <int QT, int B, int G, int CB, int XK = -1>
 __global__ void __launch_bounds__(512) gemv_run_kernel(GemvRunArgs a) {
   extern __shared__ __align__(16) uint8_t smem[];
+  if constexpr (XK >= 0) a.x_kind = XK;
   gemv_run_workgroup<QT, B, G, CB>(a, smem);
 }
 
@@ -77,15 +80,20 @@ using RunKernelFn = void (*)(GemvRunArgs);
 struct RunVariant {
   int b, g, cb;
   RunKernelFn fn;
+  RunKernelFn by_kind[2];   // float32 and bf16 activations (null: use fn)
 };
 
 #define RUN_VARIANT(QT, B, G, CB) \
-  RunVariant { B, G, CB, gemv_run_kernel<QT, B, G, CB> }
+  RunVariant { B, G, CB, gemv_run_kernel<QT, B, G, CB>, {nullptr, nullptr} }
+// the variants the default plan picks for K = 4096 and 5120 (4 rows per run, 5 loads per chunk)
+#define RUN_VARIANT_BY_KIND(QT, B, G, CB)              \
+  RunVariant { B, G, CB, gemv_run_kernel<QT, B, G, CB>, \
+               {gemv_run_kernel<QT, B, G, CB, KIND_F32>, gemv_run_kernel<QT, B, G, CB, KIND_BF16>} }
 #define RUN_VARIANTS_FOR(QT)                                                                        \
   RUN_VARIANT(QT, 1, 1, 1), RUN_VARIANT(QT, 1, 2, 1), RUN_VARIANT(QT, 1, 4, 1), RUN_VARIANT(QT, 1, 8, 1), \
-  RUN_VARIANT(QT, 1, 1, 5), RUN_VARIANT(QT, 1, 2, 5), RUN_VARIANT(QT, 1, 4, 5), RUN_VARIANT(QT, 1, 8, 5), \
+  RUN_VARIANT(QT, 1, 1, 5), RUN_VARIANT(QT, 1, 2, 5), RUN_VARIANT_BY_KIND(QT, 1, 4, 5), RUN_VARIANT(QT, 1, 8, 5), \
   RUN_VARIANT(QT, 2, 1, 1), RUN_VARIANT(QT, 2, 2, 1), RUN_VARIANT(QT, 2, 4, 1), RUN_VARIANT(QT, 2, 8, 1), \
-  RUN_VARIANT(QT, 2, 1, 5), RUN_VARIANT(QT, 2, 2, 5), RUN_VARIANT(QT, 2, 4, 5), RUN_VARIANT(QT, 2, 8, 5)
+  RUN_VARIANT(QT, 2, 1, 5), RUN_VARIANT(QT, 2, 2, 5), RUN_VARIANT_BY_KIND(QT, 2, 4, 5), RUN_VARIANT(QT, 2, 8, 5)
 
 const RunVariant kRunQ4K[] = {RUN_VARIANTS_FOR(GGML_Q4_K)};
 const RunVariant kRunQ6K[] = {RUN_VARIANTS_FOR(GGML_Q6_K)};
@@ -344,7 +352,8 @@ int launch_gemv_run(int qt, const void* x, int x_kind, const uint8_t* w, void* o
   a.waves = p.waves;
   const int64_t runs = (N + p.g - 1) / p.g;
   const unsigned grid = static_cast<unsigned>((runs + p.waves - 1) / p.waves);
-  hipLaunchKernelGGL(v->fn, dim3(grid), dim3(p.waves * 64), lds, stream, a);
+  const RunKernelFn fn = (x_kind == KIND_F32 || x_kind == KIND_BF16) && v->by_kind[x_kind] ? v->by_kind[x_kind] : v->fn;
+  hipLaunchKernelGGL(fn, dim3(grid), dim3(p.waves * 64), lds, stream, a);
   return static_cast<int>(hipGetLastError());
 }
 
