@@ -380,6 +380,7 @@ using StreamKernelFn = void (*)(GemvStreamArgs);
 // `fuse`: plain projection, gate/up pair with SiLU, or projection plus residual.
 struct StreamVariant {
   int qt, b, d;
+  int s;         // activation groups (of 8 values) per thread fetched up front
   bool long_k;
   int fuse;
   StreamKernelFn fn;
@@ -387,14 +388,14 @@ struct StreamVariant {
 };
 
 #define STREAM_VARIANT(QT, B, D) \
-  StreamVariant { QT, B, D, false, FUSE_NONE, gemv_stream_kernel<QT, B, D, (B <= 2 ? 2 : 1)>, {nullptr, nullptr, nullptr, nullptr} }
+  StreamVariant { QT, B, D, (B <= 2 ? 2 : 1), false, FUSE_NONE, gemv_stream_kernel<QT, B, D, (B <= 2 ? 2 : 1)>, {nullptr, nullptr, nullptr, nullptr} }
 #define STREAM_VARIANT_BY_KIND(QT, B, D, S, LONG_K)                                                      \
-  StreamVariant { QT, B, D, LONG_K, FUSE_NONE, gemv_stream_kernel<QT, B, D, S>,                           \
+  StreamVariant { QT, B, D, S, LONG_K, FUSE_NONE, gemv_stream_kernel<QT, B, D, S>,                        \
                   {gemv_stream_kernel<QT, B, D, S, KIND_F32>, gemv_stream_kernel<QT, B, D, S, KIND_BF16>, \
                    gemv_stream_kernel<QT, B, D, S, KIND_F16>, gemv_stream_kernel<QT, B, D, S, KIND_Q8_1>} }
 // fused epilogues: float32 and bf16 activations get instantiations of their own, the other kinds the generic one
 #define STREAM_VARIANT_FUSED_D(QT, B, D, S, LONG_K, FUSE)                                                        \
-  StreamVariant { QT, B, D, LONG_K, FUSE, gemv_stream_kernel<QT, B, D, S, -1, FUSE>,                              \
+  StreamVariant { QT, B, D, S, LONG_K, FUSE, gemv_stream_kernel<QT, B, D, S, -1, FUSE>,                           \
                   {gemv_stream_kernel<QT, B, D, S, KIND_F32, FUSE>, gemv_stream_kernel<QT, B, D, S, KIND_BF16, FUSE>, \
                    nullptr, nullptr} }
 #define STREAM_VARIANT_FUSED(QT, B, S, LONG_K, FUSE) STREAM_VARIANT_FUSED_D(QT, B, 3, S, LONG_K, FUSE)
@@ -514,7 +515,10 @@ int launch_gemv_stream(int qt, const void* x, int x_kind, const uint8_t* w, void
   }
   if (fusion.fuse == FUSE_RESIDUAL && !fusion.residual) return static_cast<int>(hipErrorInvalidValue);
   if (lds > kMaxLds) return static_cast<int>(hipErrorInvalidValue);
-  const StreamKernelFn fn = (x_kind >= KIND_F32 && x_kind <= KIND_Q8_1 && v->by_kind[x_kind]) ? v->by_kind[x_kind] : v->fn;
+  // the kind-specialised kernels stage the whole row from the groups fetched up front
+  const bool up_front = nb * 8 <= v->s * p.waves * 16;
+  const StreamKernelFn fn =
+      (up_front && x_kind >= KIND_F32 && x_kind <= KIND_Q8_1 && v->by_kind[x_kind]) ? v->by_kind[x_kind] : v->fn;
   if (lds > 64 * 1024) {
     // above the default dynamic limit: raise it for this kernel, once (no stream work)
     static const void* raised[64];

@@ -216,7 +216,9 @@ __device__ __forceinline__ void gemv_run_stage_one(int x_kind, const uint32_t (&
   }
 }
 
-template <int QT, int B, int S>
+// ALL_UP_FRONT: the caller guarantees that the S groups per thread fetched up front cover the row
+// (K/32 <= S * threads/4); the loop over the rest is then not generated.
+template <int QT, int B, int S, bool ALL_UP_FRONT = false>
 __device__ __forceinline__ void gemv_run_stage_commit(const GemvRunArgs& a, const StageRegs<B, S>& sr, uint8_t* q8,
                                                       float* rec, int* s16) {
   constexpr int Q8S = run_q8_stride<QT>();
@@ -238,7 +240,7 @@ __device__ __forceinline__ void gemv_run_stage_commit(const GemvRunArgs& a, cons
   // large K or batch: the rest - (batch row, group) items past the first S groups per row - is loaded here, P
   // items per thread at a time across the batch rows, so that a load latency is paid once per P items
   // and not once per item per row
-  const int rest = groups - S * nteams;              // groups per row still to do (may be <= 0)
+  const int rest = ALL_UP_FRONT ? 0 : groups - S * nteams;   // groups per row still to do (may be <= 0)
   if (rest > 0) {
     constexpr int P = B >= 4 ? 8 : 2;
     const int per_row = (rest + nteams - 1) / nteams;  // items of this team per batch row

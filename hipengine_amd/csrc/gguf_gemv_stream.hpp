@@ -48,8 +48,11 @@ constexpr int STREAM_PAIR_MAX_ROWS = 16;   // rows per wave the pair form can ho
 
 // XK >= 0 fixes the activation kind at compile time (the staging code of the other
 // kinds is then not generated: a decode kernel runs its prologue once per launch
-// with a cold instruction cache, so prologue code size is launch latency), XK < 0
-// reads it from the arguments.
+// with a cold instruction cache, so prologue code size is launch latency) and
+// promises that S groups of 8 values per thread cover K (K/8 <= S * threads/4), so
+// the loop over further groups is not generated either (dropping that never-taken
+// loop alone took 0.7 us off the 17408x5120 launch); XK < 0 reads the kind from the
+// arguments and takes any K.
 //
 // FUSE selects the epilogue:
 //   FUSE_PAIR      the wave walks its rows of the gate matrix and then the same rows of the up
@@ -109,7 +112,8 @@ __device__ __forceinline__ void gemv_stream_workgroup(const GemvStreamArgs& a, u
 #pragma unroll
   for (int c = 0; c < D; ++c) issue(c, ring[c]);
 
-  gemv_run_stage_commit<QT, B, S>(ra, sr, q8, rec, s16);
+  // the kind-specialised kernels are launched only where the S groups per thread fetched up front cover K
+  gemv_run_stage_commit<QT, B, S, (XK >= 0)>(ra, sr, q8, rec, s16);
   __syncthreads();
 
   const int total_rows = FUSE == FUSE_PAIR ? 2 * nrows : nrows;
