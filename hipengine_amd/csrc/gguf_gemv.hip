@@ -421,6 +421,23 @@ const StreamVariant kStream[] = {
     STREAM_VARIANT_FUSED_D(GGML_Q4_K, 1, 2, 2, false, FUSE_PAIR), STREAM_VARIANT_FUSED_D(GGML_Q4_K, 1, 2, 2, false, FUSE_RESIDUAL),
 };
 
+// The variant a launch takes: of those for (type, batch bucket, ring depth, epilogue), the one with the fewest
+// up-front groups per thread that still cover K with this many waves (nb*8 groups, 16 teams per wave);
+// if none does, the one with the most (its generic kernel loops over the rest).
+const StreamVariant* pick_stream_variant(int qt, int b, int d, int fuse, int nb, int waves) {
+  const StreamVariant* best = nullptr;
+  bool best_covers = false;
+  for (const StreamVariant& v : kStream) {
+    if (v.qt != qt || v.b != b || v.d != d || v.fuse != fuse) continue;
+    const bool covers = nb * 8 <= v.s * waves * 16;
+    if (!best || (covers && (!best_covers || v.s < best->s)) || (!covers && !best_covers && v.s > best->s)) {
+      best = &v;
+      best_covers = covers;
+    }
+  }
+  return best;
+}
+
 const StreamVariant* find_stream_variant(int qt, int b, int d, bool long_k = false, int fuse = FUSE_NONE) {
   const StreamVariant* fallback = nullptr;
   for (const StreamVariant& v : kStream) {
@@ -500,9 +517,7 @@ int launch_gemv_stream(int qt, const void* x, int x_kind, const uint8_t* w, void
                        int64_t K, int64_t N, const StreamPlan& p, hipStream_t stream,
                        const StreamFusion& fusion = StreamFusion()) {
   const int nb = static_cast<int>(K / QK_K);
-  // more than two activation groups per thread (16 teams of 4 lanes per wave): take the
-  // instantiation that fetches five up front
-  const StreamVariant* v = find_stream_variant(qt, p.b, p.d, p.waves > 0 && nb > 4 * p.waves, fusion.fuse);
+  const StreamVariant* v = p.waves > 0 ? pick_stream_variant(qt, p.b, p.d, fusion.fuse, nb, p.waves) : nullptr;
   if (!v || nb < 16 || rows > p.b || p.waves < 1 || p.waves > (p.b == 1 ? 12 : 8) || p.waves_total < p.waves ||
       (p.waves_total % p.waves) != 0 || p.waves_total > N) {
     return static_cast<int>(hipErrorInvalidValue);
