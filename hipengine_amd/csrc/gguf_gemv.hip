@@ -66,13 +66,14 @@ const Variant* find_variant(int qt, int b, int r, int cb) {
 
 // ---- run form (whole rows per wave, contiguous block runs) -------------------
 
-// XK >= 0 fixes the activation kind at compile time (less prologue code to fetch cold), XK < 0 reads it
-// from the arguments.
+// XK >= 0 fixes the activation kind at compile time and promises that the two activation groups per
+// thread fetched up front cover K (less prologue code to fetch cold), XK < 0 reads the kind from the
+// arguments and takes any K.
 template <int QT, int B, int G, int CB, int XK = -1>
 __global__ void __launch_bounds__(512) gemv_run_kernel(GemvRunArgs a) {
   extern __shared__ __align__(16) uint8_t smem[];
   if constexpr (XK >= 0) a.x_kind = XK;
-  gemv_run_workgroup<QT, B, G, CB>(a, smem);
+  gemv_run_workgroup<QT, B, G, CB, (XK >= 0)>(a, smem);
 }
 
 using RunKernelFn = void (*)(GemvRunArgs);
@@ -352,7 +353,9 @@ int launch_gemv_run(int qt, const void* x, int x_kind, const uint8_t* w, void* o
   a.waves = p.waves;
   const int64_t runs = (N + p.g - 1) / p.g;
   const unsigned grid = static_cast<unsigned>((runs + p.waves - 1) / p.waves);
-  const RunKernelFn fn = (x_kind == KIND_F32 || x_kind == KIND_BF16) && v->by_kind[x_kind] ? v->by_kind[x_kind] : v->fn;
+  const bool up_front = nb * 8 <= 2 * p.waves * 16;
+  const RunKernelFn fn =
+      up_front && (x_kind == KIND_F32 || x_kind == KIND_BF16) && v->by_kind[x_kind] ? v->by_kind[x_kind] : v->fn;
   hipLaunchKernelGGL(fn, dim3(grid), dim3(p.waves * 64), lds, stream, a);
   return static_cast<int>(hipGetLastError());
 }

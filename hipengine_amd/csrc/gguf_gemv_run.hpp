@@ -333,7 +333,8 @@ __device__ __forceinline__ float wave_sum_to_lane63(float v) {
   return v;
 }
 
-template <int QT, int B, int G, int CB>
+// ALL_UP_FRONT: the two activation groups per thread fetched up front cover K (K/32 <= 2 * threads/4).
+template <int QT, int B, int G, int CB, bool ALL_UP_FRONT = false>
 __device__ __forceinline__ void gemv_run_workgroup(const GemvRunArgs& a, uint8_t* smem) {
   using Regs = WeightRegs<GemvTraits<QT>::REGS>;
   constexpr int Q8S = run_q8_stride<QT>();
@@ -378,7 +379,7 @@ __device__ __forceinline__ void gemv_run_workgroup(const GemvRunArgs& a, uint8_t
       }
     }
     if (i0 == 0) {
-      gemv_run_stage_commit<QT, B, S>(a, sr, q8, rec, s16);
+      gemv_run_stage_commit<QT, B, S, ALL_UP_FRONT>(a, sr, q8, rec, s16);
       __syncthreads();
     }
 #pragma unroll
