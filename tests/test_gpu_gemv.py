@@ -319,9 +319,12 @@ def test_pslab_form_q5_k(dev, rows, k, n, waves, bpw, wgs):
 
 
 @pytest.mark.parametrize("quant,d,waves,waves_total", [("gguf_q4_k", 3, 4, 64), ("gguf_q4_k", 3, 10, 120),
-                                                      ("gguf_q6_k", 3, 12, 96), ("gguf_q8_0", 3, 8, 64)])
+                                                      ("gguf_q6_k", 3, 12, 96), ("gguf_q8_0", 3, 8, 64),
+                                                      ("gguf_q4_k", 2, 12, 96), ("gguf_q4_k", 2, 4, 64)])
 def test_stream_form_explicit_layouts(dev, quant, d, waves, waves_total):
-    """Stream form with explicit wave counts (up to 12 waves per workgroup at batch 1); the ring depth built is 3."""
+    """Stream form with explicit wave counts (up to 12 waves per workgroup at batch 1); ring depths built: 3, and 2
+    for Q4_K.  With 4 waves the two activation groups per thread fetched up front do not cover K = 5120, so the
+    launch takes the kernel that loops over the rest; with 10 or 12 they do and it takes the one without that loop."""
     rng = np.random.default_rng(5 + waves_total)
     rows, k, n = 1, 5120, 256
     x = rng.standard_normal((rows, k)).astype(np.float32)
