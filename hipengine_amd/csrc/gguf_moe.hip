@@ -305,9 +305,12 @@ constexpr int sel_max_threads() {
   return BLOCKS * GemvTraits<QT>::REGS <= 48 ? 1024 : 512;
 }
 
-template <int QT, int R, int CB, int MODE>
+// XK >= 0 fixes the activation kind at compile time (a decode kernel runs its staging code once, with a cold
+// instruction cache: the code of the other kinds is launch latency), XK < 0 reads it from the arguments.
+template <int QT, int R, int CB, int MODE, int XK = -1>
 __global__ void __launch_bounds__((sel_max_threads<QT, R * CB>())) selected_gemv_kernel(SelArgs s) {
   extern __shared__ __align__(16) uint8_t smem[];
+  if constexpr (XK >= 0) s.g.x_kind = XK;
   const int64_t row_bytes = static_cast<int64_t>(s.g.K / QK_K) * GemvTraits<QT>::SUPER_BYTES;
   const int64_t expert_bytes = static_cast<int64_t>(s.g.N) * row_bytes;
   GemvArgs a = s.g;
@@ -352,9 +355,10 @@ __global__ void __launch_bounds__((sel_max_threads<QT, R * CB>())) selected_gemv
 // One workgroup per (16 output rows, token); its waves are (slot, K slice) pairs, so the
 // weight blocks of all the token's experts are in flight together and the activations
 // of all slots (top_k consecutive rows of x) are quantized in one pass per K chunk.
-template <int QT, int TK, int RG>
+template <int QT, int TK, int RG, int XK = -1>
 __global__ void __launch_bounds__(1024) selected_down_sum_kernel(SelArgs s) {
   extern __shared__ __align__(16) uint8_t smem[];
+  if constexpr (XK >= 0) s.g.x_kind = XK;
   using Regs = WeightRegs<GemvTraits<QT>::REGS>;
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int ks = s.g.ks;                       // K slices per slot; waves = TK * ks
@@ -382,6 +386,10 @@ __global__ void __launch_bounds__(1024) selected_down_sum_kernel(SelArgs s) {
   const int64_t e = slot < s.top_k ? s.selected[t * s.top_k + slot] : -1;
   const bool valid = e >= 0 && e < s.num_experts;
   const uint8_t* wexp = s.g.w + (valid ? e : 0) * expert_bytes;
+  // routing weight of each slot (0 for a slot without a valid expert, whose dot is 0 too), fetched now and
+  // kept in LDS: read from memory in the final sum, slot after slot, they were a chain of eight round trips
+  float* rw = red + TK * ks * 16 * RG;
+  if (kslice == 0 && lane == 0) rw[slot] = valid ? s.routing[t * s.top_k + slot] : 0.0f;
 
   float acc[RG];
 #pragma unroll
@@ -415,11 +423,9 @@ __global__ void __launch_bounds__(1024) selected_down_sum_kernel(SelArgs s) {
   if (tid < 16 * RG && first_row + tid < s.g.N) {
     float total = 0.0f;
     for (int sl = 0; sl < s.top_k; ++sl) {
-      const int64_t es = s.selected[t * s.top_k + sl];
-      if (es < 0 || es >= s.num_experts) continue;
       float dot = 0.0f;
       for (int k = 0; k < ks; ++k) dot += red[(sl * ks + k) * 16 * RG + tid];
-      total += s.routing[t * s.top_k + sl] * dot;
+      total += rw[sl] * dot;
     }
     store_scalar(s.g.out, static_cast<int64_t>(t) * s.g.N + first_row + tid, total, s.g.out_kind);
   }
@@ -429,10 +435,13 @@ using SelFn = void (*)(SelArgs);
 struct SelVariant {
   int qt, cb, mode, max_threads;
   SelFn fn;
+  SelFn by_kind[2];   // float32 and bf16 activations
 };
 #define SEL_VARIANTS(QT, CB)                                                                                   \
-  SelVariant{QT, CB, SEL_SINGLE, sel_max_threads<QT, CB>(), selected_gemv_kernel<QT, 1, CB, SEL_SINGLE>},         \
-  SelVariant{QT, CB, SEL_DUAL_SILU, sel_max_threads<QT, 2 * CB>(), selected_gemv_kernel<QT, 2, CB, SEL_DUAL_SILU>}
+  SelVariant{QT, CB, SEL_SINGLE, sel_max_threads<QT, CB>(), selected_gemv_kernel<QT, 1, CB, SEL_SINGLE>,          \
+             {selected_gemv_kernel<QT, 1, CB, SEL_SINGLE, KIND_F32>, selected_gemv_kernel<QT, 1, CB, SEL_SINGLE, KIND_BF16>}}, \
+  SelVariant{QT, CB, SEL_DUAL_SILU, sel_max_threads<QT, 2 * CB>(), selected_gemv_kernel<QT, 2, CB, SEL_DUAL_SILU>, \
+             {selected_gemv_kernel<QT, 2, CB, SEL_DUAL_SILU, KIND_F32>, selected_gemv_kernel<QT, 2, CB, SEL_DUAL_SILU, KIND_BF16>}}
 const SelVariant kSel[] = {
     SEL_VARIANTS(GGML_Q4_K, 1), SEL_VARIANTS(GGML_Q4_K, 2), SEL_VARIANTS(GGML_Q4_K, 5),
     SEL_VARIANTS(GGML_Q6_K, 1), SEL_VARIANTS(GGML_Q6_K, 2), SEL_VARIANTS(GGML_Q6_K, 5),
@@ -467,11 +476,16 @@ int launch_selected(int qt, int mode, const void* x, int x_kind, const int64_t* 
     int rgn = 2;
     while (rgn > 1 && (N + 16 * rgn - 1) / (16 * rgn) * x_rows < 512) rgn >>= 1;
     s.g.ks = ks; s.g.nrg = rgn;
-    const size_t lds = gemv_lds_bytes(qt, 8, 1, 1, ks, 1) + static_cast<size_t>(8) * ks * 16 * rgn * 4;
+    const size_t lds = gemv_lds_bytes(qt, 8, 1, 1, ks, 1) + static_cast<size_t>(8) * ks * 16 * rgn * 4 + 8 * 4;
     if (lds > 64 * 1024) return static_cast<int>(hipErrorInvalidValue);
     const dim3 grid(static_cast<unsigned>((N + 16 * rgn - 1) / (16 * rgn)), static_cast<unsigned>(x_rows));
     const dim3 block(8 * ks * 64);
-#define LAUNCH_DOWN(QT, RGN) hipLaunchKernelGGL((selected_down_sum_kernel<QT, 8, RGN>), grid, block, lds, stream, s)
+#define LAUNCH_DOWN(QT, RGN)                                                                                   \
+  do {                                                                                                         \
+    if (x_kind == KIND_F32) hipLaunchKernelGGL((selected_down_sum_kernel<QT, 8, RGN, KIND_F32>), grid, block, lds, stream, s); \
+    else if (x_kind == KIND_BF16) hipLaunchKernelGGL((selected_down_sum_kernel<QT, 8, RGN, KIND_BF16>), grid, block, lds, stream, s); \
+    else hipLaunchKernelGGL((selected_down_sum_kernel<QT, 8, RGN>), grid, block, lds, stream, s);                \
+  } while (0)
     if (qt == GGML_Q4_K) {
       if (rgn == 2) LAUNCH_DOWN(GGML_Q4_K, 2); else LAUNCH_DOWN(GGML_Q4_K, 1);
     } else {
@@ -508,7 +522,8 @@ int launch_selected(int qt, int mode, const void* x, int x_kind, const int64_t* 
   if (lds > 64 * 1024) return static_cast<int>(hipErrorInvalidValue);
   const int rows_out = nrg * rows_out_per_group;
   const dim3 grid(static_cast<unsigned>((N + rows_out - 1) / rows_out), static_cast<unsigned>(lanes));
-  hipLaunchKernelGGL(v->fn, grid, dim3(ks * nrg * 64), lds, stream, s);
+  const SelFn fn = (x_kind == KIND_F32 || x_kind == KIND_BF16) ? v->by_kind[x_kind] : v->fn;
+  hipLaunchKernelGGL(fn, grid, dim3(ks * nrg * 64), lds, stream, s);
   return static_cast<int>(hipGetLastError());
 }
 
