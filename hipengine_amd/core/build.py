@@ -46,6 +46,7 @@ class BuildError(RuntimeError):
 class BuildArtifact:
     family: str
     key: str
+    sources_digest: str
     sources: tuple[Path, ...]
     headers: tuple[Path, ...]
     flags: tuple[str, ...]
@@ -70,7 +71,7 @@ def default_sources() -> tuple[Path, ...]:
 
 
 def default_headers() -> tuple[Path, ...]:
-    return tuple(sorted(CSRC_DIR.glob("*.hpp"))) + (_PACKAGE.parent / "include" / "hipengine_gfx950.h",)
+    return tuple(sorted(CSRC_DIR.glob("*.hpp"))) + tuple(sorted((_PACKAGE.parent / "include").glob("*.h")))
 
 
 def _compiler() -> str:
@@ -103,26 +104,54 @@ def plan_hip_build(
     for part in (_KEY_DOMAIN, Path(compiler).name, version, *flags):
         h.update(part.encode())
         h.update(b"\0")
-    for path in (*srcs, *hdrs):
-        h.update(path.name.encode())
-        h.update(b"\0")
-        h.update(path.read_bytes())
-        h.update(b"\0")
+    digest = sources_digest(srcs, hdrs)
+    h.update(digest.encode())
     key = h.hexdigest()
     out = Path(out_dir) if out_dir else LIB_DIR
     obj_dir = out / "obj"
     commands = tuple(
         (compiler, *flags, "-c", str(s), "-o", str(obj_dir / (s.stem + ".o"))) for s in srcs
     ) + ((compiler, *flags, "-shared", *(str(obj_dir / (s.stem + ".o")) for s in srcs), "-o", str(out / output_name)),)
-    return BuildArtifact(family, key, srcs, hdrs, flags, compiler, out / output_name, out / "manifest.txt", commands)
+    return BuildArtifact(family, key, digest, srcs, hdrs, flags, compiler, out / output_name, out / "manifest.txt", commands)
+
+
+def sources_digest(sources: tuple[Path, ...] | None = None, headers: tuple[Path, ...] | None = None) -> str:
+    """sha256 over the names and bytes of the sources and headers the library is built from."""
+    h = hashlib.sha256()
+    for path in (*(sources or default_sources()), *(headers or default_headers())):
+        h.update(path.name.encode())
+        h.update(b"\0")
+        h.update(path.read_bytes())
+        h.update(b"\0")
+    return h.hexdigest()
+
+
+def write_manifest(art: BuildArtifact) -> None:
+    art.manifest.write_text(
+        f"key={art.key}\nsources_digest={art.sources_digest}\nfamily={art.family}\ncompiler={art.compiler}\n"
+        f"flags={' '.join(art.flags)}\n" + "".join(f"source={s.name}\n" for s in art.sources)
+    )
+
+
+def _manifest_field(manifest: Path, name: str) -> str | None:
+    if not manifest.exists():
+        return None
+    for line in manifest.read_text().splitlines():
+        if line.startswith(name + "="):
+            return line[len(name) + 1:].strip()
+    return None
 
 
 _loaded: dict[Path, ctypes.CDLL] = {}
 
 
 def load_library(path: Path | None = None) -> ctypes.CDLL:
-    """Open the built library (memoized).  Raises if it has not been built: there is
-    no other implementation to fall back to."""
+    """Open the built library (memoized).  Raises if it has not been built, or if the in-tree
+    library was built from other sources than the ones next to it (a stale binary would silently
+    be what runs): there is no other implementation to fall back to.  When a device is present the
+    library's per-device set-up runs here, so that every entry point is graph-capturable from its
+    first launch."""
+    in_tree = path is None
     target = Path(path) if path else LIB_DIR / OUTPUT_NAME
     lib = _loaded.get(target)
     if lib is None:
@@ -131,7 +160,18 @@ def load_library(path: Path | None = None) -> ctypes.CDLL:
                 f"{target} is missing: build it with hipengine_amd.core.build.build_hip() "
                 "(hipcc --offload-arch=gfx950); the gfx950 kernels have no CPU fallback"
             )
+        if in_tree and os.environ.get("HIPENGINE_SKIP_STALE_CHECK") != "1":
+            built_from = _manifest_field(target.parent / "manifest.txt", "sources_digest")
+            if built_from != sources_digest():
+                raise BuildError(
+                    f"{target} is stale: its manifest records sources {str(built_from)[:16]}, the tree holds "
+                    f"{sources_digest()[:16]}; rebuild with hipengine_amd.core.build.build_hip()"
+                )
         lib = ctypes.CDLL(str(target))
+        init = getattr(lib, "hipengine_gfx950_init", None)
+        if init is not None:
+            init.argtypes, init.restype = [], ctypes.c_int
+            init()   # without a device this returns an error code and changes nothing; launches would fail anyway
         _loaded[target] = lib
     return lib
 
@@ -165,9 +205,6 @@ def build_hip(
         with ThreadPoolExecutor(max_workers=max(1, jobs)) as pool:
             list(pool.map(run, compile_cmds))
         run(link_cmd)
-        art.manifest.write_text(
-            f"key={art.key}\nfamily={art.family}\ncompiler={art.compiler}\nflags={' '.join(art.flags)}\n"
-            + "".join(f"source={s.name}\n" for s in art.sources)
-        )
+        write_manifest(art)
         _loaded.pop(art.output, None)
     return load_library(art.output) if load else art

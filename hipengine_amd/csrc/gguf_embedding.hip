@@ -4,6 +4,8 @@
 
 #include "gguf_dequant.hpp"
 
+#include "gguf_init.hpp"
+
 #include "../../include/hipengine_gfx950.h"
 
 namespace {
@@ -59,3 +61,8 @@ DEFINE_EMBEDDING(q4_k, GGML_Q4_K)
 DEFINE_EMBEDDING(q5_k, GGML_Q5_K)
 DEFINE_EMBEDDING(q6_k, GGML_Q6_K)
 DEFINE_EMBEDDING(q8_0, GGML_Q8_0)
+
+int hipengine_gfx950::embedding_load() {
+  hipFuncAttributes attr;
+  return static_cast<int>(hipFuncGetAttributes(&attr, reinterpret_cast<const void*>(embedding_kernel<GGML_Q4_K>)));
+}

@@ -7,8 +7,10 @@
 #include "gguf_gemv_stream.hpp"
 #include "gguf_gemv_slab.hpp"
 #include "gguf_gemv_pslab.hpp"
+#include "gguf_init.hpp"
 
 #include "../../include/hipengine_gfx950.h"
+#include "../../include/hipengine_gfx950_tuning.h"
 
 namespace {
 
@@ -125,13 +127,11 @@ using SlabKernelFn = void (*)(GemvSlabArgs);
 struct SlabVariant {
   int b, bpw;
   SlabKernelFn by_kind[4];
-  bool lds_raised[4];
 };
 #define SLAB_VARIANT(B, BPW)                                                                            \
   SlabVariant { B, BPW, {gemv_slab_q4k_kernel<B, BPW, KIND_F32>, gemv_slab_q4k_kernel<B, BPW, KIND_BF16>, \
-                         gemv_slab_q4k_kernel<B, BPW, KIND_F16>, gemv_slab_q4k_kernel<B, BPW, KIND_Q8_1>}, \
-                {false, false, false, false} }
-SlabVariant kSlab[] = {SLAB_VARIANT(1, 1), SLAB_VARIANT(1, 2), SLAB_VARIANT(2, 1), SLAB_VARIANT(2, 2),
+                         gemv_slab_q4k_kernel<B, BPW, KIND_F16>, gemv_slab_q4k_kernel<B, BPW, KIND_Q8_1>} }
+const SlabVariant kSlab[] = {SLAB_VARIANT(1, 1), SLAB_VARIANT(1, 2), SLAB_VARIANT(2, 1), SLAB_VARIANT(2, 2),
                        SLAB_VARIANT(4, 1), SLAB_VARIANT(4, 2), SLAB_VARIANT(8, 1), SLAB_VARIANT(8, 2)};
 
 struct SlabPlan {
@@ -159,8 +159,8 @@ int launch_gemv_slab(const void* x, int x_kind, const uint8_t* w, void* out, int
                      int64_t N, const SlabPlan& p, hipStream_t stream, const void* residual = nullptr,
                      const void* gate = nullptr) {
   const int nb = static_cast<int>(K / QK_K);
-  SlabVariant* v = nullptr;
-  for (SlabVariant& c : kSlab)
+  const SlabVariant* v = nullptr;
+  for (const SlabVariant& c : kSlab)
     if (c.b == p.b && c.bpw == p.bpw) v = &c;
   if (!v || rows > p.b || x_kind < KIND_F32 || x_kind > KIND_Q8_1 || p.rows_wg < 1 || p.rows_wg > SLAB_MAX_ROWS ||
       p.waves < 1 || p.waves > (p.bpw == 1 ? 16 : 12) || p.two_block_waves < 0 || p.two_block_waves > p.waves ||
@@ -170,11 +170,9 @@ int launch_gemv_slab(const void* x, int x_kind, const uint8_t* w, void* out, int
   }
   const size_t lds = gemv_slab_lds_bytes(p.b, p.waves, p.two_block_waves);
   if (lds > 160 * 1024) return static_cast<int>(hipErrorInvalidValue);
-  if (lds > 64 * 1024 && !v->lds_raised[x_kind]) {
-    const hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(v->by_kind[x_kind]),
-                                             hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
-    if (e != hipSuccess) return static_cast<int>(e);
-    v->lds_raised[x_kind] = true;
+  if (lds > 64 * 1024) {   // above the default dynamic limit: raised for every kernel by the library set-up
+    const int rc = ensure_init();
+    if (rc != static_cast<int>(hipSuccess)) return rc;
   }
   GemvSlabArgs a{x, w, out, x_kind, out_kind, rows, static_cast<int>(K), static_cast<int>(N), p.rows_wg, p.waves,
                  p.two_block_waves, residual, gate};
@@ -196,13 +194,11 @@ struct PslabVariant {
   int qt, b;
   bool phased;
   PslabKernelFn by_kind[4];
-  bool lds_raised[4];
 };
 #define PSLAB_VARIANT(QT, B, P)                                                                              \
   PslabVariant { QT, B, P, {gemv_pslab_kernel<QT, B, P, KIND_F32>, gemv_pslab_kernel<QT, B, P, KIND_BF16>,   \
-                            gemv_pslab_kernel<QT, B, P, KIND_F16>, gemv_pslab_kernel<QT, B, P, KIND_Q8_1>}, \
-                 {false, false, false, false} }
-PslabVariant kPslab[] = {PSLAB_VARIANT(GGML_Q5_K, 4, false), PSLAB_VARIANT(GGML_Q5_K, 4, true),
+                            gemv_pslab_kernel<QT, B, P, KIND_F16>, gemv_pslab_kernel<QT, B, P, KIND_Q8_1>} }
+const PslabVariant kPslab[] = {PSLAB_VARIANT(GGML_Q5_K, 4, false), PSLAB_VARIANT(GGML_Q5_K, 4, true),
                          PSLAB_VARIANT(GGML_Q5_K, 8, false), PSLAB_VARIANT(GGML_Q5_K, 8, true),
                          PSLAB_VARIANT(GGML_Q4_K, 4, false), PSLAB_VARIANT(GGML_Q4_K, 4, true),
                          PSLAB_VARIANT(GGML_Q4_K, 8, false), PSLAB_VARIANT(GGML_Q4_K, 8, true),
@@ -281,8 +277,8 @@ int launch_gemv_pslab(int qt, const void* x, int x_kind, const uint8_t* w, void*
   const int nb = static_cast<int>(K / QK_K);
   const int bpw = 1 << p.bpw_log2;
   const int64_t row_bytes = pslab_row_bytes(qt, nb);
-  PslabVariant* v = nullptr;
-  for (PslabVariant& c : kPslab)
+  const PslabVariant* v = nullptr;
+  for (const PslabVariant& c : kPslab)
     if (c.qt == qt && c.b == p.b && c.phased == (p.phases > 1)) v = &c;
   if (!v || rows < 1 || rows > p.b || x_kind < KIND_F32 || x_kind > KIND_Q8_1 || p.waves < 1 || p.waves > 12 ||
       p.bpw_log2 < 0 || p.bpw_log2 > 2 || p.waves > nb || (nb & 1) != 0 ||
@@ -293,11 +289,9 @@ int launch_gemv_pslab(int qt, const void* x, int x_kind, const uint8_t* w, void*
   }
   const size_t lds = pslab_lds_bytes(qt, p.b, p.waves, bpw);
   if (lds > kMaxLds) return static_cast<int>(hipErrorInvalidValue);
-  if (lds > 64 * 1024 && !v->lds_raised[x_kind]) {
-    const hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(v->by_kind[x_kind]),
-                                             hipFuncAttributeMaxDynamicSharedMemorySize, kMaxLds);
-    if (e != hipSuccess) return static_cast<int>(e);
-    v->lds_raised[x_kind] = true;
+  if (lds > 64 * 1024) {
+    const int rc = ensure_init();
+    if (rc != static_cast<int>(hipSuccess)) return rc;
   }
   GemvPslabArgs a{};
   a.x = x; a.w = w; a.out = out; a.residual = residual; a.gate = gate;
@@ -538,17 +532,8 @@ int launch_gemv_stream(int qt, const void* x, int x_kind, const uint8_t* w, void
   const StreamKernelFn fn =
       (up_front && x_kind >= KIND_F32 && x_kind <= KIND_Q8_1 && v->by_kind[x_kind]) ? v->by_kind[x_kind] : v->fn;
   if (lds > 64 * 1024) {
-    // above the default dynamic limit: raise it for this kernel, once (no stream work)
-    static const void* raised[64];
-    static int n_raised = 0;
-    bool done = false;
-    for (int i = 0; i < n_raised; ++i) done = done || raised[i] == reinterpret_cast<const void*>(fn);
-    if (!done) {
-      const hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(fn),
-                                               hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(kMaxLds));
-      if (e != hipSuccess) return static_cast<int>(e);
-      if (n_raised < 64) raised[n_raised++] = reinterpret_cast<const void*>(fn);
-    }
+    const int rc = ensure_init();
+    if (rc != static_cast<int>(hipSuccess)) return rc;
   }
   GemvStreamArgs a;
   a.x = x; a.w = w; a.out = out;
@@ -678,6 +663,34 @@ int launch_gemv(int qt, const void* x, int x_kind, const uint8_t* w, void* out, 
 }
 
 }  // namespace
+
+// Every slab, phased slab and stream kernel may be launched with more dynamic LDS than the 64 KB a kernel
+// gets by default; the limit is raised for all of them here, once per device, so that no launch has to.
+int hipengine_gfx950::gemv_raise_lds_limits() {
+  auto raise = [](const void* fn) {
+    return fn ? hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(kMaxLds))
+              : hipSuccess;
+  };
+  for (const SlabVariant& v : kSlab)
+    for (const SlabKernelFn fn : v.by_kind) {
+      const hipError_t e = raise(reinterpret_cast<const void*>(fn));
+      if (e != hipSuccess) return static_cast<int>(e);
+    }
+  for (const PslabVariant& v : kPslab)
+    for (const PslabKernelFn fn : v.by_kind) {
+      const hipError_t e = raise(reinterpret_cast<const void*>(fn));
+      if (e != hipSuccess) return static_cast<int>(e);
+    }
+  for (const StreamVariant& v : kStream) {
+    hipError_t e = raise(reinterpret_cast<const void*>(v.fn));
+    if (e != hipSuccess) return static_cast<int>(e);
+    for (const StreamKernelFn fn : v.by_kind) {
+      e = raise(reinterpret_cast<const void*>(fn));
+      if (e != hipSuccess) return static_cast<int>(e);
+    }
+  }
+  return static_cast<int>(hipSuccess);
+}
 
 // ---- fused: float activations in, q8_1 quantization inside the kernel -------
 

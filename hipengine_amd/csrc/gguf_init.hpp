@@ -1,0 +1,22 @@
+// Per-device set-up steps of the library, collected by hipengine_gfx950_init() (gguf_init.hip).
+// Each returns a hipError_t as int and may be called again for a device already set up.
+#pragma once
+
+namespace hipengine_gfx950 {
+
+// Raise the dynamic-LDS limit of every decode GEMV kernel that may be launched with more than 64 KB
+// (gguf_gemv.hip).  Applies to the current device.
+int gemv_raise_lds_limits();
+
+// Make the runtime load the code object of a source file now (it otherwise does so at the file's first
+// launch, which may be inside a stream capture): one per source file that has kernels and no other set-up.
+int quantize_load();
+int mmq_load();
+int moe_load();
+int embedding_load();
+
+// True once hipengine_gfx950_init() has completed for the current device; runs it otherwise.
+// Launch paths that depend on the set-up call this first.
+int ensure_init();
+
+}  // namespace hipengine_gfx950

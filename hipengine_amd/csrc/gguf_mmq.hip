@@ -13,7 +13,10 @@
 
 #include "gguf_mmq_q4k.hpp"
 
+#include "gguf_init.hpp"
+
 #include "../../include/hipengine_gfx950.h"
+#include "../../include/hipengine_gfx950_tuning.h"
 
 namespace {
 
@@ -296,3 +299,8 @@ DEFINE_MMQ_Q4(hipengine_gguf_q4_k_q8_1_mmq32_ctl_dense_bf16_bf16_out, KIND_BF16)
 
 DEFINE_MMQ_Q6(hipengine_gguf_q6_k_mmq32_q8_1_d4s4_f32_bf16_f32_out, KIND_F32)
 DEFINE_MMQ_Q6(hipengine_gguf_q6_k_mmq32_q8_1_d4s4_f32_bf16_bf16_out, KIND_BF16)
+
+int hipengine_gfx950::mmq_load() {
+  hipFuncAttributes attr;
+  return static_cast<int>(hipFuncGetAttributes(&attr, reinterpret_cast<const void*>(mmq_q6_k_d4s4_kernel)));
+}

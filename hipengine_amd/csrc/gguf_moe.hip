@@ -17,6 +17,8 @@
 #include "gguf_gemv.hpp"
 #include "gguf_mmq_q4k.hpp"
 
+#include "gguf_init.hpp"
+
 #include "../../include/hipengine_gfx950.h"
 
 namespace {
@@ -826,4 +828,9 @@ extern "C" int hipengine_qwen35_router_select(const float* logits, int64_t* sele
   hipLaunchKernelGGL(router_select_kernel, dim3(grid), dim3(waves * 64), 0, stream, logits, selected, routing, tokens,
                      logits_stride, static_cast<int>(num_experts), static_cast<int>(top_k));
   return static_cast<int>(hipGetLastError());
+}
+
+int hipengine_gfx950::moe_load() {
+  hipFuncAttributes attr;
+  return static_cast<int>(hipFuncGetAttributes(&attr, reinterpret_cast<const void*>(moe_tile_map_kernel)));
 }

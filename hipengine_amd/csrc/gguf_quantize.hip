@@ -6,6 +6,8 @@
 
 #include "gguf_common.hpp"
 
+#include "gguf_init.hpp"
+
 #include "../../include/hipengine_gfx950.h"
 
 namespace {
@@ -169,8 +171,6 @@ int launch_pack(const void* x, void* out, int64_t rows, int64_t hidden, hipStrea
 
 }  // namespace
 
-extern "C" int hipengine_gfx950_abi_version(void) { return 1; }
-
 extern "C" int hipengine_gguf_q4_k_quantize_f32_q8_1(const void* x, void* xq, int64_t rows, int64_t in_features,
                                                      hipStream_t stream) {
   return launch_q8_1(x, KIND_F32, xq, rows, in_features, stream);
@@ -202,4 +202,9 @@ extern "C" int hipengine_gfx950_moe_silu_mul_ds4_pack(const void* gate_up, int i
   hipLaunchKernelGGL(silu_mul_ds4_pack_kernel, dim3(static_cast<unsigned>(grid)), dim3(256), 0, stream, gate_up,
                      in_kind, static_cast<uint8_t*>(out), groups, inter);
   return static_cast<int>(hipGetLastError());
+}
+
+int hipengine_gfx950::quantize_load() {
+  hipFuncAttributes attr;
+  return static_cast<int>(hipFuncGetAttributes(&attr, reinterpret_cast<const void*>(pack_mmq_kernel<false>)));
 }

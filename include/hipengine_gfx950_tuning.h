@@ -1,0 +1,94 @@
+/*
+ * Tuning and measurement entry points of libhipengine_gfx950.so: the kernels of
+ * hipengine_gfx950.h with their launch layout chosen by the caller, and host-only
+ * queries of the layout the library would choose.  Parameter sweeps and benchmarks
+ * use them; nothing in a serving path needs them and none has a counterpart in
+ * hipEngine.  Same conventions as hipengine_gfx950.h (device pointers, int64 sizes,
+ * hipError_t as int, asynchronous on `stream`).
+ */
+#ifndef HIPENGINE_GFX950_TUNING_H
+#define HIPENGINE_GFX950_TUNING_H
+
+#include "hipengine_gfx950.h"
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+/* The fused GEMV with an explicit workgroup layout, for tuning sweeps: a
+ * workgroup is k_slices x row_groups waves, every wave walks blocks_per_wave
+ * 256-value blocks per chunk of rows_per_lane x 16 rows.  rows <= 8.  New here. */
+int hipengine_gfx950_gguf_q8_1_fused_gemv_tuned(int32_t ggml_type, const void* x, int32_t x_kind,
+                                                const uint8_t* qweight, void* out, int32_t out_kind, int64_t rows,
+                                                int64_t in_features, int64_t out_features, int32_t k_slices,
+                                                int32_t row_groups, int32_t blocks_per_wave, int32_t rows_per_lane,
+                                                hipengine_stream_t stream);
+
+/* The same for the "run" form of the kernel (a wave streams rows_per_wave whole
+ * rows as one contiguous run of blocks, loads_per_chunk 16-block loads at a
+ * time, `waves` waves per workgroup).  rows <= 2, rows_per_wave * (K/256) must
+ * be a multiple of 16.  New here. */
+int hipengine_gfx950_gguf_q8_1_fused_gemv_run_tuned(int32_t ggml_type, const void* x, int32_t x_kind,
+                                                    const uint8_t* qweight, void* out, int32_t out_kind,
+                                                    int64_t rows, int64_t in_features, int64_t out_features,
+                                                    int32_t rows_per_wave, int32_t loads_per_chunk, int32_t waves,
+                                                    hipengine_stream_t stream);
+
+/* The same for the "stream" form (waves_total resident waves, `waves` per
+ * workgroup, each owning a contiguous range of rows and keeping loads_in_flight
+ * 16-block loads in flight; the library builds loads_in_flight = 3 only, deeper
+ * rings measured slower).  rows <= 8, in_features >= 4096,
+ * waves_total <= out_features.  New here. */
+int hipengine_gfx950_gguf_q8_1_fused_gemv_stream_tuned(int32_t ggml_type, const void* x, int32_t x_kind,
+                                                       const uint8_t* qweight, void* out, int32_t out_kind,
+                                                       int64_t rows, int64_t in_features, int64_t out_features,
+                                                       int32_t loads_in_flight, int32_t waves, int32_t waves_total,
+                                                       hipengine_stream_t stream);
+
+/* The "slab" form for Q4_K: one workgroup per CU owns rows_per_workgroup (<= 96;
+ * 0 = ceil(out_features / 256)) consecutive output rows, its waves split K in
+ * slices of one or two 256-value blocks and run on the int8 MFMA.  rows <= 8,
+ * 1024 <= in_features <= 6144.  New here. */
+int hipengine_gfx950_gguf_q4_k_q8_1_fused_gemv_slab_tuned(const void* x, int32_t x_kind, const uint8_t* qweight,
+                                                          void* out, int32_t out_kind, int64_t rows,
+                                                          int64_t in_features, int64_t out_features,
+                                                          int32_t rows_per_workgroup, hipengine_stream_t stream);
+
+/* The phased slab form of the fused Q4_K / Q5_K / Q6_K / Q8_0 GEMV with an explicit layout
+ * (0 = the planner's choice): `waves` <= 12 waves per workgroup split K by
+ * 256-value blocks, `blocks_per_wave` (1, 2 or 4) per wave and phase, on the
+ * int8 MFMA; `workgroups` share the output rows.  rows <= 8, in_features a
+ * multiple of 512 and >= 2048, weights 4-byte aligned and < 4 GiB.  The default
+ * dispatch uses this form for batches of 3 to 8 (Q4_K: where in_features > 6144,
+ * below that its slab form).  New here. */
+int hipengine_gfx950_gguf_q8_1_fused_gemv_pslab_tuned(int32_t ggml_type, const void* x, int32_t x_kind,
+                                                      const uint8_t* qweight, void* out, int32_t out_kind,
+                                                      int64_t rows, int64_t in_features, int64_t out_features,
+                                                      int32_t waves, int32_t blocks_per_wave, int32_t workgroups,
+                                                      hipengine_stream_t stream);
+
+/* Host only: the layout the library picks for a shape, as
+ * {batch_bucket, rows_per_lane, blocks_per_wave, k_slices, row_groups}.  New here. */
+int hipengine_gfx950_gguf_gemv_default_plan(int32_t ggml_type, int64_t rows, int64_t in_features,
+                                            int64_t out_features, int32_t* plan5);
+
+/* Host only: the kernel form the default dispatch takes for the first launch of a
+ * batch, as {form, rows in that launch}: form 0 row-strided, 1 run, 2 stream,
+ * 3 slab (Q4_K on the int8 MFMA), 4 phased slab (int8 MFMA).  Weights are assumed
+ * 4-byte aligned.  New here. */
+int hipengine_gfx950_gguf_gemv_default_form(int32_t ggml_type, int64_t rows, int64_t in_features,
+                                            int64_t out_features, int32_t* form2);
+
+/* The same Q4_K x DS4 GEMM with the kernel form chosen by the caller (benchmarks
+ * and tuning; no counterpart in hipEngine).  out_kind: 0 float32, 1 bf16, 2 fp16.
+ * variant 0: the next K step is prefetched into registers (what the named entry
+ * points run); variant 1: no prefetch, one more workgroup per CU. */
+int hipengine_gfx950_gguf_q4_k_mmq_tuned(const void* xq, const uint8_t* qweight, void* out, int out_kind,
+                                         int64_t rows, int64_t in_features, int64_t out_features, int variant,
+                                         hipengine_stream_t stream);
+
+#ifdef __cplusplus
+}
+#endif
+
+#endif /* HIPENGINE_GFX950_TUNING_H */
