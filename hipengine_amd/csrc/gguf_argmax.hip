@@ -6,6 +6,10 @@
 // stage 2 reduces a row's pairs.
 
 #include "gguf_common.hpp"
+#include "gguf_init.hpp"
+
+#include <atomic>
+#include <mutex>
 
 #include "../../include/hipengine_gfx950.h"
 
@@ -77,7 +81,78 @@ __global__ void __launch_bounds__(512) argmax_stage2_kernel(const float* __restr
   }
 }
 
+// ---- stage scratch held by the library, for callers that cannot allocate ----
+//
+// One (value, index) pair per stage-1 block, HIPENGINE_GFX950_ARGMAX_NOALLOC_MAX_ENTRIES pairs at most:
+// values in the first half of the array, indices in the second.  Every device the library runs on holds
+// its own copy of the array at its own address until the process ends; `scratch` is only a host-side
+// handle, the address kernels may use is the one hipGetSymbolAddress returns with that device current.
+constexpr int64_t kNoAllocEntries = HIPENGINE_GFX950_ARGMAX_NOALLOC_MAX_ENTRIES;
+static __device__ __align__(256) uint8_t scratch[kNoAllocEntries * (sizeof(float) + sizeof(int32_t))];
+
+constexpr int kMaxDevices = 64;
+std::mutex scratch_mutex;
+std::atomic<void*> scratch_ptr[kMaxDevices];   // per device, null until set up
+
 }  // namespace
+
+namespace hipengine_gfx950 {
+
+int argmax_noalloc_setup(int device) {
+  if (device < 0 || device >= kMaxDevices) return static_cast<int>(hipErrorInvalidDevice);
+  std::lock_guard<std::mutex> lock(scratch_mutex);
+  if (scratch_ptr[device].load(std::memory_order_acquire)) return static_cast<int>(hipSuccess);
+  void* ptr = nullptr;
+  const hipError_t err = hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch));
+  if (err != hipSuccess) return static_cast<int>(err);
+  if (!ptr) return static_cast<int>(hipErrorInvalidSymbol);
+  scratch_ptr[device].store(ptr, std::memory_order_release);
+  return static_cast<int>(hipSuccess);
+}
+
+}  // namespace hipengine_gfx950
+
+namespace {
+
+int launch_argmax(const float* logits, float* block_values, int32_t* block_indices, int32_t* out_indices,
+                  float* out_values, int64_t rows, int64_t vocab_size, int64_t threads, int64_t stage1_blocks,
+                  hipStream_t stream) {
+  const unsigned t = static_cast<unsigned>(threads);
+  hipLaunchKernelGGL(argmax_stage1_kernel, dim3(static_cast<unsigned>(stage1_blocks), static_cast<unsigned>(rows)),
+                     dim3(t), 0, stream, logits, block_values, block_indices, vocab_size, stage1_blocks);
+  const hipError_t err = hipGetLastError();
+  if (err != hipSuccess) return static_cast<int>(err);
+  hipLaunchKernelGGL(argmax_stage2_kernel, dim3(static_cast<unsigned>(rows)), dim3(t), 0, stream, block_values,
+                     block_indices, out_indices, out_values, stage1_blocks);
+  return static_cast<int>(hipGetLastError());
+}
+
+}  // namespace
+
+extern "C" int hipengine_gfx950_argmax_f32_rows_i32_noalloc(const float* logits, int32_t* out_indices,
+                                                            float* out_values, int64_t rows, int64_t vocab_size,
+                                                            int64_t threads, hipStream_t stream) {
+  if (!logits || !out_indices || rows <= 0 || rows > 65535 || vocab_size <= 0 || vocab_size > 0x7FFFFFFF ||
+      !(threads == 128 || threads == 256 || threads == 512)) {
+    return static_cast<int>(hipErrorInvalidValue);
+  }
+  const int64_t stage1_blocks = (vocab_size + threads * 4 - 1) / (threads * 4);
+  if (rows * stage1_blocks > kNoAllocEntries) return static_cast<int>(hipErrorInvalidValue);   // beyond the array
+  int device = -1;
+  hipError_t err = hipGetDevice(&device);
+  if (err != hipSuccess) return static_cast<int>(err);
+  if (device < 0 || device >= kMaxDevices) return static_cast<int>(hipErrorInvalidDevice);
+  if (!scratch_ptr[device].load(std::memory_order_acquire)) {   // first call on this device without hipengine_gfx950_init()
+    const int rc = hipengine_gfx950::argmax_noalloc_setup(device);
+    if (rc != static_cast<int>(hipSuccess)) return rc;
+  }
+  // Stage 1 writes every pair stage 2 reads, so nothing of the previous call's contents is consumed.
+  uint8_t* base = static_cast<uint8_t*>(scratch_ptr[device].load(std::memory_order_acquire));
+  float* block_values = reinterpret_cast<float*>(base);
+  int32_t* block_indices = reinterpret_cast<int32_t*>(base + kNoAllocEntries * sizeof(float));
+  return launch_argmax(logits, block_values, block_indices, out_indices, out_values, rows, vocab_size, threads,
+                       stage1_blocks, stream);
+}
 
 extern "C" int hipengine_argmax_f32_rows_i32(const float* logits, float* block_values, int32_t* block_indices,
                                              int32_t* out_indices, float* out_values, int64_t rows, int64_t vocab_size,
@@ -87,12 +162,6 @@ extern "C" int hipengine_argmax_f32_rows_i32(const float* logits, float* block_v
     return static_cast<int>(hipErrorInvalidValue);
   }
   const int64_t stage1_blocks = (vocab_size + threads * 4 - 1) / (threads * 4);
-  const unsigned t = static_cast<unsigned>(threads);
-  hipLaunchKernelGGL(argmax_stage1_kernel, dim3(static_cast<unsigned>(stage1_blocks), static_cast<unsigned>(rows)),
-                     dim3(t), 0, stream, logits, block_values, block_indices, vocab_size, stage1_blocks);
-  const hipError_t err = hipGetLastError();
-  if (err != hipSuccess) return static_cast<int>(err);
-  hipLaunchKernelGGL(argmax_stage2_kernel, dim3(static_cast<unsigned>(rows)), dim3(t), 0, stream, block_values,
-                     block_indices, out_indices, out_values, stage1_blocks);
-  return static_cast<int>(hipGetLastError());
+  return launch_argmax(logits, block_values, block_indices, out_indices, out_values, rows, vocab_size, threads,
+                       stage1_blocks, stream);
 }

@@ -1,6 +1,6 @@
 // Library set-up: hipengine_gfx950_init() does, once per device, everything a launch would otherwise
 // have to do on first use through a call that is not a stream operation - raising dynamic-LDS limits,
-// loading code objects - so that every entry point can be captured into a HIP
+// looking up the address of library-held scratch - so that every entry point can be captured into a HIP
 // graph from its very first call.  Launch paths call ensure_init() and so stay correct without it.
 
 #include <hip/hip_runtime.h>
@@ -31,6 +31,8 @@ extern "C" int hipengine_gfx950_init(void) {
   std::lock_guard<std::mutex> lock(init_mutex);
   if (device_ready[device].load(std::memory_order_relaxed)) return static_cast<int>(hipSuccess);
   int rc = hipengine_gfx950::gemv_raise_lds_limits();
+  if (rc != static_cast<int>(hipSuccess)) return rc;
+  rc = hipengine_gfx950::argmax_noalloc_setup(device);
   if (rc != static_cast<int>(hipSuccess)) return rc;
   int (*const loads[])() = {hipengine_gfx950::quantize_load, hipengine_gfx950::mmq_load, hipengine_gfx950::moe_load,
                             hipengine_gfx950::embedding_load};

@@ -8,6 +8,9 @@ namespace hipengine_gfx950 {
 // (gguf_gemv.hip).  Applies to the current device.
 int gemv_raise_lds_limits();
 
+// Look up this device's address of the arg-max stage scratch (gguf_argmax.hip).  `device` must be current.
+int argmax_noalloc_setup(int device);
+
 // Make the runtime load the code object of a source file now (it otherwise does so at the file's first
 // launch, which may be inside a stream capture): one per source file that has kernels and no other set-up.
 int quantize_load();

@@ -42,6 +42,32 @@ def argmax_f32_rows_i32(logits_f32_ptr: int, block_values_f32_ptr: int, block_in
                     out_values_f32_ptr or None, rows, vocab_size, threads, stream), runtime)
 
 
+NOALLOC_MAX_ENTRIES = 65536   # HIPENGINE_GFX950_ARGMAX_NOALLOC_MAX_ENTRIES
+
+
+def argmax_f32_rows_i32_noalloc(logits_f32_ptr: int, out_indices_i32_ptr: int, out_values_f32_ptr: int | None, rows: int,
+                                vocab_size: int, *, threads: int = 256, stream: int = 0,
+                                library: ctypes.CDLL | None = None, runtime: HipRuntime | None = None) -> None:
+    """``argmax_f32_rows_i32`` on scratch the library holds itself, for callers that cannot allocate
+    (no counterpart in hipEngine).  ``rows * ceil(vocab_size / (threads * 4))`` may not exceed
+    ``NOALLOC_MAX_ENTRIES``; calls that overlap on one device share the scratch and race."""
+    if rows <= 0:
+        raise ValueError("rows must be positive")
+    if vocab_size <= 0:
+        raise ValueError("vocab_size must be positive")
+    if threads not in _ALLOWED_THREADS:
+        raise ValueError("threads must be one of 128, 256, or 512")
+    if vocab_size > 2**31 - 1:
+        raise ValueError("vocab_size must fit int32 row-wise argmax outputs")
+    if argmax_scratch_entries(rows, vocab_size, threads) > NOALLOC_MAX_ENTRIES:
+        raise ValueError(f"rows * ceil(vocab_size / (threads * 4)) exceeds the library's scratch of {NOALLOC_MAX_ENTRIES} entries")
+    validate_pointers(logits_f32_ptr=logits_f32_ptr, out_indices_i32_ptr=out_indices_i32_ptr)
+    fn = entry("hipengine_gfx950_argmax_f32_rows_i32_noalloc", [VOID, VOID, VOID, I64, I64, I64, VOID], library)
+    check_launch(fn(logits_f32_ptr, out_indices_i32_ptr, out_values_f32_ptr or None, rows, vocab_size, threads, stream),
+                 runtime)
+
+
 def register_kernels(backend: str = "hip_gfx950", *, replace: bool = False) -> None:
     register(KernelKey(backend, "argmax", "f32", "rows_i32"), argmax_f32_rows_i32, replace=replace)
     register(KernelKey(backend, "argmax", "w4_paro", "f32_rows_i32"), argmax_f32_rows_i32, replace=replace)
+    register(KernelKey(backend, "argmax", "f32", "rows_i32_noalloc"), argmax_f32_rows_i32_noalloc, replace=replace)

@@ -47,7 +47,8 @@ typedef struct ihipStream_t* hipengine_stream_t; /* == hipStream_t */
 int hipengine_gfx950_abi_version(void);
 
 /* Per-device set-up, for the device that is current: raises the dynamic-LDS limit of every kernel
- * that may need more than the default 64 KB and loads the code objects.  Call it once per device after loading the library
+ * that may need more than the default 64 KB and looks up the address of the library-held scratch of
+ * hipengine_gfx950_argmax_f32_rows_i32_noalloc.  Call it once per device after loading the library
  * and before capturing a HIP graph; after it, no entry point makes any call that is not a stream
  * operation, so every one of them can be captured from its first launch on.  Entry points that need
  * the set-up run it themselves when it has not been done (then outside of a capture, please).
@@ -228,6 +229,20 @@ int hipengine_gguf_q8_0_embedding_bf16_out(const int64_t* token_ids, const uint8
 int hipengine_argmax_f32_rows_i32(const float* logits, float* block_values, int32_t* block_indices,
                                   int32_t* out_indices, float* out_values, int64_t rows, int64_t vocab_size,
                                   int64_t threads, hipengine_stream_t stream);
+
+/* The same arg-max for callers that cannot allocate device memory (code under HIP graph capture, tight
+ * serving loops, harnesses that forbid hipMalloc): the stage scratch is a fixed array inside the library
+ * instead of two caller buffers.  It has no counterpart in hipEngine.  Same results as
+ * hipengine_argmax_f32_rows_i32 with the same `threads`.  Limit: rows * ceil(vocab_size / (threads * 4))
+ * <= HIPENGINE_GFX950_ARGMAX_NOALLOC_MAX_ENTRIES, otherwise hipErrorInvalidValue (1) and nothing is
+ * launched.  The array (512 KiB per device, held until the process ends) is shared by every call on a
+ * device: calls that overlap on one device - different streams, or two graphs replayed concurrently -
+ * race on it; calls in stream order do not.  No call allocates, frees or synchronizes; the first call on
+ * a device looks up the array's address unless hipengine_gfx950_init() has done so. */
+#define HIPENGINE_GFX950_ARGMAX_NOALLOC_MAX_ENTRIES 65536
+int hipengine_gfx950_argmax_f32_rows_i32_noalloc(const float* logits, int32_t* out_indices, float* out_values,
+                                                 int64_t rows, int64_t vocab_size, int64_t threads,
+                                                 hipengine_stream_t stream);
 
 /* Router: for each of `tokens` rows of float32 logits (row pitch logits_stride), the top_k
  * experts by logit, highest first (equal logits: lowest index), as int64 into
