@@ -4,9 +4,7 @@
 
 #include "gguf_gemv.hpp"
 #include "gguf_gemv_run.hpp"
-#include "gguf_gemv_stream.hpp"
-#include "gguf_gemv_slab.hpp"
-#include "gguf_gemv_pslab.hpp"
+#include "gguf_gemv_launch.hpp"
 #include "gguf_init.hpp"
 
 #include "../../include/hipengine_gfx950.h"
@@ -111,199 +109,6 @@ const RunVariant* find_run_variant(int qt, int b, int g, int cb) {
   return nullptr;
 }
 
-constexpr size_t kMaxLds = 160 * 1024;   // LDS of one CU
-
-// ---- slab form (Q4_K on the int8 MFMA, one workgroup per CU, waves split K) ----
-
-// BPW = 1: up to 16 waves (K <= 4096); BPW = 2: up to 12 waves (K <= 6144), whose 64
-// operand registers want the 170-register budget of a 768-thread bound.
-template <int B, int BPW, int XK>
-__global__ void __launch_bounds__(BPW == 1 ? 1024 : 768) gemv_slab_q4k_kernel(GemvSlabArgs a) {
-  extern __shared__ __align__(16) uint8_t smem[];
-  gemv_slab_q4k_workgroup<B, BPW, XK>(a, smem);
-}
-
-using SlabKernelFn = void (*)(GemvSlabArgs);
-struct SlabVariant {
-  int b, bpw;
-  SlabKernelFn by_kind[4];
-};
-#define SLAB_VARIANT(B, BPW)                                                                            \
-  SlabVariant { B, BPW, {gemv_slab_q4k_kernel<B, BPW, KIND_F32>, gemv_slab_q4k_kernel<B, BPW, KIND_BF16>, \
-                         gemv_slab_q4k_kernel<B, BPW, KIND_F16>, gemv_slab_q4k_kernel<B, BPW, KIND_Q8_1>} }
-const SlabVariant kSlab[] = {SLAB_VARIANT(1, 1), SLAB_VARIANT(1, 2), SLAB_VARIANT(2, 1), SLAB_VARIANT(2, 2),
-                       SLAB_VARIANT(4, 1), SLAB_VARIANT(4, 2), SLAB_VARIANT(8, 1), SLAB_VARIANT(8, 2)};
-
-struct SlabPlan {
-  int b, bpw, waves, two_block_waves, rows_wg;
-  bool ok;
-};
-
-// K <= 4096: one block per wave (up to 16 waves).  4352 <= K <= 6144: 12 waves, the first nb - 12 of them
-// with two blocks, so that every SIMD gets three waves and (at K = 5120) five blocks.
-SlabPlan default_slab_plan(int qt, int rows, int64_t K, int64_t N) {
-  SlabPlan p{};
-  const int nb = static_cast<int>(K / QK_K);
-  p.b = rows <= 1 ? 1 : rows <= 2 ? 2 : rows <= 4 ? 4 : 8;
-  p.bpw = nb <= 16 ? 1 : 2;
-  p.waves = p.bpw == 1 ? nb : 12;
-  p.two_block_waves = p.bpw == 1 ? 0 : nb - 12;
-  const int64_t per_cu = (N + 255) / 256;
-  p.rows_wg = static_cast<int>(per_cu < 1 ? 1 : per_cu > SLAB_MAX_ROWS ? SLAB_MAX_ROWS : per_cu);
-  p.ok = qt == GGML_Q4_K && rows >= 1 && rows <= 8 && nb >= 4 && nb <= 24 &&
-         gemv_slab_lds_bytes(p.b, p.waves, p.two_block_waves) <= 160 * 1024;
-  return p;
-}
-
-int launch_gemv_slab(const void* x, int x_kind, const uint8_t* w, void* out, int out_kind, int rows, int64_t K,
-                     int64_t N, const SlabPlan& p, hipStream_t stream, const void* residual = nullptr,
-                     const void* gate = nullptr) {
-  const int nb = static_cast<int>(K / QK_K);
-  const SlabVariant* v = nullptr;
-  for (const SlabVariant& c : kSlab)
-    if (c.b == p.b && c.bpw == p.bpw) v = &c;
-  if (!v || rows > p.b || x_kind < KIND_F32 || x_kind > KIND_Q8_1 || p.rows_wg < 1 || p.rows_wg > SLAB_MAX_ROWS ||
-      p.waves < 1 || p.waves > (p.bpw == 1 ? 16 : 12) || p.two_block_waves < 0 || p.two_block_waves > p.waves ||
-      (p.bpw == 1 && p.two_block_waves != 0) || p.waves + p.two_block_waves != nb || K > (1 << 20) ||
-      N > (1 << 30)) {
-    return static_cast<int>(hipErrorInvalidValue);
-  }
-  const size_t lds = gemv_slab_lds_bytes(p.b, p.waves, p.two_block_waves);
-  if (lds > 160 * 1024) return static_cast<int>(hipErrorInvalidValue);
-  if (lds > 64 * 1024) {   // above the default dynamic limit: raised for every kernel by the library set-up
-    const int rc = ensure_init();
-    if (rc != static_cast<int>(hipSuccess)) return rc;
-  }
-  GemvSlabArgs a{x, w, out, x_kind, out_kind, rows, static_cast<int>(K), static_cast<int>(N), p.rows_wg, p.waves,
-                 p.two_block_waves, residual, gate};
-  const unsigned grid = static_cast<unsigned>((N + p.rows_wg - 1) / p.rows_wg);
-  hipLaunchKernelGGL(v->by_kind[x_kind], dim3(grid), dim3(p.waves * 64), lds, stream, a);
-  return static_cast<int>(hipGetLastError());
-}
-
-// ---- phased slab form (Q6_K / Q8_0, and Q4_K rows too long for the slab form, on the int8 MFMA; batch 3..8) ----
-
-template <int QT, int B, bool PHASED, int XK>
-__global__ void __launch_bounds__(768) gemv_pslab_kernel(GemvPslabArgs a) {
-  extern __shared__ __align__(16) uint8_t smem[];
-  gemv_pslab_workgroup<QT, B, PHASED, XK>(a, smem);
-}
-
-using PslabKernelFn = void (*)(GemvPslabArgs);
-struct PslabVariant {
-  int qt, b;
-  bool phased;
-  PslabKernelFn by_kind[4];
-};
-#define PSLAB_VARIANT(QT, B, P)                                                                              \
-  PslabVariant { QT, B, P, {gemv_pslab_kernel<QT, B, P, KIND_F32>, gemv_pslab_kernel<QT, B, P, KIND_BF16>,   \
-                            gemv_pslab_kernel<QT, B, P, KIND_F16>, gemv_pslab_kernel<QT, B, P, KIND_Q8_1>} }
-const PslabVariant kPslab[] = {PSLAB_VARIANT(GGML_Q5_K, 4, false), PSLAB_VARIANT(GGML_Q5_K, 4, true),
-                         PSLAB_VARIANT(GGML_Q5_K, 8, false), PSLAB_VARIANT(GGML_Q5_K, 8, true),
-                         PSLAB_VARIANT(GGML_Q4_K, 4, false), PSLAB_VARIANT(GGML_Q4_K, 4, true),
-                         PSLAB_VARIANT(GGML_Q4_K, 8, false), PSLAB_VARIANT(GGML_Q4_K, 8, true),
-                         PSLAB_VARIANT(GGML_Q6_K, 4, false), PSLAB_VARIANT(GGML_Q6_K, 4, true),
-                         PSLAB_VARIANT(GGML_Q6_K, 8, false), PSLAB_VARIANT(GGML_Q6_K, 8, true),
-                         PSLAB_VARIANT(GGML_Q8_0, 4, false), PSLAB_VARIANT(GGML_Q8_0, 4, true),
-                         PSLAB_VARIANT(GGML_Q8_0, 8, false), PSLAB_VARIANT(GGML_Q8_0, 8, true)};
-
-struct PslabPlan {
-  int b, waves, bpw_log2, phases, grid;
-  bool ok;
-};
-
-size_t pslab_lds_bytes(int qt, int b, int waves, int bpw) {
-  return static_cast<size_t>(waves) * (qt == GGML_Q6_K   ? pslab_wave_bytes<GGML_Q6_K>(b, bpw)
-                                       : qt == GGML_Q4_K ? pslab_wave_bytes<GGML_Q4_K>(b, bpw)
-                                       : qt == GGML_Q5_K ? pslab_wave_bytes<GGML_Q5_K>(b, bpw)
-                                                         : pslab_wave_bytes<GGML_Q8_0>(b, bpw));
-}
-
-int64_t pslab_row_bytes(int qt, int nb) {
-  return static_cast<int64_t>(nb) * (qt == GGML_Q6_K   ? Q6_K_BYTES
-                                     : qt == GGML_Q4_K ? Q4_K_BYTES
-                                     : qt == GGML_Q5_K ? Q5_K_BYTES
-                                                       : 8 * Q8_0_BYTES);
-}
-
-int pslab_grid(int64_t N, int phases) {
-  // one phase: a workgroup per CU walks its share of the rows group by group; several phases: a
-  // workgroup has one group of at most 96 rows
-  const int64_t groups = (N + PSLAB_GROUP_ROWS - 1) / PSLAB_GROUP_ROWS;
-  const int64_t per_cu = N < 256 ? N : 256;
-  return static_cast<int>(phases == 1 ? per_cu : (groups > per_cu ? groups : per_cu));
-}
-
-// Waves and blocks per wave: the split of K/256 blocks over W <= 12 waves x bpw in {1, 2, 4} slots x phases
-// that loads the four SIMDs most evenly, preferring a single phase (activations quantized once) and more
-// waves.
-PslabPlan default_pslab_plan(int qt, int rows, int64_t K, int64_t N, const void* w) {
-  PslabPlan p{};
-  const int nb = static_cast<int>(K / QK_K);
-  const int64_t row_bytes = pslab_row_bytes(qt, nb);
-  if ((qt != GGML_Q4_K && qt != GGML_Q5_K && qt != GGML_Q6_K && qt != GGML_Q8_0) || rows < 1 || rows > 8 || nb < 8 || (nb & 1) != 0 ||
-      (reinterpret_cast<uintptr_t>(w) & 3u) != 0 || N < 1 || row_bytes >= (1 << 24) || N * row_bytes > 0xFFFF0000ll) {
-    return p;
-  }
-  p.b = rows <= 4 ? 4 : 8;
-  float best = -1.0f;
-  for (int waves = 12; waves >= 6; --waves) {
-    for (int bl2 = 0; bl2 <= 2; ++bl2) {
-      const int bpw = 1 << bl2;
-      if (waves > nb || pslab_lds_bytes(qt, p.b, waves, bpw) > kMaxLds) continue;
-      const int phases = (nb + waves * bpw - 1) / (waves * bpw);
-      // wave w owns blocks w, w + waves, ...: the SIMD (w % 4) with the most blocks sets the pace
-      int simd_blocks[4] = {0, 0, 0, 0};
-      for (int w = 0; w < waves; ++w) simd_blocks[w & 3] += (nb - w + waves - 1) / waves;
-      int worst = 0;
-      for (int v : simd_blocks) worst = v > worst ? v : worst;
-      const float score = static_cast<float>(nb) / static_cast<float>(4 * worst) -
-                          0.02f * static_cast<float>(12 - waves) + (phases == 1 ? 0.05f : 0.0f) - 0.001f * bl2;
-      if (score > best) {
-        best = score;
-        p.waves = waves; p.bpw_log2 = bl2; p.phases = phases;
-      }
-    }
-  }
-  if (best < 0.0f) return p;
-  p.grid = pslab_grid(N, p.phases);
-  p.ok = true;
-  return p;
-}
-
-int launch_gemv_pslab(int qt, const void* x, int x_kind, const uint8_t* w, void* out, int out_kind, int rows,
-                      int64_t K, int64_t N, const PslabPlan& p, hipStream_t stream, const void* residual = nullptr,
-                      const void* gate = nullptr) {
-  const int nb = static_cast<int>(K / QK_K);
-  const int bpw = 1 << p.bpw_log2;
-  const int64_t row_bytes = pslab_row_bytes(qt, nb);
-  const PslabVariant* v = nullptr;
-  for (const PslabVariant& c : kPslab)
-    if (c.qt == qt && c.b == p.b && c.phased == (p.phases > 1)) v = &c;
-  if (!v || rows < 1 || rows > p.b || x_kind < KIND_F32 || x_kind > KIND_Q8_1 || p.waves < 1 || p.waves > 12 ||
-      p.bpw_log2 < 0 || p.bpw_log2 > 2 || p.waves > nb || (nb & 1) != 0 ||
-      p.phases != (nb + p.waves * bpw - 1) / (p.waves * bpw) || p.grid < 1 ||
-      (p.phases > 1 && static_cast<int64_t>(p.grid) * PSLAB_GROUP_ROWS < N) ||
-      (reinterpret_cast<uintptr_t>(w) & 3u) != 0 || row_bytes >= (1 << 24) || N * row_bytes > 0xFFFF0000ll) {
-    return static_cast<int>(hipErrorInvalidValue);
-  }
-  const size_t lds = pslab_lds_bytes(qt, p.b, p.waves, bpw);
-  if (lds > kMaxLds) return static_cast<int>(hipErrorInvalidValue);
-  if (lds > 64 * 1024) {
-    const int rc = ensure_init();
-    if (rc != static_cast<int>(hipSuccess)) return rc;
-  }
-  GemvPslabArgs a{};
-  a.x = x; a.w = w; a.out = out; a.residual = residual; a.gate = gate;
-  a.x_kind = x_kind; a.out_kind = out_kind; a.rows = rows;
-  a.K = static_cast<int>(K); a.N = static_cast<int>(N);
-  a.waves = p.waves; a.bpw_log2 = p.bpw_log2; a.phases = p.phases;
-  a.base_rows = static_cast<int>(N / p.grid);
-  a.w_bytes = static_cast<uint32_t>((N * row_bytes + 3) & ~3ll);
-  hipLaunchKernelGGL(v->by_kind[x_kind], dim3(static_cast<unsigned>(p.grid)), dim3(p.waves * 64), lds, stream, a);
-  return static_cast<int>(hipGetLastError());
-}
-
 int gcd_int(int a, int b) { return b == 0 ? a : gcd_int(b, a % b); }
 
 struct RunPlan {
@@ -354,197 +159,6 @@ int launch_gemv_run(int qt, const void* x, int x_kind, const uint8_t* w, void* o
   return static_cast<int>(hipGetLastError());
 }
 
-
-// ---- stream form (resident waves, ring of loads in flight) --------------------
-
-// Batch 1 kernels fit 170 registers and may run 12 waves per workgroup, which lets the
-// planner pick a wave count that divides the rows evenly.
-template <int B>
-constexpr int stream_max_threads() {
-  return B == 1 ? 768 : 512;
-}
-
-template <int QT, int B, int D, int S, int XK = -1, int FUSE = FUSE_NONE>
-__global__ void __launch_bounds__((stream_max_threads<B>())) gemv_stream_kernel(GemvStreamArgs a) {
-  extern __shared__ __align__(16) uint8_t smem[];
-  gemv_stream_workgroup<QT, B, D, S, XK, FUSE>(a, smem);
-}
-
-using StreamKernelFn = void (*)(GemvStreamArgs);
-
-// `long_k`: the instantiation that fetches five activation groups (of 8 values) per thread
-// up front (batch 1 only); the other fetches two (batch 1, 2) or one (batch 4, 8).
-// `fuse`: plain projection, gate/up pair with SiLU, or projection plus residual.
-struct StreamVariant {
-  int qt, b, d;
-  int s;         // activation groups (of 8 values) per thread fetched up front
-  bool long_k;
-  int fuse;
-  StreamKernelFn fn;
-  StreamKernelFn by_kind[4];   // instantiations with the activation kind fixed (null: use fn)
-};
-
-#define STREAM_VARIANT(QT, B, D) \
-  StreamVariant { QT, B, D, (B <= 2 ? 2 : 1), false, FUSE_NONE, gemv_stream_kernel<QT, B, D, (B <= 2 ? 2 : 1)>, {nullptr, nullptr, nullptr, nullptr} }
-#define STREAM_VARIANT_BY_KIND(QT, B, D, S, LONG_K)                                                      \
-  StreamVariant { QT, B, D, S, LONG_K, FUSE_NONE, gemv_stream_kernel<QT, B, D, S>,                        \
-                  {gemv_stream_kernel<QT, B, D, S, KIND_F32>, gemv_stream_kernel<QT, B, D, S, KIND_BF16>, \
-                   gemv_stream_kernel<QT, B, D, S, KIND_F16>, gemv_stream_kernel<QT, B, D, S, KIND_Q8_1>} }
-// fused epilogues: float32 and bf16 activations get instantiations of their own, the other kinds the generic one
-#define STREAM_VARIANT_FUSED_D(QT, B, D, S, LONG_K, FUSE)                                                        \
-  StreamVariant { QT, B, D, S, LONG_K, FUSE, gemv_stream_kernel<QT, B, D, S, -1, FUSE>,                           \
-                  {gemv_stream_kernel<QT, B, D, S, KIND_F32, FUSE>, gemv_stream_kernel<QT, B, D, S, KIND_BF16, FUSE>, \
-                   nullptr, nullptr} }
-#define STREAM_VARIANT_FUSED(QT, B, S, LONG_K, FUSE) STREAM_VARIANT_FUSED_D(QT, B, 3, S, LONG_K, FUSE)
-
-const StreamVariant kStream[] = {
-    STREAM_VARIANT_BY_KIND(GGML_Q4_K, 1, 3, 2, false), STREAM_VARIANT_BY_KIND(GGML_Q4_K, 2, 3, 2, false),
-    STREAM_VARIANT_BY_KIND(GGML_Q4_K, 1, 2, 2, false),
-    STREAM_VARIANT_BY_KIND(GGML_Q6_K, 1, 3, 2, false), STREAM_VARIANT_BY_KIND(GGML_Q6_K, 2, 3, 2, false),
-    STREAM_VARIANT_BY_KIND(GGML_Q8_0, 1, 3, 2, false), STREAM_VARIANT_BY_KIND(GGML_Q8_0, 2, 3, 2, false),
-    STREAM_VARIANT_BY_KIND(GGML_Q5_K, 1, 3, 2, false), STREAM_VARIANT_BY_KIND(GGML_Q5_K, 2, 3, 2, false),
-    STREAM_VARIANT_BY_KIND(GGML_Q5_K, 1, 3, 5, true),
-    STREAM_VARIANT_BY_KIND(GGML_Q4_K, 1, 3, 5, true), STREAM_VARIANT_BY_KIND(GGML_Q6_K, 1, 3, 5, true),
-    STREAM_VARIANT_BY_KIND(GGML_Q8_0, 1, 3, 5, true),
-    STREAM_VARIANT_BY_KIND(GGML_Q4_K, 2, 3, 5, true), STREAM_VARIANT_BY_KIND(GGML_Q6_K, 2, 3, 5, true),
-    STREAM_VARIANT(GGML_Q4_K, 4, 3), STREAM_VARIANT(GGML_Q4_K, 8, 3), STREAM_VARIANT(GGML_Q6_K, 4, 3),
-    STREAM_VARIANT(GGML_Q6_K, 8, 3), STREAM_VARIANT(GGML_Q8_0, 4, 3), STREAM_VARIANT(GGML_Q8_0, 8, 3),
-    // gate/up pair with SiLU (Q4_K) and projection + residual (Q4_K, Q6_K), batch 1 and 2
-    STREAM_VARIANT_FUSED(GGML_Q4_K, 1, 2, false, FUSE_PAIR), STREAM_VARIANT_FUSED(GGML_Q4_K, 2, 2, false, FUSE_PAIR),
-    STREAM_VARIANT_FUSED(GGML_Q4_K, 1, 2, false, FUSE_RESIDUAL), STREAM_VARIANT_FUSED(GGML_Q4_K, 2, 2, false, FUSE_RESIDUAL),
-    STREAM_VARIANT_FUSED(GGML_Q6_K, 1, 2, false, FUSE_RESIDUAL), STREAM_VARIANT_FUSED(GGML_Q6_K, 2, 2, false, FUSE_RESIDUAL),
-    STREAM_VARIANT_FUSED(GGML_Q4_K, 1, 5, true, FUSE_RESIDUAL), STREAM_VARIANT_FUSED(GGML_Q6_K, 1, 5, true, FUSE_RESIDUAL),
-    // the tall Q4_K shape at batch 1 on a ring of two (see tuned_stream_plan)
-    STREAM_VARIANT_FUSED_D(GGML_Q4_K, 1, 2, 2, false, FUSE_PAIR), STREAM_VARIANT_FUSED_D(GGML_Q4_K, 1, 2, 2, false, FUSE_RESIDUAL),
-};
-
-// The variant a launch takes: of those for (type, batch bucket, ring depth, epilogue), the one with the fewest
-// up-front groups per thread that still cover K with this many waves (nb*8 groups, 16 teams per wave);
-// if none does, the one with the most (its generic kernel loops over the rest).
-const StreamVariant* pick_stream_variant(int qt, int b, int d, int fuse, int nb, int waves) {
-  const StreamVariant* best = nullptr;
-  bool best_covers = false;
-  for (const StreamVariant& v : kStream) {
-    if (v.qt != qt || v.b != b || v.d != d || v.fuse != fuse) continue;
-    const bool covers = nb * 8 <= v.s * waves * 16;
-    if (!best || (covers && (!best_covers || v.s < best->s)) || (!covers && !best_covers && v.s > best->s)) {
-      best = &v;
-      best_covers = covers;
-    }
-  }
-  return best;
-}
-
-const StreamVariant* find_stream_variant(int qt, int b, int d, bool long_k = false, int fuse = FUSE_NONE) {
-  const StreamVariant* fallback = nullptr;
-  for (const StreamVariant& v : kStream) {
-    if (v.qt != qt || v.b != b || v.d != d || v.fuse != fuse) continue;
-    if (v.long_k == long_k) return &v;
-    if (!v.long_k) fallback = &v;
-  }
-  return fallback;
-}
-
-int batch_bucket(int rows) { return rows <= 1 ? 1 : rows <= 2 ? 2 : rows <= 4 ? 4 : 8; }
-
-struct StreamPlan {
-  int b, d, waves, waves_total;
-  bool ok;
-};
-
-constexpr int kComputeUnits = 256;   // MI355X
-
-// The stream form applies to K >= 4096 (a 16-block load then spans at most two
-// rows), batch <= 2, when every resident wave gets at least a few loads.
-StreamPlan default_stream_plan(int qt, int rows, int64_t K, int64_t N) {
-  StreamPlan p{};
-  const int nb = static_cast<int>(K / QK_K);
-  p.b = batch_bucket(rows);
-  p.d = 3;
-  p.waves = 8;
-  const int64_t total_loads = N * nb / 16;
-  // 8 resident waves per CU once every wave gets 3 loads or more, else 4 per CU
-  p.waves_total = total_loads >= 6144 ? kComputeUnits * 8 : kComputeUnits * 4;
-  if (p.b == 1 && total_loads >= 6144) {
-    // whole rows per wave: 8, 10 or 12 waves per CU, whichever splits the rows most
-    // evenly (N = 5120: 2.5 rows per wave at 8, exactly 2 at 10)
-    double best = 1e9;
-    for (int w = 8; w <= 12; w += 2) {
-      const int64_t wt = static_cast<int64_t>(kComputeUnits) * w;
-      if (wt > N) break;
-      const double imbalance = static_cast<double>((N + wt - 1) / wt) * wt / static_cast<double>(N);
-      if (imbalance < best - 0.1) { best = imbalance; p.waves = w; p.waves_total = static_cast<int>(wt); }
-    }
-  }
-  // every wave should get the ring's three loads; Q4_K at batch 1 still beats the slab form with two
-  // (5120 x 5120 on 10 waves per CU: 6.7 us against 7.8)
-  const int min_loads = (qt == GGML_Q4_K && p.b == 1) ? 2 : 3;
-  p.ok = rows <= 8 && nb >= 16 && total_loads >= min_loads * static_cast<int64_t>(p.waves_total) &&
-         N >= p.waves_total && gemv_run_lds_bytes(qt, p.b, static_cast<int>(K)) <= kMaxLds &&
-         find_stream_variant(qt, p.b, p.d) != nullptr;
-  return p;
-}
-
-// The plan the entry points launch with.  A tall Q4_K matrix at batch 1 (every wave of a 12-per-CU grid still
-// gets six loads: the 17408 x 5120 gate/up shape) runs 12 waves per CU with two loads in flight each:
-// measured 12.1 us against 12.3 for 8 waves with three (the same bytes in flight, rows split 6/5
-// instead of 9/8).
-// The fused forms take the same plan as the plain projection, so that their float32 sums are the same.
-StreamPlan tuned_stream_plan(int qt, int rows, int64_t K, int64_t N) {
-  StreamPlan p = default_stream_plan(qt, rows, K, N);
-  const int64_t nb = K / QK_K;
-  const int64_t wt = static_cast<int64_t>(kComputeUnits) * 12;
-  if (p.ok && qt == GGML_Q4_K && p.b == 1 && nb <= 32 && N * nb / 16 >= 6 * wt && find_stream_variant(qt, 1, 2) != nullptr &&
-      find_stream_variant(qt, 1, 2, false, FUSE_PAIR) != nullptr && find_stream_variant(qt, 1, 2, false, FUSE_RESIDUAL) != nullptr) {
-    p.d = 2;
-    p.waves = 12;
-    p.waves_total = static_cast<int>(wt);
-  }
-  return p;
-}
-
-struct StreamFusion {
-  int fuse = FUSE_NONE;
-  const uint8_t* w_up = nullptr;
-  const void* residual = nullptr;
-  int round_mid = 0;
-};
-
-int launch_gemv_stream(int qt, const void* x, int x_kind, const uint8_t* w, void* out, int out_kind, int rows,
-                       int64_t K, int64_t N, const StreamPlan& p, hipStream_t stream,
-                       const StreamFusion& fusion = StreamFusion()) {
-  const int nb = static_cast<int>(K / QK_K);
-  const StreamVariant* v = p.waves > 0 ? pick_stream_variant(qt, p.b, p.d, fusion.fuse, nb, p.waves) : nullptr;
-  if (!v || nb < 16 || rows > p.b || p.waves < 1 || p.waves > (p.b == 1 ? 12 : 8) || p.waves_total < p.waves ||
-      (p.waves_total % p.waves) != 0 || p.waves_total > N) {
-    return static_cast<int>(hipErrorInvalidValue);
-  }
-  size_t lds = gemv_run_lds_bytes(qt, p.b, static_cast<int>(K));
-  if (fusion.fuse == FUSE_PAIR) {
-    // gate results wait per wave; a wave may hold at most STREAM_PAIR_MAX_ROWS rows
-    if (!fusion.w_up || (N + p.waves_total - 1) / p.waves_total > STREAM_PAIR_MAX_ROWS) return static_cast<int>(hipErrorInvalidValue);
-    lds += static_cast<size_t>(p.waves) * p.b * STREAM_PAIR_MAX_ROWS * sizeof(float);
-  }
-  if (fusion.fuse == FUSE_RESIDUAL && !fusion.residual) return static_cast<int>(hipErrorInvalidValue);
-  if (lds > kMaxLds) return static_cast<int>(hipErrorInvalidValue);
-  // the kind-specialised kernels stage the whole row from the groups fetched up front
-  const bool up_front = nb * 8 <= v->s * p.waves * 16;
-  const StreamKernelFn fn =
-      (up_front && x_kind >= KIND_F32 && x_kind <= KIND_Q8_1 && v->by_kind[x_kind]) ? v->by_kind[x_kind] : v->fn;
-  if (lds > 64 * 1024) {
-    const int rc = ensure_init();
-    if (rc != static_cast<int>(hipSuccess)) return rc;
-  }
-  GemvStreamArgs a;
-  a.x = x; a.w = w; a.out = out;
-  a.x_kind = x_kind; a.out_kind = out_kind;
-  a.rows = rows; a.K = static_cast<int>(K); a.N = static_cast<int>(N);
-  a.waves = p.waves; a.waves_total = p.waves_total;
-  a.base_rows = static_cast<int>(N / p.waves_total);
-  a.w_up = fusion.w_up; a.residual = fusion.residual; a.round_mid = fusion.round_mid;
-  hipLaunchKernelGGL(fn, dim3(p.waves_total / p.waves), dim3(p.waves * 64), lds, stream, a);
-  return static_cast<int>(hipGetLastError());
-}
 
 struct Plan {
   int b, r, cb, ks, nrg;
@@ -667,29 +281,10 @@ int launch_gemv(int qt, const void* x, int x_kind, const uint8_t* w, void* out, 
 // Every slab, phased slab and stream kernel may be launched with more dynamic LDS than the 64 KB a kernel
 // gets by default; the limit is raised for all of them here, once per device, so that no launch has to.
 int hipengine_gfx950::gemv_raise_lds_limits() {
-  auto raise = [](const void* fn) {
-    return fn ? hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(kMaxLds))
-              : hipSuccess;
-  };
-  for (const SlabVariant& v : kSlab)
-    for (const SlabKernelFn fn : v.by_kind) {
-      const hipError_t e = raise(reinterpret_cast<const void*>(fn));
-      if (e != hipSuccess) return static_cast<int>(e);
-    }
-  for (const PslabVariant& v : kPslab)
-    for (const PslabKernelFn fn : v.by_kind) {
-      const hipError_t e = raise(reinterpret_cast<const void*>(fn));
-      if (e != hipSuccess) return static_cast<int>(e);
-    }
-  for (const StreamVariant& v : kStream) {
-    hipError_t e = raise(reinterpret_cast<const void*>(v.fn));
-    if (e != hipSuccess) return static_cast<int>(e);
-    for (const StreamKernelFn fn : v.by_kind) {
-      e = raise(reinterpret_cast<const void*>(fn));
-      if (e != hipSuccess) return static_cast<int>(e);
-    }
-  }
-  return static_cast<int>(hipSuccess);
+  int rc = slab_raise_lds_limits();
+  if (rc == static_cast<int>(hipSuccess)) rc = pslab_raise_lds_limits();
+  if (rc == static_cast<int>(hipSuccess)) rc = stream_raise_lds_limits();
+  return rc;
 }
 
 // ---- fused: float activations in, q8_1 quantization inside the kernel -------
@@ -715,6 +310,54 @@ DEFINE_FUSED_ALL(q4_k, GGML_Q4_K)
 DEFINE_FUSED_ALL(q5_k, GGML_Q5_K)
 DEFINE_FUSED_ALL(q6_k, GGML_Q6_K)
 DEFINE_FUSED_ALL(q8_0, GGML_Q8_0)
+
+// ---- hipEngine's dense names --------------------------------------------------
+//
+// hipengine_gguf_<q>_gemv_<act>_<out>_out is what hipEngine's dense wrappers bind and what its
+// dispatcher reaches through the ("linear", quant, "gemv_*" / "prefill_*") registry keys
+// (gguf_q4_k_gemv.hip:2483-2611, gguf_k_gemv.hip:5504-5560).  Here they are the fused kernels above:
+// the activations are quantized to q8_1 inside the kernel, so results follow the q8_1 arithmetic of
+// hipEngine's dp4a kernels, not the float-activation arithmetic of the kernels of the same name there.
+
+#define DEFINE_DENSE(QNAME, QT, ANAME, AKIND, ONAME, OKIND)                                               \
+  extern "C" int hipengine_gguf_##QNAME##_gemv_##ANAME##_##ONAME##_out(                                   \
+      const void* x, const uint8_t* qweight, void* out, int64_t rows, int64_t in_features,                \
+      int64_t out_features, int64_t threads, hipStream_t stream) {                                        \
+    (void)threads;                                                                                        \
+    return launch_gemv(QT, x, AKIND, qweight, out, OKIND, rows, in_features, out_features, nullptr,       \
+                       stream);                                                                           \
+  }
+
+// Two matrices over one activation (gate and up, or k and v): out_a = W_a x, out_b = W_b x
+// (gguf_k_gemv.hip:5546-5560; Q4_K has the form for its pack8 layout only, gguf_q4_k_gemv.hip:2970).
+#define DEFINE_DENSE_DUAL(QNAME, QT, ANAME, AKIND, ONAME, OKIND)                                          \
+  extern "C" int hipengine_gguf_##QNAME##_dual_gemv_##ANAME##_##ONAME##_out(                              \
+      const void* x, const uint8_t* qweight_a, const uint8_t* qweight_b, void* out_a, void* out_b,        \
+      int64_t rows, int64_t in_features, int64_t out_features, int64_t threads, hipStream_t stream) {     \
+    (void)threads;                                                                                        \
+    if (!qweight_b || !out_b) return static_cast<int>(hipErrorInvalidValue);                              \
+    const int rc = launch_gemv(QT, x, AKIND, qweight_a, out_a, OKIND, rows, in_features, out_features,    \
+                               nullptr, stream);                                                          \
+    if (rc != static_cast<int>(hipSuccess)) return rc;                                                    \
+    return launch_gemv(QT, x, AKIND, qweight_b, out_b, OKIND, rows, in_features, out_features, nullptr,   \
+                       stream);                                                                           \
+  }
+
+#define DEFINE_DENSE_ALL(QNAME, QT)                         \
+  DEFINE_DENSE(QNAME, QT, f32, KIND_F32, f32, KIND_F32)     \
+  DEFINE_DENSE(QNAME, QT, f32, KIND_F32, fp16, KIND_F16)    \
+  DEFINE_DENSE(QNAME, QT, fp16, KIND_F16, f32, KIND_F32)    \
+  DEFINE_DENSE(QNAME, QT, fp16, KIND_F16, fp16, KIND_F16)   \
+  DEFINE_DENSE(QNAME, QT, bf16, KIND_BF16, f32, KIND_F32)   \
+  DEFINE_DENSE(QNAME, QT, bf16, KIND_BF16, fp16, KIND_F16)  \
+  DEFINE_DENSE(QNAME, QT, bf16, KIND_BF16, bf16, KIND_BF16) \
+  DEFINE_DENSE_DUAL(QNAME, QT, f32, KIND_F32, f32, KIND_F32) \
+  DEFINE_DENSE_DUAL(QNAME, QT, bf16, KIND_BF16, bf16, KIND_BF16)
+
+DEFINE_DENSE_ALL(q4_k, GGML_Q4_K)
+DEFINE_DENSE_ALL(q5_k, GGML_Q5_K)
+DEFINE_DENSE_ALL(q6_k, GGML_Q6_K)
+DEFINE_DENSE_ALL(q8_0, GGML_Q8_0)
 
 // ---- pre-quantized q8_1 activations (36-byte blocks) ------------------------
 
@@ -850,6 +493,32 @@ extern "C" int hipengine_gfx950_gguf_q8_1_fused_gemv_pslab_tuned(int32_t ggml_ty
   if (workgroups > 0) p.grid = workgroups;
   return launch_gemv_pslab(ggml_type, x, x_kind, qweight, out, out_kind, static_cast<int>(rows), in_features,
                            out_features, p, stream);
+}
+
+// ---- verification: the int32 dots of the MFMA forms -------------------------------------
+
+extern "C" int hipengine_gfx950_gguf_gemv_mfma_dots_i32(int32_t ggml_type, int32_t form, const void* xq,
+                                                        const uint8_t* qweight, int32_t* dots, float* out,
+                                                        int64_t rows, int64_t in_features, int64_t out_features,
+                                                        hipStream_t stream) {
+  if (!xq || !qweight || !dots || !out || rows <= 0 || rows > 8 || in_features <= 0 || (in_features % QK_K) != 0 ||
+      out_features <= 0) {
+    return static_cast<int>(hipErrorInvalidValue);
+  }
+  // the batch bucket of 8 rows, whatever `rows` is: one verification instantiation per kernel
+  if (form == FORM_SLAB) {
+    const SlabPlan p = default_slab_plan(ggml_type, 8, in_features, out_features);
+    if (!p.ok) return static_cast<int>(hipErrorInvalidValue);
+    return launch_gemv_slab(xq, KIND_Q8_1, qweight, out, KIND_F32, static_cast<int>(rows), in_features, out_features, p,
+                            stream, nullptr, nullptr, dots);
+  }
+  if (form == FORM_PSLAB) {
+    const PslabPlan p = default_pslab_plan(ggml_type, 8, in_features, out_features, qweight);
+    if (!p.ok) return static_cast<int>(hipErrorInvalidValue);
+    return launch_gemv_pslab(ggml_type, xq, KIND_Q8_1, qweight, out, KIND_F32, static_cast<int>(rows), in_features,
+                             out_features, p, stream, nullptr, nullptr, dots);
+  }
+  return static_cast<int>(hipErrorInvalidValue);
 }
 
 // ---- fused epilogues: gate/up pair with SiLU, projection + residual -------------------

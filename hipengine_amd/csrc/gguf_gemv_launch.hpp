@@ -1,0 +1,59 @@
+// Launch interface between the translation units of the decode GEMV: the dispatcher and C entry points
+// (gguf_gemv.hip) and the kernel families, each compiled on its own (gguf_gemv_stream.hip,
+// gguf_gemv_slab.hip, gguf_gemv_pslab.hip).  A plan says how a family would run a shape (`ok` false: it
+// does not take it); launch_* validates the plan again and launches.  All return a hipError_t as int.
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+namespace hipengine_gfx950 {
+
+constexpr size_t kMaxLds = 160 * 1024;   // LDS of one CU
+constexpr int kComputeUnits = 256;       // MI355X
+
+inline int batch_bucket(int rows) { return rows <= 1 ? 1 : rows <= 2 ? 2 : rows <= 4 ? 4 : 8; }
+
+// ---- slab form (Q4_K on the int8 MFMA, one workgroup per CU, waves split K) ----
+struct SlabPlan {
+  int b, bpw, waves, two_block_waves, rows_wg;
+  bool ok;
+};
+SlabPlan default_slab_plan(int qt, int rows, int64_t K, int64_t N);
+int launch_gemv_slab(const void* x, int x_kind, const uint8_t* w, void* out, int out_kind, int rows, int64_t K,
+                     int64_t N, const SlabPlan& p, hipStream_t stream, const void* residual = nullptr,
+                     const void* gate = nullptr, int32_t* dots_out = nullptr);
+int slab_raise_lds_limits();
+
+// ---- phased slab form (int8 MFMA; batch 3..8) ----
+struct PslabPlan {
+  int b, waves, bpw_log2, phases, grid;
+  bool ok;
+};
+PslabPlan default_pslab_plan(int qt, int rows, int64_t K, int64_t N, const void* w);
+int pslab_grid(int64_t N, int phases);
+int launch_gemv_pslab(int qt, const void* x, int x_kind, const uint8_t* w, void* out, int out_kind, int rows,
+                      int64_t K, int64_t N, const PslabPlan& p, hipStream_t stream, const void* residual = nullptr,
+                      const void* gate = nullptr, int32_t* dots_out = nullptr);
+int pslab_raise_lds_limits();
+
+// ---- stream form (resident waves, ring of loads in flight) ----
+enum StreamFuse { FUSE_NONE = 0, FUSE_PAIR = 1, FUSE_RESIDUAL = 2 };   // epilogue of the stream kernels
+struct StreamPlan {
+  int b, d, waves, waves_total;
+  bool ok;
+};
+struct StreamFusion {
+  int fuse = FUSE_NONE;
+  const uint8_t* w_up = nullptr;
+  const void* residual = nullptr;
+  int round_mid = 0;
+};
+StreamPlan default_stream_plan(int qt, int rows, int64_t K, int64_t N);
+StreamPlan tuned_stream_plan(int qt, int rows, int64_t K, int64_t N);
+int launch_gemv_stream(int qt, const void* x, int x_kind, const uint8_t* w, void* out, int out_kind, int rows,
+                       int64_t K, int64_t N, const StreamPlan& p, hipStream_t stream,
+                       const StreamFusion& fusion = StreamFusion());
+int stream_raise_lds_limits();
+
+}  // namespace hipengine_gfx950

@@ -57,6 +57,7 @@ struct GemvPslabArgs {
   int phases;      // ceil(K/256 / (W*bpw))
   int base_rows;   // N / gridDim.x; the first N % gridDim.x workgroups own one row more
   uint32_t w_bytes;   // N * row bytes, rounded up to a multiple of 4
+  int32_t* dots_out;  // verification kernels only: int32 [rows, N, K/32] (Q6_K: K/16, signed dots), as block_dots writes them
 };
 
 constexpr int PSLAB_GROUP_ROWS = 96;
@@ -101,7 +102,8 @@ constexpr int pslab_wave_bytes(int B, int bpw) {
 
 // XK fixes the activation kind at compile time: the staging code of the other kinds is then not
 // generated (it is most of the kernel's code, and cold instruction fetch is launch latency).
-template <int QT, int B, bool PHASED, int XK>
+// DUMP: the verification instantiation, which also writes every int32 sub-block dot to a.dots_out.
+template <int QT, int B, bool PHASED, int XK, bool DUMP = false>
 __device__ __forceinline__ void gemv_pslab_workgroup(const GemvPslabArgs& a, uint8_t* smem) {
   using T = PslabTraits<QT>;
   constexpr int VB = B < 4 ? B : 4;
@@ -274,7 +276,14 @@ __device__ __forceinline__ void gemv_pslab_workgroup(const GemvPslabArgs& a, uin
   };
 
   // ---- one unit: weights of block kb (image in `stage`) x activations of slot -> acc[v] for batch rows 4g+v
-  auto compute = [&](int slot, int kb, float (&acc)[VB]) {
+  // (row0, rows_here: first output row of the unit's step and how many of its 32 rows exist; DUMP only)
+  auto compute = [&](int slot, int kb, float (&acc)[VB], int row0, int rows_here) {
+    auto dump = [&](int index, int per_row, int v, int value) {
+      const int m = 4 * g + v;
+      if (m < a.rows && n < rows_here)
+        a.dots_out[(static_cast<int64_t>(m) * a.N + row0 + n) * per_row + index] = value;
+    };
+    (void)dump;
     const uint8_t* xl = xq + min(n, B - 1) * XQ_PITCH + slot * 256;     // A operand row (rows >= B: results dropped)
     const float* xdp = reinterpret_cast<const float*>(rec + slot * T::REC_SLOT);
 #pragma unroll
@@ -336,6 +345,10 @@ __device__ __forceinline__ void gemv_pslab_workgroup(const GemvPslabArgs& a, uin
           const ps_v16i r = __builtin_amdgcn_mfma_i32_32x32x16_i8(xop, wop, zero16, 0, 0, 0);
 #pragma unroll
           for (int v = 0; v < VB; ++v) dots[l][v] = r[v] + act.cs[l][v];   // signed dot: sum x*(u - 32)
+          if constexpr (DUMP) {
+#pragma unroll
+            for (int v = 0; v < VB; ++v) dump(kb * 16 + 2 * j32 + l, a.K / 16, v, dots[l][v]);
+          }
         }
         const uint32_t sw = j32 < 2 ? scw.x : j32 < 4 ? scw.y : j32 < 6 ? scw.z : scw.w;
         const int sc0 = static_cast<int>(sw << (16 - 16 * (j32 & 1) + 8)) >> 24;   // int8 scale of group 2*j32
@@ -384,6 +397,10 @@ __device__ __forceinline__ void gemv_pslab_workgroup(const GemvPslabArgs& a, uin
           }
           const ps_v4i xop = *reinterpret_cast<const ps_v4i*>(xl + sb * 32 + 16 * g);
           const ps_v16i r = __builtin_amdgcn_mfma_i32_32x32x32_i8(xop, wop, zero16, 0, 0, 0);
+          if constexpr (DUMP) {
+#pragma unroll
+            for (int v = 0; v < VB; ++v) dump(kb * 8 + sb, a.K / 32, v, r[v]);
+          }
           const ps_f4 xd4 = *reinterpret_cast<const ps_f4*>(xdp + sb * 8 + 4 * g);
           const ps_f4 xs4 = *reinterpret_cast<const ps_f4*>(xdp + 64 + sb * 8 + 4 * g);
           const uint32_t sc = ((sb < 4 ? u.sc_lo : u.sc_hi) >> (8 * (sb & 3))) & 0xFFu;
@@ -424,6 +441,10 @@ __device__ __forceinline__ void gemv_pslab_workgroup(const GemvPslabArgs& a, uin
         const ps_v4i wop = ps_v4i{static_cast<int>(ops.wv.x), static_cast<int>(ops.wv.y), static_cast<int>(ops.wv.z),
                                   static_cast<int>(ops.wv.w)};
         const ps_v16i r = __builtin_amdgcn_mfma_i32_32x32x32_i8(ops.xop, wop, zero16, 0, 0, 0);
+        if constexpr (DUMP) {
+#pragma unroll
+          for (int v = 0; v < VB; ++v) dump(kb * 8 + i, a.K / 32, v, r[v]);
+        }
 #pragma unroll
         for (int v = 0; v < VB; ++v) {
           const float tv = dw * static_cast<float>(r[v]);    // |dot| < 2^24: one rounding
@@ -476,7 +497,7 @@ __device__ __forceinline__ void gemv_pslab_workgroup(const GemvPslabArgs& a, uin
           issue(PHASED ? o1 : i1, PHASED ? i1 : o1, g1, min(PSLAB_GROUP_ROWS, nrows - g1));
         }
         float acc[VB];
-        compute(j & (bpw - 1), kb_of(j), acc);
+        compute(j & (bpw - 1), kb_of(j), acc, r_begin + g0 + 32 * t, min(grows - 32 * t, 32));
         if constexpr (PHASED) {
 #pragma unroll
           for (int u = 0; u < MAX_STEPS; ++u)

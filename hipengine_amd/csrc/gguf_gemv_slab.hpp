@@ -62,6 +62,7 @@ struct GemvSlabArgs {
   int two_block_waves;   // waves 0..two_block_waves-1 own two K blocks each, the rest one
   const void* residual;   // null, or [rows, N] of the output type: out = round(projection) + residual
   const void* gate;       // null, or [rows, N] of the output type (may be `out` itself): out = silu(gate) * round(projection)
+  int32_t* dots_out;      // verification kernels only: int32 [rows, N, K/32], every sub-block dot as the MFMA returns it
 };
 
 constexpr int SLAB_MAX_ROWS = 96;
@@ -81,7 +82,8 @@ inline size_t gemv_slab_lds_bytes(int b, int waves, int two_block_waves) {
          static_cast<size_t>(waves - two_block_waves) * slab_wave_bytes(b, 1);
 }
 
-template <int B, int BPW, int XK>
+// VERIFY: the verification instantiation, which also writes every int32 sub-block dot to a.dots_out.
+template <int B, int BPW, int XK, bool VERIFY = false>
 __device__ __forceinline__ void gemv_slab_q4k_workgroup(const GemvSlabArgs& a, uint8_t* smem) {
   constexpr int VB = B < 4 ? B : 4;                  // result registers in use per lane
   constexpr int NL = (32 * BPW * 9 + 63) / 64;       // 16-byte loads per lane and step
@@ -275,6 +277,15 @@ __device__ __forceinline__ void gemv_slab_q4k_workgroup(const GemvSlabArgs& a, u
 #pragma unroll
             for (int v = 0; v < 16; ++v) c0[v] = 0;
             const sl_v16i dots = __builtin_amdgcn_mfma_i32_32x32x32_i8(xop, wop, c0, 0, 0, 0);
+            if constexpr (VERIFY) {
+              const int row = 32 * t + n;
+#pragma unroll
+              for (int v = 0; v < VB; ++v) {
+                const int m = 4 * g + v;
+                if (m < a.rows && row < rows_wg)
+                  a.dots_out[(static_cast<int64_t>(m) * a.N + r0 + row) * (a.K / 32) + (kb0 + s) * 8 + sb] = dots[v];
+              }
+            }
             const uint32_t sc = ((sb < 4 ? u.sc_lo : u.sc_hi) >> (8 * (sb & 3))) & 0xFFu;
             const uint32_t mn = ((sb < 4 ? u.mn_lo : u.mn_hi) >> (8 * (sb & 3))) & 0xFFu;
             const float sw = d * static_cast<float>(sc);

@@ -22,6 +22,7 @@
 // padded layout of gguf_gemv_run.hpp.
 #pragma once
 
+#include "gguf_gemv_launch.hpp"
 #include "gguf_gemv_run.hpp"
 
 namespace hipengine_gfx950 {
@@ -43,7 +44,6 @@ struct GemvStreamArgs {
   int round_mid;            // FUSE_PAIR: round gate and up to the output type before the SiLU
 };
 
-enum StreamFuse { FUSE_NONE = 0, FUSE_PAIR = 1, FUSE_RESIDUAL = 2 };
 constexpr int STREAM_PAIR_MAX_ROWS = 16;   // rows per wave the pair form can hold back (gate results wait for up)
 
 // XK >= 0 fixes the activation kind at compile time (the staging code of the other

@@ -63,6 +63,28 @@ __global__ void __launch_bounds__(THREADS, 2) mmq_q4_k_ds4_kernel(MmqArgs a) {
       });
 }
 
+// Verification: the same tile engine, which also writes every int32 sub-block dot to dots[M, N, K/32].
+__global__ void __launch_bounds__(THREADS, 2) mmq_q4_k_ds4_dump_kernel(MmqArgs a, int32_t* __restrict__ dots) {
+  extern __shared__ __align__(16) uint8_t smem_raw[];
+  DenseQ4::Smem& s = *reinterpret_cast<DenseQ4::Smem*>(smem_raw);
+  const int m0 = blockIdx.x * BM, n0 = blockIdx.y * BN;
+  const int steps = a.K / 128;
+  const int64_t w_row_bytes = static_cast<int64_t>(a.K / QK_K) * Q4_K_BYTES;
+  const int64_t x_row_bytes = static_cast<int64_t>(steps) * DS4_BYTES;
+  auto row_of = [=](int row) { return static_cast<int64_t>(min(m0 + row, a.M - 1)); };
+  auto col_of = [=](int col) { return static_cast<int64_t>(min(n0 + col, a.N - 1)); };
+  auto emit = [=](int row, int col, float v) {
+    const int m = m0 + row, n = n0 + col;
+    if (m < a.M && n < a.N) store_scalar(a.out, static_cast<int64_t>(m) * a.N + n, v, a.out_kind);
+  };
+  auto dump = [=](int row, int col, int sb, int dot) {
+    const int m = m0 + row, n = n0 + col;
+    if (m < a.M && n < a.N) dots[(static_cast<int64_t>(m) * a.N + n) * (a.K / 32) + sb] = dot;
+  };
+  DenseQ4::run<true, decltype(row_of), decltype(col_of), decltype(emit), true, decltype(dump)>(
+      a.xq, x_row_bytes, a.w, w_row_bytes, steps, s, row_of, col_of, emit, dump);
+}
+
 int launch_q4(const void* xq, const uint8_t* w, void* out, int out_kind, int64_t M, int64_t K, int64_t N,
               int variant, hipStream_t stream) {
   if (!xq || !w || !out || M <= 0 || M > (1 << 20) || K <= 0 || (K % QK_K) != 0 || N <= 0 || (N % 32) != 0 ||
@@ -170,7 +192,9 @@ __device__ __forceinline__ void q6_step_store(Q6Smem& s, int tid, const Q6StepRe
   }
 }
 
-__global__ void __launch_bounds__(THREADS, 2) mmq_q6_k_d4s4_kernel(MmqArgs a) {
+// DUMP: the verification instantiation, which also writes every int32 16-value dot to dots[M, N, K/16].
+template <bool DUMP>
+__global__ void __launch_bounds__(THREADS, 2) mmq_q6_k_d4s4_kernel(MmqArgs a, int32_t* __restrict__ dots) {
   extern __shared__ __align__(16) uint8_t smem_raw[];
   Q6Smem& s = *reinterpret_cast<Q6Smem*>(smem_raw);
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
@@ -238,6 +262,17 @@ __global__ void __launch_bounds__(THREADS, 2) mmq_q6_k_d4s4_kernel(MmqArgs a) {
           xdv[4 * j] = t.x; xdv[4 * j + 1] = t.y; xdv[4 * j + 2] = t.z; xdv[4 * j + 3] = t.w;
         }
         const int col = wn * 64 + nt * 32 + lc;
+        if constexpr (DUMP) {
+#pragma unroll
+          for (int v = 0; v < 16; ++v) {
+            const int m = m0 + wm * 64 + mt * 32 + 8 * (v >> 2) + 4 * g + (v & 3), nn = n0 + col;
+            if (m < a.M && nn < a.N) {
+              int32_t* o = dots + (static_cast<int64_t>(m) * a.N + nn) * (a.K / 16) + (step * 4 + sl) * 2;
+              o[0] = cur.d0[v] - static_cast<int>(MAGIC_BITS);
+              o[1] = cur.d1[v] - static_cast<int>(MAGIC_BITS);
+            }
+          }
+        }
         const float s0 = s.sw[2 * sl][col], c0 = s.cw[2 * sl][col];
         const float s1 = s.sw[2 * sl + 1][col], c1 = s.cw[2 * sl + 1][col];
 #pragma unroll
@@ -268,7 +303,8 @@ int launch_q6(const void* xq, const uint8_t* w, void* out, int out_kind, int64_t
   MmqArgs a{static_cast<const uint8_t*>(xq), w, out, out_kind, static_cast<int>(M), static_cast<int>(K),
             static_cast<int>(N)};
   const dim3 grid(static_cast<unsigned>((M + BM - 1) / BM), static_cast<unsigned>((N + BN - 1) / BN));
-  hipLaunchKernelGGL(mmq_q6_k_d4s4_kernel, grid, dim3(THREADS), sizeof(Q6Smem), stream, a);
+  hipLaunchKernelGGL(mmq_q6_k_d4s4_kernel<false>, grid, dim3(THREADS), sizeof(Q6Smem), stream, a,
+                     static_cast<int32_t*>(nullptr));
   return static_cast<int>(hipGetLastError());
 }
 
@@ -300,7 +336,63 @@ DEFINE_MMQ_Q4(hipengine_gguf_q4_k_q8_1_mmq32_ctl_dense_bf16_bf16_out, KIND_BF16)
 DEFINE_MMQ_Q6(hipengine_gguf_q6_k_mmq32_q8_1_d4s4_f32_bf16_f32_out, KIND_F32)
 DEFINE_MMQ_Q6(hipengine_gguf_q6_k_mmq32_q8_1_d4s4_f32_bf16_bf16_out, KIND_BF16)
 
+// ---- verification: the int32 dots the MMQ kernels feed their float32 combine with ----
+
+extern "C" int hipengine_gfx950_gguf_mmq_dots_i32(int32_t ggml_type, const void* xq, const uint8_t* qweight,
+                                                  int32_t* dots, float* out, int64_t rows, int64_t in_features,
+                                                  int64_t out_features, hipStream_t stream) {
+  if (!xq || !qweight || !dots || !out || rows <= 0 || rows > (1 << 20) || in_features <= 0 ||
+      (in_features % QK_K) != 0 || out_features <= 0 || out_features > (1 << 24)) {
+    return static_cast<int>(hipErrorInvalidValue);
+  }
+  MmqArgs a{static_cast<const uint8_t*>(xq), qweight, out, KIND_F32, static_cast<int>(rows),
+            static_cast<int>(in_features), static_cast<int>(out_features)};
+  const dim3 grid(static_cast<unsigned>((rows + BM - 1) / BM), static_cast<unsigned>((out_features + BN - 1) / BN));
+  if (ggml_type == GGML_Q4_K) {
+    if ((out_features % 32) != 0) return static_cast<int>(hipErrorInvalidValue);
+    hipLaunchKernelGGL(mmq_q4_k_ds4_dump_kernel, grid, dim3(THREADS), sizeof(DenseQ4::Smem), stream, a, dots);
+  } else if (ggml_type == GGML_Q6_K) {
+    hipLaunchKernelGGL(mmq_q6_k_d4s4_kernel<true>, grid, dim3(THREADS), sizeof(Q6Smem), stream, a, dots);
+  } else {
+    return static_cast<int>(hipErrorInvalidValue);
+  }
+  return static_cast<int>(hipGetLastError());
+}
+
+// ---- prefill from bf16 activations: pack into the caller's workspace, then the MMQ ----
+
+extern "C" int hipengine_gfx950_gguf_prefill_workspace_bytes(int32_t ggml_type, int64_t rows, int64_t in_features,
+                                                             int64_t* bytes) {
+  if (!bytes || rows <= 0 || in_features <= 0 || (in_features % QK_K) != 0 ||
+      (ggml_type != GGML_Q4_K && ggml_type != GGML_Q6_K)) {
+    return static_cast<int>(hipErrorInvalidValue);
+  }
+  *bytes = rows * (in_features / 128) * (ggml_type == GGML_Q4_K ? DS4_BYTES : D4S4_BYTES);
+  return static_cast<int>(hipSuccess);
+}
+
+extern "C" int hipengine_gfx950_gguf_prefill_bf16(int32_t ggml_type, const void* x, const uint8_t* qweight, void* out,
+                                                  int32_t out_kind, int64_t rows, int64_t in_features,
+                                                  int64_t out_features, void* workspace, int64_t workspace_bytes,
+                                                  hipStream_t stream) {
+  int64_t need = 0;
+  const int rc = hipengine_gfx950_gguf_prefill_workspace_bytes(ggml_type, rows, in_features, &need);
+  if (rc != static_cast<int>(hipSuccess)) return rc;
+  if (!x || !workspace || workspace_bytes < need || (reinterpret_cast<uintptr_t>(workspace) & 15u) != 0) {
+    return static_cast<int>(hipErrorInvalidValue);
+  }
+  if (ggml_type == GGML_Q4_K) {
+    if ((out_features % 32) != 0) return static_cast<int>(hipErrorInvalidValue);
+    const int prc = hipengine_gguf_q8_1_mmq_ds4_pack_bf16(x, workspace, rows, in_features, stream);
+    if (prc != static_cast<int>(hipSuccess)) return prc;
+    return launch_q4(workspace, qweight, out, out_kind, rows, in_features, out_features, 0, stream);
+  }
+  const int prc = hipengine_gguf_q8_1_d4s4_f32_quantize_bf16(x, workspace, rows, in_features, stream);
+  if (prc != static_cast<int>(hipSuccess)) return prc;
+  return launch_q6(workspace, qweight, out, out_kind, rows, in_features, out_features, stream);
+}
+
 int hipengine_gfx950::mmq_load() {
   hipFuncAttributes attr;
-  return static_cast<int>(hipFuncGetAttributes(&attr, reinterpret_cast<const void*>(mmq_q6_k_d4s4_kernel)));
+  return static_cast<int>(hipFuncGetAttributes(&attr, reinterpret_cast<const void*>(mmq_q6_k_d4s4_kernel<false>)));
 }

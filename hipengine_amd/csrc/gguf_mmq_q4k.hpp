@@ -149,9 +149,11 @@ struct Q4Tile {
     }
   }
 
-  // One K step of MFMA work on the LDS images; acc is [NT][MT][16].
+  // One K step of MFMA work on the LDS images; acc is [NT][MT][16].  `dump(row, col, sub_block, dot)`
+  // receives every int32 sub-block dot (tile-relative row and column, sub-block of the K step) when DUMP.
+  template <bool DUMP = false, class Dump = int>
   static __device__ __forceinline__ void compute(const Smem& s, int step, int wm, int wn, int lc, int g,
-                                                 float (&acc)[NT][MT][16]) {
+                                                 float (&acc)[NT][MT][16], Dump dump = 0) {
     const int h = step & 1;
     v16i c0;
 #pragma unroll
@@ -212,6 +214,12 @@ struct Q4Tile {
           const int i = pr * NT + nt;
           v16i dnext = dcur;
           if (i + 1 < TILES) dnext = issue(i + 1);
+          if constexpr (DUMP) {
+#pragma unroll
+            for (int v = 0; v < 16; ++v)
+              dump((wm * MT + mt) * 32 + 8 * (v >> 2) + 4 * g + (v & 3), (wn * NT + nt) * 32 + lc, 2 * sp + pr / MT,
+                   dcur[v] - static_cast<int>(MMQ_MAGIC_BITS));
+          }
 #pragma unroll
           for (int v = 0; v < 16; ++v) {
             const float t = __builtin_fmaf(bits_to_float(static_cast<uint32_t>(dcur[v])), ops.sw[nt], ops.cw[nt]);   // = sw * dot, rounded once
@@ -246,10 +254,10 @@ struct Q4Tile {
 
   // The whole K loop of one output tile.  `emit(row, col, value)` receives every
   // element of the tile (tile-relative coordinates) once.
-  template <bool PREFETCH, class RowOf, class ColOf, class Emit>
+  template <bool PREFETCH, class RowOf, class ColOf, class Emit, bool DUMP = false, class Dump = int>
   static __device__ __forceinline__ void run(const uint8_t* xq, int64_t x_row_bytes, const uint8_t* w,
                                              int64_t w_row_bytes, int steps, Smem& s, RowOf row_of, ColOf col_of,
-                                             Emit emit) {
+                                             Emit emit, Dump dump = 0) {
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int wm = wave % WM, wn = wave / WM;
     const int lc = lane & 31, g = lane >> 5;
@@ -271,7 +279,11 @@ struct Q4Tile {
       // The loads of the next step are issued before this step is computed, so
       // their latency hides behind the MFMA/FMA work.
       if (PREFETCH && step + 1 < steps) load(xq, x_row_bytes, w, w_row_bytes, step + 1, tid, row_of, col_of, regs);
-      compute(s, step, wm, wn, lc, g, acc);
+      if constexpr (DUMP) {
+        compute<true>(s, step, wm, wn, lc, g, acc, [&](int row, int col, int sb, int dot) { dump(row, col, 4 * step + sb, dot); });
+      } else {
+        compute(s, step, wm, wn, lc, g, acc);
+      }
       __syncthreads();   // the next step overwrites the tiles
     }
 

@@ -241,6 +241,148 @@ __global__ void moe_invert_kernel(const int64_t* __restrict__ sorted_lanes, int6
   }
 }
 
+// ---- the count / prefix / scatter pipeline hipEngine's runner drives step by step ----
+// (runtime/qwen35_gguf_runner.py:34107-34143; kernels moe/group_scatter.hip:9-60,391-485)
+
+// counts[e] += lanes routed to e.  The caller zeroes counts (int32), as in hipEngine.
+__global__ void __launch_bounds__(256) moe_group_count_kernel(const int64_t* __restrict__ selected,
+                                                              int32_t* __restrict__ counts, int64_t lanes,
+                                                              int64_t num_experts) {
+  const int64_t lane = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x;
+  if (lane >= lanes) return;
+  const int64_t e = selected[lane];
+  if (e >= 0 && e < num_experts) atomicAdd(&counts[e], 1);
+}
+
+// One workgroup of 1024: padded_counts[e] = counts[e] rounded up to pad_multiple, expert_start = its
+// exclusive prefix, expert_start[E] = total_padded[0] = the sum.
+__global__ void __launch_bounds__(1024) moe_group_prefix_kernel(const int32_t* __restrict__ counts,
+                                                                int32_t* __restrict__ padded_counts,
+                                                                int64_t* __restrict__ expert_start,
+                                                                int64_t* __restrict__ total_padded, int num_experts,
+                                                                int64_t pad_multiple) {
+  constexpr int PER = MAX_EXPERTS / 1024;
+  __shared__ int64_t wsum[16];
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  int64_t c[PER], sum = 0;
+#pragma unroll
+  for (int k = 0; k < PER; ++k) {
+    const int e = tid * PER + k;
+    int64_t padded = 0;
+    if (e < num_experts) {
+      const int64_t n = counts[e];
+      padded = pad_multiple > 1 ? (n + pad_multiple - 1) / pad_multiple * pad_multiple : n;
+      padded_counts[e] = static_cast<int32_t>(padded);
+    }
+    c[k] = padded;
+    sum += padded;
+  }
+  int64_t isum = sum;
+#pragma unroll
+  for (int off = 1; off < 64; off <<= 1) {
+    const int64_t t = __shfl_up(isum, off);
+    if (lane >= off) isum += t;
+  }
+  if (lane == 63) wsum[wave] = isum;
+  __syncthreads();
+  int64_t base = 0;
+  for (int w = 0; w < wave; ++w) base += wsum[w];
+  int64_t offset = base + isum - sum;
+#pragma unroll
+  for (int k = 0; k < PER; ++k) {
+    const int e = tid * PER + k;
+    if (e < num_experts) { expert_start[e] = offset; offset += c[k]; }
+  }
+  if (tid == 1023) {
+    expert_start[num_experts] = base + isum;
+    total_padded[0] = base + isum;
+  }
+}
+
+// One workgroup per expert: the expert's lanes in ascending lane order from expert_start[e] on (hipEngine's
+// scatter takes its slots with atomics, in whatever order the lanes arrive; ascending order is one of the
+// orders it can produce), scatter_offsets[e] += the number placed, as the atomics would leave it.
+__global__ void __launch_bounds__(1024) moe_scatter_kernel(const int64_t* __restrict__ selected,
+                                                           const float* __restrict__ routing,
+                                                           const int64_t* __restrict__ expert_start,
+                                                           int32_t* __restrict__ scatter_offsets,
+                                                           int64_t* __restrict__ sorted_lanes,
+                                                           int64_t* __restrict__ sorted_experts,
+                                                           float* __restrict__ sorted_weights, int64_t lanes,
+                                                           const uint16_t* __restrict__ hidden,
+                                                           uint16_t* __restrict__ packed, int64_t top_k,
+                                                           int64_t hidden_size) {
+  __shared__ int wave_cnt[2][16];
+  const int64_t e = blockIdx.x;
+  const int64_t base = expert_start[e] + scatter_offsets[e];
+  const int lane_id = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  int running = 0, buf = 0;
+  for (int64_t chunk = 0; chunk < lanes; chunk += 1024, buf ^= 1) {
+    const int64_t lane = chunk + threadIdx.x;
+    const bool flag = lane < lanes && selected[lane] == e;
+    const unsigned long long ballot = __ballot(flag);
+    const int before = __popcll(ballot & ((1ull << lane_id) - 1ull));
+    if (lane_id == 0) wave_cnt[buf][wave] = __popcll(ballot);
+    __syncthreads();
+    int offset = running, total = 0;
+#pragma unroll
+    for (int w = 0; w < 16; ++w) {
+      const int c = wave_cnt[buf][w];
+      if (w < wave) offset += c;
+      total += c;
+    }
+    if (flag) {
+      const int64_t idx = base + offset + before;
+      sorted_lanes[idx] = lane;
+      if (sorted_experts) sorted_experts[idx] = e;
+      if (sorted_weights) sorted_weights[idx] = routing[lane];
+    }
+    running += total;
+  }
+  __syncthreads();   // the lanes this workgroup placed are visible to all of its threads
+  if (threadIdx.x == 0) scatter_offsets[e] += running;
+  // gather: packed[base + i, :] = hidden[sorted_lanes[base + i] / top_k, :] for the rows placed above
+  if (hidden && packed) {
+    const bool wide = (hidden_size & 7) == 0 &&
+                      ((reinterpret_cast<uintptr_t>(hidden) | reinterpret_cast<uintptr_t>(packed)) & 15u) == 0;
+    const int64_t per_row = wide ? hidden_size / 8 : hidden_size;
+    for (int64_t i = threadIdx.x; i < running * per_row; i += 1024) {
+      const int64_t r = i / per_row, c = i - r * per_row;
+      const int64_t token = sorted_lanes[base + r] / top_k;
+      if (wide) {
+        reinterpret_cast<uint4*>(packed + (base + r) * hidden_size)[c] =
+            reinterpret_cast<const uint4*>(hidden + token * hidden_size)[c];
+      } else {
+        packed[(base + r) * hidden_size + c] = hidden[token * hidden_size + c];
+      }
+    }
+  }
+}
+
+// packed[row, :] = hidden[sorted_lanes[row] / top_k, :] (16-bit elements), zeros for a negative lane or a
+// token outside [0, tokens).  16 bytes per thread where the row length allows.
+__global__ void __launch_bounds__(256) moe_gather_rows_kernel(const uint16_t* __restrict__ hidden,
+                                                              const int64_t* __restrict__ sorted_lanes,
+                                                              uint16_t* __restrict__ packed, int64_t rows,
+                                                              int64_t tokens, int64_t top_k, int64_t hidden_size) {
+  const int64_t row = blockIdx.x;
+  if (row >= rows) return;
+  const int64_t lane = sorted_lanes[row];
+  const int64_t token = lane >= 0 ? lane / top_k : -1;
+  const bool valid = token >= 0 && token < tokens;
+  const uint16_t* src = hidden + (valid ? token : 0) * hidden_size;
+  uint16_t* dst = packed + row * hidden_size;
+  if ((hidden_size & 7) == 0 && ((reinterpret_cast<uintptr_t>(hidden) | reinterpret_cast<uintptr_t>(packed)) & 15u) == 0) {
+    for (int64_t c = threadIdx.x; c < hidden_size / 8; c += blockDim.x) {
+      uint4 v = make_uint4(0u, 0u, 0u, 0u);
+      if (valid) v = reinterpret_cast<const uint4*>(src)[c];
+      reinterpret_cast<uint4*>(dst)[c] = v;
+    }
+  } else {
+    for (int64_t c = threadIdx.x; c < hidden_size; c += blockDim.x) dst[c] = valid ? src[c] : static_cast<uint16_t>(0);
+  }
+}
+
 // --------------------------------------------------------------------------
 // elementwise steps between the projections
 // --------------------------------------------------------------------------
@@ -283,11 +425,12 @@ __global__ void moe_weighted_gather_kernel(const void* __restrict__ down, const 
 // decode: selected GEMV on the q8_1 integer GEMV body
 // --------------------------------------------------------------------------
 
-enum SelMode : int { SEL_SINGLE = 0, SEL_DUAL_SILU = 1, SEL_DOWN_SUM = 2 };
+enum SelMode : int { SEL_SINGLE = 0, SEL_DUAL_SILU = 1, SEL_DOWN_SUM = 2, SEL_DUAL = 3 };
 
 struct SelArgs {
   GemvArgs g;                 // x, w (first weight), out, kinds, K, N, ks, nrg; rows = 1
   const uint8_t* w_b;         // second weight (dual)
+  void* out_b;                // second output (SEL_DUAL)
   const int64_t* selected;    // [lanes]
   const float* routing;       // [lanes] (down sum)
   int x_rows;                 // activation rows (tokens) for single/dual; tokens for down sum
@@ -299,6 +442,10 @@ struct SelArgs {
 };
 
 __device__ __forceinline__ int64_t scalar_bytes(int kind) { return kind == KIND_F32 ? 4 : 2; }
+// bytes of one activation row of K values: scalars, or 36-byte q8_1 blocks
+__device__ __forceinline__ int64_t act_row_bytes(int kind, int K) {
+  return kind == KIND_Q8_1 ? static_cast<int64_t>(K / 32) * Q8_1_BYTES : static_cast<int64_t>(K) * scalar_bytes(kind);
+}
 
 // Workgroup size cap: the CB weight blocks of a chunk have to fit the VGPR
 // budget the cap implies (128 registers at 1024 threads, 256 at 512).
@@ -322,10 +469,18 @@ __global__ void __launch_bounds__((sel_max_threads<QT, R * CB>())) selected_gemv
   if (e < 0 || e >= s.num_experts) return;
   const int per = s.lanes / s.x_rows;
   const int x_row = s.x_rows == 1 ? 0 : lane / per;
-  a.x = static_cast<const uint8_t*>(s.g.x) + static_cast<int64_t>(x_row) * s.g.K * scalar_bytes(s.g.x_kind);
+  a.x = static_cast<const uint8_t*>(s.g.x) + static_cast<int64_t>(x_row) * act_row_bytes(s.g.x_kind, s.g.K);
   a.out = static_cast<uint8_t*>(s.g.out) + static_cast<int64_t>(lane) * s.g.N * scalar_bytes(s.g.out_kind);
   if constexpr (MODE == SEL_SINGLE) {
     gemv_workgroup<QT, 1, R, CB>(a, s.g.w + e * expert_bytes, blockIdx.x * s.g.nrg * 16 * R, smem);
+  } else if constexpr (MODE == SEL_DUAL) {
+    // gate and up rows of the same index in one pass, each stored to its own output
+    static_assert(R == 2, "the dual form pairs two matrices");
+    void* out_b = static_cast<uint8_t*>(s.out_b) + static_cast<int64_t>(lane) * s.g.N * scalar_bytes(s.g.out_kind);
+    gemv_workgroup_emit<QT, 1, 2, CB, true>(
+        a, s.g.w + e * expert_bytes, blockIdx.x * s.g.nrg * 16, smem,
+        [&](int which, int row, float v) { store_scalar(which ? out_b : a.out, row, v, a.out_kind); },
+        s.w_b + e * expert_bytes);
   } else {
     // gate and up rows of the same index in one pass: one staging of the activations,
     // all weight loads of both matrices in flight together
@@ -443,7 +598,8 @@ struct SelVariant {
   SelVariant{QT, CB, SEL_SINGLE, sel_max_threads<QT, CB>(), selected_gemv_kernel<QT, 1, CB, SEL_SINGLE>,          \
              {selected_gemv_kernel<QT, 1, CB, SEL_SINGLE, KIND_F32>, selected_gemv_kernel<QT, 1, CB, SEL_SINGLE, KIND_BF16>}}, \
   SelVariant{QT, CB, SEL_DUAL_SILU, sel_max_threads<QT, 2 * CB>(), selected_gemv_kernel<QT, 2, CB, SEL_DUAL_SILU>, \
-             {selected_gemv_kernel<QT, 2, CB, SEL_DUAL_SILU, KIND_F32>, selected_gemv_kernel<QT, 2, CB, SEL_DUAL_SILU, KIND_BF16>}}
+             {selected_gemv_kernel<QT, 2, CB, SEL_DUAL_SILU, KIND_F32>, selected_gemv_kernel<QT, 2, CB, SEL_DUAL_SILU, KIND_BF16>}}, \
+  SelVariant{QT, CB, SEL_DUAL, sel_max_threads<QT, 2 * CB>(), selected_gemv_kernel<QT, 2, CB, SEL_DUAL>, {nullptr, nullptr}}
 const SelVariant kSel[] = {
     SEL_VARIANTS(GGML_Q4_K, 1), SEL_VARIANTS(GGML_Q4_K, 2), SEL_VARIANTS(GGML_Q4_K, 5),
     SEL_VARIANTS(GGML_Q6_K, 1), SEL_VARIANTS(GGML_Q6_K, 2), SEL_VARIANTS(GGML_Q6_K, 5),
@@ -451,13 +607,17 @@ const SelVariant kSel[] = {
 
 int launch_selected(int qt, int mode, const void* x, int x_kind, const int64_t* selected, const float* routing,
                     const uint8_t* w_a, const uint8_t* w_b, void* out, int out_kind, int64_t x_rows, int64_t lanes,
-                    int64_t num_experts, int64_t top_k, int64_t K, int64_t N, int round_mid, hipStream_t stream) {
+                    int64_t num_experts, int64_t top_k, int64_t K, int64_t N, int round_mid, hipStream_t stream,
+                    void* out_b = nullptr) {
+  // q8_1 blocks as activations: the single and dual forms only (their staging reads them as they are)
+  const int max_x_kind = (mode == SEL_SINGLE || mode == SEL_DUAL) ? KIND_Q8_1 : KIND_F16;
   if (!x || !selected || !w_a || !out || x_rows <= 0 || lanes <= 0 || lanes > 65535 || num_experts <= 0 || K <= 0 ||
-      (K % QK_K) != 0 || K > (1 << 20) || N <= 0 || N > (1 << 24) || x_kind < KIND_F32 || x_kind > KIND_F16 ||
+      (K % QK_K) != 0 || K > (1 << 20) || N <= 0 || N > (1 << 24) || x_kind < KIND_F32 || x_kind > max_x_kind ||
       out_kind < KIND_F32 || out_kind > KIND_F16 || (qt != GGML_Q4_K && qt != GGML_Q6_K)) {
     return static_cast<int>(hipErrorInvalidValue);
   }
-  if (mode == SEL_DUAL_SILU && !w_b) return static_cast<int>(hipErrorInvalidValue);
+  if ((mode == SEL_DUAL_SILU || mode == SEL_DUAL) && !w_b) return static_cast<int>(hipErrorInvalidValue);
+  if (mode == SEL_DUAL && !out_b) return static_cast<int>(hipErrorInvalidValue);
   if (mode == SEL_DOWN_SUM && (!routing || top_k <= 0 || top_k > 8 || lanes != x_rows * top_k)) {
     return static_cast<int>(hipErrorInvalidValue);
   }
@@ -466,7 +626,7 @@ int launch_selected(int qt, int mode, const void* x, int x_kind, const int64_t* 
   SelArgs s;
   s.g.x = x; s.g.w = w_a; s.g.out = out; s.g.x_kind = x_kind; s.g.out_kind = out_kind; s.g.rows = 1;
   s.g.K = static_cast<int>(K); s.g.N = static_cast<int>(N);
-  s.w_b = w_b; s.selected = selected; s.routing = routing;
+  s.w_b = w_b; s.out_b = out_b; s.selected = selected; s.routing = routing;
   s.x_rows = static_cast<int>(x_rows); s.lanes = static_cast<int>(lanes);
   s.num_experts = static_cast<int>(num_experts); s.top_k = static_cast<int>(top_k); s.round_mid = round_mid;
   s.pair_offset = 0;
@@ -509,10 +669,11 @@ int launch_selected(int qt, int mode, const void* x, int x_kind, const int64_t* 
   for (const SelVariant& c : kSel)
     if (c.qt == qt && c.cb == cb && c.mode == mode) v = &c;
   if (!v) return static_cast<int>(hipErrorInvalidValue);
-  const int r = mode == SEL_DUAL_SILU ? 2 : 1;
+  const bool dual = mode == SEL_DUAL_SILU || mode == SEL_DUAL;
+  const int r = dual ? 2 : 1;
   int nrg = v->max_threads / 64 / ks;
   if (nrg < 1) return static_cast<int>(hipErrorInvalidValue);
-  const int rows_out_per_group = mode == SEL_DUAL_SILU ? 16 : 16 * r;
+  const int rows_out_per_group = 16;
   while (nrg > 1 && (N + nrg * rows_out_per_group - 1) / (nrg * rows_out_per_group) * lanes < 512) nrg >>= 1;
   s.g.ks = ks; s.g.nrg = nrg;
   size_t lds = gemv_lds_bytes(qt, 1, r, cb, ks, nrg);
@@ -524,8 +685,85 @@ int launch_selected(int qt, int mode, const void* x, int x_kind, const int64_t* 
   if (lds > 64 * 1024) return static_cast<int>(hipErrorInvalidValue);
   const int rows_out = nrg * rows_out_per_group;
   const dim3 grid(static_cast<unsigned>((N + rows_out - 1) / rows_out), static_cast<unsigned>(lanes));
-  const SelFn fn = (x_kind == KIND_F32 || x_kind == KIND_BF16) ? v->by_kind[x_kind] : v->fn;
+  const SelFn fn = ((x_kind == KIND_F32 || x_kind == KIND_BF16) && v->by_kind[x_kind]) ? v->by_kind[x_kind] : v->fn;
   hipLaunchKernelGGL(fn, grid, dim3(ks * nrg * 64), lds, stream, s);
+  return static_cast<int>(hipGetLastError());
+}
+
+// --------------------------------------------------------------------------
+// grouped GEMV: compact rows (activations already gathered in expert-major order),
+// every expert's weights read once per batch of 8 of its rows
+// (kernels/hip_gfx1100/quant/gguf_q4_k_gemv.hip:378-450)
+// --------------------------------------------------------------------------
+
+struct GroupedArgs {
+  GemvArgs g;                     // x [compact_rows, K], w [E, N, row_bytes], out [compact_rows, N]
+  const int64_t* expert_start;    // [E + 1]
+  int compact_rows;
+};
+
+// grid (row tiles of nrg*16 output rows, experts).  An expert's rows [start, end) are consecutive rows of x
+// and out, so they are batch rows of the dense GEMV body; experts with one or two rows (a decode batch)
+// take its batch-2 instantiation, the others walk their rows 8 at a time.
+template <int QT, int CB>
+__global__ void __launch_bounds__(512) grouped_gemv_kernel(GroupedArgs s) {
+  extern __shared__ __align__(16) uint8_t smem[];
+  const int e = blockIdx.y;
+  const int64_t start = s.expert_start[e], end = s.expert_start[e + 1];
+  if (start < 0 || end > s.compact_rows || start >= end) return;
+  const int64_t row_bytes = static_cast<int64_t>(s.g.K / QK_K) * GemvTraits<QT>::SUPER_BYTES;
+  const uint8_t* w = s.g.w + static_cast<int64_t>(e) * s.g.N * row_bytes;
+  const int first_row = blockIdx.x * s.g.nrg * 16;
+  GemvArgs a = s.g;
+  const int64_t xb = act_row_bytes(s.g.x_kind, s.g.K), ob = static_cast<int64_t>(s.g.N) * scalar_bytes(s.g.out_kind);
+  if (end - start <= 2) {
+    a.rows = static_cast<int>(end - start);
+    a.x = static_cast<const uint8_t*>(s.g.x) + start * xb;
+    a.out = static_cast<uint8_t*>(s.g.out) + start * ob;
+    gemv_workgroup<QT, 2, 1, CB>(a, w, first_row, smem);
+    return;
+  }
+  for (int64_t base = start; base < end; base += 8) {
+    a.rows = static_cast<int>(end - base < 8 ? end - base : 8);
+    a.x = static_cast<const uint8_t*>(s.g.x) + base * xb;
+    a.out = static_cast<uint8_t*>(s.g.out) + base * ob;
+    if (base > start) __syncthreads();   // the staging area of the previous batch is still being read
+    gemv_workgroup<QT, 8, 1, CB>(a, w, first_row, smem);
+  }
+}
+
+int launch_grouped_gemv(int qt, const void* x, int x_kind, const int64_t* expert_start, const uint8_t* w, void* out,
+                        int out_kind, int64_t compact_rows, int64_t num_experts, int64_t K, int64_t N,
+                        hipStream_t stream) {
+  if (!x || !expert_start || !w || !out || compact_rows <= 0 || compact_rows > 0x7FFFFFFF || num_experts <= 0 ||
+      num_experts > 65535 || K <= 0 || (K % QK_K) != 0 || K > (1 << 20) || N <= 0 || N > (1 << 24) ||
+      x_kind < KIND_F32 || x_kind > KIND_Q8_1 || out_kind < KIND_F32 || out_kind > KIND_F16 ||
+      (qt != GGML_Q4_K && qt != GGML_Q6_K)) {
+    return static_cast<int>(hipErrorInvalidValue);
+  }
+  const int nb = static_cast<int>(K / QK_K);
+  const int ks = nb >= 4 ? 4 : nb;
+  const int per_wave = (nb + ks - 1) / ks;
+  const int cb = per_wave >= 5 ? 5 : per_wave >= 2 ? 2 : 1;
+  int nrg = 512 / 64 / ks;
+  while (nrg > 1 && (N + nrg * 16 - 1) / (nrg * 16) < 8) nrg >>= 1;
+  GroupedArgs s;
+  s.g.x = x; s.g.w = w; s.g.out = out; s.g.x_kind = x_kind; s.g.out_kind = out_kind; s.g.rows = 8;
+  s.g.K = static_cast<int>(K); s.g.N = static_cast<int>(N); s.g.ks = ks; s.g.nrg = nrg;
+  s.expert_start = expert_start;
+  s.compact_rows = static_cast<int>(compact_rows);
+  const size_t lds = gemv_lds_bytes(qt, 8, 1, cb, ks, nrg);
+  if (lds > 64 * 1024) return static_cast<int>(hipErrorInvalidValue);
+  const dim3 grid(static_cast<unsigned>((N + nrg * 16 - 1) / (nrg * 16)), static_cast<unsigned>(num_experts));
+  const dim3 block(ks * nrg * 64);
+#define LAUNCH_GROUPED(QT)                                                                          \
+  do {                                                                                              \
+    if (cb == 1) hipLaunchKernelGGL((grouped_gemv_kernel<QT, 1>), grid, block, lds, stream, s);      \
+    else if (cb == 2) hipLaunchKernelGGL((grouped_gemv_kernel<QT, 2>), grid, block, lds, stream, s); \
+    else hipLaunchKernelGGL((grouped_gemv_kernel<QT, 5>), grid, block, lds, stream, s);              \
+  } while (0)
+  if (qt == GGML_Q4_K) LAUNCH_GROUPED(GGML_Q4_K); else LAUNCH_GROUPED(GGML_Q6_K);
+#undef LAUNCH_GROUPED
   return static_cast<int>(hipGetLastError());
 }
 
@@ -712,6 +950,59 @@ extern "C" int hipengine_qwen35_moe_mmq32_tile_map(const int64_t* expert_start_c
                          32, stream);
 }
 
+extern "C" int hipengine_qwen35_moe_group_count(const int64_t* selected_experts, int32_t* counts, int64_t total_lanes,
+                                                int64_t num_experts, hipStream_t stream) {
+  if (!selected_experts || !counts || total_lanes <= 0 || total_lanes > (1ll << 30) || num_experts <= 0) {
+    return static_cast<int>(hipErrorInvalidValue);
+  }
+  hipLaunchKernelGGL(moe_group_count_kernel, dim3(static_cast<unsigned>((total_lanes + 255) / 256)), dim3(256), 0,
+                     stream, selected_experts, counts, total_lanes, num_experts);
+  return static_cast<int>(hipGetLastError());
+}
+
+extern "C" int hipengine_qwen35_moe_group_prefix(const int32_t* counts, int32_t* padded_counts, int64_t* expert_start,
+                                                 int64_t* total_padded, int64_t num_experts, int64_t pad_multiple,
+                                                 hipStream_t stream) {
+  if (!counts || !padded_counts || !expert_start || !total_padded || num_experts <= 0 || pad_multiple <= 0 ||
+      num_experts > MAX_EXPERTS) {
+    return static_cast<int>(hipErrorInvalidValue);
+  }
+  hipLaunchKernelGGL(moe_group_prefix_kernel, dim3(1), dim3(1024), 0, stream, counts, padded_counts, expert_start,
+                     total_padded, static_cast<int>(num_experts), pad_multiple);
+  return static_cast<int>(hipGetLastError());
+}
+
+extern "C" int hipengine_qwen35_moe_gather_packed_hidden_lowp(const uint16_t* hidden_states, const int64_t* sorted_lanes,
+                                                              uint16_t* packed_hidden, int64_t total_elements,
+                                                              int64_t tokens, int64_t top_k, int64_t hidden_size,
+                                                              hipStream_t stream) {
+  if (!hidden_states || !sorted_lanes || !packed_hidden || total_elements <= 0 || tokens <= 0 || top_k <= 0 ||
+      hidden_size <= 0 || (total_elements % hidden_size) != 0 || total_elements / hidden_size > 0x7FFFFFFF) {
+    return static_cast<int>(hipErrorInvalidValue);
+  }
+  const int64_t rows = total_elements / hidden_size;
+  hipLaunchKernelGGL(moe_gather_rows_kernel, dim3(static_cast<unsigned>(rows)), dim3(256), 0, stream, hidden_states,
+                     sorted_lanes, packed_hidden, rows, tokens, top_k, hidden_size);
+  return static_cast<int>(hipGetLastError());
+}
+
+extern "C" int hipengine_qwen35_moe_group_scatter_gather_lowp(
+    const uint16_t* hidden_states, const int64_t* selected_experts, const float* routing_weights,
+    const int64_t* expert_start, int32_t* scatter_offsets, int64_t* sorted_lanes, int64_t* sorted_experts,
+    float* sorted_weights, uint16_t* packed_hidden, int64_t total_lanes, int64_t num_experts, int64_t top_k,
+    int64_t hidden_size, hipStream_t stream) {
+  if (!hidden_states || !selected_experts || !routing_weights || !expert_start || !scatter_offsets || !sorted_lanes ||
+      !sorted_experts || !sorted_weights || !packed_hidden || total_lanes <= 0 || total_lanes > 0x7FFFFFFF ||
+      num_experts <= 0 || num_experts > MAX_EXPERTS || top_k <= 0 || hidden_size <= 0) {
+    return static_cast<int>(hipErrorInvalidValue);
+  }
+  // Rows of the outputs that no lane is scattered to (padding between experts) keep their contents, as in hipEngine.
+  hipLaunchKernelGGL(moe_scatter_kernel, dim3(static_cast<unsigned>(num_experts)), dim3(1024), 0, stream,
+                     selected_experts, routing_weights, expert_start, scatter_offsets, sorted_lanes, sorted_experts,
+                     sorted_weights, total_lanes, hidden_states, packed_hidden, top_k, hidden_size);
+  return static_cast<int>(hipGetLastError());
+}
+
 extern "C" int hipengine_gfx950_moe_lane_to_compact(const int64_t* sorted_lanes, int64_t* lane_to_compact,
                                                     int64_t compact_rows, int64_t total_lanes, hipStream_t stream) {
   if (!sorted_lanes || !lane_to_compact || compact_rows <= 0 || total_lanes <= 0) {
@@ -772,6 +1063,52 @@ extern "C" int hipengine_gguf_q4_k_selected_dual_silu_gemv_bf16_bf16_out(
   (void)threads;
   return launch_selected(GGML_Q4_K, SEL_DUAL_SILU, x, KIND_BF16, selected, nullptr, qweight_a, qweight_b, out,
                          KIND_BF16, x_rows, rows, num_experts, 1, in_features, out_features, 1, stream);
+}
+
+// out_a[lane] = W_a[selected[lane]] . x_row, out_b[lane] = W_b[selected[lane]] . x_row in one pass
+// (gguf_q4_k_gemv.hip:2732-2749), and the same over pre-quantized 36-byte q8_1 activation rows (:2864-2892).
+extern "C" int hipengine_gguf_q4_k_selected_dual_gemv_bf16_bf16_out(
+    const uint16_t* x, const int64_t* selected, const uint8_t* qweight_a, const uint8_t* qweight_b, uint16_t* out_a,
+    uint16_t* out_b, int64_t x_rows, int64_t rows, int64_t num_experts, int64_t in_features, int64_t out_features,
+    int64_t threads, hipStream_t stream) {
+  (void)threads;
+  return launch_selected(GGML_Q4_K, SEL_DUAL, x, KIND_BF16, selected, nullptr, qweight_a, qweight_b, out_a, KIND_BF16,
+                         x_rows, rows, num_experts, 1, in_features, out_features, 0, stream, out_b);
+}
+
+extern "C" int hipengine_gguf_q4_k_selected_dual_gemv_q8_1_dp4a_bf16_bf16_out(
+    const void* xq, const int64_t* selected, const uint8_t* qweight_a, const uint8_t* qweight_b, uint16_t* out_a,
+    uint16_t* out_b, int64_t x_rows, int64_t rows, int64_t num_experts, int64_t in_features, int64_t out_features,
+    int64_t threads, hipStream_t stream) {
+  (void)threads;
+  return launch_selected(GGML_Q4_K, SEL_DUAL, xq, KIND_Q8_1, selected, nullptr, qweight_a, qweight_b, out_a, KIND_BF16,
+                         x_rows, rows, num_experts, 1, in_features, out_features, 0, stream, out_b);
+}
+
+// Routed down projection with the weighted sum over a token's experts fused ("weighted_down" call kind,
+// loading/gguf_selected_contract.py:50-54,305-315; argument list of
+// hipengine_gguf_iq4_xs_weighted_selected_down_bf16_bf16_out, gguf_iq_gemv.hip:2276-2288).
+#define DEFINE_WEIGHTED_DOWN(QNAME, QT)                                                                              \
+  extern "C" int hipengine_gguf_##QNAME##_weighted_selected_down_bf16_bf16_out(                                      \
+      const uint16_t* x, const int64_t* selected, const float* routing_weights, const uint8_t* qweight, uint16_t* out, \
+      int64_t tokens, int64_t top_k, int64_t num_experts, int64_t in_features, int64_t out_features, int64_t threads, \
+      hipStream_t stream) {                                                                                          \
+    (void)threads;                                                                                                   \
+    if (tokens <= 0 || top_k <= 0 || tokens * top_k > 65535) return static_cast<int>(hipErrorInvalidValue);          \
+    return launch_selected(QT, SEL_DOWN_SUM, x, KIND_BF16, selected, routing_weights, qweight, nullptr, out,         \
+                           KIND_BF16, tokens, tokens * top_k, num_experts, top_k, in_features, out_features, 0,      \
+                           stream);                                                                                  \
+  }
+DEFINE_WEIGHTED_DOWN(q4_k, GGML_Q4_K)
+DEFINE_WEIGHTED_DOWN(q6_k, GGML_Q6_K)
+
+// Grouped GEMV over gathered compact rows (gguf_q4_k_gemv.hip:2634-2669).
+extern "C" int hipengine_gguf_q4_k_selected_grouped_prefill_compact_rowbatch8_bf16_bf16_out(
+    const void* x, const void* expert_start, const void* qweight, void* out, int64_t compact_rows, int64_t num_experts,
+    int64_t in_features, int64_t out_features, hipStream_t stream) {
+  return launch_grouped_gemv(GGML_Q4_K, x, KIND_BF16, static_cast<const int64_t*>(expert_start),
+                             static_cast<const uint8_t*>(qweight), out, KIND_BF16, compact_rows, num_experts,
+                             in_features, out_features, stream);
 }
 
 extern "C" int hipengine_gfx950_gguf_selected_gemv(int32_t ggml_type, int32_t mode, const void* x, int32_t x_kind,

@@ -85,7 +85,89 @@ def moe_lane_to_compact(sorted_lanes_ptr: int, lane_to_compact_ptr: int, compact
     check_launch(fn(sorted_lanes_ptr, lane_to_compact_ptr, compact_rows, total_lanes, stream), runtime)
 
 
+def _check_positive(value: int, name: str) -> None:
+    if value <= 0:
+        raise ValueError(f"{name} must be positive")
+
+
+def qwen35_moe_group_count(selected_experts_ptr: int, counts_ptr: int, total_lanes: int, num_experts: int, *,
+                           stream: int = 0, library: ctypes.CDLL | None = None,
+                           runtime: HipRuntime | None = None) -> None:
+    """Count routed lanes per expert into int32 ``counts``; the caller zeroes it (hipEngine :77-103)."""
+    _check_positive(total_lanes, "total_lanes")
+    _check_positive(num_experts, "num_experts")
+    validate_pointers(selected_experts_ptr=selected_experts_ptr, counts_ptr=counts_ptr)
+    fn = entry("hipengine_qwen35_moe_group_count", [VOID, VOID, I64, I64, VOID], library)
+    check_launch(fn(selected_experts_ptr, counts_ptr, total_lanes, num_experts, stream), runtime)
+
+
+def qwen35_moe_group_prefix(counts_ptr: int, padded_counts_ptr: int, expert_start_ptr: int, total_padded_ptr: int,
+                            num_experts: int, pad_multiple: int, *, stream: int = 0,
+                            library: ctypes.CDLL | None = None, runtime: HipRuntime | None = None) -> None:
+    """Per-expert counts -> counts padded to ``pad_multiple``, their exclusive prefix and total (hipEngine :106-146)."""
+    _check_num_experts(num_experts)
+    _check_positive(pad_multiple, "pad_multiple")
+    validate_pointers(counts_ptr=counts_ptr, padded_counts_ptr=padded_counts_ptr, expert_start_ptr=expert_start_ptr,
+                      total_padded_ptr=total_padded_ptr)
+    fn = entry("hipengine_qwen35_moe_group_prefix", [VOID] * 4 + [I64, I64, VOID], library)
+    check_launch(fn(counts_ptr, padded_counts_ptr, expert_start_ptr, total_padded_ptr, num_experts, pad_multiple, stream),
+                 runtime)
+
+
+def qwen35_moe_group_scatter_gather_lowp(hidden_states_ptr: int, selected_experts_ptr: int, routing_weights_ptr: int,
+                                         expert_start_ptr: int, scatter_offsets_ptr: int, sorted_lanes_ptr: int,
+                                         sorted_experts_ptr: int, sorted_weights_ptr: int, packed_hidden_ptr: int,
+                                         total_lanes: int, num_experts: int, top_k: int, hidden_size: int, *,
+                                         stream: int = 0, library: ctypes.CDLL | None = None,
+                                         runtime: HipRuntime | None = None) -> None:
+    """Scatter lanes into expert order and gather their 16-bit hidden rows (hipEngine :558-619).  Lanes of an
+    expert land in ascending lane order (hipEngine: arrival order); ``scatter_offsets`` (int32, zeroed by the
+    caller) ends as the per-expert lane counts."""
+    _check_positive(total_lanes, "total_lanes")
+    _check_num_experts(num_experts)
+    _check_positive(top_k, "top_k")
+    _check_positive(hidden_size, "hidden_size")
+    validate_pointers(hidden_states_ptr=hidden_states_ptr, selected_experts_ptr=selected_experts_ptr,
+                      routing_weights_ptr=routing_weights_ptr, expert_start_ptr=expert_start_ptr,
+                      scatter_offsets_ptr=scatter_offsets_ptr, sorted_lanes_ptr=sorted_lanes_ptr,
+                      sorted_experts_ptr=sorted_experts_ptr, sorted_weights_ptr=sorted_weights_ptr,
+                      packed_hidden_ptr=packed_hidden_ptr)
+    fn = entry("hipengine_qwen35_moe_group_scatter_gather_lowp", [VOID] * 9 + [I64] * 4 + [VOID], library)
+    check_launch(fn(hidden_states_ptr, selected_experts_ptr, routing_weights_ptr, expert_start_ptr, scatter_offsets_ptr,
+                    sorted_lanes_ptr, sorted_experts_ptr, sorted_weights_ptr, packed_hidden_ptr, total_lanes,
+                    num_experts, top_k, hidden_size, stream), runtime)
+
+
+def qwen35_moe_gather_packed_hidden_lowp(hidden_states_ptr: int, sorted_lanes_ptr: int, packed_hidden_ptr: int,
+                                         total_elements: int, tokens: int, top_k: int, hidden_size: int, *,
+                                         stream: int = 0, library: ctypes.CDLL | None = None,
+                                         runtime: HipRuntime | None = None) -> None:
+    """Gather 16-bit hidden rows by sorted lane ids into packed rows (hipEngine :622-668)."""
+    _check_positive(total_elements, "total_elements")
+    _check_positive(tokens, "tokens")
+    _check_positive(top_k, "top_k")
+    _check_positive(hidden_size, "hidden_size")
+    if total_elements % hidden_size != 0:
+        raise ValueError("total_elements must be a multiple of hidden_size")
+    validate_pointers(hidden_states_ptr=hidden_states_ptr, sorted_lanes_ptr=sorted_lanes_ptr,
+                      packed_hidden_ptr=packed_hidden_ptr)
+    fn = entry("hipengine_qwen35_moe_gather_packed_hidden_lowp", [VOID] * 3 + [I64] * 4 + [VOID], library)
+    check_launch(fn(hidden_states_ptr, sorted_lanes_ptr, packed_hidden_ptr, total_elements, tokens, top_k, hidden_size,
+                    stream), runtime)
+
+
 def register_kernels(backend: str = "hip_gfx950", *, replace: bool = False) -> None:
+    # keys of hipEngine's moe/group_scatter.py:713-806
+    for quant, variant in (("generic", "selected_experts"), ("w4_paro", "qwen35")):
+        register(KernelKey(backend, "moe_group_count", quant, variant), qwen35_moe_group_count, replace=replace)
+    register(KernelKey(backend, "moe_group_prefix", "w4_paro", "qwen35"), qwen35_moe_group_prefix, replace=replace)
+    register(KernelKey(backend, "moe_group_prefix", "generic", "pad_multiple"), qwen35_moe_group_prefix, replace=replace)
+    for quant, variant in (("generic", "bf16_lane_rows"), ("w4_paro", "qwen35_lowp")):
+        register(KernelKey(backend, "moe_group_scatter_gather", quant, variant), qwen35_moe_group_scatter_gather_lowp,
+                 replace=replace)
+    for quant, variant in (("generic", "bf16_lanes"), ("w4_paro", "qwen35_lowp")):
+        register(KernelKey(backend, "moe_gather_packed_hidden", quant, variant), qwen35_moe_gather_packed_hidden_lowp,
+                 replace=replace)
     register(KernelKey(backend, "moe_group_compact", "generic", "active_experts"), qwen35_moe_group_compact_active,
              replace=replace)
     register(KernelKey(backend, "moe_group_compact", "generic", "active_experts_source_rows"),

@@ -66,6 +66,87 @@ def gguf_q4_k_selected_dual_silu_gemv_bf16_bf16_out(x_ptr: int, selected_ptr: in
                     out_features, threads, stream), runtime)
 
 
+def gguf_q4_k_selected_dual_gemv_bf16_bf16_out(x_ptr: int, selected_ptr: int, qweight_a_ptr: int, qweight_b_ptr: int,
+                                               out_a_ptr: int, out_b_ptr: int, x_rows: int, rows: int,
+                                               num_experts: int, in_features: int, out_features: int, *,
+                                               threads: int = 128, stream: int = 0,
+                                               library: ctypes.CDLL | None = None,
+                                               runtime: HipRuntime | None = None) -> None:
+    """Gate and up of every lane in one pass, each to its own output (the ``dual`` call kind;
+    hipEngine ``gguf_q4_k_gemv.py`` ``gguf_q4_k_selected_dual_gemv_bf16_bf16_out``)."""
+    _validate_selected(x_rows, rows, num_experts, in_features, out_features, threads)
+    validate_pointers(x_ptr=x_ptr, selected_ptr=selected_ptr, qweight_a_ptr=qweight_a_ptr, qweight_b_ptr=qweight_b_ptr,
+                      out_a_ptr=out_a_ptr, out_b_ptr=out_b_ptr)
+    fn = entry("hipengine_gguf_q4_k_selected_dual_gemv_bf16_bf16_out", [VOID] * 6 + [I64] * 6 + [VOID], library)
+    check_launch(fn(x_ptr, selected_ptr, qweight_a_ptr, qweight_b_ptr, out_a_ptr, out_b_ptr, x_rows, rows, num_experts,
+                    in_features, out_features, threads, stream), runtime)
+
+
+def gguf_q4_k_selected_dual_gemv_q8_1_dp4a_bf16_bf16_out(xq_ptr: int, selected_ptr: int, qweight_a_ptr: int,
+                                                         qweight_b_ptr: int, out_a_ptr: int, out_b_ptr: int,
+                                                         x_rows: int, rows: int, num_experts: int, in_features: int,
+                                                         out_features: int, *, threads: int = 128, stream: int = 0,
+                                                         library: ctypes.CDLL | None = None,
+                                                         runtime: HipRuntime | None = None) -> None:
+    """The ``dual`` form over pre-quantized 36-byte q8_1 activation rows (caller-owned scratch, written by
+    ``gguf_q4_k_quantize_bf16_q8_1``)."""
+    _validate_selected(x_rows, rows, num_experts, in_features, out_features, threads)
+    validate_pointers(xq_ptr=xq_ptr, selected_ptr=selected_ptr, qweight_a_ptr=qweight_a_ptr, qweight_b_ptr=qweight_b_ptr,
+                      out_a_ptr=out_a_ptr, out_b_ptr=out_b_ptr)
+    fn = entry("hipengine_gguf_q4_k_selected_dual_gemv_q8_1_dp4a_bf16_bf16_out", [VOID] * 6 + [I64] * 6 + [VOID], library)
+    check_launch(fn(xq_ptr, selected_ptr, qweight_a_ptr, qweight_b_ptr, out_a_ptr, out_b_ptr, x_rows, rows, num_experts,
+                    in_features, out_features, threads, stream), runtime)
+
+
+def _make_weighted_down(quant: str):
+    symbol = f"hipengine_gguf_{quant}_weighted_selected_down_bf16_bf16_out"
+
+    def wrapper(x_ptr: int, selected_ptr: int, routing_weights_ptr: int, qweight_ptr: int, out_ptr: int, *,
+                tokens: int, top_k: int, num_experts: int, in_features: int, out_features: int, threads: int = 0,
+                stream: int = 0, library: ctypes.CDLL | None = None, runtime: HipRuntime | None = None) -> None:
+        if tokens <= 0:
+            raise ValueError("tokens must be positive")
+        if top_k <= 0 or top_k > 8:
+            raise ValueError("top_k must be in 1..8")
+        _validate_selected(tokens, tokens * top_k, num_experts, in_features, out_features, threads or 128)
+        validate_pointers(x_ptr=x_ptr, selected_ptr=selected_ptr, routing_weights_ptr=routing_weights_ptr,
+                          qweight_ptr=qweight_ptr, out_ptr=out_ptr)
+        fn = entry(symbol, [VOID] * 5 + [I64] * 6 + [VOID], library)
+        check_launch(fn(x_ptr, selected_ptr, routing_weights_ptr, qweight_ptr, out_ptr, tokens, top_k, num_experts,
+                        in_features, out_features, threads or 128, stream), runtime)
+
+    wrapper.__name__ = f"gguf_{quant}_weighted_selected_down_bf16_bf16_out"
+    wrapper.__doc__ = ("Routed down projection with the weighted sum over a token's experts fused: the ``weighted_down`` "
+                       "call kind, keyword geometry as in hipEngine's ``gguf_iq4_xs_weighted_selected_down_bf16_bf16_out`` "
+                       "(``gguf_iq_gemv.py:956-972``).")
+    return wrapper
+
+
+gguf_q4_k_weighted_selected_down_bf16_bf16_out = _make_weighted_down("q4_k")
+gguf_q6_k_weighted_selected_down_bf16_bf16_out = _make_weighted_down("q6_k")
+
+
+def gguf_q4_k_selected_grouped_prefill_compact_rowbatch8_bf16_bf16_out(
+        x_ptr: int, expert_start_ptr: int, qweight_ptr: int, out_ptr: int, compact_rows: int, num_experts: int,
+        in_features: int, out_features: int, *, stream: int = 0, library: ctypes.CDLL | None = None,
+        runtime: HipRuntime | None = None) -> None:
+    """Grouped GEMV over gathered compact rows: rows ``[expert_start[e], expert_start[e+1])`` of ``x`` take
+    expert ``e`` (hipEngine ``gguf_q4_k_gemv.py:1406-1451``)."""
+    if compact_rows <= 0:
+        raise ValueError("compact_rows must be positive")
+    if num_experts <= 0 or num_experts > 65535:
+        raise ValueError("num_experts must be in 1..65535")
+    if in_features <= 0 or in_features % 256 != 0:
+        raise ValueError("in_features must be positive and divisible by the GGUF block size 256")
+    if out_features <= 0:
+        raise ValueError("out_features must be positive")
+    validate_pointers(x_ptr=x_ptr, expert_start_ptr=expert_start_ptr, qweight_ptr=qweight_ptr, out_ptr=out_ptr)
+    fn = entry("hipengine_gguf_q4_k_selected_grouped_prefill_compact_rowbatch8_bf16_bf16_out",
+               [VOID] * 4 + [I64] * 4 + [VOID], library)
+    check_launch(fn(x_ptr, expert_start_ptr, qweight_ptr, out_ptr, compact_rows, num_experts, in_features, out_features,
+                    stream), runtime)
+
+
 def gguf_selected_gemv(quant: str, mode: int, x_ptr: int, selected_ptr: int, qweight_a_ptr: int, out_ptr: int,
                        x_rows: int, lanes: int, num_experts: int, in_features: int, out_features: int, *,
                        x_dtype: str = "f32", out_dtype: str = "f32", routing_weights_ptr: int = 0,
@@ -189,6 +270,21 @@ def register_kernels(backend: str = "hip_gfx950", *, replace: bool = False) -> N
              gguf_q4_k_selected_gemv_bf16_bf16_out, replace=replace)
     register(KernelKey(backend, "linear", "gguf_q4_k", "selected_dual_silu_gemv_bf16_bf16_out"),
              gguf_q4_k_selected_dual_silu_gemv_bf16_bf16_out, replace=replace)
+    register(KernelKey(backend, "linear", "gguf_q4_k", "selected_dual_gemv_bf16_bf16_out"),
+             gguf_q4_k_selected_dual_gemv_bf16_bf16_out, replace=replace)
+    register(KernelKey(backend, "linear", "gguf_q4_k", "selected_dual_gemv_q8_1_dp4a_bf16_bf16_out"),
+             gguf_q4_k_selected_dual_gemv_q8_1_dp4a_bf16_bf16_out, replace=replace)
+    register(KernelKey(backend, "moe_linear", "gguf_q4_k", "selected_grouped_prefill_compact_rowbatch8_bf16_bf16_out"),
+             gguf_q4_k_selected_grouped_prefill_compact_rowbatch8_bf16_bf16_out, replace=replace)
+    # the generic call-kind names of loading/gguf_selected_contract.py:50-54
+    register(KernelKey(backend, "moe_linear", "gguf_q4_k", "selected_gemv_decode_bf16_bf16_out"),
+             gguf_q4_k_selected_gemv_bf16_bf16_out, replace=replace)
+    register(KernelKey(backend, "moe_linear", "gguf_q4_k", "selected_dual_silu_gemv_decode_bf16_bf16_out"),
+             gguf_q4_k_selected_dual_silu_gemv_bf16_bf16_out, replace=replace)
+    register(KernelKey(backend, "moe_linear", "gguf_q4_k", "selected_weighted_down_gemv_decode_bf16_bf16_out"),
+             gguf_q4_k_weighted_selected_down_bf16_bf16_out, replace=replace)
+    register(KernelKey(backend, "moe_linear", "gguf_q6_k", "selected_weighted_down_gemv_decode_bf16_bf16_out"),
+             gguf_q6_k_weighted_selected_down_bf16_bf16_out, replace=replace)
     register(KernelKey(backend, "moe_linear", "gguf_q4_k",
                        "selected_dual_q8_1_ds4_mmq32_prefill_compact32_bf16_bf16_out"),
              gguf_q4_k_selected_dual_q8_1_ds4_mmq32_prefill_compact32_bf16_bf16_out, replace=replace)

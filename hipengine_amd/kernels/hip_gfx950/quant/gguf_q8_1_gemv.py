@@ -7,6 +7,9 @@ stream, library, runtime)`` (``kernels/hip_gfx1100/quant/gguf_q4_k_gemv.py:115-1
 
 * ``gguf_<q>_q8_1_fused_gemv_<act>_<out>_out`` take float activations and
   quantize them to q8_1 inside the kernel;
+* ``gguf_<q>_gemv_<act>_<out>_out`` / ``gguf_<q>_prefill_<act>_<out>_out`` are hipEngine's own dense names
+  (``gguf_q4_k_gemv.py:175-202,524-576``, ``gguf_k_gemv.py:1920-2049``), registered under the keys its
+  dispatcher asks for, ``("linear", quant, "gemv_*" / "prefill_*")``; they run the fused kernels;
 * ``gguf_q4_k_q8_1_dp4a_vdr_*``, ``gguf_q6_k_q8_1_dp4a_gemv_*`` and
   ``gguf_q8_0_dp4a_gemv_*`` take pre-quantized 36-byte q8_1 blocks, as
   hipEngine's ``gguf_q4_k_q8_1_dp4a_vdr_gemv.py`` / ``gguf_q8_0_dp4a_gemv.py`` do.
@@ -71,6 +74,79 @@ def _make_q8_1(name: str, symbol: str):
     wrapper.__doc__ = f"GGUF GEMV over pre-quantized 36-byte q8_1 activation blocks (C symbol ``{symbol}``)."
     return wrapper
 
+
+_DENSE_DTYPES = (("f32", "f32"), ("f32", "fp16"), ("fp16", "f32"), ("fp16", "fp16"), ("bf16", "f32"), ("bf16", "fp16"),
+                 ("bf16", "bf16"))
+_MMQ_MIN_ROWS = 32          # from here on a prefill with a workspace goes through pack + MMQ
+_PREFILL_ARGS = [I32, VOID, VOID, VOID, I32, I64, I64, I64, VOID, I64, VOID]
+
+
+def gguf_prefill_workspace_bytes(quant_key: str, rows: int, in_features: int) -> int:
+    """Bytes of the workspace a ``prefill_bf16_*`` call takes to run on the MMQ (0: that quant has none)."""
+    if quant_key not in ("gguf_q4_k", "gguf_q6_k"):
+        return 0
+    return rows * (in_features // 128) * (144 if quant_key == "gguf_q4_k" else 160)
+
+
+def _make_dense(quant: str, family: str, act: str, out: str):
+    symbol = f"hipengine_gguf_{quant}_gemv_{act}_{out}_out"
+    quant_key = f"gguf_{quant}"
+
+    def wrapper(x_ptr: int, qweight_ptr: int, out_ptr: int, rows: int, in_features: int, out_features: int, *,
+                threads: int = 128, stream: int = 0, library: ctypes.CDLL | None = None,
+                runtime: HipRuntime | None = None, workspace_ptr: int = 0, workspace_bytes: int = 0) -> None:
+        validate_linear(rows, in_features, out_features, threads)
+        validate_pointers(x_ptr=x_ptr, qweight_ptr=qweight_ptr, out_ptr=out_ptr)
+        need = gguf_prefill_workspace_bytes(quant_key, rows, in_features)
+        if (family == "prefill" and act == "bf16" and rows >= _MMQ_MIN_ROWS and workspace_ptr and need
+                and workspace_bytes >= need and (quant != "q4_k" or out_features % 32 == 0)):
+            code = entry("hipengine_gfx950_gguf_prefill_bf16", _PREFILL_ARGS, library)(
+                QUANT_KEY_TO_GGML[quant_key], x_ptr, qweight_ptr, out_ptr, _KINDS[out], rows, in_features, out_features,
+                workspace_ptr, workspace_bytes, stream)
+        else:
+            code = entry(symbol, _FUSED_ARGS, library)(x_ptr, qweight_ptr, out_ptr, rows, in_features, out_features,
+                                                       threads, stream)
+        check_launch(code, runtime)
+
+    wrapper.__name__ = f"gguf_{quant}_{family}_{act}_{out}_out"
+    wrapper.__doc__ = (
+        f"hipEngine's dense {family} entry for {quant.upper()} (C symbol ``{symbol}``): {act} activations, quantized to "
+        f"q8_1 inside the kernel, {out} output; any number of rows, 8 per launch."
+        + (" With ``workspace_ptr`` / ``workspace_bytes`` (see ``gguf_prefill_workspace_bytes``) and 32 rows or more, "
+           "bf16 activations are packed into the workspace and the int8-MFMA MMQ runs instead."
+           if family == "prefill" else ""))
+    return wrapper
+
+
+def _make_dense_dual(quant: str, act: str, out: str):
+    symbol = f"hipengine_gguf_{quant}_dual_gemv_{act}_{out}_out"
+
+    def wrapper(x_ptr: int, qweight_a_ptr: int, qweight_b_ptr: int, out_a_ptr: int, out_b_ptr: int, rows: int,
+                in_features: int, out_features: int, *, threads: int = 128, stream: int = 0,
+                library: ctypes.CDLL | None = None, runtime: HipRuntime | None = None) -> None:
+        validate_linear(rows, in_features, out_features, threads)
+        validate_pointers(x_ptr=x_ptr, qweight_a_ptr=qweight_a_ptr, qweight_b_ptr=qweight_b_ptr, out_a_ptr=out_a_ptr,
+                          out_b_ptr=out_b_ptr)
+        code = entry(symbol, [VOID] * 5 + [I64] * 4 + [VOID], library)(
+            x_ptr, qweight_a_ptr, qweight_b_ptr, out_a_ptr, out_b_ptr, rows, in_features, out_features, threads, stream)
+        check_launch(code, runtime)
+
+    wrapper.__name__ = f"gguf_{quant}_dual_gemv_{act}_{out}_out"
+    wrapper.__doc__ = (f"Two {quant.upper()} matrices over one activation: ``out_a = W_a x``, ``out_b = W_b x`` "
+                       f"(C symbol ``{symbol}``; hipEngine ``gguf_k_gemv.py`` dual wrappers).")
+    return wrapper
+
+
+DENSE: dict[tuple[str, str, str, str], object] = {}
+for _q in _QUANTS:
+    for _family in ("gemv", "prefill"):
+        for _a, _o in _DENSE_DTYPES:
+            _fn = _make_dense(_q, _family, _a, _o)
+            DENSE[(_q, _family, _a, _o)] = _fn
+            globals()[_fn.__name__] = _fn
+DENSE_DUAL = {(q, a, o): _make_dense_dual(q, a, o) for q in _QUANTS for a, o in (("f32", "f32"), ("bf16", "bf16"))}
+for _fn in DENSE_DUAL.values():
+    globals()[_fn.__name__] = _fn
 
 FUSED: dict[tuple[str, str, str], object] = {}
 for _q in _QUANTS:
@@ -261,6 +337,12 @@ def gguf_gemv_default_form(quant_key: str, rows: int, in_features: int, out_feat
 
 
 def register_kernels(backend: str = "hip_gfx950", *, replace: bool = False) -> None:
+    # the keys hipEngine's dispatcher resolves for raw-layout weights: gemv_* at one row, prefill_* above
+    # (loading/qwen35_gguf_consumer_surface.py:134-144,527-530)
+    for (quant, family, act, out), fn in DENSE.items():
+        register(KernelKey(backend, "linear", f"gguf_{quant}", f"{family}_{act}_{out}_out"), fn, replace=replace)
+    for (quant, act, out), fn in DENSE_DUAL.items():
+        register(KernelKey(backend, "linear", f"gguf_{quant}", f"dual_gemv_{act}_{out}_out"), fn, replace=replace)
     for (act, out), fn in PAIR_SILU.items():
         register(KernelKey(backend, "linear", "gguf_q4_k", f"dual_silu_gemv_{act}_{out}_out"), fn, replace=replace)
     for (quant, act, out), fn in RESIDUAL.items():

@@ -40,6 +40,40 @@ def gguf_q8_1_block_dots_i32(quant_key: str, xq_ptr: int, qweight_ptr: int, dots
                     out_features, stream), runtime)
 
 
+FORM_SLAB, FORM_PSLAB = 3, 4
+
+
+def gguf_gemv_mfma_dots_i32(quant_key: str, form: int, xq_ptr: int, qweight_ptr: int, dots_ptr: int, out_ptr: int,
+                            rows: int, in_features: int, out_features: int, *, stream: int = 0,
+                            library: ctypes.CDLL | None = None, runtime: HipRuntime | None = None) -> None:
+    """The int32 sub-block dots of the decode GEMV's MFMA forms (``FORM_SLAB``: Q4_K; ``FORM_PSLAB``: all four
+    types), written by the production kernel body: ``[rows, out_features, K/32]`` (Q6_K ``K/16``), and the
+    kernel's float32 result ``[rows, out_features]``.  ``xq``: 36-byte q8_1 blocks, ``rows <= 8``."""
+    if rows <= 0 or rows > 8 or out_features <= 0 or in_features <= 0 or in_features % 256:
+        raise ValueError("rows must be in 1..8, out_features positive and in_features divisible by 256")
+    if form not in (FORM_SLAB, FORM_PSLAB):
+        raise ValueError("form must be FORM_SLAB or FORM_PSLAB")
+    validate_pointers(xq_ptr=xq_ptr, qweight_ptr=qweight_ptr, dots_ptr=dots_ptr, out_ptr=out_ptr)
+    fn = entry("hipengine_gfx950_gguf_gemv_mfma_dots_i32", [I32, I32, VOID, VOID, VOID, VOID, I64, I64, I64, VOID], library)
+    check_launch(fn(QUANT_KEY_TO_GGML[quant_key], form, xq_ptr, qweight_ptr, dots_ptr, out_ptr, rows, in_features,
+                    out_features, stream), runtime)
+
+
+def gguf_mmq_dots_i32(quant_key: str, xq_ptr: int, qweight_ptr: int, dots_ptr: int, out_ptr: int, rows: int,
+                      in_features: int, out_features: int, *, stream: int = 0, library: ctypes.CDLL | None = None,
+                      runtime: HipRuntime | None = None) -> None:
+    """The int32 dots of the MMQ prefill GEMM (Q4_K over DS4 blocks: ``[rows, N, K/32]``; Q6_K over D4S4 blocks:
+    ``[rows, N, K/16]``, centred values) and its float32 result, from the production tile engine."""
+    if rows <= 0 or out_features <= 0 or in_features <= 0 or in_features % 256:
+        raise ValueError("rows/out_features must be positive and in_features divisible by 256")
+    if quant_key not in ("gguf_q4_k", "gguf_q6_k"):
+        raise ValueError("the MMQ takes gguf_q4_k or gguf_q6_k weights")
+    validate_pointers(xq_ptr=xq_ptr, qweight_ptr=qweight_ptr, dots_ptr=dots_ptr, out_ptr=out_ptr)
+    fn = entry("hipengine_gfx950_gguf_mmq_dots_i32", [I32, VOID, VOID, VOID, VOID, I64, I64, I64, VOID], library)
+    check_launch(fn(QUANT_KEY_TO_GGML[quant_key], xq_ptr, qweight_ptr, dots_ptr, out_ptr, rows, in_features,
+                    out_features, stream), runtime)
+
+
 def copy_bytes(src_ptr: int, dst_ptr: int, nbytes: int, *, stream: int = 0, library: ctypes.CDLL | None = None,
                runtime: HipRuntime | None = None) -> None:
     """Plain device copy kernel of a known size (calibration of HBM byte counters)."""

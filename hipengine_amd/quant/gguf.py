@@ -59,7 +59,7 @@ GGUF_QUANT_LAYOUTS: dict[GGMLQuantizationType, GGUFQuantLayout] = {
     # half d; half dmin; u8 scales[12]; u8 qs[128]
     GGMLQuantizationType.Q4_K: _blocks(GGMLQuantizationType.Q4_K, QK_K, 2 + 2 + 12 + QK_K // 2, True),
     # half d; half dmin; u8 scales[12]; u8 qh[32]; u8 qs[128]
-    GGMLQuantizationType.Q5_K: _blocks(GGMLQuantizationType.Q5_K, QK_K, 2 + 2 + 12 + QK_K // 8 + QK_K // 2, False),
+    GGMLQuantizationType.Q5_K: _blocks(GGMLQuantizationType.Q5_K, QK_K, 2 + 2 + 12 + QK_K // 8 + QK_K // 2, True),
     # u8 ql[128]; u8 qh[64]; i8 scales[16]; half d
     GGMLQuantizationType.Q6_K: _blocks(GGMLQuantizationType.Q6_K, QK_K, QK_K // 2 + QK_K // 4 + QK_K // 16 + 2, True),
 }

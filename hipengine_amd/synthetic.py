@@ -33,9 +33,9 @@ def synthetic_blocks(qtype: int | GGMLQuantizationType, out_features: int, in_fe
     q = GGMLQuantizationType(int(qtype))
     if q == GGMLQuantizationType.Q6_K:
         blk[..., 208], blk[..., 209] = lo, hi
-    else:                                    # Q4_K (d, dmin) and Q8_0 (d) keep their scale first
+    else:                                    # Q4_K / Q5_K (d, dmin) and Q8_0 (d) keep their scale first
         blk[..., 0], blk[..., 1] = lo, hi
-        if q == GGMLQuantizationType.Q4_K:
+        if q in (GGMLQuantizationType.Q4_K, GGMLQuantizationType.Q5_K):
             blk[..., 2], blk[..., 3] = lo, hi
     tile = blk.reshape(rows, nb * layout.type_size)
     reps = -(-out_features // rows)

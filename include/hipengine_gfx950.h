@@ -111,6 +111,38 @@ HIPENGINE_GFX950_DECLARE_FUSED_ALL(q5_k)
 HIPENGINE_GFX950_DECLARE_FUSED_ALL(q6_k)
 HIPENGINE_GFX950_DECLARE_FUSED_ALL(q8_0)
 
+/* hipEngine's own dense names, which its wrappers bind and its dispatcher reaches through the registry
+ * keys ("linear", quant, "gemv_<act>_<out>_out") and, for rows > 1, ("linear", quant, "prefill_<act>_<out>_out")
+ * (loading/qwen35_gguf_consumer_surface.py:134-144,527-530).  Same argument list; here they run the fused
+ * kernels above, so the arithmetic is q8_1 activations x integer weights (what hipEngine's dp4a kernels
+ * compute), not the float-activation arithmetic of hipEngine's kernels of the same name.  Any rows >= 1:
+ * batches of up to 8 rows per launch.
+ * Replace gguf_q4_k_gemv.hip:2483-2611 (Q4_K) and gguf_k_gemv.hip:5504-5545 (Q5_K, Q6_K, Q8_0). */
+#define HIPENGINE_GFX950_DECLARE_DENSE(q, a, o)                                                          \
+  int hipengine_gguf_##q##_gemv_##a##_##o##_out(                                                         \
+      const void* x, const uint8_t* qweight, void* out, int64_t rows, int64_t in_features,               \
+      int64_t out_features, int64_t threads, hipengine_stream_t stream);
+/* Two matrices over one activation, out_a = W_a x and out_b = W_b x (k and v, gate and up).
+ * Replaces gguf_k_gemv.hip:5546-5560. */
+#define HIPENGINE_GFX950_DECLARE_DENSE_DUAL(q, a, o)                                                     \
+  int hipengine_gguf_##q##_dual_gemv_##a##_##o##_out(                                                    \
+      const void* x, const uint8_t* qweight_a, const uint8_t* qweight_b, void* out_a, void* out_b,       \
+      int64_t rows, int64_t in_features, int64_t out_features, int64_t threads, hipengine_stream_t stream);
+#define HIPENGINE_GFX950_DECLARE_DENSE_ALL(q) \
+  HIPENGINE_GFX950_DECLARE_DENSE(q, f32, f32) \
+  HIPENGINE_GFX950_DECLARE_DENSE(q, f32, fp16) \
+  HIPENGINE_GFX950_DECLARE_DENSE(q, fp16, f32) \
+  HIPENGINE_GFX950_DECLARE_DENSE(q, fp16, fp16) \
+  HIPENGINE_GFX950_DECLARE_DENSE(q, bf16, f32) \
+  HIPENGINE_GFX950_DECLARE_DENSE(q, bf16, fp16) \
+  HIPENGINE_GFX950_DECLARE_DENSE(q, bf16, bf16) \
+  HIPENGINE_GFX950_DECLARE_DENSE_DUAL(q, f32, f32) \
+  HIPENGINE_GFX950_DECLARE_DENSE_DUAL(q, bf16, bf16)
+HIPENGINE_GFX950_DECLARE_DENSE_ALL(q4_k)
+HIPENGINE_GFX950_DECLARE_DENSE_ALL(q5_k)
+HIPENGINE_GFX950_DECLARE_DENSE_ALL(q6_k)
+HIPENGINE_GFX950_DECLARE_DENSE_ALL(q8_0)
+
 /* Pre-quantized: xq is [rows, in_features/32] 36-byte q8_1 blocks.
  * Q4_K replaces gguf_q4_k_q8_1_dp4a_vdr_gemv.hip:321-361 (without its
  * out_features % 8 restriction); Q8_0 replaces gguf_q8_0_dp4a_gemv.hip:345-388;
@@ -196,6 +228,20 @@ int hipengine_gguf_q6_k_mmq32_q8_1_d4s4_f32_bf16_bf16_out(const void* xq, const 
                                                           int64_t rows, int64_t in_features, int64_t out_features,
                                                           hipengine_stream_t stream);
 
+/* Prefill from bf16 activations in one call: x [rows, in_features] bf16 is packed into `workspace`
+ * (DS4 blocks for Q4_K, D4S4 for Q6_K; caller-owned, 16-byte aligned, at least the byte count
+ * hipengine_gfx950_gguf_prefill_workspace_bytes reports = rows * in_features/128 * 144 or 160) and the MMQ
+ * above runs on it: two launches.  ggml_type 12 (Q4_K, out_features % 32 == 0) or 14 (Q6_K); out_kind 0
+ * float32, 1 bf16, 2 fp16.  This is what a ("linear", quant, "prefill_bf16_*_out") caller with 32 or more
+ * rows should reach: hipEngine's prefill signature has no workspace argument, so the Python wrappers of the
+ * prefill keys take it as an optional keyword and fall back to batches of 8 rows through the GEMV without
+ * it.  New here. */
+int hipengine_gfx950_gguf_prefill_workspace_bytes(int32_t ggml_type, int64_t rows, int64_t in_features,
+                                                  int64_t* bytes);
+int hipengine_gfx950_gguf_prefill_bf16(int32_t ggml_type, const void* x, const uint8_t* qweight, void* out,
+                                       int32_t out_kind, int64_t rows, int64_t in_features, int64_t out_features,
+                                       void* workspace, int64_t workspace_bytes, hipengine_stream_t stream);
+
 /* ------------------------------------------------------------------------
  * MoE: routing index, expert-indexed decode GEMV, expert-grouped prefill MMQ
  * Expert weights are [num_experts, out_features, row_bytes] raw blocks.
@@ -276,6 +322,38 @@ int hipengine_qwen35_moe_group_compact_active_source_rows(const int64_t* selecte
                                                           int64_t num_experts, int64_t top_k,
                                                           hipengine_stream_t stream);
 
+/* The step-by-step form of the same index, as hipEngine's runner drives it
+ * (runtime/qwen35_gguf_runner.py:34107-34143): count, prefix, scatter + gather.
+ *   group_count   counts[e] (int32, zeroed by the caller) += lanes whose expert is e.
+ *                 Replaces moe/group_scatter.hip:683-705 (kernel :9-22).
+ *   group_prefix  padded_counts[e] = counts[e] rounded up to pad_multiple; expert_start[0..E] = exclusive
+ *                 prefix of the padded counts; total_padded[0] = their sum.  num_experts <= 2048.
+ *                 Replaces moe/group_scatter.hip:707-733 (kernel :24-60).
+ *   group_scatter_gather_lowp  for every lane with a valid expert e: a slot i in
+ *                 [expert_start[e] + scatter_offsets[e], ...) gets sorted_lanes[i] = lane, sorted_experts[i] = e,
+ *                 sorted_weights[i] = routing_weights[lane] and packed_hidden[i, :] = hidden_states[lane / top_k, :]
+ *                 (16-bit elements); scatter_offsets[e] (int32, zeroed by the caller) ends as the number of
+ *                 lanes placed.  hipEngine takes slots with atomics, in arrival order; here an expert's lanes
+ *                 are placed in ascending lane order, which is one of the orders it can produce and makes the
+ *                 result deterministic.  Replaces moe/group_scatter.hip:1121-1159 (kernel :419-460).
+ *   gather_packed_hidden_lowp  packed_hidden[r, :] = hidden_states[sorted_lanes[r] / top_k, :] for the
+ *                 total_elements / hidden_size rows, zeros where the lane is negative or its token is not in
+ *                 [0, tokens).  Replaces moe/group_scatter.hip:1161-1206 (kernel :462-485). */
+int hipengine_qwen35_moe_group_count(const int64_t* selected_experts, int32_t* counts, int64_t total_lanes,
+                                     int64_t num_experts, hipengine_stream_t stream);
+int hipengine_qwen35_moe_group_prefix(const int32_t* counts, int32_t* padded_counts, int64_t* expert_start,
+                                      int64_t* total_padded, int64_t num_experts, int64_t pad_multiple,
+                                      hipengine_stream_t stream);
+int hipengine_qwen35_moe_group_scatter_gather_lowp(const uint16_t* hidden_states, const int64_t* selected_experts,
+                                                   const float* routing_weights, const int64_t* expert_start,
+                                                   int32_t* scatter_offsets, int64_t* sorted_lanes,
+                                                   int64_t* sorted_experts, float* sorted_weights,
+                                                   uint16_t* packed_hidden, int64_t total_lanes, int64_t num_experts,
+                                                   int64_t top_k, int64_t hidden_size, hipengine_stream_t stream);
+int hipengine_qwen35_moe_gather_packed_hidden_lowp(const uint16_t* hidden_states, const int64_t* sorted_lanes,
+                                                   uint16_t* packed_hidden, int64_t total_elements, int64_t tokens,
+                                                   int64_t top_k, int64_t hidden_size, hipengine_stream_t stream);
+
 /* expert_start_compact[num_experts+1] -> mmq_expert_start[num_experts+1] (row
  * starts with every expert's count rounded up to 32), tile_expert[tile] (expert
  * of each 32-row tile; the first tile_capacity entries are preset to -1 when
@@ -334,6 +412,56 @@ int hipengine_gguf_q4_k_selected_dual_silu_gemv_bf16_bf16_out(const uint16_t* x,
                                                               int64_t num_experts, int64_t in_features,
                                                               int64_t out_features, int64_t threads,
                                                               hipengine_stream_t stream);
+
+/* Decode gate/up pair without the activation: out_a[lane] = W_a[selected[lane]] . x_row,
+ * out_b[lane] = W_b[selected[lane]] . x_row, one pass over both (the "dual" call kind,
+ * loading/gguf_selected_contract.py:305-315).  Replaces gguf_q4_k_gemv.hip:2732-2749. */
+int hipengine_gguf_q4_k_selected_dual_gemv_bf16_bf16_out(const uint16_t* x, const int64_t* selected,
+                                                         const uint8_t* qweight_a, const uint8_t* qweight_b,
+                                                         uint16_t* out_a, uint16_t* out_b, int64_t x_rows,
+                                                         int64_t rows, int64_t num_experts, int64_t in_features,
+                                                         int64_t out_features, int64_t threads,
+                                                         hipengine_stream_t stream);
+
+/* The same over pre-quantized activations: xq is [x_rows, in_features/32] 36-byte q8_1 blocks.
+ * Replaces gguf_q4_k_gemv.hip:2864-2892. */
+int hipengine_gguf_q4_k_selected_dual_gemv_q8_1_dp4a_bf16_bf16_out(const void* xq, const int64_t* selected,
+                                                                   const uint8_t* qweight_a,
+                                                                   const uint8_t* qweight_b, uint16_t* out_a,
+                                                                   uint16_t* out_b, int64_t x_rows, int64_t rows,
+                                                                   int64_t num_experts, int64_t in_features,
+                                                                   int64_t out_features, int64_t threads,
+                                                                   hipengine_stream_t stream);
+
+/* Routed down projection with the weighted sum fused (the "weighted_down" call kind,
+ * loading/gguf_selected_contract.py:50-54,305-315): x is [tokens*top_k, in_features] bf16, one row per lane;
+ * out[t, :] = sum over the token's slots s = 0..top_k-1, in that order, of
+ * routing_weights[t*top_k+s] * (W[selected[t*top_k+s]] . x[t*top_k+s]); lanes with an expert id outside
+ * [0, num_experts) are skipped.  top_k <= 8, tokens*top_k <= 65535.  hipEngine has this call kind for its
+ * IQ families only; the argument list is that of hipengine_gguf_iq4_xs_weighted_selected_down_bf16_bf16_out
+ * (gguf_iq_gemv.hip:2276-2288). */
+int hipengine_gguf_q4_k_weighted_selected_down_bf16_bf16_out(const uint16_t* x, const int64_t* selected,
+                                                             const float* routing_weights, const uint8_t* qweight,
+                                                             uint16_t* out, int64_t tokens, int64_t top_k,
+                                                             int64_t num_experts, int64_t in_features,
+                                                             int64_t out_features, int64_t threads,
+                                                             hipengine_stream_t stream);
+int hipengine_gguf_q6_k_weighted_selected_down_bf16_bf16_out(const uint16_t* x, const int64_t* selected,
+                                                             const float* routing_weights, const uint8_t* qweight,
+                                                             uint16_t* out, int64_t tokens, int64_t top_k,
+                                                             int64_t num_experts, int64_t in_features,
+                                                             int64_t out_features, int64_t threads,
+                                                             hipengine_stream_t stream);
+
+/* Grouped GEMV over gathered rows: x is [compact_rows, in_features] bf16 in expert-major order (the
+ * packed_hidden of the routing index), rows [expert_start[e], expert_start[e+1]) belong to expert e and
+ * out[r, :] = W[e] . x[r, :] for them; rows outside every range are left untouched.  An expert's weights
+ * are read once per batch of 8 of its rows.  num_experts <= 65535.
+ * Replaces gguf_q4_k_gemv.hip:2634-2669 (kernel :378-450; registry key
+ * ("moe_linear", "gguf_q4_k", "selected_grouped_prefill_compact_rowbatch8_bf16_bf16_out"), gguf_q4_k_gemv.py:603-612). */
+int hipengine_gguf_q4_k_selected_grouped_prefill_compact_rowbatch8_bf16_bf16_out(
+    const void* x, const void* expert_start, const void* qweight, void* out, int64_t compact_rows,
+    int64_t num_experts, int64_t in_features, int64_t out_features, hipengine_stream_t stream);
 
 /* The decode kernels with every choice explicit.  ggml_type 12 (Q4_K) or 14 (Q6_K).
  *   mode 0: out[lanes, N] = W_a[selected[lane]] . x[lane / (lanes/x_rows)]
@@ -396,6 +524,20 @@ int hipengine_gfx950_gguf_dequantize_f32(int32_t ggml_type, const uint8_t* block
 int hipengine_gfx950_gguf_q8_1_block_dots_i32(int32_t ggml_type, const void* xq, const uint8_t* qweight,
                                               int32_t* dots, int32_t* qsums, int64_t rows, int64_t in_features,
                                               int64_t out_features, hipengine_stream_t stream);
+
+/* The same dots as the kernels that run on the int8 MFMA produce them: the production kernel body with one
+ * more store per MFMA result.  form 3: the slab form (Q4_K), form 4: the phased slab form (Q4_K, Q5_K, Q6_K,
+ * Q8_0); both in their batch-8 instantiation, xq = 36-byte q8_1 blocks [rows, K/32], rows <= 8, shapes as
+ * the forms take them.  dots as above; out: float32 [rows, out_features], the kernel's normal result. */
+int hipengine_gfx950_gguf_gemv_mfma_dots_i32(int32_t ggml_type, int32_t form, const void* xq, const uint8_t* qweight,
+                                             int32_t* dots, float* out, int64_t rows, int64_t in_features,
+                                             int64_t out_features, hipengine_stream_t stream);
+
+/* The same for the MMQ prefill GEMM: ggml_type 12 (Q4_K, xq = DS4 blocks, dots int32 [rows, N, K/32]) or 14
+ * (Q6_K, xq = D4S4 blocks, dots [rows, N, K/16], of the centred 6-bit values); out: float32 [rows, N]. */
+int hipengine_gfx950_gguf_mmq_dots_i32(int32_t ggml_type, const void* xq, const uint8_t* qweight, int32_t* dots,
+                                       float* out, int64_t rows, int64_t in_features, int64_t out_features,
+                                       hipengine_stream_t stream);
 
 /* dst[0:bytes] = src[0:bytes] with a plain 16-byte-per-lane kernel (bytes % 16 == 0):
  * the known-size launch that HBM counter readings are calibrated against. */

@@ -65,16 +65,19 @@ def test_decode_gemv_full_size(dev, short, qt, n, k):
     w = synthetic_blocks(qt, n, k, seed=n + k, tile_rows=TILE)
     dw = dev.put(w)
     rng = np.random.default_rng(k)
-    x8 = (rng.standard_normal((8, k)) * 0.5).astype(np.float32)
     dout = dev.empty(8 * n * 4)
     for batch in (1, 2, 4, 8):
-        x = np.ascontiguousarray(x8[:batch])
+        # fresh activations and a freshly poisoned output for every batch: the batches take different kernel
+        # forms, and an element one of them failed to write must not pass on what the previous one left there
+        x = (rng.standard_normal((batch, k)) * 0.5).astype(np.float32)
         dx = dev.put(x)
+        dev.runtime.memset(dout.ptr, 0xFF, 8 * n * 4)         # all-ones bits: NaN as float32
         G.FUSED[(short, "f32", "f32")](dx.ptr, dw.ptr, dout.ptr, batch, k, n)
-        got = dev.get(dout, np.float32, (batch, n))
+        got = dev.get(dout, np.float32, (8, n))
         dev.free(dx)
+        assert np.all(got[batch:].view(np.uint32) == 0xFFFFFFFF)   # rows past the batch are not touched
         ref = O.gguf_quant_gemv(O.dequantize_q8_1(O.quantize_q8_1(x)), w[:TILE], qt)
-        _assert_close(got, np.tile(ref, (1, -(-n // TILE)))[:, :n])
+        _assert_close(got[:batch], np.tile(ref, (1, -(-n // TILE)))[:, :n])
     dev.free(dw, dout)
 
 

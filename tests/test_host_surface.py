@@ -115,6 +115,45 @@ def test_backend_registers_the_documented_keys(clean_registry):
     assert fn.__name__ == "gguf_q4_k_q8_1_fused_gemv_f32_f32_out"
 
 
+def test_every_raw_row_of_the_dispatch_surface_resolves_to_this_backend(clean_registry):
+    """hipEngine's dispatcher resolves, for a raw-layout weight, ("linear", weight quant, "gemv_<act>_<out>_out") and
+    rewrites gemv_ to prefill_ for rows > 1 (loading/qwen35_gguf_consumer_surface.py:134-144,527-530); with
+    missing="error" nothing may fall through to another backend.  The MoE consumers and call kinds of
+    loading/gguf_selected_contract.py:31-54 resolve too."""
+    from hipengine_amd.kernels import hip_gfx950
+
+    hip_gfx950.register_backend_kernels(replace=True)
+    raw_rows = (("bf16", "bf16"), ("bf16", "fp16"), ("bf16", "f32"), ("f32", "f32"))
+    for q in ("gguf_q4_k", "gguf_q5_k", "gguf_q6_k", "gguf_q8_0"):
+        for act, out in raw_rows:
+            for family in ("gemv", "prefill"):
+                variant = f"{family}_{act}_{out}_out"
+                assert R.is_registered(KernelKey("hip_gfx950", "linear", q, variant))
+                fn = R.resolve(backend="hip_gfx950", layer="linear", quant=q, variant=variant, missing="error")
+                assert fn.__name__ == f"{q}_{variant}"
+        assert R.resolve(backend="hip_gfx950", layer="linear", quant=q, variant="dual_gemv_bf16_bf16_out",
+                         missing="error").__name__ == f"{q}_dual_gemv_bf16_bf16_out"
+    for layer, q, variant in (
+            ("linear", "gguf_q4_k", "selected_gemv_bf16_bf16_out"),
+            ("linear", "gguf_q4_k", "selected_dual_gemv_bf16_bf16_out"),
+            ("linear", "gguf_q4_k", "selected_dual_silu_gemv_bf16_bf16_out"),
+            ("linear", "gguf_q4_k", "selected_dual_gemv_q8_1_dp4a_bf16_bf16_out"),
+            ("moe_linear", "gguf_q4_k", "selected_gemv_decode_bf16_bf16_out"),
+            ("moe_linear", "gguf_q4_k", "selected_dual_silu_gemv_decode_bf16_bf16_out"),
+            ("moe_linear", "gguf_q4_k", "selected_weighted_down_gemv_decode_bf16_bf16_out"),
+            ("moe_linear", "gguf_q6_k", "selected_weighted_down_gemv_decode_bf16_bf16_out"),
+            ("moe_linear", "gguf_q4_k", "selected_grouped_prefill_compact_rowbatch8_bf16_bf16_out"),
+            ("moe_group_count", "generic", "selected_experts"), ("moe_group_prefix", "w4_paro", "qwen35"),
+            ("moe_group_scatter_gather", "generic", "bf16_lane_rows"), ("moe_gather_packed_hidden", "generic", "bf16_lanes")):
+        assert R.is_registered(KernelKey("hip_gfx950", layer, q, variant)), (layer, q, variant)
+    # a prefill wrapper checks its arguments like hipEngine's before it touches the library
+    fn = R.resolve(backend="hip_gfx950", layer="linear", quant="gguf_q4_k", variant="prefill_bf16_bf16_out")
+    with pytest.raises(ValueError, match="divisible"):
+        fn(16, 16, 16, 40, 100, 64)
+    with pytest.raises(ValueError, match="threads"):
+        fn(16, 16, 16, 40, 256, 64, threads=7)
+
+
 def test_quant_plugin_records():
     p = quant.resolve_quant("gguf_q4_k")
     assert (p.weight_storage, p.activation_preprocess, p.compute_dtype, p.scale_granularity, p.calibration_artifact,
