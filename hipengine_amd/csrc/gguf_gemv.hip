@@ -188,14 +188,14 @@ Plan default_plan(int qt, int rows, int64_t K, int64_t N) {
 // The kernel form a batch of `chunk` <= 8 rows takes, and the rows of it that go in one launch.
 enum GemvForm { FORM_ROW_STRIDED = 0, FORM_RUN = 1, FORM_STREAM = 2, FORM_SLAB = 3, FORM_PSLAB = 4 };
 
-// Q4_K, K <= 6144: the int8 MFMA slab form wins for batches of 3 and more; at batch 2 when a slab is a single
-// 32-row step (N <= 8192); at batch 1 only below 4096 rows (above, the stream form is ~1 us faster) or where
-// the stream form does not apply.  Measured on MI355X.
+// Q4_K, K <= 6144: the int8 MFMA slab form wins for batches of 3 and more (17408x5120 at batch 3: 17.0 us against
+// 23.0 for the stream form), the stream form at batch 1 and 2 wherever it applies (batch 1: 4.5 against 6.3 us
+// at 1024x5120, 10.8 against 15.8 at 17408x5120; batch 2: 5.5 against 6.9 and 14.0 against 15.5; within 0.5 us
+// of each other at batch 2 for K = 4096, N = 5120..8192).  Measured on MI355X.
 bool slab_preferred(int qt, int chunk, int64_t K, int64_t N, const SlabPlan& sl) {
   if (!sl.ok) return false;
   if (chunk >= 3) return true;
-  if (chunk == 2) return sl.rows_wg <= 32;
-  return sl.rows_wg < 16 || (sl.rows_wg <= 32 && !default_stream_plan(qt, chunk, K, N).ok);
+  return !default_stream_plan(qt, chunk, K, N).ok;
 }
 
 GemvForm pick_form(int qt, int& chunk, int64_t K, int64_t N, const void* w) {
@@ -238,7 +238,7 @@ int launch_gemv(int qt, const void* x, int x_kind, const uint8_t* w, void* out, 
         rc = launch_gemv_pslab(qt, xr, x_kind, w, outr, out_kind, chunk, K, N, default_pslab_plan(qt, chunk, K, N, w),
                                stream);
       } else if (form == FORM_STREAM) {
-        rc = launch_gemv_stream(qt, xr, x_kind, w, outr, out_kind, chunk, K, N, tuned_stream_plan(qt, chunk, K, N),
+        rc = launch_gemv_stream(qt, xr, x_kind, w, outr, out_kind, chunk, K, N, default_stream_plan(qt, chunk, K, N),
                                 stream);
       } else {
         rc = launch_gemv_run(qt, xr, x_kind, w, outr, out_kind, chunk, K, N, default_run_plan(qt, chunk, K, N), stream);
@@ -553,7 +553,7 @@ extern "C" int hipengine_gfx950_gguf_pair_silu_gemv(int32_t ggml_type, const voi
     return launch_gemv_pslab(ggml_type, x, x_kind, qweight_up, out, out_kind, r, in_features, out_features, pu, stream,
                              nullptr, out);
   }
-  const StreamPlan sp = tuned_stream_plan(ggml_type, static_cast<int>(rows), in_features, out_features);
+  const StreamPlan sp = default_stream_plan(ggml_type, static_cast<int>(rows), in_features, out_features, FUSE_PAIR);
   if (!sp.ok) return static_cast<int>(hipErrorInvalidValue);
   StreamFusion f;
   f.fuse = FUSE_PAIR; f.w_up = qweight_up; f.round_mid = round_mid;
@@ -581,7 +581,7 @@ extern "C" int hipengine_gfx950_gguf_gemv_residual(int32_t ggml_type, const void
     return launch_gemv_pslab(ggml_type, x, x_kind, qweight, out, out_kind, static_cast<int>(rows), in_features,
                              out_features, pp, stream, residual);
   }
-  const StreamPlan sp = tuned_stream_plan(ggml_type, static_cast<int>(rows), in_features, out_features);
+  const StreamPlan sp = default_stream_plan(ggml_type, static_cast<int>(rows), in_features, out_features, FUSE_RESIDUAL);
   if (!sp.ok) return static_cast<int>(hipErrorInvalidValue);
   StreamFusion f;
   f.fuse = FUSE_RESIDUAL; f.residual = residual;

@@ -49,8 +49,7 @@ struct StreamFusion {
   const void* residual = nullptr;
   int round_mid = 0;
 };
-StreamPlan default_stream_plan(int qt, int rows, int64_t K, int64_t N);
-StreamPlan tuned_stream_plan(int qt, int rows, int64_t K, int64_t N);
+StreamPlan default_stream_plan(int qt, int rows, int64_t K, int64_t N, int fuse = FUSE_NONE);
 int launch_gemv_stream(int qt, const void* x, int x_kind, const uint8_t* w, void* out, int out_kind, int rows,
                        int64_t K, int64_t N, const StreamPlan& p, hipStream_t stream,
                        const StreamFusion& fusion = StreamFusion());

@@ -49,28 +49,26 @@ struct StreamVariant {
   StreamVariant { QT, B, D, S, LONG_K, FUSE, gemv_stream_kernel<QT, B, D, S, -1, FUSE>,                           \
                   {gemv_stream_kernel<QT, B, D, S, KIND_F32, FUSE>, gemv_stream_kernel<QT, B, D, S, KIND_BF16, FUSE>, \
                    nullptr, nullptr} }
-#define STREAM_VARIANT_FUSED(QT, B, S, LONG_K, FUSE) STREAM_VARIANT_FUSED_D(QT, B, 3, S, LONG_K, FUSE)
 
-const StreamVariant kStream[] = {
-    STREAM_VARIANT_BY_KIND(GGML_Q4_K, 1, 3, 2, false), STREAM_VARIANT_BY_KIND(GGML_Q4_K, 2, 3, 2, false),
-    STREAM_VARIANT_BY_KIND(GGML_Q4_K, 1, 2, 2, false),
-    STREAM_VARIANT_BY_KIND(GGML_Q6_K, 1, 3, 2, false), STREAM_VARIANT_BY_KIND(GGML_Q6_K, 2, 3, 2, false),
-    STREAM_VARIANT_BY_KIND(GGML_Q8_0, 1, 3, 2, false), STREAM_VARIANT_BY_KIND(GGML_Q8_0, 2, 3, 2, false),
-    STREAM_VARIANT_BY_KIND(GGML_Q5_K, 1, 3, 2, false), STREAM_VARIANT_BY_KIND(GGML_Q5_K, 2, 3, 2, false),
-    STREAM_VARIANT_BY_KIND(GGML_Q5_K, 1, 3, 5, true),
-    STREAM_VARIANT_BY_KIND(GGML_Q4_K, 1, 3, 5, true), STREAM_VARIANT_BY_KIND(GGML_Q6_K, 1, 3, 5, true),
-    STREAM_VARIANT_BY_KIND(GGML_Q8_0, 1, 3, 5, true),
-    STREAM_VARIANT_BY_KIND(GGML_Q4_K, 2, 3, 5, true), STREAM_VARIANT_BY_KIND(GGML_Q6_K, 2, 3, 5, true),
-    STREAM_VARIANT(GGML_Q4_K, 4, 3), STREAM_VARIANT(GGML_Q4_K, 8, 3), STREAM_VARIANT(GGML_Q6_K, 4, 3),
-    STREAM_VARIANT(GGML_Q6_K, 8, 3), STREAM_VARIANT(GGML_Q8_0, 4, 3), STREAM_VARIANT(GGML_Q8_0, 8, 3),
-    // gate/up pair with SiLU (Q4_K) and projection + residual (Q4_K, Q6_K), batch 1 and 2
-    STREAM_VARIANT_FUSED(GGML_Q4_K, 1, 2, false, FUSE_PAIR), STREAM_VARIANT_FUSED(GGML_Q4_K, 2, 2, false, FUSE_PAIR),
-    STREAM_VARIANT_FUSED(GGML_Q4_K, 1, 2, false, FUSE_RESIDUAL), STREAM_VARIANT_FUSED(GGML_Q4_K, 2, 2, false, FUSE_RESIDUAL),
-    STREAM_VARIANT_FUSED(GGML_Q6_K, 1, 2, false, FUSE_RESIDUAL), STREAM_VARIANT_FUSED(GGML_Q6_K, 2, 2, false, FUSE_RESIDUAL),
-    STREAM_VARIANT_FUSED(GGML_Q4_K, 1, 5, true, FUSE_RESIDUAL), STREAM_VARIANT_FUSED(GGML_Q6_K, 1, 5, true, FUSE_RESIDUAL),
-    // the tall Q4_K shape at batch 1 on a ring of two (see tuned_stream_plan)
-    STREAM_VARIANT_FUSED_D(GGML_Q4_K, 1, 2, 2, false, FUSE_PAIR), STREAM_VARIANT_FUSED_D(GGML_Q4_K, 1, 2, 2, false, FUSE_RESIDUAL),
-};
+#define STREAM_RING(D)                                                                                              \
+    STREAM_VARIANT_BY_KIND(GGML_Q4_K, 1, D, 2, false), STREAM_VARIANT_BY_KIND(GGML_Q4_K, 2, D, 2, false),               \
+    STREAM_VARIANT_BY_KIND(GGML_Q6_K, 1, D, 2, false), STREAM_VARIANT_BY_KIND(GGML_Q6_K, 2, D, 2, false),               \
+    STREAM_VARIANT_BY_KIND(GGML_Q8_0, 1, D, 2, false), STREAM_VARIANT_BY_KIND(GGML_Q8_0, 2, D, 2, false),               \
+    STREAM_VARIANT_BY_KIND(GGML_Q5_K, 1, D, 2, false), STREAM_VARIANT_BY_KIND(GGML_Q5_K, 2, D, 2, false),               \
+    STREAM_VARIANT_BY_KIND(GGML_Q5_K, 1, D, 5, true),                                                                   \
+    STREAM_VARIANT_BY_KIND(GGML_Q4_K, 1, D, 5, true), STREAM_VARIANT_BY_KIND(GGML_Q6_K, 1, D, 5, true),                 \
+    STREAM_VARIANT_BY_KIND(GGML_Q8_0, 1, D, 5, true),                                                                   \
+    STREAM_VARIANT_BY_KIND(GGML_Q4_K, 2, D, 5, true), STREAM_VARIANT_BY_KIND(GGML_Q6_K, 2, D, 5, true),                 \
+    STREAM_VARIANT(GGML_Q4_K, 4, D), STREAM_VARIANT(GGML_Q4_K, 8, D), STREAM_VARIANT(GGML_Q6_K, 4, D),                  \
+    STREAM_VARIANT(GGML_Q6_K, 8, D), STREAM_VARIANT(GGML_Q8_0, 4, D), STREAM_VARIANT(GGML_Q8_0, 8, D),                  \
+    /* gate/up pair with SiLU (Q4_K) and projection + residual (Q4_K, Q6_K), batch 1 and 2 */                           \
+    STREAM_VARIANT_FUSED_D(GGML_Q4_K, 1, D, 2, false, FUSE_PAIR), STREAM_VARIANT_FUSED_D(GGML_Q4_K, 2, D, 2, false, FUSE_PAIR),         \
+    STREAM_VARIANT_FUSED_D(GGML_Q4_K, 1, D, 2, false, FUSE_RESIDUAL), STREAM_VARIANT_FUSED_D(GGML_Q4_K, 2, D, 2, false, FUSE_RESIDUAL), \
+    STREAM_VARIANT_FUSED_D(GGML_Q6_K, 1, D, 2, false, FUSE_RESIDUAL), STREAM_VARIANT_FUSED_D(GGML_Q6_K, 2, D, 2, false, FUSE_RESIDUAL), \
+    STREAM_VARIANT_FUSED_D(GGML_Q4_K, 1, D, 5, true, FUSE_RESIDUAL), STREAM_VARIANT_FUSED_D(GGML_Q6_K, 1, D, 5, true, FUSE_RESIDUAL)
+
+const StreamVariant kStream[] = {STREAM_RING(2), STREAM_RING(3)};
+
 
 // The variant a launch takes: of those for (type, batch bucket, ring depth, epilogue), the one with the fewest
 // up-front groups per thread that still cover K with this many waves (nb*8 groups, 16 teams per wave);
@@ -89,71 +87,61 @@ const StreamVariant* pick_stream_variant(int qt, int b, int d, int fuse, int nb,
   return best;
 }
 
-const StreamVariant* find_stream_variant(int qt, int b, int d, bool long_k = false, int fuse = FUSE_NONE) {
-  const StreamVariant* fallback = nullptr;
-  for (const StreamVariant& v : kStream) {
-    if (v.qt != qt || v.b != b || v.d != d || v.fuse != fuse) continue;
-    if (v.long_k == long_k) return &v;
-    if (!v.long_k) fallback = &v;
-  }
-  return fallback;
-}
-
-
-
-
-
-
-
-
 }  // namespace
 
-// The stream form applies to K >= 4096 (a 16-block load then spans at most two
-// rows), batch <= 2, when every resident wave gets at least a few loads.
-StreamPlan default_stream_plan(int qt, int rows, int64_t K, int64_t N) {
+// Geometry of a stream launch: rows per chunk (as a shift) and chunks of the matrix.
+struct StreamGeometry {
+  int chunk_shift;
+  int64_t nchunks;
+};
+StreamGeometry stream_geometry(int nb, int64_t N) {
+  StreamGeometry g{0, 0};
+  while (((nb << g.chunk_shift) & 15) != 0) ++g.chunk_shift;          // rows per chunk: 16 / gcd(nb, 16)
+  g.nchunks = (N + (1 << g.chunk_shift) - 1) >> g.chunk_shift;
+  return g;
+}
+
+// Groups (per matrix) of the workgroup with the most chunks.
+int64_t stream_max_groups(int nb, const StreamGeometry& g, int grid) {
+  const int64_t chunks = (g.nchunks + grid - 1) / grid;
+  return ((chunks << g.chunk_shift) * nb) / 16;
+}
+
+// The stream form applies to K >= 4096 (a group of 16 blocks then spans at most two rows) and
+// batch <= 8, from one group per CU on.  One workgroup per CU, two loads in flight per wave (three measured
+// slower at every shape and batch).  Waves per workgroup: a workgroup works in rounds of `waves` groups, an
+// even number of rounds (the ring is unrolled), and a round of fewer than 8 waves is bound by the latency of
+// its loads rather than by their number; so the cost of w waves is rounds(w) * max(w, 8), and the wave
+// count is 8 unless another is more than 2 % cheaper.  Measured on MI355X at batch 1 (us, best wave count
+// against 8 waves): 17408x5120 Q4_K 11.2 (11 waves) / 11.6; 5120x5120 Q4_K 5.80 (7) / 5.86; 5120x17408 Q6_K
+// 18.6 (11) / 18.9; 151936x5120 Q6_K 108.6 (8); 6144x5120 Q4_K 5.95 (8; 5 waves, with no idle slot, 6.7).
+// The float32 row sums do not depend on the plan: a group's lanes and the order of a row's groups are fixed by
+// K alone.
+StreamPlan default_stream_plan(int qt, int rows, int64_t K, int64_t N, int fuse) {
   StreamPlan p{};
   const int nb = static_cast<int>(K / QK_K);
   p.b = batch_bucket(rows);
-  p.d = 3;
+  p.d = 2;
   p.waves = 8;
-  const int64_t total_loads = N * nb / 16;
-  // 8 resident waves per CU once every wave gets 3 loads or more, else 4 per CU
-  p.waves_total = total_loads >= 6144 ? kComputeUnits * 8 : kComputeUnits * 4;
-  if (p.b == 1 && total_loads >= 6144) {
-    // whole rows per wave: 8, 10 or 12 waves per CU, whichever splits the rows most
-    // evenly (N = 5120: 2.5 rows per wave at 8, exactly 2 at 10)
-    double best = 1e9;
-    for (int w = 8; w <= 12; w += 2) {
-      const int64_t wt = static_cast<int64_t>(kComputeUnits) * w;
-      if (wt > N) break;
-      const double imbalance = static_cast<double>((N + wt - 1) / wt) * wt / static_cast<double>(N);
-      if (imbalance < best - 0.1) { best = imbalance; p.waves = w; p.waves_total = static_cast<int>(wt); }
-    }
+  p.waves_total = 0;
+  if (rows > 8 || nb < 16 || N < 1) return p;
+  const StreamGeometry g = stream_geometry(nb, N);
+  const int grid = static_cast<int>(g.nchunks < kComputeUnits ? g.nchunks : kComputeUnits);
+  const int mats = fuse == FUSE_PAIR ? 2 : 1;
+  const int64_t groups = mats * stream_max_groups(nb, g, grid);
+  const int max_waves = p.b == 1 ? 12 : 8;
+  auto cost = [&](int w) {
+    const int64_t rounds = (groups + w - 1) / w;
+    return ((rounds + p.d - 1) / p.d * p.d) * (w < 8 ? 8 : w);
+  };
+  int64_t best = cost(8);
+  for (int w = 5; w <= max_waves; ++w) {
+    if (cost(w) * 100 < best * 98) { best = cost(w); p.waves = w; }
   }
-  // every wave should get the ring's three loads; Q4_K at batch 1 still beats the slab form with two
-  // (5120 x 5120 on 10 waves per CU: 6.7 us against 7.8)
-  const int min_loads = (qt == GGML_Q4_K && p.b == 1) ? 2 : 3;
-  p.ok = rows <= 8 && nb >= 16 && total_loads >= min_loads * static_cast<int64_t>(p.waves_total) &&
-         N >= p.waves_total && gemv_run_lds_bytes(qt, p.b, static_cast<int>(K)) <= kMaxLds &&
-         find_stream_variant(qt, p.b, p.d) != nullptr;
-  return p;
-}
-
-// The plan the entry points launch with.  A tall Q4_K matrix at batch 1 (every wave of a 12-per-CU grid still
-// gets six loads: the 17408 x 5120 gate/up shape) runs 12 waves per CU with two loads in flight each:
-// measured 12.1 us against 12.3 for 8 waves with three (the same bytes in flight, rows split 6/5
-// instead of 9/8).
-// The fused forms take the same plan as the plain projection, so that their float32 sums are the same.
-StreamPlan tuned_stream_plan(int qt, int rows, int64_t K, int64_t N) {
-  StreamPlan p = default_stream_plan(qt, rows, K, N);
-  const int64_t nb = K / QK_K;
-  const int64_t wt = static_cast<int64_t>(kComputeUnits) * 12;
-  if (p.ok && qt == GGML_Q4_K && p.b == 1 && nb <= 32 && N * nb / 16 >= 6 * wt && find_stream_variant(qt, 1, 2) != nullptr &&
-      find_stream_variant(qt, 1, 2, false, FUSE_PAIR) != nullptr && find_stream_variant(qt, 1, 2, false, FUSE_RESIDUAL) != nullptr) {
-    p.d = 2;
-    p.waves = 12;
-    p.waves_total = static_cast<int>(wt);
-  }
+  p.waves_total = p.waves * grid;
+  p.ok = N * nb / 16 >= kComputeUnits &&
+         gemv_run_lds_bytes(qt, p.b, static_cast<int>(K)) + static_cast<size_t>(groups) * 2 * p.b * sizeof(float) <= kMaxLds &&
+         pick_stream_variant(qt, p.b, p.d, fuse, nb, p.waves) != nullptr;
   return p;
 }
 
@@ -163,16 +151,27 @@ int launch_gemv_stream(int qt, const void* x, int x_kind, const uint8_t* w, void
   const int nb = static_cast<int>(K / QK_K);
   const StreamVariant* v = p.waves > 0 ? pick_stream_variant(qt, p.b, p.d, fusion.fuse, nb, p.waves) : nullptr;
   if (!v || nb < 16 || rows > p.b || p.waves < 1 || p.waves > (p.b == 1 ? 12 : 8) || p.waves_total < p.waves ||
-      (p.waves_total % p.waves) != 0 || p.waves_total > N) {
+      (p.waves_total % p.waves) != 0) {
     return static_cast<int>(hipErrorInvalidValue);
   }
-  size_t lds = gemv_run_lds_bytes(qt, p.b, static_cast<int>(K));
-  if (fusion.fuse == FUSE_PAIR) {
-    // gate results wait per wave; a wave may hold at most STREAM_PAIR_MAX_ROWS rows
-    if (!fusion.w_up || (N + p.waves_total - 1) / p.waves_total > STREAM_PAIR_MAX_ROWS) return static_cast<int>(hipErrorInvalidValue);
-    lds += static_cast<size_t>(p.waves) * p.b * STREAM_PAIR_MAX_ROWS * sizeof(float);
-  }
+  if (fusion.fuse == FUSE_PAIR && !fusion.w_up) return static_cast<int>(hipErrorInvalidValue);
   if (fusion.fuse == FUSE_RESIDUAL && !fusion.residual) return static_cast<int>(hipErrorInvalidValue);
+  const int grid = p.waves_total / p.waves;
+  const int mats = fusion.fuse == FUSE_PAIR ? 2 : 1;
+  const StreamGeometry geo = stream_geometry(nb, N);
+  const int chunk_shift = geo.chunk_shift;
+  const int64_t nchunks = geo.nchunks;
+  if (grid > nchunks) return static_cast<int>(hipErrorInvalidValue);
+  const int base_chunks = static_cast<int>(nchunks / grid);
+  int rounds[2];
+  int64_t max_groups = 0;
+  for (int big = 0; big < 2; ++big) {
+    const int64_t groups = mats * (((static_cast<int64_t>(base_chunks + big) << chunk_shift) * nb) / 16);
+    rounds[big] = static_cast<int>((groups + p.waves - 1) / p.waves);
+    max_groups = groups;
+  }
+  // the activation image, then two partial sums per group and batch row
+  const size_t lds = gemv_run_lds_bytes(qt, p.b, static_cast<int>(K)) + static_cast<size_t>(max_groups) * 2 * p.b * sizeof(float);
   if (lds > kMaxLds) return static_cast<int>(hipErrorInvalidValue);
   // the kind-specialised kernels stage the whole row from the groups fetched up front
   const bool up_front = nb * 8 <= v->s * p.waves * 16;
@@ -187,9 +186,13 @@ int launch_gemv_stream(int qt, const void* x, int x_kind, const uint8_t* w, void
   a.x_kind = x_kind; a.out_kind = out_kind;
   a.rows = rows; a.K = static_cast<int>(K); a.N = static_cast<int>(N);
   a.waves = p.waves; a.waves_total = p.waves_total;
-  a.base_rows = static_cast<int>(N / p.waves_total);
+  a.chunk_shift = chunk_shift;
+  a.base_chunks = base_chunks;
+  a.extra_chunks = static_cast<int>(nchunks - static_cast<int64_t>(base_chunks) * grid);
+  a.rounds[0] = rounds[0]; a.rounds[1] = rounds[1];
+  a.inv_nb = 1.0f / static_cast<float>(nb);
   a.w_up = fusion.w_up; a.residual = fusion.residual; a.round_mid = fusion.round_mid;
-  hipLaunchKernelGGL(fn, dim3(p.waves_total / p.waves), dim3(p.waves * 64), lds, stream, a);
+  hipLaunchKernelGGL(fn, dim3(grid), dim3(p.waves * 64), lds, stream, a);
   return static_cast<int>(hipGetLastError());
 }
 
