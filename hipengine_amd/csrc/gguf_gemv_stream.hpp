@@ -14,11 +14,11 @@
 //     workgroup, in order, are its run;
 //   * the waves of the workgroup take the groups of the run round robin (group i*waves + wave in round i).
 //     Workgroups advance at about the same pace, so at any time the whole chip reads one window of a few MB
-//     that moves through the matrix, every workgroup a different 11.5 KB of it.  Contiguous shares per
-//     workgroup or per wave instead make the launch time depend on the share's size in bytes, through the
-//     memory channels that concurrent readers then have in common: measured at 17408x5120, same bytes and same
-//     wave count, 16.5 us for shares of 16320 B per wave against 12.4 us for 17800 B, and 17.3 us for 64 rows
-//     (45 * 4096 B) per workgroup against 12.0 us for 68 rows;
+//     that moves through the matrix, every workgroup a different 11.5 KB of it, and the waves are balanced to
+//     within one group whatever the rows per workgroup and the wave count.  Measured at 17408x5120 (us per
+//     launch, 11 or 12 waves per CU): whole rows per wave 11.4; a contiguous, equal share of blocks per wave
+//     12.4 to 16.5 depending on the share's size in bytes; groups round robin within a contiguous share per
+//     workgroup 11.7 to 12.0; this form 10.8 to 11.2.
 //   * the groups do not divide evenly over the waves; the idle slots are put in round 0,
 //     so that the last round, which nothing else hides, is a full one;
 //   * D wave loads are kept in flight: after a load's registers are consumed
