@@ -330,17 +330,32 @@ DEFINE_FUSED_ALL(q8_0, GGML_Q8_0)
 
 // Two matrices over one activation (gate and up, or k and v): out_a = W_a x, out_b = W_b x
 // (gguf_k_gemv.hip:5546-5560; Q4_K has the form for its pack8 layout only, gguf_q4_k_gemv.hip:2970).
+// One launch of the stream form where it applies (rows <= 2), else one launch per matrix.
+int launch_dual(int qt, const void* x, int x_kind, const uint8_t* w_a, const uint8_t* w_b, void* out_a, void* out_b,
+                int out_kind, int64_t rows, int64_t K, int64_t N, hipStream_t stream) {
+  if (!x || !w_a || !w_b || !out_a || !out_b || rows <= 0 || K <= 0 || N <= 0 || (K % QK_K) != 0) {
+    return static_cast<int>(hipErrorInvalidValue);
+  }
+  if (rows <= 2) {
+    const StreamPlan sp = default_stream_plan(qt, static_cast<int>(rows), K, N, FUSE_DUAL);
+    if (sp.ok) {
+      StreamFusion f;
+      f.fuse = FUSE_DUAL; f.w_up = w_b; f.out_b = out_b;
+      return launch_gemv_stream(qt, x, x_kind, w_a, out_a, out_kind, static_cast<int>(rows), K, N, sp, stream, f);
+    }
+  }
+  const int rc = launch_gemv(qt, x, x_kind, w_a, out_a, out_kind, rows, K, N, nullptr, stream);
+  if (rc != static_cast<int>(hipSuccess)) return rc;
+  return launch_gemv(qt, x, x_kind, w_b, out_b, out_kind, rows, K, N, nullptr, stream);
+}
+
 #define DEFINE_DENSE_DUAL(QNAME, QT, ANAME, AKIND, ONAME, OKIND)                                          \
   extern "C" int hipengine_gguf_##QNAME##_dual_gemv_##ANAME##_##ONAME##_out(                              \
       const void* x, const uint8_t* qweight_a, const uint8_t* qweight_b, void* out_a, void* out_b,        \
       int64_t rows, int64_t in_features, int64_t out_features, int64_t threads, hipStream_t stream) {     \
     (void)threads;                                                                                        \
-    if (!qweight_b || !out_b) return static_cast<int>(hipErrorInvalidValue);                              \
-    const int rc = launch_gemv(QT, x, AKIND, qweight_a, out_a, OKIND, rows, in_features, out_features,    \
-                               nullptr, stream);                                                          \
-    if (rc != static_cast<int>(hipSuccess)) return rc;                                                    \
-    return launch_gemv(QT, x, AKIND, qweight_b, out_b, OKIND, rows, in_features, out_features, nullptr,   \
-                       stream);                                                                           \
+    return launch_dual(QT, x, AKIND, qweight_a, qweight_b, out_a, out_b, OKIND, rows, in_features,        \
+                       out_features, stream);                                                             \
   }
 
 #define DEFINE_DENSE_ALL(QNAME, QT)                         \
@@ -519,6 +534,36 @@ extern "C" int hipengine_gfx950_gguf_gemv_mfma_dots_i32(int32_t ggml_type, int32
                              out_features, p, stream, nullptr, nullptr, dots);
   }
   return static_cast<int>(hipErrorInvalidValue);
+}
+
+// ---- several matrices over one activation --------------------------------------------
+
+extern "C" int hipengine_gfx950_gguf_multi_gemv(int32_t count, const int32_t* ggml_types, const void* x, int32_t x_kind,
+                                                const uint8_t* const* qweights, void* const* outs, int32_t out_kind,
+                                                int64_t rows, int64_t in_features, const int64_t* out_features,
+                                                hipStream_t stream) {
+  if (count < 1 || count > 4 || !ggml_types || !x || !qweights || !outs || !out_features || x_kind < KIND_F32 ||
+      x_kind > KIND_Q8_1 || out_kind < KIND_F32 || out_kind > KIND_F16 || rows <= 0 || in_features <= 0 ||
+      (in_features % QK_K) != 0) {
+    return static_cast<int>(hipErrorInvalidValue);
+  }
+  int qt[4];
+  for (int i = 0; i < count; ++i) {
+    qt[i] = ggml_types[i];
+    if (!qweights[i] || !outs[i] || out_features[i] <= 0 || !find_variant(qt[i], 1, 1, 1)) {
+      return static_cast<int>(hipErrorInvalidValue);
+    }
+  }
+  if (rows <= 2 && stream_multi_ok(count, qt, static_cast<int>(rows), in_features, out_features)) {
+    return launch_gemv_stream_multi(count, qt, x, x_kind, qweights, outs, out_kind, static_cast<int>(rows), in_features,
+                                    out_features, stream);
+  }
+  for (int i = 0; i < count; ++i) {
+    const int rc = launch_gemv(qt[i], x, x_kind, qweights[i], outs[i], out_kind, rows, in_features, out_features[i],
+                               nullptr, stream);
+    if (rc != static_cast<int>(hipSuccess)) return rc;
+  }
+  return static_cast<int>(hipSuccess);
 }
 
 // ---- fused epilogues: gate/up pair with SiLU, projection + residual -------------------

@@ -38,7 +38,7 @@ int launch_gemv_pslab(int qt, const void* x, int x_kind, const uint8_t* w, void*
 int pslab_raise_lds_limits();
 
 // ---- stream form (resident waves, ring of loads in flight) ----
-enum StreamFuse { FUSE_NONE = 0, FUSE_PAIR = 1, FUSE_RESIDUAL = 2 };   // epilogue of the stream kernels
+enum StreamFuse { FUSE_NONE = 0, FUSE_PAIR = 1, FUSE_RESIDUAL = 2, FUSE_DUAL = 3 };   // epilogue of the stream kernels
 struct StreamPlan {
   int b, d, waves, waves_total;
   bool ok;
@@ -48,11 +48,17 @@ struct StreamFusion {
   const uint8_t* w_up = nullptr;
   const void* residual = nullptr;
   int round_mid = 0;
+  void* out_b = nullptr;      // FUSE_DUAL
 };
 StreamPlan default_stream_plan(int qt, int rows, int64_t K, int64_t N, int fuse = FUSE_NONE);
 int launch_gemv_stream(int qt, const void* x, int x_kind, const uint8_t* w, void* out, int out_kind, int rows,
                        int64_t K, int64_t N, const StreamPlan& p, hipStream_t stream,
                        const StreamFusion& fusion = StreamFusion());
+// Up to four matrices of any supported types over one activation (rows <= 2), one launch.
+bool stream_multi_ok(int count, const int* qt, int rows, int64_t K, const int64_t* N);
+int launch_gemv_stream_multi(int count, const int* qt, const void* x, int x_kind, const uint8_t* const* w,
+                             void* const* out, int out_kind, int rows, int64_t K, const int64_t* N,
+                             hipStream_t stream);
 int stream_raise_lds_limits();
 
 }  // namespace hipengine_gfx950

@@ -56,7 +56,8 @@ struct GemvStreamArgs {
   int extra_chunks; // instructions here); the first extra_chunks workgroups take one more
   int rounds[2];    // rounds of a workgroup with base_chunks / base_chunks + 1 chunks: ceil(groups / waves)
   float inv_nb;     // 1 / (K / 256)
-  const uint8_t* w_up;      // FUSE_PAIR: the second matrix (w is the gate); out = silu(gate.x) * (up.x)
+  const uint8_t* w_up;      // FUSE_PAIR: the second matrix (w is the gate), out = silu(gate.x) * (up.x); FUSE_DUAL: the second matrix
+  void* out_b;              // FUSE_DUAL: the second matrix's output
   const void* residual;     // FUSE_RESIDUAL: [rows, N] of the output type, added to the projection
   int round_mid;            // FUSE_PAIR: round gate and up to the output type before the SiLU
 };
@@ -74,21 +75,22 @@ struct GemvStreamArgs {
 //                  up matrix (groups do not straddle the two); the stored value is silu(gate) * up,
 //                  with gate and up rounded to the output type first when round_mid is set
 //                  (gguf_q4_k_gemv.hip:652-657);
-//   FUSE_RESIDUAL  out = round(projection) + residual in the output type (gguf_q4_k_gemv.hip:1669-1678).
+//   FUSE_RESIDUAL  out = round(projection) + residual in the output type (gguf_q4_k_gemv.hip:1669-1678);
+//   FUSE_DUAL      two matrices of one shape as in the pair form, each stored to its own output (gguf_k_gemv.hip:5546-5560).
 // The row sums of the three forms are the same floats: the groups of a matrix depend only on the workgroup's rows.
 template <int QT, int B, int D, int S, int XK = -1, int FUSE = FUSE_NONE>
-__device__ __forceinline__ void gemv_stream_workgroup(const GemvStreamArgs& a, uint8_t* smem) {
+__device__ __forceinline__ void gemv_stream_workgroup(const GemvStreamArgs& a, uint8_t* smem, int wg, int grid) {
   using Regs = WeightRegs<GemvTraits<QT>::REGS>;
   constexpr int Q8S = run_q8_stride<QT>();
   constexpr int SUPER = GemvTraits<QT>::SUPER_BYTES;
-  constexpr int MATS = FUSE == FUSE_PAIR ? 2 : 1;
+  constexpr int MATS = (FUSE == FUSE_PAIR || FUSE == FUSE_DUAL) ? 2 : 1;
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int q = lane & 3, j = lane >> 2;
   const int nb = a.K / QK_K;
 
   // the workgroup's chunks wg, wg + workgroups, ...: its run of "virtual" rows and blocks, per matrix
-  const int wg = blockIdx.x, lr = a.chunk_shift;
+  const int lr = a.chunk_shift;
   const int big = wg < a.extra_chunks ? 1 : 0;
   const int vrows = (a.base_chunks + big) << lr;
   const int total = vrows * nb;                  // blocks of the run: a multiple of 16
@@ -97,7 +99,7 @@ __device__ __forceinline__ void gemv_stream_workgroup(const GemvStreamArgs& a, u
   // round i of this wave is group g_first + i * waves of MATS * ngroups; negative or too large: idle
   const int g_first = wave - (rounds * a.waves - MATS * ngroups);
   // virtual row v is row v + (v >> lr) * gap + (wg << lr) of the matrix
-  const int gap = (static_cast<int>(gridDim.x) - 1) << lr;
+  const int gap = (grid - 1) << lr;
   const int row_off = wg << lr;
   uint8_t* q8 = smem;
   float* rec = reinterpret_cast<float*>(q8 + B * nb * Q8S);
@@ -121,7 +123,7 @@ __device__ __forceinline__ void gemv_stream_workgroup(const GemvStreamArgs& a, u
     const int g_all = g_first + i * a.waves;                         // over both matrices of the pair form
     int g = g_all;
     const uint8_t* base = a.w;
-    if constexpr (FUSE == FUSE_PAIR) {
+    if constexpr (MATS == 2) {
       if (g >= ngroups) { g -= ngroups; base = a.w_up; }
     }
     const int blk_raw = g * 16 + j;
@@ -202,6 +204,9 @@ __device__ __forceinline__ void gemv_stream_workgroup(const GemvStreamArgs& a, u
         if (a.round_mid) { gate = round_to_kind(gate, a.out_kind); up = round_to_kind(up, a.out_kind); }
         const float sig = 1.0f / (1.0f + expf(-gate));
         store_scalar(a.out, idx, gate * sig * up, a.out_kind);
+      } else if constexpr (FUSE == FUSE_DUAL) {
+        store_scalar(a.out, idx, v[0], a.out_kind);
+        store_scalar(a.out_b, idx, v[MATS - 1], a.out_kind);
       } else if constexpr (FUSE == FUSE_RESIDUAL) {
         store_scalar(a.out, idx, round_to_kind(v[0], a.out_kind) + load_scalar(a.residual, idx, a.out_kind), a.out_kind);
       } else {

@@ -256,6 +256,31 @@ def gguf_gemv_residual(quant_key: str, x_ptr: int, x_kind: str, qweight_ptr: int
     check_launch(code, runtime)
 
 
+def gguf_multi_gemv(quant_keys, x_ptr: int, x_kind: str, qweight_ptrs, out_ptrs, out_kind: str, rows: int,
+                    in_features: int, out_features, *, stream: int = 0, library: ctypes.CDLL | None = None,
+                    runtime: HipRuntime | None = None) -> None:
+    """Up to four matrices over one activation, ``out_i = W_i x`` (the q, k and v projections of an attention
+    block), whatever their GGUF types and row counts.  Rows 1-2 with ``in_features >= 4096``: one launch, the
+    workgroups divided between the matrices by their bytes; otherwise one launch per matrix.  Every output has
+    the bits its own fused GEMV call gives (C symbol ``hipengine_gfx950_gguf_multi_gemv``)."""
+    count = len(quant_keys)
+    if not (1 <= count <= 4) or len(qweight_ptrs) != count or len(out_ptrs) != count or len(out_features) != count:
+        raise ValueError("multi_gemv takes 1 to 4 matrices, with one weight, output and out_features each")
+    for n in out_features:
+        validate_linear(rows, in_features, n)
+    validate_pointers(x_ptr=x_ptr, **{f"qweight_{i}": p for i, p in enumerate(qweight_ptrs)},
+                      **{f"out_{i}": p for i, p in enumerate(out_ptrs)})
+    types = (I32 * count)(*[QUANT_KEY_TO_GGML[q] for q in quant_keys])
+    weights = (VOID * count)(*qweight_ptrs)
+    outs = (VOID * count)(*out_ptrs)
+    ns = (I64 * count)(*out_features)
+    fn = entry("hipengine_gfx950_gguf_multi_gemv",
+               [I32, ctypes.POINTER(I32), VOID, I32, ctypes.POINTER(VOID), ctypes.POINTER(VOID), I32, I64, I64,
+                ctypes.POINTER(I64), VOID], library)
+    check_launch(fn(count, types, x_ptr, _KINDS[x_kind], weights, outs, _KINDS[out_kind], rows, in_features, ns, stream),
+                 runtime)
+
+
 def _make_pair_silu(act: str, out: str):
     def wrapper(x_ptr: int, qweight_gate_ptr: int, qweight_up_ptr: int, out_ptr: int, rows: int, in_features: int,
                 out_features: int, *, stream: int = 0, library: ctypes.CDLL | None = None,
@@ -345,6 +370,7 @@ def register_kernels(backend: str = "hip_gfx950", *, replace: bool = False) -> N
         register(KernelKey(backend, "linear", f"gguf_{quant}", f"dual_gemv_{act}_{out}_out"), fn, replace=replace)
     for (act, out), fn in PAIR_SILU.items():
         register(KernelKey(backend, "linear", "gguf_q4_k", f"dual_silu_gemv_{act}_{out}_out"), fn, replace=replace)
+    register(KernelKey(backend, "linear", "gguf", "multi_gemv"), gguf_multi_gemv, replace=replace)
     for (quant, act, out), fn in RESIDUAL.items():
         register(KernelKey(backend, "linear", f"gguf_{quant}", f"gemv_{act}_residual_{out}_out"), fn, replace=replace)
     for (quant, act, out), fn in FUSED.items():

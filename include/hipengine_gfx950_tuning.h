@@ -34,11 +34,12 @@ int hipengine_gfx950_gguf_q8_1_fused_gemv_run_tuned(int32_t ggml_type, const voi
                                                     int32_t rows_per_wave, int32_t loads_per_chunk, int32_t waves,
                                                     hipengine_stream_t stream);
 
-/* The same for the "stream" form (waves_total resident waves, `waves` per
- * workgroup, each owning a contiguous range of rows and keeping loads_in_flight
- * 16-block loads in flight; the library builds loads_in_flight = 3 only, deeper
- * rings measured slower).  rows <= 8, in_features >= 4096,
- * waves_total <= out_features.  New here. */
+/* The same for the "stream" form (waves_total / waves workgroups of `waves` waves, all
+ * resident; chunks of rows dealt round robin to the workgroups, groups of 16 blocks
+ * round robin to a workgroup's waves, each wave keeping loads_in_flight loads in
+ * flight; the library builds loads_in_flight = 2 only, deeper rings measured
+ * slower).  rows <= 8, in_features >= 4096, at most one workgroup per chunk of
+ * 16 / gcd(in_features / 256, 16) rows.  New here. */
 int hipengine_gfx950_gguf_q8_1_fused_gemv_stream_tuned(int32_t ggml_type, const void* x, int32_t x_kind,
                                                        const uint8_t* qweight, void* out, int32_t out_kind,
                                                        int64_t rows, int64_t in_features, int64_t out_features,

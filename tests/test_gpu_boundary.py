@@ -18,6 +18,7 @@ from hipengine_amd.kernels.hip_gfx950.quant import gguf_moe as M
 from hipengine_amd.kernels.hip_gfx950.quant import gguf_q8_1_gemv as G
 from hipengine_amd.kernels.hip_gfx950.quant import gguf_quantize as Q
 from hipengine_amd.kernels.hip_gfx950.quant import gguf_verify as V
+from hipengine_amd.synthetic import synthetic_blocks
 
 pytestmark = pytest.mark.gpu
 
@@ -116,7 +117,7 @@ def test_prefill_key_with_workspace_runs_the_mmq(dev, quant, n):
 
 
 @pytest.mark.parametrize("quant", ["gguf_q4_k", "gguf_q6_k", "gguf_q8_0"])
-@pytest.mark.parametrize("rows", [1, 8])
+@pytest.mark.parametrize("rows", [1, 2, 8])
 def test_dense_dual_gemv(dev, quant, rows):
     """Two matrices over one activation (k and v of an attention block): each output equals the single GEMV's."""
     k, n = 5120, 1024
@@ -134,6 +135,42 @@ def test_dense_dual_gemv(dev, quant, rows):
         G.FUSED[(short, "bf16", "bf16")](dx.ptr, w_dev.ptr, ds.ptr, rows, k, n)
         assert np.array_equal(got, dev.get(ds, np.uint16, (rows, n)))
     dev.free(dx, dwa, dwb, da, db, ds)
+
+
+@pytest.mark.parametrize("rows", [1, 2, 3])
+@pytest.mark.parametrize("mats", [(("gguf_q4_k", 640), ("gguf_q4_k", 256), ("gguf_q6_k", 256)),
+                                  (("gguf_q8_0", 130), ("gguf_q5_k", 1021)),
+                                  (("gguf_q6_k", 96), ("gguf_q4_k", 64), ("gguf_q4_k", 32), ("gguf_q8_0", 7))],
+                         ids=["qkv", "two_ragged", "four_small"])
+def test_multi_gemv_matches_the_single_calls_and_the_oracle(dev, rows, mats):
+    """Several matrices of mixed types and row counts over one activation: one launch at rows <= 2 (a launch per
+    matrix above); every output has the bits of its own fused GEMV call and meets the oracle's tolerance."""
+    k = 5120
+    rng = np.random.default_rng(31 + rows)
+    x = rng.standard_normal((rows, k)).astype(np.float32)
+    # Q5_K has no quantizer in the oracle: random valid blocks
+    ws = [synthetic_blocks(QT[q], n, k, seed=5 + i, tile_rows=n) if q == "gguf_q5_k" else O.random_weight(QT[q], n, k, seed=5 + i)
+          for i, (q, n) in enumerate(mats)]
+    fn = _resolve("linear", "gguf", "multi_gemv")
+    dx = dev.put(x)
+    dws = [dev.put(w) for w in ws]
+    outs = [dev.empty(rows * n * 4) for _, n in mats]
+    single = [dev.empty(rows * n * 4) for _, n in mats]
+    for o, (_, n) in zip(outs, mats):
+        dev.runtime.memset(o.ptr, 0xFF, rows * n * 4)
+    fn([q for q, _ in mats], dx.ptr, "f32", [d.ptr for d in dws], [o.ptr for o in outs], "f32", rows, k,
+       [n for _, n in mats], stream=0, runtime=dev.runtime)
+    xq = O.dequantize_q8_1(O.quantize_q8_1(x))
+    for (q, n), w, dw, o, sgl in zip(mats, ws, dws, outs, single):
+        G.FUSED[(q.removeprefix("gguf_"), "f32", "f32")](dx.ptr, dw.ptr, sgl.ptr, rows, k, n)
+        got = dev.get(o, np.float32, (rows, n)).copy()
+        alone = dev.get(sgl, np.float32, (rows, n))
+        if rows > 2 or G.gguf_gemv_default_form(q, rows, k, n)[0] == "stream":
+            # the same kernel form as the call of its own: the same float32 sums
+            assert np.array_equal(got.view(np.uint32), alone.view(np.uint32)), (q, n)
+        _close(got, O.gguf_quant_gemv(xq, w, QT[q]))
+        _close(alone, O.gguf_quant_gemv(xq, w, QT[q]))
+    dev.free(dx, *dws, *outs, *single)
 
 
 # ---- MoE call kinds -------------------------------------------------------------------------

@@ -318,24 +318,27 @@ def test_pslab_form_q5_k(dev, rows, k, n, waves, bpw, wgs):
         _check_f32(default, xq, w, O.GGML_Q5_K)
 
 
-@pytest.mark.parametrize("quant,d,waves,waves_total", [("gguf_q4_k", 3, 4, 64), ("gguf_q4_k", 3, 10, 120),
-                                                      ("gguf_q6_k", 3, 12, 96), ("gguf_q8_0", 3, 8, 64),
-                                                      ("gguf_q4_k", 2, 12, 96), ("gguf_q4_k", 2, 4, 64)])
-def test_stream_form_explicit_layouts(dev, quant, d, waves, waves_total):
-    """Stream form with explicit wave counts (up to 12 waves per workgroup at batch 1); ring depths built: 3, and 2
-    for Q4_K.  With 4 waves the two activation groups per thread fetched up front do not cover K = 5120, so the
-    launch takes the kernel that loops over the rest; with 10 or 12 they do and it takes the one without that loop."""
+@pytest.mark.parametrize("quant,d,waves,waves_total,n", [("gguf_q4_k", 2, 4, 64, 256), ("gguf_q4_k", 2, 10, 120, 256),
+                                                        ("gguf_q6_k", 2, 12, 96, 256), ("gguf_q8_0", 2, 8, 64, 256),
+                                                        ("gguf_q4_k", 2, 12, 96, 1021), ("gguf_q5_k", 2, 5, 35, 333),
+                                                        ("gguf_q6_k", 2, 7, 7 * 64, 255)])
+def test_stream_form_explicit_layouts(dev, quant, d, waves, waves_total, n):
+    """Stream form with explicit wave and workgroup counts (up to 12 waves per workgroup at batch 1, ring depth 2),
+    also with row counts that leave the last chunk of 4 rows partial and the workgroups with unequal chunk counts.
+    With 4 waves the two activation groups per thread fetched up front do not cover K = 5120, so the launch takes
+    the kernel that loops over the rest; with 10 or 12 they do and it takes the one without that loop."""
     rng = np.random.default_rng(5 + waves_total)
-    rows, k, n = 1, 5120, 256
+    rows, k = 1, 5120
     x = rng.standard_normal((rows, k)).astype(np.float32)
-    w = O.random_weight(QT[quant], n, k, seed=3)
+    qt = O.GGML_Q5_K if quant == "gguf_q5_k" else QT[quant]
+    w = _random_q5_k(n, k, seed=3) if quant == "gguf_q5_k" else O.random_weight(qt, n, k, seed=3)
     dx, dw = dev.put(x), dev.put(w)
     dout = dev.empty(rows * n * 4)
     G.gguf_q8_1_fused_gemv_stream_tuned(quant, dx.ptr, "f32", dw.ptr, dout.ptr, "f32", rows, k, n, loads_in_flight=d,
                                         waves=waves, waves_total=waves_total)
     got = dev.get(dout, np.float32, (rows, n))
     dev.free(dx, dw, dout)
-    _check_f32(got, O.quantize_q8_1(x), w, QT[quant])
+    _check_f32(got, O.quantize_q8_1(x), w, qt)
 
 
 def test_output_canaries_untouched(dev):
