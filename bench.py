@@ -138,6 +138,25 @@ class Harness:
                 "weight_host": w, "x_host": x, "spread_us": groups}
 
 
+    def read_ceiling_case(self, nbytes: int, steps: int, warmup: int):
+        """Seconds per launch of the library's read-only probe (resident waves, 16 bytes per lane, loads only) over
+        buffers of `nbytes`, rotated like the weights of a GEMV case: what a launch that only reads reaches."""
+        from hipengine_amd.kernels.hip_gfx950.quant.gguf_verify import read_probe
+
+        copies = max(2, -(-2 * MALL_BYTES // nbytes))
+        bufs = [self.memory.malloc(nbytes, runtime=self.rt) for _ in range(copies)]
+        for b in bufs:
+            self.rt.memset(b.ptr, 0x5A, nbytes)
+        best = None
+        for waves, depth in ((8, 4), (12, 2), (16, 2)):
+            _, ev = self.time_launches(lambda i: read_probe(bufs[i % copies].ptr, nbytes, waves_per_workgroup=waves,
+                                                            loads_in_flight=depth), steps, warmup)
+            if best is None or ev < best[0]:
+                best = (ev, waves, depth)
+        for b in bufs:
+            self.memory.free(b)
+        return best
+
     def ffn_case(self, rows: int, steps: int, warmup: int, seed: int = 7):
         """Dense 27B FFN at decode: gate/up pair with SiLU fused (one launch) and the down projection with the
         residual add fused (one launch), against the unfused sequence (3 GEMVs; its SiLU and add kernels are
@@ -440,6 +459,14 @@ def main() -> None:
                 "GB/s": round(lbytes / lsec / 1e9, 1), "frac_hbm": round(lbytes / lsec / 1e9 / HBM_PEAK_GBS, 4),
                 "tok_per_s_64_layers_matmuls_only": round(batch / (64 * lsec), 1)}
 
+        # what a launch that only reads the same bytes reaches, for the headline weight and for the lm_head
+        for label, nbytes in (("50MB", 17408 * 20 * 144), ("638MB", 151936 * 20 * 210)):
+            sec, waves, depth = h.read_ceiling_case(nbytes, steps, max(5, args.warmup // 5))
+            extra[f"read_only_ceiling_{label}"] = {
+                "what": "library read probe: 256 workgroups of resident waves, 16-byte loads only, rotating buffers",
+                "us": round(sec * 1e6, 2), "GB/s": round(nbytes / sec / 1e9, 1),
+                "frac_hbm": round(nbytes / sec / 1e9 / HBM_PEAK_GBS, 4), "waves_per_cu": waves, "loads_in_flight": depth}
+
         ev_f, ev_u, wbytes = h.ffn_case(1, steps, max(5, args.warmup // 5))
         extra["ffn_27b_b1_fused_pair_silu_and_down_residual"] = {
             "us": round(ev_f * 1e6, 1), "launches": 2, "GB/s": round(wbytes / ev_f / 1e9, 1),
@@ -474,6 +501,9 @@ def main() -> None:
                 "us": round(sec * 1e6, 1), "expert_GB/s": round(touched / sec / 1e9, 1),
                 "int8_TOPS": round(ops / sec / 1e12, 2), "launches": 2 if tokens <= 8 else 10}
 
+    # the MMQ half of the metric, as a second roofline object: int8 operations 2*M*N*K of the Q4_K prefill GEMM at
+    # M = 2048 over its HIP-event time, against the dense int8 MFMA peak
+    mmq_sec, mmq_ops = h.mmq_case("q4_k", 2048, 5120, 17408, max(10, args.steps // 50), 2)
     result = {
         "metric": METRIC,
         "value": round(gbs, 2),
@@ -491,7 +521,12 @@ def main() -> None:
                    "weight_copies_rotated": main_case["copies"], "bytes_per_step": main_case["bytes"]},
         "roofline": {"bound": "hbm", "achieved": round(achieved, 2), "peak": HBM_PEAK_GBS, "unit": "GB/s",
                      "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": measured_traffic(),
-                     "kernel_us": round(main_case["event_s"] * 1e6, 3)},
+                     "kernel_us": round(main_case["event_s"] * 1e6, 3),
+                     "traffic_source": str(TRAFFIC_FILE.relative_to(ROOT)) if measured_traffic() is not None else None},
+        "roofline_mmq": {"bound": "int8_mfma", "achieved": round(mmq_ops / mmq_sec / 1e12, 2), "peak": INT8_PEAK_TOPS,
+                         "unit": "TOP/s", "frac": round(mmq_ops / mmq_sec / 1e12 / INT8_PEAK_TOPS, 4),
+                         "kernel_us": round(mmq_sec * 1e6, 1),
+                         "workload": "Q4_K 17408x5120 x DS4 activations, M = 2048 (MMQ prefill GEMM)"},
         "cpu_baseline": None if args.no_cpu else cpu_baseline(main_case["weight_host"], main_case["x_host"],
                                                                main_case["bytes"]),
         "extra": extra,

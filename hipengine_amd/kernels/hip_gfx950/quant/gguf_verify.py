@@ -74,6 +74,17 @@ def gguf_mmq_dots_i32(quant_key: str, xq_ptr: int, qweight_ptr: int, dots_ptr: i
                     out_features, stream), runtime)
 
 
+def read_probe(src_ptr: int, nbytes: int, *, waves_per_workgroup: int = 8, loads_in_flight: int = 4, sink_ptr: int = 0,
+               stream: int = 0, library: ctypes.CDLL | None = None, runtime: HipRuntime | None = None) -> None:
+    """Read-only pass over a device buffer with the streaming GEMV's load shape (the ceiling a launch that only
+    reads reaches; C symbol ``hipengine_gfx950_read_probe``)."""
+    if nbytes < 1024:
+        raise ValueError("nbytes must be at least 1024")
+    validate_pointers(src_ptr=src_ptr)
+    fn = entry("hipengine_gfx950_read_probe", [VOID, I64, I32, I32, VOID, VOID], library)
+    check_launch(fn(src_ptr, nbytes, waves_per_workgroup, loads_in_flight, sink_ptr or None, stream), runtime)
+
+
 def copy_bytes(src_ptr: int, dst_ptr: int, nbytes: int, *, stream: int = 0, library: ctypes.CDLL | None = None,
                runtime: HipRuntime | None = None) -> None:
     """Plain device copy kernel of a known size (calibration of HBM byte counters)."""
