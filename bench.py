@@ -37,8 +37,8 @@ if str(ROOT) not in sys.path:
 HBM_PEAK_GBS = 8000.0          # MI355X HBM3E, published
 INT8_PEAK_TOPS = 5000.0        # dense int8 MFMA, published
 METRIC = "Q4_K decode GEMV GB/s (% HBM peak); MMQ prefill int8 TOPS (% MFMA peak)"
-GGML = {"q8_0": 8, "q4_k": 12, "q6_k": 14}
-BLOCK = {"q8_0": (32, 34), "q4_k": (256, 144), "q6_k": (256, 210)}
+GGML = {"q8_0": 8, "q4_k": 12, "q5_k": 13, "q6_k": 14}
+BLOCK = {"q8_0": (32, 34), "q4_k": (256, 144), "q5_k": (256, 176), "q6_k": (256, 210)}
 MALL_BYTES = 256 << 20
 PREWARM_S = 0.15               # untimed launches ahead of every timed region (clock ramp after idle)
 TRAFFIC_FILE = ROOT / "profiles" / "gemv_stream_q4k_17408x5120_b1_pmc.md"
@@ -277,7 +277,8 @@ class Harness:
             fn = M.gguf_q4_k_q8_1_mmq32_vdr_dense_bf16_f32_out
         else:
             Q.gguf_q8_1_d4s4_f32_quantize_bf16(dx.ptr, dxq.ptr, m, k)
-            fn = M.gguf_q6_k_mmq32_q8_1_d4s4_f32_bf16_f32_out
+            fn = (M.gguf_q5_k_mmq32_q8_1_d4s4_f32_bf16_f32_out if quant == "q5_k"
+                  else M.gguf_q6_k_mmq32_q8_1_d4s4_f32_bf16_f32_out)
         _, ev = self.time_launches(lambda i: fn(dxq.ptr, dw.ptr, dout.ptr, m, k, n), steps, warmup)
         for buf in (dw, dx, dxq, dout):
             self.memory.free(buf)
@@ -491,6 +492,7 @@ def main() -> None:
             "mmq_q4_k_17408x5120_m2048": ("q4_k", 2048, 5120, 17408),
             "mmq_q4_k_17408x5120_m8192": ("q4_k", 8192, 5120, 17408),
             "mmq_q6_k_5120x17408_m2048": ("q6_k", 2048, 17408, 5120),
+            "mmq_q5_k_17408x5120_m2048": ("q5_k", 2048, 5120, 17408),
         }.items():
             sec, ops = h.mmq_case(quant, m, kk, nn, msteps, 2)
             extra[name] = {"us": round(sec * 1e6, 1), "int8_TOPS": round(ops / sec / 1e12, 1),

@@ -54,8 +54,8 @@ __global__ void __launch_bounds__(Tile::THREADS, MIN_WAVES) mmq_q4_k_ds4_kernel(
   typename Tile::Smem& s = *reinterpret_cast<typename Tile::Smem*>(smem_raw);
   const int m0 = blockIdx.x * Tile::BM, n0 = blockIdx.y * Tile::BN;
   const int steps = a.K / 128;
-  const int64_t w_row_bytes = static_cast<int64_t>(a.K / QK_K) * Q4_K_BYTES;
-  const int64_t x_row_bytes = static_cast<int64_t>(steps) * DS4_BYTES;
+  const int64_t w_row_bytes = static_cast<int64_t>(a.K / QK_K) * Tile::W_BLOCK;
+  const int64_t x_row_bytes = static_cast<int64_t>(steps) * Tile::A_BYTES;
   Tile::template run<PREFETCH>(
       a.xq, x_row_bytes, a.w, w_row_bytes, steps, s,
       [=](int row) { return static_cast<int64_t>(min(m0 + row, a.M - 1)); },
@@ -74,13 +74,14 @@ void launch_q4_tile(const MmqArgs& a, hipStream_t stream) {
 }
 
 // Verification: the same tile engine, which also writes every int32 sub-block dot to dots[M, N, K/32].
-__global__ void __launch_bounds__(THREADS, 2) mmq_q4_k_ds4_dump_kernel(MmqArgs a, int32_t* __restrict__ dots) {
+template <class Tile>
+__global__ void __launch_bounds__(Tile::THREADS, 2) mmq_tile_dump_kernel(MmqArgs a, int32_t* __restrict__ dots) {
   extern __shared__ __align__(16) uint8_t smem_raw[];
-  DenseQ4::Smem& s = *reinterpret_cast<DenseQ4::Smem*>(smem_raw);
-  const int m0 = blockIdx.x * BM, n0 = blockIdx.y * BN;
+  typename Tile::Smem& s = *reinterpret_cast<typename Tile::Smem*>(smem_raw);
+  const int m0 = blockIdx.x * Tile::BM, n0 = blockIdx.y * Tile::BN;
   const int steps = a.K / 128;
-  const int64_t w_row_bytes = static_cast<int64_t>(a.K / QK_K) * Q4_K_BYTES;
-  const int64_t x_row_bytes = static_cast<int64_t>(steps) * DS4_BYTES;
+  const int64_t w_row_bytes = static_cast<int64_t>(a.K / QK_K) * Tile::W_BLOCK;
+  const int64_t x_row_bytes = static_cast<int64_t>(steps) * Tile::A_BYTES;
   auto row_of = [=](int row) { return static_cast<int64_t>(min(m0 + row, a.M - 1)); };
   auto col_of = [=](int col) { return static_cast<int64_t>(min(n0 + col, a.N - 1)); };
   auto emit = [=](int row, int col, float v) {
@@ -91,7 +92,7 @@ __global__ void __launch_bounds__(THREADS, 2) mmq_q4_k_ds4_dump_kernel(MmqArgs a
     const int m = m0 + row, n = n0 + col;
     if (m < a.M && n < a.N) dots[(static_cast<int64_t>(m) * a.N + n) * (a.K / 32) + sb] = dot;
   };
-  DenseQ4::run<true, decltype(row_of), decltype(col_of), decltype(emit), true, decltype(dump)>(
+  Tile::template run<true, decltype(row_of), decltype(col_of), decltype(emit), true, decltype(dump)>(
       a.xq, x_row_bytes, a.w, w_row_bytes, steps, s, row_of, col_of, emit, dump);
 }
 
@@ -335,6 +336,30 @@ DEFINE_MMQ_Q4(hipengine_gguf_q4_k_q8_1_mmq32_vdr_dense_bf16_bf16_out, KIND_BF16)
 DEFINE_MMQ_Q4(hipengine_gguf_q4_k_q8_1_mmq32_ctl_dense_bf16_f32_out, KIND_F32)
 DEFINE_MMQ_Q4(hipengine_gguf_q4_k_q8_1_mmq32_ctl_dense_bf16_bf16_out, KIND_BF16)
 
+// Q5_K x D4S4: the same tile engine with the fifth bit and float32 activation scales and sums.
+using DenseQ5 = Q4Tile<2, 2, 2, 2, MMQ_Q5K_D4S4>;
+
+int launch_q5(const void* xq, const uint8_t* w, void* out, int out_kind, int64_t M, int64_t K, int64_t N,
+              hipStream_t stream) {
+  if (!xq || !w || !out || M <= 0 || M > (1 << 20) || K <= 0 || (K % QK_K) != 0 || N <= 0 || (N % 32) != 0 ||
+      N > (1 << 24) || out_kind < KIND_F32 || out_kind > KIND_F16) {
+    return static_cast<int>(hipErrorInvalidValue);
+  }
+  MmqArgs a{static_cast<const uint8_t*>(xq), w, out, out_kind, static_cast<int>(M), static_cast<int>(K),
+            static_cast<int>(N)};
+  launch_q4_tile<DenseQ5, true, 2>(a, stream);
+  return static_cast<int>(hipGetLastError());
+}
+
+#define DEFINE_MMQ_Q5(SYMBOL, OKIND)                                                                        \
+  extern "C" int SYMBOL(const void* xq, const uint8_t* qweight, void* out, int64_t rows, int64_t in_features, \
+                        int64_t out_features, hipStream_t stream) {                                         \
+    return launch_q5(xq, qweight, out, OKIND, rows, in_features, out_features, stream);                     \
+  }
+
+DEFINE_MMQ_Q5(hipengine_gguf_q5_k_mmq32_q8_1_d4s4_f32_bf16_f32_out, KIND_F32)
+DEFINE_MMQ_Q5(hipengine_gguf_q5_k_mmq32_q8_1_d4s4_f32_bf16_bf16_out, KIND_BF16)
+
 #define DEFINE_MMQ_Q6(SYMBOL, OKIND)                                                                        \
   extern "C" int SYMBOL(const void* xq, const uint8_t* qweight, void* out, int64_t rows, int64_t in_features, \
                         int64_t out_features, hipStream_t stream) {                                         \
@@ -358,7 +383,10 @@ extern "C" int hipengine_gfx950_gguf_mmq_dots_i32(int32_t ggml_type, const void*
   const dim3 grid(static_cast<unsigned>((rows + BM - 1) / BM), static_cast<unsigned>((out_features + BN - 1) / BN));
   if (ggml_type == GGML_Q4_K) {
     if ((out_features % 32) != 0) return static_cast<int>(hipErrorInvalidValue);
-    hipLaunchKernelGGL(mmq_q4_k_ds4_dump_kernel, grid, dim3(THREADS), sizeof(DenseQ4::Smem), stream, a, dots);
+    hipLaunchKernelGGL(mmq_tile_dump_kernel<DenseQ4>, grid, dim3(THREADS), sizeof(DenseQ4::Smem), stream, a, dots);
+  } else if (ggml_type == GGML_Q5_K) {
+    if ((out_features % 32) != 0) return static_cast<int>(hipErrorInvalidValue);
+    hipLaunchKernelGGL(mmq_tile_dump_kernel<DenseQ5>, grid, dim3(THREADS), sizeof(DenseQ5::Smem), stream, a, dots);
   } else if (ggml_type == GGML_Q6_K) {
     hipLaunchKernelGGL(mmq_q6_k_d4s4_kernel<true>, grid, dim3(THREADS), sizeof(Q6Smem), stream, a, dots);
   } else {
@@ -372,7 +400,7 @@ extern "C" int hipengine_gfx950_gguf_mmq_dots_i32(int32_t ggml_type, const void*
 extern "C" int hipengine_gfx950_gguf_prefill_workspace_bytes(int32_t ggml_type, int64_t rows, int64_t in_features,
                                                              int64_t* bytes) {
   if (!bytes || rows <= 0 || in_features <= 0 || (in_features % QK_K) != 0 ||
-      (ggml_type != GGML_Q4_K && ggml_type != GGML_Q6_K)) {
+      (ggml_type != GGML_Q4_K && ggml_type != GGML_Q5_K && ggml_type != GGML_Q6_K)) {
     return static_cast<int>(hipErrorInvalidValue);
   }
   *bytes = rows * (in_features / 128) * (ggml_type == GGML_Q4_K ? DS4_BYTES : D4S4_BYTES);
@@ -397,6 +425,10 @@ extern "C" int hipengine_gfx950_gguf_prefill_bf16(int32_t ggml_type, const void*
   }
   const int prc = hipengine_gguf_q8_1_d4s4_f32_quantize_bf16(x, workspace, rows, in_features, stream);
   if (prc != static_cast<int>(hipSuccess)) return prc;
+  if (ggml_type == GGML_Q5_K) {
+    if ((out_features % 32) != 0) return static_cast<int>(hipErrorInvalidValue);
+    return launch_q5(workspace, qweight, out, out_kind, rows, in_features, out_features, stream);
+  }
   return launch_q6(workspace, qweight, out, out_kind, rows, in_features, out_features, stream);
 }
 

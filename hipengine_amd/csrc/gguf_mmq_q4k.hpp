@@ -43,13 +43,29 @@ typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
 constexpr uint32_t MMQ_MAGIC_BITS = 0x4B400000u;   // float 12582912 = 1.5 * 2^23
 constexpr float MMQ_MAGIC = 12582912.0f;
 
-template <int MT_, int NT_, int WM_, int WN_>
+// FMT selects the operand formats of the same engine:
+//   MMQ_Q4K_DS4   Q4_K weights x DS4 activations (fp16 scale and raw sum per 32 values, 144-byte blocks);
+//   MMQ_Q5K_D4S4  Q5_K weights x D4S4 activations (float32 scale and raw sum per 32 values, 160-byte blocks):
+//                 out = sum_j (d*sc_j)*xd_j*dot_j - (dmin*mn_j)*s4_j (gguf_k_mmq_prefill.hip:563-572,655-664).
+//                 The fifth bit of a value comes from the block's qh bytes (bit s of qh[l] for sub-block s,
+//                 value l), which travel to LDS beside the nibbles; the float32 raw sum enters the fp16 MFMA of
+//                 the min term as a high and a low fp16 part (two MFMAs, the product with mn <= 63 exact).
+enum MmqFormat : int { MMQ_Q4K_DS4 = 0, MMQ_Q5K_D4S4 = 1 };
+
+template <int MT_, int NT_, int WM_, int WN_, int FMT = MMQ_Q4K_DS4>
 struct Q4Tile {
   static constexpr int MT = MT_, NT = NT_, WM = WM_, WN = WN_;
+  static constexpr bool Q5 = FMT == MMQ_Q5K_D4S4;
   static constexpr int BM = 32 * MT * WM, BN = 32 * NT * WN, THREADS = 64 * WM * WN;
-  static constexpr int A_STRIDE = DS4_BYTES;   // 144 B = 9 x 16 B: conflict free for b128 reads
-  static constexpr int W_STRIDE = 80;          // 64 nibble bytes per K step, padded to 5 x 16 B
-  static constexpr int A_CHUNKS = BM * 9, W_CHUNKS = BN * 4, H_ITEMS = BN + BM;
+  static constexpr int A_BYTES = Q5 ? D4S4_BYTES : DS4_BYTES;   // activation block
+  static constexpr int A_PARTS = A_BYTES / 16;                  // 9 or 10 chunks of 16 bytes
+  static constexpr int A_QS = Q5 ? 32 : 16;                     // offset of the 128 int8 values in the block
+  static constexpr int A_STRIDE = Q5 ? 176 : DS4_BYTES;         // 9 or 11 x 16 B: conflict free for b128 reads
+  static constexpr int W_BLOCK = Q5 ? Q5_K_BYTES : Q4_K_BYTES;
+  static constexpr int W_QS = Q5 ? 48 : 16;                     // offset of the 128 nibble bytes in the block
+  static constexpr int W_PARTS = Q5 ? 6 : 4;                    // 16-byte chunks per column and K step: 4 of nibbles (+ 2 of qh)
+  static constexpr int W_STRIDE = Q5 ? 112 : 80;                // 64 nibble bytes (+ 32 qh bytes) per K step, padded to 5 / 7 x 16 B
+  static constexpr int A_CHUNKS = BM * A_PARTS, W_CHUNKS = BN * W_PARTS, H_ITEMS = BN + BM;
   static constexpr int A_PER = (A_CHUNKS + THREADS - 1) / THREADS;
   static constexpr int W_PER = (W_CHUNKS + THREADS - 1) / THREADS;
   static constexpr int H_PER = (H_ITEMS + THREADS - 1) / THREADS;
@@ -62,14 +78,16 @@ struct Q4Tile {
     float xd[4][BM];             // activation scale per sub-block of the step, by row
     float dmin[BN];
     _Float16 mnh[BN][8];         // 6-bit mins as fp16
-    _Float16 xsh[BM][8];         // activation sums of the Q4_K block (fp16 in the DS4 block already)
+    _Float16 xsh[BM][8];         // activation sums of the weight block (fp16 in the DS4 block already; D4S4: high part)
+    _Float16 xsl[Q5 ? BM : 1][8];   // D4S4: low part of the float32 sums
   };
 
   // Registers of one K step in flight between global memory and LDS.
   struct Regs {
     u32x4 pa[A_PER];
     u32x4 pw[W_PER];
-    u32x4 ph[H_PER];   // item < BN: Q4_K block header of that column; else DS4 header of row item-BN
+    u32x4 ph[H_PER];   // item < BN: weight block header of that column; else activation block header of row item-BN
+    u32x4 ph2[Q5 ? H_PER : 1];   // D4S4: the second half of a row's header (the four float32 sums)
   };
 
   // `row_of(r)` / `col_of(c)` give the activation row (in DS4 blocks of x_row_bytes
@@ -84,23 +102,27 @@ struct Q4Tile {
 #pragma unroll
     for (int i = 0; i < A_PER; ++i) {
       const int c = min(tid + i * THREADS, A_CHUNKS - 1);
-      const int row = c / 9, part = c - row * 9;
-      r.pa[i] = *reinterpret_cast<const u32x4*>(xq + row_of(row) * x_row_bytes + static_cast<int64_t>(step) * DS4_BYTES +
+      const int row = c / A_PARTS, part = c - row * A_PARTS;
+      r.pa[i] = *reinterpret_cast<const u32x4*>(xq + row_of(row) * x_row_bytes + static_cast<int64_t>(step) * A_BYTES +
                                                 part * 16);
     }
 #pragma unroll
     for (int i = 0; i < W_PER; ++i) {
       const int c = min(tid + i * THREADS, W_CHUNKS - 1);
-      const int col = c >> 2, part = c & 3;
-      r.pw[i] = *reinterpret_cast<const u32x4*>(w + col_of(col) * w_row_bytes + static_cast<int64_t>(kb) * Q4_K_BYTES + 16 +
-                                                h * 64 + part * 16);
+      const int col = c / W_PARTS, part = c - col * W_PARTS;
+      // parts 0..3: the step's 64 nibble bytes; Q5_K parts 4, 5: the block's 32 qh bytes (both steps read them)
+      const int off = part < 4 ? W_QS + h * 64 + part * 16 : 16 + (part - 4) * 16;
+      r.pw[i] = *reinterpret_cast<const u32x4*>(w + col_of(col) * w_row_bytes + static_cast<int64_t>(kb) * W_BLOCK + off);
     }
 #pragma unroll
     for (int i = 0; i < H_PER; ++i) {
       const int item = min(tid + i * THREADS, H_ITEMS - 1);
-      const uint8_t* hp = item < BN ? w + col_of(item) * w_row_bytes + static_cast<int64_t>(kb) * Q4_K_BYTES
-                                    : xq + row_of(item - BN) * x_row_bytes + static_cast<int64_t>(step) * DS4_BYTES;
+      const uint8_t* hp = item < BN ? w + col_of(item) * w_row_bytes + static_cast<int64_t>(kb) * W_BLOCK
+                                    : xq + row_of(item - BN) * x_row_bytes + static_cast<int64_t>(step) * A_BYTES;
       r.ph[i] = *reinterpret_cast<const u32x4*>(hp);
+      if constexpr (Q5) {
+        if (item >= BN) r.ph2[i] = *reinterpret_cast<const u32x4*>(hp + 16);
+      }
     }
   }
 
@@ -108,13 +130,20 @@ struct Q4Tile {
     const int h = step & 1;
 #pragma unroll
     for (int i = 0; i < A_PER; ++i) {
-      const int c = tid + i * THREADS;           // 144-byte rows are contiguous in LDS: offset c*16
-      if (c < A_CHUNKS) *reinterpret_cast<u32x4*>(s.xa + c * 16) = r.pa[i];
+      const int c = tid + i * THREADS;           // DS4: 144-byte rows are contiguous in LDS, offset c*16
+      if (c < A_CHUNKS) {
+        if constexpr (Q5) {
+          const int row = c / A_PARTS, part = c - row * A_PARTS;
+          *reinterpret_cast<u32x4*>(s.xa + row * A_STRIDE + part * 16) = r.pa[i];
+        } else {
+          *reinterpret_cast<u32x4*>(s.xa + c * 16) = r.pa[i];
+        }
+      }
     }
 #pragma unroll
     for (int i = 0; i < W_PER; ++i) {
       const int c = tid + i * THREADS;
-      if (c < W_CHUNKS) *reinterpret_cast<u32x4*>(s.wq + (c >> 2) * W_STRIDE + (c & 3) * 16) = r.pw[i];
+      if (c < W_CHUNKS) *reinterpret_cast<u32x4*>(s.wq + (c / W_PARTS) * W_STRIDE + (c % W_PARTS) * 16) = r.pw[i];
     }
 #pragma unroll
     for (int i = 0; i < H_PER; ++i) {
@@ -142,8 +171,16 @@ struct Q4Tile {
         const int row = item - BN;
 #pragma unroll
         for (int j = 0; j < 4; ++j) {
-          s.xd[j][row] = f16_bits_to_float(ph[j] & 0xFFFFu);
-          s.xsh[row][4 * h + j] = __builtin_bit_cast(_Float16, static_cast<uint16_t>(ph[j] >> 16));
+          if constexpr (Q5) {
+            s.xd[j][row] = bits_to_float(ph[j]);
+            const float sum = bits_to_float(r.ph2[i][j]);
+            const _Float16 hi = static_cast<_Float16>(sum);
+            s.xsh[row][4 * h + j] = hi;
+            s.xsl[row][4 * h + j] = static_cast<_Float16>(sum - static_cast<float>(hi));
+          } else {
+            s.xd[j][row] = f16_bits_to_float(ph[j] & 0xFFFFu);
+            s.xsh[row][4 * h + j] = __builtin_bit_cast(_Float16, static_cast<uint16_t>(ph[j] >> 16));
+          }
         }
       }
     }
@@ -169,6 +206,16 @@ struct Q4Tile {
                       static_cast<int>(q4k_low(qs.z)), static_cast<int>(q4k_low(qs.w))};
         whi[nt] = v4i{static_cast<int>(q4k_high(qs.x)), static_cast<int>(q4k_high(qs.y)),
                       static_cast<int>(q4k_high(qs.z)), static_cast<int>(q4k_high(qs.w))};
+        if constexpr (Q5) {
+          // values 16g..16g+15 of sub-blocks s0 = 4h + 2sp (low nibbles) and s0 + 1 (high): bit 4 is bit s of qh[l]
+          const u32x4 qh = *reinterpret_cast<const u32x4*>(s.wq + col * W_STRIDE + 64 + 16 * g);
+          const int s0 = 4 * h + 2 * sp;
+#pragma unroll
+          for (int e = 0; e < 4; ++e) {
+            wlo[nt][e] |= static_cast<int>(((qh[e] >> s0) & 0x01010101u) << 4);
+            whi[nt][e] |= static_cast<int>(((qh[e] >> (s0 + 1)) & 0x01010101u) << 4);
+          }
+        }
       }
       // The 2*MT*NT MFMAs of this nibble pair, software-pipelined: the MFMA of tile i+1 is issued
       // before the 32 scale FMAs of tile i, so the matrix pipe works while the VALU does.
@@ -178,7 +225,7 @@ struct Q4Tile {
       for (int half = 0; half < 2; ++half)
 #pragma unroll
         for (int mt = 0; mt < MT; ++mt)
-          xop[half][mt] = *reinterpret_cast<const v4i*>(s.xa + ((wm * MT + mt) * 32 + lc) * A_STRIDE + 16 +
+          xop[half][mt] = *reinterpret_cast<const v4i*>(s.xa + ((wm * MT + mt) * 32 + lc) * A_STRIDE + A_QS +
                                                         (2 * sp + half) * 32 + 16 * g);
       auto issue = [&](int i) {
         const int half = i / (MT * NT), mt = (i / NT) % MT, nt = i % NT;
@@ -243,7 +290,11 @@ struct Q4Tile {
           v16f z;
 #pragma unroll
           for (int v = 0; v < 16; ++v) z[v] = 0.0f;
-          const v16f t = __builtin_amdgcn_mfma_f32_32x32x8f16(xs, mn, z, 0, 0, 0);
+          v16f t = __builtin_amdgcn_mfma_f32_32x32x8f16(xs, mn, z, 0, 0, 0);
+          if constexpr (Q5) {
+            const v4h xl = *reinterpret_cast<const v4h*>(&s.xsl[arow][4 * g]);
+            t = __builtin_amdgcn_mfma_f32_32x32x8f16(xl, mn, t, 0, 0, 0);
+          }
           const float nd = -s.dmin[col];
 #pragma unroll
           for (int v = 0; v < 16; ++v) acc[nt][mt][v] = __builtin_fmaf(nd, t[v], acc[nt][mt][v]);

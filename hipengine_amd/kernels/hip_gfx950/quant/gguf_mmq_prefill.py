@@ -48,6 +48,10 @@ gguf_q4_k_q8_1_mmq32_ctl_dense_bf16_f32_out = _make(
 gguf_q4_k_q8_1_mmq32_ctl_dense_bf16_bf16_out = _make(
     "gguf_q4_k_q8_1_mmq32_ctl_dense_bf16_bf16_out", "hipengine_gguf_q4_k_q8_1_mmq32_ctl_dense_bf16_bf16_out", 32)
 
+gguf_q5_k_mmq32_q8_1_d4s4_f32_bf16_f32_out = _make(
+    "gguf_q5_k_mmq32_q8_1_d4s4_f32_bf16_f32_out", "hipengine_gguf_q5_k_mmq32_q8_1_d4s4_f32_bf16_f32_out", 32)
+gguf_q5_k_mmq32_q8_1_d4s4_f32_bf16_bf16_out = _make(
+    "gguf_q5_k_mmq32_q8_1_d4s4_f32_bf16_bf16_out", "hipengine_gguf_q5_k_mmq32_q8_1_d4s4_f32_bf16_bf16_out", 32)
 gguf_q6_k_mmq32_q8_1_d4s4_f32_bf16_f32_out = _make(
     "gguf_q6_k_mmq32_q8_1_d4s4_f32_bf16_f32_out", "hipengine_gguf_q6_k_mmq32_q8_1_d4s4_f32_bf16_f32_out", 1)
 gguf_q6_k_mmq32_q8_1_d4s4_f32_bf16_bf16_out = _make(
@@ -76,6 +80,10 @@ _Q4 = (
 def register_kernels(backend: str = "hip_gfx950", *, replace: bool = False) -> None:
     for variant, fn in _Q4:
         register(KernelKey(backend, "linear", "gguf_q4_k", variant), fn, replace=replace)
+    register(KernelKey(backend, "linear", "gguf_q5_k", "mmq32_q8_1_d4s4_f32_bf16_f32_out"),
+             gguf_q5_k_mmq32_q8_1_d4s4_f32_bf16_f32_out, replace=replace)
+    register(KernelKey(backend, "linear", "gguf_q5_k", "mmq32_q8_1_d4s4_f32_bf16_bf16_out"),
+             gguf_q5_k_mmq32_q8_1_d4s4_f32_bf16_bf16_out, replace=replace)
     register(KernelKey(backend, "linear", "gguf_q6_k", "mmq32_q8_1_d4s4_f32_bf16_f32_out"),
              gguf_q6_k_mmq32_q8_1_d4s4_f32_bf16_f32_out, replace=replace)
     register(KernelKey(backend, "linear", "gguf_q6_k", "mmq32_q8_1_d4s4_f32_bf16_bf16_out"),

@@ -227,6 +227,17 @@ int hipengine_gguf_q4_k_q8_1_mmq32_ctl_dense_bf16_bf16_out(const void* xq, const
                                                            int64_t rows, int64_t in_features, int64_t out_features,
                                                            hipengine_stream_t stream);
 
+/* Raw Q5_K weights x D4S4 activations ([rows, in_features/128] 160-byte blocks, float32 scale and raw sum per
+ * 32 values): sum_j (d*sc_j)*xd_j*dot_j - (dmin*mn_j)*s4_j per 32-wide sub-block, dot of the 5-bit values.
+ * Replaces gguf_k_mmq_prefill.hip:2557-2589 with NAME = gguf_q5_k (kernel :517-685, qtype 5); the pipe and mb4
+ * names of the same export block are scheduling variants of this kernel there and are not exported here. */
+int hipengine_gguf_q5_k_mmq32_q8_1_d4s4_f32_bf16_f32_out(const void* xq, const uint8_t* qweight, void* out,
+                                                         int64_t rows, int64_t in_features, int64_t out_features,
+                                                         hipengine_stream_t stream);
+int hipengine_gguf_q5_k_mmq32_q8_1_d4s4_f32_bf16_bf16_out(const void* xq, const uint8_t* qweight, void* out,
+                                                          int64_t rows, int64_t in_features, int64_t out_features,
+                                                          hipengine_stream_t stream);
+
 /* Raw Q6_K weights x D4S4 activations ([rows, in_features/128] 160-byte blocks
  * {float d4[4]; float s4[4]; int8 qs[128]}): sum over 32-value groups of
  * xd_g * (s0*dot0 + s1*dot1), s = d*scale_i8 per 16 values, dots of the centred
@@ -241,9 +252,9 @@ int hipengine_gguf_q6_k_mmq32_q8_1_d4s4_f32_bf16_bf16_out(const void* xq, const 
                                                           hipengine_stream_t stream);
 
 /* Prefill from bf16 activations in one call: x [rows, in_features] bf16 is packed into `workspace`
- * (DS4 blocks for Q4_K, D4S4 for Q6_K; caller-owned, 16-byte aligned, at least the byte count
+ * (DS4 blocks for Q4_K, D4S4 for Q5_K and Q6_K; caller-owned, 16-byte aligned, at least the byte count
  * hipengine_gfx950_gguf_prefill_workspace_bytes reports = rows * in_features/128 * 144 or 160) and the MMQ
- * above runs on it: two launches.  ggml_type 12 (Q4_K, out_features % 32 == 0) or 14 (Q6_K); out_kind 0
+ * above runs on it: two launches.  ggml_type 12 (Q4_K), 13 (Q5_K; both out_features % 32 == 0) or 14 (Q6_K); out_kind 0
  * float32, 1 bf16, 2 fp16.  This is what a ("linear", quant, "prefill_bf16_*_out") caller with 32 or more
  * rows should reach: hipEngine's prefill signature has no workspace argument, so the Python wrappers of the
  * prefill keys take it as an optional keyword and fall back to batches of 8 rows through the GEMV without
@@ -545,7 +556,8 @@ int hipengine_gfx950_gguf_gemv_mfma_dots_i32(int32_t ggml_type, int32_t form, co
                                              int32_t* dots, float* out, int64_t rows, int64_t in_features,
                                              int64_t out_features, hipengine_stream_t stream);
 
-/* The same for the MMQ prefill GEMM: ggml_type 12 (Q4_K, xq = DS4 blocks, dots int32 [rows, N, K/32]) or 14
+/* The same for the MMQ prefill GEMM: ggml_type 12 (Q4_K, xq = DS4 blocks, dots int32 [rows, N, K/32]), 13 (Q5_K,
+ * xq = D4S4 blocks, dots [rows, N, K/32]) or 14
  * (Q6_K, xq = D4S4 blocks, dots [rows, N, K/16], of the centred 6-bit values); out: float32 [rows, N]. */
 int hipengine_gfx950_gguf_mmq_dots_i32(int32_t ggml_type, const void* xq, const uint8_t* qweight, int32_t* dots,
                                        float* out, int64_t rows, int64_t in_features, int64_t out_features,

@@ -561,10 +561,10 @@ def block_dots_q8_0(qs_i8: np.ndarray, qweight: np.ndarray) -> np.ndarray:
     return np.einsum("rjk,njk->rnj", qs_i8.astype(np.int32), w, optimize=True).astype(np.int32)
 
 
-def _q4_k_scales_f32(qweight: np.ndarray) -> tuple[np.ndarray, np.ndarray]:
-    """(d*sc, dmin*mn) per (row, sub-block) as float32 ``[N, K/32]``."""
+def _q4_k_scales_f32(qweight: np.ndarray, block_bytes: int = Q4_K_BLOCK_BYTES) -> tuple[np.ndarray, np.ndarray]:
+    """(d*sc, dmin*mn) per (row, sub-block) as float32 ``[N, K/32]``; Q5_K blocks carry the same 16-byte header."""
     n = qweight.shape[0]
-    blocks, _ = _as_blocks(qweight, Q4_K_BLOCK_BYTES)
+    blocks, _ = _as_blocks(qweight, block_bytes)
     sc, mn = q4_k_scale_min(blocks[:, 4:16])
     ds = (_fp16_field(blocks, 0)[:, None] * sc.astype(np.float32)).astype(np.float32)
     dm = (_fp16_field(blocks, 2)[:, None] * mn.astype(np.float32)).astype(np.float32)
@@ -617,6 +617,17 @@ def mmq_q4_k_ds4(xds4, qweight, dtype=np.float64) -> np.ndarray:
     main = (ds[None].astype(dtype) * xd[:, None, :].astype(dtype) * dots.astype(dtype)).sum(axis=-1)
     corr = xs.astype(dtype) @ dm.astype(dtype).T
     return main - corr
+
+
+def mmq_q5_k_d4s4(xd4s4, qweight, dtype=np.float64) -> np.ndarray:
+    """D4S4 x Q5_K MMQ: ``sum_j xd_j*(d*sc_j)*dot_j - (dmin*mn_j)*s4_j`` with the float32 raw sum of the
+    32 activation values (gguf_k_mmq_prefill.hip:563-572 scales, :655-664 combine)."""
+    xd, xs, qs = d4s4_fields(xd4s4)
+    qw = np.asarray(qweight)
+    dots, _ = block_dots_q5_k(qs, qw)
+    ds, dm = _q4_k_scales_f32(qw, Q5_K_BLOCK_BYTES)
+    main = (ds[None].astype(dtype) * xd[:, None, :].astype(dtype) * dots.astype(dtype)).sum(axis=-1)
+    return main - xs.astype(dtype) @ dm.astype(dtype).T
 
 
 def mmq_q6_k_d4s4(xd4s4, qweight, dtype=np.float64) -> np.ndarray:

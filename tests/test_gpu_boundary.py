@@ -85,7 +85,7 @@ def test_dispatcher_keys_called_like_launch_raw(dev, quant, act, out):
     dev.free(dw)
 
 
-@pytest.mark.parametrize("quant,n", [("gguf_q4_k", 352), ("gguf_q6_k", 333)])
+@pytest.mark.parametrize("quant,n", [("gguf_q4_k", 352), ("gguf_q6_k", 333), ("gguf_q5_k", 160)])
 def test_prefill_key_with_workspace_runs_the_mmq(dev, quant, n):
     """prefill_bf16_f32_out with 32 rows or more and a caller-owned workspace packs the activations and runs the
     int8-MFMA MMQ: results equal the MMQ formula of the oracle, and agree with the workspace-free route (GEMV in
@@ -93,7 +93,8 @@ def test_prefill_key_with_workspace_runs_the_mmq(dev, quant, n):
     rows, k = 70, 1024
     rng = np.random.default_rng(3)
     xb = O.f32_to_bf16_bits((rng.standard_normal((rows, k)) * 0.25).astype(np.float32))
-    w = O.random_weight(QT[quant], n, k, seed=5)
+    w = (synthetic_blocks(QT[quant], n, k, seed=5, tile_rows=n) if quant == "gguf_q5_k"
+         else O.random_weight(QT[quant], n, k, seed=5))
     fn = _resolve("linear", quant, "prefill_bf16_f32_out")
     need = G.gguf_prefill_workspace_bytes(quant, rows, k)
     assert need == rows * (k // 128) * (144 if quant == "gguf_q4_k" else 160)
@@ -107,6 +108,9 @@ def test_prefill_key_with_workspace_runs_the_mmq(dev, quant, n):
     if quant == "gguf_q4_k":
         want_pack = O.pack_q8_1_ds4(xb)
         ref = O.mmq_q4_k_ds4(want_pack, w)
+    elif quant == "gguf_q5_k":
+        want_pack = O.pack_q8_1_d4s4(xb)
+        ref = O.mmq_q5_k_d4s4(want_pack, w)
     else:
         want_pack = O.pack_q8_1_d4s4(xb)
         ref = O.mmq_q6_k_d4s4(want_pack, w)
@@ -380,18 +384,25 @@ def test_gemv_mfma_forms_int32_dots_bit_exact(dev, quant, form, k, n, rows):
     _close(out, O.gguf_quant_gemv(O.dequantize_q8_1(xq), w, qt))
 
 
-@pytest.mark.parametrize("quant,rows,k,n", [("gguf_q4_k", 150, 1024, 160), ("gguf_q6_k", 129, 768, 130)])
+@pytest.mark.parametrize("quant,rows,k,n", [("gguf_q4_k", 150, 1024, 160), ("gguf_q6_k", 129, 768, 130),
+                                            ("gguf_q5_k", 131, 1280, 96)])
 def test_mmq_int32_dots_bit_exact(dev, quant, rows, k, n):
     """The int32 tiles of the MMQ prefill GEMM (v_mfma_i32_32x32x32_i8 / 32x32x16) against the oracle's integer
     dots of the same packed activations; ragged tiles in both dimensions."""
     rng = np.random.default_rng(rows + k)
     xb = O.f32_to_bf16_bits((rng.standard_normal((rows, k)) * 0.3).astype(np.float32))
-    w = O.random_weight(QT[quant], n, k, seed=9)
+    w = (synthetic_blocks(QT[quant], n, k, seed=9, tile_rows=n) if quant == "gguf_q5_k"
+         else O.random_weight(QT[quant], n, k, seed=9))
     if quant == "gguf_q4_k":
         xq = O.pack_q8_1_ds4(xb)
         qs = O.ds4_fields(xq)[2].reshape(rows, k // 32, 32)
         want, per = O.block_dots_q4_k(qs, w)[0], k // 32
         ref = O.mmq_q4_k_ds4(xq, w)
+    elif quant == "gguf_q5_k":
+        xq = O.pack_q8_1_d4s4(xb)
+        qs = O.d4s4_fields(xq)[2].reshape(rows, k // 32, 32)
+        want, per = O.block_dots_q5_k(qs, w)[0], k // 32
+        ref = O.mmq_q5_k_d4s4(xq, w)
     else:
         xq = O.pack_q8_1_d4s4(xb)
         qs = O.d4s4_fields(xq)[2].reshape(rows, k // 32, 32)

@@ -141,6 +141,49 @@ def test_q6_k_mmq_closed_form_bf16_and_determinism(dev):
     assert np.array_equal(b16, O.f32_to_bf16_bits(f32))
 
 
+def _random_q5_k(n, k, seed):
+    """Random valid Q5_K blocks (the oracle has no fp32 -> Q5_K quantizer): every field drawn uniformly."""
+    rng = np.random.default_rng(seed)
+    nblk = n * (k // 256)
+    blk = O.pack_q5_k_blocks(rng.integers(0, 32, size=(nblk, 8, 32), dtype=np.uint8),
+                             rng.integers(0, 64, size=(nblk, 8), dtype=np.uint8),
+                             rng.integers(0, 64, size=(nblk, 8), dtype=np.uint8),
+                             (rng.random(nblk) * 0.05).astype(np.float32), (rng.random(nblk) * 0.02).astype(np.float32))
+    return blk.reshape(n, -1)
+
+
+@pytest.mark.parametrize("rows,k,n", [(1, 256, 32), (7, 512, 64), (128, 1024, 128), (130, 768, 160), (300, 5120, 224)])
+def test_q5_k_mmq_matches_formula_and_cpu_reference(dev, rows, k, n):
+    """Q5_K x D4S4 (gguf_k_mmq_prefill.hip:655-664) on the tile engine of the Q4_K GEMM: the formula in float64,
+    and the reference CPU GEMV on the dequantized activations (which differs in the min term only: xd * sum(q8)
+    against the raw float32 sum, so the gate there is the looser one hipEngine's own q8_1 tests use)."""
+    xb = _bf16_rows(3 * rows + k + n, rows, k, scale=0.1, offset=0.002)
+    d4 = O.pack_q8_1_d4s4(xb)
+    w = _random_q5_k(n, k, seed=k + n + 2)
+    got = _run_q4(dev, M.gguf_q5_k_mmq32_q8_1_d4s4_f32_bf16_f32_out, d4, w, rows, k, n)
+    want = O.mmq_q5_k_d4s4(d4, w)
+    assert O.max_rel_err(got, want) <= 1e-3 and O.cosine(got, want) >= 0.99999
+    xd, _, qs = O.d4s4_fields(d4)
+    xdeq = (xd[..., None] * qs.astype(np.float32)).reshape(rows, k)
+    ref = O.gguf_quant_gemv(xdeq, w, O.GGML_Q5_K)
+    assert O.cosine(got, ref) >= 0.9995
+    np.testing.assert_allclose(got, ref, rtol=2e-2, atol=1e-2 * (np.abs(ref).max() + 1))
+
+
+def test_q5_k_mmq_bf16_and_determinism(dev):
+    rows, k, n = 70, 512, 96
+    xb = _bf16_rows(17, rows, k, scale=0.125)
+    d4 = O.pack_q8_1_d4s4(xb)
+    w = O.closed_form_q5_k(n, k)
+    f32 = _run_q4(dev, M.gguf_q5_k_mmq32_q8_1_d4s4_f32_bf16_f32_out, d4, w, rows, k, n)
+    again = _run_q4(dev, M.gguf_q5_k_mmq32_q8_1_d4s4_f32_bf16_f32_out, d4, w, rows, k, n)
+    want = O.mmq_q5_k_d4s4(d4, w)
+    assert O.max_rel_err(f32, want) <= 1e-3 and O.cosine(f32, want) >= 0.99999
+    assert np.array_equal(f32.view(np.uint32), again.view(np.uint32))
+    b16 = _run_q4(dev, M.gguf_q5_k_mmq32_q8_1_d4s4_f32_bf16_bf16_out, d4, w, rows, k, n, out_dtype=np.uint16)
+    assert np.array_equal(b16, O.f32_to_bf16_bits(f32))
+
+
 def test_mmq_wrapper_rejects_bad_shapes(dev):
     f = M.gguf_q4_k_q8_1_mmq32_vdr_dense_bf16_f32_out
     with pytest.raises(ValueError, match="divisible"):

@@ -351,6 +351,22 @@ def test_mmq_formulas_against_float64():
     want = (d[..., None].astype(np.float64) * q).reshape(rows, k) @ O.dequantize(w6, O.GGML_Q6_K).astype(np.float64).T
     np.testing.assert_allclose(O.mmq_q6_k_d4s4(d4, w6), want, rtol=1e-9, atol=1e-9 * np.abs(want).max())
     assert O.max_rel_err(C.mmq_q6_k_d4s4(d4, w6), want) < 2e-4
+    # Q5_K x D4S4: the Q4_K structure with 5-bit values and the float32 raw sum; an independent float64 evaluation
+    # from the unpacked fields, and the dequantize-matmul identity it must stay close to (they differ in the min
+    # term only: raw sum of the activations against xd * sum(q8))
+    from hipengine_amd.synthetic import synthetic_blocks
+    w5 = synthetic_blocks(O.GGML_Q5_K, n, k, seed=6, tile_rows=n)
+    b5 = w5.reshape(-1, 176)
+    sc5, mn5 = O.q4_k_scale_min(b5[:, 4:16])
+    dsc5 = (b5[:, 0:2].copy().view(np.float16).astype(np.float64) * sc5).reshape(n, -1)
+    dm5 = (b5[:, 2:4].copy().view(np.float16).astype(np.float64) * mn5).reshape(n, -1)
+    q5 = O.q5_k_quants(b5).reshape(n, -1, 32).astype(np.float64)
+    d, s4, q = O.d4s4_fields(d4)
+    want = np.einsum("rj,nj,rjk,njk->rn", d.astype(np.float64), dsc5, q.astype(np.float64), q5) - s4.astype(np.float64) @ dm5.T
+    got5 = O.mmq_q5_k_d4s4(d4, w5)
+    np.testing.assert_allclose(got5, want, rtol=1e-9, atol=1e-9 * np.abs(want).max())
+    deq = (d[..., None].astype(np.float64) * q).reshape(rows, k) @ O.dequantize(w5, O.GGML_Q5_K).astype(np.float64).T
+    assert O.cosine(got5, deq) > 0.9999
 
 
 # ---------------------------------------------------------------- fp16 / bf16 helpers of the C restatement
