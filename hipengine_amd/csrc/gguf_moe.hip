@@ -738,7 +738,7 @@ int launch_grouped_gemv(int qt, const void* x, int x_kind, const int64_t* expert
   if (!x || !expert_start || !w || !out || compact_rows <= 0 || compact_rows > 0x7FFFFFFF || num_experts <= 0 ||
       num_experts > 65535 || K <= 0 || (K % QK_K) != 0 || K > (1 << 20) || N <= 0 || N > (1 << 24) ||
       x_kind < KIND_F32 || x_kind > KIND_Q8_1 || out_kind < KIND_F32 || out_kind > KIND_F16 ||
-      (qt != GGML_Q4_K && qt != GGML_Q6_K)) {
+      (qt != GGML_Q4_K && qt != GGML_Q5_K && qt != GGML_Q6_K && qt != GGML_Q8_0)) {
     return static_cast<int>(hipErrorInvalidValue);
   }
   const int nb = static_cast<int>(K / QK_K);
@@ -762,7 +762,10 @@ int launch_grouped_gemv(int qt, const void* x, int x_kind, const int64_t* expert
     else if (cb == 2) hipLaunchKernelGGL((grouped_gemv_kernel<QT, 2>), grid, block, lds, stream, s); \
     else hipLaunchKernelGGL((grouped_gemv_kernel<QT, 5>), grid, block, lds, stream, s);              \
   } while (0)
-  if (qt == GGML_Q4_K) LAUNCH_GROUPED(GGML_Q4_K); else LAUNCH_GROUPED(GGML_Q6_K);
+  if (qt == GGML_Q4_K) LAUNCH_GROUPED(GGML_Q4_K);
+  else if (qt == GGML_Q5_K) LAUNCH_GROUPED(GGML_Q5_K);
+  else if (qt == GGML_Q6_K) LAUNCH_GROUPED(GGML_Q6_K);
+  else LAUNCH_GROUPED(GGML_Q8_0);
 #undef LAUNCH_GROUPED
   return static_cast<int>(hipGetLastError());
 }
@@ -1108,6 +1111,15 @@ extern "C" int hipengine_gguf_q4_k_selected_grouped_prefill_compact_rowbatch8_bf
     int64_t in_features, int64_t out_features, hipStream_t stream) {
   return launch_grouped_gemv(GGML_Q4_K, x, KIND_BF16, static_cast<const int64_t*>(expert_start),
                              static_cast<const uint8_t*>(qweight), out, KIND_BF16, compact_rows, num_experts,
+                             in_features, out_features, stream);
+}
+
+// The same for expert weights of any of the four block types and any activation / output kind.
+extern "C" int hipengine_gfx950_gguf_grouped_gemv(int32_t ggml_type, const void* x, int32_t x_kind,
+                                                  const int64_t* expert_start, const uint8_t* qweight, void* out,
+                                                  int32_t out_kind, int64_t compact_rows, int64_t num_experts,
+                                                  int64_t in_features, int64_t out_features, hipStream_t stream) {
+  return launch_grouped_gemv(ggml_type, x, x_kind, expert_start, qweight, out, out_kind, compact_rows, num_experts,
                              in_features, out_features, stream);
 }
 

@@ -147,6 +147,28 @@ def gguf_q4_k_selected_grouped_prefill_compact_rowbatch8_bf16_bf16_out(
                     stream), runtime)
 
 
+def gguf_grouped_gemv(quant: str, x_ptr: int, expert_start_ptr: int, qweight_ptr: int, out_ptr: int,
+                      compact_rows: int, num_experts: int, in_features: int, out_features: int, *,
+                      x_dtype: str = "bf16", out_dtype: str = "bf16", stream: int = 0,
+                      library: ctypes.CDLL | None = None, runtime: HipRuntime | None = None) -> None:
+    """The grouped GEMV for expert weights of any of the four block types (``hipengine_gfx950_gguf_grouped_gemv``)."""
+    if quant not in QUANT_KEY_TO_GGML:
+        raise ValueError("quant must be one of " + ", ".join(sorted(QUANT_KEY_TO_GGML)))
+    if compact_rows <= 0:
+        raise ValueError("compact_rows must be positive")
+    if num_experts <= 0 or num_experts > 65535:
+        raise ValueError("num_experts must be in 1..65535")
+    if in_features <= 0 or in_features % 256 != 0:
+        raise ValueError("in_features must be positive and divisible by the GGUF block size 256")
+    if out_features <= 0:
+        raise ValueError("out_features must be positive")
+    validate_pointers(x_ptr=x_ptr, expert_start_ptr=expert_start_ptr, qweight_ptr=qweight_ptr, out_ptr=out_ptr)
+    fn = entry("hipengine_gfx950_gguf_grouped_gemv", [I32, VOID, I32, VOID, VOID, VOID, I32, I64, I64, I64, I64, VOID],
+               library)
+    check_launch(fn(QUANT_KEY_TO_GGML[quant], x_ptr, _KIND[x_dtype], expert_start_ptr, qweight_ptr, out_ptr,
+                    _KIND[out_dtype], compact_rows, num_experts, in_features, out_features, stream), runtime)
+
+
 def gguf_selected_gemv(quant: str, mode: int, x_ptr: int, selected_ptr: int, qweight_a_ptr: int, out_ptr: int,
                        x_rows: int, lanes: int, num_experts: int, in_features: int, out_features: int, *,
                        x_dtype: str = "f32", out_dtype: str = "f32", routing_weights_ptr: int = 0,
@@ -288,6 +310,9 @@ def register_kernels(backend: str = "hip_gfx950", *, replace: bool = False) -> N
     register(KernelKey(backend, "moe_linear", "gguf_q4_k",
                        "selected_dual_q8_1_ds4_mmq32_prefill_compact32_bf16_bf16_out"),
              gguf_q4_k_selected_dual_q8_1_ds4_mmq32_prefill_compact32_bf16_bf16_out, replace=replace)
+    for _q in ("gguf_q4_k", "gguf_q5_k", "gguf_q6_k", "gguf_q8_0"):
+        register(KernelKey(backend, "moe_linear", _q, "grouped_gemv_rowbatch8"),
+                 (lambda q: lambda *a, **k: gguf_grouped_gemv(q, *a, **k))(_q), replace=replace)
     register(KernelKey(backend, "moe_linear", "gguf_q4_k", "grouped_mmq32_q8_1_ds4"), gguf_q4_k_grouped_mmq,
              replace=replace)
     for quant in ("gguf_q4_k", "gguf_q6_k"):

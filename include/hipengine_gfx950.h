@@ -486,6 +486,18 @@ int hipengine_gguf_q4_k_selected_grouped_prefill_compact_rowbatch8_bf16_bf16_out
     const void* x, const void* expert_start, const void* qweight, void* out, int64_t compact_rows,
     int64_t num_experts, int64_t in_features, int64_t out_features, hipengine_stream_t stream);
 
+/* Grouped GEMV over gathered compact rows for expert weights of any of the four block types: rows
+ * [expert_start[e], expert_start[e+1]) of x [compact_rows, in_features] (x_kind 0 f32, 1 bf16, 2 fp16, 3 q8_1
+ * blocks) take expert e of qweight [num_experts, out_features, row_bytes]; out [compact_rows, out_features] of
+ * out_kind.  An expert's weights are read once per 8 of its rows.  The form of
+ * hipengine_gguf_q4_k_selected_grouped_prefill_compact_rowbatch8_bf16_bf16_out for Q5_K, Q6_K and Q8_0 experts
+ * (the 35B-A3B shared expert is Q8_0) in the raw layout; hipEngine's grouped kernels for those types take its
+ * RDNA3 layouts (t16 / pack8).  New here. */
+int hipengine_gfx950_gguf_grouped_gemv(int32_t ggml_type, const void* x, int32_t x_kind, const int64_t* expert_start,
+                                       const uint8_t* qweight, void* out, int32_t out_kind, int64_t compact_rows,
+                                       int64_t num_experts, int64_t in_features, int64_t out_features,
+                                       hipengine_stream_t stream);
+
 /* The decode kernels with every choice explicit.  ggml_type 12 (Q4_K) or 14 (Q6_K).
  *   mode 0: out[lanes, N] = W_a[selected[lane]] . x[lane / (lanes/x_rows)]
  *   mode 1: out[lanes, N] = silu(gate) * up with W_a = gate, W_b = up; round_mid != 0

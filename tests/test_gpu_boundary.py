@@ -280,6 +280,33 @@ def test_grouped_gemv_over_compact_rows(dev, tokens):
         assert O.max_rel_err(O.bf16_bits_to_f32(got[r:r + 1]), ref, floor_frac=1e-2) <= 8e-3, r
 
 
+@pytest.mark.parametrize("quant", ["gguf_q5_k", "gguf_q6_k", "gguf_q8_0"])
+def test_grouped_gemv_other_expert_types(dev, quant):
+    """The grouped GEMV for Q5_K, Q6_K and Q8_0 expert weights in the raw layout (float32 in and out): experts
+    with 1, 2, several and more than 8 rows, and experts with none."""
+    experts, hidden, inter = 6, 1024, 96
+    counts = np.array([1, 0, 2, 11, 0, 5])
+    start = np.concatenate([[0], np.cumsum(counts)]).astype(np.int64)
+    total = int(start[-1])
+    rng = np.random.default_rng(77)
+    x = (rng.standard_normal((total, hidden)) * 0.5).astype(np.float32)
+    w = np.stack([synthetic_blocks(QT[quant], inter, hidden, seed=20 + e, tile_rows=inter) if quant == "gguf_q5_k"
+                  else O.random_weight(QT[quant], inter, hidden, seed=20 + e) for e in range(experts)])
+    fn = _resolve("moe_linear", quant, "grouped_gemv_rowbatch8")
+    dx, des, dw = dev.put(x), dev.put(start), dev.put(w)
+    dout = dev.empty((total + 1) * inter * 4, fill=0xEE)
+    fn(dx.ptr, des.ptr, dw.ptr, dout.ptr, total, experts, hidden, inter, x_dtype="f32", out_dtype="f32", stream=0,
+       runtime=dev.runtime)
+    got = dev.get(dout, np.float32, (total + 1, inter))
+    dev.free(dx, des, dw, dout)
+    assert np.all(got[total].view(np.uint32) == 0xEEEEEEEE)
+    x_deq = O.dequantize_q8_1(O.quantize_q8_1(x))
+    for e in range(experts):
+        lo, hi = int(start[e]), int(start[e + 1])
+        if hi > lo:
+            _close(got[lo:hi], O.gguf_quant_gemv(x_deq[lo:hi], w[e], QT[quant]))
+
+
 # ---- the runner's step-by-step routing index ----------------------------------------------------
 
 @pytest.mark.parametrize("tokens,top_k,experts,pad", [(1, 8, 256, 1), (8, 8, 256, 1), (333, 4, 60, 1), (2048, 8, 256, 1),
