@@ -328,8 +328,8 @@ class Harness:
             for name, nbytes in (("es", (experts + 1) * 8), ("act", experts * 8), ("actn", 8), ("sl", lanes * 8),
                                  ("c2s", lanes * 8), ("sw", lanes * 4), ("ms", (experts + 1) * 8), ("te", cap * 8),
                                  ("mt", 8), ("l2c", lanes * 8), ("xq", tokens * (hidden // 128) * 144),
-                                 ("gu", lanes * 2 * inter * 4),
-                                 ("mq", lanes * (inter // 128) * 144), ("down", lanes * hidden * 4)):
+                                 ("gu", lanes * 2 * inter * 2),
+                                 ("mq", lanes * (inter // 128) * 144), ("down", lanes * hidden * 2)):
                 b[name] = mem.malloc(nbytes, runtime=rt)
             mmq_rows = cap * 32     # upper bound known on the host; unused tiles are marked -1
 
@@ -341,15 +341,16 @@ class Harness:
                                              tile_capacity=cap)
                 GS.moe_lane_to_compact(b["sl"].ptr, b["l2c"].ptr, lanes, lanes)
                 Q.gguf_q8_1_mmq_ds4_pack_bf16(b["x"].ptr, b["xq"].ptr, tokens, hidden)
+                # intermediates in bf16, hipEngine's own types for this chain (the named gate|up entry stores bf16)
                 M.gguf_q4_k_grouped_mmq(b["xq"].ptr, b["es"].ptr, b["ms"].ptr, b["te"].ptr, b["wg"].ptr, b["gu"].ptr,
                                         lanes, tokens, hidden, inter, experts, mmq_rows,
                                         compact_to_source_ptr=b["c2s"].ptr, qweight_b_ptr=b["wu"].ptr,
-                                        out_features_b=inter)
-                M.moe_silu_mul_ds4_pack(b["gu"].ptr, b["mq"].ptr, lanes, inter, in_dtype="f32")
+                                        out_features_b=inter, out_dtype="bf16")
+                M.moe_silu_mul_ds4_pack(b["gu"].ptr, b["mq"].ptr, lanes, inter, in_dtype="bf16")
                 M.gguf_q4_k_grouped_mmq(b["mq"].ptr, b["es"].ptr, b["ms"].ptr, b["te"].ptr, b["wd"].ptr, b["down"].ptr,
-                                        lanes, lanes, inter, hidden, experts, mmq_rows)
+                                        lanes, lanes, inter, hidden, experts, mmq_rows, out_dtype="bf16")
                 M.moe_weighted_gather_sum(b["down"].ptr, b["l2c"].ptr, b["wts"].ptr, b["out"].ptr, tokens, top_k, hidden,
-                                          lanes)
+                                          lanes, in_dtype="bf16")
         _, ev = self.time_launches(chain, steps, warmup)
         for buf in bufs.values():
             mem.free(buf)

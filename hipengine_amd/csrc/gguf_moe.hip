@@ -421,6 +421,66 @@ __global__ void moe_weighted_gather_kernel(const void* __restrict__ down, const 
   store_scalar(out, t * hidden + h, acc, out_kind);
 }
 
+// The same sums for hidden % 8 == 0 and top_k <= 8, eight consecutive features per thread: a token's slot
+// indices and weights are fetched first, then all of its rows' 16- or 32-byte pieces are in flight together
+// (the scalar form above is a chain of top_k dependent 2- or 4-byte loads per thread).
+template <int IN_KIND>
+__global__ void __launch_bounds__(256) moe_weighted_gather8_kernel(const void* __restrict__ down,
+                                                                   const int64_t* __restrict__ lane_to_compact,
+                                                                   const float* __restrict__ routing,
+                                                                   void* __restrict__ out, int64_t tokens, int top_k,
+                                                                   int64_t hidden, int64_t compact_rows, int out_kind) {
+  const int64_t t = blockIdx.y;
+  const int64_t h = (static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x) * 8;
+  if (t >= tokens || h >= hidden) return;
+  int64_t c[8];
+  float wgt[8];
+#pragma unroll
+  for (int s = 0; s < 8; ++s) {
+    const bool on = s < top_k;
+    c[s] = on ? lane_to_compact[t * top_k + s] : -1;
+    wgt[s] = on ? routing[t * top_k + s] : 0.0f;
+  }
+  float v[8][8];
+#pragma unroll
+  for (int s = 0; s < 8; ++s) {
+    const bool live = c[s] >= 0 && c[s] < compact_rows;
+    const int64_t base = (live ? c[s] : 0) * hidden + h;
+    if constexpr (IN_KIND == KIND_F32) {
+      const float4 lo = *reinterpret_cast<const float4*>(static_cast<const float*>(down) + base);
+      const float4 hi = *reinterpret_cast<const float4*>(static_cast<const float*>(down) + base + 4);
+      v[s][0] = lo.x; v[s][1] = lo.y; v[s][2] = lo.z; v[s][3] = lo.w;
+      v[s][4] = hi.x; v[s][5] = hi.y; v[s][6] = hi.z; v[s][7] = hi.w;
+    } else {
+      const uint4 p = *reinterpret_cast<const uint4*>(static_cast<const uint16_t*>(down) + base);
+      const uint32_t w32[4] = {p.x, p.y, p.z, p.w};
+#pragma unroll
+      for (int e = 0; e < 4; ++e) {
+        v[s][2 * e] = IN_KIND == KIND_BF16 ? bf16_bits_to_float(w32[e] & 0xFFFFu) : f16_bits_to_float(w32[e] & 0xFFFFu);
+        v[s][2 * e + 1] = IN_KIND == KIND_BF16 ? bf16_bits_to_float(w32[e] >> 16) : f16_bits_to_float(w32[e] >> 16);
+      }
+    }
+  }
+  float res[8];
+#pragma unroll
+  for (int e = 0; e < 8; ++e) {
+    float acc = 0.0f;
+#pragma unroll
+    for (int s = 0; s < 8; ++s) {
+      if (s < top_k && c[s] >= 0 && c[s] < compact_rows) acc += wgt[s] * v[s][e];
+    }
+    res[e] = acc;
+  }
+  if (out_kind == KIND_F32) {
+    float* o = static_cast<float*>(out) + t * hidden + h;
+    *reinterpret_cast<float4*>(o) = float4{res[0], res[1], res[2], res[3]};
+    *reinterpret_cast<float4*>(o + 4) = float4{res[4], res[5], res[6], res[7]};
+  } else {
+#pragma unroll
+    for (int e = 0; e < 8; ++e) store_scalar(out, t * hidden + h + e, res[e], out_kind);
+  }
+}
+
 // --------------------------------------------------------------------------
 // decode: selected GEMV on the q8_1 integer GEMV body
 // --------------------------------------------------------------------------
@@ -1039,6 +1099,21 @@ extern "C" int hipengine_gfx950_moe_weighted_gather_sum(const void* down, const 
       hidden <= 0 || compact_rows <= 0 || in_kind < KIND_F32 || in_kind > KIND_F16 || out_kind < KIND_F32 ||
       out_kind > KIND_F16) {
     return static_cast<int>(hipErrorInvalidValue);
+  }
+  if ((hidden % 8) == 0 && top_k <= 8 && ((reinterpret_cast<uintptr_t>(down) | reinterpret_cast<uintptr_t>(out)) & 15u) == 0) {
+    const dim3 grid(static_cast<unsigned>((hidden / 8 + 255) / 256), static_cast<unsigned>(tokens));
+    const int k = static_cast<int>(top_k);
+    if (in_kind == KIND_F32) {
+      hipLaunchKernelGGL(moe_weighted_gather8_kernel<KIND_F32>, grid, dim3(256), 0, stream, down, lane_to_compact,
+                         routing_weights, out, tokens, k, hidden, compact_rows, out_kind);
+    } else if (in_kind == KIND_BF16) {
+      hipLaunchKernelGGL(moe_weighted_gather8_kernel<KIND_BF16>, grid, dim3(256), 0, stream, down, lane_to_compact,
+                         routing_weights, out, tokens, k, hidden, compact_rows, out_kind);
+    } else {
+      hipLaunchKernelGGL(moe_weighted_gather8_kernel<KIND_F16>, grid, dim3(256), 0, stream, down, lane_to_compact,
+                         routing_weights, out, tokens, k, hidden, compact_rows, out_kind);
+    }
+    return static_cast<int>(hipGetLastError());
   }
   hipLaunchKernelGGL(moe_weighted_gather_kernel, dim3(static_cast<unsigned>((hidden + 255) / 256),
                                                       static_cast<unsigned>(tokens)),

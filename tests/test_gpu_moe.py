@@ -345,6 +345,64 @@ def test_prefill_chain_matches_cpu_moe(dev, tokens, experts):
     assert np.all(np.isfinite(got))
 
 
+def test_prefill_chain_with_bf16_intermediates(dev):
+    """The same chain with hipEngine's own intermediate types: gate|up through the named bf16 entry, SiLU*up +
+    DS4 pack from bf16, down projection stored as bf16, gather from bf16.  Every stage is held to the float32
+    stage on the same inputs (bf16 output = bf16_round(float32 output) bit for bit, packed bytes equal to the
+    oracle's), the end to the reference CPU MoE with the gate hipEngine's q8_1 tests use."""
+    tokens, experts, top_k, hidden, inter = 96, 16, 8, 2048, 512
+    sel, wts = _routing(79, tokens, top_k, experts)
+    host, d = _device_index(dev, sel, wts, experts)
+    total, lanes = host["total"], tokens * top_k
+    wg = _experts(O.GGML_Q4_K, experts, inter, hidden, seed=4)
+    wu = _experts(O.GGML_Q4_K, experts, inter, hidden, seed=5)
+    wd = _experts(O.GGML_Q4_K, experts, hidden, inter, seed=6)
+    x = (np.random.default_rng(9).standard_normal((tokens, hidden)) * 0.3).astype(np.float32)
+    xb = O.f32_to_bf16_bits(x)
+    dxb, dg, du, dd = dev.put(xb), dev.put(wg), dev.put(wu), dev.put(wd)
+    dxq = dev.empty(tokens * (hidden // 128) * 144)
+    Q.gguf_q8_1_mmq_ds4_pack_bf16(dxb.ptr, dxq.ptr, tokens, hidden)
+    idx = (d["expert_start"].ptr, d["mmq_start"].ptr, d["tile_expert"].ptr)
+    # gate|up: named bf16 entry against the float32 form
+    dgu32, dgu16 = dev.empty(total * 2 * inter * 4), dev.empty(total * 2 * inter * 2)
+    M.gguf_q4_k_grouped_mmq(dxq.ptr, *idx, dg.ptr, dgu32.ptr, total, tokens, hidden, inter, experts, host["mmq_total"],
+                            compact_to_source_ptr=d["c2s"].ptr, qweight_b_ptr=du.ptr, out_features_b=inter)
+    M.gguf_q4_k_selected_dual_q8_1_ds4_mmq32_prefill_compact32_bf16_bf16_out(
+        dxq.ptr, d["c2s"].ptr, *idx, dg.ptr, du.ptr, dgu16.ptr, total, hidden, inter, inter, experts, host["mmq_total"])
+    gu16 = dev.get(dgu16, np.uint16, (total, 2 * inter)).copy()
+    assert np.array_equal(gu16, O.f32_to_bf16_bits(dev.get(dgu32, np.float32, (total, 2 * inter))))
+    # SiLU*up + DS4 pack from the bf16 gate|up: the oracle's bytes
+    dmq = dev.empty(total * (inter // 128) * 144)
+    M.moe_silu_mul_ds4_pack(dgu16.ptr, dmq.ptr, total, inter, in_dtype="bf16")
+    guf = O.bf16_bits_to_f32(gu16)
+    mid_bits = O.f32_to_bf16_bits((O.silu(guf[:, :inter]) * guf[:, inter:]).astype(np.float32))
+    got_mq = dev.get(dmq, np.uint8, (total, inter // 128, 144)).copy()
+    want_mq = O.pack_q8_1_ds4(mid_bits)
+    assert np.mean(got_mq != want_mq) < 2e-3          # silu through expf on the device: a few last-place differences
+    # down: bf16 store of the float32 result on the same packed intermediate
+    ddown32, ddown16 = dev.empty(total * hidden * 4), dev.empty(total * hidden * 2)
+    M.gguf_q4_k_grouped_mmq(dmq.ptr, *idx, dd.ptr, ddown32.ptr, total, total, inter, hidden, experts, host["mmq_total"])
+    M.gguf_q4_k_grouped_mmq(dmq.ptr, *idx, dd.ptr, ddown16.ptr, total, total, inter, hidden, experts, host["mmq_total"],
+                            out_dtype="bf16")
+    down16 = dev.get(ddown16, np.uint16, (total, hidden)).copy()
+    assert np.array_equal(down16, O.f32_to_bf16_bits(dev.get(ddown32, np.float32, (total, hidden))))
+    # ordered weighted gather from bf16 rows
+    dout = dev.empty(tokens * hidden * 4)
+    M.moe_weighted_gather_sum(ddown16.ptr, d["l2c"].ptr, d["w"].ptr, dout.ptr, tokens, top_k, hidden, total,
+                              in_dtype="bf16")
+    got = dev.get(dout, np.float32, (tokens, hidden)).copy()
+    dev.free(dxb, dg, du, dd, dxq, dgu32, dgu16, dmq, ddown32, ddown16, dout, *d.values())
+    downf = O.bf16_bits_to_f32(down16)
+    want_out = np.zeros((tokens, hidden), dtype=np.float64)
+    for lane in range(lanes):
+        want_out[lane // top_k] += np.float64(wts.reshape(-1)[lane]) * downf[host["l2c"][lane]]
+    assert O.max_rel_err(got, want_out.astype(np.float32), floor_frac=1e-3) <= 1e-4
+    pick = np.arange(0, tokens, 8)
+    ref = O.moe_selected_ffn(O.bf16_bits_to_f32(xb)[pick], sel[pick], wts[pick], wg, wu, wd)
+    assert O.cosine(got[pick], ref) >= 0.999
+    np.testing.assert_allclose(got[pick], ref, rtol=2e-2, atol=5e-2 * np.abs(ref).max())
+
+
 def test_moe_wrappers_reject_bad_arguments(dev):
     with pytest.raises(ValueError, match="num_experts"):
         GS.qwen35_moe_mmq32_tile_map(1, 1, 1, 1, 0)
