@@ -695,8 +695,11 @@ int launch_selected(int qt, int mode, const void* x, int x_kind, const int64_t* 
     // waves = 8 slots x ks K slices <= 16; one or two groups of 16 rows per workgroup, one as
     // long as the grid stays above ~2 workgroups per CU
     const int ks = nb >= 2 ? 2 : 1;
-    int rgn = 2;
-    while (rgn > 1 && (N + 16 * rgn - 1) / (16 * rgn) * x_rows < 512) rgn >>= 1;
+    // one workgroup per CU is resident (16 waves of ~80 registers): the fewest row groups per workgroup that
+    // keep the grid within one round of 256 workgroups (measured, E=256 k=8 H=2048 I=512: T=4 8.4 us against
+    // 12.7 with twice the workgroups, T=8 12.4 against 16.3)
+    int rgn = 1;
+    while (rgn < 4 && (N + 16 * rgn - 1) / (16 * rgn) * x_rows > 256) rgn <<= 1;   // 256 CUs
     s.g.ks = ks; s.g.nrg = rgn;
     const size_t lds = gemv_lds_bytes(qt, 8, 1, 1, ks, 1) + static_cast<size_t>(8) * ks * 16 * rgn * 4 + 8 * 4;
     if (lds > 64 * 1024) return static_cast<int>(hipErrorInvalidValue);
@@ -709,9 +712,9 @@ int launch_selected(int qt, int mode, const void* x, int x_kind, const int64_t* 
     else hipLaunchKernelGGL((selected_down_sum_kernel<QT, 8, RGN>), grid, block, lds, stream, s);                \
   } while (0)
     if (qt == GGML_Q4_K) {
-      if (rgn == 2) LAUNCH_DOWN(GGML_Q4_K, 2); else LAUNCH_DOWN(GGML_Q4_K, 1);
+      if (rgn == 4) LAUNCH_DOWN(GGML_Q4_K, 4); else if (rgn == 2) LAUNCH_DOWN(GGML_Q4_K, 2); else LAUNCH_DOWN(GGML_Q4_K, 1);
     } else {
-      if (rgn == 2) LAUNCH_DOWN(GGML_Q6_K, 2); else LAUNCH_DOWN(GGML_Q6_K, 1);
+      if (rgn == 4) LAUNCH_DOWN(GGML_Q6_K, 4); else if (rgn == 2) LAUNCH_DOWN(GGML_Q6_K, 2); else LAUNCH_DOWN(GGML_Q6_K, 1);
     }
 #undef LAUNCH_DOWN
     return static_cast<int>(hipGetLastError());
@@ -722,9 +725,6 @@ int launch_selected(int qt, int mode, const void* x, int x_kind, const int64_t* 
   if (nb <= 8) { ks = nb; cb = 1; }
   else if (nb <= 16) { ks = 8; cb = 2; }
   else { ks = 4; cb = 5; }
-  // many lanes: half the K slices, twice the rows per workgroup (the staging of the
-  // activations is per workgroup, so a grid far above the CU count only repeats it)
-  if (nb == 8 && lanes * ((N + 31) / 32) > 768) { ks = 4; cb = 2; }
   const SelVariant* v = nullptr;
   for (const SelVariant& c : kSel)
     if (c.qt == qt && c.cb == cb && c.mode == mode) v = &c;
@@ -734,7 +734,9 @@ int launch_selected(int qt, int mode, const void* x, int x_kind, const int64_t* 
   int nrg = v->max_threads / 64 / ks;
   if (nrg < 1) return static_cast<int>(hipErrorInvalidValue);
   const int rows_out_per_group = 16;
-  while (nrg > 1 && (N + nrg * rows_out_per_group - 1) / (nrg * rows_out_per_group) * lanes < 512) nrg >>= 1;
+  // 16 rows per workgroup until the grid passes 2048 workgroups (measured, gate/up of 64 lanes x 512 rows, K = 2048:
+  // 16.0 us at 16 rows per workgroup, 17.9 at 32, 18.5 with four K slices of two blocks)
+  while (nrg > 1 && (N + nrg * rows_out_per_group - 1) / (nrg * rows_out_per_group) * lanes < 2048) nrg >>= 1;
   s.g.ks = ks; s.g.nrg = nrg;
   size_t lds = gemv_lds_bytes(qt, 1, r, cb, ks, nrg);
   if (mode == SEL_DUAL_SILU) {
