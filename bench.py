@@ -315,12 +315,12 @@ class Harness:
             b["x"] = mem.to_device(x, runtime=rt)
             b["mid"] = mem.malloc(lanes * inter * 4, runtime=rt)
 
-            def chain(_i):
+            def chain(_i, stream=0):
                 M.gguf_selected_gemv("gguf_q4_k", M.SEL_DUAL_SILU, b["x"].ptr, b["sel"].ptr, b["wg"].ptr, b["mid"].ptr,
-                                     tokens, lanes, experts, hidden, inter, qweight_b_ptr=b["wu"].ptr)
+                                     tokens, lanes, experts, hidden, inter, qweight_b_ptr=b["wu"].ptr, stream=stream)
                 M.gguf_selected_gemv("gguf_q4_k", M.SEL_DOWN_SUM, b["mid"].ptr, b["sel"].ptr, b["wd"].ptr, b["out"].ptr,
                                      tokens, lanes, experts, inter, hidden, routing_weights_ptr=b["wts"].ptr,
-                                     top_k=top_k)
+                                     top_k=top_k, stream=stream)
         else:
             xb = (x.view(np.uint32) >> 16).astype(np.uint16)
             cap = lanes // 32 + experts
@@ -352,6 +352,29 @@ class Harness:
                 M.moe_weighted_gather_sum(b["down"].ptr, b["l2c"].ptr, b["wts"].ptr, b["out"].ptr, tokens, top_k, hidden,
                                           lanes, in_dtype="bf16")
         _, ev = self.time_launches(chain, steps, warmup)
+        self.last_moe_graph_s = None
+        if tokens <= 8:
+            # the same chain 16 times in one HIP graph: the GPU time without the host's launch rate
+            # (two ctypes launches take ~12 us on the host, as long as the two kernels)
+            reps = 16
+            stream = rt.stream_create()
+            rt.stream_begin_capture(stream)
+            for _ in range(reps):
+                chain(0, stream)
+            graph = rt.stream_end_capture(stream)
+            graph_exec = rt.graph_instantiate(graph)
+            for _ in range(3):
+                rt.graph_launch(graph_exec, stream)
+            rt.stream_synchronize(stream)
+            rt.event_record(self.ev0, stream)
+            for _ in range(max(4, steps // reps)):
+                rt.graph_launch(graph_exec, stream)
+            rt.event_record(self.ev1, stream)
+            rt.stream_synchronize(stream)
+            self.last_moe_graph_s = rt.event_elapsed_time_ms(self.ev0, self.ev1) * 1e-3 / (max(4, steps // reps) * reps)
+            rt.graph_exec_destroy(graph_exec)
+            rt.graph_destroy(graph)
+            rt.stream_destroy(stream)
         for buf in bufs.values():
             mem.free(buf)
         ops = 2.0 * lanes * (2 * inter * hidden + hidden * inter)
@@ -503,6 +526,8 @@ def main() -> None:
             extra[f"moe_q4_k_e256_k8_h2048_i512_t{tokens}"] = {
                 "us": round(sec * 1e6, 1), "expert_GB/s": round(touched / sec / 1e9, 1),
                 "int8_TOPS": round(ops / sec / 1e12, 2), "launches": 2 if tokens <= 8 else 10}
+            if h.last_moe_graph_s:
+                extra[f"moe_q4_k_e256_k8_h2048_i512_t{tokens}"]["hip_graph_us"] = round(h.last_moe_graph_s * 1e6, 1)
 
     # the MMQ half of the metric, as a second roofline object: int8 operations 2*M*N*K of the Q4_K prefill GEMM at
     # M = 2048 over its HIP-event time, against the dense int8 MFMA peak
