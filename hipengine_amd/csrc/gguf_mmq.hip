@@ -120,22 +120,26 @@ int launch_q4(const void* xq, const uint8_t* w, void* out, int out_kind, int64_t
 constexpr int A6_STRIDE = 176;   // 160-byte D4S4 block padded to 11 x 16 B
 constexpr int W6_STRIDE = 144;   // 128 centred int8 values padded to 9 x 16 B
 
+// COLS: columns of the workgroup's tile, 128 (each wave 64 x 64) or 64 (each wave 64 x 32: twice the tiles for
+// a narrow N, whose 128-wide tiles leave a last round mostly empty).
+template <int COLS>
 struct Q6Smem {
   uint8_t xa[BM * A6_STRIDE];
-  uint8_t w8[BN * W6_STRIDE];
-  float sw[8][BN];     // d * scale of the 8 16-value groups of the step, by column
-  float cw[8][BN];     // -MAGIC * sw (exact: d has 11 significant bits, the scale 8)
+  uint8_t w8[COLS * W6_STRIDE];
+  float sw[8][COLS];   // d * scale of the 8 16-value groups of the step, by column
+  float cw[8][COLS];   // -MAGIC * sw (exact: d has 11 significant bits, the scale 8)
   float xd[4][BM];     // activation scale per 32 values, by row
 };
 
 struct Q6StepRegs {
   u32x4 pa[5];         // 128 rows x 10 chunks = 1280 = 5 per thread
   u32x4 qla, qlb, qh;  // 16 bytes each of the column tid/2, byte offset 16*(tid&1)
-  uint2 sc;            // threads 0..127: the 8 scales of column tid
-  uint32_t d;          //                 and its fp16 d
-  u32x4 xd;            // threads 128..255: the four float scales of row tid-128
+  uint2 sc;            // threads 0..COLS-1: the 8 scales of column tid
+  uint32_t d;          //                    and its fp16 d
+  u32x4 xd;            // threads COLS..COLS+127: the four float scales of row tid-COLS
 };
 
+template <int COLS>
 __device__ __forceinline__ void q6_step_load(const MmqArgs& a, int step, int m0, int n0, int64_t w_row_bytes,
                                              int64_t x_row_bytes, int tid, Q6StepRegs& r) {
   const int kb = step >> 1, hh = step & 1;
@@ -146,7 +150,7 @@ __device__ __forceinline__ void q6_step_load(const MmqArgs& a, int step, int m0,
     const int m = min(m0 + row, a.M - 1);
     r.pa[i] = *reinterpret_cast<const u32x4*>(a.xq + m * x_row_bytes + static_cast<int64_t>(step) * D4S4_BYTES + part * 16);
   }
-  {
+  if (tid < 2 * COLS) {
     const int n = min(n0 + (tid >> 1), a.N - 1);
     const uint8_t* blk = a.w + n * w_row_bytes + static_cast<int64_t>(kb) * Q6_K_BYTES;
     const int o = (tid & 1) * 16;
@@ -155,24 +159,25 @@ __device__ __forceinline__ void q6_step_load(const MmqArgs& a, int step, int m0,
     r.qlb = u32x4{y.x, y.y, y.z, y.w};
     r.qh = u32x4{z.x, z.y, z.z, z.w};
   }
-  if (tid < BN) {
+  if (tid < COLS) {
     const uint8_t* blk = a.w + min(n0 + tid, a.N - 1) * w_row_bytes + static_cast<int64_t>(kb) * Q6_K_BYTES;
     r.sc = load8(blk + 192 + 8 * hh);
     r.d = load2(blk + 208);
-  } else {
-    r.xd = *reinterpret_cast<const u32x4*>(a.xq + min(m0 + tid - BN, a.M - 1) * x_row_bytes +
+  } else if (tid < COLS + BM) {
+    r.xd = *reinterpret_cast<const u32x4*>(a.xq + min(m0 + tid - COLS, a.M - 1) * x_row_bytes +
                                            static_cast<int64_t>(step) * D4S4_BYTES);
   }
 }
 
-__device__ __forceinline__ void q6_step_store(Q6Smem& s, int tid, const Q6StepRegs& r) {
+template <int COLS>
+__device__ __forceinline__ void q6_step_store(Q6Smem<COLS>& s, int tid, const Q6StepRegs& r) {
 #pragma unroll
   for (int i = 0; i < 5; ++i) {
     const int c = tid + i * THREADS;
     const int row = c / 10, part = c - row * 10;
     *reinterpret_cast<u32x4*>(s.xa + row * A6_STRIDE + part * 16) = r.pa[i];
   }
-  {
+  if (tid < 2 * COLS) {
     u32x4 q0, q1, q2, q3;   // the four 32-value quarters of the half, bytes o..o+15 of each
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
@@ -185,7 +190,7 @@ __device__ __forceinline__ void q6_step_store(Q6Smem& s, int tid, const Q6StepRe
     *reinterpret_cast<u32x4*>(dst + 64) = q2;
     *reinterpret_cast<u32x4*>(dst + 96) = q3;
   }
-  if (tid < BN) {
+  if (tid < COLS) {
     const float d = f16_bits_to_float(r.d & 0xFFFFu);
 #pragma unroll
     for (int j = 0; j < 8; ++j) {
@@ -195,52 +200,54 @@ __device__ __forceinline__ void q6_step_store(Q6Smem& s, int tid, const Q6StepRe
       s.sw[j][tid] = sw;
       s.cw[j][tid] = -MAGIC * sw;
     }
-  } else {
+  } else if (tid < COLS + BM) {
 #pragma unroll
-    for (int j = 0; j < 4; ++j) s.xd[j][tid - BN] = bits_to_float(r.xd[j]);
+    for (int j = 0; j < 4; ++j) s.xd[j][tid - COLS] = bits_to_float(r.xd[j]);
   }
 }
 
 // DUMP: the verification instantiation, which also writes every int32 16-value dot to dots[M, N, K/16].
-template <bool DUMP>
+template <bool DUMP, int COLS = BN>
 __global__ void __launch_bounds__(THREADS, 2) mmq_q6_k_d4s4_kernel(MmqArgs a, int32_t* __restrict__ dots) {
+  static_assert(COLS == 128 || COLS == 64, "two wave columns of one or two 32-wide tiles");
+  constexpr int NT = COLS / 64;                   // 32-wide n tiles per wave
   extern __shared__ __align__(16) uint8_t smem_raw[];
-  Q6Smem& s = *reinterpret_cast<Q6Smem*>(smem_raw);
+  Q6Smem<COLS>& s = *reinterpret_cast<Q6Smem<COLS>*>(smem_raw);
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int wm = wave & 1, wn = wave >> 1;
   const int lc = lane & 31, g = lane >> 5;
-  const int m0 = blockIdx.x * BM, n0 = blockIdx.y * BN;
+  const int m0 = blockIdx.x * BM, n0 = blockIdx.y * COLS;
   const int steps = a.K / 128;
   const int64_t w_row_bytes = static_cast<int64_t>(a.K / QK_K) * Q6_K_BYTES;
   const int64_t x_row_bytes = static_cast<int64_t>(steps) * D4S4_BYTES;
 
-  float acc[2][2][16];
+  float acc[NT][2][16];
 #pragma unroll
-  for (int i = 0; i < 2; ++i)
+  for (int i = 0; i < NT; ++i)
 #pragma unroll
     for (int j = 0; j < 2; ++j)
 #pragma unroll
       for (int v = 0; v < 16; ++v) acc[i][j][v] = 0.0f;
 
   Q6StepRegs regs;
-  q6_step_load(a, 0, m0, n0, w_row_bytes, x_row_bytes, tid, regs);
+  q6_step_load<COLS>(a, 0, m0, n0, w_row_bytes, x_row_bytes, tid, regs);
 
   for (int step = 0; step < steps; ++step) {
     q6_step_store(s, tid, regs);
     __syncthreads();
-    if (step + 1 < steps) q6_step_load(a, step + 1, m0, n0, w_row_bytes, x_row_bytes, tid, regs);
+    if (step + 1 < steps) q6_step_load<COLS>(a, step + 1, m0, n0, w_row_bytes, x_row_bytes, tid, regs);
 
     v16i ci;
 #pragma unroll
     for (int v = 0; v < 16; ++v) ci[v] = static_cast<int>(MAGIC_BITS);
 #pragma unroll
     for (int sl = 0; sl < 4; ++sl) {            // 32 activation values share one scale
-      long wop[2][2];                            // [n tile][16-value group]
+      long wop[NT][2];                           // [n tile][16-value group]
 #pragma unroll
-      for (int nt = 0; nt < 2; ++nt)
+      for (int nt = 0; nt < NT; ++nt)
 #pragma unroll
         for (int t = 0; t < 2; ++t)
-          wop[nt][t] = *reinterpret_cast<const long*>(s.w8 + (wn * 64 + nt * 32 + lc) * W6_STRIDE + 32 * sl + 16 * t + 8 * g);
+          wop[nt][t] = *reinterpret_cast<const long*>(s.w8 + (wn * 32 * NT + nt * 32 + lc) * W6_STRIDE + 32 * sl + 16 * t + 8 * g);
       long xop[2][2];                            // [m tile][16-value group]
 #pragma unroll
       for (int mt = 0; mt < 2; ++mt) {
@@ -248,11 +255,12 @@ __global__ void __launch_bounds__(THREADS, 2) mmq_q6_k_d4s4_kernel(MmqArgs a, in
         xop[mt][0] = *reinterpret_cast<const long*>(ap);
         xop[mt][1] = *reinterpret_cast<const long*>(ap + 16);
       }
-      // Software pipeline over the four (m tile, n tile) pairs: the two MFMAs of pair i+1 are issued before
+      // Software pipeline over the 2 * NT (m tile, n tile) pairs: the two MFMAs of pair i+1 are issued before
       // the scale arithmetic of pair i.
+      constexpr int PAIRS = 2 * NT;
       struct Dots { v16i d0, d1; };
       auto issue = [&](int i) {
-        const int mt = i >> 1, nt = i & 1;
+        const int mt = i / NT, nt = i % NT;
         Dots r;
         r.d0 = __builtin_amdgcn_mfma_i32_32x32x16_i8(xop[mt][0], wop[nt][0], ci, 0, 0, 0);
         r.d1 = __builtin_amdgcn_mfma_i32_32x32x16_i8(xop[mt][1], wop[nt][1], ci, 0, 0, 0);
@@ -260,17 +268,17 @@ __global__ void __launch_bounds__(THREADS, 2) mmq_q6_k_d4s4_kernel(MmqArgs a, in
       };
       Dots cur = issue(0);
 #pragma unroll
-      for (int i = 0; i < 4; ++i) {
-        const int mt = i >> 1, nt = i & 1;
+      for (int i = 0; i < PAIRS; ++i) {
+        const int mt = i / NT, nt = i % NT;
         Dots next = cur;
-        if (i + 1 < 4) next = issue(i + 1);
+        if (i + 1 < PAIRS) next = issue(i + 1);
         float xdv[16];
 #pragma unroll
         for (int j = 0; j < 4; ++j) {
           const float4 t = *reinterpret_cast<const float4*>(&s.xd[sl][wm * 64 + mt * 32 + 8 * j + 4 * g]);
           xdv[4 * j] = t.x; xdv[4 * j + 1] = t.y; xdv[4 * j + 2] = t.z; xdv[4 * j + 3] = t.w;
         }
-        const int col = wn * 64 + nt * 32 + lc;
+        const int col = wn * 32 * NT + nt * 32 + lc;
         if constexpr (DUMP) {
 #pragma unroll
           for (int v = 0; v < 16; ++v) {
@@ -297,12 +305,15 @@ __global__ void __launch_bounds__(THREADS, 2) mmq_q6_k_d4s4_kernel(MmqArgs a, in
   }
 
 #pragma unroll
-  for (int nt = 0; nt < 2; ++nt)
+  for (int nt = 0; nt < NT; ++nt)
 #pragma unroll
     for (int mt = 0; mt < 2; ++mt)
-      store_tile(a, acc[nt][mt], m0 + wm * 64 + mt * 32 + 4 * g, n0 + wn * 64 + nt * 32 + lc);
+      store_tile(a, acc[nt][mt], m0 + wm * 64 + mt * 32 + 4 * g, n0 + wn * 32 * NT + nt * 32 + lc);
 }
 
+#ifndef Q6_TILE_CHOICE
+#define Q6_TILE_CHOICE(wide_fill, narrow_fill) ((wide_fill) < 0.7 && (narrow_fill) > (wide_fill) + 0.1)
+#endif
 int launch_q6(const void* xq, const uint8_t* w, void* out, int out_kind, int64_t M, int64_t K, int64_t N,
               hipStream_t stream) {
   if (!xq || !w || !out || M <= 0 || M > (1 << 20) || K <= 0 || (K % QK_K) != 0 || N <= 0 || N > (1 << 24) ||
@@ -311,9 +322,21 @@ int launch_q6(const void* xq, const uint8_t* w, void* out, int out_kind, int64_t
   }
   MmqArgs a{static_cast<const uint8_t*>(xq), w, out, out_kind, static_cast<int>(M), static_cast<int>(K),
             static_cast<int>(N)};
-  const dim3 grid(static_cast<unsigned>((M + BM - 1) / BM), static_cast<unsigned>((N + BN - 1) / BN));
-  hipLaunchKernelGGL(mmq_q6_k_d4s4_kernel<false>, grid, dim3(THREADS), sizeof(Q6Smem), stream, a,
-                     static_cast<int32_t*>(nullptr));
+  // 128-wide tiles unless their last round of the 512 resident workgroups would be less than half full and
+  // 64-wide tiles fill their rounds better (N = 5120 at M = 2048: 640 tiles = 1.25 rounds against 1280 = 2.5)
+  const int64_t m_tiles = (M + BM - 1) / BM;
+  const int64_t wide = m_tiles * ((N + 127) / 128), narrow = m_tiles * ((N + 63) / 64);
+  const int64_t slots = 2 * 256;
+  auto fill = [&](int64_t tiles) { return static_cast<double>(tiles) / static_cast<double>((tiles + slots - 1) / slots * slots); };
+  if (Q6_TILE_CHOICE(fill(wide), fill(narrow))) {
+    const dim3 grid(static_cast<unsigned>(m_tiles), static_cast<unsigned>((N + 63) / 64));
+    hipLaunchKernelGGL((mmq_q6_k_d4s4_kernel<false, 64>), grid, dim3(THREADS), sizeof(Q6Smem<64>), stream, a,
+                       static_cast<int32_t*>(nullptr));
+  } else {
+    const dim3 grid(static_cast<unsigned>(m_tiles), static_cast<unsigned>((N + BN - 1) / BN));
+    hipLaunchKernelGGL((mmq_q6_k_d4s4_kernel<false, 128>), grid, dim3(THREADS), sizeof(Q6Smem<128>), stream, a,
+                       static_cast<int32_t*>(nullptr));
+  }
   return static_cast<int>(hipGetLastError());
 }
 
@@ -388,7 +411,7 @@ extern "C" int hipengine_gfx950_gguf_mmq_dots_i32(int32_t ggml_type, const void*
     if ((out_features % 32) != 0) return static_cast<int>(hipErrorInvalidValue);
     hipLaunchKernelGGL(mmq_tile_dump_kernel<DenseQ5>, grid, dim3(THREADS), sizeof(DenseQ5::Smem), stream, a, dots);
   } else if (ggml_type == GGML_Q6_K) {
-    hipLaunchKernelGGL(mmq_q6_k_d4s4_kernel<true>, grid, dim3(THREADS), sizeof(Q6Smem), stream, a, dots);
+    hipLaunchKernelGGL((mmq_q6_k_d4s4_kernel<true, 128>), grid, dim3(THREADS), sizeof(Q6Smem<128>), stream, a, dots);
   } else {
     return static_cast<int>(hipErrorInvalidValue);
   }
@@ -434,5 +457,5 @@ extern "C" int hipengine_gfx950_gguf_prefill_bf16(int32_t ggml_type, const void*
 
 int hipengine_gfx950::mmq_load() {
   hipFuncAttributes attr;
-  return static_cast<int>(hipFuncGetAttributes(&attr, reinterpret_cast<const void*>(mmq_q6_k_d4s4_kernel<false>)));
+  return static_cast<int>(hipFuncGetAttributes(&attr, reinterpret_cast<const void*>(mmq_q6_k_d4s4_kernel<false, 128>)));
 }

@@ -127,6 +127,24 @@ def test_q6_k_mmq_matches_formula_and_cpu_reference(dev, rows, k, n):
     assert O.max_rel_err(got, ref) <= 1e-3 and O.cosine(got, ref) >= 0.99999
 
 
+def test_q6_k_mmq_narrow_tiles(dev):
+    """A shape whose 128-wide tiles would leave the last round of resident workgroups a quarter full takes 64-wide
+    tiles (20 x 32 = 640 tiles against 1280): sampled rows against the formula, every row against the wide-tile
+    result of the same columns computed as two half-width problems is not needed - the sums of an element do not
+    depend on the tile, so a second shape that takes wide tiles on the same data must give the same bits."""
+    rows, k, n = 2560, 256, 4096
+    xb = _bf16_rows(21, rows, k, scale=0.1, offset=0.002)
+    d4 = O.pack_q8_1_d4s4(xb)
+    w = O.random_weight(O.GGML_Q6_K, n, k, seed=31)
+    got = _run_q4(dev, M.gguf_q6_k_mmq32_q8_1_d4s4_f32_bf16_f32_out, d4, w, rows, k, n)
+    pick = np.array([0, 1, 31, 32, 127, 128, 1000, 2047, 2048, 2559])
+    want = O.mmq_q6_k_d4s4(d4[pick], w)
+    assert O.max_rel_err(got[pick], want) <= 1e-3 and O.cosine(got[pick], want) >= 0.99999
+    # the first 128 rows alone are one row of tiles: 32 wide tiles, filled 6 %, so the wide kernel runs them
+    wide = _run_q4(dev, M.gguf_q6_k_mmq32_q8_1_d4s4_f32_bf16_f32_out, d4[:128], w, 128, k, n)
+    assert np.array_equal(got[:128].view(np.uint32), wide.view(np.uint32))
+
+
 def test_q6_k_mmq_closed_form_bf16_and_determinism(dev):
     rows, k, n = 70, 512, 96
     xb = _bf16_rows(13, rows, k, scale=0.125)
