@@ -387,8 +387,66 @@ DEFINE_Q8_1(hipengine_gguf_q4_k_q8_1_dp4a_vdr_bf16_f32_out, GGML_Q4_K, KIND_F32)
 DEFINE_Q8_1(hipengine_gguf_q4_k_q8_1_dp4a_vdr_bf16_bf16_out, GGML_Q4_K, KIND_BF16)
 DEFINE_Q8_1(hipengine_gguf_q6_k_q8_1_dp4a_gemv_bf16_f32_out, GGML_Q6_K, KIND_F32)
 DEFINE_Q8_1(hipengine_gguf_q6_k_q8_1_dp4a_gemv_bf16_bf16_out, GGML_Q6_K, KIND_BF16)
-DEFINE_Q8_1(hipengine_gguf_q8_0_dp4a_gemv_f32_f32_out, GGML_Q8_0, KIND_F32)
-DEFINE_Q8_1(hipengine_gguf_q8_0_dp4a_gemv_bf16_bf16_out, GGML_Q8_0, KIND_BF16)
+DEFINE_Q8_1(hipengine_gguf_q4_k_q8_1_dp4a_ctl_bf16_f32_out, GGML_Q4_K, KIND_F32)
+DEFINE_Q8_1(hipengine_gguf_q4_k_q8_1_dp4a_ctl_bf16_bf16_out, GGML_Q4_K, KIND_BF16)
+
+// The Q8_0 entry points carry a `threads` argument before the stream (ignored, as in hipEngine).  The split
+// forms take two or three matrices over the same q8_1 activations, each with its own output buffer.
+static int launch_q8_0_split(int count, const void* xq, const uint8_t* const* qweights, void* const* outs, int out_kind,
+                             int64_t rows, int64_t in_features, const int64_t* out_features, hipStream_t stream) {
+  if (!xq || rows <= 0 || in_features <= 0 || (in_features % QK_K) != 0) return static_cast<int>(hipErrorInvalidValue);
+  int qt[4];
+  for (int i = 0; i < count; ++i) {
+    qt[i] = GGML_Q8_0;
+    if (!qweights[i] || !outs[i] || out_features[i] <= 0) return static_cast<int>(hipErrorInvalidValue);
+  }
+  if (rows <= 2 && stream_multi_ok(count, qt, static_cast<int>(rows), in_features, out_features)) {
+    return launch_gemv_stream_multi(count, qt, xq, KIND_Q8_1, qweights, outs, out_kind, static_cast<int>(rows),
+                                    in_features, out_features, stream);
+  }
+  for (int i = 0; i < count; ++i) {
+    const int rc = launch_gemv(GGML_Q8_0, xq, KIND_Q8_1, qweights[i], outs[i], out_kind, rows, in_features,
+                               out_features[i], nullptr, stream);
+    if (rc != static_cast<int>(hipSuccess)) return rc;
+  }
+  return static_cast<int>(hipSuccess);
+}
+
+#define DEFINE_Q8_0_DP4A(SUFFIX, OKIND)                                                                             \
+  extern "C" int hipengine_gguf_q8_0_dp4a_gemv_##SUFFIX(const void* xq, const uint8_t* qweight, void* out,          \
+                                                        int64_t rows, int64_t in_features, int64_t out_features,    \
+                                                        int64_t /*threads*/, hipStream_t stream) {                  \
+    return launch_gemv(GGML_Q8_0, xq, KIND_Q8_1, qweight, out, OKIND, rows, in_features, out_features, nullptr,     \
+                       stream);                                                                                     \
+  }                                                                                                                 \
+  extern "C" int hipengine_gguf_q8_0_dp4a_rowtile4_gemv_##SUFFIX(const void* xq, const uint8_t* qweight, void* out, \
+                                                                 int64_t rows, int64_t in_features,                 \
+                                                                 int64_t out_features, int64_t /*threads*/,         \
+                                                                 hipStream_t stream) {                              \
+    return launch_gemv(GGML_Q8_0, xq, KIND_Q8_1, qweight, out, OKIND, rows, in_features, out_features, nullptr,     \
+                       stream);                                                                                     \
+  }                                                                                                                 \
+  extern "C" int hipengine_gguf_q8_0_dp4a_dual_split_rowtile4_gemv_##SUFFIX(                                        \
+      const void* xq, const uint8_t* qweight_a, const uint8_t* qweight_b, void* out_a, void* out_b, int64_t rows,   \
+      int64_t in_features, int64_t out_features_a, int64_t out_features_b, int64_t /*threads*/,                     \
+      hipStream_t stream) {                                                                                         \
+    const uint8_t* const w[2] = {qweight_a, qweight_b};                                                             \
+    void* const o[2] = {out_a, out_b};                                                                              \
+    const int64_t n[2] = {out_features_a, out_features_b};                                                          \
+    return launch_q8_0_split(2, xq, w, o, OKIND, rows, in_features, n, stream);                                     \
+  }                                                                                                                 \
+  extern "C" int hipengine_gguf_q8_0_dp4a_triple_split_rowtile4_gemv_##SUFFIX(                                      \
+      const void* xq, const uint8_t* qweight_a, const uint8_t* qweight_b, const uint8_t* qweight_c, void* out_a,    \
+      void* out_b, void* out_c, int64_t rows, int64_t in_features, int64_t out_features_a, int64_t out_features_b,  \
+      int64_t out_features_c, int64_t /*threads*/, hipStream_t stream) {                                            \
+    const uint8_t* const w[3] = {qweight_a, qweight_b, qweight_c};                                                  \
+    void* const o[3] = {out_a, out_b, out_c};                                                                       \
+    const int64_t n[3] = {out_features_a, out_features_b, out_features_c};                                          \
+    return launch_q8_0_split(3, xq, w, o, OKIND, rows, in_features, n, stream);                                     \
+  }
+
+DEFINE_Q8_0_DP4A(f32_f32_out, KIND_F32)
+DEFINE_Q8_0_DP4A(bf16_bf16_out, KIND_BF16)
 
 // ---- explicit layout, for tuning sweeps --------------------------------------
 

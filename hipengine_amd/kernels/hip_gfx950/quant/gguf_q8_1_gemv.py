@@ -11,8 +11,8 @@ stream, library, runtime)`` (``kernels/hip_gfx1100/quant/gguf_q4_k_gemv.py:115-1
   (``gguf_q4_k_gemv.py:175-202,524-576``, ``gguf_k_gemv.py:1920-2049``), registered under the keys its
   dispatcher asks for, ``("linear", quant, "gemv_*" / "prefill_*")``; they run the fused kernels;
 * ``gguf_q4_k_q8_1_dp4a_vdr_*``, ``gguf_q6_k_q8_1_dp4a_gemv_*`` and
-  ``gguf_q8_0_dp4a_gemv_*`` take pre-quantized 36-byte q8_1 blocks, as
-  hipEngine's ``gguf_q4_k_q8_1_dp4a_vdr_gemv.py`` / ``gguf_q8_0_dp4a_gemv.py`` do.
+  ``gguf_q8_0_dp4a_[rowtile4_|dual_split_rowtile4_|triple_split_rowtile4_]gemv_*`` take pre-quantized 36-byte
+  q8_1 blocks, as hipEngine's ``gguf_q4_k_q8_1_dp4a_vdr_gemv.py`` / ``gguf_q8_0_dp4a_gemv.py`` do.
 """
 
 from __future__ import annotations
@@ -163,10 +163,43 @@ gguf_q6_k_q8_1_dp4a_gemv_bf16_f32_out = _make_q8_1(
     "gguf_q6_k_q8_1_dp4a_gemv_bf16_f32_out", "hipengine_gguf_q6_k_q8_1_dp4a_gemv_bf16_f32_out")
 gguf_q6_k_q8_1_dp4a_gemv_bf16_bf16_out = _make_q8_1(
     "gguf_q6_k_q8_1_dp4a_gemv_bf16_bf16_out", "hipengine_gguf_q6_k_q8_1_dp4a_gemv_bf16_bf16_out")
-gguf_q8_0_dp4a_gemv_f32_f32_out = _make_q8_1(
-    "gguf_q8_0_dp4a_gemv_f32_f32_out", "hipengine_gguf_q8_0_dp4a_gemv_f32_f32_out")
-gguf_q8_0_dp4a_gemv_bf16_bf16_out = _make_q8_1(
-    "gguf_q8_0_dp4a_gemv_bf16_bf16_out", "hipengine_gguf_q8_0_dp4a_gemv_bf16_bf16_out")
+gguf_q4_k_q8_1_dp4a_ctl_bf16_f32_out = _make_q8_1(
+    "gguf_q4_k_q8_1_dp4a_ctl_bf16_f32_out", "hipengine_gguf_q4_k_q8_1_dp4a_ctl_bf16_f32_out")
+gguf_q4_k_q8_1_dp4a_ctl_bf16_bf16_out = _make_q8_1(
+    "gguf_q4_k_q8_1_dp4a_ctl_bf16_bf16_out", "hipengine_gguf_q4_k_q8_1_dp4a_ctl_bf16_bf16_out")
+
+
+def _make_q8_0_dp4a(name: str, count: int):
+    """hipEngine's Q8_0 entries over q8_1 activations (``gguf_q8_0_dp4a_gemv.py:124-400``): ``count`` weights and
+    outputs, then rows, in_features, one out_features per weight, a ``threads`` slot (passed as 0, as hipEngine's
+    wrappers do) and the stream."""
+    symbol = f"hipengine_{name}"
+    argtypes = [VOID] * (1 + 2 * count) + [I64] * (2 + count) + [I64, VOID]
+
+    def wrapper(xq_ptr: int, *args: int, stream: int = 0, library: ctypes.CDLL | None = None,
+                runtime: HipRuntime | None = None) -> None:
+        if len(args) != 3 * count + 2:
+            raise TypeError(f"{name} takes xq_ptr, {count} weight and {count} output pointers, rows, in_features and "
+                            f"{count} out_features")
+        pointers, (rows, in_features, *out_features) = args[:2 * count], args[2 * count:]
+        for n in out_features:
+            validate_linear(rows, in_features, n, 128)
+        validate_pointers(xq_ptr=xq_ptr, **{f"ptr_{i}": p for i, p in enumerate(pointers)})
+        check_launch(entry(symbol, argtypes, library)(xq_ptr, *pointers, rows, in_features, *out_features, 0, stream),
+                     runtime)
+
+    wrapper.__name__ = name
+    wrapper.__doc__ = (f"GGUF Q8_0 GEMV of {count} matri{'x' if count == 1 else 'ces'} over pre-quantized q8_1 "
+                       f"activation blocks (C symbol ``{symbol}``).")
+    return wrapper
+
+
+Q8_0_DP4A: dict[str, object] = {}
+for _shape, _count in (("", 1), ("rowtile4_", 1), ("dual_split_rowtile4_", 2), ("triple_split_rowtile4_", 3)):
+    for _suffix in ("f32_f32_out", "bf16_bf16_out"):
+        _fn = _make_q8_0_dp4a(f"gguf_q8_0_dp4a_{_shape}gemv_{_suffix}", _count)
+        Q8_0_DP4A[f"q8_1_dp4a_{_shape}gemv_{_suffix}"] = _fn
+        globals()[_fn.__name__] = _fn
 
 _TUNED_ARGS = [I32, VOID, I32, VOID, VOID, I32, I64, I64, I64, I32, I32, I32, I32, VOID]
 
@@ -381,7 +414,8 @@ def register_kernels(backend: str = "hip_gfx950", *, replace: bool = False) -> N
         ("gguf_q4_k", "q8_1_dp4a_vdr_bf16_bf16_out", gguf_q4_k_q8_1_dp4a_vdr_bf16_bf16_out),
         ("gguf_q6_k", "q8_1_dp4a_gemv_bf16_f32_out", gguf_q6_k_q8_1_dp4a_gemv_bf16_f32_out),
         ("gguf_q6_k", "q8_1_dp4a_gemv_bf16_bf16_out", gguf_q6_k_q8_1_dp4a_gemv_bf16_bf16_out),
-        ("gguf_q8_0", "q8_1_dp4a_gemv_f32_f32_out", gguf_q8_0_dp4a_gemv_f32_f32_out),
-        ("gguf_q8_0", "q8_1_dp4a_gemv_bf16_bf16_out", gguf_q8_0_dp4a_gemv_bf16_bf16_out),
+        ("gguf_q4_k", "q8_1_dp4a_ctl_bf16_f32_out", gguf_q4_k_q8_1_dp4a_ctl_bf16_f32_out),
+        ("gguf_q4_k", "q8_1_dp4a_ctl_bf16_bf16_out", gguf_q4_k_q8_1_dp4a_ctl_bf16_bf16_out),
+        *(("gguf_q8_0", variant, fn) for variant, fn in Q8_0_DP4A.items()),
     ):
         register(KernelKey(backend, "linear", quant, variant), fn, replace=replace)

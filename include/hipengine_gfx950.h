@@ -160,11 +160,54 @@ int hipengine_gguf_q6_k_q8_1_dp4a_gemv_bf16_f32_out(const void* xq, const uint8_
 int hipengine_gguf_q6_k_q8_1_dp4a_gemv_bf16_bf16_out(const void* xq, const uint8_t* qweight, void* out, int64_t rows,
                                                      int64_t in_features, int64_t out_features,
                                                      hipengine_stream_t stream);
+/* The "ctl" names of the same Q4_K kernel (gguf_q4_k_q8_1_dp4a_vdr_gemv.hip:348-364: a second code shape of the
+ * same arithmetic in hipEngine; one kernel here). */
+int hipengine_gguf_q4_k_q8_1_dp4a_ctl_bf16_f32_out(const void* xq, const uint8_t* qweight, void* out, int64_t rows,
+                                                   int64_t in_features, int64_t out_features,
+                                                   hipengine_stream_t stream);
+int hipengine_gguf_q4_k_q8_1_dp4a_ctl_bf16_bf16_out(const void* xq, const uint8_t* qweight, void* out, int64_t rows,
+                                                    int64_t in_features, int64_t out_features,
+                                                    hipengine_stream_t stream);
+
+/* Q8_0 weights over pre-quantized q8_1 activations (gguf_q8_0_dp4a_gemv.hip:345-387).  As in hipEngine these
+ * carry a `threads` argument before the stream, which is ignored.  The "rowtile4" names (lines 389-437) are
+ * hipEngine's variant that reuses a weight row across four activation rows; here every batch already does,
+ * so they run the same kernels.  in_features must be a multiple of 256 (hipEngine: of 32). */
 int hipengine_gguf_q8_0_dp4a_gemv_f32_f32_out(const void* xq, const uint8_t* qweight, void* out, int64_t rows,
-                                              int64_t in_features, int64_t out_features, hipengine_stream_t stream);
+                                              int64_t in_features, int64_t out_features, int64_t threads,
+                                              hipengine_stream_t stream);
 int hipengine_gguf_q8_0_dp4a_gemv_bf16_bf16_out(const void* xq, const uint8_t* qweight, void* out, int64_t rows,
-                                                int64_t in_features, int64_t out_features,
+                                                int64_t in_features, int64_t out_features, int64_t threads,
                                                 hipengine_stream_t stream);
+int hipengine_gguf_q8_0_dp4a_rowtile4_gemv_f32_f32_out(const void* xq, const uint8_t* qweight, void* out, int64_t rows,
+                                                       int64_t in_features, int64_t out_features, int64_t threads,
+                                                       hipengine_stream_t stream);
+int hipengine_gguf_q8_0_dp4a_rowtile4_gemv_bf16_bf16_out(const void* xq, const uint8_t* qweight, void* out,
+                                                         int64_t rows, int64_t in_features, int64_t out_features,
+                                                         int64_t threads, hipengine_stream_t stream);
+
+/* Two or three Q8_0 matrices over the same q8_1 activations, each with its own contiguous output
+ * [rows, out_features_i] (gguf_q8_0_dp4a_gemv.hip:439-600: the q/k/v or gate/up projections of a block in one
+ * launch).  rows <= 2 take one launch of the streaming kernel shared among the matrices by their sizes; larger
+ * batches run one launch per matrix.  Every output is bit-equal to the single-matrix call's. */
+int hipengine_gguf_q8_0_dp4a_dual_split_rowtile4_gemv_f32_f32_out(const void* xq, const uint8_t* qweight_a,
+                                                                  const uint8_t* qweight_b, void* out_a, void* out_b,
+                                                                  int64_t rows, int64_t in_features,
+                                                                  int64_t out_features_a, int64_t out_features_b,
+                                                                  int64_t threads, hipengine_stream_t stream);
+int hipengine_gguf_q8_0_dp4a_dual_split_rowtile4_gemv_bf16_bf16_out(const void* xq, const uint8_t* qweight_a,
+                                                                    const uint8_t* qweight_b, void* out_a, void* out_b,
+                                                                    int64_t rows, int64_t in_features,
+                                                                    int64_t out_features_a, int64_t out_features_b,
+                                                                    int64_t threads, hipengine_stream_t stream);
+int hipengine_gguf_q8_0_dp4a_triple_split_rowtile4_gemv_f32_f32_out(
+    const void* xq, const uint8_t* qweight_a, const uint8_t* qweight_b, const uint8_t* qweight_c, void* out_a,
+    void* out_b, void* out_c, int64_t rows, int64_t in_features, int64_t out_features_a, int64_t out_features_b,
+    int64_t out_features_c, int64_t threads, hipengine_stream_t stream);
+int hipengine_gguf_q8_0_dp4a_triple_split_rowtile4_gemv_bf16_bf16_out(
+    const void* xq, const uint8_t* qweight_a, const uint8_t* qweight_b, const uint8_t* qweight_c, void* out_a,
+    void* out_b, void* out_c, int64_t rows, int64_t in_features, int64_t out_features_a, int64_t out_features_b,
+    int64_t out_features_c, int64_t threads, hipengine_stream_t stream);
 
 /* Up to four matrices over one activation, out_i = W_i x: the q, k and v projections of an attention block,
  * whatever their types (each of Q4_K, Q5_K, Q6_K, Q8_0) and row counts.  qweights, outs and out_features are

@@ -213,6 +213,49 @@ def test_prequantized_gemv_matches_fused_bit_for_bit(dev, quant, fn):
     _check_f32(pre, xq, w, QT[quant])
 
 
+@pytest.mark.parametrize("rows,k,sizes,suffix", [
+    (1, 5120, (1024, 256, 512), "f32_f32_out"),      # one launch shared among the matrices
+    (2, 4096, (768, 130), "bf16_bf16_out"),          # ragged second matrix
+    (1, 1024, (48, 80, 16), "bf16_bf16_out"),        # too small to share a launch: one launch per matrix
+    (6, 2048, (96, 40, 72), "f32_f32_out"),          # more than two activation rows
+    (11, 1024, (64, 33), "f32_f32_out"),             # more than eight
+])
+def test_q8_0_dp4a_family_takes_hipengine_argument_lists(dev, rows, k, sizes, suffix):
+    """gguf_q8_0_dp4a_{,rowtile4_,dual_split_rowtile4_,triple_split_rowtile4_}gemv_*: the argument lists of
+    hipEngine's exports (a `threads` slot before the stream; one output buffer and row count per matrix).  Every
+    output equals the single-matrix call's bit for bit and the oracle's q8_1 x Q8_0 GEMV within float32 noise."""
+    rng = np.random.default_rng(1234 + rows)
+    x = rng.standard_normal((rows, k)).astype(np.float32)
+    xq = O.quantize_q8_1(x)
+    ws = [O.random_weight(O.GGML_Q8_0, n, k, seed=50 + i) for i, n in enumerate(sizes)]
+    bf16 = suffix.startswith("bf16")
+    width, dtype = (2, np.uint16) if bf16 else (4, np.float32)
+    dxq = dev.put(xq)
+    dws = [dev.put(w) for w in ws]
+
+    def run(name, weights, ns):
+        outs = [dev.empty(rows * n * width) for n in ns]
+        getattr(G, name)(dxq.ptr, *[w.ptr for w in weights], *[o.ptr for o in outs], rows, k, *ns)
+        got = [dev.get(o, dtype, (rows, n)) for o, n in zip(outs, ns)]
+        dev.free(*outs)
+        return got
+
+    single = [run(f"gguf_q8_0_dp4a_gemv_{suffix}", [dw], [n])[0] for dw, n in zip(dws, sizes)]
+    tiled = [run(f"gguf_q8_0_dp4a_rowtile4_gemv_{suffix}", [dw], [n])[0] for dw, n in zip(dws, sizes)]
+    shape = {2: "dual", 3: "triple"}[len(sizes)]
+    split = run(f"gguf_q8_0_dp4a_{shape}_split_rowtile4_gemv_{suffix}", dws, list(sizes))
+    dev.free(dxq, *dws)
+    for one, four, many, w in zip(single, tiled, split, ws):
+        assert np.array_equal(one, four)
+        assert np.array_equal(one, many)
+        ref = O.gemv_q8_1_q8_0(xq, w).astype(np.float32)
+        if bf16:      # the bf16 output is the float32 result rounded to nearest even
+            assert O.max_rel_err(O.bf16_bits_to_f32(one), ref) <= 2.0 ** -8
+        else:
+            assert O.max_rel_err(one, ref) <= REL_TOL
+            assert O.cosine(one, ref) >= COS_MIN
+
+
 def test_more_than_eight_rows_and_determinism(dev):
     rng = np.random.default_rng(44)
     rows, k, n = 19, 1024, 48
