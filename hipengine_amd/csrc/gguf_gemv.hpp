@@ -44,7 +44,12 @@ struct GemvArgs {
   int N;
   int ks;               // K-slices per workgroup
   int nrg;              // row groups per workgroup
+  const void* x_up;     // KIND_SILU_BF16 only: the second bf16 operand, the activation is bf16(silu(x) * x_up)
 };
+
+// Activation kind of the expert-selected down projection that takes the gate and up rows as they are
+// (bf16) and forms bf16(silu(gate) * up) while staging (gguf_k_gemv.hip:1813-1866).  Not part of the C ABI.
+constexpr int KIND_SILU_BF16 = 4;
 
 // Q4_K and Q5_K share the header (d, dmin, 6-bit scales and mins) and the min term.
 constexpr bool gemv_has_mins(int qt) { return qt == GGML_Q4_K || qt == GGML_Q5_K; }
@@ -310,9 +315,18 @@ __device__ __forceinline__ void gemv_stage_activations(const GemvArgs& a, int kc
             v0 = v.x; v1 = v.y; v2 = v.z; v3 = v.w;
           } else {
             const uint2 v = *reinterpret_cast<const uint2*>(static_cast<const uint16_t*>(a.x) + k0);
-            if (a.x_kind == KIND_BF16) {
+            if (a.x_kind == KIND_BF16 || a.x_kind == KIND_SILU_BF16) {
               v0 = bf16_bits_to_float(v.x & 0xFFFFu); v1 = bf16_bits_to_float(v.x >> 16);
               v2 = bf16_bits_to_float(v.y & 0xFFFFu); v3 = bf16_bits_to_float(v.y >> 16);
+              if (a.x_kind == KIND_SILU_BF16) {
+                const uint2 u = *reinterpret_cast<const uint2*>(static_cast<const uint16_t*>(a.x_up) + k0);
+                const auto act = [](float g, uint32_t up_bits) {
+                  const float silu = g / (1.0f + expf(-g));
+                  return bf16_bits_to_float(float_to_bf16_bits(silu * bf16_bits_to_float(up_bits)));
+                };
+                v0 = act(v0, u.x & 0xFFFFu); v1 = act(v1, u.x >> 16);
+                v2 = act(v2, u.y & 0xFFFFu); v3 = act(v3, u.y >> 16);
+              }
             } else {
               v0 = f16_bits_to_float(v.x & 0xFFFFu); v1 = f16_bits_to_float(v.x >> 16);
               v2 = f16_bits_to_float(v.y & 0xFFFFu); v3 = f16_bits_to_float(v.y >> 16);

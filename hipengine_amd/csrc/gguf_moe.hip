@@ -530,6 +530,9 @@ __global__ void __launch_bounds__((sel_max_threads<QT, R * CB>())) selected_gemv
   const int per = s.lanes / s.x_rows;
   const int x_row = s.x_rows == 1 ? 0 : lane / per;
   a.x = static_cast<const uint8_t*>(s.g.x) + static_cast<int64_t>(x_row) * act_row_bytes(s.g.x_kind, s.g.K);
+  if constexpr (XK == KIND_SILU_BF16) {
+    a.x_up = static_cast<const uint8_t*>(s.g.x_up) + static_cast<int64_t>(x_row) * act_row_bytes(s.g.x_kind, s.g.K);
+  }
   a.out = static_cast<uint8_t*>(s.g.out) + static_cast<int64_t>(lane) * s.g.N * scalar_bytes(s.g.out_kind);
   if constexpr (MODE == SEL_SINGLE) {
     gemv_workgroup<QT, 1, R, CB>(a, s.g.w + e * expert_bytes, blockIdx.x * s.g.nrg * 16 * R, smem);
@@ -653,29 +656,41 @@ struct SelVariant {
   int qt, cb, mode, max_threads;
   SelFn fn;
   SelFn by_kind[2];   // float32 and bf16 activations
+  SelFn silu_pair;    // single form over bf16(silu(gate) * up)
 };
-#define SEL_VARIANTS(QT, CB)                                                                                   \
+#define SEL_SINGLE_VARIANT(QT, CB)                                                                             \
   SelVariant{QT, CB, SEL_SINGLE, sel_max_threads<QT, CB>(), selected_gemv_kernel<QT, 1, CB, SEL_SINGLE>,          \
-             {selected_gemv_kernel<QT, 1, CB, SEL_SINGLE, KIND_F32>, selected_gemv_kernel<QT, 1, CB, SEL_SINGLE, KIND_BF16>}}, \
+             {selected_gemv_kernel<QT, 1, CB, SEL_SINGLE, KIND_F32>, selected_gemv_kernel<QT, 1, CB, SEL_SINGLE, KIND_BF16>}, \
+             selected_gemv_kernel<QT, 1, CB, SEL_SINGLE, KIND_SILU_BF16>}
+#define SEL_VARIANTS(QT, CB)                                                                                   \
+  SEL_SINGLE_VARIANT(QT, CB),                                                                                  \
   SelVariant{QT, CB, SEL_DUAL_SILU, sel_max_threads<QT, 2 * CB>(), selected_gemv_kernel<QT, 2, CB, SEL_DUAL_SILU>, \
-             {selected_gemv_kernel<QT, 2, CB, SEL_DUAL_SILU, KIND_F32>, selected_gemv_kernel<QT, 2, CB, SEL_DUAL_SILU, KIND_BF16>}}, \
-  SelVariant{QT, CB, SEL_DUAL, sel_max_threads<QT, 2 * CB>(), selected_gemv_kernel<QT, 2, CB, SEL_DUAL>, {nullptr, nullptr}}
+             {selected_gemv_kernel<QT, 2, CB, SEL_DUAL_SILU, KIND_F32>, selected_gemv_kernel<QT, 2, CB, SEL_DUAL_SILU, KIND_BF16>}, \
+             nullptr},                                                                                         \
+  SelVariant{QT, CB, SEL_DUAL, sel_max_threads<QT, 2 * CB>(), selected_gemv_kernel<QT, 2, CB, SEL_DUAL>,          \
+             {nullptr, nullptr}, nullptr}
+// Q4_K and Q6_K experts take every form; Q5_K and Q8_0 experts the single form (a projection per launch)
 const SelVariant kSel[] = {
     SEL_VARIANTS(GGML_Q4_K, 1), SEL_VARIANTS(GGML_Q4_K, 2), SEL_VARIANTS(GGML_Q4_K, 5),
     SEL_VARIANTS(GGML_Q6_K, 1), SEL_VARIANTS(GGML_Q6_K, 2), SEL_VARIANTS(GGML_Q6_K, 5),
+    SEL_SINGLE_VARIANT(GGML_Q5_K, 1), SEL_SINGLE_VARIANT(GGML_Q5_K, 2), SEL_SINGLE_VARIANT(GGML_Q5_K, 5),
+    SEL_SINGLE_VARIANT(GGML_Q8_0, 1), SEL_SINGLE_VARIANT(GGML_Q8_0, 2), SEL_SINGLE_VARIANT(GGML_Q8_0, 5),
 };
 
 int launch_selected(int qt, int mode, const void* x, int x_kind, const int64_t* selected, const float* routing,
                     const uint8_t* w_a, const uint8_t* w_b, void* out, int out_kind, int64_t x_rows, int64_t lanes,
                     int64_t num_experts, int64_t top_k, int64_t K, int64_t N, int round_mid, hipStream_t stream,
-                    void* out_b = nullptr) {
-  // q8_1 blocks as activations: the single and dual forms only (their staging reads them as they are)
+                    void* out_b = nullptr, const void* x_up = nullptr) {
+  // q8_1 blocks as activations: the single and dual forms only (their staging reads them as they are);
+  // x_up: the single form over bf16(silu(x) * x_up), both bf16
   const int max_x_kind = (mode == SEL_SINGLE || mode == SEL_DUAL) ? KIND_Q8_1 : KIND_F16;
   if (!x || !selected || !w_a || !out || x_rows <= 0 || lanes <= 0 || lanes > 65535 || num_experts <= 0 || K <= 0 ||
       (K % QK_K) != 0 || K > (1 << 20) || N <= 0 || N > (1 << 24) || x_kind < KIND_F32 || x_kind > max_x_kind ||
-      out_kind < KIND_F32 || out_kind > KIND_F16 || (qt != GGML_Q4_K && qt != GGML_Q6_K)) {
+      out_kind < KIND_F32 || out_kind > KIND_F16 ||
+      (qt != GGML_Q4_K && qt != GGML_Q6_K && !(mode == SEL_SINGLE && (qt == GGML_Q5_K || qt == GGML_Q8_0)))) {
     return static_cast<int>(hipErrorInvalidValue);
   }
+  if (x_up && (mode != SEL_SINGLE || x_kind != KIND_BF16)) return static_cast<int>(hipErrorInvalidValue);
   if ((mode == SEL_DUAL_SILU || mode == SEL_DUAL) && !w_b) return static_cast<int>(hipErrorInvalidValue);
   if (mode == SEL_DUAL && !out_b) return static_cast<int>(hipErrorInvalidValue);
   if (mode == SEL_DOWN_SUM && (!routing || top_k <= 0 || top_k > 8 || lanes != x_rows * top_k)) {
@@ -686,6 +701,7 @@ int launch_selected(int qt, int mode, const void* x, int x_kind, const int64_t* 
   SelArgs s;
   s.g.x = x; s.g.w = w_a; s.g.out = out; s.g.x_kind = x_kind; s.g.out_kind = out_kind; s.g.rows = 1;
   s.g.K = static_cast<int>(K); s.g.N = static_cast<int>(N);
+  s.g.x_up = x_up;
   s.w_b = w_b; s.out_b = out_b; s.selected = selected; s.routing = routing;
   s.x_rows = static_cast<int>(x_rows); s.lanes = static_cast<int>(lanes);
   s.num_experts = static_cast<int>(num_experts); s.top_k = static_cast<int>(top_k); s.round_mid = round_mid;
@@ -747,7 +763,9 @@ int launch_selected(int qt, int mode, const void* x, int x_kind, const int64_t* 
   if (lds > 64 * 1024) return static_cast<int>(hipErrorInvalidValue);
   const int rows_out = nrg * rows_out_per_group;
   const dim3 grid(static_cast<unsigned>((N + rows_out - 1) / rows_out), static_cast<unsigned>(lanes));
-  const SelFn fn = ((x_kind == KIND_F32 || x_kind == KIND_BF16) && v->by_kind[x_kind]) ? v->by_kind[x_kind] : v->fn;
+  const SelFn fn = x_up ? v->silu_pair
+                   : ((x_kind == KIND_F32 || x_kind == KIND_BF16) && v->by_kind[x_kind]) ? v->by_kind[x_kind] : v->fn;
+  if (!fn) return static_cast<int>(hipErrorInvalidValue);
   hipLaunchKernelGGL(fn, grid, dim3(ks * nrg * 64), lds, stream, s);
   return static_cast<int>(hipGetLastError());
 }
@@ -1135,6 +1153,28 @@ extern "C" int hipengine_gguf_q4_k_selected_gemv_bf16_bf16_out(const uint16_t* x
   return launch_selected(GGML_Q4_K, SEL_SINGLE, x, KIND_BF16, selected, nullptr, qweight, nullptr, out, KIND_BF16,
                          x_rows, rows, num_experts, 1, in_features, out_features, 0, stream);
 }
+
+// The same for Q5_K / Q6_K / Q8_0 experts, and their down projection over bf16(silu(gate) * up) formed from the
+// gate and up rows while the activations are staged (gguf_k_gemv.hip:5586-5599, kernel :1813-1866).
+#define DEFINE_SELECTED_K(QNAME, QT)                                                                                 \
+  extern "C" int hipengine_gguf_##QNAME##_selected_gemv_bf16_bf16_out(                                               \
+      const uint16_t* x, const int64_t* selected, const uint8_t* qweight, uint16_t* out, int64_t x_rows,             \
+      int64_t rows, int64_t num_experts, int64_t in_features, int64_t out_features, int64_t /*threads*/,            \
+      hipStream_t stream) {                                                                                          \
+    return launch_selected(QT, SEL_SINGLE, x, KIND_BF16, selected, nullptr, qweight, nullptr, out, KIND_BF16, x_rows, \
+                           rows, num_experts, 1, in_features, out_features, 0, stream);                              \
+  }                                                                                                                  \
+  extern "C" int hipengine_gguf_##QNAME##_selected_silu_gemv_bf16_bf16_out(                                          \
+      const uint16_t* gate, const uint16_t* up, const int64_t* selected, const uint8_t* qweight, uint16_t* out,      \
+      int64_t x_rows, int64_t rows, int64_t num_experts, int64_t in_features, int64_t out_features,                  \
+      int64_t /*threads*/, hipStream_t stream) {                                                                     \
+    if (!up) return static_cast<int>(hipErrorInvalidValue);                                                          \
+    return launch_selected(QT, SEL_SINGLE, gate, KIND_BF16, selected, nullptr, qweight, nullptr, out, KIND_BF16,     \
+                           x_rows, rows, num_experts, 1, in_features, out_features, 0, stream, nullptr, up);         \
+  }
+DEFINE_SELECTED_K(q5_k, GGML_Q5_K)
+DEFINE_SELECTED_K(q6_k, GGML_Q6_K)
+DEFINE_SELECTED_K(q8_0, GGML_Q8_0)
 
 extern "C" int hipengine_gguf_q4_k_selected_dual_silu_gemv_bf16_bf16_out(
     const uint16_t* x, const int64_t* selected, const uint8_t* qweight_a, const uint8_t* qweight_b, uint16_t* out,

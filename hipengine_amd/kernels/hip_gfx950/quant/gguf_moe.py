@@ -51,6 +51,47 @@ def gguf_q4_k_selected_gemv_bf16_bf16_out(x_ptr: int, selected_ptr: int, qweight
                     threads, stream), runtime)
 
 
+def _make_selected_k(quant: str):
+    """``gguf_<q>_selected_gemv_bf16_bf16_out`` and ``gguf_<q>_selected_silu_gemv_bf16_bf16_out`` for Q5_K, Q6_K and
+    Q8_0 experts (hipEngine ``gguf_k_gemv.py:229-232,497,713-716,789-792,1587-1634``)."""
+    single_symbol = f"hipengine_gguf_{quant}_selected_gemv_bf16_bf16_out"
+    silu_symbol = f"hipengine_gguf_{quant}_selected_silu_gemv_bf16_bf16_out"
+
+    def single(x_ptr: int, selected_ptr: int, qweight_ptr: int, out_ptr: int, x_rows: int, rows: int,
+               num_experts: int, in_features: int, out_features: int, *, threads: int = 128, stream: int = 0,
+               library: ctypes.CDLL | None = None, runtime: HipRuntime | None = None) -> None:
+        _validate_selected(x_rows, rows, num_experts, in_features, out_features, threads)
+        validate_pointers(x_ptr=x_ptr, selected_ptr=selected_ptr, qweight_ptr=qweight_ptr, out_ptr=out_ptr)
+        fn = entry(single_symbol, [VOID] * 4 + [I64] * 6 + [VOID], library)
+        check_launch(fn(x_ptr, selected_ptr, qweight_ptr, out_ptr, x_rows, rows, num_experts, in_features,
+                        out_features, threads, stream), runtime)
+
+    def silu(gate_ptr: int, up_ptr: int, selected_ptr: int, qweight_ptr: int, out_ptr: int, x_rows: int, rows: int,
+             num_experts: int, in_features: int, out_features: int, *, threads: int = 128, stream: int = 0,
+             library: ctypes.CDLL | None = None, runtime: HipRuntime | None = None) -> None:
+        _validate_selected(x_rows, rows, num_experts, in_features, out_features, threads)
+        validate_pointers(gate_ptr=gate_ptr, up_ptr=up_ptr, selected_ptr=selected_ptr, qweight_ptr=qweight_ptr,
+                          out_ptr=out_ptr)
+        fn = entry(silu_symbol, [VOID] * 5 + [I64] * 6 + [VOID], library)
+        check_launch(fn(gate_ptr, up_ptr, selected_ptr, qweight_ptr, out_ptr, x_rows, rows, num_experts, in_features,
+                        out_features, threads, stream), runtime)
+
+    single.__name__ = f"gguf_{quant}_selected_gemv_bf16_bf16_out"
+    single.__doc__ = (f"``out[lane] = W[selected[lane]] . x[lane // (rows // x_rows)]`` for {quant.upper()} experts, "
+                      f"bf16 in and out (C symbol ``{single_symbol}``).")
+    silu.__name__ = f"gguf_{quant}_selected_silu_gemv_bf16_bf16_out"
+    silu.__doc__ = (f"``out[lane] = W[selected[lane]] . bf16(silu(gate[r]) * up[r])``, ``r = lane // (rows // x_rows)``, "
+                    f"for {quant.upper()} experts (C symbol ``{silu_symbol}``).")
+    return single, silu
+
+
+SELECTED_K: dict[str, tuple[object, object]] = {}
+for _quant in ("q5_k", "q6_k", "q8_0"):
+    SELECTED_K[_quant] = _make_selected_k(_quant)
+    for _fn in SELECTED_K[_quant]:
+        globals()[_fn.__name__] = _fn
+
+
 def gguf_q4_k_selected_dual_silu_gemv_bf16_bf16_out(x_ptr: int, selected_ptr: int, qweight_a_ptr: int,
                                                     qweight_b_ptr: int, out_ptr: int, x_rows: int, rows: int,
                                                     num_experts: int, in_features: int, out_features: int, *,
@@ -292,6 +333,10 @@ def register_kernels(backend: str = "hip_gfx950", *, replace: bool = False) -> N
              gguf_q4_k_selected_gemv_bf16_bf16_out, replace=replace)
     register(KernelKey(backend, "linear", "gguf_q4_k", "selected_dual_silu_gemv_bf16_bf16_out"),
              gguf_q4_k_selected_dual_silu_gemv_bf16_bf16_out, replace=replace)
+    for quant, (single, silu) in SELECTED_K.items():     # keys of hipEngine's gguf_k_gemv.py:1938,1987-1989,2022-2023
+        register(KernelKey(backend, "linear", f"gguf_{quant}", "selected_gemv_bf16_bf16_out"), single, replace=replace)
+        register(KernelKey(backend, "linear", f"gguf_{quant}", "selected_silu_gemv_bf16_bf16_out"), silu,
+                 replace=replace)
     register(KernelKey(backend, "linear", "gguf_q4_k", "selected_dual_gemv_bf16_bf16_out"),
              gguf_q4_k_selected_dual_gemv_bf16_bf16_out, replace=replace)
     register(KernelKey(backend, "linear", "gguf_q4_k", "selected_dual_gemv_q8_1_dp4a_bf16_bf16_out"),

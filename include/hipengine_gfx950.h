@@ -469,6 +469,23 @@ int hipengine_gguf_q4_k_selected_gemv_bf16_bf16_out(const uint16_t* x, const int
                                                     int64_t out_features, int64_t threads,
                                                     hipengine_stream_t stream);
 
+/* The same for Q5_K, Q6_K and Q8_0 experts (gguf_k_gemv.hip:5586-5592, macro instances :5619-5621), and their
+ * down projection that takes the gate and up rows [x_rows, in_features] (bf16) as they are: the activation of
+ * lane r is bf16(silu(gate) * up) of row r / (rows / x_rows), silu(g) = g / (1 + expf(-g)), formed while the
+ * activations are staged and quantized to q8_1 (gguf_k_gemv.hip:5593-5599, kernel :1813-1866). */
+#define HIPENGINE_GFX950_DECLARE_SELECTED_K(q)                                                                     \
+  int hipengine_gguf_##q##_selected_gemv_bf16_bf16_out(                                                            \
+      const uint16_t* x, const int64_t* selected, const uint8_t* qweight, uint16_t* out, int64_t x_rows,           \
+      int64_t rows, int64_t num_experts, int64_t in_features, int64_t out_features, int64_t threads,               \
+      hipengine_stream_t stream);                                                                                  \
+  int hipengine_gguf_##q##_selected_silu_gemv_bf16_bf16_out(                                                       \
+      const uint16_t* gate, const uint16_t* up, const int64_t* selected, const uint8_t* qweight, uint16_t* out,    \
+      int64_t x_rows, int64_t rows, int64_t num_experts, int64_t in_features, int64_t out_features,                \
+      int64_t threads, hipengine_stream_t stream);
+HIPENGINE_GFX950_DECLARE_SELECTED_K(q5_k)
+HIPENGINE_GFX950_DECLARE_SELECTED_K(q6_k)
+HIPENGINE_GFX950_DECLARE_SELECTED_K(q8_0)
+
 /* Decode gate/up pair: out[lane, n] = silu(bf16(gate)) * bf16(up), gate and up
  * rounded to bf16 before the activation as in gguf_q4_k_gemv.hip:732-736.
  * Replaces gguf_q4_k_gemv.hip:2751-2767. */

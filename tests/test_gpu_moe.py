@@ -189,6 +189,63 @@ def test_selected_gemv_bf16_entry_points(dev):
         assert O.max_rel_err(dual[lane], want, floor_frac=2e-2) <= 2e-2
 
 
+def _random_q5_k(n, k, seed):
+    rng = np.random.default_rng(seed)
+    nblk = n * (k // 256)
+    blk = O.pack_q5_k_blocks(rng.integers(0, 32, size=(nblk, 8, 32), dtype=np.uint8),
+                             rng.integers(0, 64, size=(nblk, 8), dtype=np.uint8),
+                             rng.integers(0, 64, size=(nblk, 8), dtype=np.uint8),
+                             (rng.random(nblk) * 0.05).astype(np.float32), (rng.random(nblk) * 0.02).astype(np.float32))
+    return blk.reshape(n, -1)
+
+
+@pytest.mark.parametrize("quant,qt", [("q5_k", O.GGML_Q5_K), ("q6_k", O.GGML_Q6_K), ("q8_0", O.GGML_Q8_0)])
+@pytest.mark.parametrize("tokens,top_k,experts,k,n", [(1, 8, 12, 512, 2048), (3, 4, 6, 2048, 272), (2, 2, 5, 4352, 40)])
+def test_selected_gemv_and_silu_down_for_other_expert_types(dev, quant, qt, tokens, top_k, experts, k, n):
+    """gguf_<q>_selected_gemv_bf16_bf16_out and gguf_<q>_selected_silu_gemv_bf16_bf16_out for Q5_K / Q6_K / Q8_0
+    experts: the plain projection over `tokens` rows fanned out to tokens * top_k lanes, and the down projection
+    whose activation is bf16(silu(gate) * up) of the lane's own row (x_rows == rows)."""
+    rng = np.random.default_rng(k + n + tokens)
+    sel, _ = _routing(k + n, tokens, top_k, experts)
+    if tokens > 1:
+        sel[1, 0] = experts                              # an invalid lane stays unwritten
+    base = _random_q5_k(n, k, seed=8) if qt == O.GGML_Q5_K else O.random_weight(qt, n, k, seed=8)
+    w = O.stack_experts(base, experts, seed=2)
+    lanes = tokens * top_k
+    single, silu = M.SELECTED_K[quant]
+    dsel, dw = dev.put(sel), dev.put(w)
+
+    xb = O.f32_to_bf16_bits((rng.standard_normal((tokens, k)) * 0.5).astype(np.float32))
+    dx = dev.put(xb)
+    dout = dev.empty(lanes * n * 2, fill=0x7F)
+    single(dx.ptr, dsel.ptr, dw.ptr, dout.ptr, tokens, lanes, experts, k, n)
+    got_single = dev.get(dout, np.uint16, (lanes, n))
+    dev.free(dx, dout)
+
+    gate = O.f32_to_bf16_bits((rng.standard_normal((lanes, k)) * 1.5).astype(np.float32))
+    up = O.f32_to_bf16_bits(rng.standard_normal((lanes, k)).astype(np.float32))
+    dg, du = dev.put(gate), dev.put(up)
+    dout = dev.empty(lanes * n * 2, fill=0x7F)
+    silu(dg.ptr, du.ptr, dsel.ptr, dw.ptr, dout.ptr, lanes, lanes, experts, k, n)
+    got_silu = dev.get(dout, np.uint16, (lanes, n))
+    dev.free(dg, du, dout, dsel, dw)
+
+    xf = O.bf16_bits_to_f32(xb)
+    act = O.bf16_bits_to_f32(O.f32_to_bf16_bits(O.silu(O.bf16_bits_to_f32(gate)) * O.bf16_bits_to_f32(up)))
+    for lane in range(lanes):
+        e = int(sel.reshape(-1)[lane])
+        if e >= experts:
+            assert np.all(got_single[lane] == 0x7F7F) and np.all(got_silu[lane] == 0x7F7F)
+            continue
+        # bf16 outputs: half a bf16 ulp (2^-9) on top of the float32 gate
+        ref = _ref_lane(xf[lane // top_k], w[e], qt)
+        assert O.max_rel_err(O.bf16_bits_to_f32(got_single[lane]), ref, floor_frac=1e-2) <= 6e-3
+        assert O.cosine(O.bf16_bits_to_f32(got_single[lane]), ref) >= 0.9999
+        ref = _ref_lane(act[lane], w[e], qt)
+        assert O.max_rel_err(O.bf16_bits_to_f32(got_silu[lane]), ref, floor_frac=1e-2) <= 6e-3
+        assert O.cosine(O.bf16_bits_to_f32(got_silu[lane]), ref) >= 0.9999
+
+
 @pytest.mark.parametrize("tokens,experts", [(1, 32), (8, 32), (1, 256), (8, 256)])
 def test_decode_chain_matches_cpu_moe(dev, tokens, experts):
     """dual SiLU GEMV -> routed down sum (two launches) against the reference CPU MoE FFN."""
