@@ -347,3 +347,47 @@ def test_gguf_container_round_trip_and_errors(tmp_path):
                        version=2)
     assert GG.scan_gguf(v2).version == 2 and GG.scan_gguf(v2).alignment == 32
     assert GG.scan_gguf(v2).tensor("w").byte_shape == (3, 68)
+
+
+def test_gguf_reader_on_a_container_packed_without_this_package(tmp_path):
+    """tests/golden/tiny_v3.gguf is packed field by field with `struct` (tests/golden/make_tiny_gguf.py), not by
+    this package's writer; content and expectations are those of hipEngine's reader test
+    (tests/test_unit_gguf_reader.py:54-142): reversed ggml dimensions, 32-byte alignment of the payload, string and
+    float arrays, F32 / BF16 / Q8_0 payloads."""
+    from pathlib import Path
+
+    import numpy as np
+
+    from hipengine_amd.loading import gguf as GG
+    from oracle import gguf_oracle as O
+
+    golden = Path(__file__).parent / "golden" / "tiny_v3.gguf"
+    info = GG.scan_gguf(golden)
+    assert info.version == 3 and info.alignment == 32 and info.architecture == "toy" and info.file_type == 7
+    assert info.metadata["toy.context_length"] == 16
+    assert info.metadata["tokenizer.ggml.tokens"] == ["a", "b"]
+    assert info.metadata["tokenizer.ggml.scores"] == pytest.approx([0.25, -0.5])
+    assert info.tensor_count == 3 and info.names_with_prefix("dense") == ("dense.weight",)
+    assert info.tensor_data_offset == 448                       # 435 header bytes rounded up to 32
+    dense, bf16, q8 = info.require(["dense.weight", "bf16.weight", "q8.weight"])
+    assert dense.shape == (2, 3) and dense.ggml_shape == (3, 2) and dense.ggml_type_name == "F32" and dense.nbytes == 24
+    assert bf16.byte_shape == (2,) and bf16.nbytes == 4
+    assert q8.shape == (1, 32) and q8.byte_shape == (1, 34) and q8.nbytes == 34
+    assert (dense.data_offset, bf16.data_offset, q8.data_offset) == (448, 480, 512)
+    reader = GG.GGUFReader(golden)
+    assert np.array_equal(reader.tensor_data("dense.weight"), np.arange(6, dtype=np.float32).reshape(2, 3))
+    assert np.array_equal(O.bf16_bits_to_f32(np.asarray(reader.tensor_data("bf16.weight"))), np.float32([1.0, -2.5]))
+    assert np.array_equal(O.dequantize(np.asarray(reader.tensor_data("q8.weight")), O.GGML_Q8_0)[0],
+                          np.arange(-16, 16, dtype=np.float32) * 2.0)
+    with pytest.raises(GG.MissingGGUFTensorError, match="missing required GGUF tensors: absent"):
+        info.require(["dense.weight", "absent"])
+    # the committed file is what the generator writes
+    script = golden.with_name("make_tiny_gguf.py").read_text().replace('with_name("tiny_v3.gguf")', f'with_name("{tmp_path.name}.gguf")')
+    probe = golden.with_name(f"{tmp_path.name}.gguf")
+    try:
+        namespace = {"__file__": str(golden.with_name("make_tiny_gguf.py")), "__name__": "make_tiny_gguf"}
+        exec(compile(script, "make_tiny_gguf.py", "exec"), namespace)
+        namespace["main"]()
+        assert probe.read_bytes() == golden.read_bytes()
+    finally:
+        probe.unlink(missing_ok=True)
