@@ -369,6 +369,24 @@ int launch_dual(int qt, const void* x, int x_kind, const uint8_t* w_a, const uin
   DEFINE_DENSE_DUAL(QNAME, QT, f32, KIND_F32, f32, KIND_F32) \
   DEFINE_DENSE_DUAL(QNAME, QT, bf16, KIND_BF16, bf16, KIND_BF16)
 
+// hipEngine's "rowtile" names (batches of 2 to 8 rows that reuse each weight row across the batch,
+// gguf_q4_k_gemv.hip:2496-2533, gguf_k_gemv.hip:5600-5617): every batch here does, so they are the same launch.
+#define DEFINE_ROWTILE(QNAME, QT, ANAME, AKIND, ONAME, OKIND)                                             \
+  extern "C" int hipengine_gguf_##QNAME##_gemv_rowtile_##ANAME##_##ONAME##_out(                           \
+      const void* x, const uint8_t* qweight, void* out, int64_t rows, int64_t in_features,                \
+      int64_t out_features, int64_t /*threads*/, hipStream_t stream) {                                    \
+    return launch_gemv(QT, x, AKIND, qweight, out, OKIND, rows, in_features, out_features, nullptr,       \
+                       stream);                                                                           \
+  }
+#define DEFINE_ROWTILE_ALL(QNAME, QT)                        \
+  DEFINE_ROWTILE(QNAME, QT, f32, KIND_F32, f32, KIND_F32)    \
+  DEFINE_ROWTILE(QNAME, QT, bf16, KIND_BF16, f32, KIND_F32)  \
+  DEFINE_ROWTILE(QNAME, QT, bf16, KIND_BF16, bf16, KIND_BF16)
+DEFINE_ROWTILE_ALL(q4_k, GGML_Q4_K)
+DEFINE_ROWTILE_ALL(q5_k, GGML_Q5_K)
+DEFINE_ROWTILE_ALL(q6_k, GGML_Q6_K)
+DEFINE_ROWTILE_ALL(q8_0, GGML_Q8_0)
+
 DEFINE_DENSE_ALL(q4_k, GGML_Q4_K)
 DEFINE_DENSE_ALL(q5_k, GGML_Q5_K)
 DEFINE_DENSE_ALL(q6_k, GGML_Q6_K)

@@ -144,6 +144,25 @@ __global__ void __launch_bounds__(256) silu_mul_ds4_pack_kernel(const void* __re
   ds4_pack_group(v, amax, g, e, out);
 }
 
+// The DS4 pack of rows gathered through the routing index: output row r is the pack of token
+// sorted_lanes[r] / top_k; a negative lane or a token outside [0, tokens) packs as a row of zeros
+// (gguf_q4_k_q8_1_selected_prefill.hip:705-772).  Bytes equal a row gather followed by the plain pack.
+__global__ void __launch_bounds__(256) gather_ds4_pack_kernel(const uint16_t* __restrict__ hidden_states,
+                                                              const int64_t* __restrict__ sorted_lanes,
+                                                              uint8_t* __restrict__ out, int64_t total_groups,
+                                                              int64_t groups_per_row, int64_t tokens, int64_t top_k) {
+  const int64_t g = static_cast<int64_t>(blockIdx.x) * 32 + (threadIdx.x >> 3);
+  const int e = threadIdx.x & 7;
+  if (g >= total_groups) return;
+  const int64_t row = g / groups_per_row, within = g - row * groups_per_row;
+  const int64_t lane = sorted_lanes[row];
+  const int64_t token = lane >= 0 ? lane / top_k : -1;
+  float v[4] = {0.0f, 0.0f, 0.0f, 0.0f};
+  if (token >= 0 && token < tokens) load4_values(hidden_states, KIND_BF16, (token * groups_per_row + within) * 32 + e * 4, v);
+  const float amax = oct_max(fmaxf(fmaxf(fabsf(v[0]), fabsf(v[1])), fmaxf(fabsf(v[2]), fabsf(v[3]))));
+  ds4_pack_group(v, amax, g, e, out);
+}
+
 int launch_q8_1(const void* x, int kind, void* xq, int64_t rows, int64_t in_features, hipStream_t stream) {
   if (!x || !xq || rows <= 0 || in_features <= 0 || (in_features % 32) != 0) {
     return static_cast<int>(hipErrorInvalidValue);
@@ -184,6 +203,21 @@ extern "C" int hipengine_gguf_q4_k_quantize_bf16_q8_1(const void* x, void* xq, i
 extern "C" int hipengine_gguf_q8_1_mmq_ds4_pack_bf16(const void* x, void* out, int64_t rows, int64_t hidden,
                                                      hipStream_t stream) {
   return launch_pack<false>(x, out, rows, hidden, stream);
+}
+
+extern "C" int hipengine_gguf_q8_1_mmq_gather_ds4_pack_bf16(const uint16_t* hidden_states, const int64_t* sorted_lanes,
+                                                            void* out, int64_t rows, int64_t hidden, int64_t tokens,
+                                                            int64_t top_k, hipStream_t stream) {
+  if (!hidden_states || !sorted_lanes || !out || rows <= 0 || hidden <= 0 || (hidden % 128) != 0 || tokens <= 0 ||
+      top_k <= 0) {
+    return static_cast<int>(hipErrorInvalidValue);
+  }
+  const int64_t groups = rows * (hidden / 32);
+  const int64_t grid = (groups + 31) / 32;
+  if (grid > 0x7FFFFFFF) return static_cast<int>(hipErrorInvalidValue);
+  hipLaunchKernelGGL(gather_ds4_pack_kernel, dim3(static_cast<unsigned>(grid)), dim3(256), 0, stream, hidden_states,
+                     sorted_lanes, static_cast<uint8_t*>(out), groups, hidden / 32, tokens, top_k);
+  return static_cast<int>(hipGetLastError());
 }
 
 extern "C" int hipengine_gguf_q8_1_d4s4_f32_quantize_bf16(const void* x, void* out, int64_t rows, int64_t hidden,

@@ -89,7 +89,7 @@ def gguf_prefill_workspace_bytes(quant_key: str, rows: int, in_features: int) ->
 
 
 def _make_dense(quant: str, family: str, act: str, out: str):
-    symbol = f"hipengine_gguf_{quant}_gemv_{act}_{out}_out"
+    symbol = f"hipengine_gguf_{quant}_gemv_{'rowtile_' if family == 'gemv_rowtile' else ''}{act}_{out}_out"
     quant_key = f"gguf_{quant}"
 
     def wrapper(x_ptr: int, qweight_ptr: int, out_ptr: int, rows: int, in_features: int, out_features: int, *,
@@ -144,6 +144,11 @@ for _q in _QUANTS:
             _fn = _make_dense(_q, _family, _a, _o)
             DENSE[(_q, _family, _a, _o)] = _fn
             globals()[_fn.__name__] = _fn
+for _q in _QUANTS:       # hipEngine's rowtile names (gguf_q4_k_gemv.py:1517-1519,1552-1554): the same launch
+    for _a, _o in (("f32", "f32"), ("bf16", "f32"), ("bf16", "bf16")):
+        _fn = _make_dense(_q, "gemv_rowtile", _a, _o)
+        DENSE[(_q, "gemv_rowtile", _a, _o)] = _fn
+        globals()[_fn.__name__] = _fn
 DENSE_DUAL = {(q, a, o): _make_dense_dual(q, a, o) for q in _QUANTS for a, o in (("f32", "f32"), ("bf16", "bf16"))}
 for _fn in DENSE_DUAL.values():
     globals()[_fn.__name__] = _fn
@@ -398,7 +403,8 @@ def register_kernels(backend: str = "hip_gfx950", *, replace: bool = False) -> N
     # the keys hipEngine's dispatcher resolves for raw-layout weights: gemv_* at one row, prefill_* above
     # (loading/qwen35_gguf_consumer_surface.py:134-144,527-530)
     for (quant, family, act, out), fn in DENSE.items():
-        register(KernelKey(backend, "linear", f"gguf_{quant}", f"{family}_{act}_{out}_out"), fn, replace=replace)
+        variant = family[len("gemv_"):] if family == "gemv_rowtile" else family     # "rowtile_<act>_<out>_out"
+        register(KernelKey(backend, "linear", f"gguf_{quant}", f"{variant}_{act}_{out}_out"), fn, replace=replace)
     for (quant, act, out), fn in DENSE_DUAL.items():
         register(KernelKey(backend, "linear", f"gguf_{quant}", f"dual_gemv_{act}_{out}_out"), fn, replace=replace)
     for (act, out), fn in PAIR_SILU.items():

@@ -46,6 +46,22 @@ def gguf_q8_1_mmq_ds4_pack_bf16(x_ptr: int, xq_ptr: int, rows: int, hidden: int,
     _quantize("hipengine_gguf_q8_1_mmq_ds4_pack_bf16", x_ptr, xq_ptr, rows, hidden, 128, stream, library, runtime)
 
 
+def gguf_q8_1_mmq_gather_ds4_pack_bf16(hidden_bf16_ptr: int, sorted_lanes_ptr: int, out_q8_ptr: int, rows: int,
+                                       hidden: int, tokens: int, top_k: int, *, stream: int = 0,
+                                       library: ctypes.CDLL | None = None, runtime: HipRuntime | None = None) -> None:
+    """Gather + DS4 pack in one pass (hipEngine ``gguf_q4_k_q8_1_selected_prefill.py:432-490``): output row ``r`` is
+    the pack of token ``sorted_lanes[r] // top_k`` of the bf16 ``[tokens, hidden]`` input, a row of zeros for a
+    negative lane or a token outside the input.  ``rows`` counts packed lanes."""
+    for name, value in (("rows", rows), ("hidden", hidden), ("tokens", tokens), ("top_k", top_k)):
+        if value <= 0:
+            raise ValueError(f"{name} must be positive")
+    if hidden % 128 != 0:
+        raise ValueError("hidden must be divisible by DS4 Q8_1 MMQ block size 128")
+    validate_pointers(hidden_bf16_ptr=hidden_bf16_ptr, sorted_lanes_ptr=sorted_lanes_ptr, out_q8_ptr=out_q8_ptr)
+    fn = entry("hipengine_gguf_q8_1_mmq_gather_ds4_pack_bf16", [VOID, VOID, VOID, I64, I64, I64, I64, VOID], library)
+    check_launch(fn(hidden_bf16_ptr, sorted_lanes_ptr, out_q8_ptr, rows, hidden, tokens, top_k, stream), runtime)
+
+
 def gguf_q8_1_d4s4_f32_quantize_bf16(x_ptr: int, xq_ptr: int, rows: int, hidden: int, *, stream: int = 0,
                                      library: ctypes.CDLL | None = None, runtime: HipRuntime | None = None) -> None:
     """bf16 ``[rows, hidden]`` -> ``[rows, hidden/128]`` 160-byte D4S4 blocks."""
@@ -70,6 +86,7 @@ def register_kernels(backend: str = "hip_gfx950", *, replace: bool = False) -> N
         ("q8_1", "f32", gguf_q4_k_quantize_f32_q8_1),
         ("q8_1", "bf16", gguf_q4_k_quantize_bf16_q8_1),
         ("q8_1_ds4", "bf16", gguf_q8_1_mmq_ds4_pack_bf16),
+        ("q8_1_ds4", "gather_bf16", gguf_q8_1_mmq_gather_ds4_pack_bf16),
         ("q8_1_d4s4_f32", "bf16", gguf_q8_1_d4s4_f32_quantize_bf16),
     ):
         register(KernelKey(backend, "activation_quant", quant, variant), fn, replace=replace)

@@ -76,6 +76,14 @@ int hipengine_gguf_q4_k_quantize_bf16_q8_1(const void* x, void* xq, int64_t rows
 int hipengine_gguf_q8_1_mmq_ds4_pack_bf16(const void* x, void* out, int64_t rows, int64_t hidden,
                                           hipengine_stream_t stream);
 
+/* The same pack of rows gathered through the routing index, in one pass: output row r (of `rows` packed lanes)
+ * is the pack of token sorted_lanes[r] / top_k of hidden_states [tokens, hidden]; a negative lane or a token
+ * outside the input packs as a row of zeros.  Bytes equal hipengine_qwen35_moe_gather_packed_hidden_lowp followed
+ * by the plain pack.  Replaces gguf_q4_k_q8_1_selected_prefill.hip:5596-5614 (kernel :705-772). */
+int hipengine_gguf_q8_1_mmq_gather_ds4_pack_bf16(const uint16_t* hidden_states, const int64_t* sorted_lanes,
+                                                 void* out, int64_t rows, int64_t hidden, int64_t tokens,
+                                                 int64_t top_k, hipengine_stream_t stream);
+
 /* bf16 [rows, hidden] -> 160-byte D4S4 blocks {float d4[4]; float s4[4]; int8 qs[128]}:
  * d = amax/127 (float32), q = clamp(roundf(x/d), -128, 127).  hidden % 128 == 0.
  * Replaces gguf_k_mmq_prefill.hip:2515-2540 (kernel :264-307). */
@@ -128,7 +136,16 @@ HIPENGINE_GFX950_DECLARE_FUSED_ALL(q8_0)
   int hipengine_gguf_##q##_dual_gemv_##a##_##o##_out(                                                    \
       const void* x, const uint8_t* qweight_a, const uint8_t* qweight_b, void* out_a, void* out_b,       \
       int64_t rows, int64_t in_features, int64_t out_features, int64_t threads, hipengine_stream_t stream);
+/* The "rowtile" names of the same (hipEngine's kernels for 2 to 8 rows that reuse a weight row across the batch;
+ * every batch here does): gguf_q4_k_gemv.hip:2496-2533, gguf_k_gemv.hip:5600-5617. */
+#define HIPENGINE_GFX950_DECLARE_ROWTILE(q, a, o)                                                        \
+  int hipengine_gguf_##q##_gemv_rowtile_##a##_##o##_out(                                                 \
+      const void* x, const uint8_t* qweight, void* out, int64_t rows, int64_t in_features,               \
+      int64_t out_features, int64_t threads, hipengine_stream_t stream);
 #define HIPENGINE_GFX950_DECLARE_DENSE_ALL(q) \
+  HIPENGINE_GFX950_DECLARE_ROWTILE(q, f32, f32) \
+  HIPENGINE_GFX950_DECLARE_ROWTILE(q, bf16, f32) \
+  HIPENGINE_GFX950_DECLARE_ROWTILE(q, bf16, bf16) \
   HIPENGINE_GFX950_DECLARE_DENSE(q, f32, f32) \
   HIPENGINE_GFX950_DECLARE_DENSE(q, f32, fp16) \
   HIPENGINE_GFX950_DECLARE_DENSE(q, fp16, f32) \

@@ -85,6 +85,29 @@ def test_dispatcher_keys_called_like_launch_raw(dev, quant, act, out):
     dev.free(dw)
 
 
+@pytest.mark.parametrize("quant", ["gguf_q4_k", "gguf_q6_k", "gguf_q8_0"])
+def test_rowtile_keys_are_the_batch_launch(dev, quant):
+    """("linear", quant, "rowtile_<act>_<out>_out") (gguf_q4_k_gemv.py:1552-1554) for 2 to 8 rows: the bits of the
+    prefill_* key on the same input."""
+    k, n = 2048, 200
+    rng = np.random.default_rng(k)
+    w = O.random_weight(QT[quant], n, k, seed=17)
+    dw = dev.put(w)
+    for rows, act, out in ((2, "f32", "f32"), (4, "bf16", "f32"), (8, "bf16", "bf16")):
+        xin, _ = _act(rng.standard_normal((rows, k)).astype(np.float32), act)
+        dx = dev.put(xin)
+        got = []
+        for family in ("rowtile", "prefill"):
+            dout = dev.empty(rows * n * (4 if out == "f32" else 2))
+            _resolve("linear", quant, f"{family}_{act}_{out}_out")(dx.ptr, dw.ptr, dout.ptr, rows, k, n, stream=0,
+                                                                   runtime=dev.runtime, threads=128, library=dev.library)
+            got.append(dev.get(dout, np.float32 if out == "f32" else np.uint16, (rows, n)))
+            dev.free(dout)
+        dev.free(dx)
+        assert np.array_equal(got[0].view(np.uint8), got[1].view(np.uint8))
+    dev.free(dw)
+
+
 @pytest.mark.parametrize("quant,n", [("gguf_q4_k", 352), ("gguf_q6_k", 333), ("gguf_q5_k", 160)])
 def test_prefill_key_with_workspace_runs_the_mmq(dev, quant, n):
     """prefill_bf16_f32_out with 32 rows or more and a caller-owned workspace packs the activations and runs the

@@ -48,6 +48,32 @@ def test_ds4_and_d4s4_pack_bytes(dev, rows, k):
     dev.free(dx)
 
 
+@pytest.mark.parametrize("tokens,top_k,k", [(1, 8, 2048), (7, 4, 512), (40, 2, 1280)])
+def test_gather_ds4_pack_bytes(dev, tokens, top_k, k):
+    """gguf_q8_1_mmq_gather_ds4_pack_bf16: the bytes of a row gather through sorted_lanes followed by the plain DS4
+    pack; lanes that are negative or name a token outside the input pack as rows of zeros (scale 0, sum 0)."""
+    xb = _bf16_rows(tokens + k, tokens, k)
+    lanes = tokens * top_k
+    rng = np.random.default_rng(lanes)
+    sorted_lanes = rng.permutation(lanes).astype(np.int64)
+    if lanes > 4:
+        sorted_lanes[1] = -1
+        sorted_lanes[3] = lanes + 5
+    src = sorted_lanes // top_k
+    gathered = np.zeros((lanes, k), dtype=np.uint16)
+    ok = (sorted_lanes >= 0) & (src < tokens)
+    gathered[ok] = xb[src[ok]]
+    want = O.pack_q8_1_ds4(gathered)
+    dx, dl = dev.put(xb), dev.put(sorted_lanes)
+    dq = dev.empty(lanes * (k // 128) * 144)
+    Q.gguf_q8_1_mmq_gather_ds4_pack_bf16(dx.ptr, dl.ptr, dq.ptr, lanes, k, tokens, top_k)
+    got = dev.get(dq, np.uint8, want.shape)
+    dev.free(dx, dl, dq)
+    assert np.array_equal(got, want)
+    with pytest.raises(ValueError):
+        Q.gguf_q8_1_mmq_gather_ds4_pack_bf16(1, 1, 1, lanes, k + 64, tokens, top_k)
+
+
 def _run_q4(dev, fn, ds4, w, rows, k, n, out_dtype=np.float32):
     dxq, dw = dev.put(ds4), dev.put(w)
     dout = dev.empty(rows * n * np.dtype(out_dtype).itemsize)
