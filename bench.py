@@ -1,7 +1,7 @@
 #!/usr/bin/env python3
 """Benchmark of the gfx950 GGUF k-quant matmul path on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-extra] [--no-cpu] [--pmc-pass [--pmc-shape quant,rows,K,N | mmq,quant,M,K,N]]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-extra] [--no-cpu] [--pmc-pass [--pmc-shape quant,rows,K,N | mmq,quant,M,K,N | moe,T]]
 
 One "step" is one pass of the hot path over one batch of synthetic input: the
 fused q8_1 decode GEMV of a Q4_K 17408x5120 weight at batch 1 (the shape the
@@ -411,7 +411,8 @@ def main() -> None:
                     help="hardware-counter pass: a 256 MiB calibration copy, then the headline kernel only")
     ap.add_argument("--pmc-shape", default="",
                     help="with --pmc-pass: launch this GEMV case instead of the headline one, as quant,rows,K,N "
-                         "(e.g. q6_k,8,5120,151936), or an MMQ prefill GEMM as mmq,quant,M,K,N (e.g. mmq,q4_k,2048,5120,17408)")
+                         "(e.g. q6_k,8,5120,151936), or an MMQ prefill GEMM as mmq,quant,M,K,N (e.g. mmq,q4_k,2048,5120,17408), "
+                         "or the selected-expert FFN chain of T tokens as moe,T")
     args = ap.parse_args()
     if args.gpus != 1:
         raise SystemExit("bench.py measures one GPU: this path is single-GPU (run with --gpus 1)")
@@ -429,6 +430,12 @@ def main() -> None:
         for _ in range(3):
             copy_bytes(src.ptr, dst.ptr, nbytes)
         h.rt.device_synchronize()
+        if args.pmc_shape.startswith("moe,"):
+            tokens = int(args.pmc_shape.split(",")[1])
+            sec, touched, ops = h.moe_case(tokens, 4, 1)
+            print(json.dumps({"pmc_pass": True, "copy_bytes": nbytes, "moe_tokens": tokens, "expert_bytes": touched,
+                              "int8_ops": ops}))
+            return
         if args.pmc_shape.startswith("mmq,"):
             _, pq, pm, pk, pn = args.pmc_shape.split(",")
             sec, ops = h.mmq_case(pq, int(pm), int(pk), int(pn), 4, 1)
