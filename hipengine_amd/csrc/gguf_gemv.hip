@@ -661,6 +661,11 @@ extern "C" int hipengine_gfx950_gguf_pair_silu_gemv(int32_t ggml_type, const voi
     const int r = static_cast<int>(rows);
     const SlabPlan sl = default_slab_plan(ggml_type, r, in_features, out_features);
     if (sl.ok) {
+      // one launch where a workgroup's rows of both matrices fit its partial-sum buffer (up to 72 x 256 rows)
+      if (sl.rows_wg <= SLAB_PAIR_ROWS) {
+        return launch_gemv_slab(x, x_kind, qweight_gate, out, out_kind, r, in_features, out_features, sl, stream, nullptr,
+                                nullptr, nullptr, qweight_up);
+      }
       const int rc = launch_gemv_slab(x, x_kind, qweight_gate, out, out_kind, r, in_features, out_features, sl, stream);
       if (rc != static_cast<int>(hipSuccess)) return rc;
       return launch_gemv_slab(x, x_kind, qweight_up, out, out_kind, r, in_features, out_features, sl, stream, nullptr, out);

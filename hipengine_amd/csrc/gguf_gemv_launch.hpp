@@ -19,10 +19,11 @@ struct SlabPlan {
   int b, bpw, waves, two_block_waves, rows_wg;
   bool ok;
 };
+constexpr int SLAB_PAIR_ROWS = 72;   // rows per workgroup up to which the gate/up pair runs as one slab launch
 SlabPlan default_slab_plan(int qt, int rows, int64_t K, int64_t N);
 int launch_gemv_slab(const void* x, int x_kind, const uint8_t* w, void* out, int out_kind, int rows, int64_t K,
                      int64_t N, const SlabPlan& p, hipStream_t stream, const void* residual = nullptr,
-                     const void* gate = nullptr, int32_t* dots_out = nullptr);
+                     const void* gate = nullptr, int32_t* dots_out = nullptr, const uint8_t* w_up = nullptr);
 int slab_raise_lds_limits();
 
 // ---- phased slab form (int8 MFMA; batch 3..8) ----

@@ -7,6 +7,8 @@
 
 namespace hipengine_gfx950 {
 
+static_assert(SLAB_PAIR_ROWS == SLAB_MAX_PAIR_ROWS, "launcher and kernel agree on the pair limit");
+
 namespace {
 // ---- slab form (Q4_K on the int8 MFMA, one workgroup per CU, waves split K) ----
 
@@ -16,6 +18,13 @@ template <int B, int BPW, int XK>
 __global__ void __launch_bounds__(BPW == 1 ? 1024 : 768) gemv_slab_q4k_kernel(GemvSlabArgs a) {
   extern __shared__ __align__(16) uint8_t smem[];
   gemv_slab_q4k_workgroup<B, BPW, XK>(a, smem);
+}
+
+// gate and up in one launch: out = silu(round(gate.x)) * round(up.x)
+template <int B, int BPW, int XK>
+__global__ void __launch_bounds__(BPW == 1 ? 1024 : 768) gemv_slab_q4k_pair_kernel(GemvSlabArgs a) {
+  extern __shared__ __align__(16) uint8_t smem[];
+  gemv_slab_q4k_workgroup<B, BPW, XK, false, true>(a, smem);
 }
 
 template <int B, int BPW>
@@ -28,12 +37,16 @@ using SlabKernelFn = void (*)(GemvSlabArgs);
 struct SlabVariant {
   int b, bpw;
   SlabKernelFn by_kind[4];
+  SlabKernelFn pair_by_kind[4];   // batch buckets 4 and 8 (batch 1 and 2 pair on the stream form)
 };
-#define SLAB_VARIANT(B, BPW)                                                                            \
-  SlabVariant { B, BPW, {gemv_slab_q4k_kernel<B, BPW, KIND_F32>, gemv_slab_q4k_kernel<B, BPW, KIND_BF16>, \
-                         gemv_slab_q4k_kernel<B, BPW, KIND_F16>, gemv_slab_q4k_kernel<B, BPW, KIND_Q8_1>} }
+#define SLAB_KINDS(KERNEL, B, BPW) \
+  {KERNEL<B, BPW, KIND_F32>, KERNEL<B, BPW, KIND_BF16>, KERNEL<B, BPW, KIND_F16>, KERNEL<B, BPW, KIND_Q8_1>}
+#define SLAB_VARIANT(B, BPW) SlabVariant { B, BPW, SLAB_KINDS(gemv_slab_q4k_kernel, B, BPW), {nullptr, nullptr, nullptr, nullptr} }
+#define SLAB_VARIANT_PAIR(B, BPW) \
+  SlabVariant { B, BPW, SLAB_KINDS(gemv_slab_q4k_kernel, B, BPW), SLAB_KINDS(gemv_slab_q4k_pair_kernel, B, BPW) }
 const SlabVariant kSlab[] = {SLAB_VARIANT(1, 1), SLAB_VARIANT(1, 2), SLAB_VARIANT(2, 1), SLAB_VARIANT(2, 2),
-                       SLAB_VARIANT(4, 1), SLAB_VARIANT(4, 2), SLAB_VARIANT(8, 1), SLAB_VARIANT(8, 2)};
+                             SLAB_VARIANT_PAIR(4, 1), SLAB_VARIANT_PAIR(4, 2), SLAB_VARIANT_PAIR(8, 1),
+                             SLAB_VARIANT_PAIR(8, 2)};
 
 
 
@@ -58,7 +71,7 @@ SlabPlan default_slab_plan(int qt, int rows, int64_t K, int64_t N) {
 
 int launch_gemv_slab(const void* x, int x_kind, const uint8_t* w, void* out, int out_kind, int rows, int64_t K,
                      int64_t N, const SlabPlan& p, hipStream_t stream, const void* residual,
-                     const void* gate, int32_t* dots_out) {
+                     const void* gate, int32_t* dots_out, const uint8_t* w_up) {
   const int nb = static_cast<int>(K / QK_K);
   const SlabVariant* v = nullptr;
   for (const SlabVariant& c : kSlab)
@@ -75,10 +88,14 @@ int launch_gemv_slab(const void* x, int x_kind, const uint8_t* w, void* out, int
     const int rc = ensure_init();
     if (rc != static_cast<int>(hipSuccess)) return rc;
   }
+  // the pair kernels keep 2 x rows_wg partial sums per batch row, and take no other epilogue
+  if (w_up && (p.rows_wg > SLAB_MAX_PAIR_ROWS || residual || gate || dots_out || !v->pair_by_kind[x_kind])) {
+    return static_cast<int>(hipErrorInvalidValue);
+  }
   GemvSlabArgs a{x, w, out, x_kind, out_kind, rows, static_cast<int>(K), static_cast<int>(N), p.rows_wg, p.waves,
-                 p.two_block_waves, residual, gate, dots_out};
+                 p.two_block_waves, residual, gate, w_up, dots_out};
   const unsigned grid = static_cast<unsigned>((N + p.rows_wg - 1) / p.rows_wg);
-  SlabKernelFn fn = v->by_kind[x_kind];
+  SlabKernelFn fn = w_up ? v->pair_by_kind[x_kind] : v->by_kind[x_kind];
   if (dots_out) {   // verification: q8_1 activations, batch bucket 8, either block count
     if (x_kind != KIND_Q8_1 || p.b != 8) return static_cast<int>(hipErrorInvalidValue);
     fn = p.bpw == 1 ? gemv_slab_q4k_dump_kernel<8, 1> : gemv_slab_q4k_dump_kernel<8, 2>;
@@ -93,12 +110,13 @@ int launch_gemv_slab(const void* x, int x_kind, const uint8_t* w, void* out, int
 
 int slab_raise_lds_limits() {
   for (const SlabVariant& v : kSlab)
-    for (const auto fn : v.by_kind) {
-      if (!fn) continue;
-      const hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(fn), hipFuncAttributeMaxDynamicSharedMemorySize,
-                                               static_cast<int>(kMaxLds));
-      if (e != hipSuccess) return static_cast<int>(e);
-    }
+    for (const auto& fns : {v.by_kind, v.pair_by_kind})
+      for (int kind = 0; kind < 4; ++kind) {
+        if (!fns[kind]) continue;
+        const hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(fns[kind]),
+                                                 hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(kMaxLds));
+        if (e != hipSuccess) return static_cast<int>(e);
+      }
   return static_cast<int>(hipSuccess);
 }
 

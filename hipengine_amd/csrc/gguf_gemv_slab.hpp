@@ -62,10 +62,12 @@ struct GemvSlabArgs {
   int two_block_waves;   // waves 0..two_block_waves-1 own two K blocks each, the rest one
   const void* residual;   // null, or [rows, N] of the output type: out = round(projection) + residual
   const void* gate;       // null, or [rows, N] of the output type (may be `out` itself): out = silu(gate) * round(projection)
+  const uint8_t* w_up;    // pair kernels only: the second matrix (w is the gate), out = silu(round(gate.x)) * round(up.x)
   int32_t* dots_out;      // verification kernels only: int32 [rows, N, K/32], every sub-block dot as the MFMA returns it
 };
 
 constexpr int SLAB_MAX_ROWS = 96;
+constexpr int SLAB_MAX_PAIR_ROWS = 72;   // rows per workgroup and matrix of the pair kernels: 2 x 72 partial sums per batch row
 
 template <int BPW>
 constexpr int slab_row_pitch() { return BPW == 1 ? 144 : 304; }
@@ -83,14 +85,21 @@ inline size_t gemv_slab_lds_bytes(int b, int waves, int two_block_waves) {
 }
 
 // VERIFY: the verification instantiation, which also writes every int32 sub-block dot to a.dots_out.
-template <int B, int BPW, int XK, bool VERIFY = false>
+// PAIR: the workgroup walks its rows of the gate matrix (a.w), then the same rows of the up matrix (a.w_up), and
+// stores silu(round(gate)) * round(up): the arithmetic of a gate launch followed by an up launch with a.gate set,
+// in one launch (one staging of the activations, no round trip of the gate through memory).
+template <int B, int BPW, int XK, bool VERIFY = false, bool PAIR = false>
 __device__ __forceinline__ void gemv_slab_q4k_workgroup(const GemvSlabArgs& a, uint8_t* smem) {
+  static_assert(!(PAIR && VERIFY), "the verification kernel takes one matrix");
   constexpr int VB = B < 4 ? B : 4;                  // result registers in use per lane
   constexpr int NL = (32 * BPW * 9 + 63) / 64;       // 16-byte loads per lane and step
-  constexpr int MAX_STEPS = SLAB_MAX_ROWS / 32;
+  constexpr int NM = PAIR ? 2 : 1;                   // matrices
+  constexpr int STEPS_PER = SLAB_MAX_ROWS / 32;      // steps per matrix
+  constexpr int MAX_STEPS = NM * STEPS_PER;
+  constexpr int RED_ROWS = PAIR ? 2 * SLAB_MAX_PAIR_ROWS : SLAB_MAX_ROWS;   // partial sums per batch row
   constexpr int EARLY_TAIL_ROWS = 7;                 // a last step of at most this many rows is done first
   constexpr int NLT = (EARLY_TAIL_ROWS * BPW * 9 + 63) / 64;
-  static_assert(B * SLAB_MAX_ROWS * 4 <= 32 * slab_pitch(1), "partial sums must fit the weight piece");
+  static_assert(B * RED_ROWS * 4 <= 32 * slab_pitch(1), "partial sums must fit the weight piece");
   const int x_kind = XK >= 0 ? XK : a.x_kind;
 
   const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -111,7 +120,7 @@ __device__ __forceinline__ void gemv_slab_q4k_workgroup(const GemvSlabArgs& a, u
   const int rows_wg = min(a.rows_wg, a.N - r0);
   const int steps = (rows_wg + 31) >> 5;
   const int row_bytes = nb * Q4_K_BYTES;
-  const uint8_t* wbase = a.w + static_cast<int64_t>(r0) * row_bytes + kb0 * Q4_K_BYTES;
+  const int64_t wg_offset = static_cast<int64_t>(r0) * row_bytes + kb0 * Q4_K_BYTES;
 
   uint8_t* wq = smem + wave_off;
   float* rec = reinterpret_cast<float*>(wq + REC);   // [BPW*8 sub-blocks][xd[8], xd*qsum[8]]
@@ -173,36 +182,51 @@ __device__ __forceinline__ void gemv_slab_q4k_workgroup(const GemvSlabArgs& a, u
   // Buffer loads: a descriptor over this wave's K slice of the slab (the hardware returns
   // zeros past its end), a 32-bit lane offset and a scalar step offset: no 64-bit
   // address arithmetic per load.
+  const int slab_bytes = (rows_wg - 1) * row_bytes + blocks_w * Q4_K_BYTES;
   const __amdgpu_buffer_rsrc_t wrsrc = __builtin_amdgcn_make_buffer_rsrc(
-      const_cast<uint8_t*>(wbase), 0, (rows_wg - 1) * row_bytes + blocks_w * Q4_K_BYTES, 0x00020000);
-  auto issue = [&](int t, sl_u32x4 (&dst)[NL]) {
+      const_cast<uint8_t*>(a.w + wg_offset), 0, slab_bytes, 0x00020000);
+  // the pair kernels' second matrix (the same slab of rows of a.w_up)
+  const __amdgpu_buffer_rsrc_t wrsrc_up = __builtin_amdgcn_make_buffer_rsrc(
+      const_cast<uint8_t*>((PAIR ? a.w_up : a.w) + wg_offset), 0, slab_bytes, 0x00020000);
+  // step t of matrix m
+  auto issue = [&](int m, int t, sl_u32x4 (&dst)[NL]) {
     const int last = rows_wg - 32 * t - 1;           // >= 0 for t < steps
-    walk([&](int i, int row, int col16) {
-      dst[i] = __builtin_amdgcn_raw_buffer_load_b128(wrsrc, min(row, last) * row_bytes + col16, t * 32 * row_bytes, 0);
-    });
+    if (PAIR && m) {
+      walk([&](int i, int row, int col16) {
+        dst[i] = __builtin_amdgcn_raw_buffer_load_b128(wrsrc_up, min(row, last) * row_bytes + col16, t * 32 * row_bytes, 0);
+      });
+    } else {
+      walk([&](int i, int row, int col16) {
+        dst[i] = __builtin_amdgcn_raw_buffer_load_b128(wrsrc, min(row, last) * row_bytes + col16, t * 32 * row_bytes, 0);
+      });
+    }
   };
   // A short last step (N = 17408: 68 rows per slab = 32 + 32 + 4) is loaded up front into its own
   // few registers and computed first, while the first full step is still on its way; done
   // last, it would cost a whole step of MFMA and scale work with nothing left to overlap.
   const int tail_rows = rows_wg & 31;
   const bool early_tail = steps > 1 && tail_rows >= 1 && tail_rows <= EARLY_TAIL_ROWS;
-  sl_u32x4 tbuf[NLT];
+  sl_u32x4 tbuf[NM][NLT];
   if (early_tail) {
     walk([&](int i, int row, int col16) {
-      if (i < NLT)
-        tbuf[i] = __builtin_amdgcn_raw_buffer_load_b128(wrsrc, min(row, tail_rows - 1) * row_bytes + col16,
-                                                        (steps - 1) * 32 * row_bytes, 0);
+      if (i < NLT) {
+        tbuf[0][i] = __builtin_amdgcn_raw_buffer_load_b128(wrsrc, min(row, tail_rows - 1) * row_bytes + col16,
+                                                           (steps - 1) * 32 * row_bytes, 0);
+        if constexpr (PAIR)
+          tbuf[1][i] = __builtin_amdgcn_raw_buffer_load_b128(wrsrc_up, min(row, tail_rows - 1) * row_bytes + col16,
+                                                             (steps - 1) * 32 * row_bytes, 0);
+      }
     });
   }
   // batch 8 holds 64 registers of fetched activations: its first weight loads wait until half of
   // them are quantized (they are not needed before the staging is done)
-  if constexpr (B < 8) issue(0, buf);
+  if constexpr (B < 8) issue(0, 0, buf);
 
   // ---- quantize the slice into LDS
 #pragma unroll
   for (int p = 0; p < PASSES; ++p) {
     if constexpr (B >= 8) {
-      if (p == PASSES / 2) issue(0, buf);
+      if (p == PASSES / 2) issue(0, 0, buf);
     }
     if (p >= passes) continue;
     const int gid = p * 16 + quad;
@@ -249,7 +273,9 @@ __device__ __forceinline__ void gemv_slab_q4k_workgroup(const GemvSlabArgs& a, u
     __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
   };
 
-  auto compute = [&](int t) {
+  // `slot` = matrix * STEPS_PER + step: where the result is filed
+  auto compute = [&](int slot) {
+    const int t = slot;     // the verification kernel has one matrix
     float acc[VB];
 #pragma unroll
     for (int v = 0; v < VB; ++v) acc[v] = 0.0f;
@@ -315,45 +341,58 @@ __device__ __forceinline__ void gemv_slab_q4k_workgroup(const GemvSlabArgs& a, u
 #pragma unroll
     for (int u = 0; u < MAX_STEPS; ++u)
 #pragma unroll
-      for (int v = 0; v < VB; ++v) done[u][v] = (u == t) ? acc[v] : done[u][v];
+      for (int v = 0; v < VB; ++v) done[u][v] = (u == slot) ? acc[v] : done[u][v];
   };
 
+  // the full steps of the matrices in turn: q = matrix * full_steps + step
   const int full_steps = early_tail ? steps - 1 : steps;
+  const int nfull = NM * full_steps;
 #pragma unroll 1
-  for (int t = early_tail ? -1 : 0; t < full_steps; ++t) {
-    if (t < 0) {
+  for (int q = early_tail ? -NM : 0; q < nfull; ++q) {
+    if (q < 0) {
+      const int mt = q + NM;     // the short last step of matrix mt
       walk([&](int i, int row, int col16) {
-        if (i < NLT) *reinterpret_cast<sl_u32x4*>(wq + row * PITCH + col16) = tbuf[i];   // rows 0..7
+        if (i < NLT) *reinterpret_cast<sl_u32x4*>(wq + row * PITCH + col16) = (PAIR && mt) ? tbuf[NM - 1][i] : tbuf[0][i];   // rows 0..7
       });
       __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
       __builtin_amdgcn_wave_barrier();
       __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
     } else {
       to_lds(buf);
-      if (t + 1 < full_steps) issue(t + 1, buf);
+      const int qn = q + 1;
+      if (qn < nfull) issue(qn >= full_steps, qn >= full_steps ? qn - full_steps : qn, buf);
     }
-    compute(t < 0 ? steps - 1 : t);
+    compute(q < 0 ? (q + NM) * STEPS_PER + steps - 1 : q >= full_steps ? STEPS_PER + q - full_steps : q);
   }
 
-  // ---- K-slice reduction: each wave's partial sums [batch row][SLAB_MAX_ROWS] replace its weight piece
+  // ---- K-slice reduction: each wave's partial sums [batch row][RED_ROWS] replace its weight piece
+  // (pair kernels: the rows of the up matrix follow the rows_wg rows of the gate matrix)
   float* red = reinterpret_cast<float*>(wq);
 #pragma unroll
-  for (int t = 0; t < MAX_STEPS; ++t) {
+  for (int u = 0; u < MAX_STEPS; ++u) {
 #pragma unroll
     for (int v = 0; v < VB; ++v) {
-      const int m = 4 * g + v, rl = 32 * t + n;
-      if (m < B && rl < rows_wg) red[m * SLAB_MAX_ROWS + rl] = done[t][v];
+      const int m = 4 * g + v, rl = 32 * (u % STEPS_PER) + n;
+      if (m < B && rl < rows_wg) red[m * RED_ROWS + (u / STEPS_PER) * rows_wg + rl] = done[u][v];
     }
   }
   __syncthreads();
   for (int idx = tid; idx < a.rows * rows_wg; idx += blockDim.x) {
     const int m = idx / rows_wg, rl = idx - m * rows_wg;
-    float v = 0.0f;
+    float v = 0.0f, v_up = 0.0f;
     for (int s = 0; s < a.waves; ++s) {
       const int off = s < t2 ? s * slab_wave_bytes(B, 2) : t2 * slab_wave_bytes(B, 2) + (s - t2) * slab_wave_bytes(B, 1);
-      v += reinterpret_cast<const float*>(smem + off)[m * SLAB_MAX_ROWS + rl];
+      v += reinterpret_cast<const float*>(smem + off)[m * RED_ROWS + rl];
+      if constexpr (PAIR) v_up += reinterpret_cast<const float*>(smem + off)[m * RED_ROWS + rows_wg + rl];
     }
     const int64_t oi = static_cast<int64_t>(m) * a.N + r0 + rl;
+    if constexpr (PAIR) {
+      // what the gate launch stores and the up launch reads back and applies (gguf_q4_k_gemv.hip:652-657)
+      const float gt = round_to_kind(v, a.out_kind);
+      const float sig = 1.0f / (1.0f + expf(-gt));
+      store_scalar(a.out, oi, gt * sig * round_to_kind(v_up, a.out_kind), a.out_kind);
+      continue;
+    }
     if (a.residual) v = round_to_kind(v, a.out_kind) + load_scalar(a.residual, oi, a.out_kind);
     if (a.gate) {   // the up half of a gate/up pair: the gate projection is already stored, rounded (gguf_q4_k_gemv.hip:652-657)
       const float gt = load_scalar(a.gate, oi, a.out_kind);

@@ -246,9 +246,11 @@ int hipengine_gfx950_gguf_multi_gemv(int32_t count, const int32_t* ggml_types, c
  * (runtime/qwen35_gguf_layer_ffn.py:519-538) falls back to the unfused sequence when no fused kernel
  * applies; so must a caller here when this returns 1).  rows <= 2: Q4_K, in_features >= 4096 and
  * out_features large enough for the stream form (a 27B FFN is), one launch.  rows 3..8: any of the four
- * types, two launches on the int8 MFMA forms - the gate projection is stored to `out` and the up
- * projection's epilogue reads it back, which is the round_mid arithmetic: a 16-bit out_kind needs
- * round_mid != 0.  New here. */
+ * types on the int8 MFMA forms, out = silu(round(gate)) * round(up) with both rounded to the output type
+ * (the round_mid arithmetic: a 16-bit out_kind needs round_mid != 0) - one launch for Q4_K with
+ * in_features <= 6144 and out_features <= 72 * 256 (a workgroup walks its rows of the gate matrix, then the
+ * same rows of the up matrix), else a gate launch that stores to `out` and an up launch whose epilogue reads
+ * it back; both give the same bits.  New here. */
 int hipengine_gfx950_gguf_pair_silu_gemv(int32_t ggml_type, const void* x, int32_t x_kind, const uint8_t* qweight_gate,
                                          const uint8_t* qweight_up, void* out, int32_t out_kind, int64_t rows,
                                          int64_t in_features, int64_t out_features, int32_t round_mid,

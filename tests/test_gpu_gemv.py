@@ -452,14 +452,14 @@ def test_pair_silu_gemv(dev, rows, kind, round_mid):
 
 
 @pytest.mark.parametrize("quant,rows,k,n,kind,round_mid", [
-    ("gguf_q4_k", 8, 5120, 600, "bf16", True),      # slab form, gate stored then read by the up launch
+    ("gguf_q4_k", 8, 5120, 600, "bf16", True),      # slab form, gate and up in one launch
     ("gguf_q4_k", 4, 5120, 300, "f32", False),
     ("gguf_q6_k", 5, 5120, 300, "bf16", True),      # phased slab, one phase
     ("gguf_q4_k", 8, 17408, 200, "f32", False),     # phased slab, several phases
 ])
 def test_pair_silu_gemv_batch_3_to_8(dev, quant, rows, k, n, kind, round_mid):
-    """Gate/up pair at batch 3..8: two launches on the MFMA forms, out = silu(stored gate) * round(up), against
-    the unfused kernels' own gate and up outputs."""
+    """Gate/up pair at batch 3..8 on the MFMA forms (one launch on the Q4_K slab form, gate launch then up launch
+    elsewhere): out = silu(round(gate)) * round(up), against the unfused kernels' own gate and up outputs."""
     rng = np.random.default_rng(15 + rows + n)
     x = rng.standard_normal((rows, k)).astype(np.float32)
     if kind == "bf16":
@@ -486,6 +486,44 @@ def test_pair_silu_gemv_batch_3_to_8(dev, quant, rows, k, n, kind, round_mid):
     if kind != "f32":
         with pytest.raises(G.FusedFormUnavailable):
             G.gguf_pair_silu_gemv(quant, 16, kind, 16, 16, 16, kind, rows, k, n, round_mid=False)
+
+
+@pytest.mark.parametrize("rows,k,n,kind", [
+    (8, 5120, 17408, "f32"),      # 68 rows per workgroup and matrix: two full steps and an early 4-row step, twice
+    (3, 2048, 10240, "bf16"),     # one block per wave; 40 rows: a full step and a step of 8
+    (5, 5120, 8960, "f32"),       # 35 rows: one full step, an early step of 3
+    (8, 4096, 18432, "bf16"),     # 72 rows: the most a pair launch takes
+    (4, 5120, 18500, "f32"),      # 73 rows: past it, gate launch then up launch
+    (6, 5120, 700, "bf16"),       # ragged last workgroup
+])
+def test_pair_silu_gemv_slab_one_launch(dev, rows, k, n, kind):
+    """The Q4_K gate/up pair at batch 3..8 as ONE slab launch (a workgroup walks its rows of the gate matrix, then
+    the same rows of the up matrix): out = silu(round(gate)) * round(up) against the single-matrix launches' own
+    gate and up outputs, over the step shapes of the slab (full steps, early short steps, ragged ends)."""
+    from hipengine_amd.synthetic import synthetic_blocks
+
+    rng = np.random.default_rng(rows * 1000 + n)
+    x = (rng.standard_normal((rows, k)) * 0.5).astype(np.float32)
+    wg = synthetic_blocks(O.GGML_Q4_K, n, k, seed=31)
+    wu = synthetic_blocks(O.GGML_Q4_K, n, k, seed=32)
+    xin = x if kind == "f32" else O.f32_to_bf16_bits(x)
+    dx, dg, du = dev.put(xin), dev.put(wg), dev.put(wu)
+    esz = 4 if kind == "f32" else 2
+    dout, dgate, dup = dev.empty(rows * n * esz, fill=0x7B), dev.empty(rows * n * esz), dev.empty(rows * n * esz)
+    G.gguf_pair_silu_gemv("gguf_q4_k", dx.ptr, kind, dg.ptr, du.ptr, dout.ptr, kind, rows, k, n, round_mid=True)
+    G.FUSED[("q4_k", kind, kind)](dx.ptr, dg.ptr, dgate.ptr, rows, k, n)
+    G.FUSED[("q4_k", kind, kind)](dx.ptr, du.ptr, dup.ptr, rows, k, n)
+    dt = np.float32 if kind == "f32" else np.uint16
+    got, gate, up = (dev.get(b, dt, (rows, n)) for b in (dout, dgate, dup))
+    dev.free(dx, dg, du, dout, dgate, dup)
+    if kind == "bf16":
+        got, gate, up = (O.bf16_bits_to_f32(a) for a in (got, gate, up))
+    want = (O.silu(gate) * up).astype(np.float32)
+    assert np.all(np.isfinite(got))
+    # the device's expf and the final rounding to the output type are the only differences
+    tol = 2.0 ** -7 if kind == "bf16" else 1e-5
+    assert np.max(np.abs(got - want)) <= tol * max(1.0, float(np.max(np.abs(want))))
+    assert O.cosine(got, want) >= 0.99999
 
 
 @pytest.mark.parametrize("quant,rows,k,n,kind", [("gguf_q6_k", 1, 17408, 5120, "bf16"), ("gguf_q4_k", 2, 4096, 4096, "bf16"),
