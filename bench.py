@@ -507,7 +507,7 @@ def main() -> None:
 
         ev_f, ev_u, wbytes = h.ffn_case(8, steps, max(5, args.warmup // 5))
         extra["ffn_27b_b8_pair_silu_and_down_residual"] = {
-            "us": round(ev_f * 1e6, 1), "launches": 3, "GB/s": round(wbytes / ev_f / 1e9, 1),
+            "us": round(ev_f * 1e6, 1), "launches": 2, "GB/s": round(wbytes / ev_f / 1e9, 1),
             "frac_hbm": round(wbytes / ev_f / 1e9 / HBM_PEAK_GBS, 4),
             "unfused_3_gemv_us": round(ev_u * 1e6, 1)}
 
@@ -516,6 +516,12 @@ def main() -> None:
             "eager_us_per_layer": round(eager * 1e6, 1), "hip_graph_us_per_layer": round(replay * 1e6, 1),
             "GB/s_graph": round(lbytes / replay / 1e9, 1), "frac_hbm_graph": round(lbytes / replay / 1e9 / HBM_PEAK_GBS, 4),
             "tok_per_s_64_layers_matmuls_only_graph": round(1.0 / (64 * replay), 1)}
+
+        eager, replay, lbytes = h.layer_graph_case(8, max(10, steps // 8), 3)
+        extra["layer_27b_b8_fused_4_launches"] = {
+            "eager_us_per_layer": round(eager * 1e6, 1), "hip_graph_us_per_layer": round(replay * 1e6, 1),
+            "GB/s_graph": round(lbytes / replay / 1e9, 1), "frac_hbm_graph": round(lbytes / replay / 1e9 / HBM_PEAK_GBS, 4),
+            "tok_per_s_64_layers_matmuls_only_graph": round(8.0 / (64 * replay), 1)}
 
         msteps = max(5, args.steps // 50)
         for name, (quant, m, kk, nn) in {

@@ -330,7 +330,8 @@ DEFINE_FUSED_ALL(q8_0, GGML_Q8_0)
 
 // Two matrices over one activation (gate and up, or k and v): out_a = W_a x, out_b = W_b x
 // (gguf_k_gemv.hip:5546-5560; Q4_K has the form for its pack8 layout only, gguf_q4_k_gemv.hip:2970).
-// One launch of the stream form where it applies (rows <= 2), else one launch per matrix.
+// One launch of the stream form where it applies (rows <= 2) or of the Q4_K slab form (rows 3..8), else one
+// launch per matrix.
 int launch_dual(int qt, const void* x, int x_kind, const uint8_t* w_a, const uint8_t* w_b, void* out_a, void* out_b,
                 int out_kind, int64_t rows, int64_t K, int64_t N, hipStream_t stream) {
   if (!x || !w_a || !w_b || !out_a || !out_b || rows <= 0 || K <= 0 || N <= 0 || (K % QK_K) != 0) {
@@ -342,6 +343,17 @@ int launch_dual(int qt, const void* x, int x_kind, const uint8_t* w_a, const uin
       StreamFusion f;
       f.fuse = FUSE_DUAL; f.w_up = w_b; f.out_b = out_b;
       return launch_gemv_stream(qt, x, x_kind, w_a, out_a, out_kind, static_cast<int>(rows), K, N, sp, stream, f);
+    }
+  }
+  if (rows >= 3 && rows <= 8 && qt == GGML_Q4_K) {   // both on the slab form: one launch of it
+    int chunk = static_cast<int>(rows);
+    const int q2[2] = {qt, qt};
+    const int64_t n2[2] = {N, N};
+    if (pick_form(qt, chunk, K, N, w_a) == FORM_SLAB && chunk == rows &&
+        slab_multi_ok(2, q2, static_cast<int>(rows), K, n2)) {
+      const uint8_t* const w2[2] = {w_a, w_b};
+      void* const o2[2] = {out_a, out_b};
+      return launch_gemv_slab_multi(2, x, x_kind, w2, o2, out_kind, static_cast<int>(rows), K, n2, stream);
     }
   }
   const int rc = launch_gemv(qt, x, x_kind, w_a, out_a, out_kind, rows, K, N, nullptr, stream);
@@ -634,7 +646,33 @@ extern "C" int hipengine_gfx950_gguf_multi_gemv(int32_t count, const int32_t* gg
     return launch_gemv_stream_multi(count, qt, x, x_kind, qweights, outs, out_kind, static_cast<int>(rows), in_features,
                                     out_features, stream);
   }
+  // batch 3..8: the Q4_K matrices that take the slab form share one launch of it, the others go one by one
+  bool done[4] = {false, false, false, false};
+  if (rows >= 3 && rows <= 8) {
+    int sq[4];
+    const uint8_t* sw[4];
+    void* so[4];
+    int64_t sn[4];
+    int picked = 0;
+    for (int i = 0; i < count; ++i) {
+      int chunk = static_cast<int>(rows);
+      if (qt[i] == GGML_Q4_K && pick_form(qt[i], chunk, in_features, out_features[i], qweights[i]) == FORM_SLAB &&
+          chunk == rows) {
+        sq[picked] = qt[i]; sw[picked] = qweights[i]; so[picked] = outs[i]; sn[picked] = out_features[i];
+        ++picked;
+      }
+    }
+    if (picked >= 2 && slab_multi_ok(picked, sq, static_cast<int>(rows), in_features, sn)) {
+      const int rc = launch_gemv_slab_multi(picked, x, x_kind, sw, so, out_kind, static_cast<int>(rows), in_features, sn,
+                                            stream);
+      if (rc != static_cast<int>(hipSuccess)) return rc;
+      for (int i = 0; i < count; ++i) {
+        for (int j = 0; j < picked; ++j) done[i] = done[i] || (so[j] == outs[i]);
+      }
+    }
+  }
   for (int i = 0; i < count; ++i) {
+    if (done[i]) continue;
     const int rc = launch_gemv(qt[i], x, x_kind, qweights[i], outs[i], out_kind, rows, in_features, out_features[i],
                                nullptr, stream);
     if (rc != static_cast<int>(hipSuccess)) return rc;

@@ -24,6 +24,9 @@ SlabPlan default_slab_plan(int qt, int rows, int64_t K, int64_t N);
 int launch_gemv_slab(const void* x, int x_kind, const uint8_t* w, void* out, int out_kind, int rows, int64_t K,
                      int64_t N, const SlabPlan& p, hipStream_t stream, const void* residual = nullptr,
                      const void* gate = nullptr, int32_t* dots_out = nullptr, const uint8_t* w_up = nullptr);
+bool slab_multi_ok(int count, const int* qt, int rows, int64_t K, const int64_t* N);
+int launch_gemv_slab_multi(int count, const void* x, int x_kind, const uint8_t* const* w, void* const* out, int out_kind,
+                           int rows, int64_t K, const int64_t* N, hipStream_t stream);
 int slab_raise_lds_limits();
 
 // ---- phased slab form (int8 MFMA; batch 3..8) ----

@@ -17,33 +17,48 @@ namespace {
 template <int B, int BPW, int XK>
 __global__ void __launch_bounds__(BPW == 1 ? 1024 : 768) gemv_slab_q4k_kernel(GemvSlabArgs a) {
   extern __shared__ __align__(16) uint8_t smem[];
-  gemv_slab_q4k_workgroup<B, BPW, XK>(a, smem);
+  gemv_slab_q4k_workgroup<B, BPW, XK>(a, smem, blockIdx.x);
+}
+
+// several matrices over one activation (q | k, k | v, ...): every workgroup runs the single-matrix body on its matrix
+template <int B, int BPW, int XK>
+__global__ void __launch_bounds__(BPW == 1 ? 1024 : 768) gemv_slab_q4k_multi_kernel(GemvSlabMultiArgs m) {
+  extern __shared__ __align__(16) uint8_t smem[];
+  const int wg = blockIdx.x;
+  int i = 0;
+  while (i + 1 < m.count && wg >= m.wg_end[i]) ++i;
+  gemv_slab_q4k_workgroup<B, BPW, XK>(m.sub[i], smem, wg - (i ? m.wg_end[i - 1] : 0));
 }
 
 // gate and up in one launch: out = silu(round(gate.x)) * round(up.x)
 template <int B, int BPW, int XK>
 __global__ void __launch_bounds__(BPW == 1 ? 1024 : 768) gemv_slab_q4k_pair_kernel(GemvSlabArgs a) {
   extern __shared__ __align__(16) uint8_t smem[];
-  gemv_slab_q4k_workgroup<B, BPW, XK, false, true>(a, smem);
+  gemv_slab_q4k_workgroup<B, BPW, XK, false, true>(a, smem, blockIdx.x);
 }
 
 template <int B, int BPW>
 __global__ void __launch_bounds__(BPW == 1 ? 1024 : 768) gemv_slab_q4k_dump_kernel(GemvSlabArgs a) {
   extern __shared__ __align__(16) uint8_t smem[];
-  gemv_slab_q4k_workgroup<B, BPW, KIND_Q8_1, true>(a, smem);
+  gemv_slab_q4k_workgroup<B, BPW, KIND_Q8_1, true>(a, smem, blockIdx.x);
 }
 
 using SlabKernelFn = void (*)(GemvSlabArgs);
+using SlabMultiKernelFn = void (*)(GemvSlabMultiArgs);
 struct SlabVariant {
   int b, bpw;
   SlabKernelFn by_kind[4];
-  SlabKernelFn pair_by_kind[4];   // batch buckets 4 and 8 (batch 1 and 2 pair on the stream form)
+  SlabKernelFn pair_by_kind[4];         // batch buckets 4 and 8 (batch 1 and 2 pair on the stream form)
+  SlabMultiKernelFn multi_by_kind[4];   // batch buckets 4 and 8 (batch 1 and 2 share a launch of the stream form)
 };
 #define SLAB_KINDS(KERNEL, B, BPW) \
   {KERNEL<B, BPW, KIND_F32>, KERNEL<B, BPW, KIND_BF16>, KERNEL<B, BPW, KIND_F16>, KERNEL<B, BPW, KIND_Q8_1>}
-#define SLAB_VARIANT(B, BPW) SlabVariant { B, BPW, SLAB_KINDS(gemv_slab_q4k_kernel, B, BPW), {nullptr, nullptr, nullptr, nullptr} }
-#define SLAB_VARIANT_PAIR(B, BPW) \
-  SlabVariant { B, BPW, SLAB_KINDS(gemv_slab_q4k_kernel, B, BPW), SLAB_KINDS(gemv_slab_q4k_pair_kernel, B, BPW) }
+#define SLAB_VARIANT(B, BPW)                                                                             \
+  SlabVariant { B, BPW, SLAB_KINDS(gemv_slab_q4k_kernel, B, BPW), {nullptr, nullptr, nullptr, nullptr}, \
+                {nullptr, nullptr, nullptr, nullptr} }
+#define SLAB_VARIANT_PAIR(B, BPW)                                                                               \
+  SlabVariant { B, BPW, SLAB_KINDS(gemv_slab_q4k_kernel, B, BPW), SLAB_KINDS(gemv_slab_q4k_pair_kernel, B, BPW), \
+                SLAB_KINDS(gemv_slab_q4k_multi_kernel, B, BPW) }
 const SlabVariant kSlab[] = {SLAB_VARIANT(1, 1), SLAB_VARIANT(1, 2), SLAB_VARIANT(2, 1), SLAB_VARIANT(2, 2),
                              SLAB_VARIANT_PAIR(4, 1), SLAB_VARIANT_PAIR(4, 2), SLAB_VARIANT_PAIR(8, 1),
                              SLAB_VARIANT_PAIR(8, 2)};
@@ -108,6 +123,60 @@ int launch_gemv_slab(const void* x, int x_kind, const uint8_t* w, void* out, int
 }
 
 
+// Up to four Q4_K matrices over one activation (batch 3..8) in one launch: the 256 workgroups are shared out in
+// proportion to the matrices' rows, every matrix with its own rows per workgroup.
+bool slab_multi_ok(int count, const int* qt, int rows, int64_t K, const int64_t* N) {
+  if (count < 2 || count > SLAB_MAX_MATRICES || rows < 3 || rows > 8) return false;
+  int64_t total = 0;
+  for (int i = 0; i < count; ++i) {
+    if (qt[i] != GGML_Q4_K || !default_slab_plan(qt[i], rows, K, N[i]).ok) return false;
+    total += N[i];
+  }
+  // every matrix needs a workgroup, and no workgroup more than SLAB_MAX_ROWS rows (checked again by the launcher)
+  return total <= static_cast<int64_t>(SLAB_MAX_ROWS) * (kComputeUnits - count);
+}
+
+int launch_gemv_slab_multi(int count, const void* x, int x_kind, const uint8_t* const* w, void* const* out, int out_kind,
+                           int rows, int64_t K, const int64_t* N, hipStream_t stream) {
+  if (count < 2 || count > SLAB_MAX_MATRICES || x_kind < KIND_F32 || x_kind > KIND_Q8_1) {
+    return static_cast<int>(hipErrorInvalidValue);
+  }
+  const SlabPlan p = default_slab_plan(GGML_Q4_K, rows, K, N[0]);
+  const SlabVariant* v = nullptr;
+  for (const SlabVariant& c : kSlab)
+    if (c.b == p.b && c.bpw == p.bpw) v = &c;
+  if (!p.ok || !v || !v->multi_by_kind[x_kind]) return static_cast<int>(hipErrorInvalidValue);
+  int64_t total = 0;
+  for (int i = 0; i < count; ++i) total += N[i];
+  GemvSlabMultiArgs m;
+  m.count = count;
+  int used = 0;
+  for (int i = 0; i < count; ++i) {
+    // a share of the CUs in proportion to the rows, at least one workgroup; the rows per workgroup follow
+    int64_t share = N[i] * kComputeUnits / total;      // rounded down: the shares stay within one round of workgroups
+    if (share < 1) share = 1;
+    int64_t rows_wg = (N[i] + share - 1) / share;
+    if (rows_wg > SLAB_MAX_ROWS) rows_wg = SLAB_MAX_ROWS;
+    const int64_t wgs = (N[i] + rows_wg - 1) / rows_wg;
+    if (!w[i] || !out[i] || N[i] <= 0 || N[i] > (1 << 30) || used + wgs > (1 << 20)) {
+      return static_cast<int>(hipErrorInvalidValue);
+    }
+    m.sub[i] = GemvSlabArgs{x, w[i], out[i], x_kind, out_kind, rows, static_cast<int>(K), static_cast<int>(N[i]),
+                            static_cast<int>(rows_wg), p.waves, p.two_block_waves, nullptr, nullptr, nullptr, nullptr};
+    used += static_cast<int>(wgs);
+    m.wg_end[i] = used;
+  }
+  for (int i = count; i < SLAB_MAX_MATRICES; ++i) { m.sub[i] = m.sub[0]; m.wg_end[i] = used; }
+  const size_t lds = gemv_slab_lds_bytes(p.b, p.waves, p.two_block_waves);
+  if (lds > 160 * 1024) return static_cast<int>(hipErrorInvalidValue);
+  if (lds > 64 * 1024) {
+    const int rc = ensure_init();
+    if (rc != static_cast<int>(hipSuccess)) return rc;
+  }
+  hipLaunchKernelGGL(v->multi_by_kind[x_kind], dim3(static_cast<unsigned>(used)), dim3(p.waves * 64), lds, stream, m);
+  return static_cast<int>(hipGetLastError());
+}
+
 int slab_raise_lds_limits() {
   for (const SlabVariant& v : kSlab)
     for (const auto& fns : {v.by_kind, v.pair_by_kind})
@@ -117,6 +186,13 @@ int slab_raise_lds_limits() {
                                                  hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(kMaxLds));
         if (e != hipSuccess) return static_cast<int>(e);
       }
+  for (const SlabVariant& v : kSlab)
+    for (const auto fn : v.multi_by_kind) {
+      if (!fn) continue;
+      const hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(fn), hipFuncAttributeMaxDynamicSharedMemorySize,
+                                               static_cast<int>(kMaxLds));
+      if (e != hipSuccess) return static_cast<int>(e);
+    }
   return static_cast<int>(hipSuccess);
 }
 

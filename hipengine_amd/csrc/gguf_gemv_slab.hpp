@@ -67,6 +67,15 @@ struct GemvSlabArgs {
 };
 
 constexpr int SLAB_MAX_ROWS = 96;
+constexpr int SLAB_MAX_MATRICES = 4;
+
+// Several matrices over one activation in one launch: workgroups [wg_end[i-1], wg_end[i]) take matrix i
+// (its own row count, rows per workgroup, weight and output; the same K, batch and layout).
+struct GemvSlabMultiArgs {
+  GemvSlabArgs sub[SLAB_MAX_MATRICES];
+  int wg_end[SLAB_MAX_MATRICES];
+  int count;
+};
 constexpr int SLAB_MAX_PAIR_ROWS = 72;   // rows per workgroup and matrix of the pair kernels: 2 x 72 partial sums per batch row
 
 template <int BPW>
@@ -88,8 +97,9 @@ inline size_t gemv_slab_lds_bytes(int b, int waves, int two_block_waves) {
 // PAIR: the workgroup walks its rows of the gate matrix (a.w), then the same rows of the up matrix (a.w_up), and
 // stores silu(round(gate)) * round(up): the arithmetic of a gate launch followed by an up launch with a.gate set,
 // in one launch (one staging of the activations, no round trip of the gate through memory).
+// `wg`: the workgroup's index among those of this matrix (the multi-matrix kernel hands every matrix a range).
 template <int B, int BPW, int XK, bool VERIFY = false, bool PAIR = false>
-__device__ __forceinline__ void gemv_slab_q4k_workgroup(const GemvSlabArgs& a, uint8_t* smem) {
+__device__ __forceinline__ void gemv_slab_q4k_workgroup(const GemvSlabArgs& a, uint8_t* smem, int wg) {
   static_assert(!(PAIR && VERIFY), "the verification kernel takes one matrix");
   constexpr int VB = B < 4 ? B : 4;                  // result registers in use per lane
   constexpr int NL = (32 * BPW * 9 + 63) / 64;       // 16-byte loads per lane and step
@@ -116,7 +126,7 @@ __device__ __forceinline__ void gemv_slab_q4k_workgroup(const GemvSlabArgs& a, u
   const int XQ = REC + blocks_w * 8 * 16 * 4;
   const int wave_off = wave < t2 ? wave * slab_wave_bytes(B, 2)
                                  : t2 * slab_wave_bytes(B, 2) + (wave - t2) * slab_wave_bytes(B, 1);
-  const int r0 = static_cast<int>(blockIdx.x) * a.rows_wg;
+  const int r0 = wg * a.rows_wg;
   const int rows_wg = min(a.rows_wg, a.N - r0);
   const int steps = (rows_wg + 31) >> 5;
   const int row_bytes = nb * Q4_K_BYTES;

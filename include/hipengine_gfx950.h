@@ -131,7 +131,8 @@ HIPENGINE_GFX950_DECLARE_FUSED_ALL(q8_0)
       const void* x, const uint8_t* qweight, void* out, int64_t rows, int64_t in_features,               \
       int64_t out_features, int64_t threads, hipengine_stream_t stream);
 /* Two matrices over one activation, out_a = W_a x and out_b = W_b x (k and v, gate and up): one launch for
- * rows <= 2 and in_features >= 4096, else one per matrix.  Replaces gguf_k_gemv.hip:5546-5560. */
+ * rows <= 2 and in_features >= 4096, and for Q4_K with in_features <= 6144 at rows 3..8, else one per matrix.
+ * Replaces gguf_k_gemv.hip:5546-5560. */
 #define HIPENGINE_GFX950_DECLARE_DENSE_DUAL(q, a, o)                                                     \
   int hipengine_gguf_##q##_dual_gemv_##a##_##o##_out(                                                    \
       const void* x, const uint8_t* qweight_a, const uint8_t* qweight_b, void* out_a, void* out_b,       \
@@ -231,7 +232,9 @@ int hipengine_gguf_q8_0_dp4a_triple_split_rowtile4_gemv_bf16_bf16_out(
  * host arrays of `count` entries, read before the call returns; x [rows, in_features] of x_kind, every out_i
  * [rows, out_features[i]] of out_kind.  rows <= 2 and in_features >= 4096: one launch, the workgroups divided
  * between the matrices in proportion to their bytes, each matrix computed in the stream form (the float32 sums
- * of its own call wherever that takes the stream form too); otherwise one launch per matrix.  hipEngine has the form for
+ * of its own call wherever that takes the stream form too).  rows 3..8: the Q4_K matrices with in_features <= 6144
+ * share one launch of the slab form (the 256 workgroups divided in proportion to their rows; the bits of their
+ * own calls), the others take a launch each.  Otherwise one launch per matrix.  hipEngine has the form for
  * two and three Q8_0 matrices (gguf_q8_0_dp4a_gemv.hip:100-340).  New here. */
 int hipengine_gfx950_gguf_multi_gemv(int32_t count, const int32_t* ggml_types, const void* x, int32_t x_kind,
                                      const uint8_t* const* qweights, void* const* outs, int32_t out_kind,

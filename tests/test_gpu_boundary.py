@@ -164,14 +164,15 @@ def test_dense_dual_gemv(dev, quant, rows):
     dev.free(dx, dwa, dwb, da, db, ds)
 
 
-@pytest.mark.parametrize("rows", [1, 2, 3])
+@pytest.mark.parametrize("rows", [1, 2, 3, 5, 8])
 @pytest.mark.parametrize("mats", [(("gguf_q4_k", 640), ("gguf_q4_k", 256), ("gguf_q6_k", 256)),
                                   (("gguf_q8_0", 130), ("gguf_q5_k", 1021)),
                                   (("gguf_q6_k", 96), ("gguf_q4_k", 64), ("gguf_q4_k", 32), ("gguf_q8_0", 7))],
                          ids=["qkv", "two_ragged", "four_small"])
 def test_multi_gemv_matches_the_single_calls_and_the_oracle(dev, rows, mats):
-    """Several matrices of mixed types and row counts over one activation: one launch at rows <= 2 (a launch per
-    matrix above); every output has the bits of its own fused GEMV call and meets the oracle's tolerance."""
+    """Several matrices of mixed types and row counts over one activation: one launch at rows <= 2; at rows 3..8 the
+    Q4_K matrices share one launch of the slab form and the others go one by one; every output has the bits of its
+    own fused GEMV call and meets the oracle's tolerance."""
     k = 5120
     rng = np.random.default_rng(31 + rows)
     x = rng.standard_normal((rows, k)).astype(np.float32)
@@ -197,6 +198,29 @@ def test_multi_gemv_matches_the_single_calls_and_the_oracle(dev, rows, mats):
             assert np.array_equal(got.view(np.uint32), alone.view(np.uint32)), (q, n)
         _close(got, O.gguf_quant_gemv(xq, w, QT[q]))
         _close(alone, O.gguf_quant_gemv(xq, w, QT[q]))
+    dev.free(dx, *dws, *outs, *single)
+
+
+@pytest.mark.parametrize("rows", [4, 8])
+def test_multi_gemv_attention_shapes_batch_3_to_8(dev, rows):
+    """q | k | v of a 27B-shape attention block (Q4_K 5120 and 1024 rows, Q6_K 1024 rows, K = 5120) at batch 4 and 8:
+    q and k share one slab launch (213 + 42 workgroups), v takes the phased slab; bits of the single calls."""
+    k = 5120
+    mats = (("gguf_q4_k", 5120), ("gguf_q4_k", 1024), ("gguf_q6_k", 1024))
+    rng = np.random.default_rng(77 + rows)
+    x = rng.standard_normal((rows, k)).astype(np.float32)
+    ws = [synthetic_blocks(QT[q], n, k, seed=50 + i) for i, (q, n) in enumerate(mats)]
+    fn = _resolve("linear", "gguf", "multi_gemv")
+    dx = dev.put(x)
+    dws = [dev.put(w) for w in ws]
+    outs = [dev.empty(rows * n * 4, fill=0x7C) for _, n in mats]
+    single = [dev.empty(rows * n * 4) for _, n in mats]
+    fn([q for q, _ in mats], dx.ptr, "f32", [d.ptr for d in dws], [o.ptr for o in outs], "f32", rows, k,
+       [n for _, n in mats], stream=0, runtime=dev.runtime)
+    for (q, n), dw, o, sgl in zip(mats, dws, outs, single):
+        G.FUSED[(q.removeprefix("gguf_"), "f32", "f32")](dx.ptr, dw.ptr, sgl.ptr, rows, k, n)
+        got, alone = dev.get(o, np.float32, (rows, n)).copy(), dev.get(sgl, np.float32, (rows, n))
+        assert np.array_equal(got.view(np.uint32), alone.view(np.uint32)), (q, n)
     dev.free(dx, *dws, *outs, *single)
 
 
