@@ -120,16 +120,35 @@ __global__ void __launch_bounds__(1024) moe_place_kernel(const int64_t* __restri
   const int count = static_cast<int>(expert_start[e + 1] - base);
   if (count <= 0) return;
   const int lane_id = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  constexpr int PER = 4;                        // consecutive lanes per thread and chunk
+  constexpr int64_t CHUNK = 1024 * PER;
   int running = 0, buf = 0;
-  // the selection of the next chunk is loaded before this chunk's barrier
-  int64_t sel_next = threadIdx.x < lanes ? selected[threadIdx.x] : -1;
-  for (int64_t chunk = 0; chunk < lanes && running < count; chunk += 1024, buf ^= 1) {
-    const int64_t lane = chunk + threadIdx.x;
-    const bool flag = lane < lanes && sel_next == e;
-    sel_next = lane + 1024 < lanes ? selected[lane + 1024] : -1;
-    const unsigned long long ballot = __ballot(flag);
-    const int before = __popcll(ballot & ((1ull << lane_id) - 1ull));
-    if (lane_id == 0) wave_cnt[buf][wave] = __popcll(ballot);
+  // the selections of the next chunk are loaded before this chunk's barrier
+  int64_t sel_next[PER];
+#pragma unroll
+  for (int j = 0; j < PER; ++j) {
+    const int64_t lane = static_cast<int64_t>(threadIdx.x) * PER + j;
+    sel_next[j] = lane < lanes ? selected[lane] : -1;
+  }
+  for (int64_t chunk = 0; chunk < lanes && running < count; chunk += CHUNK, buf ^= 1) {
+    const int64_t lane0 = chunk + static_cast<int64_t>(threadIdx.x) * PER;
+    bool flag[PER];
+    int mine = 0;
+#pragma unroll
+    for (int j = 0; j < PER; ++j) {
+      flag[j] = lane0 + j < lanes && sel_next[j] == e;
+      mine += flag[j] ? 1 : 0;
+      sel_next[j] = lane0 + CHUNK + j < lanes ? selected[lane0 + CHUNK + j] : -1;
+    }
+    // lanes of this expert in the threads before this one of the wave (ascending lane order: thread, then j)
+    int before = 0, wave_total = 0;
+#pragma unroll
+    for (int j = 0; j < PER; ++j) {
+      const unsigned long long ballot = __ballot(flag[j]);
+      before += __popcll(ballot & ((1ull << lane_id) - 1ull));
+      wave_total += __popcll(ballot);
+    }
+    if (lane_id == 0) wave_cnt[buf][wave] = wave_total;
     __syncthreads();      // one barrier per chunk: the count buffers alternate
     int offset = running, total = 0;
 #pragma unroll
@@ -138,12 +157,19 @@ __global__ void __launch_bounds__(1024) moe_place_kernel(const int64_t* __restri
       if (w < wave) offset += c;
       total += c;
     }
-    if (flag) {
-      const int64_t idx = base + offset + before;
-      sorted_lanes[idx] = lane;
-      if (sorted_experts) sorted_experts[idx] = e;
-      if (compact_to_source) compact_to_source[idx] = lane / top_k;
-      if (sorted_weights) sorted_weights[idx] = routing[lane];
+    if (mine) {
+      int64_t idx = base + offset + before;
+#pragma unroll
+      for (int j = 0; j < PER; ++j) {
+        if (flag[j]) {
+          const int64_t lane = lane0 + j;
+          sorted_lanes[idx] = lane;
+          if (sorted_experts) sorted_experts[idx] = e;
+          if (compact_to_source) compact_to_source[idx] = lane / top_k;
+          if (sorted_weights) sorted_weights[idx] = routing[lane];
+          ++idx;
+        }
+      }
     }
     running += total;
   }
