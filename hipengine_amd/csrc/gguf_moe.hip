@@ -37,7 +37,8 @@ constexpr int MAX_EXPERTS = 2048;
 __global__ void __launch_bounds__(1024) moe_count_prefix_kernel(const int64_t* __restrict__ selected,
                                                                 int64_t* __restrict__ expert_start,
                                                                 int64_t* __restrict__ active_experts,
-                                                                int64_t* __restrict__ active_count, int64_t lanes,
+                                                                int64_t* __restrict__ active_count,
+                                                                int64_t* __restrict__ lane_to_compact, int64_t lanes,
                                                                 int num_experts) {
   __shared__ int cnt[MAX_EXPERTS];
   __shared__ int act[MAX_EXPERTS];
@@ -53,8 +54,10 @@ __global__ void __launch_bounds__(1024) moe_count_prefix_kernel(const int64_t* _
       e[u] = i < lanes ? selected[i] : -1;
     }
 #pragma unroll
-    for (int u = 0; u < 8; ++u)
+    for (int u = 0; u < 8; ++u) {
       if (e[u] >= 0 && e[u] < num_experts) atomicAdd(&cnt[static_cast<int>(e[u])], 1);
+      else if (lane_to_compact && i0 + u * 1024 < lanes) lane_to_compact[i0 + u * 1024] = -1;   // a lane of no expert
+    }
   }
   __syncthreads();
   {
@@ -112,7 +115,8 @@ __global__ void __launch_bounds__(1024) moe_place_kernel(const int64_t* __restri
                                                          int64_t* __restrict__ sorted_lanes,
                                                          int64_t* __restrict__ sorted_experts,
                                                          int64_t* __restrict__ compact_to_source,
-                                                         float* __restrict__ sorted_weights, int64_t lanes,
+                                                         float* __restrict__ sorted_weights,
+                                                         int64_t* __restrict__ lane_to_compact, int64_t lanes,
                                                          int64_t top_k) {
   __shared__ int wave_cnt[2][16];
   const int64_t e = blockIdx.x;
@@ -167,6 +171,7 @@ __global__ void __launch_bounds__(1024) moe_place_kernel(const int64_t* __restri
           if (sorted_experts) sorted_experts[idx] = e;
           if (compact_to_source) compact_to_source[idx] = lane / top_k;
           if (sorted_weights) sorted_weights[idx] = routing[lane];
+          if (lane_to_compact) lane_to_compact[lane] = idx;
           ++idx;
         }
       }
@@ -177,15 +182,17 @@ __global__ void __launch_bounds__(1024) moe_place_kernel(const int64_t* __restri
 
 int launch_compact(const int64_t* selected, const float* routing, int64_t* expert_start, int64_t* active_experts,
                    int64_t* active_count, int64_t* sorted_lanes, int64_t* sorted_experts, int64_t* compact_to_source,
-                   float* sorted_weights, int64_t lanes, int64_t num_experts, int64_t top_k, hipStream_t stream) {
+                   float* sorted_weights, int64_t lanes, int64_t num_experts, int64_t top_k, hipStream_t stream,
+                   int64_t* lane_to_compact = nullptr) {
   if (!selected || !expert_start || !sorted_lanes || (sorted_weights && !routing) || lanes <= 0 || lanes > (1ll << 30) ||
       num_experts <= 0 || num_experts > MAX_EXPERTS || top_k <= 0) {
     return static_cast<int>(hipErrorInvalidValue);
   }
   hipLaunchKernelGGL(moe_count_prefix_kernel, dim3(1), dim3(1024), 0, stream, selected, expert_start, active_experts,
-                     active_count, lanes, static_cast<int>(num_experts));
+                     active_count, lane_to_compact, lanes, static_cast<int>(num_experts));
   hipLaunchKernelGGL(moe_place_kernel, dim3(static_cast<unsigned>(num_experts)), dim3(1024), 0, stream, selected, routing,
-                     expert_start, sorted_lanes, sorted_experts, compact_to_source, sorted_weights, lanes, top_k);
+                     expert_start, sorted_lanes, sorted_experts, compact_to_source, sorted_weights, lane_to_compact, lanes,
+                     top_k);
   return static_cast<int>(hipGetLastError());
 }
 
@@ -1050,6 +1057,18 @@ extern "C" int hipengine_qwen35_moe_group_compact_active_source_rows(
     int64_t total_lanes, int64_t num_experts, int64_t top_k, hipStream_t stream) {
   return launch_compact(selected_experts, routing_weights, expert_start, active_experts, active_count, sorted_lanes,
                         nullptr, compact_to_source, sorted_weights, total_lanes, num_experts, top_k, stream);
+}
+
+// The same index with the inverse (lane -> compact position, -1 for a lane of no expert) written by the same two
+// launches, instead of a fill and a scatter after them.
+extern "C" int hipengine_gfx950_moe_group_compact_index(
+    const int64_t* selected_experts, const float* routing_weights, int64_t* expert_start, int64_t* active_experts,
+    int64_t* active_count, int64_t* sorted_lanes, int64_t* compact_to_source, float* sorted_weights,
+    int64_t* lane_to_compact, int64_t total_lanes, int64_t num_experts, int64_t top_k, hipStream_t stream) {
+  if (!lane_to_compact) return static_cast<int>(hipErrorInvalidValue);
+  return launch_compact(selected_experts, routing_weights, expert_start, active_experts, active_count, sorted_lanes,
+                        nullptr, compact_to_source, sorted_weights, total_lanes, num_experts, top_k, stream,
+                        lane_to_compact);
 }
 
 extern "C" int hipengine_qwen35_moe_mmq32_tile_map(const int64_t* expert_start_compact, int64_t* mmq_expert_start,

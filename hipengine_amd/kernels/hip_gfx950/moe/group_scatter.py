@@ -60,6 +60,24 @@ def qwen35_moe_group_compact_active_source_rows(selected_experts_ptr: int, routi
                     stream), runtime)
 
 
+def moe_group_compact_index(selected_experts_ptr: int, routing_weights_ptr: int, expert_start_ptr: int,
+                            active_experts_ptr: int, active_count_ptr: int, sorted_lanes_ptr: int,
+                            compact_to_source_ptr: int, sorted_weights_ptr: int, lane_to_compact_ptr: int,
+                            total_lanes: int, num_experts: int, top_k: int, *, stream: int = 0,
+                            library: ctypes.CDLL | None = None, runtime: HipRuntime | None = None) -> None:
+    """``qwen35_moe_group_compact_active_source_rows`` and ``moe_lane_to_compact`` in the two launches of the former
+    (C symbol ``hipengine_gfx950_moe_group_compact_index``): the same arrays, bit for bit."""
+    _check_num_experts(num_experts)
+    if total_lanes <= 0 or top_k <= 0:
+        raise ValueError("total_lanes and top_k must be positive")
+    validate_pointers(selected_experts_ptr=selected_experts_ptr, expert_start_ptr=expert_start_ptr,
+                      sorted_lanes_ptr=sorted_lanes_ptr, lane_to_compact_ptr=lane_to_compact_ptr)
+    fn = entry("hipengine_gfx950_moe_group_compact_index", [VOID] * 9 + [I64, I64, I64, VOID], library)
+    check_launch(fn(selected_experts_ptr, routing_weights_ptr, expert_start_ptr, active_experts_ptr, active_count_ptr,
+                    sorted_lanes_ptr, compact_to_source_ptr, sorted_weights_ptr, lane_to_compact_ptr, total_lanes,
+                    num_experts, top_k, stream), runtime)
+
+
 def qwen35_moe_mmq32_tile_map(expert_start_compact_ptr: int, mmq_expert_start_ptr: int, tile_expert_ptr: int,
                               mmq_total_ptr: int, num_experts: int, *, tile_capacity: int = 0, stream: int = 0,
                               library: ctypes.CDLL | None = None, runtime: HipRuntime | None = None) -> None:

@@ -457,6 +457,15 @@ int hipengine_qwen35_moe_mmq32_tile_map(const int64_t* expert_start_compact, int
 int hipengine_gfx950_moe_lane_to_compact(const int64_t* sorted_lanes, int64_t* lane_to_compact, int64_t compact_rows,
                                          int64_t total_lanes, hipengine_stream_t stream);
 
+/* hipengine_qwen35_moe_group_compact_active_source_rows and hipengine_gfx950_moe_lane_to_compact in the two
+ * launches of the former: the placement writes lane_to_compact[lane] as it files the lane, the counting pass
+ * writes -1 for the lanes of no expert.  Same arrays, bit for bit.  New here. */
+int hipengine_gfx950_moe_group_compact_index(const int64_t* selected_experts, const float* routing_weights,
+                                             int64_t* expert_start, int64_t* active_experts, int64_t* active_count,
+                                             int64_t* sorted_lanes, int64_t* compact_to_source, float* sorted_weights,
+                                             int64_t* lane_to_compact, int64_t total_lanes, int64_t num_experts,
+                                             int64_t top_k, hipengine_stream_t stream);
+
 /* gate_up[rows, 2*inter] (gate columns first) -> out[rows, inter] = gate*sigmoid(gate)*up.
  * Kinds: 0 float32, 1 bf16, 2 fp16.  The step between the gate/up and the down
  * projection (fused/paro_silu silu_mul_separate_out_bf16 in hipEngine). */

@@ -76,6 +76,18 @@ def _device_index(dev, sel, w, num_experts, tile_capacity=0):
         GS.moe_lane_to_compact(d["sorted_lanes"].ptr, d["l2c"].ptr, total, lanes)
         host["l2c"] = dev.get(d["l2c"], np.int64, (lanes,))
     host["total"] = total
+    # the combined entry: the same index and the inverse in two launches
+    es2, sl2, c2s2, sw2 = dev.empty((num_experts + 1) * 8), dev.empty(lanes * 8, fill=0xFF), dev.empty(lanes * 8, fill=0xFF), dev.empty(lanes * 4, fill=0)
+    act2, actn2, l2c2 = dev.empty(num_experts * 8, fill=0xFF), dev.empty(8), dev.empty(lanes * 8, fill=0x22)
+    GS.moe_group_compact_index(d["sel"].ptr, d["w"].ptr, es2.ptr, act2.ptr, actn2.ptr, sl2.ptr, c2s2.ptr, sw2.ptr, l2c2.ptr,
+                               lanes, num_experts, top_k)
+    assert np.array_equal(dev.get(es2, np.int64, (num_experts + 1,)), host["expert_start"])
+    assert np.array_equal(dev.get(sl2, np.int64, (lanes,))[:total], host["sorted_lanes"][:total])
+    assert np.array_equal(dev.get(c2s2, np.int64, (lanes,))[:total], host["c2s"][:total])
+    assert np.array_equal(dev.get(sw2, np.float32, (lanes,))[:total].view(np.uint32), host["sorted_w"][:total].view(np.uint32))
+    if total > 0:
+        assert np.array_equal(dev.get(l2c2, np.int64, (lanes,)), host["l2c"])
+    dev.free(es2, sl2, c2s2, sw2, act2, actn2, l2c2)
     return host, d
 
 
