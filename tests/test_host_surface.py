@@ -273,7 +273,22 @@ def test_moe_wrappers_validate_before_touching_the_device():
     with pytest.raises(ValueError, match="x_rows \\* top_k"):
         M.gguf_selected_gemv("gguf_q4_k", M.SEL_DOWN_SUM, 1, 1, 1, 1, 2, 9, 4, 256, 32, routing_weights_ptr=1, top_k=4)
     with pytest.raises(ValueError, match="gguf_q4_k or gguf_q6_k"):
-        M.gguf_selected_gemv("gguf_q8_0", M.SEL_SINGLE, 1, 1, 1, 1, 1, 8, 4, 256, 32)
+        M.gguf_selected_gemv("gguf_q8_0", M.SEL_DUAL_SILU, 1, 1, 1, 1, 1, 8, 4, 256, 32, qweight_b_ptr=1)
+    single, silu = M.SELECTED_K["q6_k"]
+    with pytest.raises(ValueError, match="multiple of x_rows"):
+        single(1, 1, 1, 1, 3, 8, 4, 256, 32)
+    with pytest.raises(ValueError, match="non-null"):
+        silu(1, 0, 1, 1, 1, 8, 8, 4, 256, 32)
+    from hipengine_amd.kernels.hip_gfx950.quant import gguf_q8_1_gemv as G
+    with pytest.raises(TypeError, match="2 weight and 2 output pointers"):
+        G.gguf_q8_0_dp4a_dual_split_rowtile4_gemv_f32_f32_out(1, 1, 1, 1, 1, 4, 256, 8)
+    with pytest.raises(ValueError, match="divisible"):
+        G.gguf_q8_0_dp4a_triple_split_rowtile4_gemv_bf16_bf16_out(1, 1, 1, 1, 1, 1, 1, 4, 100, 8, 8, 8)
+    with pytest.raises(ValueError, match="hidden must be divisible"):
+        from hipengine_amd.kernels.hip_gfx950.quant import gguf_quantize as Q
+        Q.gguf_q8_1_mmq_gather_ds4_pack_bf16(1, 1, 1, 8, 192, 1, 8)
+    with pytest.raises(ValueError, match="num_experts"):
+        GS.moe_group_compact_index(1, 1, 1, 1, 1, 1, 1, 1, 1, 8, 4096, 8)
     with pytest.raises(ValueError, match="multiples of 32"):
         M.gguf_q4_k_grouped_mmq(1, 1, 1, 1, 1, 1, 8, 8, 256, 40, 4, 32)
     with pytest.raises(ValueError, match="multiple of 32"):
