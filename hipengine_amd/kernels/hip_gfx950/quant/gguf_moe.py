@@ -360,5 +360,5 @@ def register_kernels(backend: str = "hip_gfx950", *, replace: bool = False) -> N
                  (lambda q: lambda *a, **k: gguf_grouped_gemv(q, *a, **k))(_q), replace=replace)
     register(KernelKey(backend, "moe_linear", "gguf_q4_k", "grouped_mmq32_q8_1_ds4"), gguf_q4_k_grouped_mmq,
              replace=replace)
-    for quant in ("gguf_q4_k", "gguf_q6_k"):
+    for quant in ("gguf_q4_k", "gguf_q5_k", "gguf_q6_k", "gguf_q8_0"):     # Q5_K and Q8_0: the single form
         register(KernelKey(backend, "moe_linear", quant, "selected_gemv_q8_1"), gguf_selected_gemv, replace=replace)

@@ -148,13 +148,15 @@ def _ref_lane(x_row, w_e, qt):
     return O.gguf_quant_gemv(O.dequantize_q8_1(xq), w_e, qt)[0]
 
 
-@pytest.mark.parametrize("quant,qt", [("gguf_q4_k", O.GGML_Q4_K), ("gguf_q6_k", O.GGML_Q6_K)])
+@pytest.mark.parametrize("quant,qt", [("gguf_q4_k", O.GGML_Q4_K), ("gguf_q6_k", O.GGML_Q6_K), ("gguf_q5_k", O.GGML_Q5_K),
+                                      ("gguf_q8_0", O.GGML_Q8_0)])
 @pytest.mark.parametrize("tokens,top_k,experts,k,n", [(1, 8, 16, 2048, 512), (3, 4, 8, 512, 2048), (5, 2, 6, 1280, 80)])
 def test_selected_gemv_single(dev, quant, qt, tokens, top_k, experts, k, n):
     sel, _ = _routing(k + n, tokens, top_k, experts)
     if tokens > 1:
         sel[1, 0] = -1                                   # an invalid lane stays unwritten
-    w = _experts(qt, experts, n, k, seed=3)
+    w = (O.stack_experts(_random_q5_k(n, k, seed=3), experts, seed=3) if qt == O.GGML_Q5_K
+         else _experts(qt, experts, n, k, seed=3))
     x = np.random.default_rng(9).standard_normal((tokens, k)).astype(np.float32)
     lanes = tokens * top_k
     dx, dsel, dw = dev.put(x), dev.put(sel), dev.put(w)
