@@ -16,6 +16,7 @@
 
 #include "gguf_gemv.hpp"
 #include "gguf_mmq_q4k.hpp"
+#include "gguf_mmq_q6k.hpp"
 
 #include "gguf_init.hpp"
 
@@ -982,6 +983,106 @@ int launch_moe_mmq(const void* xq, const int64_t* compact_to_source, const int64
 }
 
 
+// --------------------------------------------------------------------------
+// prefill: expert-grouped Q6_K x D4S4 MMQ.  The tile engine of the dense GEMM over a map of 128-row tiles
+// (expert per tile, built by the tile-map kernel with tile_rows = 128), rows gathered through
+// compact_to_source; workgroup = (column tile of 64, row tile).
+// --------------------------------------------------------------------------
+
+struct MoeQ6Args {
+  const uint8_t* xq;                 // D4S4 blocks [source_rows, K/128]
+  const int64_t* compact_to_source;  // [compact_rows] or null (compact row i reads source row i)
+  const int64_t* expert_start_compact;
+  const int64_t* expert_start_tiles; // row starts rounded up to 128 per expert
+  const int64_t* tile_expert;        // [total_rows/128]
+  const uint8_t* w_a;
+  const uint8_t* w_b;
+  void* out;                         // [compact_rows, Na + Nb]
+  int out_kind;
+  int compact_rows, source_rows, K, Na, Nb, num_experts;
+  int64_t expert_stride_rows;
+  int tiles_a;
+};
+
+constexpr int MOE_Q6_COLS = 64;   // the 128-wide tile spills in this kernel (the row map on top of 243 registers)
+
+__global__ void __launch_bounds__(Q6_THREADS, 2) moe_mmq_q6_k_kernel(MoeQ6Args a) {
+  extern __shared__ __align__(16) uint8_t smem_raw[];
+  Q6Smem<MOE_Q6_COLS>& s = *reinterpret_cast<Q6Smem<MOE_Q6_COLS>*>(smem_raw);
+  int* src_row = reinterpret_cast<int*>(smem_raw + sizeof(Q6Smem<MOE_Q6_COLS>));
+
+  const int tile_row = blockIdx.y;
+  const int64_t e = a.tile_expert[tile_row];
+  if (e < 0 || e >= a.num_experts) return;
+  const bool use_b = static_cast<int>(blockIdx.x) >= a.tiles_a;
+  const int n0 = (use_b ? blockIdx.x - a.tiles_a : blockIdx.x) * MOE_Q6_COLS;
+  const int local_n = use_b ? a.Nb : a.Na;
+  const int64_t compact_base = a.expert_start_compact[e];
+  const int64_t count = a.expert_start_compact[e + 1] - compact_base;
+  const int64_t row0 = static_cast<int64_t>(tile_row) * Q6_BM - a.expert_start_tiles[e];
+  const int64_t remaining = count - row0;
+  if (row0 < 0 || remaining <= 0) return;
+  const int valid_rows = remaining >= Q6_BM ? Q6_BM : static_cast<int>(remaining);
+  const int64_t first_compact = compact_base + row0;
+  if (compact_base < 0 || first_compact + valid_rows > a.compact_rows) return;
+
+  const int steps = a.K / 128;
+  const int64_t w_row_bytes = static_cast<int64_t>(a.K / QK_K) * Q6_K_BYTES;
+  const int64_t x_row_bytes = static_cast<int64_t>(steps) * D4S4_BYTES;
+  const int64_t stride_rows = a.expert_stride_rows > 0 ? a.expert_stride_rows : local_n;
+  const uint8_t* w = (use_b ? a.w_b : a.w_a) + e * stride_rows * w_row_bytes;
+
+  if (threadIdx.x < Q6_BM) {
+    const int64_t crow = first_compact + min(static_cast<int>(threadIdx.x), valid_rows - 1);
+    int64_t src = a.compact_to_source ? a.compact_to_source[crow] : crow;
+    src = src < 0 ? 0 : (src >= a.source_rows ? a.source_rows - 1 : src);
+    src_row[threadIdx.x] = static_cast<int>(src);
+  }
+  __syncthreads();
+
+  const int64_t out_stride = static_cast<int64_t>(a.Na) + a.Nb;
+  const int col_base = (use_b ? a.Na : 0) + n0;
+  q6_tile_run<false, MOE_Q6_COLS>(
+      a.xq, x_row_bytes, w, w_row_bytes, steps, s,
+      [=](int row) { return static_cast<int64_t>(src_row[row]); },
+      [=](int col) { return static_cast<int64_t>(min(n0 + col, local_n - 1)); },
+      [=](int row, int col, float v) {
+        if (row < valid_rows && n0 + col < local_n)
+          store_scalar(a.out, (first_compact + row) * out_stride + col_base + col, v, a.out_kind);
+      });
+}
+
+int launch_moe_mmq_q6(const void* xq, const int64_t* compact_to_source, const int64_t* expert_start_compact,
+                      const int64_t* expert_start_tiles, const int64_t* tile_expert, const uint8_t* w_a,
+                      const uint8_t* w_b, void* out, int out_kind, int64_t compact_rows, int64_t source_rows, int64_t K,
+                      int64_t Na, int64_t Nb, int64_t num_experts, int64_t total_rows, int64_t expert_stride_rows,
+                      hipStream_t stream) {
+  if (!xq || !expert_start_compact || !expert_start_tiles || !tile_expert || !w_a || !out || compact_rows <= 0 ||
+      compact_rows > (1 << 24) || source_rows <= 0 || source_rows > (1 << 24) || K <= 0 || (K % QK_K) != 0 ||
+      Na <= 0 || Nb < 0 || (Nb > 0 && !w_b) || Na + Nb > (1 << 24) || num_experts <= 0 || total_rows <= 0 ||
+      (total_rows % Q6_BM) != 0 || total_rows / Q6_BM > 65535 || expert_stride_rows < 0 || out_kind < KIND_F32 ||
+      out_kind > KIND_F16) {
+    return static_cast<int>(hipErrorInvalidValue);
+  }
+  MoeQ6Args a;
+  a.xq = static_cast<const uint8_t*>(xq);
+  a.compact_to_source = compact_to_source;
+  a.expert_start_compact = expert_start_compact;
+  a.expert_start_tiles = expert_start_tiles;
+  a.tile_expert = tile_expert;
+  a.w_a = w_a; a.w_b = w_b; a.out = out; a.out_kind = out_kind;
+  a.compact_rows = static_cast<int>(compact_rows); a.source_rows = static_cast<int>(source_rows);
+  a.K = static_cast<int>(K); a.Na = static_cast<int>(Na); a.Nb = static_cast<int>(Nb);
+  a.num_experts = static_cast<int>(num_experts);
+  a.expert_stride_rows = expert_stride_rows;
+  a.tiles_a = static_cast<int>((Na + MOE_Q6_COLS - 1) / MOE_Q6_COLS);
+  const int tiles_b = static_cast<int>((Nb + MOE_Q6_COLS - 1) / MOE_Q6_COLS);
+  const dim3 grid(static_cast<unsigned>(a.tiles_a + tiles_b), static_cast<unsigned>(total_rows / Q6_BM));
+  hipLaunchKernelGGL(moe_mmq_q6_k_kernel, grid, dim3(Q6_THREADS), sizeof(Q6Smem<MOE_Q6_COLS>) + Q6_BM * sizeof(int),
+                     stream, a);
+  return static_cast<int>(hipGetLastError());
+}
+
 // ---- router: top-k experts of a row of logits and the softmax of their logits --------
 //
 // One wave per token.  Lane l keeps the logits of experts l, l+64, ... (up to 16 of them,
@@ -1323,6 +1424,32 @@ extern "C" int hipengine_gfx950_gguf_q4_k_grouped_mmq(const void* x_q8, const in
   return launch_moe_mmq(x_q8, compact_to_source, expert_start_compact, expert_start_mmq32, tile_expert, qweight_a,
                         qweight_b, out, out_kind, compact_rows, source_rows, in_features, out_features_a,
                         out_features_b, num_experts, mmq_total_rows, expert_stride_rows, stream);
+}
+
+// The expert-grouped MMQ for Q6_K expert weights over D4S4 activation blocks: out[compact row, :] =
+// [W_a[e] | W_b[e]] x, e the expert that owns the compact row.  The tile map is one of 128-row tiles
+// (hipengine_gfx950_moe_tile_map with tile_rows = 128): total_rows a multiple of 128.
+extern "C" int hipengine_gfx950_gguf_q6_k_grouped_mmq(const void* x_d4s4, const int64_t* compact_to_source,
+                                                      const int64_t* expert_start_compact,
+                                                      const int64_t* expert_start_tiles, const int64_t* tile_expert,
+                                                      const uint8_t* qweight_a, const uint8_t* qweight_b, void* out,
+                                                      int32_t out_kind, int64_t compact_rows, int64_t source_rows,
+                                                      int64_t in_features, int64_t out_features_a,
+                                                      int64_t out_features_b, int64_t num_experts,
+                                                      int64_t total_rows, int64_t expert_stride_rows,
+                                                      hipStream_t stream) {
+  return launch_moe_mmq_q6(x_d4s4, compact_to_source, expert_start_compact, expert_start_tiles, tile_expert, qweight_a,
+                           qweight_b, out, out_kind, compact_rows, source_rows, in_features, out_features_a,
+                           out_features_b, num_experts, total_rows, expert_stride_rows, stream);
+}
+
+// The tile map for tiles of any height (hipengine_qwen35_moe_mmq32_tile_map is the 32-row one).
+extern "C" int hipengine_gfx950_moe_tile_map(const int64_t* expert_start_compact, int64_t* tile_expert_start,
+                                             int64_t* tile_expert, int64_t* total_out, int64_t num_experts,
+                                             int64_t tile_capacity, int32_t tile_rows, hipStream_t stream) {
+  if (tile_rows != 32 && tile_rows != 64 && tile_rows != 128) return static_cast<int>(hipErrorInvalidValue);
+  return launch_tile_map(expert_start_compact, tile_expert_start, tile_expert, total_out, num_experts, tile_capacity,
+                         tile_rows, stream);
 }
 
 extern "C" int hipengine_qwen35_router_select(const float* logits, int64_t* selected, float* routing, int64_t tokens,

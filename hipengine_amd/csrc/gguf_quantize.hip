@@ -83,6 +83,31 @@ __device__ __forceinline__ void ds4_pack_group(const float (&v)[4], float amax, 
   }
 }
 
+// One lane's share (4 of 32 values) of a D4S4 group: ties away from zero, clamp -128..127, float32 scale and sum
+// (four sequential adds per lane, then an xor tree over the 8 lanes: 4, 2, 1).
+__device__ __forceinline__ void d4s4_pack_group(const float (&v)[4], float amax, int64_t g, int e, uint8_t* out) {
+  const int64_t blk_idx = g >> 2;
+  const int grp = static_cast<int>(g & 3);
+  float s = ((v[0] + v[1]) + v[2]) + v[3];
+  s += dpp_f<DPP_ROW_SHL4>(s);
+  s += dpp_f<DPP_ROW_SHL2>(s);
+  s += dpp_f<DPP_ROW_SHL1>(s);
+  const float d = amax == 0.0f ? 0.0f : amax / 127.0f;
+  uint32_t packed = 0;
+  if (d != 0.0f) {
+    packed = pack_i8x4(max(-128, min(127, static_cast<int>(roundf(v[0] / d)))),
+                       max(-128, min(127, static_cast<int>(roundf(v[1] / d)))),
+                       max(-128, min(127, static_cast<int>(roundf(v[2] / d)))),
+                       max(-128, min(127, static_cast<int>(roundf(v[3] / d)))));
+  }
+  uint8_t* blk = out + blk_idx * D4S4_BYTES;
+  *reinterpret_cast<uint32_t*>(blk + 32 + grp * 32 + 4 * e) = packed;
+  if (e == 0) {
+    *reinterpret_cast<float*>(blk + 4 * grp) = d;
+    *reinterpret_cast<float*>(blk + 16 + 4 * grp) = s;
+  }
+}
+
 // DS4 (ties-to-even, clamp +-127, fp16 scale and sum) or D4S4 (ties away,
 // clamp -128..127, float32 scale and sum).  One group of 8 lanes per 32 values;
 // a 128-value block is four consecutive groups.
@@ -95,28 +120,8 @@ __global__ void __launch_bounds__(256) pack_mmq_kernel(const uint16_t* __restric
   float v[4];
   load4_values(x, KIND_BF16, g * 32 + e * 4, v);
   const float amax = oct_max(fmaxf(fmaxf(fabsf(v[0]), fabsf(v[1])), fmaxf(fabsf(v[2]), fabsf(v[3]))));
-  const int64_t blk_idx = g >> 2;
-  const int grp = static_cast<int>(g & 3);
   if constexpr (D4S4) {
-    // four sequential adds per lane, then an xor tree over the 8 lanes (4, 2, 1)
-    float s = ((v[0] + v[1]) + v[2]) + v[3];
-    s += dpp_f<DPP_ROW_SHL4>(s);
-    s += dpp_f<DPP_ROW_SHL2>(s);
-    s += dpp_f<DPP_ROW_SHL1>(s);
-    const float d = amax == 0.0f ? 0.0f : amax / 127.0f;
-    uint32_t packed = 0;
-    if (d != 0.0f) {
-      packed = pack_i8x4(max(-128, min(127, static_cast<int>(roundf(v[0] / d)))),
-                         max(-128, min(127, static_cast<int>(roundf(v[1] / d)))),
-                         max(-128, min(127, static_cast<int>(roundf(v[2] / d)))),
-                         max(-128, min(127, static_cast<int>(roundf(v[3] / d)))));
-    }
-    uint8_t* blk = out + blk_idx * D4S4_BYTES;
-    *reinterpret_cast<uint32_t*>(blk + 32 + grp * 32 + 4 * e) = packed;
-    if (e == 0) {
-      *reinterpret_cast<float*>(blk + 4 * grp) = d;
-      *reinterpret_cast<float*>(blk + 16 + 4 * grp) = s;
-    }
+    d4s4_pack_group(v, amax, g, e, out);
   } else {
     ds4_pack_group(v, amax, g, e, out);
   }
@@ -124,6 +129,7 @@ __global__ void __launch_bounds__(256) pack_mmq_kernel(const uint16_t* __restric
 
 // gate_up [rows, 2*inter] (gate columns first) -> DS4 blocks of bf16_round(silu(gate) * up):
 // the bytes the two-step path (SiLU*up to bf16, then the DS4 pack) produces.
+template <bool D4S4>
 __global__ void __launch_bounds__(256) silu_mul_ds4_pack_kernel(const void* __restrict__ gate_up, int in_kind,
                                                                 uint8_t* __restrict__ out, int64_t total_groups,
                                                                 int64_t inter) {
@@ -141,7 +147,11 @@ __global__ void __launch_bounds__(256) silu_mul_ds4_pack_kernel(const void* __re
     v[i] = bf16_bits_to_float(float_to_bf16_bits(gate[i] * sig * up[i]));
   }
   const float amax = oct_max(fmaxf(fmaxf(fabsf(v[0]), fabsf(v[1])), fmaxf(fabsf(v[2]), fabsf(v[3]))));
-  ds4_pack_group(v, amax, g, e, out);
+  if constexpr (D4S4) {
+    d4s4_pack_group(v, amax, g, e, out);
+  } else {
+    ds4_pack_group(v, amax, g, e, out);
+  }
 }
 
 // The DS4 pack of rows gathered through the routing index: output row r is the pack of token
@@ -233,7 +243,21 @@ extern "C" int hipengine_gfx950_moe_silu_mul_ds4_pack(const void* gate_up, int i
   const int64_t groups = rows * (inter / 32);
   const int64_t grid = (groups + 31) / 32;
   if (grid > 0x7FFFFFFF) return static_cast<int>(hipErrorInvalidValue);
-  hipLaunchKernelGGL(silu_mul_ds4_pack_kernel, dim3(static_cast<unsigned>(grid)), dim3(256), 0, stream, gate_up,
+  hipLaunchKernelGGL(silu_mul_ds4_pack_kernel<false>, dim3(static_cast<unsigned>(grid)), dim3(256), 0, stream, gate_up,
+                     in_kind, static_cast<uint8_t*>(out), groups, inter);
+  return static_cast<int>(hipGetLastError());
+}
+
+// The same into D4S4 blocks (what the Q5_K / Q6_K MMQ kernels take).
+extern "C" int hipengine_gfx950_moe_silu_mul_d4s4_pack(const void* gate_up, int in_kind, void* out, int64_t rows,
+                                                       int64_t inter, hipStream_t stream) {
+  if (!gate_up || !out || rows <= 0 || inter <= 0 || (inter % 128) != 0 || in_kind < KIND_F32 || in_kind > KIND_F16) {
+    return static_cast<int>(hipErrorInvalidValue);
+  }
+  const int64_t groups = rows * (inter / 32);
+  const int64_t grid = (groups + 31) / 32;
+  if (grid > 0x7FFFFFFF) return static_cast<int>(hipErrorInvalidValue);
+  hipLaunchKernelGGL(silu_mul_ds4_pack_kernel<true>, dim3(static_cast<unsigned>(grid)), dim3(256), 0, stream, gate_up,
                      in_kind, static_cast<uint8_t*>(out), groups, inter);
   return static_cast<int>(hipGetLastError());
 }

@@ -60,6 +60,22 @@ def qwen35_moe_group_compact_active_source_rows(selected_experts_ptr: int, routi
                     stream), runtime)
 
 
+def moe_tile_map(expert_start_compact_ptr: int, tile_expert_start_ptr: int, tile_expert_ptr: int, total_ptr: int,
+                 num_experts: int, *, tile_rows: int = 32, tile_capacity: int = 0, stream: int = 0,
+                 library: ctypes.CDLL | None = None, runtime: HipRuntime | None = None) -> None:
+    """``qwen35_moe_mmq32_tile_map`` for tiles of 32, 64 or 128 rows (C symbol ``hipengine_gfx950_moe_tile_map``)."""
+    _check_num_experts(num_experts)
+    if tile_rows not in (32, 64, 128):
+        raise ValueError("tile_rows must be 32, 64 or 128")
+    if tile_capacity < 0:
+        raise ValueError("tile_capacity must be non-negative")
+    validate_pointers(expert_start_compact_ptr=expert_start_compact_ptr, tile_expert_start_ptr=tile_expert_start_ptr,
+                      tile_expert_ptr=tile_expert_ptr, total_ptr=total_ptr)
+    fn = entry("hipengine_gfx950_moe_tile_map", [VOID] * 4 + [I64, I64, ctypes.c_int32, VOID], library)
+    check_launch(fn(expert_start_compact_ptr, tile_expert_start_ptr, tile_expert_ptr, total_ptr, num_experts,
+                    tile_capacity, tile_rows, stream), runtime)
+
+
 def moe_group_compact_index(selected_experts_ptr: int, routing_weights_ptr: int, expert_start_ptr: int,
                             active_experts_ptr: int, active_count_ptr: int, sorted_lanes_ptr: int,
                             compact_to_source_ptr: int, sorted_weights_ptr: int, lane_to_compact_ptr: int,

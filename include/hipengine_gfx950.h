@@ -480,6 +480,11 @@ int hipengine_gfx950_moe_silu_mul(const void* gate_up, void* out, int64_t rows, 
 int hipengine_gfx950_moe_silu_mul_ds4_pack(const void* gate_up, int in_kind, void* out, int64_t rows, int64_t inter,
                                            hipengine_stream_t stream);
 
+/* The same into 160-byte D4S4 blocks (byte for byte hipengine_gfx950_moe_silu_mul with bf16 out followed by
+ * hipengine_gguf_q8_1_d4s4_f32_quantize_bf16): the activations of a Q5_K / Q6_K down projection.  New here. */
+int hipengine_gfx950_moe_silu_mul_d4s4_pack(const void* gate_up, int in_kind, void* out, int64_t rows, int64_t inter,
+                                            hipengine_stream_t stream);
+
 /* out[t, h] = sum over slots s = 0..top_k-1, in that order, of
  * routing_weights[t*top_k+s] * down[lane_to_compact[t*top_k+s], h]; lanes mapped
  * to -1 are skipped.  tokens <= 65535.  New here (see lane_to_compact). */
@@ -632,6 +637,27 @@ int hipengine_gfx950_gguf_q4_k_grouped_mmq(const void* x_q8, const int64_t* comp
                                            int64_t out_features_a, int64_t out_features_b, int64_t num_experts,
                                            int64_t mmq_total_rows, int64_t expert_stride_rows,
                                            hipengine_stream_t stream);
+
+/* The expert-grouped MMQ for Q6_K expert weights [num_experts, out_features, K/256 * 210] over D4S4 activation
+ * blocks (hipengine_gguf_q8_1_d4s4_f32_quantize_bf16 or hipengine_gfx950_moe_silu_mul_d4s4_pack):
+ * out[compact row, :] = [W_a[e] | W_b[e]] x, e the expert that owns the compact row; the arithmetic of
+ * hipengine_gguf_q6_k_mmq32_q8_1_d4s4_f32_bf16_*_out per expert.  The tile map is one of 128-row tiles
+ * (hipengine_gfx950_moe_tile_map with tile_rows = 128): total_rows a multiple of 128 with at most 65535 tiles.
+ * Any out_features; out_kind 0 float32, 1 bf16, 2 fp16; compact_to_source and the second weight optional.
+ * hipEngine has no grouped MMQ for Q6_K experts (its grouped kernels for them take its RDNA3 layouts).  New here. */
+int hipengine_gfx950_gguf_q6_k_grouped_mmq(const void* x_d4s4, const int64_t* compact_to_source,
+                                           const int64_t* expert_start_compact, const int64_t* expert_start_tiles,
+                                           const int64_t* tile_expert, const uint8_t* qweight_a,
+                                           const uint8_t* qweight_b, void* out, int32_t out_kind,
+                                           int64_t compact_rows, int64_t source_rows, int64_t in_features,
+                                           int64_t out_features_a, int64_t out_features_b, int64_t num_experts,
+                                           int64_t total_rows, int64_t expert_stride_rows,
+                                           hipengine_stream_t stream);
+
+/* hipengine_qwen35_moe_mmq32_tile_map for tiles of tile_rows = 32, 64 or 128 rows.  New here. */
+int hipengine_gfx950_moe_tile_map(const int64_t* expert_start_compact, int64_t* tile_expert_start,
+                                  int64_t* tile_expert, int64_t* total_out, int64_t num_experts,
+                                  int64_t tile_capacity, int32_t tile_rows, hipengine_stream_t stream);
 
 /* ------------------------------------------------------------------------
  * Verification exports: the integer unpack and the int32 sub-block dots the

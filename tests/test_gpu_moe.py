@@ -334,6 +334,68 @@ def test_grouped_mmq_matches_dense_formula_per_expert(dev, tokens, top_k, expert
     dev.free(*d.values())
 
 
+@pytest.mark.parametrize("tokens,top_k,experts,k,na,nb,identity", [
+    (40, 4, 8, 512, 96, 40, False),        # ragged widths, experts of a few rows
+    (300, 4, 6, 1024, 200, 0, False),      # experts of several 128-row tiles (about 200 rows each)
+    (64, 1, 5, 768, 130, 64, True),        # compact rows read as they are (an already gathered intermediate)
+])
+def test_grouped_mmq_q6_k_matches_dense_formula_per_expert(dev, tokens, top_k, experts, k, na, nb, identity):
+    """The expert-grouped MMQ for Q6_K experts over D4S4 blocks and a map of 128-row tiles: per expert the float64
+    value of the dense Q6_K x D4S4 formula on the rows it owns; rows of no expert and tiles past an expert's rows
+    stay unwritten."""
+    sel, wts = _routing(tokens * 5 + k, tokens, top_k, experts, bad=tokens > 20)
+    host, d = _device_index(dev, sel, wts, experts)
+    total, lanes = host["total"], tokens * top_k
+    rows_src = total if identity else tokens
+    x = (np.random.default_rng(k).standard_normal((rows_src, k)) * 0.2).astype(np.float32)
+    d4s4 = O.pack_q8_1_d4s4(O.f32_to_bf16_bits(x))
+    w_a = _experts(O.GGML_Q6_K, experts, na, k, seed=13)
+    w_b = _experts(O.GGML_Q6_K, experts, nb, k, seed=14) if nb else None
+    cap = lanes // 128 + experts
+    ts, te, tt = dev.empty((experts + 1) * 8), dev.empty(cap * 8, fill=0x11), dev.empty(8)
+    GS.moe_tile_map(d["expert_start"].ptr, ts.ptr, te.ptr, tt.ptr, experts, tile_rows=128, tile_capacity=cap)
+    want_map = O.tile_map(host["expert_start"], experts, 128, cap)
+    assert np.array_equal(dev.get(ts, np.int64, (experts + 1,)), want_map["tile_expert_start"])
+    assert np.array_equal(dev.get(te, np.int64, (cap,)), want_map["tile_expert"])
+    assert int(dev.get(tt, np.int64, (1,))[0]) == want_map["total"]
+    dxq, dwa = dev.put(d4s4), dev.put(w_a)
+    dwb = dev.put(w_b) if nb else None
+    dout = dev.empty((total + 1) * (na + nb) * 4, fill=0x7D)
+    M.gguf_q6_k_grouped_mmq(dxq.ptr, d["expert_start"].ptr, ts.ptr, te.ptr, dwa.ptr, dout.ptr, total, rows_src, k, na,
+                            experts, cap * 128, compact_to_source_ptr=0 if identity else d["c2s"].ptr,
+                            qweight_b_ptr=dwb.ptr if dwb else 0, out_features_b=nb)
+    got = dev.get(dout, np.float32, (total + 1, na + nb))
+    dev.free(dxq, dwa, dout, ts, te, tt, *([dwb] if dwb else []))
+    assert np.all(got[total].view(np.uint32) == 0x7D7D7D7D)
+    es = host["expert_start"]
+    for e in range(experts):
+        lo, hi = int(es[e]), int(es[e + 1])
+        if hi == lo:
+            continue
+        src = np.arange(lo, hi) if identity else host["c2s"][lo:hi]
+        want_a = O.mmq_q6_k_d4s4(d4s4[src], w_a[e])
+        assert O.max_rel_err(got[lo:hi, :na], want_a) <= REL_TOL and O.cosine(got[lo:hi, :na], want_a) >= COS_MIN
+        if nb:
+            want_b = O.mmq_q6_k_d4s4(d4s4[src], w_b[e])
+            assert O.max_rel_err(got[lo:hi, na:], want_b) <= REL_TOL and O.cosine(got[lo:hi, na:], want_b) >= COS_MIN
+    dev.free(*d.values())
+
+
+def test_silu_mul_d4s4_pack_bytes(dev):
+    """SiLU * up fused with the D4S4 pack: the bytes of the two-step path (SiLU * up to bf16, then the pack)."""
+    rows, inter = 37, 384
+    rng = np.random.default_rng(5)
+    gu = O.f32_to_bf16_bits((rng.standard_normal((rows, 2 * inter)) * 1.5).astype(np.float32))
+    dgu = dev.put(gu)
+    mid, want, got = dev.empty(rows * inter * 2), dev.empty(rows * (inter // 128) * 160), dev.empty(rows * (inter // 128) * 160)
+    M.moe_silu_mul(dgu.ptr, mid.ptr, rows, inter, in_dtype="bf16", out_dtype="bf16")
+    Q.gguf_q8_1_d4s4_f32_quantize_bf16(mid.ptr, want.ptr, rows, inter)
+    M.moe_silu_mul_d4s4_pack(dgu.ptr, got.ptr, rows, inter, in_dtype="bf16")
+    a, b = dev.get(got, np.uint8, (rows, inter // 128, 160)), dev.get(want, np.uint8, (rows, inter // 128, 160))
+    dev.free(dgu, mid, want, got)
+    assert np.array_equal(a, b)
+
+
 def test_grouped_mmq_bf16_named_entry(dev):
     tokens, top_k, experts, k, na, nb = 64, 4, 8, 1024, 128, 128
     sel, wts = _routing(31, tokens, top_k, experts)

@@ -293,6 +293,16 @@ def test_moe_wrappers_validate_before_touching_the_device():
         M.gguf_q4_k_grouped_mmq(1, 1, 1, 1, 1, 1, 8, 8, 256, 40, 4, 32)
     with pytest.raises(ValueError, match="multiple of 32"):
         M.gguf_q4_k_grouped_mmq(1, 1, 1, 1, 1, 1, 8, 8, 256, 64, 4, 40)
+    with pytest.raises(ValueError, match="multiple of 128"):
+        M.gguf_q6_k_grouped_mmq(1, 1, 1, 1, 1, 1, 8, 8, 256, 64, 4, 64)
+    with pytest.raises(ValueError, match="divisible by the GGUF block size"):
+        M.gguf_q6_k_grouped_mmq(1, 1, 1, 1, 1, 1, 8, 8, 384, 64, 4, 128)
+    with pytest.raises(ValueError, match="non-null"):
+        M.gguf_q6_k_grouped_mmq(1, 1, 1, 0, 1, 1, 8, 8, 256, 64, 4, 128)
+    with pytest.raises(ValueError, match="tile_rows"):
+        GS.moe_tile_map(1, 1, 1, 1, 8, tile_rows=48)
+    with pytest.raises(ValueError, match="inter"):
+        M.moe_silu_mul_d4s4_pack(1, 1, 4, 100)
 
 
 def test_gguf_container_round_trip_and_errors(tmp_path):
