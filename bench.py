@@ -285,8 +285,8 @@ class Harness:
         return ev, 2.0 * m * n * k
 
     def moe_case(self, tokens: int, steps: int, warmup: int, experts: int = 256, top_k: int = 8, hidden: int = 2048,
-                 inter: int = 512):
-        """Selected-expert FFN (Q4_K gate/up/down): the two-launch decode chain for
+                 inter: int = 512, down_quant: str = "q4_k"):
+        """Selected-expert FFN (Q4_K gate/up, Q4_K or Q6_K down): the two-launch decode chain for
         tokens <= 8, the grouped-MMQ prefill chain (index, pack, gate|up, SiLU, pack,
         down, ordered gather) above.  Returns seconds per chain and the bytes of
         distinct expert weights it touches."""
@@ -299,7 +299,8 @@ class Harness:
         rng = np.random.default_rng(tokens)
         wg = synthetic_blocks(GGML["q4_k"], experts * inter, hidden, seed=5)
         wu = synthetic_blocks(GGML["q4_k"], experts * inter, hidden, seed=6)
-        wd = synthetic_blocks(GGML["q4_k"], experts * hidden, inter, seed=7)
+        wd = synthetic_blocks(GGML[down_quant], experts * hidden, inter, seed=7)
+        q6_down = down_quant == "q6_k"
         sel = np.stack([rng.permutation(experts)[:top_k] for _ in range(tokens)]).astype(np.int64)
         wts = rng.random((tokens, top_k)).astype(np.float32)
         wts /= wts.sum(axis=1, keepdims=True)
@@ -309,7 +310,7 @@ class Harness:
                 "sel": mem.to_device(sel, runtime=rt), "wts": mem.to_device(wts, runtime=rt),
                 "out": mem.malloc(tokens * hidden * 4, runtime=rt)}
         b = bufs
-        per_expert = (2 * inter * (hidden // 256) + hidden * (inter // 256)) * 144
+        per_expert = 2 * inter * (hidden // 256) * 144 + hidden * (inter // 256) * (210 if q6_down else 144)
         touched = len(np.unique(sel)) * per_expert
         if tokens <= 8:
             b["x"] = mem.to_device(x, runtime=rt)
@@ -318,7 +319,7 @@ class Harness:
             def chain(_i, stream=0):
                 M.gguf_selected_gemv("gguf_q4_k", M.SEL_DUAL_SILU, b["x"].ptr, b["sel"].ptr, b["wg"].ptr, b["mid"].ptr,
                                      tokens, lanes, experts, hidden, inter, qweight_b_ptr=b["wu"].ptr, stream=stream)
-                M.gguf_selected_gemv("gguf_q4_k", M.SEL_DOWN_SUM, b["mid"].ptr, b["sel"].ptr, b["wd"].ptr, b["out"].ptr,
+                M.gguf_selected_gemv("gguf_" + down_quant, M.SEL_DOWN_SUM, b["mid"].ptr, b["sel"].ptr, b["wd"].ptr, b["out"].ptr,
                                      tokens, lanes, experts, inter, hidden, routing_weights_ptr=b["wts"].ptr,
                                      top_k=top_k, stream=stream)
         else:
@@ -329,9 +330,13 @@ class Harness:
                                  ("c2s", lanes * 8), ("sw", lanes * 4), ("ms", (experts + 1) * 8), ("te", cap * 8),
                                  ("mt", 8), ("l2c", lanes * 8), ("xq", tokens * (hidden // 128) * 144),
                                  ("gu", lanes * 2 * inter * 2),
-                                 ("mq", lanes * (inter // 128) * 144), ("down", lanes * hidden * 2)):
+                                 ("mq", lanes * (inter // 128) * 160), ("down", lanes * hidden * 2)):
                 b[name] = mem.malloc(nbytes, runtime=rt)
             mmq_rows = cap * 32     # upper bound known on the host; unused tiles are marked -1
+            cap128 = lanes // 128 + experts
+            if q6_down:             # the Q6_K tile engine takes 128-row tiles: a second tile map
+                for name, nbytes in (("ms128", (experts + 1) * 8), ("te128", cap128 * 8), ("mt128", 8)):
+                    b[name] = mem.malloc(nbytes, runtime=rt)
 
             def chain(_i):
                 GS.moe_group_compact_index(b["sel"].ptr, b["wts"].ptr, b["es"].ptr, b["act"].ptr, b["actn"].ptr,
@@ -344,9 +349,18 @@ class Harness:
                                         lanes, tokens, hidden, inter, experts, mmq_rows,
                                         compact_to_source_ptr=b["c2s"].ptr, qweight_b_ptr=b["wu"].ptr,
                                         out_features_b=inter, out_dtype="bf16")
-                M.moe_silu_mul_ds4_pack(b["gu"].ptr, b["mq"].ptr, lanes, inter, in_dtype="bf16")
-                M.gguf_q4_k_grouped_mmq(b["mq"].ptr, b["es"].ptr, b["ms"].ptr, b["te"].ptr, b["wd"].ptr, b["down"].ptr,
-                                        lanes, lanes, inter, hidden, experts, mmq_rows, out_dtype="bf16")
+                if q6_down:
+                    GS.moe_tile_map(b["es"].ptr, b["ms128"].ptr, b["te128"].ptr, b["mt128"].ptr, experts, tile_rows=128,
+                                    tile_capacity=cap128)
+                    M.moe_silu_mul_d4s4_pack(b["gu"].ptr, b["mq"].ptr, lanes, inter, in_dtype="bf16")
+                    M.gguf_q6_k_grouped_mmq(b["mq"].ptr, b["es"].ptr, b["ms128"].ptr, b["te128"].ptr, b["wd"].ptr,
+                                            b["down"].ptr, lanes, lanes, inter, hidden, experts, cap128 * 128,
+                                            out_dtype="bf16")
+                else:
+                    M.moe_silu_mul_ds4_pack(b["gu"].ptr, b["mq"].ptr, lanes, inter, in_dtype="bf16")
+                    M.gguf_q4_k_grouped_mmq(b["mq"].ptr, b["es"].ptr, b["ms"].ptr, b["te"].ptr, b["wd"].ptr,
+                                            b["down"].ptr, lanes, lanes, inter, hidden, experts, mmq_rows,
+                                            out_dtype="bf16")
                 M.moe_weighted_gather_sum(b["down"].ptr, b["l2c"].ptr, b["wts"].ptr, b["out"].ptr, tokens, top_k, hidden,
                                           lanes, in_dtype="bf16")
         _, ev = self.time_launches(chain, steps, warmup)
@@ -539,6 +553,12 @@ def main() -> None:
                 "int8_TOPS": round(ops / sec / 1e12, 2), "launches": 2 if tokens <= 8 else 8}
             if h.last_moe_graph_s:
                 extra[f"moe_q4_k_e256_k8_h2048_i512_t{tokens}"]["hip_graph_us"] = round(h.last_moe_graph_s * 1e6, 1)
+        for tokens in (1, 2048):    # the same FFN with Q6_K down experts (what a Q4_K_M file holds in half its layers)
+            sec, touched, ops = h.moe_case(tokens, max(10, args.steps // 10) if tokens <= 8 else msteps, 3,
+                                           down_quant="q6_k")
+            extra[f"moe_q4_k_gate_up_q6_k_down_e256_k8_h2048_i512_t{tokens}"] = {
+                "us": round(sec * 1e6, 1), "expert_GB/s": round(touched / sec / 1e9, 1),
+                "int8_TOPS": round(ops / sec / 1e12, 2), "launches": 2 if tokens <= 8 else 9}
 
     # the MMQ half of the metric, as a second roofline object: int8 operations 2*M*N*K of the Q4_K prefill GEMM at
     # M = 2048 over its HIP-event time, against the dense int8 MFMA peak

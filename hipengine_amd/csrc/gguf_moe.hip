@@ -889,9 +889,10 @@ int launch_grouped_gemv(int qt, const void* x, int x_kind, const int64_t* expert
 // --------------------------------------------------------------------------
 
 using MoeQ4 = Q4Tile<1, 2, 1, 4>;   // 32 compact rows x 256 columns, four waves side by side
+using MoeQ5 = Q4Tile<1, 2, 1, 4, MMQ_Q5K_D4S4>;   // the same tile for Q5_K experts over D4S4 blocks
 
 struct MoeMmqArgs {
-  const uint8_t* xq;                 // DS4 blocks [source_rows, K/128]
+  const uint8_t* xq;                 // DS4 (Q4_K) or D4S4 (Q5_K) blocks [source_rows, K/128]
   const int64_t* compact_to_source;  // [compact_rows] or null (compact row i reads source row i)
   const int64_t* expert_start_compact;
   const int64_t* expert_start_tiles; // row starts rounded up to 32 per expert
@@ -905,33 +906,34 @@ struct MoeMmqArgs {
   int tiles_a;
 };
 
-__global__ void __launch_bounds__(MoeQ4::THREADS, 2) moe_mmq_q4_k_kernel(MoeMmqArgs a) {
+template <class Tile>
+__global__ void __launch_bounds__(Tile::THREADS, 2) moe_mmq_kernel(MoeMmqArgs a) {
   extern __shared__ __align__(16) uint8_t smem_raw[];
-  MoeQ4::Smem& s = *reinterpret_cast<MoeQ4::Smem*>(smem_raw);
-  int* src_row = reinterpret_cast<int*>(smem_raw + sizeof(MoeQ4::Smem));
+  typename Tile::Smem& s = *reinterpret_cast<typename Tile::Smem*>(smem_raw);
+  int* src_row = reinterpret_cast<int*>(smem_raw + sizeof(typename Tile::Smem));
 
   const int tile_row = blockIdx.y;
   const int64_t e = a.tile_expert[tile_row];
   if (e < 0 || e >= a.num_experts) return;
   const bool use_b = static_cast<int>(blockIdx.x) >= a.tiles_a;
-  const int n0 = (use_b ? blockIdx.x - a.tiles_a : blockIdx.x) * MoeQ4::BN;
+  const int n0 = (use_b ? blockIdx.x - a.tiles_a : blockIdx.x) * Tile::BN;
   const int local_n = use_b ? a.Nb : a.Na;
   const int64_t compact_base = a.expert_start_compact[e];
   const int64_t count = a.expert_start_compact[e + 1] - compact_base;
-  const int64_t row0 = static_cast<int64_t>(tile_row) * MoeQ4::BM - a.expert_start_tiles[e];
+  const int64_t row0 = static_cast<int64_t>(tile_row) * Tile::BM - a.expert_start_tiles[e];
   const int64_t remaining = count - row0;
   if (row0 < 0 || remaining <= 0) return;
-  const int valid_rows = remaining >= MoeQ4::BM ? MoeQ4::BM : static_cast<int>(remaining);
+  const int valid_rows = remaining >= Tile::BM ? Tile::BM : static_cast<int>(remaining);
   const int64_t first_compact = compact_base + row0;
-  if (first_compact + valid_rows > a.compact_rows) return;
+  if (compact_base < 0 || first_compact + valid_rows > a.compact_rows) return;
 
   const int steps = a.K / 128;
-  const int64_t w_row_bytes = static_cast<int64_t>(a.K / QK_K) * Q4_K_BYTES;
-  const int64_t x_row_bytes = static_cast<int64_t>(steps) * DS4_BYTES;
+  const int64_t w_row_bytes = static_cast<int64_t>(a.K / QK_K) * Tile::W_BLOCK;
+  const int64_t x_row_bytes = static_cast<int64_t>(steps) * Tile::A_BYTES;
   const int64_t stride_rows = a.expert_stride_rows > 0 ? a.expert_stride_rows : local_n;
   const uint8_t* w = (use_b ? a.w_b : a.w_a) + e * stride_rows * w_row_bytes;
 
-  if (threadIdx.x < MoeQ4::BM) {
+  if (threadIdx.x < Tile::BM) {
     const int64_t crow = first_compact + min(static_cast<int>(threadIdx.x), valid_rows - 1);
     int64_t src = a.compact_to_source ? a.compact_to_source[crow] : crow;
     src = src < 0 ? 0 : (src >= a.source_rows ? a.source_rows - 1 : src);
@@ -941,7 +943,7 @@ __global__ void __launch_bounds__(MoeQ4::THREADS, 2) moe_mmq_q4_k_kernel(MoeMmqA
 
   const int64_t out_stride = static_cast<int64_t>(a.Na) + a.Nb;
   const int col_base = (use_b ? a.Na : 0) + n0;
-  MoeQ4::run<true>(
+  Tile::template run<true>(
       a.xq, x_row_bytes, w, w_row_bytes, steps, s,
       [=](int row) { return static_cast<int64_t>(src_row[row]); },
       [=](int col) { return static_cast<int64_t>(min(n0 + col, local_n - 1)); },
@@ -951,6 +953,7 @@ __global__ void __launch_bounds__(MoeQ4::THREADS, 2) moe_mmq_q4_k_kernel(MoeMmqA
       });
 }
 
+template <class Tile>
 int launch_moe_mmq(const void* xq, const int64_t* compact_to_source, const int64_t* expert_start_compact,
                    const int64_t* expert_start_tiles, const int64_t* tile_expert, const uint8_t* w_a,
                    const uint8_t* w_b, void* out, int out_kind, int64_t compact_rows, int64_t source_rows, int64_t K,
@@ -974,10 +977,10 @@ int launch_moe_mmq(const void* xq, const int64_t* compact_to_source, const int64
   a.K = static_cast<int>(K); a.Na = static_cast<int>(Na); a.Nb = static_cast<int>(Nb);
   a.num_experts = static_cast<int>(num_experts);
   a.expert_stride_rows = expert_stride_rows;
-  a.tiles_a = static_cast<int>((Na + MoeQ4::BN - 1) / MoeQ4::BN);
-  const int tiles_b = static_cast<int>((Nb + MoeQ4::BN - 1) / MoeQ4::BN);
+  a.tiles_a = static_cast<int>((Na + Tile::BN - 1) / Tile::BN);
+  const int tiles_b = static_cast<int>((Nb + Tile::BN - 1) / Tile::BN);
   const dim3 grid(static_cast<unsigned>(a.tiles_a + tiles_b), static_cast<unsigned>(total_rows / 32));
-  hipLaunchKernelGGL(moe_mmq_q4_k_kernel, grid, dim3(MoeQ4::THREADS), sizeof(MoeQ4::Smem) + MoeQ4::BM * sizeof(int),
+  hipLaunchKernelGGL(moe_mmq_kernel<Tile>, grid, dim3(Tile::THREADS), sizeof(typename Tile::Smem) + Tile::BM * sizeof(int),
                      stream, a);
   return static_cast<int>(hipGetLastError());
 }
@@ -1407,7 +1410,7 @@ extern "C" int hipengine_gguf_q4_k_selected_dual_q8_1_ds4_mmq32_prefill_compact3
   if (!compact_to_source) return static_cast<int>(hipErrorInvalidValue);
   // As in hipEngine, the activation rows are addressed through compact_to_source only; the
   // source row count is not part of this signature, so the clamp is the compact row count.
-  return launch_moe_mmq(x_q8, compact_to_source, expert_start_compact, expert_start_mmq32, tile_expert, qweight_a,
+  return launch_moe_mmq<MoeQ4>(x_q8, compact_to_source, expert_start_compact, expert_start_mmq32, tile_expert, qweight_a,
                         qweight_b, out, KIND_BF16, compact_rows, compact_rows, in_features, out_features_a,
                         out_features_b, num_experts, mmq_total_rows, expert_stride_rows, stream);
 }
@@ -1421,9 +1424,24 @@ extern "C" int hipengine_gfx950_gguf_q4_k_grouped_mmq(const void* x_q8, const in
                                                       int64_t out_features_b, int64_t num_experts,
                                                       int64_t mmq_total_rows, int64_t expert_stride_rows,
                                                       hipStream_t stream) {
-  return launch_moe_mmq(x_q8, compact_to_source, expert_start_compact, expert_start_mmq32, tile_expert, qweight_a,
+  return launch_moe_mmq<MoeQ4>(x_q8, compact_to_source, expert_start_compact, expert_start_mmq32, tile_expert, qweight_a,
                         qweight_b, out, out_kind, compact_rows, source_rows, in_features, out_features_a,
                         out_features_b, num_experts, mmq_total_rows, expert_stride_rows, stream);
+}
+
+// The same for Q5_K expert weights over D4S4 activation blocks (the 32-row tile map).
+extern "C" int hipengine_gfx950_gguf_q5_k_grouped_mmq(const void* x_d4s4, const int64_t* compact_to_source,
+                                                      const int64_t* expert_start_compact,
+                                                      const int64_t* expert_start_mmq32, const int64_t* tile_expert,
+                                                      const uint8_t* qweight_a, const uint8_t* qweight_b, void* out,
+                                                      int32_t out_kind, int64_t compact_rows, int64_t source_rows,
+                                                      int64_t in_features, int64_t out_features_a,
+                                                      int64_t out_features_b, int64_t num_experts,
+                                                      int64_t mmq_total_rows, int64_t expert_stride_rows,
+                                                      hipStream_t stream) {
+  return launch_moe_mmq<MoeQ5>(x_d4s4, compact_to_source, expert_start_compact, expert_start_mmq32, tile_expert,
+                               qweight_a, qweight_b, out, out_kind, compact_rows, source_rows, in_features,
+                               out_features_a, out_features_b, num_experts, mmq_total_rows, expert_stride_rows, stream);
 }
 
 // The expert-grouped MMQ for Q6_K expert weights over D4S4 activation blocks: out[compact row, :] =

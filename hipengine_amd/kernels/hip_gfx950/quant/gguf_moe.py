@@ -276,7 +276,8 @@ def gguf_q4_k_grouped_mmq(x_q8_ptr: int, expert_start_compact_ptr: int, expert_s
                           in_features: int, out_features_a: int, num_experts: int, mmq_total_rows: int, *,
                           compact_to_source_ptr: int = 0, qweight_b_ptr: int = 0, out_features_b: int = 0,
                           out_dtype: str = "f32", expert_stride_rows: int = 0, stream: int = 0,
-                          library: ctypes.CDLL | None = None, runtime: HipRuntime | None = None) -> None:
+                          library: ctypes.CDLL | None = None, runtime: HipRuntime | None = None,
+                          _symbol: str = "hipengine_gfx950_gguf_q4_k_grouped_mmq") -> None:
     """The grouped MMQ with explicit output type, optional row map and optional second weight."""
     _validate_grouped(compact_rows, in_features, out_features_a, out_features_b, num_experts, mmq_total_rows)
     if source_rows <= 0:
@@ -284,11 +285,22 @@ def gguf_q4_k_grouped_mmq(x_q8_ptr: int, expert_start_compact_ptr: int, expert_s
     validate_pointers(x_q8_ptr=x_q8_ptr, expert_start_compact_ptr=expert_start_compact_ptr,
                       expert_start_mmq32_ptr=expert_start_mmq32_ptr, tile_expert_ptr=tile_expert_ptr,
                       qweight_a_ptr=qweight_a_ptr, out_ptr=out_ptr)
-    fn = entry("hipengine_gfx950_gguf_q4_k_grouped_mmq", [VOID] * 8 + [I32] + [I64] * 8 + [VOID], library)
+    fn = entry(_symbol, [VOID] * 8 + [I32] + [I64] * 8 + [VOID], library)
     check_launch(fn(x_q8_ptr, compact_to_source_ptr or None, expert_start_compact_ptr, expert_start_mmq32_ptr,
                     tile_expert_ptr, qweight_a_ptr, qweight_b_ptr or None, out_ptr, _KIND[out_dtype], compact_rows,
                     source_rows, in_features, out_features_a, out_features_b, num_experts, mmq_total_rows,
                     expert_stride_rows, stream), runtime)
+
+
+def gguf_q5_k_grouped_mmq(x_d4s4_ptr: int, expert_start_compact_ptr: int, expert_start_mmq32_ptr: int,
+                          tile_expert_ptr: int, qweight_a_ptr: int, out_ptr: int, compact_rows: int, source_rows: int,
+                          in_features: int, out_features_a: int, num_experts: int, mmq_total_rows: int,
+                          **kwargs) -> None:
+    """``gguf_q4_k_grouped_mmq`` for Q5_K experts over D4S4 activation blocks (the same 32-row tile map and
+    keyword arguments; C symbol ``hipengine_gfx950_gguf_q5_k_grouped_mmq``)."""
+    gguf_q4_k_grouped_mmq(x_d4s4_ptr, expert_start_compact_ptr, expert_start_mmq32_ptr, tile_expert_ptr,
+                          qweight_a_ptr, out_ptr, compact_rows, source_rows, in_features, out_features_a, num_experts,
+                          mmq_total_rows, _symbol="hipengine_gfx950_gguf_q5_k_grouped_mmq", **kwargs)
 
 
 def moe_silu_mul(gate_up_ptr: int, out_ptr: int, rows: int, inter: int, *, in_dtype: str = "f32",
@@ -398,6 +410,8 @@ def register_kernels(backend: str = "hip_gfx950", *, replace: bool = False) -> N
     register(KernelKey(backend, "moe_linear", "gguf_q4_k", "grouped_mmq32_q8_1_ds4"), gguf_q4_k_grouped_mmq,
              replace=replace)
     register(KernelKey(backend, "moe_linear", "gguf_q6_k", "grouped_mmq128_q8_1_d4s4"), gguf_q6_k_grouped_mmq,
+             replace=replace)
+    register(KernelKey(backend, "moe_linear", "gguf_q5_k", "grouped_mmq32_q8_1_d4s4"), gguf_q5_k_grouped_mmq,
              replace=replace)
     for quant in ("gguf_q4_k", "gguf_q5_k", "gguf_q6_k", "gguf_q8_0"):     # Q5_K and Q8_0: the single form
         register(KernelKey(backend, "moe_linear", quant, "selected_gemv_q8_1"), gguf_selected_gemv, replace=replace)

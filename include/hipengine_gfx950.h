@@ -638,6 +638,19 @@ int hipengine_gfx950_gguf_q4_k_grouped_mmq(const void* x_q8, const int64_t* comp
                                            int64_t mmq_total_rows, int64_t expert_stride_rows,
                                            hipengine_stream_t stream);
 
+/* hipengine_gfx950_gguf_q4_k_grouped_mmq for Q5_K expert weights [num_experts, out_features, K/256 * 176] over D4S4
+ * activation blocks: the same arguments, tile map (32-row tiles) and limits; the arithmetic of
+ * hipengine_gguf_q5_k_mmq32_q8_1_d4s4_f32_bf16_*_out per expert.  hipEngine has no grouped MMQ for Q5_K experts.
+ * New here. */
+int hipengine_gfx950_gguf_q5_k_grouped_mmq(const void* x_d4s4, const int64_t* compact_to_source,
+                                           const int64_t* expert_start_compact, const int64_t* expert_start_mmq32,
+                                           const int64_t* tile_expert, const uint8_t* qweight_a,
+                                           const uint8_t* qweight_b, void* out, int32_t out_kind,
+                                           int64_t compact_rows, int64_t source_rows, int64_t in_features,
+                                           int64_t out_features_a, int64_t out_features_b, int64_t num_experts,
+                                           int64_t mmq_total_rows, int64_t expert_stride_rows,
+                                           hipengine_stream_t stream);
+
 /* The expert-grouped MMQ for Q6_K expert weights [num_experts, out_features, K/256 * 210] over D4S4 activation
  * blocks (hipengine_gguf_q8_1_d4s4_f32_quantize_bf16 or hipengine_gfx950_moe_silu_mul_d4s4_pack):
  * out[compact row, :] = [W_a[e] | W_b[e]] x, e the expert that owns the compact row; the arithmetic of

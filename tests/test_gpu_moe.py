@@ -381,6 +381,40 @@ def test_grouped_mmq_q6_k_matches_dense_formula_per_expert(dev, tokens, top_k, e
     dev.free(*d.values())
 
 
+@pytest.mark.parametrize("tokens,top_k,experts,k,na,nb", [(40, 4, 8, 512, 96, 64), (120, 8, 12, 1024, 288, 0)])
+def test_grouped_mmq_q5_k_matches_dense_formula_per_expert(dev, tokens, top_k, experts, k, na, nb):
+    """The expert-grouped MMQ for Q5_K experts over D4S4 blocks (the 32-row tile map of the Q4_K one): per expert the
+    float64 value of the dense Q5_K x D4S4 formula on the rows it owns."""
+    sel, wts = _routing(tokens * 7 + k, tokens, top_k, experts, bad=True)
+    host, d = _device_index(dev, sel, wts, experts)
+    total = host["total"]
+    x = (np.random.default_rng(k + 1).standard_normal((tokens, k)) * 0.2).astype(np.float32)
+    d4s4 = O.pack_q8_1_d4s4(O.f32_to_bf16_bits(x))
+    w_a = O.stack_experts(_random_q5_k(na, k, seed=21), experts, seed=2)
+    w_b = O.stack_experts(_random_q5_k(nb, k, seed=22), experts, seed=3) if nb else None
+    dxq, dwa = dev.put(d4s4), dev.put(w_a)
+    dwb = dev.put(w_b) if nb else None
+    dout = dev.empty((total + 1) * (na + nb) * 4, fill=0x7D)
+    M.gguf_q5_k_grouped_mmq(dxq.ptr, d["expert_start"].ptr, d["mmq_start"].ptr, d["tile_expert"].ptr, dwa.ptr, dout.ptr,
+                            total, tokens, k, na, experts, host["mmq_total"], compact_to_source_ptr=d["c2s"].ptr,
+                            qweight_b_ptr=dwb.ptr if dwb else 0, out_features_b=nb)
+    got = dev.get(dout, np.float32, (total + 1, na + nb))
+    dev.free(dxq, dwa, dout, *([dwb] if dwb else []))
+    assert np.all(got[total].view(np.uint32) == 0x7D7D7D7D)
+    es = host["expert_start"]
+    for e in range(experts):
+        lo, hi = int(es[e]), int(es[e + 1])
+        if hi == lo:
+            continue
+        src = host["c2s"][lo:hi]
+        want_a = O.mmq_q5_k_d4s4(d4s4[src], w_a[e])
+        assert O.max_rel_err(got[lo:hi, :na], want_a) <= REL_TOL and O.cosine(got[lo:hi, :na], want_a) >= COS_MIN
+        if nb:
+            want_b = O.mmq_q5_k_d4s4(d4s4[src], w_b[e])
+            assert O.max_rel_err(got[lo:hi, na:], want_b) <= REL_TOL and O.cosine(got[lo:hi, na:], want_b) >= COS_MIN
+    dev.free(*d.values())
+
+
 def test_silu_mul_d4s4_pack_bytes(dev):
     """SiLU * up fused with the D4S4 pack: the bytes of the two-step path (SiLU * up to bf16, then the pack)."""
     rows, inter = 37, 384

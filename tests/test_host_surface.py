@@ -293,6 +293,8 @@ def test_moe_wrappers_validate_before_touching_the_device():
         M.gguf_q4_k_grouped_mmq(1, 1, 1, 1, 1, 1, 8, 8, 256, 40, 4, 32)
     with pytest.raises(ValueError, match="multiple of 32"):
         M.gguf_q4_k_grouped_mmq(1, 1, 1, 1, 1, 1, 8, 8, 256, 64, 4, 40)
+    with pytest.raises(ValueError, match="multiples of 32"):
+        M.gguf_q5_k_grouped_mmq(1, 1, 1, 1, 1, 1, 8, 8, 256, 40, 4, 32)
     with pytest.raises(ValueError, match="multiple of 128"):
         M.gguf_q6_k_grouped_mmq(1, 1, 1, 1, 1, 1, 8, 8, 256, 64, 4, 64)
     with pytest.raises(ValueError, match="divisible by the GGUF block size"):
