@@ -1086,6 +1086,213 @@ int launch_moe_mmq_q6(const void* xq, const int64_t* compact_to_source, const in
   return static_cast<int>(hipGetLastError());
 }
 
+// ---- MoE tail and the next RMSNorm ---------------------------------------------------
+//
+//   selected  = the token's routed sum, already rounded to bf16 (TAIL_AGGREGATE), or formed here from its slot rows
+//               in slot order, acc = acc + value * weight in float32 with both roundings, then rounded to bf16
+//               (TAIL_SLOTS: rows [token * rows + slot]; TAIL_GATHER: compact rows through lane_to_compact, a lane of
+//               no expert contributes nothing)
+//   residual' = bf16((residual + selected) + sigmoid(gate_logits[token * gate_stride]) * shared)
+//   norm      = bf16((residual' * 1 / sqrt(mean(residual'^2) + eps)) * norm_weight)
+//   (kernels/cpu_reference/ops.py:33-102; kernels/hip_gfx1100/fused/paro_combine.hip:452-482,575-700)
+//
+// One workgroup per token.  With features % 8 == 0 and features <= 8192 a thread owns up to four 8-value pieces,
+// keeps residual' in registers between the two passes and moves 16 bytes per access, a group of up to eight slot
+// rows in flight at a time; any other width takes one value per access and reads residual' back.
+enum TailMode : int { TAIL_AGGREGATE = 0, TAIL_SLOTS = 1, TAIL_GATHER = 2 };
+
+struct MoeTailArgs {
+  const uint16_t* selected;
+  const float* routing;
+  const int64_t* lane_to_compact;
+  const uint16_t* shared;
+  const float* gate_logits;
+  const uint16_t* residual;
+  const float* norm_weight;
+  uint16_t* norm_out;
+  uint16_t* residual_out;
+  int64_t features, gate_stride, compact_rows;
+  int rows;
+  float eps;
+};
+
+__device__ __forceinline__ void bf16x8_to_float(const uint4 p, float (&v)[8]) {
+  const uint32_t w[4] = {p.x, p.y, p.z, p.w};
+#pragma unroll
+  for (int e = 0; e < 4; ++e) {
+    v[2 * e] = bf16_bits_to_float(w[e] & 0xFFFFu);
+    v[2 * e + 1] = bf16_bits_to_float(w[e] >> 16);
+  }
+}
+
+// A product and a sum that stay two roundings (the compiler contracts a * b + c into one otherwise, and HIP's
+// __fmul_rn / __fadd_rn are the plain operators).
+__device__ __forceinline__ float mul_rn(float a, float b) {
+#pragma clang fp contract(off)
+  return a * b;
+}
+__device__ __forceinline__ float add_rn(float a, float b) {
+#pragma clang fp contract(off)
+  return a + b;
+}
+
+__device__ __forceinline__ float tail_combine(float residual, float selected, float gate, float shared) {
+  return bf16_bits_to_float(float_to_bf16_bits(add_rn(add_rn(residual, selected), mul_rn(gate, shared))));
+}
+
+// row of `selected` that slot s of the token reads, or -1
+template <int MODE>
+__device__ __forceinline__ int64_t tail_slot_row(const MoeTailArgs& a, int64_t lane) {
+  if constexpr (MODE == TAIL_GATHER) {
+    const int64_t c = a.lane_to_compact[lane];
+    return (c >= 0 && c < a.compact_rows) ? c : -1;
+  }
+  return lane;
+}
+
+template <int MODE, bool VEC>
+__global__ void __launch_bounds__(256) moe_tail_rmsnorm_kernel(MoeTailArgs a) {
+  constexpr int NC = 4;   // 8-value pieces per thread: features <= 256 * 8 * NC
+  const int64_t token = blockIdx.x;
+  const int tid = threadIdx.x;
+  const int64_t base = token * a.features;
+  const float gate = 1.0f / (1.0f + expf(-a.gate_logits[token * a.gate_stride]));
+  const int64_t lane0 = token * a.rows;
+  float sumsq = 0.0f;
+  float keep[NC][8];
+
+  if constexpr (VEC) {
+    const int64_t pieces = a.features >> 3;
+#pragma unroll
+    for (int i = 0; i < NC; ++i) {
+      const int64_t col = (static_cast<int64_t>(tid) + i * 256) * 8;
+      if (col >= pieces * 8) continue;
+      float sel[8], res[8], sh[8];
+      bf16x8_to_float(*reinterpret_cast<const uint4*>(a.residual + base + col), res);
+      bf16x8_to_float(*reinterpret_cast<const uint4*>(a.shared + base + col), sh);
+      if constexpr (MODE == TAIL_AGGREGATE) {
+        bf16x8_to_float(*reinterpret_cast<const uint4*>(a.selected + base + col), sel);
+      } else {
+        float acc[8];
+#pragma unroll
+        for (int e = 0; e < 8; ++e) acc[e] = 0.0f;
+        for (int s0 = 0; s0 < a.rows; s0 += 8) {
+          int64_t row[8];
+          float wgt[8];
+          uint4 piece[8];
+#pragma unroll
+          for (int s = 0; s < 8; ++s) {
+            const bool on = s0 + s < a.rows;
+            row[s] = on ? tail_slot_row<MODE>(a, lane0 + s0 + s) : -1;
+            wgt[s] = on ? a.routing[lane0 + s0 + s] : 0.0f;
+          }
+#pragma unroll
+          for (int s = 0; s < 8; ++s)
+            piece[s] = *reinterpret_cast<const uint4*>(a.selected + (row[s] >= 0 ? row[s] : 0) * a.features + col);
+#pragma unroll
+          for (int s = 0; s < 8; ++s) {
+            if (row[s] < 0) continue;
+            float v[8];
+            bf16x8_to_float(piece[s], v);
+#pragma unroll
+            for (int e = 0; e < 8; ++e) acc[e] = add_rn(acc[e], mul_rn(v[e], wgt[s]));
+          }
+        }
+#pragma unroll
+        for (int e = 0; e < 8; ++e) sel[e] = bf16_bits_to_float(float_to_bf16_bits(acc[e]));
+      }
+      uint32_t packed[4];
+#pragma unroll
+      for (int e = 0; e < 8; ++e) {
+        const float v = tail_combine(res[e], sel[e], gate, sh[e]);
+        keep[i][e] = v;
+        sumsq += v * v;
+        const uint32_t bits = float_to_bits(v) >> 16;     // v is a bf16 value already
+        packed[e >> 1] = (e & 1) ? (packed[e >> 1] | (bits << 16)) : bits;
+      }
+      *reinterpret_cast<uint4*>(a.residual_out + base + col) = make_uint4(packed[0], packed[1], packed[2], packed[3]);
+    }
+  } else {
+    for (int64_t col = tid; col < a.features; col += 256) {
+      float sel;
+      if constexpr (MODE == TAIL_AGGREGATE) {
+        sel = bf16_bits_to_float(a.selected[base + col]);
+      } else {
+        float acc = 0.0f;
+        for (int s = 0; s < a.rows; ++s) {
+          const int64_t row = tail_slot_row<MODE>(a, lane0 + s);
+          if (row < 0) continue;
+          acc = add_rn(acc, mul_rn(bf16_bits_to_float(a.selected[row * a.features + col]), a.routing[lane0 + s]));
+        }
+        sel = bf16_bits_to_float(float_to_bf16_bits(acc));
+      }
+      const float v = tail_combine(bf16_bits_to_float(a.residual[base + col]), sel, gate,
+                                   bf16_bits_to_float(a.shared[base + col]));
+      a.residual_out[base + col] = static_cast<uint16_t>(float_to_bits(v) >> 16);
+      sumsq += v * v;
+    }
+  }
+
+  __shared__ float wave_sum[4];
+#pragma unroll
+  for (int off = 32; off > 0; off >>= 1) sumsq += __shfl_xor(sumsq, off);
+  if ((tid & 63) == 0) wave_sum[tid >> 6] = sumsq;
+  __syncthreads();
+  const float total = (wave_sum[0] + wave_sum[1]) + (wave_sum[2] + wave_sum[3]);
+  const float inv_rms = 1.0f / sqrtf(total / static_cast<float>(a.features) + a.eps);
+
+  if constexpr (VEC) {
+    const int64_t pieces = a.features >> 3;
+#pragma unroll
+    for (int i = 0; i < NC; ++i) {
+      const int64_t col = (static_cast<int64_t>(tid) + i * 256) * 8;
+      if (col >= pieces * 8) continue;
+      const float4 w0 = *reinterpret_cast<const float4*>(a.norm_weight + col);
+      const float4 w1 = *reinterpret_cast<const float4*>(a.norm_weight + col + 4);
+      const float w[8] = {w0.x, w0.y, w0.z, w0.w, w1.x, w1.y, w1.z, w1.w};
+      uint32_t packed[4];
+#pragma unroll
+      for (int e = 0; e < 8; ++e) {
+        const uint32_t bits = float_to_bf16_bits(mul_rn(mul_rn(keep[i][e], inv_rms), w[e]));
+        packed[e >> 1] = (e & 1) ? (packed[e >> 1] | (bits << 16)) : bits;
+      }
+      *reinterpret_cast<uint4*>(a.norm_out + base + col) = make_uint4(packed[0], packed[1], packed[2], packed[3]);
+    }
+  } else {
+    for (int64_t col = tid; col < a.features; col += 256) {
+      const float v = bf16_bits_to_float(a.residual_out[base + col]);   // this thread's own store
+      a.norm_out[base + col] = float_to_bf16_bits(mul_rn(mul_rn(v, inv_rms), a.norm_weight[col]));
+    }
+  }
+}
+
+template <int MODE>
+int launch_moe_tail(const uint16_t* selected, const float* routing, const int64_t* lane_to_compact,
+                    const uint16_t* shared, const float* gate_logits, const uint16_t* residual,
+                    const float* norm_weight, uint16_t* norm_out, uint16_t* residual_out, int64_t tokens, int64_t rows,
+                    int64_t features, int64_t compact_rows, int64_t gate_stride, float eps, hipStream_t stream) {
+  if (!selected || !shared || !gate_logits || !residual || !norm_weight || !norm_out || !residual_out || tokens <= 0 ||
+      tokens > 0x7FFFFFFF || features <= 0 || gate_stride <= 0 || rows <= 0 || rows > 4096 ||
+      (MODE != TAIL_AGGREGATE && !routing) || (MODE == TAIL_GATHER && (!lane_to_compact || compact_rows <= 0))) {
+    return static_cast<int>(hipErrorInvalidValue);
+  }
+  MoeTailArgs a;
+  a.selected = selected; a.routing = routing; a.lane_to_compact = lane_to_compact; a.shared = shared;
+  a.gate_logits = gate_logits; a.residual = residual; a.norm_weight = norm_weight; a.norm_out = norm_out;
+  a.residual_out = residual_out; a.features = features; a.gate_stride = gate_stride; a.compact_rows = compact_rows;
+  a.rows = static_cast<int>(rows); a.eps = eps;
+  const uintptr_t align = reinterpret_cast<uintptr_t>(selected) | reinterpret_cast<uintptr_t>(shared) |
+                          reinterpret_cast<uintptr_t>(residual) | reinterpret_cast<uintptr_t>(norm_weight) |
+                          reinterpret_cast<uintptr_t>(norm_out) | reinterpret_cast<uintptr_t>(residual_out);
+  const dim3 grid(static_cast<unsigned>(tokens));
+  if ((features % 8) == 0 && features <= 8192 && (align & 15u) == 0) {
+    hipLaunchKernelGGL((moe_tail_rmsnorm_kernel<MODE, true>), grid, dim3(256), 0, stream, a);
+  } else {
+    hipLaunchKernelGGL((moe_tail_rmsnorm_kernel<MODE, false>), grid, dim3(256), 0, stream, a);
+  }
+  return static_cast<int>(hipGetLastError());
+}
+
 // ---- router: top-k experts of a row of logits and the softmax of their logits --------
 //
 // One wave per token.  Lane l keeps the logits of experts l, l+64, ... (up to 16 of them,
@@ -1258,6 +1465,36 @@ extern "C" int hipengine_gfx950_moe_silu_mul(const void* gate_up, void* out, int
   hipLaunchKernelGGL(moe_silu_mul_kernel, dim3(static_cast<unsigned>((rows * inter + 255) / 256)), dim3(256), 0, stream,
                      gate_up, out, rows, inter, in_kind, out_kind);
   return static_cast<int>(hipGetLastError());
+}
+
+// The MoE tail with the next layer's RMSNorm (bf16 rows, float32 norm weight) for a routed sum that is already
+// formed and rounded, for slot rows [tokens * rows_per_token, features] with their routing weights, and for compact
+// rows gathered through lane_to_compact.
+extern "C" int hipengine_shared_gate_combine_residual_rmsnorm_gguf_bf16_out(
+    const uint16_t* selected, const uint16_t* shared, const float* gate_logits, const uint16_t* residual,
+    const float* norm_weight, uint16_t* norm_out, uint16_t* residual_out, int64_t tokens, int64_t features,
+    int64_t gate_stride, float eps, hipStream_t stream) {
+  return launch_moe_tail<TAIL_AGGREGATE>(selected, nullptr, nullptr, shared, gate_logits, residual, norm_weight, norm_out,
+                                         residual_out, tokens, 1, features, 0, gate_stride, eps, stream);
+}
+
+extern "C" int hipengine_weighted_sum_shared_gate_combine_residual_rmsnorm_gguf_bf16_out(
+    const uint16_t* selected_values, const float* routing_weights, const uint16_t* shared, const float* gate_logits,
+    const uint16_t* residual, const float* norm_weight, uint16_t* norm_out, uint16_t* residual_out, int64_t tokens,
+    int64_t rows_per_token, int64_t features, int64_t gate_stride, float eps, hipStream_t stream) {
+  return launch_moe_tail<TAIL_SLOTS>(selected_values, routing_weights, nullptr, shared, gate_logits, residual,
+                                     norm_weight, norm_out, residual_out, tokens, rows_per_token, features, 0,
+                                     gate_stride, eps, stream);
+}
+
+extern "C" int hipengine_gfx950_moe_gather_tail_rmsnorm_bf16(
+    const uint16_t* down, const int64_t* lane_to_compact, const float* routing_weights, const uint16_t* shared,
+    const float* gate_logits, const uint16_t* residual, const float* norm_weight, uint16_t* norm_out,
+    uint16_t* residual_out, int64_t tokens, int64_t top_k, int64_t features, int64_t compact_rows, int64_t gate_stride,
+    float eps, hipStream_t stream) {
+  return launch_moe_tail<TAIL_GATHER>(down, routing_weights, lane_to_compact, shared, gate_logits, residual, norm_weight,
+                                      norm_out, residual_out, tokens, top_k, features, compact_rows, gate_stride, eps,
+                                      stream);
 }
 
 extern "C" int hipengine_gfx950_moe_weighted_gather_sum(const void* down, const int64_t* lane_to_compact,

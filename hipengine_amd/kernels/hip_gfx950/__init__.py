@@ -24,6 +24,7 @@ def register_backend_kernels(replace: bool = False) -> None:
     global _registered
     if _registered and not replace:
         return
+    from hipengine_amd.kernels.hip_gfx950.fused import paro_combine
     from hipengine_amd.kernels.hip_gfx950.linear import lm_head
     from hipengine_amd.kernels.hip_gfx950.moe import group_scatter, router
     from hipengine_amd.kernels.hip_gfx950.quant import (
@@ -42,4 +43,5 @@ def register_backend_kernels(replace: bool = False) -> None:
     router.register_kernels(BACKEND, replace=True)
     gguf_embedding.register_kernels(BACKEND, replace=True)
     lm_head.register_kernels(BACKEND, replace=True)
+    paro_combine.register_kernels(BACKEND, replace=True)
     _registered = True

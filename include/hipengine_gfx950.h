@@ -493,6 +493,36 @@ int hipengine_gfx950_moe_weighted_gather_sum(const void* down, const int64_t* la
                                              int64_t hidden, int64_t compact_rows, int in_kind, int out_kind,
                                              hipengine_stream_t stream);
 
+/* The MoE tail fused with the next layer's RMSNorm, bf16 rows and a float32 norm weight
+ * (kernels/hip_gfx1100/fused/paro_combine.hip:1505-1579; arithmetic of kernels/cpu_reference/ops.py:33-102):
+ *   residual_out = bf16((residual + selected) + sigmoid(gate_logits[token * gate_stride]) * shared)
+ *   norm_out     = bf16(residual_out / sqrt(mean(residual_out^2) + eps) * norm_weight)
+ * `selected` [tokens, features] is the routed sum, already rounded to bf16.  residual_out may be residual itself.
+ * One workgroup per token; 16-byte accesses when features % 8 == 0, features <= 8192 and the pointers are 16-byte
+ * aligned, any other shape one value at a time.  Products and sums are rounded separately, as the CPU reference
+ * does (hipEngine's HIP kernel lets the compiler contract them: results differ in the last bf16 bit now and then). */
+int hipengine_shared_gate_combine_residual_rmsnorm_gguf_bf16_out(
+    const uint16_t* selected, const uint16_t* shared, const float* gate_logits, const uint16_t* residual,
+    const float* norm_weight, uint16_t* norm_out, uint16_t* residual_out, int64_t tokens, int64_t features,
+    int64_t gate_stride, float eps, hipengine_stream_t stream);
+
+/* The same with the routed sum formed here (kernels/hip_gfx1100/fused/paro_combine.hip:1542-1579): slot rows
+ * selected_values [tokens * rows_per_token, features] (bf16) and routing_weights [tokens * rows_per_token],
+ * acc = acc + value * weight in float32 in slot order, rounded to bf16 before it is added.  rows_per_token <= 4096. */
+int hipengine_weighted_sum_shared_gate_combine_residual_rmsnorm_gguf_bf16_out(
+    const uint16_t* selected_values, const float* routing_weights, const uint16_t* shared, const float* gate_logits,
+    const uint16_t* residual, const float* norm_weight, uint16_t* norm_out, uint16_t* residual_out, int64_t tokens,
+    int64_t rows_per_token, int64_t features, int64_t gate_stride, float eps, hipengine_stream_t stream);
+
+/* The same over the compact rows of the grouped down projection: slot s of token t reads row
+ * lane_to_compact[t * top_k + s] of down [compact_rows, features]; an entry outside [0, compact_rows) contributes
+ * nothing.  Replaces hipengine_gfx950_moe_weighted_gather_sum followed by the tail.  New here. */
+int hipengine_gfx950_moe_gather_tail_rmsnorm_bf16(
+    const uint16_t* down, const int64_t* lane_to_compact, const float* routing_weights, const uint16_t* shared,
+    const float* gate_logits, const uint16_t* residual, const float* norm_weight, uint16_t* norm_out,
+    uint16_t* residual_out, int64_t tokens, int64_t top_k, int64_t features, int64_t compact_rows, int64_t gate_stride,
+    float eps, hipengine_stream_t stream);
+
 /* Decode: out[lane, :] = W[selected[lane]] . x[lane / (rows / x_rows), :] for
  * rows lanes (<= 65535) over x_rows activation rows; lanes with an expert id
  * outside [0, num_experts) are left unwritten.  Activations are quantized to

@@ -50,6 +50,10 @@ router_topk_softmax          brute-force argsort; ties -> lowest index
 mtp_moe_routing              closed form on tiny cases
 build_routing_index          invariants (prefix sums, permutation, stability,
                              compact_to_source = lane // top_k) + brute force
+moe_tail_next_rmsnorm        reference known answer with both rounding boundaries
+                             (tests/test_gpu_moe_tail_next_rmsnorm.py:98-119);
+                             scalar float64 loop on a small case within one bf16 step;
+                             slot-weighted == aggregate of the separately formed sum
 quantize_q4_k / q6_k / q8_0  the reference ships NO fp32->Q4_K/Q6_K quantizer;
                              these only shape test data.  PARITY UNPINNED
                              (and not needed: parity is defined on block
@@ -377,6 +381,60 @@ def moe_ffn_block(x, residual, selected, routing, gate_q, up_q, down_q,
     logit = xa @ np.asarray(shared_gate_logit_w, dtype=np.float32)
     gate = (np.float32(1.0) / (np.float32(1.0) + np.exp(-logit))).astype(np.float32)
     return (np.asarray(residual, dtype=np.float32) + sel_out + gate[:, None] * shared).astype(np.float32)
+
+
+def moe_tail_next_rmsnorm(selected_values, shared, gate_logits, residual, norm_weight, *, routing_weights=None,
+                          lane_to_compact=None, eps: float = 1e-6) -> tuple[np.ndarray, np.ndarray]:
+    """MoE tail and the next layer's RMSNorm with bf16 boundaries (kernels/cpu_reference/ops.py:33-102):
+    the routed sum (given, or formed in slot order in float32, product and sum rounded separately, then rounded
+    to bf16), ``residual' = bf16((residual + selected) + sigmoid(gate[:, 0]) * shared)``,
+    ``norm = bf16(residual' / sqrt(mean(residual'^2) + eps) * weight)`` (ops.py:25-29).
+    ``selected_values`` is ``[tokens, hidden]`` without ``routing_weights``, ``[tokens, top_k, hidden]`` with them,
+    or compact rows ``[compact_rows, hidden]`` with ``lane_to_compact`` ``[tokens * top_k]`` (a lane < 0 or past the
+    compact rows contributes nothing).  Float32 values in, float32 values of the bf16 results out."""
+    res = np.asarray(residual, dtype=np.float32)
+    sh = np.asarray(shared, dtype=np.float32)
+    sel = np.asarray(selected_values, dtype=np.float32)
+    w = np.asarray(norm_weight, dtype=np.float32)
+    if res.ndim != 2 or sh.shape != res.shape or w.shape != (res.shape[1],):
+        raise ValueError("residual and shared must be [tokens, hidden] and norm_weight [hidden]")
+    tokens, hidden = res.shape
+
+    def rnd(v):
+        return bf16_bits_to_f32(f32_to_bf16_bits(np.asarray(v, dtype=np.float32)))
+
+    if routing_weights is None:
+        if sel.shape != res.shape:
+            raise ValueError("an already formed routed sum must match the residual shape")
+        selected_sum = sel
+    else:
+        rw = np.asarray(routing_weights, dtype=np.float32).reshape(tokens, -1)
+        top_k = rw.shape[1]
+        if lane_to_compact is not None:
+            l2c = np.asarray(lane_to_compact, dtype=np.int64).reshape(tokens, top_k)
+            live = (l2c >= 0) & (l2c < sel.shape[0])
+            rows = sel[np.where(live, l2c, 0)]
+            rows = np.where(live[..., None], rows, np.float32(0.0))
+            rw = np.where(live, rw, np.float32(0.0))
+        else:
+            if sel.shape != (tokens, top_k, hidden):
+                raise ValueError("slot values must be [tokens, top_k, hidden]")
+            rows = sel
+        selected_sum = np.zeros_like(res)
+        for slot in range(top_k):
+            selected_sum = (selected_sum + (rows[:, slot] * rw[:, slot, None]).astype(np.float32)).astype(np.float32)
+        selected_sum = rnd(selected_sum)
+    gate = np.asarray(gate_logits, dtype=np.float32)
+    gate_first = gate if gate.ndim == 1 else gate[:, 0]
+    if gate_first.shape != (tokens,):
+        raise ValueError("gate_logits must be [tokens] or [tokens, gate_stride]")
+    sig = (np.float32(1.0) / (np.float32(1.0) + np.exp(-gate_first))).astype(np.float32)
+    combined = (res + selected_sum).astype(np.float32)
+    combined = (combined + (sig[:, None] * sh).astype(np.float32)).astype(np.float32)
+    rounded = rnd(combined)
+    variance = np.mean(rounded * rounded, axis=-1, keepdims=True, dtype=np.float32)
+    inv = np.reciprocal(np.sqrt(variance + np.float32(eps))).astype(np.float32)
+    return rounded, rnd(((rounded * inv).astype(np.float32) * w).astype(np.float32))
 
 
 # --------------------------------------------------------------------------

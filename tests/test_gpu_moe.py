@@ -17,6 +17,7 @@ import numpy as np
 import pytest
 
 from oracle import gguf_oracle as O
+from hipengine_amd.kernels.hip_gfx950.fused import paro_combine as PC
 from hipengine_amd.kernels.hip_gfx950.moe import group_scatter as GS
 from hipengine_amd.kernels.hip_gfx950.moe import router as RT
 from hipengine_amd.kernels.hip_gfx950.quant import gguf_moe as M
@@ -579,3 +580,77 @@ def test_moe_wrappers_reject_bad_arguments(dev):
         M.gguf_q4_k_selected_gemv_bf16_bf16_out(1, 1, 1, 1, 1, 8, 4, 200, 32)
     with pytest.raises(ValueError, match="multiples of 32"):
         M.gguf_q4_k_grouped_mmq(1, 1, 1, 1, 1, 1, 8, 8, 256, 40, 4, 32)
+
+
+def _bf16_steps_apart(got_bits, want_f32):
+    """|got - want| in units of the bf16 spacing at the larger magnitude, the unit no smaller than 1e-6: where the
+    three terms of order 0.2 cancel, a float32 rounding of one of them (1e-8) is many bf16 steps of the tiny sum."""
+    got = O.bf16_bits_to_f32(got_bits)
+    step = np.spacing(np.maximum(np.abs(got), np.abs(want_f32)).astype(np.float32)) * np.float32(65536.0)
+    return np.abs(got - want_f32) / np.maximum(step, np.float32(1e-6))
+
+
+@pytest.mark.parametrize("tokens,hidden", [(1, 17), (3, 2048), (4, 5120), (2, 8200), (130, 256)])
+@pytest.mark.parametrize("mode", ["aggregate", "slots", "gather"])
+def test_moe_tail_next_rmsnorm(dev, mode, tokens, hidden):
+    """The MoE tail fused with the next RMSNorm (hipEngine's GGUF bf16 entries and the form that gathers compact
+    rows) against the restated CPU reference: the combined residual equal bit for bit except where the device's
+    expf moves a value across a bf16 rounding boundary (at most one step, in under 0.5 % of the values); the norm
+    within one bf16 step of the reference's norm of that residual (the sum of squares is taken in another order).  Inputs as in hipEngine's own test
+    (tests/test_gpu_moe_tail_next_rmsnorm.py:147-160): N(0, 0.2) rows, weights in (-0.5, 0.75), gate stride 3."""
+    rng = np.random.default_rng(0x21A0 + tokens * 37 + hidden + len(mode))
+    top_k, gate_stride, eps = 8, 3, 1e-6
+    bits = lambda a: O.f32_to_bf16_bits(a.astype(np.float32))
+    shared_b, residual_b = bits(rng.standard_normal((tokens, hidden)) * 0.2), bits(rng.standard_normal((tokens, hidden)) * 0.2)
+    routing = rng.uniform(-0.5, 0.75, size=(tokens, top_k)).astype(np.float32)
+    gate = rng.uniform(-4.0, 4.0, size=(tokens, gate_stride)).astype(np.float32)
+    weight = rng.uniform(0.5, 1.5, size=hidden).astype(np.float32)
+    d = {"shared": dev.put(shared_b), "residual": dev.put(residual_b), "gate": dev.put(gate), "weight": dev.put(weight),
+         "routing": dev.put(routing), "norm": dev.empty(tokens * hidden * 2, fill=0x5A),
+         "res_out": dev.empty(tokens * hidden * 2, fill=0x5A)}
+    shared, residual = O.bf16_bits_to_f32(shared_b), O.bf16_bits_to_f32(residual_b)
+    if mode == "aggregate":
+        sel_b = bits(rng.standard_normal((tokens, hidden)) * 0.2)
+        d["sel"] = dev.put(sel_b)
+        PC.shared_gate_combine_residual_rmsnorm_gguf_bf16_out(d["sel"].ptr, d["shared"].ptr, d["gate"].ptr,
+                                                              d["residual"].ptr, d["weight"].ptr, d["norm"].ptr,
+                                                              d["res_out"].ptr, tokens, hidden, gate_stride, eps)
+        want_r, want_n = O.moe_tail_next_rmsnorm(O.bf16_bits_to_f32(sel_b), shared, gate, residual, weight, eps=eps)
+    elif mode == "slots":
+        sel_b = bits(rng.standard_normal((tokens, top_k, hidden)) * 0.2)
+        d["sel"] = dev.put(sel_b)
+        PC.weighted_sum_shared_gate_combine_residual_rmsnorm_gguf_bf16_out(
+            d["sel"].ptr, d["routing"].ptr, d["shared"].ptr, d["gate"].ptr, d["residual"].ptr, d["weight"].ptr,
+            d["norm"].ptr, d["res_out"].ptr, tokens, top_k, hidden, gate_stride, eps)
+        want_r, want_n = O.moe_tail_next_rmsnorm(O.bf16_bits_to_f32(sel_b), shared, gate, residual, weight,
+                                                 routing_weights=routing, eps=eps)
+    else:
+        compact_rows = tokens * top_k - 2 if tokens > 1 else tokens * top_k
+        l2c = rng.permutation(tokens * top_k).astype(np.int64)
+        l2c[l2c >= compact_rows] = -1                       # two lanes of no expert
+        sel_b = bits(rng.standard_normal((compact_rows, hidden)) * 0.2)
+        d["sel"], d["l2c"] = dev.put(sel_b), dev.put(l2c)
+        PC.moe_gather_tail_rmsnorm_bf16(d["sel"].ptr, d["l2c"].ptr, d["routing"].ptr, d["shared"].ptr, d["gate"].ptr,
+                                        d["residual"].ptr, d["weight"].ptr, d["norm"].ptr, d["res_out"].ptr, tokens,
+                                        top_k, hidden, compact_rows, gate_stride, eps)
+        want_r, want_n = O.moe_tail_next_rmsnorm(O.bf16_bits_to_f32(sel_b), shared, gate, residual, weight,
+                                                 routing_weights=routing, lane_to_compact=l2c, eps=eps)
+    got_r = dev.get(d["res_out"], np.uint16, (tokens, hidden))
+    got_n = dev.get(d["norm"], np.uint16, (tokens, hidden))
+    # in place: the combined residual over the residual it read
+    PC.shared_gate_combine_residual_rmsnorm_gguf_bf16_out(d["res_out"].ptr, d["shared"].ptr, d["gate"].ptr,
+                                                          d["residual"].ptr, d["weight"].ptr, d["norm"].ptr,
+                                                          d["residual"].ptr, tokens, hidden, gate_stride, eps)
+    again_r = dev.get(d["residual"], np.uint16, (tokens, hidden))
+    want_again, _ = O.moe_tail_next_rmsnorm(O.bf16_bits_to_f32(got_r), shared, gate, residual, weight, eps=eps)
+    dev.free(*d.values())
+    apart_r = _bf16_steps_apart(got_r, want_r)
+    assert apart_r.max() <= 1.0 and np.mean(apart_r == 0) >= 0.995, (apart_r.max(), np.mean(apart_r == 0))
+    # the norm of the combined residual the device formed (where that is a step off, so is its norm)
+    zeros = np.zeros((tokens, hidden), np.float32)
+    _, norm_of_got = O.moe_tail_next_rmsnorm(zeros, zeros, gate, O.bf16_bits_to_f32(got_r), weight, eps=eps)
+    apart_n = _bf16_steps_apart(got_n, norm_of_got)
+    assert apart_n.max() <= 1.0 and np.mean(apart_n == 0) >= 0.97, (apart_n.max(), np.mean(apart_n == 0))
+    assert np.mean(_bf16_steps_apart(got_n, want_n) == 0) >= 0.97
+    apart_again = _bf16_steps_apart(again_r, want_again)
+    assert apart_again.max() <= 1.0 and np.mean(apart_again == 0) >= 0.995

@@ -303,6 +303,13 @@ def test_moe_wrappers_validate_before_touching_the_device():
         M.gguf_q6_k_grouped_mmq(1, 1, 1, 0, 1, 1, 8, 8, 256, 64, 4, 128)
     with pytest.raises(ValueError, match="tile_rows"):
         GS.moe_tile_map(1, 1, 1, 1, 8, tile_rows=48)
+    from hipengine_amd.kernels.hip_gfx950.fused import paro_combine as PC
+    with pytest.raises(ValueError, match="features must be positive"):
+        PC.shared_gate_combine_residual_rmsnorm_gguf_bf16_out(1, 1, 1, 1, 1, 1, 1, 4, 0, 1)
+    with pytest.raises(ValueError, match="rows_per_token must be positive"):
+        PC.weighted_sum_shared_gate_combine_residual_rmsnorm_gguf_bf16_out(1, 1, 1, 1, 1, 1, 1, 1, 4, 0, 64, 1)
+    with pytest.raises(ValueError, match="non-null"):
+        PC.moe_gather_tail_rmsnorm_bf16(1, 0, 1, 1, 1, 1, 1, 1, 1, 4, 8, 64, 32, 1)
     with pytest.raises(ValueError, match="inter"):
         M.moe_silu_mul_d4s4_pack(1, 1, 4, 100)
 

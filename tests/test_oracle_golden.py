@@ -529,3 +529,54 @@ def test_q5_k_block_dots_against_int64_brute_force():
             for j in range(k // 32):
                 assert dots[r, row, j] == int(np.dot(qs[r, j].astype(np.int64), deq[row, j * 32:(j + 1) * 32]))
         assert np.array_equal(qsum[r], qs[r].astype(np.int64).sum(axis=-1))
+
+
+def test_moe_tail_next_rmsnorm_reference_known_answer_and_scalar_loop():
+    """The reference's own known answer (tests/test_gpu_moe_tail_next_rmsnorm.py:98-119: both rounding boundaries,
+    gate taken from column 0), a float64 scalar loop within one bf16 step, and the three input forms agreeing."""
+    selected = np.asarray([[[0.5, -1.0], [0.5, -1.0]]], dtype=np.float32)
+    rounded, normed = O.moe_tail_next_rmsnorm(selected, np.asarray([[2.0, 4.0]], np.float32),
+                                              np.asarray([[0.0, 99.0]], np.float32), np.asarray([[3.0, -1.0]], np.float32),
+                                              np.ones(2, np.float32), routing_weights=np.asarray([[1.0, 1.0]], np.float32))
+    assert np.array_equal(rounded, np.asarray([[5.0, -1.0]], np.float32))
+    scale = np.float32(1.0 / np.sqrt(np.mean(rounded * rounded, axis=-1, keepdims=True) + 1e-6))
+    assert np.array_equal(normed, O.bf16_bits_to_f32(O.f32_to_bf16_bits(rounded * scale)))
+
+    rng = np.random.default_rng(31)
+    tokens, top_k, hidden = 3, 4, 24
+    bf = lambda a: O.bf16_bits_to_f32(O.f32_to_bf16_bits(a.astype(np.float32)))
+    slots = bf(rng.standard_normal((tokens, top_k, hidden)) * 0.3)
+    shared, residual = bf(rng.standard_normal((tokens, hidden)) * 0.3), bf(rng.standard_normal((tokens, hidden)))
+    routing = rng.uniform(-0.5, 0.75, (tokens, top_k)).astype(np.float32)
+    gate = rng.uniform(-4, 4, (tokens, 3)).astype(np.float32)
+    weight = rng.uniform(0.5, 1.5, hidden).astype(np.float32)
+    got_r, got_n = O.moe_tail_next_rmsnorm(slots, shared, gate, residual, weight, routing_weights=routing, eps=1e-5)
+    for t in range(tokens):
+        row, routed = np.empty(hidden), np.empty(hidden)
+        for h in range(hidden):
+            routed[h] = sum(float(slots[t, s, h]) * float(routing[t, s]) for s in range(top_k))
+            row[h] = float(residual[t, h]) + routed[h] + float(shared[t, h]) / (1.0 + np.exp(-float(gate[t, 0])))
+        # two bf16 roundings on the way: half a step of the routed sum, then half a step of the result
+        assert np.all(np.abs(got_r[t] - row) <= (np.abs(routed) + np.abs(row)) * 2.0 ** -8 + 1e-6)
+        norm = got_r[t].astype(np.float64) / np.sqrt(np.mean(got_r[t].astype(np.float64) ** 2) + 1e-5) * weight
+        assert np.all(np.abs(got_n[t] - norm) <= np.abs(norm) * 2.0 ** -8 + 1e-6)
+    # the aggregate form on the separately formed sum, and the gathered form on a permutation of the rows
+    agg = np.zeros((tokens, hidden), np.float32)
+    for s in range(top_k):
+        agg = (agg + (slots[:, s] * routing[:, s, None]).astype(np.float32)).astype(np.float32)
+    r2, n2 = O.moe_tail_next_rmsnorm(bf(agg), shared, gate, residual, weight, eps=1e-5)
+    assert np.array_equal(r2, got_r) and np.array_equal(n2, got_n)
+    perm = rng.permutation(tokens * top_k)
+    compact = np.empty((tokens * top_k, hidden), np.float32)
+    compact[perm] = slots.reshape(-1, hidden)
+    r3, n3 = O.moe_tail_next_rmsnorm(compact, shared, gate, residual, weight, routing_weights=routing,
+                                     lane_to_compact=perm, eps=1e-5)
+    assert np.array_equal(r3, got_r) and np.array_equal(n3, got_n)
+    dropped = perm.copy().reshape(tokens, top_k)
+    dropped[1, 2] = -1
+    r4, _ = O.moe_tail_next_rmsnorm(compact, shared, gate, residual, weight, routing_weights=routing,
+                                    lane_to_compact=dropped, eps=1e-5)
+    routing0 = routing.copy()
+    routing0[1, 2] = 0.0
+    r5, _ = O.moe_tail_next_rmsnorm(slots, shared, gate, residual, weight, routing_weights=routing0, eps=1e-5)
+    assert np.array_equal(r4, r5)
