@@ -277,8 +277,9 @@ class Harness:
             fn = M.gguf_q4_k_q8_1_mmq32_vdr_dense_bf16_f32_out
         else:
             Q.gguf_q8_1_d4s4_f32_quantize_bf16(dx.ptr, dxq.ptr, m, k)
-            fn = (M.gguf_q5_k_mmq32_q8_1_d4s4_f32_bf16_f32_out if quant == "q5_k"
-                  else M.gguf_q6_k_mmq32_q8_1_d4s4_f32_bf16_f32_out)
+            fn = {"q5_k": M.gguf_q5_k_mmq32_q8_1_d4s4_f32_bf16_f32_out,
+                  "q6_k": M.gguf_q6_k_mmq32_q8_1_d4s4_f32_bf16_f32_out,
+                  "q8_0": M.gguf_q8_0_mmq32_q8_1_d4s4_f32_bf16_f32_out}[quant]
         _, ev = self.time_launches(lambda i: fn(dxq.ptr, dw.ptr, dout.ptr, m, k, n), steps, warmup)
         for buf in (dw, dx, dxq, dout):
             self.memory.free(buf)
@@ -542,6 +543,7 @@ def main() -> None:
             "mmq_q4_k_17408x5120_m8192": ("q4_k", 8192, 5120, 17408),
             "mmq_q6_k_5120x17408_m2048": ("q6_k", 2048, 17408, 5120),
             "mmq_q5_k_17408x5120_m2048": ("q5_k", 2048, 5120, 17408),
+            "mmq_q8_0_5120x5120_m2048": ("q8_0", 2048, 5120, 5120),
         }.items():
             sec, ops = h.mmq_case(quant, m, kk, nn, msteps, 2)
             extra[name] = {"us": round(sec * 1e6, 1), "int8_TOPS": round(ops / sec / 1e12, 1),

@@ -13,6 +13,7 @@
 
 #include "gguf_mmq_q4k.hpp"
 #include "gguf_mmq_q6k.hpp"
+#include "gguf_mmq_q8_0.hpp"
 
 #include "gguf_init.hpp"
 
@@ -158,6 +159,61 @@ int launch_q6(const void* xq, const uint8_t* w, void* out, int out_kind, int64_t
   return static_cast<int>(hipGetLastError());
 }
 
+// --------------------------------------------------------------------------
+// Q8_0 x D4S4: the tile engine of gguf_mmq_q8_0.hpp over the dense problem.
+// DUMP: the verification instantiation, which also writes every int32 block dot to dots[M, N, K/32].
+// --------------------------------------------------------------------------
+template <bool DUMP, int COLS = BN>
+__global__ void __launch_bounds__(THREADS, 2) mmq_q8_0_d4s4_kernel(MmqArgs a, int32_t* __restrict__ dots) {
+  extern __shared__ __align__(16) uint8_t smem_raw[];
+  Q8Smem<COLS>& s = *reinterpret_cast<Q8Smem<COLS>*>(smem_raw);
+  const int m0 = blockIdx.x * BM, n0 = blockIdx.y * COLS;
+  const int steps = a.K / 128;
+  const int64_t w_row_bytes = static_cast<int64_t>(a.K / 32) * Q8_0_BYTES;
+  const int64_t x_row_bytes = static_cast<int64_t>(steps) * D4S4_BYTES;
+  auto row_of = [=](int row) { return static_cast<int64_t>(min(m0 + row, a.M - 1)); };
+  auto col_of = [=](int col) { return static_cast<int64_t>(min(n0 + col, a.N - 1)); };
+  auto emit = [=](int row, int col, float v) {
+    const int m = m0 + row, n = n0 + col;
+    if (m < a.M && n < a.N) store_scalar(a.out, static_cast<int64_t>(m) * a.N + n, v, a.out_kind);
+  };
+  if constexpr (DUMP) {
+    q8_tile_run<true, COLS>(a.xq, x_row_bytes, a.w, w_row_bytes, steps, s, row_of, col_of, emit,
+                            [=](int row, int col, int block, int dot) {
+                              const int m = m0 + row, n = n0 + col;
+                              if (m < a.M && n < a.N) dots[(static_cast<int64_t>(m) * a.N + n) * (a.K / 32) + block] = dot;
+                            });
+  } else {
+    q8_tile_run<false, COLS>(a.xq, x_row_bytes, a.w, w_row_bytes, steps, s, row_of, col_of, emit);
+  }
+}
+
+int launch_q8_0(const void* xq, const uint8_t* w, void* out, int out_kind, int64_t M, int64_t K, int64_t N,
+                hipStream_t stream) {
+  if (!xq || !w || !out || M <= 0 || M > (1 << 20) || K <= 0 || (K % 128) != 0 || N <= 0 || N > (1 << 24) ||
+      out_kind < KIND_F32 || out_kind > KIND_F16) {
+    return static_cast<int>(hipErrorInvalidValue);
+  }
+  MmqArgs a{static_cast<const uint8_t*>(xq), w, out, out_kind, static_cast<int>(M), static_cast<int>(K),
+            static_cast<int>(N)};
+  // the tile width by the rule of the Q6_K launch: 64-wide tiles where they fill the rounds of resident
+  // workgroups better
+  const int64_t m_tiles = (M + BM - 1) / BM;
+  const int64_t wide = m_tiles * ((N + 127) / 128), narrow = m_tiles * ((N + 63) / 64);
+  const int64_t slots = 2 * 256;
+  auto fill = [&](int64_t tiles) { return static_cast<double>(tiles) / static_cast<double>((tiles + slots - 1) / slots * slots); };
+  if (Q6_TILE_CHOICE(fill(wide), fill(narrow))) {
+    const dim3 grid(static_cast<unsigned>(m_tiles), static_cast<unsigned>((N + 63) / 64));
+    hipLaunchKernelGGL((mmq_q8_0_d4s4_kernel<false, 64>), grid, dim3(THREADS), sizeof(Q8Smem<64>), stream, a,
+                       static_cast<int32_t*>(nullptr));
+  } else {
+    const dim3 grid(static_cast<unsigned>(m_tiles), static_cast<unsigned>((N + BN - 1) / BN));
+    hipLaunchKernelGGL((mmq_q8_0_d4s4_kernel<false, 128>), grid, dim3(THREADS), sizeof(Q8Smem<128>), stream, a,
+                       static_cast<int32_t*>(nullptr));
+  }
+  return static_cast<int>(hipGetLastError());
+}
+
 }  // namespace
 
 extern "C" int hipengine_gfx950_gguf_q4_k_mmq_tuned(const void* xq, const uint8_t* qweight, void* out, int out_kind,
@@ -212,13 +268,22 @@ DEFINE_MMQ_Q5(hipengine_gguf_q5_k_mmq32_q8_1_d4s4_f32_bf16_bf16_out, KIND_BF16)
 DEFINE_MMQ_Q6(hipengine_gguf_q6_k_mmq32_q8_1_d4s4_f32_bf16_f32_out, KIND_F32)
 DEFINE_MMQ_Q6(hipengine_gguf_q6_k_mmq32_q8_1_d4s4_f32_bf16_bf16_out, KIND_BF16)
 
+#define DEFINE_MMQ_Q8_0(SYMBOL, OKIND)                                                                      \
+  extern "C" int SYMBOL(const void* xq, const uint8_t* qweight, void* out, int64_t rows, int64_t in_features, \
+                        int64_t out_features, hipStream_t stream) {                                         \
+    return launch_q8_0(xq, qweight, out, OKIND, rows, in_features, out_features, stream);                   \
+  }
+
+DEFINE_MMQ_Q8_0(hipengine_gguf_q8_0_mmq32_q8_1_d4s4_f32_bf16_f32_out, KIND_F32)
+DEFINE_MMQ_Q8_0(hipengine_gguf_q8_0_mmq32_q8_1_d4s4_f32_bf16_bf16_out, KIND_BF16)
+
 // ---- verification: the int32 dots the MMQ kernels feed their float32 combine with ----
 
 extern "C" int hipengine_gfx950_gguf_mmq_dots_i32(int32_t ggml_type, const void* xq, const uint8_t* qweight,
                                                   int32_t* dots, float* out, int64_t rows, int64_t in_features,
                                                   int64_t out_features, hipStream_t stream) {
   if (!xq || !qweight || !dots || !out || rows <= 0 || rows > (1 << 20) || in_features <= 0 ||
-      (in_features % QK_K) != 0 || out_features <= 0 || out_features > (1 << 24)) {
+      (in_features % (ggml_type == GGML_Q8_0 ? 128 : QK_K)) != 0 || out_features <= 0 || out_features > (1 << 24)) {
     return static_cast<int>(hipErrorInvalidValue);
   }
   MmqArgs a{static_cast<const uint8_t*>(xq), qweight, out, KIND_F32, static_cast<int>(rows),
@@ -232,6 +297,8 @@ extern "C" int hipengine_gfx950_gguf_mmq_dots_i32(int32_t ggml_type, const void*
     hipLaunchKernelGGL(mmq_tile_dump_kernel<DenseQ5>, grid, dim3(THREADS), sizeof(DenseQ5::Smem), stream, a, dots);
   } else if (ggml_type == GGML_Q6_K) {
     hipLaunchKernelGGL((mmq_q6_k_d4s4_kernel<true, 128>), grid, dim3(THREADS), sizeof(Q6Smem<128>), stream, a, dots);
+  } else if (ggml_type == GGML_Q8_0) {
+    hipLaunchKernelGGL((mmq_q8_0_d4s4_kernel<true, 128>), grid, dim3(THREADS), sizeof(Q8Smem<128>), stream, a, dots);
   } else {
     return static_cast<int>(hipErrorInvalidValue);
   }
@@ -242,8 +309,8 @@ extern "C" int hipengine_gfx950_gguf_mmq_dots_i32(int32_t ggml_type, const void*
 
 extern "C" int hipengine_gfx950_gguf_prefill_workspace_bytes(int32_t ggml_type, int64_t rows, int64_t in_features,
                                                              int64_t* bytes) {
-  if (!bytes || rows <= 0 || in_features <= 0 || (in_features % QK_K) != 0 ||
-      (ggml_type != GGML_Q4_K && ggml_type != GGML_Q5_K && ggml_type != GGML_Q6_K)) {
+  if (!bytes || rows <= 0 || in_features <= 0 || (in_features % (ggml_type == GGML_Q8_0 ? 128 : QK_K)) != 0 ||
+      (ggml_type != GGML_Q4_K && ggml_type != GGML_Q5_K && ggml_type != GGML_Q6_K && ggml_type != GGML_Q8_0)) {
     return static_cast<int>(hipErrorInvalidValue);
   }
   *bytes = rows * (in_features / 128) * (ggml_type == GGML_Q4_K ? DS4_BYTES : D4S4_BYTES);
@@ -272,6 +339,7 @@ extern "C" int hipengine_gfx950_gguf_prefill_bf16(int32_t ggml_type, const void*
     if ((out_features % 32) != 0) return static_cast<int>(hipErrorInvalidValue);
     return launch_q5(workspace, qweight, out, out_kind, rows, in_features, out_features, stream);
   }
+  if (ggml_type == GGML_Q8_0) return launch_q8_0(workspace, qweight, out, out_kind, rows, in_features, out_features, stream);
   return launch_q6(workspace, qweight, out, out_kind, rows, in_features, out_features, stream);
 }
 

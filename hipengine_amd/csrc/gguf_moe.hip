@@ -17,6 +17,7 @@
 #include "gguf_gemv.hpp"
 #include "gguf_mmq_q4k.hpp"
 #include "gguf_mmq_q6k.hpp"
+#include "gguf_mmq_q8_0.hpp"
 
 #include "gguf_init.hpp"
 
@@ -1009,10 +1010,24 @@ struct MoeQ6Args {
 
 constexpr int MOE_Q6_COLS = 64;   // the 128-wide tile spills in this kernel (the row map on top of 243 registers)
 
-__global__ void __launch_bounds__(Q6_THREADS, 2) moe_mmq_q6_k_kernel(MoeQ6Args a) {
+// QT: GGML_Q6_K (the Q6_K tile engine) or GGML_Q8_0 (the Q8_0 one); the same tile shape and row map.
+template <int QT>
+struct MoeWideTile {
+  using Smem = Q6Smem<MOE_Q6_COLS>;
+  static constexpr int64_t row_bytes(int K) { return static_cast<int64_t>(K / QK_K) * Q6_K_BYTES; }
+};
+template <>
+struct MoeWideTile<GGML_Q8_0> {
+  using Smem = Q8Smem<MOE_Q6_COLS>;
+  static constexpr int64_t row_bytes(int K) { return static_cast<int64_t>(K / 32) * Q8_0_BYTES; }
+};
+
+template <int QT>
+__global__ void __launch_bounds__(Q6_THREADS, 2) moe_mmq_wide_kernel(MoeQ6Args a) {
+  using Smem = typename MoeWideTile<QT>::Smem;
   extern __shared__ __align__(16) uint8_t smem_raw[];
-  Q6Smem<MOE_Q6_COLS>& s = *reinterpret_cast<Q6Smem<MOE_Q6_COLS>*>(smem_raw);
-  int* src_row = reinterpret_cast<int*>(smem_raw + sizeof(Q6Smem<MOE_Q6_COLS>));
+  Smem& s = *reinterpret_cast<Smem*>(smem_raw);
+  int* src_row = reinterpret_cast<int*>(smem_raw + sizeof(Smem));
 
   const int tile_row = blockIdx.y;
   const int64_t e = a.tile_expert[tile_row];
@@ -1030,7 +1045,7 @@ __global__ void __launch_bounds__(Q6_THREADS, 2) moe_mmq_q6_k_kernel(MoeQ6Args a
   if (compact_base < 0 || first_compact + valid_rows > a.compact_rows) return;
 
   const int steps = a.K / 128;
-  const int64_t w_row_bytes = static_cast<int64_t>(a.K / QK_K) * Q6_K_BYTES;
+  const int64_t w_row_bytes = MoeWideTile<QT>::row_bytes(a.K);
   const int64_t x_row_bytes = static_cast<int64_t>(steps) * D4S4_BYTES;
   const int64_t stride_rows = a.expert_stride_rows > 0 ? a.expert_stride_rows : local_n;
   const uint8_t* w = (use_b ? a.w_b : a.w_a) + e * stride_rows * w_row_bytes;
@@ -1045,23 +1060,28 @@ __global__ void __launch_bounds__(Q6_THREADS, 2) moe_mmq_q6_k_kernel(MoeQ6Args a
 
   const int64_t out_stride = static_cast<int64_t>(a.Na) + a.Nb;
   const int col_base = (use_b ? a.Na : 0) + n0;
-  q6_tile_run<false, MOE_Q6_COLS>(
-      a.xq, x_row_bytes, w, w_row_bytes, steps, s,
-      [=](int row) { return static_cast<int64_t>(src_row[row]); },
-      [=](int col) { return static_cast<int64_t>(min(n0 + col, local_n - 1)); },
-      [=](int row, int col, float v) {
-        if (row < valid_rows && n0 + col < local_n)
-          store_scalar(a.out, (first_compact + row) * out_stride + col_base + col, v, a.out_kind);
-      });
+  auto row_of = [=](int row) { return static_cast<int64_t>(src_row[row]); };
+  auto col_of = [=](int col) { return static_cast<int64_t>(min(n0 + col, local_n - 1)); };
+  auto emit = [=](int row, int col, float v) {
+    if (row < valid_rows && n0 + col < local_n)
+      store_scalar(a.out, (first_compact + row) * out_stride + col_base + col, v, a.out_kind);
+  };
+  if constexpr (QT == GGML_Q8_0) {
+    q8_tile_run<false, MOE_Q6_COLS>(a.xq, x_row_bytes, w, w_row_bytes, steps, s, row_of, col_of, emit);
+  } else {
+    q6_tile_run<false, MOE_Q6_COLS>(a.xq, x_row_bytes, w, w_row_bytes, steps, s, row_of, col_of, emit);
+  }
 }
 
-int launch_moe_mmq_q6(const void* xq, const int64_t* compact_to_source, const int64_t* expert_start_compact,
+template <int QT>
+int launch_moe_mmq_wide(const void* xq, const int64_t* compact_to_source, const int64_t* expert_start_compact,
                       const int64_t* expert_start_tiles, const int64_t* tile_expert, const uint8_t* w_a,
                       const uint8_t* w_b, void* out, int out_kind, int64_t compact_rows, int64_t source_rows, int64_t K,
                       int64_t Na, int64_t Nb, int64_t num_experts, int64_t total_rows, int64_t expert_stride_rows,
                       hipStream_t stream) {
   if (!xq || !expert_start_compact || !expert_start_tiles || !tile_expert || !w_a || !out || compact_rows <= 0 ||
-      compact_rows > (1 << 24) || source_rows <= 0 || source_rows > (1 << 24) || K <= 0 || (K % QK_K) != 0 ||
+      compact_rows > (1 << 24) || source_rows <= 0 || source_rows > (1 << 24) || K <= 0 ||
+      (K % (QT == GGML_Q8_0 ? 128 : QK_K)) != 0 ||
       Na <= 0 || Nb < 0 || (Nb > 0 && !w_b) || Na + Nb > (1 << 24) || num_experts <= 0 || total_rows <= 0 ||
       (total_rows % Q6_BM) != 0 || total_rows / Q6_BM > 65535 || expert_stride_rows < 0 || out_kind < KIND_F32 ||
       out_kind > KIND_F16) {
@@ -1081,8 +1101,8 @@ int launch_moe_mmq_q6(const void* xq, const int64_t* compact_to_source, const in
   a.tiles_a = static_cast<int>((Na + MOE_Q6_COLS - 1) / MOE_Q6_COLS);
   const int tiles_b = static_cast<int>((Nb + MOE_Q6_COLS - 1) / MOE_Q6_COLS);
   const dim3 grid(static_cast<unsigned>(a.tiles_a + tiles_b), static_cast<unsigned>(total_rows / Q6_BM));
-  hipLaunchKernelGGL(moe_mmq_q6_k_kernel, grid, dim3(Q6_THREADS), sizeof(Q6Smem<MOE_Q6_COLS>) + Q6_BM * sizeof(int),
-                     stream, a);
+  hipLaunchKernelGGL(moe_mmq_wide_kernel<QT>, grid, dim3(Q6_THREADS),
+                     sizeof(typename MoeWideTile<QT>::Smem) + Q6_BM * sizeof(int), stream, a);
   return static_cast<int>(hipGetLastError());
 }
 
@@ -1693,9 +1713,26 @@ extern "C" int hipengine_gfx950_gguf_q6_k_grouped_mmq(const void* x_d4s4, const 
                                                       int64_t out_features_b, int64_t num_experts,
                                                       int64_t total_rows, int64_t expert_stride_rows,
                                                       hipStream_t stream) {
-  return launch_moe_mmq_q6(x_d4s4, compact_to_source, expert_start_compact, expert_start_tiles, tile_expert, qweight_a,
-                           qweight_b, out, out_kind, compact_rows, source_rows, in_features, out_features_a,
-                           out_features_b, num_experts, total_rows, expert_stride_rows, stream);
+  return launch_moe_mmq_wide<GGML_Q6_K>(x_d4s4, compact_to_source, expert_start_compact, expert_start_tiles,
+                                        tile_expert, qweight_a, qweight_b, out, out_kind, compact_rows, source_rows,
+                                        in_features, out_features_a, out_features_b, num_experts, total_rows,
+                                        expert_stride_rows, stream);
+}
+
+// The same for Q8_0 expert weights (34-byte blocks): in_features a multiple of 128.
+extern "C" int hipengine_gfx950_gguf_q8_0_grouped_mmq(const void* x_d4s4, const int64_t* compact_to_source,
+                                                      const int64_t* expert_start_compact,
+                                                      const int64_t* expert_start_tiles, const int64_t* tile_expert,
+                                                      const uint8_t* qweight_a, const uint8_t* qweight_b, void* out,
+                                                      int32_t out_kind, int64_t compact_rows, int64_t source_rows,
+                                                      int64_t in_features, int64_t out_features_a,
+                                                      int64_t out_features_b, int64_t num_experts,
+                                                      int64_t total_rows, int64_t expert_stride_rows,
+                                                      hipStream_t stream) {
+  return launch_moe_mmq_wide<GGML_Q8_0>(x_d4s4, compact_to_source, expert_start_compact, expert_start_tiles,
+                                        tile_expert, qweight_a, qweight_b, out, out_kind, compact_rows, source_rows,
+                                        in_features, out_features_a, out_features_b, num_experts, total_rows,
+                                        expert_stride_rows, stream);
 }
 
 // The tile map for tiles of any height (hipengine_qwen35_moe_mmq32_tile_map is the 32-row one).

@@ -17,19 +17,20 @@ from hipengine_amd.kernels.registry import KernelKey, register
 _ARGS = [VOID, VOID, VOID, I64, I64, I64, VOID]
 
 
-def _validate(rows: int, hidden: int, out_features: int, out_multiple: int) -> None:
+def _validate(rows: int, hidden: int, out_features: int, out_multiple: int, hidden_multiple: int = 256) -> None:
     if rows <= 0 or rows > (1 << 20):
         raise ValueError("rows must be in 1..2^20")
-    if hidden <= 0 or hidden % 256 != 0:
-        raise ValueError("hidden must be positive and divisible by the GGUF block size 256")
+    if hidden <= 0 or hidden % hidden_multiple != 0:
+        raise ValueError("hidden must be positive and divisible by " +
+                         ("the GGUF block size 256" if hidden_multiple == 256 else f"{hidden_multiple}"))
     if out_features <= 0 or out_features % out_multiple != 0:
         raise ValueError(f"out_features must be positive and divisible by {out_multiple}")
 
 
-def _make(name: str, symbol: str, out_multiple: int):
+def _make(name: str, symbol: str, out_multiple: int, hidden_multiple: int = 256):
     def wrapper(xq_ptr: int, qweight_ptr: int, out_ptr: int, rows: int, hidden: int, out_features: int, *,
                 stream: int = 0, library: ctypes.CDLL | None = None, runtime: HipRuntime | None = None) -> None:
-        _validate(rows, hidden, out_features, out_multiple)
+        _validate(rows, hidden, out_features, out_multiple, hidden_multiple)
         validate_pointers(xq_ptr=xq_ptr, qweight_ptr=qweight_ptr, out_ptr=out_ptr)
         check_launch(entry(symbol, _ARGS, library)(xq_ptr, qweight_ptr, out_ptr, rows, hidden, out_features, stream),
                      runtime)
@@ -56,6 +57,12 @@ gguf_q6_k_mmq32_q8_1_d4s4_f32_bf16_f32_out = _make(
     "gguf_q6_k_mmq32_q8_1_d4s4_f32_bf16_f32_out", "hipengine_gguf_q6_k_mmq32_q8_1_d4s4_f32_bf16_f32_out", 1)
 gguf_q6_k_mmq32_q8_1_d4s4_f32_bf16_bf16_out = _make(
     "gguf_q6_k_mmq32_q8_1_d4s4_f32_bf16_bf16_out", "hipengine_gguf_q6_k_mmq32_q8_1_d4s4_f32_bf16_bf16_out", 1)
+
+# Q8_0 x D4S4 (new here: hipEngine has no MMQ for Q8_0): 128 values per D4S4 block
+gguf_q8_0_mmq32_q8_1_d4s4_f32_bf16_f32_out = _make(
+    "gguf_q8_0_mmq32_q8_1_d4s4_f32_bf16_f32_out", "hipengine_gguf_q8_0_mmq32_q8_1_d4s4_f32_bf16_f32_out", 1, 128)
+gguf_q8_0_mmq32_q8_1_d4s4_f32_bf16_bf16_out = _make(
+    "gguf_q8_0_mmq32_q8_1_d4s4_f32_bf16_bf16_out", "hipengine_gguf_q8_0_mmq32_q8_1_d4s4_f32_bf16_bf16_out", 1, 128)
 
 
 def gguf_q4_k_q8_1_mmq_tuned(xq_ptr: int, qweight_ptr: int, out_ptr: int, rows: int, hidden: int, out_features: int, *,
@@ -88,3 +95,7 @@ def register_kernels(backend: str = "hip_gfx950", *, replace: bool = False) -> N
              gguf_q6_k_mmq32_q8_1_d4s4_f32_bf16_f32_out, replace=replace)
     register(KernelKey(backend, "linear", "gguf_q6_k", "mmq32_q8_1_d4s4_f32_bf16_bf16_out"),
              gguf_q6_k_mmq32_q8_1_d4s4_f32_bf16_bf16_out, replace=replace)
+    register(KernelKey(backend, "linear", "gguf_q8_0", "mmq32_q8_1_d4s4_f32_bf16_f32_out"),
+             gguf_q8_0_mmq32_q8_1_d4s4_f32_bf16_f32_out, replace=replace)
+    register(KernelKey(backend, "linear", "gguf_q8_0", "mmq32_q8_1_d4s4_f32_bf16_bf16_out"),
+             gguf_q8_0_mmq32_q8_1_d4s4_f32_bf16_bf16_out, replace=replace)

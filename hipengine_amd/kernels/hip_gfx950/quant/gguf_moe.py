@@ -341,13 +341,15 @@ def gguf_q6_k_grouped_mmq(x_d4s4_ptr: int, expert_start_compact_ptr: int, expert
                           in_features: int, out_features_a: int, num_experts: int, total_rows: int, *,
                           compact_to_source_ptr: int = 0, qweight_b_ptr: int = 0, out_features_b: int = 0,
                           out_dtype: str = "f32", expert_stride_rows: int = 0, stream: int = 0,
-                          library: ctypes.CDLL | None = None, runtime: HipRuntime | None = None) -> None:
+                          library: ctypes.CDLL | None = None, runtime: HipRuntime | None = None,
+                          _symbol: str = "hipengine_gfx950_gguf_q6_k_grouped_mmq", _block: int = 256) -> None:
     """The expert-grouped MMQ for Q6_K experts over D4S4 activation blocks and a map of 128-row tiles
     (``hipengine_gfx950_gguf_q6_k_grouped_mmq``; tile map from ``group_scatter.moe_tile_map(..., tile_rows=128)``)."""
     if compact_rows <= 0 or num_experts <= 0 or source_rows <= 0:
         raise ValueError("compact_rows, source_rows and num_experts must be positive")
-    if in_features <= 0 or in_features % 256 != 0:
-        raise ValueError("in_features must be positive and divisible by the GGUF block size 256")
+    if in_features <= 0 or in_features % _block != 0:
+        raise ValueError("in_features must be positive and divisible by " +
+                         ("the GGUF block size 256" if _block == 256 else f"{_block}"))
     if out_features_a <= 0 or out_features_b < 0:
         raise ValueError("out_features_a must be positive and out_features_b non-negative")
     if total_rows <= 0 or total_rows % 128 != 0:
@@ -355,11 +357,21 @@ def gguf_q6_k_grouped_mmq(x_d4s4_ptr: int, expert_start_compact_ptr: int, expert
     validate_pointers(x_d4s4_ptr=x_d4s4_ptr, expert_start_compact_ptr=expert_start_compact_ptr,
                       expert_start_tiles_ptr=expert_start_tiles_ptr, tile_expert_ptr=tile_expert_ptr,
                       qweight_a_ptr=qweight_a_ptr, out_ptr=out_ptr)
-    fn = entry("hipengine_gfx950_gguf_q6_k_grouped_mmq", [VOID] * 8 + [I32] + [I64] * 8 + [VOID], library)
+    fn = entry(_symbol, [VOID] * 8 + [I32] + [I64] * 8 + [VOID], library)
     check_launch(fn(x_d4s4_ptr, compact_to_source_ptr or None, expert_start_compact_ptr, expert_start_tiles_ptr,
                     tile_expert_ptr, qweight_a_ptr, qweight_b_ptr or None, out_ptr, _KIND[out_dtype], compact_rows,
                     source_rows, in_features, out_features_a, out_features_b, num_experts, total_rows,
                     expert_stride_rows, stream), runtime)
+
+
+def gguf_q8_0_grouped_mmq(x_d4s4_ptr: int, expert_start_compact_ptr: int, expert_start_tiles_ptr: int,
+                          tile_expert_ptr: int, qweight_a_ptr: int, out_ptr: int, compact_rows: int, source_rows: int,
+                          in_features: int, out_features_a: int, num_experts: int, total_rows: int, **kwargs) -> None:
+    """``gguf_q6_k_grouped_mmq`` for Q8_0 experts (the same 128-row tile map and keyword arguments, in_features a
+    multiple of 128; C symbol ``hipengine_gfx950_gguf_q8_0_grouped_mmq``)."""
+    gguf_q6_k_grouped_mmq(x_d4s4_ptr, expert_start_compact_ptr, expert_start_tiles_ptr, tile_expert_ptr, qweight_a_ptr,
+                          out_ptr, compact_rows, source_rows, in_features, out_features_a, num_experts, total_rows,
+                          _symbol="hipengine_gfx950_gguf_q8_0_grouped_mmq", _block=128, **kwargs)
 
 
 def moe_weighted_gather_sum(down_ptr: int, lane_to_compact_ptr: int, routing_weights_ptr: int, out_ptr: int,
@@ -412,6 +424,8 @@ def register_kernels(backend: str = "hip_gfx950", *, replace: bool = False) -> N
     register(KernelKey(backend, "moe_linear", "gguf_q6_k", "grouped_mmq128_q8_1_d4s4"), gguf_q6_k_grouped_mmq,
              replace=replace)
     register(KernelKey(backend, "moe_linear", "gguf_q5_k", "grouped_mmq32_q8_1_d4s4"), gguf_q5_k_grouped_mmq,
+             replace=replace)
+    register(KernelKey(backend, "moe_linear", "gguf_q8_0", "grouped_mmq128_q8_1_d4s4"), gguf_q8_0_grouped_mmq,
              replace=replace)
     for quant in ("gguf_q4_k", "gguf_q5_k", "gguf_q6_k", "gguf_q8_0"):     # Q5_K and Q8_0: the single form
         register(KernelKey(backend, "moe_linear", quant, "selected_gemv_q8_1"), gguf_selected_gemv, replace=replace)

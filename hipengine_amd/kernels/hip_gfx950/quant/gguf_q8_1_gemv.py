@@ -83,7 +83,7 @@ _PREFILL_ARGS = [I32, VOID, VOID, VOID, I32, I64, I64, I64, VOID, I64, VOID]
 
 def gguf_prefill_workspace_bytes(quant_key: str, rows: int, in_features: int) -> int:
     """Bytes of the workspace a ``prefill_bf16_*`` call takes to run on the MMQ (0: that quant has none)."""
-    if quant_key not in ("gguf_q4_k", "gguf_q5_k", "gguf_q6_k"):
+    if quant_key not in ("gguf_q4_k", "gguf_q5_k", "gguf_q6_k", "gguf_q8_0") or in_features % 128:
         return 0
     return rows * (in_features // 128) * (144 if quant_key == "gguf_q4_k" else 160)
 
@@ -99,7 +99,7 @@ def _make_dense(quant: str, family: str, act: str, out: str):
         validate_pointers(x_ptr=x_ptr, qweight_ptr=qweight_ptr, out_ptr=out_ptr)
         need = gguf_prefill_workspace_bytes(quant_key, rows, in_features)
         if (family == "prefill" and act == "bf16" and rows >= _MMQ_MIN_ROWS and workspace_ptr and need
-                and workspace_bytes >= need and (quant == "q6_k" or out_features % 32 == 0)):
+                and workspace_bytes >= need and (quant in ("q6_k", "q8_0") or out_features % 32 == 0)):
             code = entry("hipengine_gfx950_gguf_prefill_bf16", _PREFILL_ARGS, library)(
                 QUANT_KEY_TO_GGML[quant_key], x_ptr, qweight_ptr, out_ptr, _KINDS[out], rows, in_features, out_features,
                 workspace_ptr, workspace_bytes, stream)

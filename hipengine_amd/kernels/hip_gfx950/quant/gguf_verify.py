@@ -62,13 +62,14 @@ def gguf_gemv_mfma_dots_i32(quant_key: str, form: int, xq_ptr: int, qweight_ptr:
 def gguf_mmq_dots_i32(quant_key: str, xq_ptr: int, qweight_ptr: int, dots_ptr: int, out_ptr: int, rows: int,
                       in_features: int, out_features: int, *, stream: int = 0, library: ctypes.CDLL | None = None,
                       runtime: HipRuntime | None = None) -> None:
-    """The int32 dots of the MMQ prefill GEMM (Q4_K over DS4 blocks and Q5_K over D4S4 blocks: ``[rows, N, K/32]``;
-    Q6_K over D4S4 blocks: ``[rows, N, K/16]``, centred values) and its float32 result, from the production tile
-    engine."""
-    if rows <= 0 or out_features <= 0 or in_features <= 0 or in_features % 256:
-        raise ValueError("rows/out_features must be positive and in_features divisible by 256")
-    if quant_key not in ("gguf_q4_k", "gguf_q5_k", "gguf_q6_k"):
-        raise ValueError("the MMQ takes gguf_q4_k, gguf_q5_k or gguf_q6_k weights")
+    """The int32 dots of the MMQ prefill GEMM (Q4_K over DS4 blocks, Q5_K and Q8_0 over D4S4 blocks:
+    ``[rows, N, K/32]``; Q6_K over D4S4 blocks: ``[rows, N, K/16]``, centred values) and its float32 result, from
+    the production tile engine."""
+    if quant_key not in ("gguf_q4_k", "gguf_q5_k", "gguf_q6_k", "gguf_q8_0"):
+        raise ValueError("the MMQ takes gguf_q4_k, gguf_q5_k, gguf_q6_k or gguf_q8_0 weights")
+    block = 128 if quant_key == "gguf_q8_0" else 256
+    if rows <= 0 or out_features <= 0 or in_features <= 0 or in_features % block:
+        raise ValueError(f"rows/out_features must be positive and in_features divisible by {block}")
     validate_pointers(xq_ptr=xq_ptr, qweight_ptr=qweight_ptr, dots_ptr=dots_ptr, out_ptr=out_ptr)
     fn = entry("hipengine_gfx950_gguf_mmq_dots_i32", [I32, VOID, VOID, VOID, VOID, I64, I64, I64, VOID], library)
     check_launch(fn(QUANT_KEY_TO_GGML[quant_key], xq_ptr, qweight_ptr, dots_ptr, out_ptr, rows, in_features,

@@ -316,10 +316,22 @@ int hipengine_gguf_q6_k_mmq32_q8_1_d4s4_f32_bf16_bf16_out(const void* xq, const 
                                                           int64_t rows, int64_t in_features, int64_t out_features,
                                                           hipengine_stream_t stream);
 
+/* Raw Q8_0 weights ([out_features, in_features/32 * 34]) x D4S4 activations: sum over the 32-value blocks of
+ * xd_b * d_b * dot_b, the q8_1 x Q8_0 formula (gguf_q8_0_dp4a_gemv.hip:100-137) with the float32 activation scales
+ * of the D4S4 block, on the int8 MFMA.  in_features a multiple of 128; any out_features >= 1.  hipEngine has no MMQ
+ * for Q8_0 (its Q8_0 prefill names run the GEMV over row chunks); named after the k-quant MMQ entries.  New here. */
+int hipengine_gguf_q8_0_mmq32_q8_1_d4s4_f32_bf16_f32_out(const void* xq, const uint8_t* qweight, void* out,
+                                                         int64_t rows, int64_t in_features, int64_t out_features,
+                                                         hipengine_stream_t stream);
+int hipengine_gguf_q8_0_mmq32_q8_1_d4s4_f32_bf16_bf16_out(const void* xq, const uint8_t* qweight, void* out,
+                                                          int64_t rows, int64_t in_features, int64_t out_features,
+                                                          hipengine_stream_t stream);
+
 /* Prefill from bf16 activations in one call: x [rows, in_features] bf16 is packed into `workspace`
- * (DS4 blocks for Q4_K, D4S4 for Q5_K and Q6_K; caller-owned, 16-byte aligned, at least the byte count
+ * (DS4 blocks for Q4_K, D4S4 for Q5_K, Q6_K and Q8_0; caller-owned, 16-byte aligned, at least the byte count
  * hipengine_gfx950_gguf_prefill_workspace_bytes reports = rows * in_features/128 * 144 or 160) and the MMQ
- * above runs on it: two launches.  ggml_type 12 (Q4_K), 13 (Q5_K; both out_features % 32 == 0) or 14 (Q6_K); out_kind 0
+ * above runs on it: two launches.  ggml_type 12 (Q4_K), 13 (Q5_K; both out_features % 32 == 0), 14 (Q6_K) or 8
+ * (Q8_0, in_features % 128 == 0); out_kind 0
  * float32, 1 bf16, 2 fp16.  This is what a ("linear", quant, "prefill_bf16_*_out") caller with 32 or more
  * rows should reach: hipEngine's prefill signature has no workspace argument, so the Python wrappers of the
  * prefill keys take it as an optional keyword and fall back to batches of 8 rows through the GEMV without
@@ -697,6 +709,18 @@ int hipengine_gfx950_gguf_q6_k_grouped_mmq(const void* x_d4s4, const int64_t* co
                                            int64_t total_rows, int64_t expert_stride_rows,
                                            hipengine_stream_t stream);
 
+/* hipengine_gfx950_gguf_q6_k_grouped_mmq for Q8_0 expert weights [num_experts, out_features, K/32 * 34]: the same
+ * arguments, 128-row tile map and limits, in_features a multiple of 128; the arithmetic of
+ * hipengine_gguf_q8_0_mmq32_q8_1_d4s4_f32_bf16_*_out per expert.  New here. */
+int hipengine_gfx950_gguf_q8_0_grouped_mmq(const void* x_d4s4, const int64_t* compact_to_source,
+                                           const int64_t* expert_start_compact, const int64_t* expert_start_tiles,
+                                           const int64_t* tile_expert, const uint8_t* qweight_a,
+                                           const uint8_t* qweight_b, void* out, int32_t out_kind,
+                                           int64_t compact_rows, int64_t source_rows, int64_t in_features,
+                                           int64_t out_features_a, int64_t out_features_b, int64_t num_experts,
+                                           int64_t total_rows, int64_t expert_stride_rows,
+                                           hipengine_stream_t stream);
+
 /* hipengine_qwen35_moe_mmq32_tile_map for tiles of tile_rows = 32, 64 or 128 rows.  New here. */
 int hipengine_gfx950_moe_tile_map(const int64_t* expert_start_compact, int64_t* tile_expert_start,
                                   int64_t* tile_expert, int64_t* total_out, int64_t num_experts,
@@ -729,8 +753,9 @@ int hipengine_gfx950_gguf_gemv_mfma_dots_i32(int32_t ggml_type, int32_t form, co
                                              int64_t out_features, hipengine_stream_t stream);
 
 /* The same for the MMQ prefill GEMM: ggml_type 12 (Q4_K, xq = DS4 blocks, dots int32 [rows, N, K/32]), 13 (Q5_K,
- * xq = D4S4 blocks, dots [rows, N, K/32]) or 14
- * (Q6_K, xq = D4S4 blocks, dots [rows, N, K/16], of the centred 6-bit values); out: float32 [rows, N]. */
+ * xq = D4S4 blocks, dots [rows, N, K/32]), 14
+ * (Q6_K, xq = D4S4 blocks, dots [rows, N, K/16], of the centred 6-bit values) or 8 (Q8_0, xq = D4S4 blocks, dots
+ * [rows, N, K/32]); out: float32 [rows, N]. */
 int hipengine_gfx950_gguf_mmq_dots_i32(int32_t ggml_type, const void* xq, const uint8_t* qweight, int32_t* dots,
                                        float* out, int64_t rows, int64_t in_features, int64_t out_features,
                                        hipengine_stream_t stream);

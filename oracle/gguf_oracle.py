@@ -43,6 +43,7 @@ quantize_q8_1                float64 brute force, invariants (|q|<=127,
 pack_q8_1_ds4                same, half-to-even tie case, fp16 clamp case
 pack_q8_1_d4s4               same, summation tree spelled out independently
 block_dots_*                 int64 einsum over independently unpacked integers
+mmq_q8_0_d4s4                float64 product of the dequantized weight and activations
 gemv_q8_1_* / mmq_*          float64 evaluation of the same formula
                              (tests/test_gpu_gguf_q4_k_q8_1_mmq_prefill.py
                              :115-165 style)
@@ -686,6 +687,20 @@ def mmq_q5_k_d4s4(xd4s4, qweight, dtype=np.float64) -> np.ndarray:
     ds, dm = _q4_k_scales_f32(qw, Q5_K_BLOCK_BYTES)
     main = (ds[None].astype(dtype) * xd[:, None, :].astype(dtype) * dots.astype(dtype)).sum(axis=-1)
     return main - xs.astype(dtype) @ dm.astype(dtype).T
+
+
+def mmq_q8_0_d4s4(xd4s4, qweight, dtype=np.float64) -> np.ndarray:
+    """D4S4 x Q8_0 MMQ: ``sum_b xd_b * wd_b * dot_b`` over the 32-value blocks: the q8_1 x Q8_0 formula
+    (gguf_q8_0_dp4a_gemv.hip:100-137) with the float32 activation scales of the D4S4 block
+    (gguf_k_mmq_prefill.hip:655-664).  hipEngine has no such kernel; pinned by the float64 product of the
+    dequantized weight with the dequantized activations."""
+    xd, _, qs = d4s4_fields(xd4s4)
+    qw = np.asarray(qweight)
+    n = qw.shape[0]
+    blocks, _ = _as_blocks(qw, Q8_0_BLOCK_BYTES)
+    wd = _fp16_field(blocks, 0).reshape(n, -1)
+    dots = block_dots_q8_0(qs, qw)
+    return (wd[None].astype(dtype) * xd[:, None, :].astype(dtype) * dots.astype(dtype)).sum(axis=-1)
 
 
 def mmq_q6_k_d4s4(xd4s4, qweight, dtype=np.float64) -> np.ndarray:

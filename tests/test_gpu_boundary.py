@@ -108,7 +108,7 @@ def test_rowtile_keys_are_the_batch_launch(dev, quant):
     dev.free(dw)
 
 
-@pytest.mark.parametrize("quant,n", [("gguf_q4_k", 352), ("gguf_q6_k", 333), ("gguf_q5_k", 160)])
+@pytest.mark.parametrize("quant,n", [("gguf_q4_k", 352), ("gguf_q6_k", 333), ("gguf_q5_k", 160), ("gguf_q8_0", 75)])
 def test_prefill_key_with_workspace_runs_the_mmq(dev, quant, n):
     """prefill_bf16_f32_out with 32 rows or more and a caller-owned workspace packs the activations and runs the
     int8-MFMA MMQ: results equal the MMQ formula of the oracle, and agree with the workspace-free route (GEMV in
@@ -134,6 +134,9 @@ def test_prefill_key_with_workspace_runs_the_mmq(dev, quant, n):
     elif quant == "gguf_q5_k":
         want_pack = O.pack_q8_1_d4s4(xb)
         ref = O.mmq_q5_k_d4s4(want_pack, w)
+    elif quant == "gguf_q8_0":
+        want_pack = O.pack_q8_1_d4s4(xb)
+        ref = O.mmq_q8_0_d4s4(want_pack, w)
     else:
         want_pack = O.pack_q8_1_d4s4(xb)
         ref = O.mmq_q6_k_d4s4(want_pack, w)
@@ -459,7 +462,7 @@ def test_gemv_mfma_forms_int32_dots_bit_exact(dev, quant, form, k, n, rows):
 
 
 @pytest.mark.parametrize("quant,rows,k,n", [("gguf_q4_k", 150, 1024, 160), ("gguf_q6_k", 129, 768, 130),
-                                            ("gguf_q5_k", 131, 1280, 96)])
+                                            ("gguf_q5_k", 131, 1280, 96), ("gguf_q8_0", 133, 640, 77)])
 def test_mmq_int32_dots_bit_exact(dev, quant, rows, k, n):
     """The int32 tiles of the MMQ prefill GEMM (v_mfma_i32_32x32x32_i8 / 32x32x16) against the oracle's integer
     dots of the same packed activations; ragged tiles in both dimensions."""
@@ -477,6 +480,11 @@ def test_mmq_int32_dots_bit_exact(dev, quant, rows, k, n):
         qs = O.d4s4_fields(xq)[2].reshape(rows, k // 32, 32)
         want, per = O.block_dots_q5_k(qs, w)[0], k // 32
         ref = O.mmq_q5_k_d4s4(xq, w)
+    elif quant == "gguf_q8_0":
+        xq = O.pack_q8_1_d4s4(xb)
+        qs = O.d4s4_fields(xq)[2].reshape(rows, k // 32, 32)
+        want, per = O.block_dots_q8_0(qs, w), k // 32
+        ref = O.mmq_q8_0_d4s4(xq, w)
     else:
         xq = O.pack_q8_1_d4s4(xb)
         qs = O.d4s4_fields(xq)[2].reshape(rows, k // 32, 32)

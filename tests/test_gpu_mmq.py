@@ -185,6 +185,31 @@ def test_q6_k_mmq_closed_form_bf16_and_determinism(dev):
     assert np.array_equal(b16, O.f32_to_bf16_bits(f32))
 
 
+@pytest.mark.parametrize("rows,k,n", [(1, 128, 1), (7, 384, 33), (128, 1024, 128), (130, 640, 160), (300, 5120, 200),
+                                      (2560, 256, 4096)])
+def test_q8_0_mmq_matches_formula_and_cpu_reference(dev, rows, k, n):
+    """Q8_0 x D4S4 on the int8 MFMA (K a multiple of 128, any N; the last shape takes 64-wide tiles): the formula in
+    float64, the reference CPU GEMV on the dequantized activations, bf16 output = bf16(float32 output), repeatable."""
+    xb = _bf16_rows(3 * rows + k + n, rows, k, scale=0.1, offset=0.002)
+    d4 = O.pack_q8_1_d4s4(xb)
+    w = O.random_weight(O.GGML_Q8_0, n, k, seed=k + n + 2)
+    got = _run_q4(dev, M.gguf_q8_0_mmq32_q8_1_d4s4_f32_bf16_f32_out, d4, w, rows, k, n)
+    pick = np.arange(rows) if rows <= 300 else np.array([0, 1, 31, 32, 127, 128, 1000, 2047, 2048, 2559])
+    want = O.mmq_q8_0_d4s4(d4[pick], w)
+    assert O.max_rel_err(got[pick], want) <= 1e-3 and O.cosine(got[pick], want) >= 0.99999
+    xd, _, qs = O.d4s4_fields(d4[pick])
+    xdeq = (xd[..., None] * qs.astype(np.float32)).reshape(len(pick), k)
+    ref = O.gguf_quant_gemv(xdeq, w, O.GGML_Q8_0)
+    assert O.max_rel_err(got[pick], ref) <= 1e-3 and O.cosine(got[pick], ref) >= 0.99999
+    again = _run_q4(dev, M.gguf_q8_0_mmq32_q8_1_d4s4_f32_bf16_f32_out, d4, w, rows, k, n)
+    assert np.array_equal(got.view(np.uint32), again.view(np.uint32))
+    b16 = _run_q4(dev, M.gguf_q8_0_mmq32_q8_1_d4s4_f32_bf16_bf16_out, d4, w, rows, k, n, out_dtype=np.uint16)
+    assert np.array_equal(b16, O.f32_to_bf16_bits(got))
+    if rows > 300:      # the first 128 rows alone take wide tiles: the same bits
+        wide = _run_q4(dev, M.gguf_q8_0_mmq32_q8_1_d4s4_f32_bf16_f32_out, d4[:128], w, 128, k, n)
+        assert np.array_equal(got[:128].view(np.uint32), wide.view(np.uint32))
+
+
 def _random_q5_k(n, k, seed):
     """Random valid Q5_K blocks (the oracle has no fp32 -> Q5_K quantizer): every field drawn uniformly."""
     rng = np.random.default_rng(seed)

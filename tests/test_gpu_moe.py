@@ -340,18 +340,21 @@ def test_grouped_mmq_matches_dense_formula_per_expert(dev, tokens, top_k, expert
     (300, 4, 6, 1024, 200, 0, False),      # experts of several 128-row tiles (about 200 rows each)
     (64, 1, 5, 768, 130, 64, True),        # compact rows read as they are (an already gathered intermediate)
 ])
-def test_grouped_mmq_q6_k_matches_dense_formula_per_expert(dev, tokens, top_k, experts, k, na, nb, identity):
-    """The expert-grouped MMQ for Q6_K experts over D4S4 blocks and a map of 128-row tiles: per expert the float64
-    value of the dense Q6_K x D4S4 formula on the rows it owns; rows of no expert and tiles past an expert's rows
+@pytest.mark.parametrize("quant", ["q6_k", "q8_0"])
+def test_grouped_mmq_q6_k_matches_dense_formula_per_expert(dev, quant, tokens, top_k, experts, k, na, nb, identity):
+    """The expert-grouped MMQ for Q6_K and for Q8_0 experts over D4S4 blocks and a map of 128-row tiles: per expert
+    the float64 value of the dense formula on the rows it owns; rows of no expert and tiles past an expert's rows
     stay unwritten."""
+    qt, run, formula = ((O.GGML_Q6_K, M.gguf_q6_k_grouped_mmq, O.mmq_q6_k_d4s4) if quant == "q6_k"
+                        else (O.GGML_Q8_0, M.gguf_q8_0_grouped_mmq, O.mmq_q8_0_d4s4))
     sel, wts = _routing(tokens * 5 + k, tokens, top_k, experts, bad=tokens > 20)
     host, d = _device_index(dev, sel, wts, experts)
     total, lanes = host["total"], tokens * top_k
     rows_src = total if identity else tokens
     x = (np.random.default_rng(k).standard_normal((rows_src, k)) * 0.2).astype(np.float32)
     d4s4 = O.pack_q8_1_d4s4(O.f32_to_bf16_bits(x))
-    w_a = _experts(O.GGML_Q6_K, experts, na, k, seed=13)
-    w_b = _experts(O.GGML_Q6_K, experts, nb, k, seed=14) if nb else None
+    w_a = _experts(qt, experts, na, k, seed=13)
+    w_b = _experts(qt, experts, nb, k, seed=14) if nb else None
     cap = lanes // 128 + experts
     ts, te, tt = dev.empty((experts + 1) * 8), dev.empty(cap * 8, fill=0x11), dev.empty(8)
     GS.moe_tile_map(d["expert_start"].ptr, ts.ptr, te.ptr, tt.ptr, experts, tile_rows=128, tile_capacity=cap)
@@ -362,9 +365,8 @@ def test_grouped_mmq_q6_k_matches_dense_formula_per_expert(dev, tokens, top_k, e
     dxq, dwa = dev.put(d4s4), dev.put(w_a)
     dwb = dev.put(w_b) if nb else None
     dout = dev.empty((total + 1) * (na + nb) * 4, fill=0x7D)
-    M.gguf_q6_k_grouped_mmq(dxq.ptr, d["expert_start"].ptr, ts.ptr, te.ptr, dwa.ptr, dout.ptr, total, rows_src, k, na,
-                            experts, cap * 128, compact_to_source_ptr=0 if identity else d["c2s"].ptr,
-                            qweight_b_ptr=dwb.ptr if dwb else 0, out_features_b=nb)
+    run(dxq.ptr, d["expert_start"].ptr, ts.ptr, te.ptr, dwa.ptr, dout.ptr, total, rows_src, k, na, experts, cap * 128,
+        compact_to_source_ptr=0 if identity else d["c2s"].ptr, qweight_b_ptr=dwb.ptr if dwb else 0, out_features_b=nb)
     got = dev.get(dout, np.float32, (total + 1, na + nb))
     dev.free(dxq, dwa, dout, ts, te, tt, *([dwb] if dwb else []))
     assert np.all(got[total].view(np.uint32) == 0x7D7D7D7D)
@@ -374,10 +376,10 @@ def test_grouped_mmq_q6_k_matches_dense_formula_per_expert(dev, tokens, top_k, e
         if hi == lo:
             continue
         src = np.arange(lo, hi) if identity else host["c2s"][lo:hi]
-        want_a = O.mmq_q6_k_d4s4(d4s4[src], w_a[e])
+        want_a = formula(d4s4[src], w_a[e])
         assert O.max_rel_err(got[lo:hi, :na], want_a) <= REL_TOL and O.cosine(got[lo:hi, :na], want_a) >= COS_MIN
         if nb:
-            want_b = O.mmq_q6_k_d4s4(d4s4[src], w_b[e])
+            want_b = formula(d4s4[src], w_b[e])
             assert O.max_rel_err(got[lo:hi, na:], want_b) <= REL_TOL and O.cosine(got[lo:hi, na:], want_b) >= COS_MIN
     dev.free(*d.values())
 

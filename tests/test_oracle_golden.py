@@ -351,6 +351,10 @@ def test_mmq_formulas_against_float64():
     want = (d[..., None].astype(np.float64) * q).reshape(rows, k) @ O.dequantize(w6, O.GGML_Q6_K).astype(np.float64).T
     np.testing.assert_allclose(O.mmq_q6_k_d4s4(d4, w6), want, rtol=1e-9, atol=1e-9 * np.abs(want).max())
     assert O.max_rel_err(C.mmq_q6_k_d4s4(d4, w6), want) < 2e-4
+    # Q8_0 x D4S4: exactly the product of the dequantized weight with the dequantized activations (no min term)
+    w8 = O.random_weight(O.GGML_Q8_0, n, k, seed=8)
+    want = (d[..., None].astype(np.float64) * q).reshape(rows, k) @ O.dequantize(w8, O.GGML_Q8_0).astype(np.float64).T
+    np.testing.assert_allclose(O.mmq_q8_0_d4s4(d4, w8), want, rtol=1e-9, atol=1e-9 * np.abs(want).max())
     # Q5_K x D4S4: the Q4_K structure with 5-bit values and the float32 raw sum; an independent float64 evaluation
     # from the unpacked fields, and the dequantize-matmul identity it must stay close to (they differ in the min
     # term only: raw sum of the activations against xd * sum(q8))
