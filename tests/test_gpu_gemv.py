@@ -625,3 +625,35 @@ def test_q5_k_fused_gemv_and_block_dots(dev, rows, k, n):
         assert np.array_equal(dots, want_dots)
         ref = O.gguf_quant_gemv(O.dequantize_q8_1(xq), w, O.GGML_Q5_K)
         assert O.max_rel_err(got, ref) <= REL_TOL and O.cosine(got, ref) >= COS_MIN
+
+
+def _sweep_cases():
+    """48 seeded (quant, rows, K, N, activation type) draws: every batch size, K from one block to 34 blocks, N from
+    1 to a few thousand, so that every kernel form the launcher picks (stream, run, row-strided, slab, phased slab)
+    and its ragged edges are met on shapes no other test names."""
+    rng = np.random.default_rng(20240611)
+    cases = []
+    for i in range(48):
+        quant = ("gguf_q4_k", "gguf_q5_k", "gguf_q6_k", "gguf_q8_0")[i % 4]
+        rows = int(rng.integers(1, 9))
+        k = 256 * int(rng.choice([1, 2, 3, 5, 8, 11, 16, 20, 24, 34]))
+        n = int(rng.choice([1, 7, 31, 64, 100, 257, 640, 1000, 2049, 3333, 5120]))
+        cases.append((quant, rows, k, n, "bf16" if i % 3 == 0 else "f32"))
+    return cases
+
+
+@pytest.mark.parametrize("quant,rows,k,n,act", _sweep_cases())
+def test_fused_gemv_seeded_shape_sweep(dev, quant, rows, k, n, act):
+    rng = np.random.default_rng(rows * 1000003 + k * 101 + n)
+    x = (rng.standard_normal((rows, k)) * 0.5).astype(np.float32)
+    if act == "bf16":
+        x = O.bf16_bits_to_f32(O.f32_to_bf16_bits(x))
+    qt = O.GGML_Q5_K if quant == "gguf_q5_k" else QT[quant]
+    w = _random_q5_k(n, k, seed=k + n) if quant == "gguf_q5_k" else O.random_weight(qt, n, k, seed=k + n)
+    xin = x if act == "f32" else O.f32_to_bf16_bits(x)
+    dx, dw, dout = dev.put(xin), dev.put(w), dev.empty((rows * n + 4) * 4, fill=0x6B)
+    G.FUSED[(quant[5:], act, "f32")](dx.ptr, dw.ptr, dout.ptr, rows, k, n)
+    got = dev.get(dout, np.float32, (rows * n + 4,)).copy()
+    dev.free(dx, dw, dout)
+    assert np.all(got[rows * n:].view(np.uint32) == 0x6B6B6B6B)          # nothing past the output
+    _check_f32(got[:rows * n].reshape(rows, n), O.quantize_q8_1(x), w, qt)

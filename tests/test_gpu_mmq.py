@@ -261,3 +261,42 @@ def test_mmq_wrapper_rejects_bad_shapes(dev):
         f(1, 1, 1, 4, 256, 40)
     with pytest.raises(ValueError, match="rows"):
         f(1, 1, 1, 0, 256, 32)
+
+
+def _mmq_sweep_cases():
+    """32 seeded (quant, M, K, N) draws with ragged tiles in both dimensions and K from one step to 20."""
+    rng = np.random.default_rng(77001)
+    cases = []
+    for i in range(32):
+        quant = ("q4_k", "q5_k", "q6_k", "q8_0")[i % 4]
+        m = int(rng.choice([1, 5, 31, 33, 64, 127, 129, 200, 257, 385]))
+        k = (128 if quant == "q8_0" else 256) * int(rng.choice([1, 2, 3, 5, 8, 10]))
+        n = int(rng.choice([1, 33, 63, 65, 127, 129, 200, 320, 513]))
+        if quant in ("q4_k", "q5_k"):
+            n = (n + 31) // 32 * 32          # these two take out_features in multiples of 32
+        cases.append((quant, m, k, n))
+    return cases
+
+
+@pytest.mark.parametrize("quant,rows,k,n", _mmq_sweep_cases())
+def test_mmq_seeded_shape_sweep(dev, quant, rows, k, n):
+    xb = _bf16_rows(rows + 3 * k + 7 * n, rows, k, scale=0.2, offset=0.001)
+    if quant == "q4_k":
+        xq, w = O.pack_q8_1_ds4(xb), O.random_weight(O.GGML_Q4_K, n, k, seed=n + k)
+        fn, want = M.gguf_q4_k_q8_1_mmq32_vdr_dense_bf16_f32_out, O.mmq_q4_k_ds4(xq, w)
+    elif quant == "q5_k":
+        xq, w = O.pack_q8_1_d4s4(xb), _random_q5_k(n, k, seed=n + k)
+        fn, want = M.gguf_q5_k_mmq32_q8_1_d4s4_f32_bf16_f32_out, O.mmq_q5_k_d4s4(xq, w)
+    elif quant == "q6_k":
+        xq, w = O.pack_q8_1_d4s4(xb), O.random_weight(O.GGML_Q6_K, n, k, seed=n + k)
+        fn, want = M.gguf_q6_k_mmq32_q8_1_d4s4_f32_bf16_f32_out, O.mmq_q6_k_d4s4(xq, w)
+    else:
+        xq, w = O.pack_q8_1_d4s4(xb), O.random_weight(O.GGML_Q8_0, n, k, seed=n + k)
+        fn, want = M.gguf_q8_0_mmq32_q8_1_d4s4_f32_bf16_f32_out, O.mmq_q8_0_d4s4(xq, w)
+    dxq, dw, dout = dev.put(xq), dev.put(w), dev.empty((rows * n + 4) * 4, fill=0x6B)
+    fn(dxq.ptr, dw.ptr, dout.ptr, rows, k, n)
+    got = dev.get(dout, np.float32, (rows * n + 4,)).copy()
+    dev.free(dxq, dw, dout)
+    assert np.all(got[rows * n:].view(np.uint32) == 0x6B6B6B6B)          # nothing past the output
+    got = got[:rows * n].reshape(rows, n)
+    assert O.max_rel_err(got, want) <= 1e-3 and O.cosine(got, want) >= 0.99999
