@@ -630,7 +630,7 @@ __global__ void __launch_bounds__(1024) selected_down_sum_kernel(SelArgs s) {
   float* xd = reinterpret_cast<float*>(q8 + TK * chunk_elems);
   float* xs = xd + TK * chunk_sb;
   int* s16 = reinterpret_cast<int*>(xs);
-  float* red = (QT == GGML_Q4_K) ? xs + TK * chunk_sb
+  float* red = gemv_has_mins(QT)  ? xs + TK * chunk_sb
              : (QT == GGML_Q6_K) ? reinterpret_cast<float*>(s16 + TK * chunk_sb * 2)
                                  : xs;                                  // [TK][ks][16 * RG]
   GemvArgs a = s.g;
@@ -704,12 +704,13 @@ struct SelVariant {
              nullptr},                                                                                         \
   SelVariant{QT, CB, SEL_DUAL, sel_max_threads<QT, 2 * CB>(), selected_gemv_kernel<QT, 2, CB, SEL_DUAL>,          \
              {nullptr, nullptr}, nullptr}
-// Q4_K and Q6_K experts take every form; Q5_K and Q8_0 experts the single form (a projection per launch)
+// Q4_K and Q6_K experts take every form at every K; Q5_K and Q8_0 experts the two-matrix forms up to K = 4096
+// (16 blocks per row: beyond that a lane would hold two matrices x five blocks of 17-20 registers)
 const SelVariant kSel[] = {
     SEL_VARIANTS(GGML_Q4_K, 1), SEL_VARIANTS(GGML_Q4_K, 2), SEL_VARIANTS(GGML_Q4_K, 5),
     SEL_VARIANTS(GGML_Q6_K, 1), SEL_VARIANTS(GGML_Q6_K, 2), SEL_VARIANTS(GGML_Q6_K, 5),
-    SEL_SINGLE_VARIANT(GGML_Q5_K, 1), SEL_SINGLE_VARIANT(GGML_Q5_K, 2), SEL_SINGLE_VARIANT(GGML_Q5_K, 5),
-    SEL_SINGLE_VARIANT(GGML_Q8_0, 1), SEL_SINGLE_VARIANT(GGML_Q8_0, 2), SEL_SINGLE_VARIANT(GGML_Q8_0, 5),
+    SEL_VARIANTS(GGML_Q5_K, 1), SEL_VARIANTS(GGML_Q5_K, 2), SEL_SINGLE_VARIANT(GGML_Q5_K, 5),
+    SEL_VARIANTS(GGML_Q8_0, 1), SEL_VARIANTS(GGML_Q8_0, 2), SEL_SINGLE_VARIANT(GGML_Q8_0, 5),
 };
 
 int launch_selected(int qt, int mode, const void* x, int x_kind, const int64_t* selected, const float* routing,
@@ -722,7 +723,7 @@ int launch_selected(int qt, int mode, const void* x, int x_kind, const int64_t* 
   if (!x || !selected || !w_a || !out || x_rows <= 0 || lanes <= 0 || lanes > 65535 || num_experts <= 0 || K <= 0 ||
       (K % QK_K) != 0 || K > (1 << 20) || N <= 0 || N > (1 << 24) || x_kind < KIND_F32 || x_kind > max_x_kind ||
       out_kind < KIND_F32 || out_kind > KIND_F16 ||
-      (qt != GGML_Q4_K && qt != GGML_Q6_K && !(mode == SEL_SINGLE && (qt == GGML_Q5_K || qt == GGML_Q8_0)))) {
+      (qt != GGML_Q4_K && qt != GGML_Q5_K && qt != GGML_Q6_K && qt != GGML_Q8_0)) {
     return static_cast<int>(hipErrorInvalidValue);
   }
   if (x_up && (mode != SEL_SINGLE || x_kind != KIND_BF16)) return static_cast<int>(hipErrorInvalidValue);
@@ -750,7 +751,8 @@ int launch_selected(int qt, int mode, const void* x, int x_kind, const int64_t* 
     // keep the grid within one round of 256 workgroups (measured, E=256 k=8 H=2048 I=512: T=4 8.4 us against
     // 12.7 with twice the workgroups, T=8 12.4 against 16.3)
     int rgn = 1;
-    while (rgn < 4 && (N + 16 * rgn - 1) / (16 * rgn) * x_rows > 256) rgn <<= 1;   // 256 CUs
+    const int max_rgn = qt == GGML_Q5_K ? 2 : 4;   // four row groups of 20-register Q5_K blocks spill
+    while (rgn < max_rgn && (N + 16 * rgn - 1) / (16 * rgn) * x_rows > 256) rgn <<= 1;   // 256 CUs
     s.g.ks = ks; s.g.nrg = rgn;
     const size_t lds = gemv_lds_bytes(qt, 8, 1, 1, ks, 1) + static_cast<size_t>(8) * ks * 16 * rgn * 4 + 8 * 4;
     if (lds > 64 * 1024) return static_cast<int>(hipErrorInvalidValue);
@@ -762,11 +764,15 @@ int launch_selected(int qt, int mode, const void* x, int x_kind, const int64_t* 
     else if (x_kind == KIND_BF16) hipLaunchKernelGGL((selected_down_sum_kernel<QT, 8, RGN, KIND_BF16>), grid, block, lds, stream, s); \
     else hipLaunchKernelGGL((selected_down_sum_kernel<QT, 8, RGN>), grid, block, lds, stream, s);                \
   } while (0)
-    if (qt == GGML_Q4_K) {
-      if (rgn == 4) LAUNCH_DOWN(GGML_Q4_K, 4); else if (rgn == 2) LAUNCH_DOWN(GGML_Q4_K, 2); else LAUNCH_DOWN(GGML_Q4_K, 1);
-    } else {
-      if (rgn == 4) LAUNCH_DOWN(GGML_Q6_K, 4); else if (rgn == 2) LAUNCH_DOWN(GGML_Q6_K, 2); else LAUNCH_DOWN(GGML_Q6_K, 1);
-    }
+#define LAUNCH_DOWN_QT(QT)                                                                                    \
+  do {                                                                                                         \
+    if (rgn == 4) LAUNCH_DOWN(QT, 4); else if (rgn == 2) LAUNCH_DOWN(QT, 2); else LAUNCH_DOWN(QT, 1);          \
+  } while (0)
+    if (qt == GGML_Q4_K) LAUNCH_DOWN_QT(GGML_Q4_K);
+    else if (qt == GGML_Q5_K) { if (rgn == 2) LAUNCH_DOWN(GGML_Q5_K, 2); else LAUNCH_DOWN(GGML_Q5_K, 1); }
+    else if (qt == GGML_Q6_K) LAUNCH_DOWN_QT(GGML_Q6_K);
+    else LAUNCH_DOWN_QT(GGML_Q8_0);
+#undef LAUNCH_DOWN_QT
 #undef LAUNCH_DOWN
     return static_cast<int>(hipGetLastError());
   }

@@ -217,8 +217,10 @@ def gguf_selected_gemv(quant: str, mode: int, x_ptr: int, selected_ptr: int, qwe
                        library: ctypes.CDLL | None = None, runtime: HipRuntime | None = None) -> None:
     """The decode kernels with every choice explicit (``hipengine_gfx950_gguf_selected_gemv``):
     mode 0 single, 1 gate/up with SiLU, 2 routed down projection summed per token."""
-    if quant not in ("gguf_q4_k", "gguf_q6_k") and not (mode == SEL_SINGLE and quant in ("gguf_q5_k", "gguf_q8_0")):
-        raise ValueError("quant must be gguf_q4_k or gguf_q6_k (the single form also takes gguf_q5_k and gguf_q8_0)")
+    if quant not in ("gguf_q4_k", "gguf_q5_k", "gguf_q6_k", "gguf_q8_0"):
+        raise ValueError("quant must be gguf_q4_k, gguf_q5_k, gguf_q6_k or gguf_q8_0")
+    if mode == SEL_DUAL_SILU and quant in ("gguf_q5_k", "gguf_q8_0") and in_features > 4096:
+        raise ValueError("the gate/up form takes gguf_q5_k and gguf_q8_0 experts up to in_features 4096")
     if mode not in (SEL_SINGLE, SEL_DUAL_SILU, SEL_DOWN_SUM):
         raise ValueError("mode must be 0, 1 or 2")
     if mode == SEL_DOWN_SUM:
@@ -427,5 +429,5 @@ def register_kernels(backend: str = "hip_gfx950", *, replace: bool = False) -> N
              replace=replace)
     register(KernelKey(backend, "moe_linear", "gguf_q8_0", "grouped_mmq128_q8_1_d4s4"), gguf_q8_0_grouped_mmq,
              replace=replace)
-    for quant in ("gguf_q4_k", "gguf_q5_k", "gguf_q6_k", "gguf_q8_0"):     # Q5_K and Q8_0: the single form
+    for quant in ("gguf_q4_k", "gguf_q5_k", "gguf_q6_k", "gguf_q8_0"):
         register(KernelKey(backend, "moe_linear", quant, "selected_gemv_q8_1"), gguf_selected_gemv, replace=replace)

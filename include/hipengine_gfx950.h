@@ -636,7 +636,8 @@ int hipengine_gfx950_gguf_grouped_gemv(int32_t ggml_type, const void* x, int32_t
                                        int64_t num_experts, int64_t in_features, int64_t out_features,
                                        hipengine_stream_t stream);
 
-/* The decode kernels with every choice explicit.  ggml_type 12 (Q4_K) or 14 (Q6_K).
+/* The decode kernels with every choice explicit.  ggml_type 12 (Q4_K), 13 (Q5_K), 14 (Q6_K) or 8 (Q8_0); mode 1 takes
+ * Q5_K and Q8_0 experts up to in_features 4096.
  *   mode 0: out[lanes, N] = W_a[selected[lane]] . x[lane / (lanes/x_rows)]
  *   mode 1: out[lanes, N] = silu(gate) * up with W_a = gate, W_b = up; round_mid != 0
  *           rounds gate and up to the output type first

@@ -296,6 +296,39 @@ def test_decode_chain_matches_cpu_moe(dev, tokens, experts):
     np.testing.assert_allclose(got, ref, rtol=2e-2, atol=2e-2 * np.abs(ref).max())
 
 
+@pytest.mark.parametrize("quant,qt", [("gguf_q5_k", O.GGML_Q5_K), ("gguf_q6_k", O.GGML_Q6_K), ("gguf_q8_0", O.GGML_Q8_0)])
+@pytest.mark.parametrize("tokens,hidden,inter", [(1, 1024, 512), (5, 4096, 256), (8, 2048, 768)])
+def test_decode_chain_for_other_expert_types(dev, quant, qt, tokens, hidden, inter):
+    """The two-launch decode chain (gate/up with SiLU, routed down sum) for Q5_K, Q6_K and Q8_0 experts: each stage
+    against the reference arithmetic on the same quantized inputs (4, 16 and 8 blocks per gate/up row: one block and
+    two blocks per lane and K slice)."""
+    top_k, experts = 8, 12
+    sel, wts = _routing(tokens + hidden, tokens, top_k, experts)
+    make = ((lambda n, k, seed: O.stack_experts(_random_q5_k(n, k, seed), experts, seed=seed % 5)) if qt == O.GGML_Q5_K
+            else (lambda n, k, seed: _experts(qt, experts, n, k, seed=seed)))
+    wg, wu, wd = make(inter, hidden, 1), make(inter, hidden, 2), make(hidden, inter, 3)
+    x = (np.random.default_rng(tokens).standard_normal((tokens, hidden)) * 0.3).astype(np.float32)
+    lanes = tokens * top_k
+    dx, dsel, dwt = dev.put(x), dev.put(sel), dev.put(wts)
+    dg, du, dd = dev.put(wg), dev.put(wu), dev.put(wd)
+    dmid, dout = dev.empty(lanes * inter * 4), dev.empty(tokens * hidden * 4)
+    M.gguf_selected_gemv(quant, M.SEL_DUAL_SILU, dx.ptr, dsel.ptr, dg.ptr, dmid.ptr, tokens, lanes, experts,
+                         hidden, inter, qweight_b_ptr=du.ptr)
+    M.gguf_selected_gemv(quant, M.SEL_DOWN_SUM, dmid.ptr, dsel.ptr, dd.ptr, dout.ptr, tokens, lanes, experts,
+                         inter, hidden, routing_weights_ptr=dwt.ptr, top_k=top_k)
+    mid = dev.get(dmid, np.float32, (lanes, inter))
+    got = dev.get(dout, np.float32, (tokens, hidden))
+    dev.free(dx, dsel, dwt, dg, du, dd, dmid, dout)
+    want = np.zeros((tokens, hidden), dtype=np.float32)
+    for lane in range(lanes):
+        t, e = lane // top_k, int(sel.reshape(-1)[lane])
+        g, u = _ref_lane(x[t], wg[e], qt), _ref_lane(x[t], wu[e], qt)
+        ref_mid = (O.silu(g) * u).astype(np.float32)
+        assert O.max_rel_err(mid[lane], ref_mid) <= REL_TOL and O.cosine(mid[lane], ref_mid) >= COS_MIN
+        want[t] += wts.reshape(-1)[lane] * _ref_lane(mid[lane], wd[e], qt)
+    assert O.max_rel_err(got, want) <= REL_TOL and O.cosine(got, want) >= COS_MIN
+
+
 def _grouped(dev, host, d, ds4, w_a, w_b, rows_src, k, na, nb, experts, identity=False, out_dtype="f32"):
     total = host["total"]
     dxq, dwa = dev.put(ds4), dev.put(w_a)

@@ -272,8 +272,10 @@ def test_moe_wrappers_validate_before_touching_the_device():
         M.gguf_q4_k_selected_gemv_bf16_bf16_out(0, 1, 1, 1, 1, 8, 4, 256, 32)
     with pytest.raises(ValueError, match="x_rows \\* top_k"):
         M.gguf_selected_gemv("gguf_q4_k", M.SEL_DOWN_SUM, 1, 1, 1, 1, 2, 9, 4, 256, 32, routing_weights_ptr=1, top_k=4)
-    with pytest.raises(ValueError, match="gguf_q4_k or gguf_q6_k"):
-        M.gguf_selected_gemv("gguf_q8_0", M.SEL_DUAL_SILU, 1, 1, 1, 1, 1, 8, 4, 256, 32, qweight_b_ptr=1)
+    with pytest.raises(ValueError, match="up to in_features 4096"):
+        M.gguf_selected_gemv("gguf_q8_0", M.SEL_DUAL_SILU, 1, 1, 1, 1, 1, 8, 4, 4352, 32, qweight_b_ptr=1)
+    with pytest.raises(ValueError, match="quant must be"):
+        M.gguf_selected_gemv("gguf_q3_k", M.SEL_SINGLE, 1, 1, 1, 1, 1, 8, 4, 256, 32)
     single, silu = M.SELECTED_K["q6_k"]
     with pytest.raises(ValueError, match="multiple of x_rows"):
         single(1, 1, 1, 1, 3, 8, 4, 256, 32)
