@@ -60,6 +60,38 @@ __global__ void __launch_bounds__(256) quantize_q8_1_kernel(const void* __restri
   }
 }
 
+// Two planes of 36-byte blocks (gguf_q4_k_gemv.hip:777-829): plane 0 is the plain quantization, plane 1, at
+// +total_groups blocks, the same quantization of what plane 0 leaves, x - float(half d0) * q0 (the product has 19
+// significant bits, so the subtraction is one rounding however it is contracted).
+__global__ void __launch_bounds__(256) quantize_q8_1x2_kernel(const void* __restrict__ x, int kind,
+                                                              uint8_t* __restrict__ xq, int64_t total_groups) {
+  const int64_t g = static_cast<int64_t>(blockIdx.x) * 32 + (threadIdx.x >> 3);
+  const int e = threadIdx.x & 7;
+  if (g >= total_groups) return;   // uniform for the 8 lanes of a group
+  float v[4];
+  load4_values(x, kind, g * 32 + e * 4, v);
+#pragma unroll
+  for (int plane = 0; plane < 2; ++plane) {
+    const float amax = oct_max(fmaxf(fmaxf(fabsf(v[0]), fabsf(v[1])), fmaxf(fabsf(v[2]), fabsf(v[3]))));
+    const float sum = oct_tree_sum32(v[0], v[1], v[2], v[3]);
+    const float d = amax / 127.0f;
+    int q[4] = {0, 0, 0, 0};
+    if (amax != 0.0f) {
+#pragma unroll
+      for (int i = 0; i < 4; ++i) q[i] = max(-128, min(127, static_cast<int>(roundf(v[i] / d))));
+    }
+    uint8_t* blk = xq + (plane * total_groups + g) * Q8_1_BYTES;
+    *reinterpret_cast<uint32_t*>(blk + 4 + 4 * e) = pack_i8x4(q[0], q[1], q[2], q[3]);
+    const uint16_t dh = float_to_f16_bits(d);
+    if (e == 0) {
+      *reinterpret_cast<uint32_t*>(blk) = static_cast<uint32_t>(dh) | (static_cast<uint32_t>(float_to_f16_bits(sum)) << 16);
+    }
+    const float dq = f16_bits_to_float(dh);
+#pragma unroll
+    for (int i = 0; i < 4; ++i) v[i] = v[i] - dq * static_cast<float>(q[i]);
+  }
+}
+
 constexpr float kFp16Max = 65504.0f;
 
 // One lane's share (4 of 32 values) of a DS4 group: ties-to-even, clamp +-127, fp16 scale and sum.
@@ -208,6 +240,17 @@ extern "C" int hipengine_gguf_q4_k_quantize_f32_q8_1(const void* x, void* xq, in
 extern "C" int hipengine_gguf_q4_k_quantize_bf16_q8_1(const void* x, void* xq, int64_t rows, int64_t in_features,
                                                       hipStream_t stream) {
   return launch_q8_1(x, KIND_BF16, xq, rows, in_features, stream);
+}
+
+extern "C" int hipengine_gguf_q4_k_quantize_bf16_q8_1x2(const void* x, void* xq, int64_t rows, int64_t in_features,
+                                                        hipStream_t stream) {
+  if (!x || !xq || rows <= 0 || in_features <= 0 || (in_features % 32) != 0) return static_cast<int>(hipErrorInvalidValue);
+  const int64_t groups = rows * (in_features / 32);
+  const int64_t grid = (groups + 31) / 32;
+  if (grid > 0x7FFFFFFF) return static_cast<int>(hipErrorInvalidValue);
+  hipLaunchKernelGGL(quantize_q8_1x2_kernel, dim3(static_cast<unsigned>(grid)), dim3(256), 0, stream, x, KIND_BF16,
+                     static_cast<uint8_t*>(xq), groups);
+  return static_cast<int>(hipGetLastError());
 }
 
 extern "C" int hipengine_gguf_q8_1_mmq_ds4_pack_bf16(const void* x, void* out, int64_t rows, int64_t hidden,

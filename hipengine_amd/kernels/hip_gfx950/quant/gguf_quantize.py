@@ -40,6 +40,14 @@ def gguf_q4_k_quantize_bf16_q8_1(x_ptr: int, xq_ptr: int, rows: int, in_features
     _quantize("hipengine_gguf_q4_k_quantize_bf16_q8_1", x_ptr, xq_ptr, rows, in_features, 32, stream, library, runtime)
 
 
+def gguf_q4_k_quantize_bf16_q8_1x2(x_ptr: int, xq_ptr: int, rows: int, in_features: int, *, stream: int = 0,
+                                   library: ctypes.CDLL | None = None, runtime: HipRuntime | None = None) -> None:
+    """bf16 ``[rows, in_features]`` -> two planes ``[2, rows, in_features/32]`` of 36-byte q8_1 blocks: the plain
+    quantization and the same quantization of its residual (``gguf_q4_k_gemv.py:1195-1233``).  The planes are
+    consecutive, so a pre-quantized GEMV over ``2 * rows`` rows yields the two partial products to add."""
+    _quantize("hipengine_gguf_q4_k_quantize_bf16_q8_1x2", x_ptr, xq_ptr, rows, in_features, 32, stream, library, runtime)
+
+
 def gguf_q8_1_mmq_ds4_pack_bf16(x_ptr: int, xq_ptr: int, rows: int, hidden: int, *, stream: int = 0,
                                 library: ctypes.CDLL | None = None, runtime: HipRuntime | None = None) -> None:
     """bf16 ``[rows, hidden]`` -> ``[rows, hidden/128]`` 144-byte DS4 blocks."""
@@ -85,6 +93,7 @@ def register_kernels(backend: str = "hip_gfx950", *, replace: bool = False) -> N
     for quant, variant, fn in (
         ("q8_1", "f32", gguf_q4_k_quantize_f32_q8_1),
         ("q8_1", "bf16", gguf_q4_k_quantize_bf16_q8_1),
+        ("q8_1x2", "bf16", gguf_q4_k_quantize_bf16_q8_1x2),
         ("q8_1_ds4", "bf16", gguf_q8_1_mmq_ds4_pack_bf16),
         ("q8_1_ds4", "gather_bf16", gguf_q8_1_mmq_gather_ds4_pack_bf16),
         ("q8_1_d4s4_f32", "bf16", gguf_q8_1_d4s4_f32_quantize_bf16),

@@ -68,6 +68,13 @@ int hipengine_gguf_q4_k_quantize_f32_q8_1(const void* x, void* xq, int64_t rows,
 int hipengine_gguf_q4_k_quantize_bf16_q8_1(const void* x, void* xq, int64_t rows, int64_t in_features,
                                            hipengine_stream_t stream);
 
+/* bf16 [rows, in_features] -> two planes [2, rows, in_features/32] of block_q8_1: plane 0 is the quantization above,
+ * plane 1 (at + rows * in_features/32 blocks) the same quantization of the residual x - float(half d0) * q0.
+ * Replaces gguf_q4_k_gemv.hip:2844-2852 (kernel :777-829).  hipEngine's consumers of the two planes take its RDNA3
+ * weight layouts; here the planes are 2 * rows rows of the pre-quantized q8_1 GEMV, whose two results add up. */
+int hipengine_gguf_q4_k_quantize_bf16_q8_1x2(const void* x, void* xq, int64_t rows, int64_t in_features,
+                                             hipengine_stream_t stream);
+
 /* bf16 [rows, hidden] -> 144-byte DS4 blocks {half ds4[8]; int8 qs[128]},
  * [rows, hidden/128]: per 32 values scale = min(65504, amax/127),
  * q = clamp(rint(x/scale), -127, 127), ds4[2g] = half(scale), ds4[2g+1] = half(sum).

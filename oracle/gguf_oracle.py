@@ -40,6 +40,9 @@ dequant_q5_k                 block builder inverse (reference generator restated
 quantize_q8_1                float64 brute force, invariants (|q|<=127,
                              q[argmax]=+-127, zero block), tie cases built
                              from exact binary fractions
+quantize_q8_1x2              plane 0 = quantize_q8_1; the two planes reconstruct x to 2^-13 of the
+                             block's amax (float64 check); a block plane 0 represents exactly
+                             has a zero plane 1
 pack_q8_1_ds4                same, half-to-even tie case, fp16 clamp case
 pack_q8_1_d4s4               same, summation tree spelled out independently
 block_dots_*                 int64 einsum over independently unpacked integers
@@ -477,6 +480,16 @@ def quantize_q8_1(x) -> np.ndarray:
     out[..., 2:4] = _tree_sum32(g).astype(np.float16)[..., None].view(np.uint8)
     out[..., 4:] = q.view(np.uint8)
     return out
+
+
+def quantize_q8_1x2(x) -> np.ndarray:
+    """Two planes of q8_1 blocks, uint8 ``[2, rows, K/32, 36]`` (gguf_q4_k_gemv.hip:777-829): plane 0 is
+    ``quantize_q8_1(x)``; plane 1 the same quantization of the residual ``x - float(half d0) * q0``."""
+    xa = np.ascontiguousarray(x, dtype=np.float32)
+    p0 = quantize_q8_1(xa)
+    d0, _, q0 = q8_1_fields(p0)
+    residual = (xa.reshape(q0.shape) - (d0[..., None] * q0.astype(np.float32)).astype(np.float32)).astype(np.float32)
+    return np.stack([p0, quantize_q8_1(residual.reshape(xa.shape))])
 
 
 def q8_1_fields(xq) -> tuple[np.ndarray, np.ndarray, np.ndarray]:

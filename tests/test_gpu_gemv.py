@@ -657,3 +657,30 @@ def test_fused_gemv_seeded_shape_sweep(dev, quant, rows, k, n, act):
     dev.free(dx, dw, dout)
     assert np.all(got[rows * n:].view(np.uint32) == 0x6B6B6B6B)          # nothing past the output
     _check_f32(got[:rows * n].reshape(rows, n), O.quantize_q8_1(x), w, qt)
+
+
+@pytest.mark.parametrize("rows,k", [(1, 32), (3, 5120), (8, 2048)])
+def test_q8_1x2_planes_bytes_and_gemv_over_both(dev, rows, k):
+    """The two-plane quantizer byte for byte; the pre-quantized GEMV over the planes as 2 * rows rows gives two
+    partial products whose sum is closer to the float GEMV on the unquantized activations than plane 0 alone (what
+    is left is the fp16 rounding of the blocks' raw sums, which the Q4_K min term of a pre-quantized GEMV reads)."""
+    rng = np.random.default_rng(rows + k)
+    x = (rng.standard_normal((rows, k)) * 0.7).astype(np.float32)
+    x[0, :32] = 0.0
+    xb = O.f32_to_bf16_bits(x)
+    want = O.quantize_q8_1x2(O.bf16_bits_to_f32(xb))
+    dx, dq = dev.put(xb), dev.empty(2 * rows * (k // 32) * 36, fill=0x33)
+    Q.gguf_q4_k_quantize_bf16_q8_1x2(dx.ptr, dq.ptr, rows, k)
+    got = dev.get(dq, np.uint8, want.shape).copy()
+    assert np.array_equal(got, want)
+    if k % 256 == 0 and 2 * rows <= 8:
+        n = 96
+        w = O.random_weight(O.GGML_Q4_K, n, k, seed=3)
+        dw, dout = dev.put(w), dev.empty(2 * rows * n * 4)
+        G.gguf_q4_k_q8_1_dp4a_vdr_bf16_f32_out(dq.ptr, dw.ptr, dout.ptr, 2 * rows, k, n)
+        parts = dev.get(dout, np.float32, (2, rows, n)).copy()
+        dev.free(dw, dout)
+        ref = O.gguf_quant_gemv(O.bf16_bits_to_f32(xb), w, O.GGML_Q4_K)
+        both, one = O.max_rel_err(parts[0] + parts[1], ref), O.max_rel_err(parts[0], ref)
+        assert both <= 5e-3 and both < 0.6 * one, (both, one)
+    dev.free(dx, dq)

@@ -584,3 +584,21 @@ def test_moe_tail_next_rmsnorm_reference_known_answer_and_scalar_loop():
     routing0[1, 2] = 0.0
     r5, _ = O.moe_tail_next_rmsnorm(slots, shared, gate, residual, weight, routing_weights=routing0, eps=1e-5)
     assert np.array_equal(r4, r5)
+
+
+def test_quantize_q8_1x2_planes():
+    """Plane 0 is the plain quantizer; plane 1 quantizes what plane 0 leaves, so the two planes together are within
+    half a step of the second scale (|residual| <= d0/2 + fp16 rounding of d0, so d1 <= amax/127 * 0.52 / 127); a block
+    that plane 0 represents exactly leaves a zero plane."""
+    rng = np.random.default_rng(12)
+    x = O.bf16_bits_to_f32(O.f32_to_bf16_bits((rng.standard_normal((5, 256)) * 3.0).astype(np.float32)))
+    x[1, 32:64] = np.arange(-16, 16) * 0.25
+    x[1, 63] = 127 * 0.25                       # d = 0.25 exactly: q = x / 0.25, nothing left
+    planes = O.quantize_q8_1x2(x)
+    assert planes.shape == (2, 5, 8, 36) and np.array_equal(planes[0], O.quantize_q8_1(x))
+    d0, _, q0 = O.q8_1_fields(planes[0])
+    d1, s1, q1 = O.q8_1_fields(planes[1])
+    recon = d0[..., None].astype(np.float64) * q0 + d1[..., None].astype(np.float64) * q1
+    amax = np.abs(x.reshape(5, 8, 32)).max(axis=-1, keepdims=True)
+    assert np.all(np.abs(recon - x.reshape(5, 8, 32)) <= amax * 2.0 ** -13 + 1e-12)
+    assert np.all(q1[1, 1] == 0) and d1[1, 1] == 0 and s1[1, 1] == 0
