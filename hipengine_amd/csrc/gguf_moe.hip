@@ -33,10 +33,61 @@ constexpr int MAX_EXPERTS = 2048;
 // routing index
 // --------------------------------------------------------------------------
 
+// Exclusive prefix of the per-expert counts in cnt[0..num_experts) (LDS, replaced by the prefix) -> expert_start[0..E],
+// and the ascending list of the experts with a non-zero count; all 1024 threads of the workgroup call it after a
+// barrier that made cnt complete.  PER consecutive experts per thread, a shuffle scan per wave, the wave totals
+// through LDS (a single thread walking 256 counters in LDS costs ~10 us of read latency).
+__device__ __forceinline__ void moe_prefix_active_block(int* cnt, int* act, int* totals, int num_experts,
+                                                        int64_t* __restrict__ expert_start,
+                                                        int64_t* __restrict__ active_experts,
+                                                        int64_t* __restrict__ active_count) {
+  constexpr int PER = MAX_EXPERTS / 1024;
+  __shared__ int wsum[16], wnz[16];
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  int c[PER], sum = 0, nz = 0;
+#pragma unroll
+  for (int k = 0; k < PER; ++k) {
+    const int e = tid * PER + k;
+    c[k] = e < num_experts ? cnt[e] : 0;
+    sum += c[k];
+    nz += c[k] > 0 ? 1 : 0;
+  }
+  int isum = sum, inz = nz;
+#pragma unroll
+  for (int off = 1; off < 64; off <<= 1) {
+    const int t = __shfl_up(isum, off), u = __shfl_up(inz, off);
+    if (lane >= off) { isum += t; inz += u; }
+  }
+  if (lane == 63) { wsum[wave] = isum; wnz[wave] = inz; }
+  __syncthreads();
+  int base = 0, base_nz = 0;
+  for (int w = 0; w < wave; ++w) { base += wsum[w]; base_nz += wnz[w]; }
+  int offset = base + isum - sum, rank = base_nz + inz - nz;
+#pragma unroll
+  for (int k = 0; k < PER; ++k) {
+    const int e = tid * PER + k;
+    if (e < num_experts) {
+      cnt[e] = offset;
+      if (c[k] > 0) act[rank++] = e;
+      offset += c[k];
+    }
+  }
+  if (tid == 1023) { totals[0] = base + isum; totals[1] = base_nz + inz; }
+  __syncthreads();
+  for (int e = threadIdx.x; e < num_experts; e += 1024) expert_start[e] = cnt[e];
+  if (active_experts)
+    for (int i = threadIdx.x; i < totals[1]; i += 1024) active_experts[i] = act[i];
+  if (threadIdx.x == 0) {
+    expert_start[num_experts] = totals[0];
+    if (active_count) active_count[0] = totals[1];
+  }
+}
+
 // One workgroup: histogram of the selected experts in LDS (integer atomics, so the
 // result does not depend on order), exclusive prefix -> expert_start[0..E],
 // ascending list of the experts that own at least one lane.
-__global__ void __launch_bounds__(1024) moe_count_prefix_kernel(const int64_t* __restrict__ selected,
+template <class ID>
+__global__ void __launch_bounds__(1024) moe_count_prefix_kernel(const ID* __restrict__ selected,
                                                                 int64_t* __restrict__ expert_start,
                                                                 int64_t* __restrict__ active_experts,
                                                                 int64_t* __restrict__ active_count,
@@ -62,56 +113,26 @@ __global__ void __launch_bounds__(1024) moe_count_prefix_kernel(const int64_t* _
     }
   }
   __syncthreads();
-  {
-    // exclusive prefix of the counts and rank among the non-empty experts, over the whole workgroup:
-    // PER consecutive experts per thread, a shuffle scan per wave, the wave totals through LDS
-    // (a single thread walking 256 counters in LDS costs ~10 us of read latency)
-    constexpr int PER = MAX_EXPERTS / 1024;
-    __shared__ int wsum[16], wnz[16];
-    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-    int c[PER], sum = 0, nz = 0;
-#pragma unroll
-    for (int k = 0; k < PER; ++k) {
-      const int e = tid * PER + k;
-      c[k] = e < num_experts ? cnt[e] : 0;
-      sum += c[k];
-      nz += c[k] > 0 ? 1 : 0;
-    }
-    int isum = sum, inz = nz;
-#pragma unroll
-    for (int off = 1; off < 64; off <<= 1) {
-      const int t = __shfl_up(isum, off), u = __shfl_up(inz, off);
-      if (lane >= off) { isum += t; inz += u; }
-    }
-    if (lane == 63) { wsum[wave] = isum; wnz[wave] = inz; }
-    __syncthreads();
-    int base = 0, base_nz = 0;
-    for (int w = 0; w < wave; ++w) { base += wsum[w]; base_nz += wnz[w]; }
-    int offset = base + isum - sum, rank = base_nz + inz - nz;
-#pragma unroll
-    for (int k = 0; k < PER; ++k) {
-      const int e = tid * PER + k;
-      if (e < num_experts) {
-        cnt[e] = offset;
-        if (c[k] > 0) act[rank++] = e;
-        offset += c[k];
-      }
-    }
-    if (tid == 1023) { totals[0] = base + isum; totals[1] = base_nz + inz; }
-  }
+  moe_prefix_active_block(cnt, act, totals, num_experts, expert_start, active_experts, active_count);
+}
+
+// The prefix and the active list from counts that are already in memory (one workgroup of 1024 threads).
+__global__ void __launch_bounds__(1024) moe_prefix_active_kernel(const int32_t* __restrict__ counts,
+                                                                 int64_t* __restrict__ expert_start,
+                                                                 int64_t* __restrict__ active_experts,
+                                                                 int64_t* __restrict__ active_count, int num_experts) {
+  __shared__ int cnt[MAX_EXPERTS];
+  __shared__ int act[MAX_EXPERTS];
+  __shared__ int totals[2];
+  for (int e = threadIdx.x; e < num_experts; e += 1024) cnt[e] = counts[e] > 0 ? counts[e] : 0;
   __syncthreads();
-  for (int e = threadIdx.x; e < num_experts; e += 1024) expert_start[e] = cnt[e];
-  if (active_experts)
-    for (int i = threadIdx.x; i < totals[1]; i += 1024) active_experts[i] = act[i];
-  if (threadIdx.x == 0) {
-    expert_start[num_experts] = totals[0];
-    if (active_count) active_count[0] = totals[1];
-  }
+  moe_prefix_active_block(cnt, act, totals, num_experts, expert_start, active_experts, active_count);
 }
 
 // One workgroup per expert: writes its lanes in ascending lane order (wave
 // ballots keep the order) into [expert_start[e], expert_start[e+1]).
-__global__ void __launch_bounds__(1024) moe_place_kernel(const int64_t* __restrict__ selected,
+template <class ID>
+__global__ void __launch_bounds__(1024) moe_place_kernel(const ID* __restrict__ selected,
                                                          const float* __restrict__ routing,
                                                          const int64_t* __restrict__ expert_start,
                                                          int64_t* __restrict__ sorted_lanes,
@@ -182,7 +203,8 @@ __global__ void __launch_bounds__(1024) moe_place_kernel(const int64_t* __restri
   }
 }
 
-int launch_compact(const int64_t* selected, const float* routing, int64_t* expert_start, int64_t* active_experts,
+template <class ID>
+int launch_compact(const ID* selected, const float* routing, int64_t* expert_start, int64_t* active_experts,
                    int64_t* active_count, int64_t* sorted_lanes, int64_t* sorted_experts, int64_t* compact_to_source,
                    float* sorted_weights, int64_t lanes, int64_t num_experts, int64_t top_k, hipStream_t stream,
                    int64_t* lane_to_compact = nullptr) {
@@ -190,9 +212,9 @@ int launch_compact(const int64_t* selected, const float* routing, int64_t* exper
       num_experts <= 0 || num_experts > MAX_EXPERTS || top_k <= 0) {
     return static_cast<int>(hipErrorInvalidValue);
   }
-  hipLaunchKernelGGL(moe_count_prefix_kernel, dim3(1), dim3(1024), 0, stream, selected, expert_start, active_experts,
+  hipLaunchKernelGGL(moe_count_prefix_kernel<ID>, dim3(1), dim3(1024), 0, stream, selected, expert_start, active_experts,
                      active_count, lane_to_compact, lanes, static_cast<int>(num_experts));
-  hipLaunchKernelGGL(moe_place_kernel, dim3(static_cast<unsigned>(num_experts)), dim3(1024), 0, stream, selected, routing,
+  hipLaunchKernelGGL(moe_place_kernel<ID>, dim3(static_cast<unsigned>(num_experts)), dim3(1024), 0, stream, selected, routing,
                      expert_start, sorted_lanes, sorted_experts, compact_to_source, sorted_weights, lane_to_compact, lanes,
                      top_k);
   return static_cast<int>(hipGetLastError());
@@ -1466,6 +1488,81 @@ extern "C" int hipengine_qwen35_moe_group_scatter_gather_lowp(
                      selected_experts, routing_weights, expert_start, scatter_offsets, sorted_lanes, sorted_experts,
                      sorted_weights, total_lanes, hidden_states, packed_hidden, top_k, hidden_size);
   return static_cast<int>(hipGetLastError());
+}
+
+// hipEngine's "parallel" compaction variants produce the same arrays as its stable ones (one workgroup per expert,
+// wave ballots keep ascending lane order: moe/group_scatter.hip:256-326), which is how the index is built here anyway.
+extern "C" int hipengine_qwen35_moe_group_compact_active_parallel(
+    const int64_t* selected_experts, const float* routing_weights, int64_t* expert_start, int64_t* active_experts,
+    int64_t* active_count, int64_t* sorted_lanes, int64_t* sorted_experts, float* sorted_weights, int64_t total_lanes,
+    int64_t num_experts, hipStream_t stream) {
+  return hipengine_qwen35_moe_group_compact_active(selected_experts, routing_weights, expert_start, active_experts,
+                                                   active_count, sorted_lanes, sorted_experts, sorted_weights,
+                                                   total_lanes, num_experts, stream);
+}
+
+extern "C" int hipengine_qwen35_moe_group_compact_active_source_rows_parallel(
+    const int64_t* selected_experts, const float* routing_weights, int64_t* expert_start, int64_t* active_experts,
+    int64_t* active_count, int64_t* sorted_lanes, int64_t* compact_to_source, float* sorted_weights,
+    int64_t total_lanes, int64_t num_experts, int64_t top_k, hipStream_t stream) {
+  return hipengine_qwen35_moe_group_compact_active_source_rows(selected_experts, routing_weights, expert_start,
+                                                               active_experts, active_count, sorted_lanes,
+                                                               compact_to_source, sorted_weights, total_lanes,
+                                                               num_experts, top_k, stream);
+}
+
+extern "C" int hipengine_qwen35_moe_group_compact_active_i32_parallel(
+    const int32_t* selected_experts, const float* routing_weights, int64_t* expert_start, int64_t* active_experts,
+    int64_t* active_count, int64_t* sorted_lanes, int64_t* sorted_experts, float* sorted_weights, int64_t total_lanes,
+    int64_t num_experts, hipStream_t stream) {
+  return launch_compact(selected_experts, routing_weights, expert_start, active_experts, active_count, sorted_lanes,
+                        sorted_experts, nullptr, sorted_weights, total_lanes, num_experts, 1, stream);
+}
+
+extern "C" int hipengine_qwen35_moe_group_prefix_active(const int32_t* counts, int64_t* expert_start,
+                                                        int64_t* active_experts, int64_t* active_count,
+                                                        int64_t num_experts, hipStream_t stream) {
+  if (!counts || !expert_start || !active_experts || !active_count || num_experts <= 0 || num_experts > MAX_EXPERTS) {
+    return static_cast<int>(hipErrorInvalidValue);
+  }
+  hipLaunchKernelGGL(moe_prefix_active_kernel, dim3(1), dim3(1024), 0, stream, counts, expert_start, active_experts,
+                     active_count, static_cast<int>(num_experts));
+  return static_cast<int>(hipGetLastError());
+}
+
+extern "C" int hipengine_qwen35_moe_group_scatter(const int64_t* selected_experts, const float* routing_weights,
+                                                  const int64_t* expert_start, int32_t* scatter_offsets,
+                                                  int64_t* sorted_lanes, int64_t* sorted_experts, float* sorted_weights,
+                                                  int64_t total_lanes, int64_t num_experts,
+                                                  bool include_routing_weights, hipStream_t stream) {
+  if (!selected_experts || !expert_start || !scatter_offsets || !sorted_lanes || !sorted_experts ||
+      (include_routing_weights && (!routing_weights || !sorted_weights)) || total_lanes <= 0 ||
+      total_lanes > 0x7FFFFFFF || num_experts <= 0 || num_experts > MAX_EXPERTS) {
+    return static_cast<int>(hipErrorInvalidValue);
+  }
+  hipLaunchKernelGGL(moe_scatter_kernel, dim3(static_cast<unsigned>(num_experts)), dim3(1024), 0, stream,
+                     selected_experts, routing_weights, expert_start, scatter_offsets, sorted_lanes, sorted_experts,
+                     include_routing_weights ? sorted_weights : nullptr, total_lanes,
+                     static_cast<const uint16_t*>(nullptr), static_cast<uint16_t*>(nullptr), static_cast<int64_t>(1),
+                     static_cast<int64_t>(0));
+  return static_cast<int>(hipGetLastError());
+}
+
+// The tile map for hipEngine's other tile heights: 16 rows (its WMMA tiles) and 64.
+extern "C" int hipengine_qwen35_moe_wmma_tile_map(const int64_t* expert_start_compact, int64_t* wmma_expert_start,
+                                                  int64_t* tile_expert, int64_t* wmma_total_out, int64_t num_experts,
+                                                  int64_t tile_capacity, hipStream_t stream) {
+  if (tile_capacity < 0) return static_cast<int>(hipErrorInvalidValue);
+  return launch_tile_map(expert_start_compact, wmma_expert_start, tile_expert, wmma_total_out, num_experts,
+                         tile_capacity, 16, stream);
+}
+
+extern "C" int hipengine_qwen35_moe_mmq64_tile_map(const int64_t* expert_start_compact, int64_t* mmq_expert_start,
+                                                   int64_t* tile_expert, int64_t* mmq_total_out, int64_t num_experts,
+                                                   int64_t tile_capacity, hipStream_t stream) {
+  if (tile_capacity < 0) return static_cast<int>(hipErrorInvalidValue);
+  return launch_tile_map(expert_start_compact, mmq_expert_start, tile_expert, mmq_total_out, num_experts,
+                         tile_capacity, 64, stream);
 }
 
 extern "C" int hipengine_gfx950_moe_lane_to_compact(const int64_t* sorted_lanes, int64_t* lane_to_compact,

@@ -26,10 +26,10 @@ def _check_num_experts(num_experts: int) -> None:
 def qwen35_moe_group_compact_active(selected_experts_ptr: int, routing_weights_ptr: int, expert_start_ptr: int,
                                     active_experts_ptr: int, active_count_ptr: int, sorted_lanes_ptr: int,
                                     sorted_experts_ptr: int, sorted_weights_ptr: int, total_lanes: int,
-                                    num_experts: int, *, stream: int = 0, library: ctypes.CDLL | None = None,
-                                    runtime: HipRuntime | None = None) -> None:
+                                    num_experts: int, *, parallel: bool = False, stream: int = 0,
+                                    library: ctypes.CDLL | None = None, runtime: HipRuntime | None = None) -> None:
     """Expert-major compaction: starts, active list, lanes (ascending within an
-    expert), experts and weights in that order."""
+    expert), experts and weights in that order.  ``parallel`` is accepted for signature compatibility."""
     _check_num_experts(num_experts)
     if total_lanes <= 0:
         raise ValueError("total_lanes must be positive")
@@ -106,6 +106,90 @@ def qwen35_moe_mmq32_tile_map(expert_start_compact_ptr: int, mmq_expert_start_pt
     fn = entry("hipengine_qwen35_moe_mmq32_tile_map", [VOID] * 4 + [I64, I64, VOID], library)
     check_launch(fn(expert_start_compact_ptr, mmq_expert_start_ptr, tile_expert_ptr, mmq_total_ptr, num_experts,
                     tile_capacity, stream), runtime)
+
+
+def qwen35_moe_group_compact_active_parallel(*args, **kwargs) -> None:
+    """hipEngine's parallel compaction (``moe/group_scatter.py:310-314``): the same arrays from the same kernels."""
+    kwargs["parallel"] = True
+    qwen35_moe_group_compact_active(*args, **kwargs)
+
+
+def qwen35_moe_group_compact_active_source_rows_parallel(*args, **kwargs) -> None:
+    """hipEngine's parallel compaction with source rows (``moe/group_scatter.py:372-379``)."""
+    kwargs["parallel"] = True
+    qwen35_moe_group_compact_active_source_rows(*args, **kwargs)
+
+
+def qwen35_moe_group_compact_active_i32_parallel(selected_experts_ptr: int, routing_weights_ptr: int,
+                                                 expert_start_ptr: int, active_experts_ptr: int, active_count_ptr: int,
+                                                 sorted_lanes_ptr: int, sorted_experts_ptr: int, sorted_weights_ptr: int,
+                                                 total_lanes: int, num_experts: int, *, stream: int = 0,
+                                                 library: ctypes.CDLL | None = None,
+                                                 runtime: HipRuntime | None = None) -> None:
+    """The compaction for int32 selected-expert ids (``moe/group_scatter.py:317-369``)."""
+    _check_num_experts(num_experts)
+    if total_lanes <= 0:
+        raise ValueError("total_lanes must be positive")
+    validate_pointers(selected_experts_ptr=selected_experts_ptr, routing_weights_ptr=routing_weights_ptr,
+                      expert_start_ptr=expert_start_ptr, sorted_lanes_ptr=sorted_lanes_ptr,
+                      sorted_weights_ptr=sorted_weights_ptr)
+    fn = entry("hipengine_qwen35_moe_group_compact_active_i32_parallel", [VOID] * 8 + [I64, I64, VOID], library)
+    check_launch(fn(selected_experts_ptr, routing_weights_ptr, expert_start_ptr, active_experts_ptr, active_count_ptr,
+                    sorted_lanes_ptr, sorted_experts_ptr, sorted_weights_ptr, total_lanes, num_experts, stream), runtime)
+
+
+def qwen35_moe_group_prefix_active(counts_ptr: int, expert_start_ptr: int, active_experts_ptr: int,
+                                   active_count_ptr: int, num_experts: int, *, stream: int = 0,
+                                   library: ctypes.CDLL | None = None, runtime: HipRuntime | None = None) -> None:
+    """int32 counts -> int64 compact starts ``[num_experts + 1]`` and the ascending list of the experts with rows
+    (``moe/group_scatter.py:147-181``)."""
+    _check_num_experts(num_experts)
+    validate_pointers(counts_ptr=counts_ptr, expert_start_ptr=expert_start_ptr, active_experts_ptr=active_experts_ptr,
+                      active_count_ptr=active_count_ptr)
+    fn = entry("hipengine_qwen35_moe_group_prefix_active", [VOID] * 4 + [I64, VOID], library)
+    check_launch(fn(counts_ptr, expert_start_ptr, active_experts_ptr, active_count_ptr, num_experts, stream), runtime)
+
+
+def qwen35_moe_group_scatter(selected_experts_ptr: int, routing_weights_ptr: int, expert_start_ptr: int,
+                             scatter_offsets_ptr: int, sorted_lanes_ptr: int, sorted_experts_ptr: int,
+                             sorted_weights_ptr: int, total_lanes: int, num_experts: int, *,
+                             include_routing_weights: bool = True, stream: int = 0,
+                             library: ctypes.CDLL | None = None, runtime: HipRuntime | None = None) -> None:
+    """Scatter of the lanes into per-expert compact order from given starts; the caller zeroes the offsets
+    (``moe/group_scatter.py:505-555``).  hipEngine's scatter takes its slots with atomics in arrival order; here an
+    expert's lanes are placed in ascending order, one of the orders that can produce."""
+    _check_positive(total_lanes, "total_lanes")
+    _check_num_experts(num_experts)
+    validate_pointers(selected_experts_ptr=selected_experts_ptr, expert_start_ptr=expert_start_ptr,
+                      scatter_offsets_ptr=scatter_offsets_ptr, sorted_lanes_ptr=sorted_lanes_ptr,
+                      sorted_experts_ptr=sorted_experts_ptr)
+    if include_routing_weights:
+        validate_pointers(routing_weights_ptr=routing_weights_ptr, sorted_weights_ptr=sorted_weights_ptr)
+    fn = entry("hipengine_qwen35_moe_group_scatter", [VOID] * 7 + [I64, I64, ctypes.c_bool, VOID], library)
+    check_launch(fn(selected_experts_ptr, routing_weights_ptr or None, expert_start_ptr, scatter_offsets_ptr,
+                    sorted_lanes_ptr, sorted_experts_ptr, sorted_weights_ptr or None, total_lanes, num_experts,
+                    bool(include_routing_weights), stream), runtime)
+
+
+def _tile_map(symbol: str, rows: int):
+    def wrapper(expert_start_compact_ptr: int, tile_expert_start_ptr: int, tile_expert_ptr: int, total_ptr: int,
+                num_experts: int, *, tile_capacity: int = 0, stream: int = 0, library: ctypes.CDLL | None = None,
+                runtime: HipRuntime | None = None) -> None:
+        _check_num_experts(num_experts)
+        if tile_capacity < 0:
+            raise ValueError("tile_capacity must be non-negative")
+        validate_pointers(expert_start_compact_ptr=expert_start_compact_ptr, tile_expert_start_ptr=tile_expert_start_ptr,
+                          tile_expert_ptr=tile_expert_ptr, total_ptr=total_ptr)
+        fn = entry(symbol, [VOID] * 4 + [I64, I64, VOID], library)
+        check_launch(fn(expert_start_compact_ptr, tile_expert_start_ptr, tile_expert_ptr, total_ptr, num_experts,
+                        tile_capacity, stream), runtime)
+
+    wrapper.__doc__ = f"Compact expert starts -> {rows}-row tile starts and the tile -> expert map (``{symbol}``)."
+    return wrapper
+
+
+qwen35_moe_wmma_tile_map = _tile_map("hipengine_qwen35_moe_wmma_tile_map", 16)      # moe/group_scatter.py:382-420
+qwen35_moe_mmq64_tile_map = _tile_map("hipengine_qwen35_moe_mmq64_tile_map", 64)    # moe/group_scatter.py:464-502
 
 
 def moe_lane_to_compact(sorted_lanes_ptr: int, lane_to_compact_ptr: int, compact_rows: int, total_lanes: int, *,
@@ -207,4 +291,16 @@ def register_kernels(backend: str = "hip_gfx950", *, replace: bool = False) -> N
     register(KernelKey(backend, "moe_group_compact", "generic", "active_experts_source_rows"),
              qwen35_moe_group_compact_active_source_rows, replace=replace)
     register(KernelKey(backend, "moe_mmq_tile_map", "generic", "tile32"), qwen35_moe_mmq32_tile_map, replace=replace)
+    register(KernelKey(backend, "moe_mmq_tile_map", "generic", "tile64"), qwen35_moe_mmq64_tile_map, replace=replace)
+    for quant, variant in (("generic", "tile16"), ("w4_paro", "qwen35")):
+        register(KernelKey(backend, "moe_wmma_tile_map", quant, variant), qwen35_moe_wmma_tile_map, replace=replace)
+    register(KernelKey(backend, "moe_group_prefix", "generic", "active_experts"), qwen35_moe_group_prefix_active,
+             replace=replace)
+    register(KernelKey(backend, "moe_group_compact", "generic", "active_experts_parallel"),
+             qwen35_moe_group_compact_active_parallel, replace=replace)
+    register(KernelKey(backend, "moe_group_compact", "generic", "active_experts_i32_parallel"),
+             qwen35_moe_group_compact_active_i32_parallel, replace=replace)
+    register(KernelKey(backend, "moe_group_compact", "generic", "active_experts_source_rows_parallel"),
+             qwen35_moe_group_compact_active_source_rows_parallel, replace=replace)
+    register(KernelKey(backend, "moe_group_scatter", "w4_paro", "qwen35"), qwen35_moe_group_scatter, replace=replace)
     register(KernelKey(backend, "moe_lane_to_compact", "generic", "sorted_lanes"), moe_lane_to_compact, replace=replace)

@@ -22,6 +22,7 @@
 #ifndef HIPENGINE_GFX950_H
 #define HIPENGINE_GFX950_H
 
+#include <stdbool.h>
 #include <stdint.h>
 
 #ifdef __cplusplus
@@ -469,6 +470,46 @@ int hipengine_qwen35_moe_gather_packed_hidden_lowp(const uint16_t* hidden_states
 int hipengine_qwen35_moe_mmq32_tile_map(const int64_t* expert_start_compact, int64_t* mmq_expert_start,
                                         int64_t* tile_expert, int64_t* mmq_total_out, int64_t num_experts,
                                         int64_t tile_capacity, hipengine_stream_t stream);
+
+/* The same map for hipEngine's other tile heights: 16 rows (moe/group_scatter.hip:994-1021) and 64 (:1054-1083). */
+int hipengine_qwen35_moe_wmma_tile_map(const int64_t* expert_start_compact, int64_t* wmma_expert_start,
+                                       int64_t* tile_expert, int64_t* wmma_total_out, int64_t num_experts,
+                                       int64_t tile_capacity, hipengine_stream_t stream);
+int hipengine_qwen35_moe_mmq64_tile_map(const int64_t* expert_start_compact, int64_t* mmq_expert_start,
+                                        int64_t* tile_expert, int64_t* mmq_total_out, int64_t num_experts,
+                                        int64_t tile_capacity, hipengine_stream_t stream);
+
+/* hipEngine's "parallel" compaction names (moe/group_scatter.hip:909-992): the arrays of the stable compaction above,
+ * which they equal there too (one workgroup per expert, ascending lanes); the i32 form takes int32 expert ids. */
+int hipengine_qwen35_moe_group_compact_active_parallel(const int64_t* selected_experts, const float* routing_weights,
+                                                       int64_t* expert_start, int64_t* active_experts,
+                                                       int64_t* active_count, int64_t* sorted_lanes,
+                                                       int64_t* sorted_experts, float* sorted_weights,
+                                                       int64_t total_lanes, int64_t num_experts,
+                                                       hipengine_stream_t stream);
+int hipengine_qwen35_moe_group_compact_active_source_rows_parallel(
+    const int64_t* selected_experts, const float* routing_weights, int64_t* expert_start, int64_t* active_experts,
+    int64_t* active_count, int64_t* sorted_lanes, int64_t* compact_to_source, float* sorted_weights,
+    int64_t total_lanes, int64_t num_experts, int64_t top_k, hipengine_stream_t stream);
+int hipengine_qwen35_moe_group_compact_active_i32_parallel(const int32_t* selected_experts, const float* routing_weights,
+                                                           int64_t* expert_start, int64_t* active_experts,
+                                                           int64_t* active_count, int64_t* sorted_lanes,
+                                                           int64_t* sorted_experts, float* sorted_weights,
+                                                           int64_t total_lanes, int64_t num_experts,
+                                                           hipengine_stream_t stream);
+
+/* int32 counts [num_experts] -> expert_start [num_experts + 1] (exclusive prefix), the ascending list of the experts
+ * with a positive count and their number (moe/group_scatter.hip:735-758). */
+int hipengine_qwen35_moe_group_prefix_active(const int32_t* counts, int64_t* expert_start, int64_t* active_experts,
+                                             int64_t* active_count, int64_t num_experts, hipengine_stream_t stream);
+
+/* Scatter of the lanes into per-expert order from given starts; scatter_offsets [num_experts] is zeroed by the caller
+ * and ends as the per-expert counts (moe/group_scatter.hip:1085-1118).  hipEngine takes an expert's slots with atomics
+ * in arrival order; here its lanes land in ascending order (one of those orders, and a deterministic one). */
+int hipengine_qwen35_moe_group_scatter(const int64_t* selected_experts, const float* routing_weights,
+                                       const int64_t* expert_start, int32_t* scatter_offsets, int64_t* sorted_lanes,
+                                       int64_t* sorted_experts, float* sorted_weights, int64_t total_lanes,
+                                       int64_t num_experts, bool include_routing_weights, hipengine_stream_t stream);
 
 /* lane_to_compact[total_lanes]: position of each lane in sorted_lanes, -1 for a
  * dropped lane.  New here (hipEngine scatters with atomics instead,

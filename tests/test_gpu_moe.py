@@ -92,6 +92,66 @@ def _device_index(dev, sel, w, num_experts, tile_capacity=0):
     return host, d
 
 
+@pytest.mark.parametrize("tokens,top_k,experts,bad", [(1, 8, 256, False), (300, 4, 64, True), (77, 2, 5, True)])
+def test_routing_index_other_entry_names(dev, tokens, top_k, experts, bad):
+    """hipEngine's other names for the same index, each against the oracle's arrays: the "parallel" compactions (int64
+    and int32 expert ids), the prefix with the active list from counts in memory, the scatter from given starts
+    (ascending lanes; offsets end as the counts), and the tile maps of 16- and 64-row tiles."""
+    sel, w = _routing(tokens + experts, tokens, top_k, experts, bad)
+    want = O.build_routing_index(sel, w, experts)
+    total, lanes = want["total"], tokens * top_k
+    dsel, dsel32, dw = dev.put(sel), dev.put(sel.astype(np.int32)), dev.put(w)
+
+    def outputs():
+        return {"es": dev.empty((experts + 1) * 8), "act": dev.empty(experts * 8, fill=0xFF), "actn": dev.empty(8),
+                "sl": dev.empty(lanes * 8, fill=0xFF), "aux": dev.empty(lanes * 8, fill=0xFF), "sw": dev.empty(lanes * 4)}
+
+    def check(o, aux_want):
+        assert np.array_equal(dev.get(o["es"], np.int64, (experts + 1,)), want["expert_start"])
+        assert int(dev.get(o["actn"], np.int64, (1,))[0]) == want["active_count"]
+        assert np.array_equal(dev.get(o["act"], np.int64, (experts,))[:want["active_count"]], want["active_experts"])
+        assert np.array_equal(dev.get(o["sl"], np.int64, (lanes,))[:total], want["sorted_lanes"])
+        assert np.array_equal(dev.get(o["aux"], np.int64, (lanes,))[:total], aux_want)
+        assert np.array_equal(dev.get(o["sw"], np.float32, (lanes,))[:total].view(np.uint32),
+                              want["sorted_weights"].view(np.uint32))
+        dev.free(*o.values())
+
+    sorted_experts = sel.reshape(-1)[want["sorted_lanes"]]
+    o = outputs()
+    GS.qwen35_moe_group_compact_active_parallel(dsel.ptr, dw.ptr, o["es"].ptr, o["act"].ptr, o["actn"].ptr, o["sl"].ptr,
+                                                o["aux"].ptr, o["sw"].ptr, lanes, experts)
+    check(o, sorted_experts)
+    o = outputs()
+    GS.qwen35_moe_group_compact_active_i32_parallel(dsel32.ptr, dw.ptr, o["es"].ptr, o["act"].ptr, o["actn"].ptr,
+                                                    o["sl"].ptr, o["aux"].ptr, o["sw"].ptr, lanes, experts)
+    check(o, sorted_experts)
+    o = outputs()
+    GS.qwen35_moe_group_compact_active_source_rows_parallel(dsel.ptr, dw.ptr, o["es"].ptr, o["act"].ptr, o["actn"].ptr,
+                                                            o["sl"].ptr, o["aux"].ptr, o["sw"].ptr, lanes, experts, top_k)
+    check(o, want["compact_to_source"])
+
+    # count -> prefix with the active list -> scatter from the starts
+    o = outputs()
+    counts, offsets = dev.empty(experts * 4, fill=0), dev.empty(experts * 4, fill=0)
+    GS.qwen35_moe_group_count(dsel.ptr, counts.ptr, lanes, experts)
+    GS.qwen35_moe_group_prefix_active(counts.ptr, o["es"].ptr, o["act"].ptr, o["actn"].ptr, experts)
+    GS.qwen35_moe_group_scatter(dsel.ptr, dw.ptr, o["es"].ptr, offsets.ptr, o["sl"].ptr, o["aux"].ptr, o["sw"].ptr,
+                                lanes, experts)
+    assert np.array_equal(dev.get(offsets, np.int32, (experts,)), np.diff(want["expert_start"]).astype(np.int32))
+    es_dev = o["es"]
+    for rows, fn in ((16, GS.qwen35_moe_wmma_tile_map), (64, GS.qwen35_moe_mmq64_tile_map)):
+        cap = lanes // rows + experts + 1
+        ts, te, tt = dev.empty((experts + 1) * 8), dev.empty(cap * 8, fill=0x11), dev.empty(8)
+        fn(es_dev.ptr, ts.ptr, te.ptr, tt.ptr, experts, tile_capacity=cap)
+        tm = O.tile_map(want["expert_start"], experts, rows, cap)
+        assert np.array_equal(dev.get(ts, np.int64, (experts + 1,)), tm["tile_expert_start"])
+        assert np.array_equal(dev.get(te, np.int64, (cap,)), tm["tile_expert"])
+        assert int(dev.get(tt, np.int64, (1,))[0]) == tm["total"]
+        dev.free(ts, te, tt)
+    check(o, sorted_experts)
+    dev.free(dsel, dsel32, dw, counts, offsets)
+
+
 @pytest.mark.parametrize("tokens,experts,top_k,stride", [(1, 256, 8, 256), (7, 256, 8, 257), (33, 60, 4, 64),
                                                         (5, 1024, 16, 1024), (3, 8, 8, 8), (2048, 256, 8, 256)])
 def test_router_select(dev, tokens, experts, top_k, stride):

@@ -305,6 +305,14 @@ def test_moe_wrappers_validate_before_touching_the_device():
         M.gguf_q6_k_grouped_mmq(1, 1, 1, 0, 1, 1, 8, 8, 256, 64, 4, 128)
     with pytest.raises(ValueError, match="tile_rows"):
         GS.moe_tile_map(1, 1, 1, 1, 8, tile_rows=48)
+    with pytest.raises(ValueError, match="total_lanes must be positive"):
+        GS.qwen35_moe_group_scatter(1, 1, 1, 1, 1, 1, 1, 0, 8)
+    with pytest.raises(ValueError, match="non-null"):
+        GS.qwen35_moe_group_scatter(1, 0, 1, 1, 1, 1, 1, 16, 8)          # weights asked for, no pointer
+    with pytest.raises(ValueError, match="num_experts"):
+        GS.qwen35_moe_group_prefix_active(1, 1, 1, 1, 0)
+    with pytest.raises(ValueError, match="tile_capacity"):
+        GS.qwen35_moe_wmma_tile_map(1, 1, 1, 1, 8, tile_capacity=-2)
     from hipengine_amd.kernels.hip_gfx950.fused import paro_combine as PC
     with pytest.raises(ValueError, match="features must be positive"):
         PC.shared_gate_combine_residual_rmsnorm_gguf_bf16_out(1, 1, 1, 1, 1, 1, 1, 4, 0, 1)
