@@ -268,6 +268,15 @@ DEFINE_MMQ_Q5(hipengine_gguf_q5_k_mmq32_q8_1_d4s4_f32_bf16_bf16_out, KIND_BF16)
 DEFINE_MMQ_Q6(hipengine_gguf_q6_k_mmq32_q8_1_d4s4_f32_bf16_f32_out, KIND_F32)
 DEFINE_MMQ_Q6(hipengine_gguf_q6_k_mmq32_q8_1_d4s4_f32_bf16_bf16_out, KIND_BF16)
 
+// hipEngine's scheduling variants of the same GEMMs (gguf_k_mmq_prefill.hip:2565-2578 "pipe" and "mb4",
+// :2315-2366 "direct_dp4a"): one kernel form here, the same results.
+DEFINE_MMQ_Q5(hipengine_gguf_q5_k_mmq32_pipe_q8_1_d4s4_f32_bf16_bf16_out, KIND_BF16)
+DEFINE_MMQ_Q5(hipengine_gguf_q5_k_mmq32_mb4_q8_1_d4s4_f32_bf16_bf16_out, KIND_BF16)
+DEFINE_MMQ_Q5(hipengine_gguf_q5_k_mmq32_direct_dp4a_q8_1_d4s4_f32_bf16_bf16_out, KIND_BF16)
+DEFINE_MMQ_Q5(hipengine_gguf_q5_k_mmq32_direct_dp4a_q8_1_d4s4_f32_bf16_f32_out, KIND_F32)
+DEFINE_MMQ_Q6(hipengine_gguf_q6_k_mmq32_pipe_q8_1_d4s4_f32_bf16_bf16_out, KIND_BF16)
+DEFINE_MMQ_Q6(hipengine_gguf_q6_k_mmq32_mb4_q8_1_d4s4_f32_bf16_bf16_out, KIND_BF16)
+
 #define DEFINE_MMQ_Q8_0(SYMBOL, OKIND)                                                                      \
   extern "C" int SYMBOL(const void* xq, const uint8_t* qweight, void* out, int64_t rows, int64_t in_features, \
                         int64_t out_features, hipStream_t stream) {                                         \

@@ -1775,6 +1775,18 @@ extern "C" int hipengine_gguf_q4_k_selected_dual_q8_1_ds4_mmq32_prefill_compact3
                         out_features_b, num_experts, mmq_total_rows, expert_stride_rows, stream);
 }
 
+// hipEngine's 32 x 128 tile variant of the same GEMM (gguf_q4_k_q8_1_selected_prefill.hip:7510-7548): no expert
+// stride argument.
+extern "C" int hipengine_gguf_q4_k_selected_dual_q8_1_ds4_mmq32x128_prefill_compact32_bf16_bf16_out(
+    const void* x_q8, const int64_t* compact_to_source, const int64_t* expert_start_compact,
+    const int64_t* expert_start_mmq32, const int64_t* tile_expert, const uint8_t* qweight_a, const uint8_t* qweight_b,
+    uint16_t* out, int64_t compact_rows, int64_t in_features, int64_t out_features_a, int64_t out_features_b,
+    int64_t num_experts, int64_t mmq_total_rows, hipStream_t stream) {
+  return hipengine_gguf_q4_k_selected_dual_q8_1_ds4_mmq32_prefill_compact32_bf16_bf16_out(
+      x_q8, compact_to_source, expert_start_compact, expert_start_mmq32, tile_expert, qweight_a, qweight_b, out,
+      compact_rows, in_features, out_features_a, out_features_b, num_experts, mmq_total_rows, 0, stream);
+}
+
 extern "C" int hipengine_gfx950_gguf_q4_k_grouped_mmq(const void* x_q8, const int64_t* compact_to_source,
                                                       const int64_t* expert_start_compact,
                                                       const int64_t* expert_start_mmq32, const int64_t* tile_expert,

@@ -58,6 +58,18 @@ gguf_q6_k_mmq32_q8_1_d4s4_f32_bf16_f32_out = _make(
 gguf_q6_k_mmq32_q8_1_d4s4_f32_bf16_bf16_out = _make(
     "gguf_q6_k_mmq32_q8_1_d4s4_f32_bf16_bf16_out", "hipengine_gguf_q6_k_mmq32_q8_1_d4s4_f32_bf16_bf16_out", 1)
 
+# hipEngine's scheduling variants of the Q5_K GEMM (gguf_k_mmq_prefill.py:459-640): the one kernel form here
+gguf_q5_k_mmq32_pipe_q8_1_d4s4_f32_bf16_bf16_out = _make(
+    "gguf_q5_k_mmq32_pipe_q8_1_d4s4_f32_bf16_bf16_out", "hipengine_gguf_q5_k_mmq32_pipe_q8_1_d4s4_f32_bf16_bf16_out", 32)
+gguf_q5_k_mmq32_mb4_q8_1_d4s4_f32_bf16_bf16_out = _make(
+    "gguf_q5_k_mmq32_mb4_q8_1_d4s4_f32_bf16_bf16_out", "hipengine_gguf_q5_k_mmq32_mb4_q8_1_d4s4_f32_bf16_bf16_out", 32)
+gguf_q5_k_mmq32_direct_dp4a_q8_1_d4s4_f32_bf16_bf16_out = _make(
+    "gguf_q5_k_mmq32_direct_dp4a_q8_1_d4s4_f32_bf16_bf16_out",
+    "hipengine_gguf_q5_k_mmq32_direct_dp4a_q8_1_d4s4_f32_bf16_bf16_out", 32)
+gguf_q5_k_mmq32_direct_dp4a_q8_1_d4s4_f32_bf16_f32_out = _make(
+    "gguf_q5_k_mmq32_direct_dp4a_q8_1_d4s4_f32_bf16_f32_out",
+    "hipengine_gguf_q5_k_mmq32_direct_dp4a_q8_1_d4s4_f32_bf16_f32_out", 32)
+
 # Q8_0 x D4S4 (new here: hipEngine has no MMQ for Q8_0): 128 values per D4S4 block
 gguf_q8_0_mmq32_q8_1_d4s4_f32_bf16_f32_out = _make(
     "gguf_q8_0_mmq32_q8_1_d4s4_f32_bf16_f32_out", "hipengine_gguf_q8_0_mmq32_q8_1_d4s4_f32_bf16_f32_out", 1, 128)
@@ -91,6 +103,11 @@ def register_kernels(backend: str = "hip_gfx950", *, replace: bool = False) -> N
              gguf_q5_k_mmq32_q8_1_d4s4_f32_bf16_f32_out, replace=replace)
     register(KernelKey(backend, "linear", "gguf_q5_k", "mmq32_q8_1_d4s4_f32_bf16_bf16_out"),
              gguf_q5_k_mmq32_q8_1_d4s4_f32_bf16_bf16_out, replace=replace)
+    for variant, fn in (("mmq32_pipe_q8_1_d4s4_f32_bf16_bf16_out", gguf_q5_k_mmq32_pipe_q8_1_d4s4_f32_bf16_bf16_out),
+                        ("mmq32_mb4_q8_1_d4s4_f32_bf16_bf16_out", gguf_q5_k_mmq32_mb4_q8_1_d4s4_f32_bf16_bf16_out),
+                        ("mmq32_direct_dp4a_q8_1_d4s4_f32_bf16_bf16_out", gguf_q5_k_mmq32_direct_dp4a_q8_1_d4s4_f32_bf16_bf16_out),
+                        ("mmq32_direct_dp4a_q8_1_d4s4_f32_bf16_f32_out", gguf_q5_k_mmq32_direct_dp4a_q8_1_d4s4_f32_bf16_f32_out)):
+        register(KernelKey(backend, "linear", "gguf_q5_k", variant), fn, replace=replace)
     register(KernelKey(backend, "linear", "gguf_q6_k", "mmq32_q8_1_d4s4_f32_bf16_f32_out"),
              gguf_q6_k_mmq32_q8_1_d4s4_f32_bf16_f32_out, replace=replace)
     register(KernelKey(backend, "linear", "gguf_q6_k", "mmq32_q8_1_d4s4_f32_bf16_bf16_out"),

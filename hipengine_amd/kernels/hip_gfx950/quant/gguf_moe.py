@@ -273,6 +273,25 @@ def gguf_q4_k_selected_dual_q8_1_ds4_mmq32_prefill_compact32_bf16_bf16_out(
                     num_experts, mmq_total_rows, expert_stride_rows, stream), runtime)
 
 
+def gguf_q4_k_selected_dual_q8_1_ds4_mmq32x128_prefill_compact32_bf16_bf16_out(
+        x_q8_ptr: int, compact_to_source_ptr: int, expert_start_compact_ptr: int, expert_start_mmq32_ptr: int,
+        mmq_tile_expert_ptr: int, qweight_a_ptr: int, qweight_b_ptr: int, out_ptr: int, compact_rows: int,
+        in_features: int, out_features_a: int, out_features_b: int, num_experts: int, mmq_total_rows: int, *,
+        stream: int = 0, library: ctypes.CDLL | None = None, runtime: HipRuntime | None = None) -> None:
+    """hipEngine's 128-wide K pass of the same GEMM (``gguf_q4_k_q8_1_selected_prefill.py:1895-1960``): identical
+    arithmetic, the one kernel form here."""
+    _validate_grouped(compact_rows, in_features, out_features_a, out_features_b, num_experts, mmq_total_rows)
+    validate_pointers(x_q8_ptr=x_q8_ptr, compact_to_source_ptr=compact_to_source_ptr,
+                      expert_start_compact_ptr=expert_start_compact_ptr, expert_start_mmq32_ptr=expert_start_mmq32_ptr,
+                      mmq_tile_expert_ptr=mmq_tile_expert_ptr, qweight_a_ptr=qweight_a_ptr, qweight_b_ptr=qweight_b_ptr,
+                      out_ptr=out_ptr)
+    fn = entry("hipengine_gguf_q4_k_selected_dual_q8_1_ds4_mmq32x128_prefill_compact32_bf16_bf16_out",
+               [VOID] * 8 + [I64] * 6 + [VOID], library)
+    check_launch(fn(x_q8_ptr, compact_to_source_ptr, expert_start_compact_ptr, expert_start_mmq32_ptr,
+                    mmq_tile_expert_ptr, qweight_a_ptr, qweight_b_ptr, out_ptr, compact_rows, in_features,
+                    out_features_a, out_features_b, num_experts, mmq_total_rows, stream), runtime)
+
+
 def gguf_q4_k_grouped_mmq(x_q8_ptr: int, expert_start_compact_ptr: int, expert_start_mmq32_ptr: int,
                           tile_expert_ptr: int, qweight_a_ptr: int, out_ptr: int, compact_rows: int, source_rows: int,
                           in_features: int, out_features_a: int, num_experts: int, mmq_total_rows: int, *,
@@ -418,6 +437,9 @@ def register_kernels(backend: str = "hip_gfx950", *, replace: bool = False) -> N
     register(KernelKey(backend, "moe_linear", "gguf_q4_k",
                        "selected_dual_q8_1_ds4_mmq32_prefill_compact32_bf16_bf16_out"),
              gguf_q4_k_selected_dual_q8_1_ds4_mmq32_prefill_compact32_bf16_bf16_out, replace=replace)
+    register(KernelKey(backend, "moe_linear", "gguf_q4_k",
+                       "selected_dual_q8_1_ds4_mmq32x128_prefill_compact32_bf16_bf16_out"),
+             gguf_q4_k_selected_dual_q8_1_ds4_mmq32x128_prefill_compact32_bf16_bf16_out, replace=replace)
     for _q in ("gguf_q4_k", "gguf_q5_k", "gguf_q6_k", "gguf_q8_0"):
         register(KernelKey(backend, "moe_linear", _q, "grouped_gemv_rowbatch8"),
                  (lambda q: lambda *a, **k: gguf_grouped_gemv(q, *a, **k))(_q), replace=replace)

@@ -324,6 +324,28 @@ int hipengine_gguf_q6_k_mmq32_q8_1_d4s4_f32_bf16_bf16_out(const void* xq, const 
                                                           int64_t rows, int64_t in_features, int64_t out_features,
                                                           hipengine_stream_t stream);
 
+/* hipEngine's scheduling variants of the two GEMMs above (gguf_k_mmq_prefill.hip:2565-2578 "pipe" and "mb4",
+ * :2315-2366 "direct_dp4a"): the same arguments and results from the one kernel form here (Q5_K: out_features % 32
+ * == 0, which hipEngine's direct_dp4a form does not ask for). */
+int hipengine_gguf_q5_k_mmq32_pipe_q8_1_d4s4_f32_bf16_bf16_out(const void* xq, const uint8_t* qweight, void* out,
+                                                               int64_t rows, int64_t in_features,
+                                                               int64_t out_features, hipengine_stream_t stream);
+int hipengine_gguf_q5_k_mmq32_mb4_q8_1_d4s4_f32_bf16_bf16_out(const void* xq, const uint8_t* qweight, void* out,
+                                                              int64_t rows, int64_t in_features, int64_t out_features,
+                                                              hipengine_stream_t stream);
+int hipengine_gguf_q5_k_mmq32_direct_dp4a_q8_1_d4s4_f32_bf16_bf16_out(const void* xq, const uint8_t* qweight, void* out,
+                                                                      int64_t rows, int64_t in_features,
+                                                                      int64_t out_features, hipengine_stream_t stream);
+int hipengine_gguf_q5_k_mmq32_direct_dp4a_q8_1_d4s4_f32_bf16_f32_out(const void* xq, const uint8_t* qweight, void* out,
+                                                                     int64_t rows, int64_t in_features,
+                                                                     int64_t out_features, hipengine_stream_t stream);
+int hipengine_gguf_q6_k_mmq32_pipe_q8_1_d4s4_f32_bf16_bf16_out(const void* xq, const uint8_t* qweight, void* out,
+                                                               int64_t rows, int64_t in_features,
+                                                               int64_t out_features, hipengine_stream_t stream);
+int hipengine_gguf_q6_k_mmq32_mb4_q8_1_d4s4_f32_bf16_bf16_out(const void* xq, const uint8_t* qweight, void* out,
+                                                              int64_t rows, int64_t in_features, int64_t out_features,
+                                                              hipengine_stream_t stream);
+
 /* Raw Q8_0 weights ([out_features, in_features/32 * 34]) x D4S4 activations: sum over the 32-value blocks of
  * xd_b * d_b * dot_b, the q8_1 x Q8_0 formula (gguf_q8_0_dp4a_gemv.hip:100-137) with the float32 activation scales
  * of the D4S4 block, on the int8 MFMA.  in_features a multiple of 128; any out_features >= 1.  hipEngine has no MMQ
@@ -715,6 +737,14 @@ int hipengine_gguf_q4_k_selected_dual_q8_1_ds4_mmq32_prefill_compact32_bf16_bf16
     const uint8_t* qweight_b, uint16_t* out, int64_t compact_rows, int64_t in_features, int64_t out_features_a,
     int64_t out_features_b, int64_t num_experts, int64_t mmq_total_rows, int64_t expert_stride_rows,
     hipengine_stream_t stream);
+
+/* hipEngine's 32 x 128 tile variant of the same GEMM (gguf_q4_k_q8_1_selected_prefill.hip:7510-7548): the same
+ * arguments without the expert stride, the same results. */
+int hipengine_gguf_q4_k_selected_dual_q8_1_ds4_mmq32x128_prefill_compact32_bf16_bf16_out(
+    const void* x_q8, const int64_t* compact_to_source, const int64_t* expert_start_compact,
+    const int64_t* expert_start_mmq32, const int64_t* tile_expert, const uint8_t* qweight_a, const uint8_t* qweight_b,
+    uint16_t* out, int64_t compact_rows, int64_t in_features, int64_t out_features_a, int64_t out_features_b,
+    int64_t num_experts, int64_t mmq_total_rows, hipengine_stream_t stream);
 
 /* The same with the output kind explicit (0 float32, 1 bf16, 2 fp16), the source
  * row count given (indices are clamped to it), compact_to_source optional (NULL:

@@ -300,3 +300,25 @@ def test_mmq_seeded_shape_sweep(dev, quant, rows, k, n):
     assert np.all(got[rows * n:].view(np.uint32) == 0x6B6B6B6B)          # nothing past the output
     got = got[:rows * n].reshape(rows, n)
     assert O.max_rel_err(got, want) <= 1e-3 and O.cosine(got, want) >= 0.99999
+
+
+def test_q5_k_and_q6_k_mmq_variant_names_are_the_same_gemm(dev):
+    """hipEngine's pipe / mb4 / direct_dp4a names: the bits of the plain entries."""
+    rows, k, n = 70, 512, 96
+    xb = _bf16_rows(3, rows, k, scale=0.2)
+    d4 = O.pack_q8_1_d4s4(xb)
+    w5 = _random_q5_k(n, k, seed=4)
+    base16 = _run_q4(dev, M.gguf_q5_k_mmq32_q8_1_d4s4_f32_bf16_bf16_out, d4, w5, rows, k, n, out_dtype=np.uint16)
+    base32 = _run_q4(dev, M.gguf_q5_k_mmq32_q8_1_d4s4_f32_bf16_f32_out, d4, w5, rows, k, n)
+    for fn in (M.gguf_q5_k_mmq32_pipe_q8_1_d4s4_f32_bf16_bf16_out, M.gguf_q5_k_mmq32_mb4_q8_1_d4s4_f32_bf16_bf16_out,
+               M.gguf_q5_k_mmq32_direct_dp4a_q8_1_d4s4_f32_bf16_bf16_out):
+        assert np.array_equal(_run_q4(dev, fn, d4, w5, rows, k, n, out_dtype=np.uint16), base16)
+    got = _run_q4(dev, M.gguf_q5_k_mmq32_direct_dp4a_q8_1_d4s4_f32_bf16_f32_out, d4, w5, rows, k, n)
+    assert np.array_equal(got.view(np.uint32), base32.view(np.uint32))
+    from hipengine_amd.kernels.hip_gfx950._launch import I64, VOID, check_launch, entry
+    w6 = O.random_weight(O.GGML_Q6_K, n, k, seed=6)
+    base6 = _run_q4(dev, M.gguf_q6_k_mmq32_q8_1_d4s4_f32_bf16_bf16_out, d4, w6, rows, k, n, out_dtype=np.uint16)
+    for name in ("pipe", "mb4"):
+        sym = entry(f"hipengine_gguf_q6_k_mmq32_{name}_q8_1_d4s4_f32_bf16_bf16_out", [VOID, VOID, VOID, I64, I64, I64, VOID])
+        fn = lambda xq, w, out, r, kk, nn, sym=sym: check_launch(sym(xq, w, out, r, kk, nn, 0), None)
+        assert np.array_equal(_run_q4(dev, fn, d4, w6, rows, k, n, out_dtype=np.uint16), base6)

@@ -540,9 +540,15 @@ def test_grouped_mmq_bf16_named_entry(dev):
     M.gguf_q4_k_selected_dual_q8_1_ds4_mmq32_prefill_compact32_bf16_bf16_out(
         dxq.ptr, d["c2s"].ptr, d["expert_start"].ptr, d["mmq_start"].ptr, d["tile_expert"].ptr, dwa.ptr, dwb.ptr,
         dout.ptr, total, k, na, nb, experts, host["mmq_total"])
-    b16 = dev.get(dout, np.uint16, (total, na + nb))
+    b16 = dev.get(dout, np.uint16, (total, na + nb)).copy()
+    dev.runtime.memset(dout.ptr, 0, total * (na + nb) * 2)
+    M.gguf_q4_k_selected_dual_q8_1_ds4_mmq32x128_prefill_compact32_bf16_bf16_out(
+        dxq.ptr, d["c2s"].ptr, d["expert_start"].ptr, d["mmq_start"].ptr, d["tile_expert"].ptr, dwa.ptr, dwb.ptr,
+        dout.ptr, total, k, na, nb, experts, host["mmq_total"])
+    wide = dev.get(dout, np.uint16, (total, na + nb)).copy()
     dev.free(dxq, dwa, dwb, dout, *d.values())
     assert np.array_equal(b16, O.f32_to_bf16_bits(f32))
+    assert np.array_equal(wide, b16)              # hipEngine's 32 x 128 variant name: the same GEMM
 
 
 @pytest.mark.parametrize("tokens,experts", [(256, 32), (2048, 256)])
