@@ -404,6 +404,41 @@ DEFINE_DENSE_ALL(q5_k, GGML_Q5_K)
 DEFINE_DENSE_ALL(q6_k, GGML_Q6_K)
 DEFINE_DENSE_ALL(q8_0, GGML_Q8_0)
 
+// hipEngine's per-shape tuning variants of the dense GEMV for Q5_K / Q6_K / Q8_0 (row batches, column tiles, wave
+// layouts, pipelining: gguf_k_gemv.hip:5665-5702,5869-5960,6161-6255): the same 8 arguments and the same product;
+// the launcher here picks the kernel form from the shape, so each of them is the dense launch (any shape, where
+// hipEngine restricts some of them to the shapes they were tuned for).
+#define DEFINE_DENSE_VARIANT(SYMBOL, QT, AKIND, OKIND)                                                    \
+  extern "C" int SYMBOL(const void* x, const uint8_t* qweight, void* out, int64_t rows, int64_t in_features, \
+                        int64_t out_features, int64_t /*threads*/, hipStream_t stream) {                  \
+    return launch_gemv(QT, x, AKIND, qweight, out, OKIND, rows, in_features, out_features, nullptr, stream); \
+  }
+#define DEFINE_DENSE_VARIANT_BF16(PREFIX, QT)                          \
+  DEFINE_DENSE_VARIANT(PREFIX##_bf16_bf16_out, QT, KIND_BF16, KIND_BF16) \
+  DEFINE_DENSE_VARIANT(PREFIX##_bf16_f32_out, QT, KIND_BF16, KIND_F32)
+DEFINE_DENSE_VARIANT_BF16(hipengine_gguf_q5_k_gemv_rowbatch8, GGML_Q5_K)
+DEFINE_DENSE_VARIANT_BF16(hipengine_gguf_q5_k_gemv_rowbatch32, GGML_Q5_K)
+DEFINE_DENSE_VARIANT_BF16(hipengine_gguf_q6_k_gemv_rowbatch8, GGML_Q6_K)
+DEFINE_DENSE_VARIANT_BF16(hipengine_gguf_q6_k_gemv_rowbatch32, GGML_Q6_K)
+DEFINE_DENSE_VARIANT_BF16(hipengine_gguf_q5_k_gemv_coltile2_rowbatch16, GGML_Q5_K)
+DEFINE_DENSE_VARIANT_BF16(hipengine_gguf_q5_k_gemv_coltile4_rowbatch8, GGML_Q5_K)
+DEFINE_DENSE_VARIANT_BF16(hipengine_gguf_q6_k_gemv_coltile2_rowbatch16, GGML_Q6_K)
+DEFINE_DENSE_VARIANT_BF16(hipengine_gguf_q6_k_gemv_coltile4_rowbatch8, GGML_Q6_K)
+DEFINE_DENSE_VARIANT_BF16(hipengine_gguf_q5_k_wave32x2_gemv_decode, GGML_Q5_K)
+DEFINE_DENSE_VARIANT_BF16(hipengine_gguf_q5_k_wave32x2_fixed_meta_gemv_decode, GGML_Q5_K)
+DEFINE_DENSE_VARIANT_BF16(hipengine_gguf_q5_k_wave32x2_swar_pair_fixed_meta_gemv_decode, GGML_Q5_K)
+DEFINE_DENSE_VARIANT(hipengine_gguf_q6_k_wave32x2_fixed_meta_gemv_decode_bf16_bf16_out, GGML_Q6_K, KIND_BF16, KIND_BF16)
+DEFINE_DENSE_VARIANT(hipengine_gguf_q6_k_gemv_dpp_wave_reduction_coltile4_rowbatch8_bf16_bf16_out, GGML_Q6_K, KIND_BF16, KIND_BF16)
+DEFINE_DENSE_VARIANT(hipengine_gguf_q6_k_gemv_dpp_wave_reduction_coltile2_rowbatch16_bf16_f32_out, GGML_Q6_K, KIND_BF16, KIND_F32)
+DEFINE_DENSE_VARIANT(hipengine_gguf_q6_k_gemv_dpp_wave_reduction_full_group_compute_coltile4_rowbatch8_bf16_bf16_out, GGML_Q6_K, KIND_BF16, KIND_BF16)
+DEFINE_DENSE_VARIANT(hipengine_gguf_q6_k_gemv_dpp_wave_reduction_full_group_compute_coltile2_rowbatch16_bf16_f32_out, GGML_Q6_K, KIND_BF16, KIND_F32)
+DEFINE_DENSE_VARIANT(hipengine_gguf_q8_0_gemv_coltile4_rowbatch8_pipelined_f32_f32_out, GGML_Q8_0, KIND_F32, KIND_F32)
+DEFINE_DENSE_VARIANT(hipengine_gguf_q8_0_gemv_coltile8_rowbatch4_pipelined_f32_f32_out, GGML_Q8_0, KIND_F32, KIND_F32)
+DEFINE_DENSE_VARIANT(hipengine_gguf_q8_0_gemv_coltile8_rowbatch4_wave_scale_f32_f32_out, GGML_Q8_0, KIND_F32, KIND_F32)
+DEFINE_DENSE_VARIANT(hipengine_gguf_q8_0_gemv_coltile8_rowbatch4_wave_scale_pipelined_f32_f32_out, GGML_Q8_0, KIND_F32, KIND_F32)
+DEFINE_DENSE_VARIANT(hipengine_gguf_q8_0_gemv_coltile8_rowbatch4_wave_scale_pipelined_dpp_f32_f32_out, GGML_Q8_0, KIND_F32, KIND_F32)
+DEFINE_DENSE_VARIANT(hipengine_gguf_q8_0_gemv_coltile8_rowbatch4_wave_scale_pipelined_dpp_checked_full_rows_f32_f32_out, GGML_Q8_0, KIND_F32, KIND_F32)
+
 // ---- pre-quantized q8_1 activations (36-byte blocks) ------------------------
 
 #define DEFINE_Q8_1(SYMBOL, QT, OKIND)                                                                   \
@@ -679,6 +714,25 @@ extern "C" int hipengine_gfx950_gguf_multi_gemv(int32_t count, const int32_t* gg
   }
   return static_cast<int>(hipSuccess);
 }
+
+// hipEngine's Q5_K pair decode names (two matrices of different heights over one bf16 activation row,
+// gguf_k_gemv.hip:6175-6255): the multi-matrix launch above.
+#define DEFINE_Q5_K_PAIR(SYMBOL, OKIND)                                                                       \
+  extern "C" int SYMBOL(const void* x, const uint8_t* qweight_a, const uint8_t* qweight_b, void* out_a, void* out_b, \
+                        int64_t rows, int64_t in_features, int64_t out_features_a, int64_t out_features_b,       \
+                        int64_t /*threads*/, hipStream_t stream) {                                             \
+    const int32_t types[2] = {GGML_Q5_K, GGML_Q5_K};                                                           \
+    const uint8_t* const weights[2] = {qweight_a, qweight_b};                                                  \
+    void* const outs[2] = {out_a, out_b};                                                                      \
+    const int64_t heights[2] = {out_features_a, out_features_b};                                               \
+    return hipengine_gfx950_gguf_multi_gemv(2, types, x, KIND_BF16, weights, outs, OKIND, rows, in_features,   \
+                                            heights, stream);                                                  \
+  }
+DEFINE_Q5_K_PAIR(hipengine_gguf_q5_k_pair_wave32x2_gemv_decode_bf16_f32_out, KIND_F32)
+DEFINE_Q5_K_PAIR(hipengine_gguf_q5_k_pair_wave32x2_fixed_meta_gemv_decode_bf16_bf16_out, KIND_BF16)
+DEFINE_Q5_K_PAIR(hipengine_gguf_q5_k_pair_wave32x2_fixed_meta_gemv_decode_bf16_f32_out, KIND_F32)
+DEFINE_Q5_K_PAIR(hipengine_gguf_q5_k_pair_wave32x2_swar_pair_fixed_meta_gemv_decode_bf16_bf16_out, KIND_BF16)
+DEFINE_Q5_K_PAIR(hipengine_gguf_q5_k_pair_wave32x2_swar_pair_fixed_meta_gemv_decode_bf16_f32_out, KIND_F32)
 
 // ---- fused epilogues: gate/up pair with SiLU, projection + residual -------------------
 

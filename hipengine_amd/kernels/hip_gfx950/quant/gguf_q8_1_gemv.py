@@ -399,6 +399,74 @@ def gguf_gemv_default_form(quant_key: str, rows: int, in_features: int, out_feat
     return GEMV_FORMS[form[0]], int(form[1])
 
 
+# hipEngine's per-shape tuning variants of the dense GEMV (gguf_k_gemv.py: rowbatch / coltile / wave32x2 / pipelined
+# forms for Q5_K, Q6_K and Q8_0): the dense launch under those names.  (quant, variant) -> wrapper.
+_DENSE_VARIANT_NAMES = (
+    *((q, f"gemv_rowbatch{rb}_bf16_{o}_out") for q in ("q5_k", "q6_k") for rb in (8, 32) for o in ("bf16", "f32")),
+    *((q, f"gemv_coltile{c}_rowbatch{r}_bf16_{o}_out") for q in ("q5_k", "q6_k") for c, r in ((2, 16), (4, 8))
+      for o in ("bf16", "f32")),
+    *(("q5_k", f"wave32x2{m}_gemv_decode_bf16_{o}_out") for m in ("", "_fixed_meta", "_swar_pair_fixed_meta")
+      for o in ("bf16", "f32")),
+    ("q6_k", "wave32x2_fixed_meta_gemv_decode_bf16_bf16_out"),
+    ("q6_k", "gemv_dpp_wave_reduction_coltile4_rowbatch8_bf16_bf16_out"),
+    ("q6_k", "gemv_dpp_wave_reduction_coltile2_rowbatch16_bf16_f32_out"),
+    ("q6_k", "gemv_dpp_wave_reduction_full_group_compute_coltile4_rowbatch8_bf16_bf16_out"),
+    ("q6_k", "gemv_dpp_wave_reduction_full_group_compute_coltile2_rowbatch16_bf16_f32_out"),
+    ("q8_0", "gemv_coltile4_rowbatch8_pipelined_f32_f32_out"),
+    ("q8_0", "gemv_coltile8_rowbatch4_pipelined_f32_f32_out"),
+    ("q8_0", "gemv_coltile8_rowbatch4_wave_scale_f32_f32_out"),
+    ("q8_0", "gemv_coltile8_rowbatch4_wave_scale_pipelined_f32_f32_out"),
+    ("q8_0", "gemv_coltile8_rowbatch4_wave_scale_pipelined_dpp_f32_f32_out"),
+    ("q8_0", "gemv_coltile8_rowbatch4_wave_scale_pipelined_dpp_checked_full_rows_f32_f32_out"),
+)
+
+
+def _make_dense_variant(quant: str, variant: str):
+    symbol = f"hipengine_gguf_{quant}_{variant}"
+
+    def wrapper(x_ptr: int, qweight_ptr: int, out_ptr: int, rows: int, in_features: int, out_features: int, *,
+                threads: int = 128, stream: int = 0, library: ctypes.CDLL | None = None,
+                runtime: HipRuntime | None = None) -> None:
+        validate_linear(rows, in_features, out_features, threads)
+        validate_pointers(x_ptr=x_ptr, qweight_ptr=qweight_ptr, out_ptr=out_ptr)
+        check_launch(entry(symbol, _FUSED_ARGS, library)(x_ptr, qweight_ptr, out_ptr, rows, in_features, out_features,
+                                                         threads, stream), runtime)
+
+    wrapper.__name__ = f"gguf_{quant}_{variant}"
+    wrapper.__doc__ = f"hipEngine's tuning variant ``{symbol}``: the dense GEMV launch (any shape)."
+    return wrapper
+
+
+DENSE_VARIANTS = {(q, v): _make_dense_variant(q, v) for q, v in _DENSE_VARIANT_NAMES}
+_PAIR_ARGS = [VOID, VOID, VOID, VOID, VOID, I64, I64, I64, I64, I64, VOID]
+
+
+def _make_q5_k_pair(variant: str):
+    symbol = f"hipengine_gguf_q5_k_{variant}"
+
+    def wrapper(x_ptr: int, qweight_a_ptr: int, qweight_b_ptr: int, out_a_ptr: int, out_b_ptr: int, rows: int,
+                in_features: int, out_features_a: int, out_features_b: int, *, threads: int = 128, stream: int = 0,
+                library: ctypes.CDLL | None = None, runtime: HipRuntime | None = None) -> None:
+        validate_linear(rows, in_features, out_features_a, threads)
+        validate_linear(rows, in_features, out_features_b, threads)
+        validate_pointers(x_ptr=x_ptr, qweight_a_ptr=qweight_a_ptr, qweight_b_ptr=qweight_b_ptr, out_a_ptr=out_a_ptr,
+                          out_b_ptr=out_b_ptr)
+        check_launch(entry(symbol, _PAIR_ARGS, library)(x_ptr, qweight_a_ptr, qweight_b_ptr, out_a_ptr, out_b_ptr, rows,
+                                                        in_features, out_features_a, out_features_b, threads, stream),
+                     runtime)
+
+    wrapper.__name__ = f"gguf_q5_k_{variant}"
+    wrapper.__doc__ = (f"hipEngine's Q5_K pair decode ``{symbol}``: two matrices of different heights over one bf16 "
+                       "activation, one multi-matrix launch.")
+    return wrapper
+
+
+Q5_K_PAIR = {v: _make_q5_k_pair(v) for v in (
+    "pair_wave32x2_gemv_decode_bf16_f32_out", "pair_wave32x2_fixed_meta_gemv_decode_bf16_bf16_out",
+    "pair_wave32x2_fixed_meta_gemv_decode_bf16_f32_out", "pair_wave32x2_swar_pair_fixed_meta_gemv_decode_bf16_bf16_out",
+    "pair_wave32x2_swar_pair_fixed_meta_gemv_decode_bf16_f32_out")}
+
+
 def register_kernels(backend: str = "hip_gfx950", *, replace: bool = False) -> None:
     # the keys hipEngine's dispatcher resolves for raw-layout weights: gemv_* at one row, prefill_* above
     # (loading/qwen35_gguf_consumer_surface.py:134-144,527-530)
@@ -410,6 +478,10 @@ def register_kernels(backend: str = "hip_gfx950", *, replace: bool = False) -> N
     for (act, out), fn in PAIR_SILU.items():
         register(KernelKey(backend, "linear", "gguf_q4_k", f"dual_silu_gemv_{act}_{out}_out"), fn, replace=replace)
     register(KernelKey(backend, "linear", "gguf", "multi_gemv"), gguf_multi_gemv, replace=replace)
+    for (quant, variant), fn in DENSE_VARIANTS.items():
+        register(KernelKey(backend, "linear", f"gguf_{quant}", variant), fn, replace=replace)
+    for variant, fn in Q5_K_PAIR.items():
+        register(KernelKey(backend, "linear", "gguf_q5_k", variant), fn, replace=replace)
     for (quant, act, out), fn in RESIDUAL.items():
         register(KernelKey(backend, "linear", f"gguf_{quant}", f"gemv_{act}_residual_{out}_out"), fn, replace=replace)
     for (quant, act, out), fn in FUSED.items():

@@ -169,6 +169,48 @@ HIPENGINE_GFX950_DECLARE_DENSE_ALL(q5_k)
 HIPENGINE_GFX950_DECLARE_DENSE_ALL(q6_k)
 HIPENGINE_GFX950_DECLARE_DENSE_ALL(q8_0)
 
+/* hipEngine's per-shape tuning variants of the dense GEMV for Q5_K / Q6_K / Q8_0 (row batches, column tiles, wave
+ * layouts, pipelining; gguf_k_gemv.hip:5665-5702, 5823-5960, 6161-6255): the same 8 arguments and product as the
+ * dense names above and the same launch here, for any shape (hipEngine restricts some to the shapes they were tuned
+ * for).  The pair names take two Q5_K matrices of different heights over one bf16 activation. */
+#define HIPENGINE_GFX950_DECLARE_DENSE_VARIANT(name)                                                     \
+  int name(const void* x, const uint8_t* qweight, void* out, int64_t rows, int64_t in_features,          \
+           int64_t out_features, int64_t threads, hipengine_stream_t stream);
+#define HIPENGINE_GFX950_DECLARE_DENSE_VARIANT_BF16(prefix)        \
+  HIPENGINE_GFX950_DECLARE_DENSE_VARIANT(prefix##_bf16_bf16_out)   \
+  HIPENGINE_GFX950_DECLARE_DENSE_VARIANT(prefix##_bf16_f32_out)
+HIPENGINE_GFX950_DECLARE_DENSE_VARIANT_BF16(hipengine_gguf_q5_k_gemv_rowbatch8)
+HIPENGINE_GFX950_DECLARE_DENSE_VARIANT_BF16(hipengine_gguf_q5_k_gemv_rowbatch32)
+HIPENGINE_GFX950_DECLARE_DENSE_VARIANT_BF16(hipengine_gguf_q6_k_gemv_rowbatch8)
+HIPENGINE_GFX950_DECLARE_DENSE_VARIANT_BF16(hipengine_gguf_q6_k_gemv_rowbatch32)
+HIPENGINE_GFX950_DECLARE_DENSE_VARIANT_BF16(hipengine_gguf_q5_k_gemv_coltile2_rowbatch16)
+HIPENGINE_GFX950_DECLARE_DENSE_VARIANT_BF16(hipengine_gguf_q5_k_gemv_coltile4_rowbatch8)
+HIPENGINE_GFX950_DECLARE_DENSE_VARIANT_BF16(hipengine_gguf_q6_k_gemv_coltile2_rowbatch16)
+HIPENGINE_GFX950_DECLARE_DENSE_VARIANT_BF16(hipengine_gguf_q6_k_gemv_coltile4_rowbatch8)
+HIPENGINE_GFX950_DECLARE_DENSE_VARIANT_BF16(hipengine_gguf_q5_k_wave32x2_gemv_decode)
+HIPENGINE_GFX950_DECLARE_DENSE_VARIANT_BF16(hipengine_gguf_q5_k_wave32x2_fixed_meta_gemv_decode)
+HIPENGINE_GFX950_DECLARE_DENSE_VARIANT_BF16(hipengine_gguf_q5_k_wave32x2_swar_pair_fixed_meta_gemv_decode)
+HIPENGINE_GFX950_DECLARE_DENSE_VARIANT(hipengine_gguf_q6_k_wave32x2_fixed_meta_gemv_decode_bf16_bf16_out)
+HIPENGINE_GFX950_DECLARE_DENSE_VARIANT(hipengine_gguf_q6_k_gemv_dpp_wave_reduction_coltile4_rowbatch8_bf16_bf16_out)
+HIPENGINE_GFX950_DECLARE_DENSE_VARIANT(hipengine_gguf_q6_k_gemv_dpp_wave_reduction_coltile2_rowbatch16_bf16_f32_out)
+HIPENGINE_GFX950_DECLARE_DENSE_VARIANT(hipengine_gguf_q6_k_gemv_dpp_wave_reduction_full_group_compute_coltile4_rowbatch8_bf16_bf16_out)
+HIPENGINE_GFX950_DECLARE_DENSE_VARIANT(hipengine_gguf_q6_k_gemv_dpp_wave_reduction_full_group_compute_coltile2_rowbatch16_bf16_f32_out)
+HIPENGINE_GFX950_DECLARE_DENSE_VARIANT(hipengine_gguf_q8_0_gemv_coltile4_rowbatch8_pipelined_f32_f32_out)
+HIPENGINE_GFX950_DECLARE_DENSE_VARIANT(hipengine_gguf_q8_0_gemv_coltile8_rowbatch4_pipelined_f32_f32_out)
+HIPENGINE_GFX950_DECLARE_DENSE_VARIANT(hipengine_gguf_q8_0_gemv_coltile8_rowbatch4_wave_scale_f32_f32_out)
+HIPENGINE_GFX950_DECLARE_DENSE_VARIANT(hipengine_gguf_q8_0_gemv_coltile8_rowbatch4_wave_scale_pipelined_f32_f32_out)
+HIPENGINE_GFX950_DECLARE_DENSE_VARIANT(hipengine_gguf_q8_0_gemv_coltile8_rowbatch4_wave_scale_pipelined_dpp_f32_f32_out)
+HIPENGINE_GFX950_DECLARE_DENSE_VARIANT(hipengine_gguf_q8_0_gemv_coltile8_rowbatch4_wave_scale_pipelined_dpp_checked_full_rows_f32_f32_out)
+#define HIPENGINE_GFX950_DECLARE_Q5_K_PAIR(name)                                                          \
+  int name(const void* x, const uint8_t* qweight_a, const uint8_t* qweight_b, void* out_a, void* out_b, int64_t rows, \
+           int64_t in_features, int64_t out_features_a, int64_t out_features_b, int64_t threads,           \
+           hipengine_stream_t stream);
+HIPENGINE_GFX950_DECLARE_Q5_K_PAIR(hipengine_gguf_q5_k_pair_wave32x2_gemv_decode_bf16_f32_out)
+HIPENGINE_GFX950_DECLARE_Q5_K_PAIR(hipengine_gguf_q5_k_pair_wave32x2_fixed_meta_gemv_decode_bf16_bf16_out)
+HIPENGINE_GFX950_DECLARE_Q5_K_PAIR(hipengine_gguf_q5_k_pair_wave32x2_fixed_meta_gemv_decode_bf16_f32_out)
+HIPENGINE_GFX950_DECLARE_Q5_K_PAIR(hipengine_gguf_q5_k_pair_wave32x2_swar_pair_fixed_meta_gemv_decode_bf16_bf16_out)
+HIPENGINE_GFX950_DECLARE_Q5_K_PAIR(hipengine_gguf_q5_k_pair_wave32x2_swar_pair_fixed_meta_gemv_decode_bf16_f32_out)
+
 /* Pre-quantized: xq is [rows, in_features/32] 36-byte q8_1 blocks.
  * Q4_K replaces gguf_q4_k_q8_1_dp4a_vdr_gemv.hip:321-361 (without its
  * out_features % 8 restriction); Q8_0 replaces gguf_q8_0_dp4a_gemv.hip:345-388;

@@ -498,3 +498,44 @@ def test_mmq_int32_dots_bit_exact(dev, quant, rows, k, n):
     dev.free(dxq, dw, ddots, dout)
     assert np.array_equal(got, want.astype(np.int32))
     _close(out, ref)
+
+
+def test_dense_tuning_variant_names_are_the_dense_launch(dev):
+    """hipEngine's per-shape variant names of the Q5_K / Q6_K / Q8_0 GEMV: the bits of the dense entry of the same
+    types, at a shape none of them was tuned for; the Q5_K pair names against two single launches."""
+    rows, k, n = 3, 1024, 200
+    rng = np.random.default_rng(5)
+    x = (rng.standard_normal((rows, k)) * 0.4).astype(np.float32)
+    weights = {"q5_k": synthetic_blocks(O.GGML_Q5_K, n, k, seed=2, tile_rows=n), "q6_k": O.random_weight(O.GGML_Q6_K, n, k, seed=2),
+               "q8_0": O.random_weight(O.GGML_Q8_0, n, k, seed=2)}
+    dw = {q: dev.put(w) for q, w in weights.items()}
+    dx = {"f32": dev.put(x), "bf16": dev.put(O.f32_to_bf16_bits(x))}
+    base = {}
+    for (quant, variant), fn in G.DENSE_VARIANTS.items():
+        act, out = variant.split("_")[-3], variant.split("_")[-2]
+        item = 4 if out == "f32" else 2
+        key = (quant, act, out)
+        if key not in base:
+            dout = dev.empty(rows * n * item)
+            G.DENSE[(quant, "gemv", act, out)](dx[act].ptr, dw[quant].ptr, dout.ptr, rows, k, n)
+            base[key] = dev.get(dout, np.uint8, (rows * n * item,)).copy()
+            dev.free(dout)
+        dout = dev.empty(rows * n * item, fill=0x3C)
+        fn(dx[act].ptr, dw[quant].ptr, dout.ptr, rows, k, n)
+        assert np.array_equal(dev.get(dout, np.uint8, (rows * n * item,)), base[key]), variant
+        dev.free(dout)
+    nb = 72
+    wb = synthetic_blocks(O.GGML_Q5_K, nb, k, seed=9, tile_rows=nb)
+    dwb = dev.put(wb)
+    for variant, fn in G.Q5_K_PAIR.items():
+        out = variant.split("_")[-2]
+        item = 4 if out == "f32" else 2
+        da, db, sa, sb = (dev.empty(rows * m * item, fill=0x3C) for m in (n, nb, n, nb))
+        fn(dx["bf16"].ptr, dw["q5_k"].ptr, dwb.ptr, da.ptr, db.ptr, rows, k, n, nb)
+        single = G.DENSE[("q5_k", "gemv", "bf16", out)]
+        single(dx["bf16"].ptr, dw["q5_k"].ptr, sa.ptr, rows, k, n)
+        single(dx["bf16"].ptr, dwb.ptr, sb.ptr, rows, k, nb)
+        assert np.array_equal(dev.get(da, np.uint8, (rows * n * item,)), dev.get(sa, np.uint8, (rows * n * item,))), variant
+        assert np.array_equal(dev.get(db, np.uint8, (rows * nb * item,)), dev.get(sb, np.uint8, (rows * nb * item,))), variant
+        dev.free(da, db, sa, sb)
+    dev.free(dwb, *dw.values(), *dx.values())
