@@ -1341,6 +1341,99 @@ int launch_moe_tail(const uint16_t* selected, const float* routing, const int64_
   return static_cast<int>(hipGetLastError());
 }
 
+// ---- router logits: logits[t, e] = hidden[t, :] . weight[e, :] in float32 (moe/router.hip:36-80) --------
+//
+// An unquantized product in front of the selection: hidden rows in float32, bf16 or fp16, weight rows in float32
+// or in the 16-bit type of the hidden rows.  A wave owns 8 tokens x 4 weight rows; a lane walks K in pieces of 8
+// values (16- and 32-byte loads), so a weight row is read once per 8 tokens and a hidden row once per 4 weight rows.
+// Lanes are summed by a butterfly, the order of which differs from hipEngine's shared-memory tree: logits agree to
+// float32 rounding, not bit for bit.
+constexpr int RL_TOKENS = 8, RL_ROWS = 4, RL_WAVES = 4;
+
+template <int KIND>
+__device__ __forceinline__ void load8_as_float(const void* base, int64_t index, float (&v)[8]) {
+  if constexpr (KIND == KIND_F32) {
+    const float4 lo = *reinterpret_cast<const float4*>(static_cast<const float*>(base) + index);
+    const float4 hi = *reinterpret_cast<const float4*>(static_cast<const float*>(base) + index + 4);
+    v[0] = lo.x; v[1] = lo.y; v[2] = lo.z; v[3] = lo.w; v[4] = hi.x; v[5] = hi.y; v[6] = hi.z; v[7] = hi.w;
+  } else {
+    const uint4 p = *reinterpret_cast<const uint4*>(static_cast<const uint16_t*>(base) + index);
+    const uint32_t w[4] = {p.x, p.y, p.z, p.w};
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+      v[2 * e] = KIND == KIND_BF16 ? bf16_bits_to_float(w[e] & 0xFFFFu) : f16_bits_to_float(w[e] & 0xFFFFu);
+      v[2 * e + 1] = KIND == KIND_BF16 ? bf16_bits_to_float(w[e] >> 16) : f16_bits_to_float(w[e] >> 16);
+    }
+  }
+}
+
+template <int HK, int WK>
+__global__ void __launch_bounds__(64 * RL_WAVES) router_logits_kernel(const void* __restrict__ hidden,
+                                                                      const void* __restrict__ weight,
+                                                                      float* __restrict__ logits, int64_t tokens,
+                                                                      int64_t hidden_size, int64_t num_rows) {
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int64_t row0 = (static_cast<int64_t>(blockIdx.x) * RL_WAVES + wave) * RL_ROWS;
+  const int64_t tok0 = static_cast<int64_t>(blockIdx.y) * RL_TOKENS;
+  if (row0 >= num_rows) return;     // whole waves leave; no workgroup barrier below
+  float acc[RL_TOKENS][RL_ROWS];
+#pragma unroll
+  for (int t = 0; t < RL_TOKENS; ++t)
+#pragma unroll
+    for (int r = 0; r < RL_ROWS; ++r) acc[t][r] = 0.0f;
+  const int64_t whole = hidden_size & ~static_cast<int64_t>(7);
+  for (int64_t k = static_cast<int64_t>(lane) * 8; k < whole; k += 64 * 8) {
+    float h[RL_TOKENS][8];
+#pragma unroll
+    for (int t = 0; t < RL_TOKENS; ++t) load8_as_float<HK>(hidden, min(tok0 + t, tokens - 1) * hidden_size + k, h[t]);
+#pragma unroll
+    for (int r = 0; r < RL_ROWS; ++r) {
+      float w[8];
+      load8_as_float<WK>(weight, min(row0 + r, num_rows - 1) * hidden_size + k, w);
+#pragma unroll
+      for (int t = 0; t < RL_TOKENS; ++t)
+#pragma unroll
+        for (int e = 0; e < 8; ++e) acc[t][r] = __builtin_fmaf(h[t][e], w[e], acc[t][r]);
+    }
+  }
+  for (int64_t k = whole + lane; k < hidden_size; k += 64) {     // a row length that is not a multiple of 8
+#pragma unroll
+    for (int r = 0; r < RL_ROWS; ++r) {
+      const float w = load_scalar(weight, min(row0 + r, num_rows - 1) * hidden_size + k, WK);
+#pragma unroll
+      for (int t = 0; t < RL_TOKENS; ++t)
+        acc[t][r] = __builtin_fmaf(load_scalar(hidden, min(tok0 + t, tokens - 1) * hidden_size + k, HK), w, acc[t][r]);
+    }
+  }
+#pragma unroll
+  for (int t = 0; t < RL_TOKENS; ++t)
+#pragma unroll
+    for (int r = 0; r < RL_ROWS; ++r) {
+      float v = acc[t][r];
+#pragma unroll
+      for (int off = 32; off > 0; off >>= 1) v += __shfl_xor(v, off);
+      if (lane == 0 && tok0 + t < tokens && row0 + r < num_rows) logits[(tok0 + t) * num_rows + row0 + r] = v;
+    }
+}
+
+template <int HK, int WK>
+int launch_router_logits(const void* hidden, const void* weight, float* logits, int64_t tokens, int64_t hidden_size,
+                         int64_t num_rows, int64_t threads, hipStream_t stream) {
+  const int64_t h_item = HK == KIND_F32 ? 4 : 2, w_item = WK == KIND_F32 ? 4 : 2;
+  if (!hidden || !weight || !logits || tokens <= 0 || tokens > (1 << 24) || hidden_size <= 0 || num_rows <= 0 ||
+      num_rows > (1 << 24) || !(threads == 64 || threads == 128 || threads == 256 || threads == 512) ||
+      // the 16- and 32-byte loads: rows of 8-value pieces must start on their natural alignment
+      (hidden_size >= 8 && (((hidden_size * h_item) % 16) != 0 || ((hidden_size * w_item) % 16) != 0 ||
+                            (reinterpret_cast<uintptr_t>(hidden) & 15u) != 0 || (reinterpret_cast<uintptr_t>(weight) & 15u) != 0))) {
+    return static_cast<int>(hipErrorInvalidValue);
+  }
+  const dim3 grid(static_cast<unsigned>((num_rows + RL_WAVES * RL_ROWS - 1) / (RL_WAVES * RL_ROWS)),
+                  static_cast<unsigned>((tokens + RL_TOKENS - 1) / RL_TOKENS));
+  hipLaunchKernelGGL((router_logits_kernel<HK, WK>), grid, dim3(64 * RL_WAVES), 0, stream, hidden, weight, logits, tokens,
+                     hidden_size, num_rows);
+  return static_cast<int>(hipGetLastError());
+}
+
 // ---- router: top-k experts of a row of logits and the softmax of their logits --------
 //
 // One wave per token.  Lane l keeps the logits of experts l, l+64, ... (up to 16 of them,
@@ -1858,6 +1951,18 @@ extern "C" int hipengine_gfx950_moe_tile_map(const int64_t* expert_start_compact
   return launch_tile_map(expert_start_compact, tile_expert_start, tile_expert, total_out, num_experts, tile_capacity,
                          tile_rows, stream);
 }
+
+// Router logits in front of the selection; `threads` is accepted and ignored.
+#define DEFINE_ROUTER_LOGITS(SYMBOL, HK, WK)                                                                    \
+  extern "C" int SYMBOL(const void* hidden, const void* weight, float* logits, int64_t tokens, int64_t hidden_size, \
+                        int64_t num_rows, int64_t threads, hipStream_t stream) {                                 \
+    return launch_router_logits<HK, WK>(hidden, weight, logits, tokens, hidden_size, num_rows, threads, stream);  \
+  }
+DEFINE_ROUTER_LOGITS(hipengine_qwen35_router_logits_bf16, KIND_BF16, KIND_BF16)
+DEFINE_ROUTER_LOGITS(hipengine_qwen35_router_logits_fp16, KIND_F16, KIND_F16)
+DEFINE_ROUTER_LOGITS(hipengine_qwen35_router_logits_bf16_f32w, KIND_BF16, KIND_F32)
+DEFINE_ROUTER_LOGITS(hipengine_qwen35_router_logits_fp16_f32w, KIND_F16, KIND_F32)
+DEFINE_ROUTER_LOGITS(hipengine_qwen35_router_logits_f32_f32w, KIND_F32, KIND_F32)
 
 extern "C" int hipengine_qwen35_router_select(const float* logits, int64_t* selected, float* routing, int64_t tokens,
                                               int64_t logits_stride, int64_t num_experts, int64_t top_k,

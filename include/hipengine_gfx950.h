@@ -462,6 +462,28 @@ int hipengine_gfx950_argmax_f32_rows_i32_noalloc(const float* logits, int32_t* o
                                                  int64_t rows, int64_t vocab_size, int64_t threads,
                                                  hipengine_stream_t stream);
 
+/* Router logits, the product in front of the selection: logits[t, e] = hidden[t, :] . weight[e, :] accumulated in
+ * float32 (moe/router.hip:36-80, entries :960-1037,1140-1160,1250-1275).  hidden [tokens, hidden_size] in bf16, fp16 or
+ * float32; weight [num_rows, hidden_size] in the same 16-bit type or in float32 (`_f32w`); logits float32
+ * [tokens, num_rows].  Rows of 8 values or more must be 16-byte aligned (hidden_size * element size a multiple of
+ * 16).  `threads` (64, 128, 256 or 512) is accepted and ignored.  Sums are taken in another order than hipEngine's
+ * shared-memory tree: equal to float32 rounding. */
+int hipengine_qwen35_router_logits_bf16(const void* hidden, const void* weight, float* logits, int64_t tokens,
+                                        int64_t hidden_size, int64_t num_rows, int64_t threads,
+                                        hipengine_stream_t stream);
+int hipengine_qwen35_router_logits_fp16(const void* hidden, const void* weight, float* logits, int64_t tokens,
+                                        int64_t hidden_size, int64_t num_rows, int64_t threads,
+                                        hipengine_stream_t stream);
+int hipengine_qwen35_router_logits_bf16_f32w(const void* hidden, const void* weight, float* logits, int64_t tokens,
+                                             int64_t hidden_size, int64_t num_rows, int64_t threads,
+                                             hipengine_stream_t stream);
+int hipengine_qwen35_router_logits_fp16_f32w(const void* hidden, const void* weight, float* logits, int64_t tokens,
+                                             int64_t hidden_size, int64_t num_rows, int64_t threads,
+                                             hipengine_stream_t stream);
+int hipengine_qwen35_router_logits_f32_f32w(const void* hidden, const void* weight, float* logits, int64_t tokens,
+                                            int64_t hidden_size, int64_t num_rows, int64_t threads,
+                                            hipengine_stream_t stream);
+
 /* Router: for each of `tokens` rows of float32 logits (row pitch logits_stride), the top_k
  * experts by logit, highest first (equal logits: lowest index), as int64 into
  * selected[tokens*top_k], and the softmax over those top_k logits into

@@ -50,6 +50,7 @@ mmq_q8_0_d4s4                float64 product of the dequantized weight and activ
 gemv_q8_1_* / mmq_*          float64 evaluation of the same formula
                              (tests/test_gpu_gguf_q4_k_q8_1_mmq_prefill.py
                              :115-165 style)
+router_logits                float64 matmul (a float32 matmul by definition)
 router_topk_softmax          brute-force argsort; ties -> lowest index
 mtp_moe_routing              closed form on tiny cases
 build_routing_index          invariants (prefix sums, permutation, stability,
@@ -733,6 +734,12 @@ def mmq_q6_k_d4s4(xd4s4, qweight, dtype=np.float64) -> np.ndarray:
 # --------------------------------------------------------------------------
 # routing
 # --------------------------------------------------------------------------
+
+def router_logits(hidden, weight) -> np.ndarray:
+    """``logits[t, e] = hidden[t] . weight[e]`` as a float32 matmul of float32 values
+    (kernels/cpu_reference/ops.py:609, the first step of the routing reference)."""
+    return np.matmul(np.asarray(hidden, dtype=np.float32), np.asarray(weight, dtype=np.float32).T).astype(np.float32)
+
 
 def router_topk_softmax(logits, top_k: int) -> tuple[np.ndarray, np.ndarray]:
     """Device router (moe/router.hip:628-715): iterative argmax on the logits

@@ -152,6 +152,48 @@ def test_routing_index_other_entry_names(dev, tokens, top_k, experts, bad):
     dev.free(dsel, dsel32, dw, counts, offsets)
 
 
+@pytest.mark.parametrize("tokens,hidden,rows", [(1, 2048, 256), (9, 2048, 257), (130, 512, 60), (3, 20, 5)])
+@pytest.mark.parametrize("name,hk,wk", [("bf16", "bf16", "bf16"), ("fp16", "fp16", "fp16"), ("bf16_f32w", "bf16", "f32"),
+                                        ("fp16_f32w", "fp16", "f32"), ("f32_f32w", "f32", "f32")])
+def test_router_logits(dev, name, hk, wk, tokens, hidden, rows):
+    """Router logits against the float32 matmul of the reference on the same (rounded) values: float32 rounding apart
+    (another summation order); then the selection of the device logits is the oracle's selection of those logits."""
+    if hidden % 8 and (hk != "f32" or wk != "f32") and (hidden * 2) % 16:
+        pytest.skip("16-bit rows shorter than their alignment")
+    rng = np.random.default_rng(tokens + hidden + rows)
+    x = (rng.standard_normal((tokens, hidden)) * 0.5).astype(np.float32)
+    w = (rng.standard_normal((rows, hidden)) * 0.05).astype(np.float32)
+
+    def encode(a, kind):
+        if kind == "bf16":
+            b = O.f32_to_bf16_bits(a)
+            return b, O.bf16_bits_to_f32(b)
+        if kind == "fp16":
+            h = a.astype(np.float16)
+            return h.view(np.uint16), h.astype(np.float32)
+        return a, a
+
+    xb, xf = encode(x, hk)
+    wb, wf = encode(w, wk)
+    dx, dw, dl = dev.put(xb), dev.put(wb), dev.empty(tokens * rows * 4, fill=0x7C)
+    getattr(RT, f"qwen35_router_logits_{name}")(dx.ptr, dw.ptr, dl.ptr, tokens, hidden, rows)
+    got = dev.get(dl, np.float32, (tokens, rows)).copy()
+    want = O.router_logits(xf, wf)
+    exact = xf.astype(np.float64) @ wf.astype(np.float64).T
+    scale = np.abs(xf).astype(np.float64) @ np.abs(wf).astype(np.float64).T
+    assert np.all(np.abs(got - exact) <= scale * 2.0 ** -20 + 1e-30)          # float32 accumulation of `hidden` terms
+    assert np.all(np.abs(want - exact) <= scale * 2.0 ** -20 + 1e-30)
+    if rows >= 8:
+        top_k = 8
+        dsel, dr = dev.empty(tokens * top_k * 8), dev.empty(tokens * top_k * 4)
+        RT.qwen35_router_select(dl.ptr, dsel.ptr, dr.ptr, tokens, rows, rows, top_k)
+        sel = dev.get(dsel, np.int64, (tokens, top_k))
+        want_sel, _ = O.router_topk_softmax(got, top_k)
+        assert np.array_equal(sel, want_sel)
+        dev.free(dsel, dr)
+    dev.free(dx, dw, dl)
+
+
 @pytest.mark.parametrize("tokens,experts,top_k,stride", [(1, 256, 8, 256), (7, 256, 8, 257), (33, 60, 4, 64),
                                                         (5, 1024, 16, 1024), (3, 8, 8, 8), (2048, 256, 8, 256)])
 def test_router_select(dev, tokens, experts, top_k, stride):
