@@ -1416,6 +1416,136 @@ __global__ void __launch_bounds__(64 * RL_WAVES) router_logits_kernel(const void
     }
 }
 
+// Decode batches (tokens <= 8): the four waves of a workgroup split K instead of the rows, so that a row of 2048 values
+// is one 8-value piece per lane with every load of the workgroup in flight at once (the kernel above walks K in a
+// loop of dependent round trips: 13.8 us at one token against the few microseconds of a 2 MB read).  TT tokens x
+// RL_ROWS weight rows per workgroup; partial sums of the waves meet in LDS.
+template <int HK, int WK, int TT>
+__global__ void __launch_bounds__(64 * RL_WAVES) router_logits_decode_kernel(const void* __restrict__ hidden,
+                                                                             const void* __restrict__ weight,
+                                                                             float* __restrict__ logits, int64_t tokens,
+                                                                             int64_t hidden_size, int64_t num_rows) {
+  __shared__ float part[RL_WAVES][TT][RL_ROWS];
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int64_t row0 = static_cast<int64_t>(blockIdx.x) * RL_ROWS;
+  float acc[TT][RL_ROWS];
+#pragma unroll
+  for (int t = 0; t < TT; ++t)
+#pragma unroll
+    for (int r = 0; r < RL_ROWS; ++r) acc[t][r] = 0.0f;
+  const int64_t whole = hidden_size & ~static_cast<int64_t>(7);
+  for (int64_t k = (static_cast<int64_t>(wave) * 64 + lane) * 8; k < whole; k += 64 * RL_WAVES * 8) {
+    float h[TT][8];
+#pragma unroll
+    for (int t = 0; t < TT; ++t) load8_as_float<HK>(hidden, min(static_cast<int64_t>(t), tokens - 1) * hidden_size + k, h[t]);
+#pragma unroll
+    for (int r = 0; r < RL_ROWS; ++r) {
+      float w[8];
+      load8_as_float<WK>(weight, min(row0 + r, num_rows - 1) * hidden_size + k, w);
+#pragma unroll
+      for (int t = 0; t < TT; ++t)
+#pragma unroll
+        for (int e = 0; e < 8; ++e) acc[t][r] = __builtin_fmaf(h[t][e], w[e], acc[t][r]);
+    }
+  }
+  for (int64_t k = whole + wave * 64 + lane; k < hidden_size; k += 64 * RL_WAVES) {
+#pragma unroll
+    for (int r = 0; r < RL_ROWS; ++r) {
+      const float w = load_scalar(weight, min(row0 + r, num_rows - 1) * hidden_size + k, WK);
+#pragma unroll
+      for (int t = 0; t < TT; ++t)
+        acc[t][r] = __builtin_fmaf(load_scalar(hidden, min(static_cast<int64_t>(t), tokens - 1) * hidden_size + k, HK), w,
+                                   acc[t][r]);
+    }
+  }
+#pragma unroll
+  for (int t = 0; t < TT; ++t)
+#pragma unroll
+    for (int r = 0; r < RL_ROWS; ++r) {
+      float v = acc[t][r];
+#pragma unroll
+      for (int off = 32; off > 0; off >>= 1) v += __shfl_xor(v, off);
+      if (lane == 0) part[wave][t][r] = v;
+    }
+  __syncthreads();
+  if (threadIdx.x < TT * RL_ROWS) {
+    const int t = threadIdx.x / RL_ROWS, r = threadIdx.x % RL_ROWS;
+    if (t < tokens && row0 + r < num_rows)
+      logits[static_cast<int64_t>(t) * num_rows + row0 + r] = (part[0][t][r] + part[1][t][r]) + (part[2][t][r] + part[3][t][r]);
+  }
+}
+
+// Prefill batches with bf16 hidden rows: the product on the bf16 MFMA (v_mfma_f32_32x32x16_bf16).  A float32 weight is
+// split into three bf16 parts that add up to it exactly (8 + 8 + 8 significant bits, each the truncation of what the
+// parts before it leave), and the hidden values are bf16 already, so every product is exact in float32 and the sums
+// have float32 accuracy: three MFMAs per 16 values instead of 16 x 32 x 32 FMAs (the kernel further up takes 73 us
+// for 2048 tokens x 256 rows x 2048, most of it float32 FMAs and conversions).  A workgroup owns 32 tokens x 32
+// rows; its four waves take a quarter of K each and meet in LDS.  Operands go from global memory straight into
+// registers: lane (n = l % 32, g = l / 32) holds values 8g..8g+7 of the 16 of row n, on both sides alike.
+typedef __bf16 rl_v8bf __attribute__((ext_vector_type(8)));
+typedef float rl_v16f __attribute__((ext_vector_type(16)));
+
+template <int WK>
+__global__ void __launch_bounds__(256) router_logits_mfma_kernel(const uint16_t* __restrict__ hidden,
+                                                                 const void* __restrict__ weight,
+                                                                 float* __restrict__ logits, int64_t tokens,
+                                                                 int64_t hidden_size, int64_t num_rows) {
+  __shared__ float part[4][16][64];
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int n = lane & 31, g = lane >> 5;
+  const int64_t row0 = static_cast<int64_t>(blockIdx.x) * 32, tok0 = static_cast<int64_t>(blockIdx.y) * 32;
+  const int64_t k_per_wave = hidden_size / 4;                       // a multiple of 16
+  const uint16_t* hrow = hidden + min(tok0 + n, tokens - 1) * hidden_size + wave * k_per_wave + 8 * g;
+  const int64_t wbase = min(row0 + n, num_rows - 1) * hidden_size + wave * k_per_wave + 8 * g;
+  // one accumulator per weight part: three independent MFMA chains instead of one of three times the length
+  rl_v16f acc, acc_mid, acc_lo;
+#pragma unroll
+  for (int v = 0; v < 16; ++v) { acc[v] = 0.0f; acc_mid[v] = 0.0f; acc_lo[v] = 0.0f; }
+#pragma unroll 4
+  for (int64_t k = 0; k < k_per_wave; k += 16) {
+    const uint4 hx = *reinterpret_cast<const uint4*>(hrow + k);
+    const rl_v8bf a = __builtin_bit_cast(rl_v8bf, hx);
+    if constexpr (WK == KIND_F32) {
+      const float* wp = static_cast<const float*>(weight) + wbase + k;
+      const float4 w0 = *reinterpret_cast<const float4*>(wp), w1 = *reinterpret_cast<const float4*>(wp + 4);
+      const float w[8] = {w0.x, w0.y, w0.z, w0.w, w1.x, w1.y, w1.z, w1.w};
+      uint32_t hi[4], mid[4], lo[4];
+#pragma unroll
+      for (int e = 0; e < 4; ++e) {
+        uint32_t p[3][2];
+#pragma unroll
+        for (int h = 0; h < 2; ++h) {
+          const float x = w[2 * e + h];
+          const uint32_t b0 = float_to_bits(x) & 0xFFFF0000u;
+          const float r1 = x - bits_to_float(b0);
+          const uint32_t b1 = float_to_bits(r1) & 0xFFFF0000u;
+          const float r2 = r1 - bits_to_float(b1);
+          p[0][h] = b0; p[1][h] = b1; p[2][h] = float_to_bits(r2) & 0xFFFF0000u;
+        }
+        hi[e] = (p[0][0] >> 16) | p[0][1];
+        mid[e] = (p[1][0] >> 16) | p[1][1];
+        lo[e] = (p[2][0] >> 16) | p[2][1];
+      }
+      acc_lo = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, __builtin_bit_cast(rl_v8bf, make_uint4(lo[0], lo[1], lo[2], lo[3])), acc_lo, 0, 0, 0);
+      acc_mid = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, __builtin_bit_cast(rl_v8bf, make_uint4(mid[0], mid[1], mid[2], mid[3])), acc_mid, 0, 0, 0);
+      acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, __builtin_bit_cast(rl_v8bf, make_uint4(hi[0], hi[1], hi[2], hi[3])), acc, 0, 0, 0);
+    } else {
+      const uint4 wx = *reinterpret_cast<const uint4*>(static_cast<const uint16_t*>(weight) + wbase + k);
+      acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, __builtin_bit_cast(rl_v8bf, wx), acc, 0, 0, 0);
+    }
+  }
+#pragma unroll
+  for (int v = 0; v < 16; ++v) part[wave][v][lane] = acc[v] + (acc_mid[v] + acc_lo[v]);   // small parts first
+  __syncthreads();
+  // lane holds weight row n and tokens 8*(v/4) + 4*g + v%4 of the tile
+  for (int i = threadIdx.x; i < 16 * 64; i += 256) {
+    const int v = i >> 6, l = i & 63;
+    const int64_t tok = tok0 + 8 * (v >> 2) + 4 * (l >> 5) + (v & 3), row = row0 + (l & 31);
+    if (tok < tokens && row < num_rows)
+      logits[tok * num_rows + row] = (part[0][v][l] + part[1][v][l]) + (part[2][v][l] + part[3][v][l]);
+  }
+}
+
 template <int HK, int WK>
 int launch_router_logits(const void* hidden, const void* weight, float* logits, int64_t tokens, int64_t hidden_size,
                          int64_t num_rows, int64_t threads, hipStream_t stream) {
@@ -1426,6 +1556,28 @@ int launch_router_logits(const void* hidden, const void* weight, float* logits, 
       (hidden_size >= 8 && (((hidden_size * h_item) % 16) != 0 || ((hidden_size * w_item) % 16) != 0 ||
                             (reinterpret_cast<uintptr_t>(hidden) & 15u) != 0 || (reinterpret_cast<uintptr_t>(weight) & 15u) != 0))) {
     return static_cast<int>(hipErrorInvalidValue);
+  }
+  if (tokens <= 8) {
+    const dim3 dgrid(static_cast<unsigned>((num_rows + RL_ROWS - 1) / RL_ROWS));
+    if (tokens == 1) {
+      hipLaunchKernelGGL((router_logits_decode_kernel<HK, WK, 1>), dgrid, dim3(64 * RL_WAVES), 0, stream, hidden, weight,
+                         logits, tokens, hidden_size, num_rows);
+    } else if (tokens <= 4) {
+      hipLaunchKernelGGL((router_logits_decode_kernel<HK, WK, 4>), dgrid, dim3(64 * RL_WAVES), 0, stream, hidden, weight,
+                         logits, tokens, hidden_size, num_rows);
+    } else {
+      hipLaunchKernelGGL((router_logits_decode_kernel<HK, WK, 8>), dgrid, dim3(64 * RL_WAVES), 0, stream, hidden, weight,
+                         logits, tokens, hidden_size, num_rows);
+    }
+    return static_cast<int>(hipGetLastError());
+  }
+  if constexpr (HK == KIND_BF16 && (WK == KIND_F32 || WK == KIND_BF16)) {
+    if (tokens >= 32 && (hidden_size % 64) == 0) {
+      const dim3 mgrid(static_cast<unsigned>((num_rows + 31) / 32), static_cast<unsigned>((tokens + 31) / 32));
+      hipLaunchKernelGGL((router_logits_mfma_kernel<WK>), mgrid, dim3(256), 0, stream,
+                         static_cast<const uint16_t*>(hidden), weight, logits, tokens, hidden_size, num_rows);
+      return static_cast<int>(hipGetLastError());
+    }
   }
   const dim3 grid(static_cast<unsigned>((num_rows + RL_WAVES * RL_ROWS - 1) / (RL_WAVES * RL_ROWS)),
                   static_cast<unsigned>((tokens + RL_TOKENS - 1) / RL_TOKENS));

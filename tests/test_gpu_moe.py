@@ -152,7 +152,8 @@ def test_routing_index_other_entry_names(dev, tokens, top_k, experts, bad):
     dev.free(dsel, dsel32, dw, counts, offsets)
 
 
-@pytest.mark.parametrize("tokens,hidden,rows", [(1, 2048, 256), (9, 2048, 257), (130, 512, 60), (3, 20, 5)])
+@pytest.mark.parametrize("tokens,hidden,rows", [(1, 2048, 256), (9, 2048, 257), (130, 512, 60), (3, 20, 5), (7, 1024, 64),
+                                                (300, 2048, 256), (33, 192, 40), (64, 1000, 33)])
 @pytest.mark.parametrize("name,hk,wk", [("bf16", "bf16", "bf16"), ("fp16", "fp16", "fp16"), ("bf16_f32w", "bf16", "f32"),
                                         ("fp16_f32w", "fp16", "f32"), ("f32_f32w", "f32", "f32")])
 def test_router_logits(dev, name, hk, wk, tokens, hidden, rows):
