@@ -296,9 +296,12 @@ __device__ __forceinline__ void gemv_stage_activations(const GemvArgs& a, int kc
   const int nb = a.K / QK_K;
   const int blocks_here = min(chunk_blocks, nb - kc);
   const int groups = blocks_here * 8;
-#pragma unroll
-  for (int b = 0; b < B; ++b) {
-    for (int j = team; j < groups; j += nteams) {
+  // (batch row, group) pairs over all the teams at once: with few groups per row (a short K chunk and many rows)
+  // a loop over the rows outside would leave most teams idle and make the rows' loads a chain of round trips
+  {
+    for (int idx = team; idx < B * groups; idx += nteams) {
+      const int b = B == 1 ? 0 : idx / groups;
+      const int j = B == 1 ? idx : idx - b * groups;
       uint32_t packed = 0;
       float xd = 0.0f;
       if (b < a.rows) {
