@@ -1428,6 +1428,7 @@ __global__ void __launch_bounds__(64 * RL_WAVES) router_logits_decode_kernel(con
   __shared__ float part[RL_WAVES][TT][RL_ROWS];
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const int64_t row0 = static_cast<int64_t>(blockIdx.x) * RL_ROWS;
+  const int64_t tok0 = static_cast<int64_t>(blockIdx.y) * TT;
   float acc[TT][RL_ROWS];
 #pragma unroll
   for (int t = 0; t < TT; ++t)
@@ -1437,7 +1438,7 @@ __global__ void __launch_bounds__(64 * RL_WAVES) router_logits_decode_kernel(con
   for (int64_t k = (static_cast<int64_t>(wave) * 64 + lane) * 8; k < whole; k += 64 * RL_WAVES * 8) {
     float h[TT][8];
 #pragma unroll
-    for (int t = 0; t < TT; ++t) load8_as_float<HK>(hidden, min(static_cast<int64_t>(t), tokens - 1) * hidden_size + k, h[t]);
+    for (int t = 0; t < TT; ++t) load8_as_float<HK>(hidden, min(tok0 + t, tokens - 1) * hidden_size + k, h[t]);
 #pragma unroll
     for (int r = 0; r < RL_ROWS; ++r) {
       float w[8];
@@ -1454,7 +1455,7 @@ __global__ void __launch_bounds__(64 * RL_WAVES) router_logits_decode_kernel(con
       const float w = load_scalar(weight, min(row0 + r, num_rows - 1) * hidden_size + k, WK);
 #pragma unroll
       for (int t = 0; t < TT; ++t)
-        acc[t][r] = __builtin_fmaf(load_scalar(hidden, min(static_cast<int64_t>(t), tokens - 1) * hidden_size + k, HK), w,
+        acc[t][r] = __builtin_fmaf(load_scalar(hidden, min(tok0 + t, tokens - 1) * hidden_size + k, HK), w,
                                    acc[t][r]);
     }
   }
@@ -1470,8 +1471,8 @@ __global__ void __launch_bounds__(64 * RL_WAVES) router_logits_decode_kernel(con
   __syncthreads();
   if (threadIdx.x < TT * RL_ROWS) {
     const int t = threadIdx.x / RL_ROWS, r = threadIdx.x % RL_ROWS;
-    if (t < tokens && row0 + r < num_rows)
-      logits[static_cast<int64_t>(t) * num_rows + row0 + r] = (part[0][t][r] + part[1][t][r]) + (part[2][t][r] + part[3][t][r]);
+    if (tok0 + t < tokens && row0 + r < num_rows)
+      logits[(tok0 + t) * num_rows + row0 + r] = (part[0][t][r] + part[1][t][r]) + (part[2][t][r] + part[3][t][r]);
   }
 }
 
@@ -1558,15 +1559,13 @@ int launch_router_logits(const void* hidden, const void* weight, float* logits, 
     return static_cast<int>(hipErrorInvalidValue);
   }
   if (tokens <= 8) {
-    const dim3 dgrid(static_cast<unsigned>((num_rows + RL_ROWS - 1) / RL_ROWS));
+    // one token, or groups of four tokens (eight tokens as one group measured 9.7 us against the 3 us of one token)
+    const dim3 dgrid(static_cast<unsigned>((num_rows + RL_ROWS - 1) / RL_ROWS), tokens <= 4 ? 1u : 2u);
     if (tokens == 1) {
       hipLaunchKernelGGL((router_logits_decode_kernel<HK, WK, 1>), dgrid, dim3(64 * RL_WAVES), 0, stream, hidden, weight,
                          logits, tokens, hidden_size, num_rows);
-    } else if (tokens <= 4) {
-      hipLaunchKernelGGL((router_logits_decode_kernel<HK, WK, 4>), dgrid, dim3(64 * RL_WAVES), 0, stream, hidden, weight,
-                         logits, tokens, hidden_size, num_rows);
     } else {
-      hipLaunchKernelGGL((router_logits_decode_kernel<HK, WK, 8>), dgrid, dim3(64 * RL_WAVES), 0, stream, hidden, weight,
+      hipLaunchKernelGGL((router_logits_decode_kernel<HK, WK, 4>), dgrid, dim3(64 * RL_WAVES), 0, stream, hidden, weight,
                          logits, tokens, hidden_size, num_rows);
     }
     return static_cast<int>(hipGetLastError());
@@ -1588,57 +1587,85 @@ int launch_router_logits(const void* hidden, const void* weight, float* logits, 
 
 // ---- router: top-k experts of a row of logits and the softmax of their logits --------
 //
-// One wave per token.  Lane l keeps the logits of experts l, l+64, ... (up to 16 of them,
-// so num_experts <= 1024) in registers.  top_k times: every lane's best remaining
-// (value, index), a butterfly maximum over the wave that prefers the lower index on
-// equal values, and the owner retires its entry.  The winners' logits sit in lanes
-// 0..top_k-1 at the end, where the softmax over them is taken
+// One wave per token.  Lane l keeps the experts l, l+64, ... (PER of them: 4 up to 256 experts, 16 up to 1024) in
+// registers as 64-bit keys: the logit's bits mapped so that unsigned order is float order, above the complement of
+// the expert index, so the largest key is the largest logit and, among equals, the lowest index; 0 stands for "no
+// candidate" (past num_experts, NaN, a logit at or below the lowest float, a retired winner).  top_k times: every
+// lane's largest key, the maximum over the wave (four DPP exchanges inside each row of 16 lanes, then the four rows
+// through scalar registers: no trip through LDS, which made a round cost 0.85 us), and the owner retires its entry.
+// The winners' logits sit in lanes 0..top_k-1 at the end, where the softmax over them is taken
 // (max = the first winner, denominator floored at 1e-20: router.hip:628-715).
 constexpr int ROUTER_MAX_PER_LANE = 16;
 constexpr float ROUTER_LOWEST = -3.4028234663852886e38f;
+constexpr int DPP_ROW_MIRROR = 0x140;   // lane i <-> lane 15-i inside each row of 16
 
+struct RouterKey {
+  uint32_t hi, lo;
+};
+__device__ __forceinline__ bool router_key_above(const RouterKey& a, const RouterKey& b) {
+  return a.hi > b.hi || (a.hi == b.hi && a.lo > b.lo);
+}
+template <int CTRL>
+__device__ __forceinline__ RouterKey router_key_dpp_max(const RouterKey& k) {
+  const RouterKey o{static_cast<uint32_t>(dpp_i<CTRL>(static_cast<int>(k.hi))),
+                    static_cast<uint32_t>(dpp_i<CTRL>(static_cast<int>(k.lo)))};
+  return router_key_above(o, k) ? o : k;
+}
+
+template <int PER>
 __global__ void __launch_bounds__(256) router_select_kernel(const float* __restrict__ logits,
                                                             int64_t* __restrict__ selected,
                                                             float* __restrict__ routing, int64_t tokens,
                                                             int64_t logits_stride, int num_experts, int top_k) {
   const int lane = threadIdx.x & 63;
   const int64_t token = static_cast<int64_t>(blockIdx.x) * (blockDim.x >> 6) + (threadIdx.x >> 6);
-  if (token >= tokens) return;
+  if (token >= tokens) return;      // whole waves leave: the lane exchanges below see full waves
   const float* row = logits + token * logits_stride;
-  float vals[ROUTER_MAX_PER_LANE];
+  RouterKey keys[PER];
 #pragma unroll
-  for (int i = 0; i < ROUTER_MAX_PER_LANE; ++i) {
+  for (int i = 0; i < PER; ++i) {
     const int ex = lane + 64 * i;
-    vals[i] = ex < num_experts ? row[ex] : ROUTER_LOWEST;
+    const float f = ex < num_experts ? row[ex] : ROUTER_LOWEST;
+    const uint32_t raw = float_to_bits(f);
+    const uint32_t bits = raw == 0x80000000u ? 0u : raw;     // -0 and +0 are equal logits
+    const bool candidate = f > ROUTER_LOWEST;     // false for NaN too
+    keys[i].hi = candidate ? ((bits & 0x80000000u) ? ~bits : (bits | 0x80000000u)) : 0u;
+    keys[i].lo = candidate ? ~static_cast<uint32_t>(ex) : 0u;
   }
   float mine = 0.0f;    // lane p < top_k: logit of the p-th winner
   for (int pos = 0; pos < top_k; ++pos) {
-    float best = ROUTER_LOWEST;
-    int best_i = -1;
+    RouterKey best = keys[0];
 #pragma unroll
-    for (int i = 0; i < ROUTER_MAX_PER_LANE; ++i) {
-      const int ex = lane + 64 * i;
-      if (ex < num_experts && vals[i] > best) { best = vals[i]; best_i = ex; }   // strict: lowest index of equals
+    for (int i = 1; i < PER; ++i) best = router_key_above(keys[i], best) ? keys[i] : best;
+    best = router_key_dpp_max<DPP_QUAD_XOR1>(best);
+    best = router_key_dpp_max<DPP_QUAD_XOR2>(best);
+    best = router_key_dpp_max<DPP_ROW_HALF_MIRROR>(best);
+    best = router_key_dpp_max<DPP_ROW_MIRROR>(best);       // every lane: the maximum of its row of 16
+    RouterKey win{static_cast<uint32_t>(__builtin_amdgcn_readlane(static_cast<int>(best.hi), 0)),
+                  static_cast<uint32_t>(__builtin_amdgcn_readlane(static_cast<int>(best.lo), 0))};
+#pragma unroll
+    for (int r = 1; r < 4; ++r) {
+      const RouterKey o{static_cast<uint32_t>(__builtin_amdgcn_readlane(static_cast<int>(best.hi), 16 * r)),
+                        static_cast<uint32_t>(__builtin_amdgcn_readlane(static_cast<int>(best.lo), 16 * r))};
+      win = router_key_above(o, win) ? o : win;
     }
-    // (a retired expert holds ROUTER_LOWEST, which the strict comparison never picks)
+    const bool any = win.hi != 0u;
+    const uint32_t wbits = (win.hi & 0x80000000u) ? (win.hi & 0x7FFFFFFFu) : ~win.hi;
+    if (lane == pos) mine = any ? bits_to_float(wbits) : ROUTER_LOWEST;
+    if (lane == 0) selected[token * top_k + pos] = any ? static_cast<int64_t>(~win.lo) : -1;
 #pragma unroll
-    for (int off = 1; off < 64; off <<= 1) {
-      const float ov = __shfl_xor(best, off);
-      const int oi = __shfl_xor(best_i, off);
-      const bool take = oi >= 0 && (best_i < 0 || ov > best || (ov == best && oi < best_i));
-      best = take ? ov : best;
-      best_i = take ? oi : best_i;
+    for (int i = 0; i < PER; ++i) {
+      const bool gone = keys[i].hi == win.hi && keys[i].lo == win.lo;
+      keys[i].hi = gone ? 0u : keys[i].hi;
+      keys[i].lo = gone ? 0u : keys[i].lo;
     }
-    if (lane == pos) mine = best;
-    if (lane == 0) selected[token * top_k + pos] = best_i;
-#pragma unroll
-    for (int i = 0; i < ROUTER_MAX_PER_LANE; ++i)
-      if (lane + 64 * i == best_i) vals[i] = ROUTER_LOWEST;
   }
-  const float top = __shfl(mine, 0);
+  const float top = bits_to_float(static_cast<uint32_t>(__builtin_amdgcn_readlane(static_cast<int>(float_to_bits(mine)), 0)));
   const float ev = lane < top_k ? expf(mine - top) : 0.0f;
   float denom = 0.0f;
-  for (int p = 0; p < top_k; ++p) denom += __shfl(ev, p);   // in position order, as the reference sums
+  for (int p = 0; p < top_k; ++p) {      // in position order, as the reference sums
+    denom += bits_to_float(static_cast<uint32_t>(__builtin_amdgcn_readlane(static_cast<int>(float_to_bits(ev)), p)));
+  }
   denom = fmaxf(denom, 1.0e-20f);
   if (lane < top_k) routing[token * top_k + lane] = ev / denom;
 }
@@ -2127,8 +2154,13 @@ extern "C" int hipengine_qwen35_router_select(const float* logits, int64_t* sele
   }
   const int waves = 4;   // tokens per workgroup; `threads` is accepted and ignored
   const unsigned grid = static_cast<unsigned>((tokens + waves - 1) / waves);
-  hipLaunchKernelGGL(router_select_kernel, dim3(grid), dim3(waves * 64), 0, stream, logits, selected, routing, tokens,
-                     logits_stride, static_cast<int>(num_experts), static_cast<int>(top_k));
+  if (num_experts <= 64 * 4) {
+    hipLaunchKernelGGL(router_select_kernel<4>, dim3(grid), dim3(waves * 64), 0, stream, logits, selected, routing,
+                       tokens, logits_stride, static_cast<int>(num_experts), static_cast<int>(top_k));
+  } else {
+    hipLaunchKernelGGL(router_select_kernel<ROUTER_MAX_PER_LANE>, dim3(grid), dim3(waves * 64), 0, stream, logits,
+                       selected, routing, tokens, logits_stride, static_cast<int>(num_experts), static_cast<int>(top_k));
+  }
   return static_cast<int>(hipGetLastError());
 }
 

@@ -206,6 +206,9 @@ def test_router_select(dev, tokens, experts, top_k, stride):
     logits[0, : min(experts, 6)] = 0.75             # equal logits
     if tokens > 1:
         logits[1, :experts] = -2.5                  # a whole row of equal logits
+    if tokens > 2 and experts >= 8:
+        logits[2, :experts] = -np.abs(logits[2, :experts]) - 0.5
+        logits[2, [5, 1, 6]] = [-0.0, 0.0, -0.0]    # zeros of either sign are equal: lowest index first
     dl = dev.put(logits)
     dsel, dw = dev.empty(tokens * top_k * 8, fill=0xFF), dev.empty(tokens * top_k * 4, fill=0xFF)
     RT.qwen35_router_select(dl.ptr, dsel.ptr, dw.ptr, tokens, stride, experts, top_k)
