@@ -285,6 +285,26 @@ class Harness:
             self.memory.free(buf)
         return ev, 2.0 * m * n * k
 
+    def router_case(self, tokens: int, steps: int, warmup: int, experts: int = 256, top_k: int = 8, hidden: int = 2048):
+        """Router of a MoE layer: logits = bf16 hidden rows x float32 router weight, then top-k + softmax.
+        Returns HIP-event seconds per launch of each (from Python: short kernels measure the host's launch rate)."""
+        from hipengine_amd.kernels.hip_gfx950.moe import router as RT
+
+        rt, mem = self.rt, self.memory
+        rng = np.random.default_rng(100 + tokens)
+        x = mem.to_device(rng.integers(0x3C00, 0x3F00, size=(tokens, hidden)).astype(np.uint16), runtime=rt)
+        w = mem.to_device((rng.standard_normal((experts, hidden)) * 0.05).astype(np.float32), runtime=rt)
+        lg = mem.malloc(tokens * experts * 4, runtime=rt)
+        sel = mem.malloc(tokens * top_k * 8, runtime=rt)
+        ro = mem.malloc(tokens * top_k * 4, runtime=rt)
+        logits = lambda i: RT.qwen35_router_logits_bf16_f32w(x.ptr, w.ptr, lg.ptr, tokens, hidden, experts)
+        select = lambda i: RT.qwen35_router_select(lg.ptr, sel.ptr, ro.ptr, tokens, experts, experts, top_k)
+        t_logits = self.time_launches(logits, steps, warmup)[1]
+        t_select = self.time_launches(select, steps, warmup)[1]
+        for buf in (x, w, lg, sel, ro):
+            mem.free(buf)
+        return t_logits, t_select
+
     def moe_case(self, tokens: int, steps: int, warmup: int, experts: int = 256, top_k: int = 8, hidden: int = 2048,
                  inter: int = 512, down_quant: str = "q4_k"):
         """Selected-expert FFN (Q4_K gate/up, Q4_K or Q6_K down): the two-launch decode chain for
@@ -555,6 +575,10 @@ def main() -> None:
                 "int8_TOPS": round(ops / sec / 1e12, 2), "launches": 2 if tokens <= 8 else 8}
             if h.last_moe_graph_s:
                 extra[f"moe_q4_k_e256_k8_h2048_i512_t{tokens}"]["hip_graph_us"] = round(h.last_moe_graph_s * 1e6, 1)
+        for tokens in (1, 8, 2048):
+            t_logits, t_select = h.router_case(tokens, max(10, args.steps // 10), 3)
+            extra[f"router_e256_k8_h2048_t{tokens}"] = {"logits_us": round(t_logits * 1e6, 1),
+                                                         "select_us": round(t_select * 1e6, 1)}
         for tokens in (1, 2048):    # the same FFN with Q6_K down experts (what a Q4_K_M file holds in half its layers)
             sec, touched, ops = h.moe_case(tokens, max(10, args.steps // 10) if tokens <= 8 else msteps, 3,
                                            down_quant="q6_k")
