@@ -186,7 +186,7 @@ Plan default_plan(int qt, int rows, int64_t K, int64_t N) {
 }
 
 // The kernel form a batch of `chunk` <= 8 rows takes, and the rows of it that go in one launch.
-enum GemvForm { FORM_ROW_STRIDED = 0, FORM_RUN = 1, FORM_STREAM = 2, FORM_SLAB = 3, FORM_PSLAB = 4 };
+enum GemvForm { FORM_ROW_STRIDED = 0, FORM_RUN = 1, FORM_STREAM = 2, FORM_SLAB = 3, FORM_PSLAB = 4, FORM_DSLAB = 5 };
 
 // Q4_K, K <= 6144: the int8 MFMA slab form wins for batches of 3 and more (17408x5120 at batch 3: 17.0 us against
 // 23.0 for the stream form), the stream form at batch 1 and 2 wherever it applies (batch 1: 4.5 against 6.3 us
@@ -198,7 +198,19 @@ bool slab_preferred(int qt, int chunk, int64_t K, int64_t N, const SlabPlan& sl)
   return !default_stream_plan(qt, chunk, K, N).ok;
 }
 
+// The direct slab form is taken where it splits K over workgroups (rows too long for the other MFMA forms to
+// hold the quantized activations of): batch 3..8 of K >= 8192 or so.  Measured on MI355X, batch 8 / 4:
+// Q6_K 5120x17408 27.1 / 26.0 us against 38.0 / 31.9 for the phased slab, Q4_K 5120x17408 23.5 / 22.4 against
+// 28.0 / 23.1, Q8_0 5120x17408 32.6 / 31.5 against 36.8 / 30.3; where K fits one part the older forms are as fast
+// or faster (all of them are bound by VALU issue there), and at batch 1 and 2 the stream form is.
+bool dslab_preferred(int qt, int chunk, int64_t K, int64_t N, const void* w) {
+  if (chunk < 3) return false;
+  const DslabPlan dp = default_dslab_plan(qt, chunk, K, N, w);
+  return dp.ok && dp.ksplit > 1;
+}
+
 GemvForm pick_form(int qt, int& chunk, int64_t K, int64_t N, const void* w) {
+  if (dslab_preferred(qt, chunk, K, N, w)) return FORM_DSLAB;
   const SlabPlan sl = default_slab_plan(qt, chunk, K, N);
   const PslabPlan pp = default_pslab_plan(qt, chunk, K, N, w);
   // a batch of 5..8 whose quantized activations do not fit the LDS of any form that takes it whole
@@ -232,7 +244,9 @@ int launch_gemv(int qt, const void* x, int x_kind, const uint8_t* w, void* out, 
     void* outr = static_cast<uint8_t*>(out) + r0 * N * out_elem;
     if (form != FORM_ROW_STRIDED) {
       int rc;
-      if (form == FORM_SLAB) {
+      if (form == FORM_DSLAB) {
+        rc = launch_gemv_dslab(qt, xr, x_kind, w, outr, out_kind, chunk, K, N, default_dslab_plan(qt, chunk, K, N, w), stream);
+      } else if (form == FORM_SLAB) {
         rc = launch_gemv_slab(xr, x_kind, w, outr, out_kind, chunk, K, N, default_slab_plan(qt, chunk, K, N), stream);
       } else if (form == FORM_PSLAB) {
         rc = launch_gemv_pslab(qt, xr, x_kind, w, outr, out_kind, chunk, K, N, default_pslab_plan(qt, chunk, K, N, w),
@@ -284,6 +298,11 @@ int hipengine_gfx950::gemv_raise_lds_limits() {
   int rc = slab_raise_lds_limits();
   if (rc == static_cast<int>(hipSuccess)) rc = pslab_raise_lds_limits();
   if (rc == static_cast<int>(hipSuccess)) rc = stream_raise_lds_limits();
+  if (rc == static_cast<int>(hipSuccess)) {
+    int device = -1;
+    rc = static_cast<int>(hipGetDevice(&device));
+    if (rc == static_cast<int>(hipSuccess)) rc = dslab_setup(device);
+  }
   return rc;
 }
 
@@ -633,6 +652,26 @@ extern "C" int hipengine_gfx950_gguf_q8_1_fused_gemv_pslab_tuned(int32_t ggml_ty
                            out_features, p, stream);
 }
 
+extern "C" int hipengine_gfx950_gguf_q8_1_fused_gemv_dslab_tuned(int32_t ggml_type, const void* x, int32_t x_kind,
+                                                                const uint8_t* qweight, void* out, int32_t out_kind,
+                                                                int64_t rows, int64_t in_features,
+                                                                int64_t out_features, int32_t waves, int32_t ring,
+                                                                int32_t workgroups, int32_t k_parts, hipStream_t stream) {
+  if (!x || !qweight || !out || x_kind < KIND_F32 || x_kind > KIND_Q8_1 || out_kind < KIND_F32 ||
+      out_kind > KIND_F16 || rows <= 0 || rows > 8 || in_features <= 0 || (in_features % QK_K) != 0 ||
+      out_features <= 0) {
+    return static_cast<int>(hipErrorInvalidValue);
+  }
+  DslabPlan p = k_parts > 0 ? dslab_plan_for(ggml_type, static_cast<int>(rows), in_features, out_features, qweight, k_parts)
+                            : default_dslab_plan(ggml_type, static_cast<int>(rows), in_features, out_features, qweight);
+  if (!p.ok) return static_cast<int>(hipErrorInvalidValue);
+  if (waves > 0) p.waves = waves;
+  if (ring > 0) p.ring = ring;
+  if (workgroups > 0) p.row_groups = workgroups / p.ksplit > 0 ? workgroups / p.ksplit : 1;
+  return launch_gemv_dslab(ggml_type, x, x_kind, qweight, out, out_kind, static_cast<int>(rows), in_features,
+                           out_features, p, stream);
+}
+
 // ---- verification: the int32 dots of the MFMA forms -------------------------------------
 
 extern "C" int hipengine_gfx950_gguf_gemv_mfma_dots_i32(int32_t ggml_type, int32_t form, const void* xq,
@@ -649,6 +688,12 @@ extern "C" int hipengine_gfx950_gguf_gemv_mfma_dots_i32(int32_t ggml_type, int32
     if (!p.ok) return static_cast<int>(hipErrorInvalidValue);
     return launch_gemv_slab(xq, KIND_Q8_1, qweight, out, KIND_F32, static_cast<int>(rows), in_features, out_features, p,
                             stream, nullptr, nullptr, dots);
+  }
+  if (form == FORM_DSLAB) {
+    const DslabPlan p = default_dslab_plan(ggml_type, 8, in_features, out_features, qweight);
+    if (!p.ok) return static_cast<int>(hipErrorInvalidValue);
+    return launch_gemv_dslab(ggml_type, xq, KIND_Q8_1, qweight, out, KIND_F32, static_cast<int>(rows), in_features,
+                             out_features, p, stream, nullptr, nullptr, dots);
   }
   if (form == FORM_PSLAB) {
     const PslabPlan p = default_pslab_plan(ggml_type, 8, in_features, out_features, qweight);
@@ -751,6 +796,14 @@ extern "C" int hipengine_gfx950_gguf_pair_silu_gemv(int32_t ggml_type, const voi
     // round_mid arithmetic, so a 16-bit output without round_mid is not taken.
     if (!round_mid && out_kind != KIND_F32) return static_cast<int>(hipErrorInvalidValue);
     const int r = static_cast<int>(rows);
+    if (dslab_preferred(ggml_type, r, in_features, out_features, qweight_gate) &&
+        dslab_preferred(ggml_type, r, in_features, out_features, qweight_up)) {
+      const DslabPlan dg = default_dslab_plan(ggml_type, r, in_features, out_features, qweight_gate);
+      const int rc = launch_gemv_dslab(ggml_type, x, x_kind, qweight_gate, out, out_kind, r, in_features, out_features, dg, stream);
+      if (rc != static_cast<int>(hipSuccess)) return rc;
+      return launch_gemv_dslab(ggml_type, x, x_kind, qweight_up, out, out_kind, r, in_features, out_features,
+                               default_dslab_plan(ggml_type, r, in_features, out_features, qweight_up), stream, nullptr, out);
+    }
     const SlabPlan sl = default_slab_plan(ggml_type, r, in_features, out_features);
     if (sl.ok) {
       // one launch where a workgroup's rows of both matrices fit its partial-sum buffer (up to 72 x 256 rows)
@@ -787,6 +840,11 @@ extern "C" int hipengine_gfx950_gguf_gemv_residual(int32_t ggml_type, const void
       out_kind > KIND_F16 || rows <= 0 || rows > 8 || in_features <= 0 || (in_features % QK_K) != 0 ||
       out_features <= 0) {
     return static_cast<int>(hipErrorInvalidValue);
+  }
+  if (dslab_preferred(ggml_type, static_cast<int>(rows), in_features, out_features, qweight)) {
+    return launch_gemv_dslab(ggml_type, x, x_kind, qweight, out, out_kind, static_cast<int>(rows), in_features, out_features,
+                             default_dslab_plan(ggml_type, static_cast<int>(rows), in_features, out_features, qweight), stream,
+                             residual);
   }
   const SlabPlan sl = default_slab_plan(ggml_type, static_cast<int>(rows), in_features, out_features);
   if (slab_preferred(ggml_type, static_cast<int>(rows), in_features, out_features, sl)) {

@@ -41,6 +41,18 @@ int launch_gemv_pslab(int qt, const void* x, int x_kind, const uint8_t* w, void*
                       const void* gate = nullptr, int32_t* dots_out = nullptr);
 int pslab_raise_lds_limits();
 
+// ---- direct slab form (weights streamed straight into LDS, int8 MFMA; batch 2..8) ----
+struct DslabPlan {
+  int waves, ring, row_groups, ksplit, blocks_part;
+  bool ok;
+};
+DslabPlan default_dslab_plan(int qt, int rows, int64_t K, int64_t N, const void* w);
+DslabPlan dslab_plan_for(int qt, int rows, int64_t K, int64_t N, const void* w, int parts);
+int launch_gemv_dslab(int qt, const void* x, int x_kind, const uint8_t* w, void* out, int out_kind, int rows,
+                      int64_t K, int64_t N, const DslabPlan& p, hipStream_t stream, const void* residual = nullptr,
+                      const void* gate = nullptr, int32_t* dots_out = nullptr);
+int dslab_setup(int device);   // per device: dynamic-LDS limits, addresses of the split-K scratch
+
 // ---- stream form (resident waves, ring of loads in flight) ----
 enum StreamFuse { FUSE_NONE = 0, FUSE_PAIR = 1, FUSE_RESIDUAL = 2, FUSE_DUAL = 3 };   // epilogue of the stream kernels
 struct StreamPlan {

@@ -20,7 +20,7 @@ I32 = ctypes.c_int32
 ALLOWED_THREADS = frozenset({64, 128, 256})
 KIND_F32, KIND_BF16, KIND_F16, KIND_Q8_1 = 0, 1, 2, 3
 GGML_Q8_0, GGML_Q4_K, GGML_Q5_K, GGML_Q6_K = 8, 12, 13, 14
-# Q5_K: decode GEMV (all forms), dequantization and embedding lookup; the MMQ prefill takes Q4_K and Q6_K
+# the four block types every kernel family here takes (decode GEMV, MMQ prefill, MoE, dequantization, embedding)
 QUANT_KEY_TO_GGML = {"gguf_q8_0": GGML_Q8_0, "gguf_q4_k": GGML_Q4_K, "gguf_q5_k": GGML_Q5_K, "gguf_q6_k": GGML_Q6_K}
 
 _entry_cache: dict[tuple[int, str], ctypes._CFuncPtr] = {}

@@ -378,6 +378,21 @@ def gguf_q8_1_fused_gemv_pslab_tuned(quant_key: str, x_ptr: int, x_kind: str, qw
                     in_features, out_features, waves, blocks_per_wave, workgroups, stream), runtime)
 
 
+def gguf_q8_1_fused_gemv_dslab_tuned(quant_key: str, x_ptr: int, x_kind: str, qweight_ptr: int, out_ptr: int,
+                                     out_kind: str, rows: int, in_features: int, out_features: int, *,
+                                     waves: int = 0, ring: int = 0, workgroups: int = 0, k_parts: int = 0,
+                                     stream: int = 0, library: ctypes.CDLL | None = None,
+                                     runtime: HipRuntime | None = None) -> None:
+    """The direct slab form (weights streamed straight into LDS, int8 MFMA) of the fused GEMV with an explicit
+    wave count, ring depth (steps of 16 rows in flight per wave), grid and number of K parts (1, 2, 4); 0 takes
+    the planner's (tuning sweeps and tests only)."""
+    validate_linear(rows, in_features, out_features)
+    fn = entry("hipengine_gfx950_gguf_q8_1_fused_gemv_dslab_tuned",
+               [I32, VOID, I32, VOID, VOID, I32, I64, I64, I64, I32, I32, I32, I32, VOID], library)
+    check_launch(fn(QUANT_KEY_TO_GGML[quant_key], x_ptr, _KINDS[x_kind], qweight_ptr, out_ptr, _KINDS[out_kind], rows,
+                    in_features, out_features, waves, ring, workgroups, k_parts, stream), runtime)
+
+
 def gguf_gemv_default_plan(quant_key: str, rows: int, in_features: int, out_features: int, *,
                            library: ctypes.CDLL | None = None) -> dict[str, int]:
     """The workgroup layout the library picks for a shape (host only)."""
@@ -387,7 +402,7 @@ def gguf_gemv_default_plan(quant_key: str, rows: int, in_features: int, out_feat
     return dict(zip(("batch_bucket", "rows_per_lane", "blocks_per_wave", "k_slices", "row_groups"), plan))
 
 
-GEMV_FORMS = ("row_strided", "run", "stream", "slab", "phased_slab")
+GEMV_FORMS = ("row_strided", "run", "stream", "slab", "phased_slab", "direct_slab")
 
 
 def gguf_gemv_default_form(quant_key: str, rows: int, in_features: int, out_features: int, *,

@@ -40,7 +40,7 @@ def gguf_q8_1_block_dots_i32(quant_key: str, xq_ptr: int, qweight_ptr: int, dots
                     out_features, stream), runtime)
 
 
-FORM_SLAB, FORM_PSLAB = 3, 4
+FORM_SLAB, FORM_PSLAB, FORM_DSLAB = 3, 4, 5
 
 
 def gguf_gemv_mfma_dots_i32(quant_key: str, form: int, xq_ptr: int, qweight_ptr: int, dots_ptr: int, out_ptr: int,
@@ -51,8 +51,8 @@ def gguf_gemv_mfma_dots_i32(quant_key: str, form: int, xq_ptr: int, qweight_ptr:
     kernel's float32 result ``[rows, out_features]``.  ``xq``: 36-byte q8_1 blocks, ``rows <= 8``."""
     if rows <= 0 or rows > 8 or out_features <= 0 or in_features <= 0 or in_features % 256:
         raise ValueError("rows must be in 1..8, out_features positive and in_features divisible by 256")
-    if form not in (FORM_SLAB, FORM_PSLAB):
-        raise ValueError("form must be FORM_SLAB or FORM_PSLAB")
+    if form not in (FORM_SLAB, FORM_PSLAB, FORM_DSLAB):
+        raise ValueError("form must be FORM_SLAB, FORM_PSLAB or FORM_DSLAB")
     validate_pointers(xq_ptr=xq_ptr, qweight_ptr=qweight_ptr, dots_ptr=dots_ptr, out_ptr=out_ptr)
     fn = entry("hipengine_gfx950_gguf_gemv_mfma_dots_i32", [I32, I32, VOID, VOID, VOID, VOID, I64, I64, I64, VOID], library)
     check_launch(fn(QUANT_KEY_TO_GGML[quant_key], form, xq_ptr, qweight_ptr, dots_ptr, out_ptr, rows, in_features,

@@ -101,8 +101,8 @@ int hipengine_gguf_q8_1_d4s4_f32_quantize_bf16(const void* x, void* out, int64_t
 /* ------------------------------------------------------------------------
  * Decode GEMV, batch 1..8 per launch (more rows are split into launches of 8)
  *   out[r, n] = sum_k W[n, k] * x[r, k],  W raw Q4_K / Q5_K / Q6_K / Q8_0 blocks
- * in_features % 256 == 0 for all weight types.  Q5_K (arithmetic of gguf_k_gemv.hip:115-137 on q8_1
- * activations) runs the row-strided form only.
+ * in_features % 256 == 0 for all weight types.  Q5_K follows the arithmetic of gguf_k_gemv.hip:115-137 on q8_1
+ * activations (the Q4_K formula with the fifth bit taken from qh) and takes every kernel form but the Q4_K slab.
  * ------------------------------------------------------------------------ */
 
 /* Fused: x is [rows, in_features] float32 / bf16 / fp16; the q8_1 quantization
@@ -889,7 +889,7 @@ int hipengine_gfx950_gguf_q8_1_block_dots_i32(int32_t ggml_type, const void* xq,
 
 /* The same dots as the kernels that run on the int8 MFMA produce them: the production kernel body with one
  * more store per MFMA result.  form 3: the slab form (Q4_K), form 4: the phased slab form (Q4_K, Q5_K, Q6_K,
- * Q8_0); both in their batch-8 instantiation, xq = 36-byte q8_1 blocks [rows, K/32], rows <= 8, shapes as
+ * Q8_0), form 5: the direct slab form (Q4_K, Q6_K, Q8_0); all in their batch-8 instantiation, xq = 36-byte q8_1 blocks [rows, K/32], rows <= 8, shapes as
  * the forms take them.  dots as above; out: float32 [rows, out_features], the kernel's normal result. */
 int hipengine_gfx950_gguf_gemv_mfma_dots_i32(int32_t ggml_type, int32_t form, const void* xq, const uint8_t* qweight,
                                              int32_t* dots, float* out, int64_t rows, int64_t in_features,

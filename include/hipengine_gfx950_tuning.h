@@ -68,6 +68,20 @@ int hipengine_gfx950_gguf_q8_1_fused_gemv_pslab_tuned(int32_t ggml_type, const v
                                                       int32_t waves, int32_t blocks_per_wave, int32_t workgroups,
                                                       hipengine_stream_t stream);
 
+/* The direct slab form of the fused Q4_K / Q6_K / Q8_0 GEMV with an explicit layout (0 = the planner's
+ * choice): weight blocks go from global memory straight into LDS (global_load_lds), `ring` steps of 16 rows
+ * in flight per wave; `waves` <= 12 waves per workgroup split the K blocks of the workgroup's part, at most
+ * two per wave; `k_parts` (1, 2, 4) splits K over workgroups, whose partial sums meet in a scratch array the
+ * library holds (eight regions taken in turn by successive launches: more than eight such launches in flight at
+ * once on one device share a region and race) and are added in part order by the workgroup that arrives last;
+ * `workgroups` = row groups x k_parts.  rows <= 8, weights 2-byte aligned and < 4 GiB.  The default dispatch
+ * takes this form for batches of 3 to 8 where K has to be split (in_features >= 6400 for Q4_K / Q6_K).  New here. */
+int hipengine_gfx950_gguf_q8_1_fused_gemv_dslab_tuned(int32_t ggml_type, const void* x, int32_t x_kind,
+                                                      const uint8_t* qweight, void* out, int32_t out_kind,
+                                                      int64_t rows, int64_t in_features, int64_t out_features,
+                                                      int32_t waves, int32_t ring, int32_t workgroups, int32_t k_parts,
+                                                      hipengine_stream_t stream);
+
 /* Host only: the layout the library picks for a shape, as
  * {batch_bucket, rows_per_lane, blocks_per_wave, k_slices, row_groups}.  New here. */
 int hipengine_gfx950_gguf_gemv_default_plan(int32_t ggml_type, int64_t rows, int64_t in_features,
@@ -75,8 +89,8 @@ int hipengine_gfx950_gguf_gemv_default_plan(int32_t ggml_type, int64_t rows, int
 
 /* Host only: the kernel form the default dispatch takes for the first launch of a
  * batch, as {form, rows in that launch}: form 0 row-strided, 1 run, 2 stream,
- * 3 slab (Q4_K on the int8 MFMA), 4 phased slab (int8 MFMA).  Weights are assumed
- * 4-byte aligned.  New here. */
+ * 3 slab (Q4_K on the int8 MFMA), 4 phased slab (int8 MFMA), 5 direct slab (int8 MFMA, weights
+ * streamed straight into LDS, K split over workgroups).  Weights are assumed 4-byte aligned.  New here. */
 int hipengine_gfx950_gguf_gemv_default_form(int32_t ggml_type, int64_t rows, int64_t in_features,
                                             int64_t out_features, int32_t* form2);
 
