@@ -204,7 +204,9 @@ bool slab_preferred(int qt, int chunk, int64_t K, int64_t N, const SlabPlan& sl)
 // 28.0 / 23.1, Q8_0 5120x17408 32.6 / 31.5 against 36.8 / 30.3; where K fits one part the older forms are as fast
 // or faster (all of them are bound by VALU issue there), and at batch 1 and 2 the stream form is.
 bool dslab_preferred(int qt, int chunk, int64_t K, int64_t N, const void* w) {
-  if (chunk < 3) return false;
+  // K > 6144: more blocks than the waves of one workgroup hold (Q8_0 at K = 5120 would split as well, for LDS
+  // room, and measures slower than the phased slab: 17.3 against 14.7 us at 5120x5120, batch 8)
+  if (chunk < (qt == GGML_Q8_0 ? 5 : 3) || K <= 6144) return false;
   const DslabPlan dp = default_dslab_plan(qt, chunk, K, N, w);
   return dp.ok && dp.ksplit > 1;
 }

@@ -71,9 +71,9 @@ def test_abi_version_and_host_only_entry_points(library):
                                    "k_q4_b1": (12, 1, 5120, 1024)}.items():
         assert ff(qt, rows, k, n, form) == 0
         picks[name] = (form[0], form[1])
-    # 0 row-strided, 1 run, 2 stream, 3 slab, 4 phased slab; second field: batch rows of the first launch
-    assert picks == {"c1": (2, 1), "c1_b8": (3, 8), "down_b1": (2, 1), "down_b8": (4, 8), "head_b4": (4, 4), "o_b4": (4, 4),
-                     "q4_long_b8": (4, 8), "q5_b2": (2, 2), "short_k": picks["short_k"], "odd_blocks_b8": (2, 8), "o_q4_b1": (2, 1), "o_q4_b2": (2, 2), "k_q4_b1": (2, 1)}
+    # 0 row-strided, 1 run, 2 stream, 3 slab, 4 phased slab, 5 direct slab; second field: batch rows of the first launch
+    assert picks == {"c1": (2, 1), "c1_b8": (3, 8), "down_b1": (2, 1), "down_b8": (5, 8), "head_b4": (4, 4), "o_b4": (4, 4),
+                     "q4_long_b8": (5, 8), "q5_b2": (2, 2), "short_k": picks["short_k"], "odd_blocks_b8": (2, 8), "o_q4_b1": (2, 1), "o_q4_b2": (2, 2), "k_q4_b1": (2, 1)}
     assert picks["short_k"][0] in (0, 1)
     assert ff(12, 1, 100, 64, form) == 1
     # argument checks come before any HIP call: null pointers and bad sizes are refused on a host without a GPU
