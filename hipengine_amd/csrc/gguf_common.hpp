@@ -232,4 +232,22 @@ __device__ __forceinline__ uint32_t load2(const uint8_t* p) {
   return v;
 }
 
+// ---- loads from global memory straight into LDS --------------------------------------------
+//
+// global_load_lds_dwordx4 / _dword: lane l's 16 (4) bytes at `base + voff` land at LDS byte `lds` + 16 l (4 l);
+// no register holds the data while the load is in flight.  The compiler does not see these as memory
+// operations with a result: completion is waited for with s_waitcnt vmcnt (loads complete in issue order),
+// by hand or through the wait the compiler places for a load of its own that was issued later.
+typedef __attribute__((address_space(3))) uint8_t lds_u8;
+
+__device__ __forceinline__ uint32_t lds_address(const void* p) {
+  return static_cast<uint32_t>(reinterpret_cast<uintptr_t>((lds_u8*)p));
+}
+__device__ __forceinline__ void lds_dma16(const uint8_t* base, uint32_t voff, uint32_t lds) {
+  asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2" ::"s"(lds), "v"(voff), "s"(base) : "memory");
+}
+__device__ __forceinline__ void lds_dma4(const uint8_t* base, uint32_t voff, uint32_t lds) {
+  asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dword %1, %2" ::"s"(lds), "v"(voff), "s"(base) : "memory");
+}
+
 }  // namespace hipengine_gfx950

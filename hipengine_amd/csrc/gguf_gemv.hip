@@ -340,11 +340,19 @@ DEFINE_FUSED_ALL(q8_0, GGML_Q8_0)
 // the activations are quantized to q8_1 inside the kernel, so results follow the q8_1 arithmetic of
 // hipEngine's dp4a kernels, not the float-activation arithmetic of the kernels of the same name there.
 
+// The dispatcher's prefill_* keys reach the same symbols with many rows (one launch of a (out, rows) grid in
+// hipEngine, gguf_q4_k_gemv.hip:1468-1493): from 32 rows of bf16 activations on they are packed, a chunk of up to 512
+// rows at a time, into a buffer the library holds and go through the int8-MFMA MMQ - the weights are then read once
+// per 512 rows instead of once per 8.
 #define DEFINE_DENSE(QNAME, QT, ANAME, AKIND, ONAME, OKIND)                                               \
   extern "C" int hipengine_gguf_##QNAME##_gemv_##ANAME##_##ONAME##_out(                                   \
       const void* x, const uint8_t* qweight, void* out, int64_t rows, int64_t in_features,                \
       int64_t out_features, int64_t threads, hipStream_t stream) {                                        \
     (void)threads;                                                                                        \
+    if (AKIND == KIND_BF16 && x && qweight && out &&                                                      \
+        prefill_library_buffer_takes(QT, rows, in_features, out_features)) {                              \
+      return prefill_bf16_library_buffer(QT, x, qweight, out, OKIND, rows, in_features, out_features, stream); \
+    }                                                                                                     \
     return launch_gemv(QT, x, AKIND, qweight, out, OKIND, rows, in_features, out_features, nullptr,       \
                        stream);                                                                           \
   }

@@ -39,7 +39,6 @@ namespace hipengine_gfx950 {
 typedef int ds_v4i __attribute__((ext_vector_type(4)));
 typedef uint32_t ds_u32x4 __attribute__((ext_vector_type(4)));
 typedef float ds_f4 __attribute__((ext_vector_type(4)));
-typedef __attribute__((address_space(3))) uint8_t ds_lds_u8;
 
 struct GemvDslabArgs {
   const void* x;
@@ -118,20 +117,6 @@ template <int QT>
 constexpr size_t gemv_dslab_lds_bytes(int blocks_part, int waves, int ring, bool red_dedicated) {
   return static_cast<size_t>(red_dedicated ? waves * 512 * DS_GROUP : 0) +
          static_cast<size_t>(ring) * blocks_part * ds_image<QT>() + static_cast<size_t>(blocks_part) * DsTraits<QT>::REC;
-}
-
-__device__ __forceinline__ uint32_t ds_lds_addr(const void* p) {
-  return static_cast<uint32_t>(reinterpret_cast<uintptr_t>((ds_lds_u8*)p));
-}
-
-// One wave-wide load of 16 (4) bytes per lane from `base + voff` straight into LDS: lane l's bytes land at
-// lds + 16 l (4 l).  The compiler does not see it as a memory operation with a result: completion is waited
-// for with ds_wait_vm (loads complete in issue order).
-__device__ __forceinline__ void ds_dma16(const uint8_t* base, uint32_t voff, uint32_t lds) {
-  asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2" ::"s"(lds), "v"(voff), "s"(base) : "memory");
-}
-__device__ __forceinline__ void ds_dma4(const uint8_t* base, uint32_t voff, uint32_t lds) {
-  asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dword %1, %2" ::"s"(lds), "v"(voff), "s"(base) : "memory");
 }
 
 // Wait until at most n vector-memory operations of this wave are outstanding (n uniform, 0..40).
@@ -448,7 +433,7 @@ __device__ __forceinline__ void gemv_dslab_workgroup(const GemvDslabArgs& a, uin
   uint8_t* ring = ring_all + before * R * IMG;                     // this wave's R slots of nown * IMG bytes
   float* rec_all = reinterpret_cast<float*>(ring_all + a.blocks_part * R * IMG);
   const int slot_bytes = nown * IMG;
-  const uint32_t ring_lds = ds_lds_addr(ring);
+  const uint32_t ring_lds = lds_address(ring);
 
   // ---- load plan.  16-byte chunk ci = 64 k + lane of the unit's chunk section [block][row][position], then
   // dword di = 64 k + lane of its dword section [block][row][index].  vfull = the lane's offset from the first
@@ -486,13 +471,13 @@ __device__ __forceinline__ void gemv_dslab_workgroup(const GemvDslabArgs& a, uin
 #pragma unroll
     for (int k = 0; k < LC_MAX; ++k) {
       if (k < LC) {
-        if (64 * k + lane < unit_chunks) ds_dma16(base, offset(k), slot + 1024u * k);
+        if (64 * k + lane < unit_chunks) lds_dma16(base, offset(k), slot + 1024u * k);
       }
     }
 #pragma unroll
     for (int k = 0; k < LD_MAX; ++k) {
       if (k < LD) {
-        if (64 * k + lane < unit_dwords) ds_dma4(base, offset(LC_MAX + k), slot + static_cast<uint32_t>(nown * IMG_C) + 256u * k);
+        if (64 * k + lane < unit_dwords) lds_dma4(base, offset(LC_MAX + k), slot + static_cast<uint32_t>(nown * IMG_C) + 256u * k);
       }
     }
   };

@@ -34,6 +34,8 @@ extern "C" int hipengine_gfx950_init(void) {
   if (rc != static_cast<int>(hipSuccess)) return rc;
   rc = hipengine_gfx950::argmax_noalloc_setup(device);
   if (rc != static_cast<int>(hipSuccess)) return rc;
+  rc = hipengine_gfx950::prefill_pack_setup(device);
+  if (rc != static_cast<int>(hipSuccess)) return rc;
   int (*const loads[])() = {hipengine_gfx950::quantize_load, hipengine_gfx950::mmq_load, hipengine_gfx950::moe_load,
                             hipengine_gfx950::embedding_load};
   for (auto load : loads) {

@@ -17,6 +17,8 @@
 
 #include "gguf_init.hpp"
 
+#include <atomic>
+
 #include "../../include/hipengine_gfx950.h"
 #include "../../include/hipengine_gfx950_tuning.h"
 
@@ -326,6 +328,31 @@ extern "C" int hipengine_gfx950_gguf_prefill_workspace_bytes(int32_t ggml_type, 
   return static_cast<int>(hipSuccess);
 }
 
+// What the MMQ launch of a type refuses, checked before anything is enqueued (a call that is refused leaves
+// nothing in the stream and writes nothing).
+static bool prefill_shape_ok(int32_t ggml_type, const void* x, const uint8_t* qweight, const void* out, int32_t out_kind,
+                             int64_t rows, int64_t in_features, int64_t out_features) {
+  const bool type_ok = ggml_type == GGML_Q4_K || ggml_type == GGML_Q5_K || ggml_type == GGML_Q6_K || ggml_type == GGML_Q8_0;
+  return type_ok && x && qweight && out && out_kind >= KIND_F32 && out_kind <= KIND_F16 && rows > 0 && in_features > 0 &&
+         (in_features % (ggml_type == GGML_Q8_0 ? 128 : QK_K)) == 0 && out_features > 0 && out_features <= (1 << 24) &&
+         ((ggml_type != GGML_Q4_K && ggml_type != GGML_Q5_K) || (out_features % 32) == 0);
+}
+
+// rows <= 2^20 of bf16 activations: pack into `workspace`, then the MMQ of the type
+static int prefill_packed(int32_t ggml_type, const void* x, const uint8_t* qweight, void* out, int32_t out_kind, int64_t rows,
+                          int64_t in_features, int64_t out_features, void* workspace, hipStream_t stream) {
+  if (ggml_type == GGML_Q4_K) {
+    const int prc = hipengine_gguf_q8_1_mmq_ds4_pack_bf16(x, workspace, rows, in_features, stream);
+    if (prc != static_cast<int>(hipSuccess)) return prc;
+    return launch_q4(workspace, qweight, out, out_kind, rows, in_features, out_features, 0, stream);
+  }
+  const int prc = hipengine_gguf_q8_1_d4s4_f32_quantize_bf16(x, workspace, rows, in_features, stream);
+  if (prc != static_cast<int>(hipSuccess)) return prc;
+  if (ggml_type == GGML_Q5_K) return launch_q5(workspace, qweight, out, out_kind, rows, in_features, out_features, stream);
+  if (ggml_type == GGML_Q8_0) return launch_q8_0(workspace, qweight, out, out_kind, rows, in_features, out_features, stream);
+  return launch_q6(workspace, qweight, out, out_kind, rows, in_features, out_features, stream);
+}
+
 extern "C" int hipengine_gfx950_gguf_prefill_bf16(int32_t ggml_type, const void* x, const uint8_t* qweight, void* out,
                                                   int32_t out_kind, int64_t rows, int64_t in_features,
                                                   int64_t out_features, void* workspace, int64_t workspace_bytes,
@@ -333,23 +360,81 @@ extern "C" int hipengine_gfx950_gguf_prefill_bf16(int32_t ggml_type, const void*
   int64_t need = 0;
   const int rc = hipengine_gfx950_gguf_prefill_workspace_bytes(ggml_type, rows, in_features, &need);
   if (rc != static_cast<int>(hipSuccess)) return rc;
-  if (!x || !workspace || workspace_bytes < need || (reinterpret_cast<uintptr_t>(workspace) & 15u) != 0) {
+  if (!workspace || workspace_bytes < need || (reinterpret_cast<uintptr_t>(workspace) & 15u) != 0 || rows > (1 << 20) ||
+      !prefill_shape_ok(ggml_type, x, qweight, out, out_kind, rows, in_features, out_features)) {
     return static_cast<int>(hipErrorInvalidValue);
   }
-  if (ggml_type == GGML_Q4_K) {
-    if ((out_features % 32) != 0) return static_cast<int>(hipErrorInvalidValue);
-    const int prc = hipengine_gguf_q8_1_mmq_ds4_pack_bf16(x, workspace, rows, in_features, stream);
-    if (prc != static_cast<int>(hipSuccess)) return prc;
-    return launch_q4(workspace, qweight, out, out_kind, rows, in_features, out_features, 0, stream);
+  return prefill_packed(ggml_type, x, qweight, out, out_kind, rows, in_features, out_features, workspace, stream);
+}
+
+// ---- the same with a pack buffer the library holds ----
+//
+// hipEngine's dense prefill entries take any number of rows and no workspace (gguf_q4_k_gemv.hip:1468-1493).  For
+// them the packed activations of a chunk of rows go to a file-scope device array: two regions of 12 MiB, taken in
+// turn by successive calls; a call walks its rows in chunks of up to 512 (pack, MMQ, pack, MMQ ... in stream
+// order), so the weights are read once per 512 rows.  Nothing is allocated.  Calls that overlap on one device -
+// more than two in flight on different streams - share a region and race.
+namespace {
+constexpr int64_t kPackRegionBytes = 12ll << 20;
+constexpr int kPackRegions = 2;
+constexpr int64_t kPackChunkRows = 512;
+constexpr int64_t kPackMinChunkRows = 128;       // below this the chunks re-read the weights too often to pay
+constexpr int kPackMaxDevices = 64;
+__device__ __align__(256) uint8_t prefill_pack[kPackRegions * kPackRegionBytes];
+std::atomic<uint8_t*> prefill_pack_ptr[kPackMaxDevices];
+std::atomic<unsigned> prefill_next_region{0};
+}  // namespace
+
+int hipengine_gfx950::prefill_pack_setup(int device) {
+  if (device < 0 || device >= kPackMaxDevices) return static_cast<int>(hipErrorInvalidDevice);
+  if (prefill_pack_ptr[device].load(std::memory_order_acquire)) return static_cast<int>(hipSuccess);
+  void* ptr = nullptr;
+  const hipError_t err = hipGetSymbolAddress(&ptr, HIP_SYMBOL(prefill_pack));
+  if (err != hipSuccess) return static_cast<int>(err);
+  if (!ptr) return static_cast<int>(hipErrorInvalidSymbol);
+  prefill_pack_ptr[device].store(static_cast<uint8_t*>(ptr), std::memory_order_release);
+  return static_cast<int>(hipSuccess);
+}
+
+bool hipengine_gfx950::prefill_library_buffer_takes(int ggml_type, int64_t rows, int64_t in_features, int64_t out_features) {
+  if (rows < 32 || in_features <= 0 || (in_features % (ggml_type == GGML_Q8_0 ? 128 : QK_K)) != 0 || out_features <= 0 ||
+      out_features > (1 << 24) || ((ggml_type == GGML_Q4_K || ggml_type == GGML_Q5_K) && (out_features % 32) != 0)) {
+    return false;
   }
-  const int prc = hipengine_gguf_q8_1_d4s4_f32_quantize_bf16(x, workspace, rows, in_features, stream);
-  if (prc != static_cast<int>(hipSuccess)) return prc;
-  if (ggml_type == GGML_Q5_K) {
-    if ((out_features % 32) != 0) return static_cast<int>(hipErrorInvalidValue);
-    return launch_q5(workspace, qweight, out, out_kind, rows, in_features, out_features, stream);
+  const int64_t row_bytes = (in_features / 128) * (ggml_type == GGML_Q4_K ? DS4_BYTES : D4S4_BYTES);
+  const int64_t fit = kPackRegionBytes / row_bytes;
+  return fit >= kPackMinChunkRows || fit >= rows;
+}
+
+int hipengine_gfx950::prefill_bf16_library_buffer(int ggml_type, const void* x, const uint8_t* qweight, void* out, int out_kind,
+                                                  int64_t rows, int64_t in_features, int64_t out_features,
+                                                  hipStream_t stream) {
+  if (!prefill_library_buffer_takes(ggml_type, rows, in_features, out_features) ||
+      !prefill_shape_ok(ggml_type, x, qweight, out, out_kind, rows, in_features, out_features)) {
+    return static_cast<int>(hipErrorInvalidValue);
   }
-  if (ggml_type == GGML_Q8_0) return launch_q8_0(workspace, qweight, out, out_kind, rows, in_features, out_features, stream);
-  return launch_q6(workspace, qweight, out, out_kind, rows, in_features, out_features, stream);
+  int device = -1;
+  const hipError_t err = hipGetDevice(&device);
+  if (err != hipSuccess) return static_cast<int>(err);
+  if (device < 0 || device >= kPackMaxDevices) return static_cast<int>(hipErrorInvalidDevice);
+  if (!prefill_pack_ptr[device].load(std::memory_order_acquire)) {   // first call on this device without hipengine_gfx950_init()
+    const int rc = prefill_pack_setup(device);
+    if (rc != static_cast<int>(hipSuccess)) return rc;
+  }
+  uint8_t* region = prefill_pack_ptr[device].load(std::memory_order_acquire) +
+                    static_cast<int64_t>(prefill_next_region.fetch_add(1, std::memory_order_relaxed) % kPackRegions) * kPackRegionBytes;
+  const int64_t row_bytes = (in_features / 128) * (ggml_type == GGML_Q4_K ? DS4_BYTES : D4S4_BYTES);
+  int64_t chunk = kPackRegionBytes / row_bytes;
+  chunk = chunk < kPackChunkRows ? chunk : kPackChunkRows;
+  const int64_t out_elem = out_kind == KIND_F32 ? 4 : 2;
+  for (int64_t r0 = 0; r0 < rows; r0 += chunk) {
+    const int64_t n = rows - r0 < chunk ? rows - r0 : chunk;
+    const int rc = prefill_packed(ggml_type, static_cast<const uint16_t*>(x) + r0 * in_features, qweight,
+                                  static_cast<uint8_t*>(out) + r0 * out_features * out_elem, out_kind, n, in_features,
+                                  out_features, region, stream);
+    if (rc != static_cast<int>(hipSuccess)) return rc;
+  }
+  return static_cast<int>(hipSuccess);
 }
 
 int hipengine_gfx950::mmq_load() {

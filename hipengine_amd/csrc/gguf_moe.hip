@@ -1371,7 +1371,7 @@ template <int HK, int WK>
 __global__ void __launch_bounds__(64 * RL_WAVES) router_logits_kernel(const void* __restrict__ hidden,
                                                                       const void* __restrict__ weight,
                                                                       float* __restrict__ logits, int64_t tokens,
-                                                                      int64_t hidden_size, int64_t num_rows) {
+                                                                      int64_t hidden_size, int64_t num_rows, int64_t whole) {
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const int64_t row0 = (static_cast<int64_t>(blockIdx.x) * RL_WAVES + wave) * RL_ROWS;
   const int64_t tok0 = static_cast<int64_t>(blockIdx.y) * RL_TOKENS;
@@ -1381,7 +1381,7 @@ __global__ void __launch_bounds__(64 * RL_WAVES) router_logits_kernel(const void
   for (int t = 0; t < RL_TOKENS; ++t)
 #pragma unroll
     for (int r = 0; r < RL_ROWS; ++r) acc[t][r] = 0.0f;
-  const int64_t whole = hidden_size & ~static_cast<int64_t>(7);
+  // `whole`: the leading values of a row that go as 8-value pieces (16- and 32-byte loads); the rest one by one
   for (int64_t k = static_cast<int64_t>(lane) * 8; k < whole; k += 64 * 8) {
     float h[RL_TOKENS][8];
 #pragma unroll
@@ -1424,7 +1424,7 @@ template <int HK, int WK, int TT>
 __global__ void __launch_bounds__(64 * RL_WAVES) router_logits_decode_kernel(const void* __restrict__ hidden,
                                                                              const void* __restrict__ weight,
                                                                              float* __restrict__ logits, int64_t tokens,
-                                                                             int64_t hidden_size, int64_t num_rows) {
+                                                                             int64_t hidden_size, int64_t num_rows, int64_t whole) {
   __shared__ float part[RL_WAVES][TT][RL_ROWS];
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const int64_t row0 = static_cast<int64_t>(blockIdx.x) * RL_ROWS;
@@ -1434,7 +1434,6 @@ __global__ void __launch_bounds__(64 * RL_WAVES) router_logits_decode_kernel(con
   for (int t = 0; t < TT; ++t)
 #pragma unroll
     for (int r = 0; r < RL_ROWS; ++r) acc[t][r] = 0.0f;
-  const int64_t whole = hidden_size & ~static_cast<int64_t>(7);
   for (int64_t k = (static_cast<int64_t>(wave) * 64 + lane) * 8; k < whole; k += 64 * RL_WAVES * 8) {
     float h[TT][8];
 #pragma unroll
@@ -1553,25 +1552,28 @@ int launch_router_logits(const void* hidden, const void* weight, float* logits, 
   const int64_t h_item = HK == KIND_F32 ? 4 : 2, w_item = WK == KIND_F32 ? 4 : 2;
   if (!hidden || !weight || !logits || tokens <= 0 || tokens > (1 << 24) || hidden_size <= 0 || num_rows <= 0 ||
       num_rows > (1 << 24) || !(threads == 64 || threads == 128 || threads == 256 || threads == 512) ||
-      // the 16- and 32-byte loads: rows of 8-value pieces must start on their natural alignment
-      (hidden_size >= 8 && (((hidden_size * h_item) % 16) != 0 || ((hidden_size * w_item) % 16) != 0 ||
-                            (reinterpret_cast<uintptr_t>(hidden) & 15u) != 0 || (reinterpret_cast<uintptr_t>(weight) & 15u) != 0))) {
+      (reinterpret_cast<uintptr_t>(hidden) % h_item) != 0 || (reinterpret_cast<uintptr_t>(weight) % w_item) != 0) {
     return static_cast<int>(hipErrorInvalidValue);
   }
+  // the 16- and 32-byte loads want rows of 8-value pieces that start on their natural alignment; any other row
+  // length or base address goes value by value (hipEngine's kernel takes any hidden_size: moe/router.hip:1016-1024)
+  const bool vector_ok = ((hidden_size * h_item) % 16) == 0 && ((hidden_size * w_item) % 16) == 0 &&
+                         (reinterpret_cast<uintptr_t>(hidden) & 15u) == 0 && (reinterpret_cast<uintptr_t>(weight) & 15u) == 0;
+  const int64_t whole = vector_ok ? hidden_size & ~static_cast<int64_t>(7) : 0;
   if (tokens <= 8) {
     // one token, or groups of four tokens (eight tokens as one group measured 9.7 us against the 3 us of one token)
     const dim3 dgrid(static_cast<unsigned>((num_rows + RL_ROWS - 1) / RL_ROWS), tokens <= 4 ? 1u : 2u);
     if (tokens == 1) {
       hipLaunchKernelGGL((router_logits_decode_kernel<HK, WK, 1>), dgrid, dim3(64 * RL_WAVES), 0, stream, hidden, weight,
-                         logits, tokens, hidden_size, num_rows);
+                         logits, tokens, hidden_size, num_rows, whole);
     } else {
       hipLaunchKernelGGL((router_logits_decode_kernel<HK, WK, 4>), dgrid, dim3(64 * RL_WAVES), 0, stream, hidden, weight,
-                         logits, tokens, hidden_size, num_rows);
+                         logits, tokens, hidden_size, num_rows, whole);
     }
     return static_cast<int>(hipGetLastError());
   }
   if constexpr (HK == KIND_BF16 && (WK == KIND_F32 || WK == KIND_BF16)) {
-    if (tokens >= 32 && (hidden_size % 64) == 0) {
+    if (tokens >= 32 && (hidden_size % 64) == 0 && vector_ok) {
       const dim3 mgrid(static_cast<unsigned>((num_rows + 31) / 32), static_cast<unsigned>((tokens + 31) / 32));
       hipLaunchKernelGGL((router_logits_mfma_kernel<WK>), mgrid, dim3(256), 0, stream,
                          static_cast<const uint16_t*>(hidden), weight, logits, tokens, hidden_size, num_rows);
@@ -1581,7 +1583,7 @@ int launch_router_logits(const void* hidden, const void* weight, float* logits, 
   const dim3 grid(static_cast<unsigned>((num_rows + RL_WAVES * RL_ROWS - 1) / (RL_WAVES * RL_ROWS)),
                   static_cast<unsigned>((tokens + RL_TOKENS - 1) / RL_TOKENS));
   hipLaunchKernelGGL((router_logits_kernel<HK, WK>), grid, dim3(64 * RL_WAVES), 0, stream, hidden, weight, logits, tokens,
-                     hidden_size, num_rows);
+                     hidden_size, num_rows, whole);
   return static_cast<int>(hipGetLastError());
 }
 
@@ -2040,10 +2042,11 @@ extern "C" int hipengine_gguf_q4_k_selected_dual_q8_1_ds4_mmq32_prefill_compact3
     uint16_t* out, int64_t compact_rows, int64_t in_features, int64_t out_features_a, int64_t out_features_b,
     int64_t num_experts, int64_t mmq_total_rows, int64_t expert_stride_rows, hipStream_t stream) {
   if (!compact_to_source) return static_cast<int>(hipErrorInvalidValue);
-  // As in hipEngine, the activation rows are addressed through compact_to_source only; the
-  // source row count is not part of this signature, so the clamp is the compact row count.
+  // As in hipEngine, the activation rows are addressed through compact_to_source only and the source row count is
+  // not part of this signature: no upper clamp (lanes dropped from the index can leave fewer compact rows than
+  // there are tokens, and a clamp to the compact row count would then redirect the last tokens).
   return launch_moe_mmq<MoeQ4>(x_q8, compact_to_source, expert_start_compact, expert_start_mmq32, tile_expert, qweight_a,
-                        qweight_b, out, KIND_BF16, compact_rows, compact_rows, in_features, out_features_a,
+                        qweight_b, out, KIND_BF16, compact_rows, 1 << 24, in_features, out_features_a,
                         out_features_b, num_experts, mmq_total_rows, expert_stride_rows, stream);
 }
 

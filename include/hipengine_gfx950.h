@@ -48,11 +48,14 @@ typedef struct ihipStream_t* hipengine_stream_t; /* == hipStream_t */
 int hipengine_gfx950_abi_version(void);
 
 /* Per-device set-up, for the device that is current: raises the dynamic-LDS limit of every kernel
- * that may need more than the default 64 KB and looks up the address of the library-held scratch of
- * hipengine_gfx950_argmax_f32_rows_i32_noalloc.  Call it once per device after loading the library
- * and before capturing a HIP graph; after it, no entry point makes any call that is not a stream
- * operation, so every one of them can be captured from its first launch on.  Entry points that need
- * the set-up run it themselves when it has not been done (then outside of a capture, please).
+ * that may need more than the default 64 KB and looks up the addresses of the device arrays the
+ * library holds (the scratch of hipengine_gfx950_argmax_f32_rows_i32_noalloc, the pack buffer of the
+ * dense prefill entries, the partial sums of the split-K decode GEMV).  Call it once per device after
+ * loading the library and before capturing a HIP graph; after it, no entry point makes any call that
+ * is not a stream operation, so every one of them can be captured from its first launch on - except
+ * the verification exports (hipengine_gfx950_gguf_gemv_mfma_dots_i32), which set a kernel attribute
+ * on every call and are not meant for graphs.  Entry points that need the set-up run it themselves
+ * when it has not been done (then outside of a capture, please).
  * Allocates nothing; safe to call again and from several threads.  New here. */
 int hipengine_gfx950_init(void);
 
@@ -489,6 +492,11 @@ int hipengine_qwen35_router_logits_f32_f32w(const void* hidden, const void* weig
  * selected[tokens*top_k], and the softmax over those top_k logits into
  * routing[tokens*top_k].  top_k <= 16, num_experts <= 1024; `threads` in {64,128,256,512}
  * is accepted and ignored.
+ * Deviation on exact ties only: hipEngine's kernel strides the experts over `threads` threads and keeps
+ * the first maximum a thread meets, then the first over threads; with num_experts > threads two equal
+ * logits can there resolve to the higher index (expert 259 on thread 3 before expert 5 on thread 5 at
+ * 256 threads).  Here equal logits always go to the lowest index, whatever `threads` is; with
+ * num_experts <= threads the two orders are the same.
  * Replaces hipengine_qwen35_router_select (kernels/hip_gfx1100/moe/router.hip:1284-1311,
  * device function :628-715). */
 int hipengine_qwen35_router_select(const float* logits, int64_t* selected, float* routing, int64_t tokens,

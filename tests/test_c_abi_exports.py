@@ -86,3 +86,22 @@ def test_abi_version_and_host_only_entry_points(library):
     assert ps(14, 16, 0, 16, 16, 0, 8, 256 * 17, 5120, 0, 0, 0, None) == 1    # odd block count: not this form
     assert ps(14, 16, 0, 18, 16, 0, 8, 5120, 5120, 0, 0, 0, None) == 1        # weights not 4-byte aligned
     assert ps(14, 16, 0, 16, 16, 0, 8, 5120, 5120, 13, 1, 0, None) == 1       # more than 12 waves
+    ds = library.hipengine_gfx950_gguf_q8_1_fused_gemv_dslab_tuned
+    ds.argtypes = [ctypes.c_int32, ctypes.c_void_p, ctypes.c_int32, ctypes.c_void_p, ctypes.c_void_p, ctypes.c_int32,
+                   ctypes.c_int64, ctypes.c_int64, ctypes.c_int64, ctypes.c_int32, ctypes.c_int32, ctypes.c_int32,
+                   ctypes.c_int32, ctypes.c_void_p]
+    assert ds(14, None, 0, None, None, 0, 8, 5120, 5120, 0, 0, 0, 0, None) == 1
+    assert ds(13, 16, 0, 16, 16, 0, 8, 5120, 5120, 0, 0, 0, 0, None) == 1      # Q5_K: not this form
+    assert ds(14, 16, 0, 16, 16, 0, 8, 5120, 5120, 0, 0, 0, 3, None) == 1      # K parts: 1, 2 or 4
+    assert ds(14, 16, 0, 17, 16, 0, 8, 5120, 5120, 0, 0, 0, 0, None) == 1      # weights not 2-byte aligned
+    # the one-call prefill refuses what its MMQ would refuse before it packs anything: nothing is enqueued or written
+    pf = library.hipengine_gfx950_gguf_prefill_bf16
+    pf.argtypes = [ctypes.c_int32, ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p, ctypes.c_int32, ctypes.c_int64,
+                   ctypes.c_int64, ctypes.c_int64, ctypes.c_void_p, ctypes.c_int64, ctypes.c_void_p]
+    big = 1 << 30
+    assert pf(12, 16, 16, 16, 0, 64, 1024, 33, 16, big, None) == 1             # Q4_K: out_features % 32
+    assert pf(13, 16, 16, 16, 0, 64, 1024, 40, 16, big, None) == 1             # Q5_K likewise
+    assert pf(14, 16, None, 16, 0, 64, 1024, 40, 16, big, None) == 1           # no weights
+    assert pf(14, 16, 16, None, 0, 64, 1024, 40, 16, big, None) == 1           # no output
+    assert pf(14, 16, 16, 16, 7, 64, 1024, 40, 16, big, None) == 1             # output kind
+    assert pf(8, 16, 16, 16, 0, 64, 1024, (1 << 24) + 1, 16, big, None) == 1   # out_features out of range

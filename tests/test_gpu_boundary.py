@@ -110,9 +110,10 @@ def test_rowtile_keys_are_the_batch_launch(dev, quant):
 
 @pytest.mark.parametrize("quant,n", [("gguf_q4_k", 352), ("gguf_q6_k", 333), ("gguf_q5_k", 160), ("gguf_q8_0", 75)])
 def test_prefill_key_with_workspace_runs_the_mmq(dev, quant, n):
-    """prefill_bf16_f32_out with 32 rows or more and a caller-owned workspace packs the activations and runs the
-    int8-MFMA MMQ: results equal the MMQ formula of the oracle, and agree with the workspace-free route (GEMV in
-    batches of 8, GEMV-convention q8_1) to the tolerance both share against the reference CPU GEMV."""
+    """prefill_bf16_f32_out with 32 rows or more packs the activations and runs the int8-MFMA MMQ, into a
+    caller-owned workspace or - called the way hipEngine's dispatcher calls it, positionally and with no workspace -
+    into the pack buffer the library holds: the same bits either way, equal to the MMQ formula of the oracle.  Below
+    32 rows the key runs the GEMV in batches of 8 (GEMV-convention q8_1)."""
     rows, k = 70, 1024
     rng = np.random.default_rng(3)
     xb = O.f32_to_bf16_bits((rng.standard_normal((rows, k)) * 0.25).astype(np.float32))
@@ -124,10 +125,14 @@ def test_prefill_key_with_workspace_runs_the_mmq(dev, quant, n):
     dx, dw = dev.put(xb), dev.put(w)
     dws, d1, d2 = dev.empty(need), dev.empty(rows * n * 4), dev.empty(rows * n * 4)
     fn(dx.ptr, dw.ptr, d1.ptr, rows, k, n, stream=0, runtime=dev.runtime, workspace_ptr=dws.ptr, workspace_bytes=need)
-    fn(dx.ptr, dw.ptr, d2.ptr, rows, k, n, stream=0, runtime=dev.runtime)
+    fn(dx.ptr, dw.ptr, d2.ptr, rows, k, n)
+    few = 20
+    d3 = dev.empty(few * n * 4)
+    fn(dx.ptr, dw.ptr, d3.ptr, few, k, n)
     with_ws, without = dev.get(d1, np.float32, (rows, n)).copy(), dev.get(d2, np.float32, (rows, n)).copy()
+    short = dev.get(d3, np.float32, (few, n)).copy()
     packed = dev.get(dws, np.uint8, (rows, k // 128, need // rows // (k // 128)))
-    dev.free(dx, dw, dws, d1, d2)
+    dev.free(dx, dw, dws, d1, d2, d3)
     if quant == "gguf_q4_k":
         want_pack = O.pack_q8_1_ds4(xb)
         ref = O.mmq_q4_k_ds4(want_pack, w)
@@ -142,8 +147,38 @@ def test_prefill_key_with_workspace_runs_the_mmq(dev, quant, n):
         ref = O.mmq_q6_k_d4s4(want_pack, w)
     assert np.array_equal(packed.reshape(want_pack.shape), want_pack)
     _close(with_ws, ref)
-    _close(without, O.gguf_quant_gemv(O.dequantize_q8_1(O.quantize_q8_1(O.bf16_bits_to_f32(xb))), w, QT[quant]))
-    assert O.cosine(with_ws, without) >= 0.9999
+    assert np.array_equal(with_ws.view(np.uint32), without.view(np.uint32))
+    _close(short, O.gguf_quant_gemv(O.dequantize_q8_1(O.quantize_q8_1(O.bf16_bits_to_f32(xb[:few]))), w, QT[quant]))
+    assert O.cosine(with_ws[:few], short) >= 0.9999
+
+
+@pytest.mark.parametrize("quant,k,n,rows", [("gguf_q4_k", 5120, 1024, 2048), ("gguf_q6_k", 17408, 256, 1100), ("gguf_q8_0", 1024, 77, 560)])
+def test_prefill_key_chunks_through_the_library_buffer(dev, quant, k, n, rows):
+    """More rows than one chunk of the library's pack buffer holds (512): every chunk's rows equal the MMQ of the same
+    rows run on their own, bit for bit, and two calls in a row (which take the two regions of the buffer in turn) agree."""
+    rng = np.random.default_rng(rows)
+    xb = O.f32_to_bf16_bits((rng.standard_normal((rows, k)) * 0.25).astype(np.float32))
+    w = O.random_weight(QT[quant], n, k, seed=6)
+    fn = _resolve("linear", quant, "prefill_bf16_bf16_out")
+    dx, dw = dev.put(xb), dev.put(w)
+    d1, d2 = dev.empty(rows * n * 2), dev.empty(rows * n * 2)
+    fn(dx.ptr, dw.ptr, d1.ptr, rows, k, n)
+    fn(dx.ptr, dw.ptr, d2.ptr, rows, k, n)
+    a, b = dev.get(d1, np.uint16, (rows, n)).copy(), dev.get(d2, np.uint16, (rows, n)).copy()
+    assert np.array_equal(a, b)
+    # the last, ragged chunk on its own through a caller-owned workspace
+    r0 = (rows // 512) * 512 if rows % 512 else rows - 512
+    tail = rows - r0
+    need = G.gguf_prefill_workspace_bytes(quant, tail, k)
+    dws, d3 = dev.empty(need), dev.empty(tail * n * 2)
+    dxt = dev.put(xb[r0:])
+    fn(dxt.ptr, dw.ptr, d3.ptr, tail, k, n, workspace_ptr=dws.ptr, workspace_bytes=need)
+    c = dev.get(d3, np.uint16, (tail, n)).copy()
+    dev.free(dx, dw, d1, d2, dws, d3, dxt)
+    assert np.array_equal(a[r0:], c)
+    pack = O.pack_q8_1_ds4(xb[:64]) if quant == "gguf_q4_k" else O.pack_q8_1_d4s4(xb[:64])
+    ref = {"gguf_q4_k": O.mmq_q4_k_ds4, "gguf_q6_k": O.mmq_q6_k_d4s4, "gguf_q8_0": O.mmq_q8_0_d4s4}[quant](pack, w)
+    assert np.allclose(O.bf16_bits_to_f32(a[:64]), ref, rtol=2.0 ** -8, atol=1e-3 * np.abs(ref).max())
 
 
 @pytest.mark.parametrize("quant", ["gguf_q4_k", "gguf_q6_k", "gguf_q8_0"])

@@ -8,6 +8,10 @@ run of the same chain (hipEngine replays decode graphs in production: core/hip.p
 
 from __future__ import annotations
 
+import subprocess
+import sys
+from pathlib import Path
+
 import numpy as np
 import pytest
 
@@ -190,3 +194,20 @@ def test_moe_block_graph_replays_and_matches_cpu(dev):
     rt.graph_destroy(graph)
     rt.stream_destroy(stream)
     dev.free(*bufs.values())
+
+
+def test_graphs_capture_cold_in_a_fresh_process():
+    """The captures above run after other tests of the same process have launched, and so set up, the same
+    kernels.  Here a child process loads the library (whose per-device set-up is all the set-up there is) and
+    captures as its very first launches: a kernel missing from that set-up would fail the capture."""
+    code = ("from tests._device import Device\n"
+            "import tests.test_gpu_graph as t\n"
+            "d = Device()\n"
+            "t.test_decode_step_graph_replays_match_eager(d, 8)\n"
+            "t.test_moe_block_graph_replays_and_matches_cpu(d)\n"
+            "d2 = Device()\n"
+            "t.test_decode_step_graph_replays_match_eager(d2, 2)\n"
+            "print('COLD_CAPTURE_OK')\n")
+    root = Path(__file__).resolve().parents[1]
+    proc = subprocess.run([sys.executable, "-c", code], cwd=root, capture_output=True, text=True, timeout=600)
+    assert proc.returncode == 0 and "COLD_CAPTURE_OK" in proc.stdout, proc.stdout[-2000:] + proc.stderr[-4000:]

@@ -40,6 +40,13 @@ def _routing(seed, tokens, top_k, num_experts, bad=False):
     return sel, w
 
 
+def _routing_from_logits(seed, tokens, top_k, num_experts):
+    """Routing as the MoE benchmark configuration states it: router logits ~ N(0, 1), top-k of them, softmax
+    over the selected logits (the device router's arithmetic, moe/router.hip:628-715)."""
+    logits = np.random.default_rng(seed).standard_normal((tokens, num_experts)).astype(np.float32)
+    return O.router_topk_softmax(logits, top_k)
+
+
 def _device_index(dev, sel, w, num_experts, tile_capacity=0):
     """Runs compact_active_source_rows + mmq32_tile_map + lane_to_compact; returns host copies and device buffers."""
     tokens, top_k = sel.shape
@@ -153,14 +160,12 @@ def test_routing_index_other_entry_names(dev, tokens, top_k, experts, bad):
 
 
 @pytest.mark.parametrize("tokens,hidden,rows", [(1, 2048, 256), (9, 2048, 257), (130, 512, 60), (3, 20, 5), (7, 1024, 64),
-                                                (300, 2048, 256), (33, 192, 40), (64, 1000, 33)])
+                                                (300, 2048, 256), (33, 192, 40), (64, 1000, 33), (40, 77, 19), (2, 3, 9)])
 @pytest.mark.parametrize("name,hk,wk", [("bf16", "bf16", "bf16"), ("fp16", "fp16", "fp16"), ("bf16_f32w", "bf16", "f32"),
                                         ("fp16_f32w", "fp16", "f32"), ("f32_f32w", "f32", "f32")])
 def test_router_logits(dev, name, hk, wk, tokens, hidden, rows):
     """Router logits against the float32 matmul of the reference on the same (rounded) values: float32 rounding apart
     (another summation order); then the selection of the device logits is the oracle's selection of those logits."""
-    if hidden % 8 and (hk != "f32" or wk != "f32") and (hidden * 2) % 16:
-        pytest.skip("16-bit rows shorter than their alignment")
     rng = np.random.default_rng(tokens + hidden + rows)
     x = (rng.standard_normal((tokens, hidden)) * 0.5).astype(np.float32)
     w = (rng.standard_normal((rows, hidden)) * 0.05).astype(np.float32)
@@ -597,12 +602,45 @@ def test_grouped_mmq_bf16_named_entry(dev):
     assert np.array_equal(wide, b16)              # hipEngine's 32 x 128 variant name: the same GEMM
 
 
+def test_grouped_mmq_named_entry_with_mostly_dropped_lanes(dev):
+    """Most lanes name no expert, so there are fewer compact rows than tokens: under hipEngine's name (which has
+    no source row count) the last tokens' rows must still be the ones their compact_to_source entries name."""
+    tokens, top_k, experts, k, na, nb = 64, 2, 4, 512, 64, 32
+    rng = np.random.default_rng(41)
+    sel = np.full((tokens, top_k), -1, dtype=np.int64)
+    keep = [3, 17, 40, 58, 61, 63]                       # 6 tokens keep one lane each: 6 compact rows, source rows up to 63
+    for i, t in enumerate(keep):
+        sel[t, i % top_k] = i % experts
+    wts = np.full((tokens, top_k), 0.5, dtype=np.float32)
+    host, d = _device_index(dev, sel, wts, experts)
+    total = host["total"]
+    assert total == len(keep) and int(host["c2s"][:total].max()) >= total
+    x = (rng.standard_normal((tokens, k)) * 0.2).astype(np.float32)
+    ds4 = O.pack_q8_1_ds4(O.f32_to_bf16_bits(x))
+    w_a, w_b = _experts(O.GGML_Q4_K, experts, na, k, seed=23), _experts(O.GGML_Q4_K, experts, nb, k, seed=24)
+    dxq, dwa, dwb = dev.put(ds4), dev.put(w_a), dev.put(w_b)
+    dout = dev.empty(total * (na + nb) * 2, fill=0)
+    M.gguf_q4_k_selected_dual_q8_1_ds4_mmq32_prefill_compact32_bf16_bf16_out(
+        dxq.ptr, d["c2s"].ptr, d["expert_start"].ptr, d["mmq_start"].ptr, d["tile_expert"].ptr, dwa.ptr, dwb.ptr,
+        dout.ptr, total, k, na, nb, experts, host["mmq_total"])
+    got = O.bf16_bits_to_f32(dev.get(dout, np.uint16, (total, na + nb)).copy())
+    dev.free(dxq, dwa, dwb, dout, *d.values())
+    es = host["expert_start"]
+    for e in range(experts):
+        lo, hi = int(es[e]), int(es[e + 1])
+        if hi > lo:
+            src = host["c2s"][lo:hi]
+            want = np.concatenate([O.mmq_q4_k_ds4(ds4[src], w_a[e]), O.mmq_q4_k_ds4(ds4[src], w_b[e])], axis=1)
+            assert np.array_equal(O.f32_to_bf16_bits(got[lo:hi]), O.f32_to_bf16_bits(O.bf16_bits_to_f32(O.f32_to_bf16_bits(want)))) or \
+                O.max_rel_err(got[lo:hi], want, floor_frac=1e-2) <= 2.0 ** -7
+
+
 @pytest.mark.parametrize("tokens,experts", [(256, 32), (2048, 256)])
 def test_prefill_chain_matches_cpu_moe(dev, tokens, experts):
     """index -> DS4 pack -> grouped gate|up MMQ -> SiLU*up -> DS4 pack -> grouped down MMQ ->
     ordered weighted gather, against the reference CPU MoE FFN on a token subsample."""
     top_k, hidden, inter = 8, 2048, 512
-    sel, wts = _routing(77, tokens, top_k, experts)
+    sel, wts = _routing_from_logits(77, tokens, top_k, experts)
     host, d = _device_index(dev, sel, wts, experts)
     total, lanes = host["total"], tokens * top_k
     wg = _experts(O.GGML_Q4_K, experts, inter, hidden, seed=1)
@@ -635,12 +673,22 @@ def test_prefill_chain_matches_cpu_moe(dev, tokens, experts):
     mid = O.bf16_bits_to_f32(mid_bits)
     down = dev.get(ddown, np.float32, (total, hidden))
     dev.free(dxb, dg, du, dd, dxq, dgu, dmid, dmq, ddown, dout, *d.values())
+    # gate|up stage: the MMQ formula on the packed activations of each expert's rows, every fifth expert
+    x_ds4 = O.pack_q8_1_ds4(xb)
+    es, c2s = host["expert_start"], host["c2s"]
+    for e in range(0, experts, 5):
+        lo, hi = int(es[e]), int(es[e + 1])
+        if hi > lo:
+            rows_e = x_ds4[c2s[lo:hi]]
+            for half, we in ((0, wg[e]), (1, wu[e])):
+                want_gu = O.mmq_q4_k_ds4(rows_e, we)
+                got_gu = gu[lo:hi, half * inter:(half + 1) * inter]
+                assert O.max_rel_err(got_gu, want_gu) <= REL_TOL and O.cosine(got_gu, want_gu) >= COS_MIN
     # elementwise stage: bf16(silu(gate)*up) of the device's own gate|up
     want_mid = O.bf16_bits_to_f32(O.f32_to_bf16_bits((O.silu(gu[:, :inter]) * gu[:, inter:]).astype(np.float32)))
     assert O.max_rel_err(mid, want_mid, floor_frac=1e-2) <= 1e-2
     # down stage: the MMQ formula on the device's own intermediate, expert by expert
     mid_ds4 = O.pack_q8_1_ds4(mid_bits)
-    es = host["expert_start"]
     for e in range(0, experts, 5):
         lo, hi = int(es[e]), int(es[e + 1])
         if hi > lo:
