@@ -231,6 +231,48 @@ GemvForm pick_form(int qt, int& chunk, int64_t K, int64_t N, const void* w) {
   return FORM_ROW_STRIDED;
 }
 
+// What the default dispatch does with a batch of `rows` <= 8 rows of a shape: the form, the rows of the first
+// launch and that form's plan.  Planning walks variant tables and LDS budgets (about a microsecond of host time);
+// a decode loop asks for the same few shapes over and over, so each thread remembers the last ones.
+struct Choice {
+  int qt, rows, walign;
+  int64_t K, N;
+  GemvForm form;
+  int chunk;
+  SlabPlan slab;
+  PslabPlan pslab;
+  StreamPlan stream;
+  RunPlan run;
+  DslabPlan dslab;
+};
+
+const Choice& choose(int qt, int rows, int64_t K, int64_t N, const void* w) {
+  constexpr int kRemembered = 8;
+  thread_local Choice memo[kRemembered];
+  thread_local int used = 0, next = 0;
+  const int walign = static_cast<int>(reinterpret_cast<uintptr_t>(w) & 3u);
+  for (int i = 0; i < used; ++i) {
+    const Choice& c = memo[i];
+    if (c.qt == qt && c.rows == rows && c.K == K && c.N == N && c.walign == walign) return c;
+  }
+  Choice& c = memo[next];
+  next = (next + 1) % kRemembered;
+  used = used < kRemembered ? used + 1 : used;
+  c = Choice{};
+  c.qt = qt; c.rows = rows; c.walign = walign; c.K = K; c.N = N;
+  c.chunk = rows;
+  c.form = pick_form(qt, c.chunk, K, N, w);
+  switch (c.form) {
+    case FORM_DSLAB: c.dslab = default_dslab_plan(qt, c.chunk, K, N, w); break;
+    case FORM_SLAB: c.slab = default_slab_plan(qt, c.chunk, K, N); break;
+    case FORM_PSLAB: c.pslab = default_pslab_plan(qt, c.chunk, K, N, w); break;
+    case FORM_STREAM: c.stream = default_stream_plan(qt, c.chunk, K, N); break;
+    case FORM_RUN: c.run = default_run_plan(qt, c.chunk, K, N); break;
+    default: break;
+  }
+  return c;
+}
+
 int launch_gemv(int qt, const void* x, int x_kind, const uint8_t* w, void* out, int out_kind, int64_t rows, int64_t K,
                 int64_t N, const Plan* forced, hipStream_t stream) {
   if (!x || !w || !out || rows <= 0 || K <= 0 || N <= 0 || (K % QK_K) != 0 || K > (1 << 24) || N > (1 << 30)) {
@@ -240,24 +282,24 @@ int launch_gemv(int qt, const void* x, int x_kind, const uint8_t* w, void* out, 
   const int64_t out_elem = out_kind == KIND_F32 ? 4 : 2;
   for (int64_t r0 = 0; r0 < rows;) {
     int chunk = static_cast<int>(rows - r0 < 8 ? rows - r0 : 8);
-    const GemvForm form = forced ? FORM_ROW_STRIDED : pick_form(qt, chunk, K, N, w);
+    const Choice* ch = forced ? nullptr : &choose(qt, chunk, K, N, w);
+    const GemvForm form = forced ? FORM_ROW_STRIDED : ch->form;
+    if (ch) chunk = ch->chunk;
     const int64_t next_r0 = r0 + chunk;
     const void* xr = static_cast<const uint8_t*>(x) + r0 * x_row_bytes;
     void* outr = static_cast<uint8_t*>(out) + r0 * N * out_elem;
     if (form != FORM_ROW_STRIDED) {
       int rc;
       if (form == FORM_DSLAB) {
-        rc = launch_gemv_dslab(qt, xr, x_kind, w, outr, out_kind, chunk, K, N, default_dslab_plan(qt, chunk, K, N, w), stream);
+        rc = launch_gemv_dslab(qt, xr, x_kind, w, outr, out_kind, chunk, K, N, ch->dslab, stream);
       } else if (form == FORM_SLAB) {
-        rc = launch_gemv_slab(xr, x_kind, w, outr, out_kind, chunk, K, N, default_slab_plan(qt, chunk, K, N), stream);
+        rc = launch_gemv_slab(xr, x_kind, w, outr, out_kind, chunk, K, N, ch->slab, stream);
       } else if (form == FORM_PSLAB) {
-        rc = launch_gemv_pslab(qt, xr, x_kind, w, outr, out_kind, chunk, K, N, default_pslab_plan(qt, chunk, K, N, w),
-                               stream);
+        rc = launch_gemv_pslab(qt, xr, x_kind, w, outr, out_kind, chunk, K, N, ch->pslab, stream);
       } else if (form == FORM_STREAM) {
-        rc = launch_gemv_stream(qt, xr, x_kind, w, outr, out_kind, chunk, K, N, default_stream_plan(qt, chunk, K, N),
-                                stream);
+        rc = launch_gemv_stream(qt, xr, x_kind, w, outr, out_kind, chunk, K, N, ch->stream, stream);
       } else {
-        rc = launch_gemv_run(qt, xr, x_kind, w, outr, out_kind, chunk, K, N, default_run_plan(qt, chunk, K, N), stream);
+        rc = launch_gemv_run(qt, xr, x_kind, w, outr, out_kind, chunk, K, N, ch->run, stream);
       }
       if (rc != static_cast<int>(hipSuccess)) return rc;
       r0 = next_r0;

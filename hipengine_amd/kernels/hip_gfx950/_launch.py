@@ -39,6 +39,24 @@ def entry(symbol: str, argtypes: list, library: ctypes.CDLL | None = None):
     return fn
 
 
+# Argument validation in the Python wrappers (range and null-pointer checks that raise ValueError, as hipEngine's
+# wrappers do).  A caller that has validated its shapes once and launches in a loop may switch it off: the C
+# entry points check their arguments as well and return hipErrorInvalidValue.
+VALIDATE = True
+
+
+def set_validation(enabled: bool) -> None:
+    global VALIDATE
+    VALIDATE = bool(enabled)
+
+
+def lean_entry(symbol: str, argtypes: list, library: ctypes.CDLL | None = None):
+    """The configured C function itself (``argtypes`` set once, hipEngine's ``_cached_fn``:
+    ``kernels/hip_gfx1100/quant/gguf_k_gemv.py:15-32``): called positionally with the C signature, it costs
+    one ctypes call; the caller tests the returned ``hipError_t`` (0 is success)."""
+    return entry(symbol, argtypes, library)
+
+
 def check_launch(code: int, runtime: HipRuntime | None) -> None:
     if int(code) == HIP_SUCCESS:
         return

@@ -34,6 +34,7 @@ from hipengine_amd.kernels.hip_gfx950._launch import (
     validate_linear,
     validate_pointers,
 )
+from hipengine_amd.kernels.hip_gfx950 import _launch
 from hipengine_amd.kernels.registry import KernelKey, register
 
 _FUSED_ARGS = [VOID, VOID, VOID, I64, I64, I64, I64, VOID]
@@ -46,14 +47,23 @@ _KINDS = {"f32": KIND_F32, "bf16": KIND_BF16, "fp16": KIND_F16, "q8_1": KIND_Q8_
 def _make_fused(quant: str, act: str, out: str):
     symbol = f"hipengine_gguf_{quant}_q8_1_fused_gemv_{act}_{out}_out"
 
+    default_fn = []          # the configured C function of the default library, resolved at the first call
+
     def wrapper(x_ptr: int, qweight_ptr: int, out_ptr: int, rows: int, in_features: int, out_features: int, *,
                 threads: int = 128, stream: int = 0, library: ctypes.CDLL | None = None,
                 runtime: HipRuntime | None = None) -> None:
-        validate_linear(rows, in_features, out_features, threads)
-        validate_pointers(x_ptr=x_ptr, qweight_ptr=qweight_ptr, out_ptr=out_ptr)
-        code = entry(symbol, _FUSED_ARGS, library)(x_ptr, qweight_ptr, out_ptr, rows, in_features, out_features,
-                                                   threads, stream)
-        check_launch(code, runtime)
+        if _launch.VALIDATE:
+            validate_linear(rows, in_features, out_features, threads)
+            validate_pointers(x_ptr=x_ptr, qweight_ptr=qweight_ptr, out_ptr=out_ptr)
+        if library is None:
+            if not default_fn:
+                default_fn.append(entry(symbol, _FUSED_ARGS, None))
+            fn = default_fn[0]
+        else:
+            fn = entry(symbol, _FUSED_ARGS, library)
+        code = fn(x_ptr, qweight_ptr, out_ptr, rows, in_features, out_features, threads, stream)
+        if code:
+            check_launch(code, runtime)
 
     wrapper.__name__ = f"gguf_{quant}_q8_1_fused_gemv_{act}_{out}_out"
     wrapper.__doc__ = (f"GGUF {quant.upper()} GEMV, {act} activations quantized to q8_1 in the kernel, {out} output "
@@ -152,6 +162,13 @@ for _q in _QUANTS:       # hipEngine's rowtile names (gguf_q4_k_gemv.py:1517-151
 DENSE_DUAL = {(q, a, o): _make_dense_dual(q, a, o) for q in _QUANTS for a, o in (("f32", "f32"), ("bf16", "bf16"))}
 for _fn in DENSE_DUAL.values():
     globals()[_fn.__name__] = _fn
+
+def lean_fused(quant: str, act: str, out: str, library: ctypes.CDLL | None = None):
+    """The C function behind ``FUSED[(quant, act, out)]`` with its argument types set: call it as
+    ``fn(x_ptr, qweight_ptr, out_ptr, rows, in_features, out_features, threads, stream)`` and test the returned
+    ``hipError_t``.  For loops that have validated their shapes once (one ctypes call per launch)."""
+    return _launch.lean_entry(f"hipengine_gguf_{quant}_q8_1_fused_gemv_{act}_{out}_out", _FUSED_ARGS, library)
+
 
 FUSED: dict[tuple[str, str, str], object] = {}
 for _q in _QUANTS:
