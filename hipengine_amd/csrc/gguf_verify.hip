@@ -106,19 +106,40 @@ __global__ void __launch_bounds__(1024) read_probe_kernel(const uint4* __restric
 
 }  // namespace
 
+static int read_probe_launch(const void* src, int64_t bytes, int32_t waves_per_workgroup, int32_t loads_in_flight,
+                             int32_t workgroups, void* sink, hipStream_t stream);
+
 extern "C" int hipengine_gfx950_read_probe(const void* src, int64_t bytes, int32_t waves_per_workgroup,
                                            int32_t loads_in_flight, void* sink, hipStream_t stream) {
+  if (loads_in_flight == 1) return static_cast<int>(hipErrorInvalidValue);
+  return read_probe_launch(src, bytes, waves_per_workgroup, loads_in_flight, 256, sink, stream);
+}
+
+// The same probe over `workgroups` workgroups instead of one per CU: with thousands of them a wave reads one or
+// two pieces and leaves, the geometry of a launch that is not persistent.  loads_in_flight may be 1 here.
+extern "C" int hipengine_gfx950_read_probe_grid(const void* src, int64_t bytes, int32_t waves_per_workgroup,
+                                                int32_t loads_in_flight, int32_t workgroups, void* sink,
+                                                hipStream_t stream) {
+  if (workgroups < 1 || workgroups > (1 << 20)) return static_cast<int>(hipErrorInvalidValue);
+  return read_probe_launch(src, bytes, waves_per_workgroup, loads_in_flight, workgroups, sink, stream);
+}
+
+static int read_probe_launch(const void* src, int64_t bytes, int32_t waves_per_workgroup, int32_t loads_in_flight,
+                             int32_t workgroups, void* sink, hipStream_t stream) {
   if (!src || (reinterpret_cast<uintptr_t>(src) & 15) != 0 || bytes < 1024 || waves_per_workgroup < 1 || waves_per_workgroup > 16 ||
-      (loads_in_flight != 2 && loads_in_flight != 4)) {
+      (loads_in_flight != 1 && loads_in_flight != 2 && loads_in_flight != 4)) {
     return static_cast<int>(hipErrorInvalidValue);
   }
   const int64_t pieces = bytes / 1024;            // whole 1 KB pieces: every load stays inside [src, src + bytes)
-  const int grid = 256;
+  const int grid = workgroups;
   const int64_t waves_total = static_cast<int64_t>(grid) * waves_per_workgroup;
   const int64_t rounds64 = (pieces + waves_total - 1) / waves_total;
   if (rounds64 > (1 << 28)) return static_cast<int>(hipErrorInvalidValue);
   const int rounds = static_cast<int>(rounds64);
-  if (loads_in_flight == 2) {
+  if (loads_in_flight == 1) {
+    hipLaunchKernelGGL(read_probe_kernel<1>, dim3(grid), dim3(waves_per_workgroup * 64), 0, stream,
+                       static_cast<const uint4*>(src), pieces, rounds, static_cast<uint32_t*>(sink));
+  } else if (loads_in_flight == 2) {
     hipLaunchKernelGGL(read_probe_kernel<2>, dim3(grid), dim3(waves_per_workgroup * 64), 0, stream,
                        static_cast<const uint4*>(src), pieces, rounds, static_cast<uint32_t*>(sink));
   } else {

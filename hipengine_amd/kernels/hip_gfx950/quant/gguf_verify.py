@@ -87,6 +87,18 @@ def read_probe(src_ptr: int, nbytes: int, *, waves_per_workgroup: int = 8, loads
     check_launch(fn(src_ptr, nbytes, waves_per_workgroup, loads_in_flight, sink_ptr or None, stream), runtime)
 
 
+def read_probe_grid(src_ptr: int, nbytes: int, workgroups: int, *, waves_per_workgroup: int = 4, loads_in_flight: int = 1,
+                    sink_ptr: int = 0, stream: int = 0, library: ctypes.CDLL | None = None,
+                    runtime: HipRuntime | None = None) -> None:
+    """The read-only pass over ``workgroups`` workgroups instead of one per CU (thousands of them: waves that read a
+    piece or two and leave; C symbol ``hipengine_gfx950_read_probe_grid``)."""
+    if nbytes < 1024 or workgroups < 1:
+        raise ValueError("nbytes must be at least 1024 and workgroups positive")
+    validate_pointers(src_ptr=src_ptr)
+    fn = entry("hipengine_gfx950_read_probe_grid", [VOID, I64, I32, I32, I32, VOID, VOID], library)
+    check_launch(fn(src_ptr, nbytes, waves_per_workgroup, loads_in_flight, workgroups, sink_ptr or None, stream), runtime)
+
+
 def copy_bytes(src_ptr: int, dst_ptr: int, nbytes: int, *, stream: int = 0, library: ctypes.CDLL | None = None,
                runtime: HipRuntime | None = None) -> None:
     """Plain device copy kernel of a known size (calibration of HBM byte counters)."""

@@ -110,6 +110,13 @@ int hipengine_gfx950_gguf_q4_k_mmq_tuned(const void* xq, const uint8_t* qweight,
 int hipengine_gfx950_read_probe(const void* src, int64_t bytes, int32_t waves_per_workgroup, int32_t loads_in_flight,
                                 void* sink, hipengine_stream_t stream);
 
+/* The same read-only pass over `workgroups` workgroups instead of one per CU (loads_in_flight 1, 2 or 4): with
+ * thousands of workgroups every wave reads one or two pieces and leaves - the geometry of a launch that is
+ * not persistent - so that the read ceilings quoted for this part do not rest on one launch shape.  Measurement
+ * only.  New here. */
+int hipengine_gfx950_read_probe_grid(const void* src, int64_t bytes, int32_t waves_per_workgroup, int32_t loads_in_flight,
+                                     int32_t workgroups, void* sink, hipengine_stream_t stream);
+
 #ifdef __cplusplus
 }
 #endif
