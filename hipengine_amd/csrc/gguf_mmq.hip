@@ -48,10 +48,11 @@ __global__ void __launch_bounds__(Tile::THREADS, MIN_WAVES) mmq_q4_k_ds4_kernel(
   const int steps = a.K / 128;
   const int64_t w_row_bytes = static_cast<int64_t>(a.K / QK_K) * Tile::W_BLOCK;
   const int64_t x_row_bytes = static_cast<int64_t>(steps) * Tile::A_BYTES;
-  Tile::template run<PREFETCH>(
-      a.xq, x_row_bytes, a.w, w_row_bytes, steps, s,
-      [=](int row) { return static_cast<int64_t>(min(m0 + row, a.M - 1)); },
-      [=](int col) { return static_cast<int64_t>(min(n0 + col, a.N - 1)); },
+  // rows and columns relative to the tile's first: the engine keeps 32-bit byte offsets from the two bases
+  Tile::template run<PREFETCH, false>(
+      a.xq + m0 * x_row_bytes, x_row_bytes, a.w + n0 * w_row_bytes, w_row_bytes, steps, s,
+      [=](int row) { return static_cast<int64_t>(min(row, a.M - 1 - m0)); },
+      [=](int col) { return static_cast<int64_t>(min(col, a.N - 1 - n0)); },
       [=](int row, int col, float v) {
         const int m = m0 + row, n = n0 + col;
         if (m < a.M && n < a.N) store_scalar(a.out, static_cast<int64_t>(m) * a.N + n, v, a.out_kind);
@@ -74,8 +75,8 @@ __global__ void __launch_bounds__(Tile::THREADS, 2) mmq_tile_dump_kernel(MmqArgs
   const int steps = a.K / 128;
   const int64_t w_row_bytes = static_cast<int64_t>(a.K / QK_K) * Tile::W_BLOCK;
   const int64_t x_row_bytes = static_cast<int64_t>(steps) * Tile::A_BYTES;
-  auto row_of = [=](int row) { return static_cast<int64_t>(min(m0 + row, a.M - 1)); };
-  auto col_of = [=](int col) { return static_cast<int64_t>(min(n0 + col, a.N - 1)); };
+  auto row_of = [=](int row) { return static_cast<int64_t>(min(row, a.M - 1 - m0)); };
+  auto col_of = [=](int col) { return static_cast<int64_t>(min(col, a.N - 1 - n0)); };
   auto emit = [=](int row, int col, float v) {
     const int m = m0 + row, n = n0 + col;
     if (m < a.M && n < a.N) store_scalar(a.out, static_cast<int64_t>(m) * a.N + n, v, a.out_kind);
@@ -84,8 +85,8 @@ __global__ void __launch_bounds__(Tile::THREADS, 2) mmq_tile_dump_kernel(MmqArgs
     const int m = m0 + row, n = n0 + col;
     if (m < a.M && n < a.N) dots[(static_cast<int64_t>(m) * a.N + n) * (a.K / 32) + sb] = dot;
   };
-  Tile::template run<true, decltype(row_of), decltype(col_of), decltype(emit), true, decltype(dump)>(
-      a.xq, x_row_bytes, a.w, w_row_bytes, steps, s, row_of, col_of, emit, dump);
+  Tile::template run<true, false, decltype(row_of), decltype(col_of), decltype(emit), true, decltype(dump)>(
+      a.xq + m0 * x_row_bytes, x_row_bytes, a.w + n0 * w_row_bytes, w_row_bytes, steps, s, row_of, col_of, emit, dump);
 }
 
 int launch_q4(const void* xq, const uint8_t* w, void* out, int out_kind, int64_t M, int64_t K, int64_t N,

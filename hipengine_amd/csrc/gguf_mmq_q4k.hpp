@@ -30,6 +30,8 @@
 // peak: the MFMA pipe itself is mostly idle.
 #pragma once
 
+#include <type_traits>
+
 #include "gguf_common.hpp"
 
 namespace hipengine_gfx950 {
@@ -73,8 +75,8 @@ struct Q4Tile {
   struct Smem {
     uint8_t xa[BM * A_STRIDE];   // DS4 blocks of the step, as stored
     uint8_t wq[BN * W_STRIDE];   // 64 nibble bytes per column
-    float sw[4][BN];             // d*sc of the four sub-blocks of the current K step, by column
-    float cw[4][BN];             // -MAGIC * sw
+    float sw[8][BN];             // d*sc of the eight sub-blocks of the current weight block, by column (decoded at
+    float cw[8][BN];             // -MAGIC * sw                          the block's first K step, used by both)
     float xd[4][BM];             // activation scale per sub-block of the step, by row
     float dmin[BN];
     _Float16 mnh[BN][8];         // 6-bit mins as fp16
@@ -90,38 +92,74 @@ struct Q4Tile {
     u32x4 ph2[Q5 ? H_PER : 1];   // D4S4: the second half of a row's header (the four float32 sums)
   };
 
-  // `row_of(r)` / `col_of(c)` give the activation row (in DS4 blocks of x_row_bytes
-  // per row from xq) and the weight row (of w_row_bytes from w) that tile row r /
-  // tile column c read; rows and columns outside the problem are mapped to any
-  // valid one by the caller (their results are not stored).
-  template <class RowOf, class ColOf>
-  static __device__ __forceinline__ void load(const uint8_t* xq, int64_t x_row_bytes, const uint8_t* w,
-                                              int64_t w_row_bytes, int step, int tid, RowOf row_of, ColOf col_of,
-                                              Regs& r) {
-    const int kb = step >> 1, h = step & 1;
+  // What a thread fetches every K step, as byte offsets that do not change along K: from xq for its activation
+  // chunks and row headers, from w for its nibble chunks and column headers.  The step adds a scalar to the base
+  // (the loads then take a 64-bit scalar base and a 32-bit lane offset: no address arithmetic in the K loop).
+  // Callers pass bases at the tile's first row and column, so 32 bits hold any offset within a tile; a caller
+  // that gathers its rows from anywhere in a large buffer asks for 64-bit row offsets (WIDE).
+  template <bool WIDE>
+  struct Offsets {
+    using Row = typename std::conditional<WIDE, uint64_t, uint32_t>::type;
+    Row a[A_PER];
+    uint32_t w[W_PER];
+    Row h[H_PER];
+  };
+
+  template <bool WIDE, class RowOf, class ColOf>
+  static __device__ __forceinline__ Offsets<WIDE> offsets(int64_t x_row_bytes, int64_t w_row_bytes, int tid, RowOf row_of,
+                                                    ColOf col_of) {
+    Offsets<WIDE> o;
+    using Row = typename Offsets<WIDE>::Row;
 #pragma unroll
     for (int i = 0; i < A_PER; ++i) {
       const int c = min(tid + i * THREADS, A_CHUNKS - 1);
       const int row = c / A_PARTS, part = c - row * A_PARTS;
-      r.pa[i] = *reinterpret_cast<const u32x4*>(xq + row_of(row) * x_row_bytes + static_cast<int64_t>(step) * A_BYTES +
-                                                part * 16);
+      o.a[i] = static_cast<Row>(row_of(row) * x_row_bytes + part * 16);
     }
 #pragma unroll
     for (int i = 0; i < W_PER; ++i) {
       const int c = min(tid + i * THREADS, W_CHUNKS - 1);
       const int col = c / W_PARTS, part = c - col * W_PARTS;
-      // parts 0..3: the step's 64 nibble bytes; Q5_K parts 4, 5: the block's 32 qh bytes (both steps read them)
-      const int off = part < 4 ? W_QS + h * 64 + part * 16 : 16 + (part - 4) * 16;
-      r.pw[i] = *reinterpret_cast<const u32x4*>(w + col_of(col) * w_row_bytes + static_cast<int64_t>(kb) * W_BLOCK + off);
+      // parts 0..3: the step's 64 nibble bytes (the step adds 64 h); Q5_K parts 4, 5: the block's 32 qh bytes
+      o.w[i] = static_cast<uint32_t>(col_of(col) * w_row_bytes + (part < 4 ? W_QS + part * 16 : 16 + (part - 4) * 16));
     }
 #pragma unroll
     for (int i = 0; i < H_PER; ++i) {
       const int item = min(tid + i * THREADS, H_ITEMS - 1);
-      const uint8_t* hp = item < BN ? w + col_of(item) * w_row_bytes + static_cast<int64_t>(kb) * W_BLOCK
-                                    : xq + row_of(item - BN) * x_row_bytes + static_cast<int64_t>(step) * A_BYTES;
-      r.ph[i] = *reinterpret_cast<const u32x4*>(hp);
+      o.h[i] = static_cast<Row>(item < BN ? col_of(item) * w_row_bytes : row_of(item - BN) * x_row_bytes);
+    }
+    return o;
+  }
+
+  // `row_of(r)` / `col_of(c)` give the activation row (in DS4 blocks of x_row_bytes
+  // per row from xq) and the weight row (of w_row_bytes from w) that tile row r /
+  // tile column c read; rows and columns outside the problem are mapped to any
+  // valid one by the caller (their results are not stored).
+  template <bool WIDE>
+  static __device__ __forceinline__ void load(const uint8_t* xq, const uint8_t* w, int step, int tid,
+                                              const Offsets<WIDE>& o, Regs& r) {
+    const int kb = step >> 1, h = step & 1;
+    const uint8_t* xs = xq + static_cast<int64_t>(step) * A_BYTES;        // uniform
+    const uint8_t* wb = w + static_cast<int64_t>(kb) * W_BLOCK;           // uniform
+#pragma unroll
+    for (int i = 0; i < A_PER; ++i) r.pa[i] = *reinterpret_cast<const u32x4*>(xs + o.a[i]);
+#pragma unroll
+    for (int i = 0; i < W_PER; ++i) {
       if constexpr (Q5) {
-        if (item >= BN) r.ph2[i] = *reinterpret_cast<const u32x4*>(hp + 16);
+        const int part = min(tid + i * THREADS, W_CHUNKS - 1) % W_PARTS;
+        r.pw[i] = *reinterpret_cast<const u32x4*>(wb + o.w[i] + (part < 4 ? h * 64 : 0));
+      } else {
+        r.pw[i] = *reinterpret_cast<const u32x4*>(wb + h * 64 + o.w[i]);
+      }
+    }
+#pragma unroll
+    for (int i = 0; i < H_PER; ++i) {
+      const int item = min(tid + i * THREADS, H_ITEMS - 1);
+      if (item < BN) {
+        if (h == 0) r.ph[i] = *reinterpret_cast<const u32x4*>(wb + o.h[i]);   // decoded once per block
+      } else {
+        r.ph[i] = *reinterpret_cast<const u32x4*>(xs + o.h[i]);
+        if constexpr (Q5) r.ph2[i] = *reinterpret_cast<const u32x4*>(xs + o.h[i] + 16);
       }
     }
   }
@@ -150,16 +188,15 @@ struct Q4Tile {
       const int item = tid + i * THREADS;
       const u32x4 ph = r.ph[i];
       if (item < BN) {
-        const Q4KScales u = q4k_unpack_scales(ph.y, ph.z, ph.w);
-        const float d = f16_bits_to_float(ph.x & 0xFFFFu);
-        const uint32_t scw = h == 0 ? u.sc_lo : u.sc_hi;         // the step's four sub-blocks
-#pragma unroll
-        for (int j = 0; j < 4; ++j) {
-          const float sw = d * static_cast<float>((scw >> (8 * j)) & 0xFFu);
-          s.sw[j][item] = sw;
-          s.cw[j][item] = -MMQ_MAGIC * sw;
-        }
         if (h == 0) {
+          const Q4KScales u = q4k_unpack_scales(ph.y, ph.z, ph.w);
+          const float d = f16_bits_to_float(ph.x & 0xFFFFu);
+#pragma unroll
+          for (int j = 0; j < 8; ++j) {
+            const float sw = d * static_cast<float>(((j < 4 ? u.sc_lo : u.sc_hi) >> (8 * (j & 3))) & 0xFFu);
+            s.sw[j][item] = sw;
+            s.cw[j][item] = -MMQ_MAGIC * sw;
+          }
           s.dmin[item] = f16_bits_to_float(ph.x >> 16);
 #pragma unroll
           for (int j = 0; j < 8; ++j) {
@@ -247,7 +284,7 @@ struct Q4Tile {
 #pragma unroll
         for (int nt = 0; nt < NT; ++nt) {
           const int col = (wn * NT + nt) * 32 + lc;
-          o.sw[nt] = s.sw[sl][col]; o.cw[nt] = s.cw[sl][col];
+          o.sw[nt] = s.sw[4 * h + sl][col]; o.cw[nt] = s.cw[4 * h + sl][col];
         }
         return o;
       };
@@ -305,7 +342,7 @@ struct Q4Tile {
 
   // The whole K loop of one output tile.  `emit(row, col, value)` receives every
   // element of the tile (tile-relative coordinates) once.
-  template <bool PREFETCH, class RowOf, class ColOf, class Emit, bool DUMP = false, class Dump = int>
+  template <bool PREFETCH, bool WIDE_ROWS, class RowOf, class ColOf, class Emit, bool DUMP = false, class Dump = int>
   static __device__ __forceinline__ void run(const uint8_t* xq, int64_t x_row_bytes, const uint8_t* w,
                                              int64_t w_row_bytes, int steps, Smem& s, RowOf row_of, ColOf col_of,
                                              Emit emit, Dump dump = 0) {
@@ -321,15 +358,16 @@ struct Q4Tile {
 #pragma unroll
         for (int v = 0; v < 16; ++v) acc[i][j][v] = 0.0f;
 
+    const Offsets<WIDE_ROWS> offs = offsets<WIDE_ROWS>(x_row_bytes, w_row_bytes, tid, row_of, col_of);
     Regs regs;
-    if (PREFETCH) load(xq, x_row_bytes, w, w_row_bytes, 0, tid, row_of, col_of, regs);
+    if (PREFETCH) load(xq, w, 0, tid, offs, regs);
     for (int step = 0; step < steps; ++step) {
-      if (!PREFETCH) load(xq, x_row_bytes, w, w_row_bytes, step, tid, row_of, col_of, regs);
+      if (!PREFETCH) load(xq, w, step, tid, offs, regs);
       store(s, step, tid, regs);
       __syncthreads();
       // The loads of the next step are issued before this step is computed, so
       // their latency hides behind the MFMA/FMA work.
-      if (PREFETCH && step + 1 < steps) load(xq, x_row_bytes, w, w_row_bytes, step + 1, tid, row_of, col_of, regs);
+      if (PREFETCH && step + 1 < steps) load(xq, w, step + 1, tid, offs, regs);
       if constexpr (DUMP) {
         compute<true>(s, step, wm, wn, lc, g, acc, [&](int row, int col, int sb, int dot) { dump(row, col, 4 * step + sb, dot); });
       } else {

@@ -960,7 +960,7 @@ __global__ void __launch_bounds__(Tile::THREADS, 2) moe_mmq_kernel(MoeMmqArgs a)
   const int64_t w_row_bytes = static_cast<int64_t>(a.K / QK_K) * Tile::W_BLOCK;
   const int64_t x_row_bytes = static_cast<int64_t>(steps) * Tile::A_BYTES;
   const int64_t stride_rows = a.expert_stride_rows > 0 ? a.expert_stride_rows : local_n;
-  const uint8_t* w = (use_b ? a.w_b : a.w_a) + e * stride_rows * w_row_bytes;
+  const uint8_t* w = (use_b ? a.w_b : a.w_a) + (e * stride_rows + n0) * w_row_bytes;   // the tile's first column
 
   if (threadIdx.x < Tile::BM) {
     const int64_t crow = first_compact + min(static_cast<int>(threadIdx.x), valid_rows - 1);
@@ -972,10 +972,10 @@ __global__ void __launch_bounds__(Tile::THREADS, 2) moe_mmq_kernel(MoeMmqArgs a)
 
   const int64_t out_stride = static_cast<int64_t>(a.Na) + a.Nb;
   const int col_base = (use_b ? a.Na : 0) + n0;
-  Tile::template run<true>(
+  Tile::template run<true, true>(
       a.xq, x_row_bytes, w, w_row_bytes, steps, s,
       [=](int row) { return static_cast<int64_t>(src_row[row]); },
-      [=](int col) { return static_cast<int64_t>(min(n0 + col, local_n - 1)); },
+      [=](int col) { return static_cast<int64_t>(min(col, local_n - 1 - n0)); },
       [=](int row, int col, float v) {
         if (row < valid_rows && n0 + col < local_n)
           store_scalar(a.out, (first_compact + row) * out_stride + col_base + col, v, a.out_kind);
