@@ -317,7 +317,7 @@ class Harness:
         return t_logits, t_select
 
     def moe_case(self, tokens: int, steps: int, warmup: int, experts: int = 256, top_k: int = 8, hidden: int = 2048,
-                 inter: int = 512, down_quant: str = "q4_k"):
+                 inter: int = 512, down_quant: str = "q4_k", expert_pool: int | None = None):
         """Selected-expert FFN (Q4_K gate/up, Q4_K or Q6_K down): the two-launch decode chain for
         tokens <= 8, the grouped-MMQ prefill chain (index, pack, gate|up, SiLU, pack,
         down, ordered gather) above.  Returns seconds per chain and the bytes of
@@ -343,7 +343,9 @@ class Harness:
             nsets = max(1, experts // lanes)
             sel_sets = [perm[i * lanes:(i + 1) * lanes].reshape(tokens, top_k).astype(np.int64) for i in range(nsets)]
         else:
-            sel_sets = [np.stack([rng.permutation(experts)[:top_k] for _ in range(tokens)]).astype(np.int64)]
+            # expert_pool: route every token within the first expert_pool experts (their weights stay in the caches)
+            pool = experts if expert_pool is None else expert_pool
+            sel_sets = [np.stack([rng.permutation(pool)[:top_k] for _ in range(tokens)]).astype(np.int64)]
         sel = sel_sets[0]
         wts = rng.random((tokens, top_k)).astype(np.float32)
         wts /= wts.sum(axis=1, keepdims=True)
@@ -492,13 +494,13 @@ def main() -> None:
         h.rt.device_synchronize()
         if args.pmc_shape.startswith("moe,"):
             tokens = int(args.pmc_shape.split(",")[1])
-            sec, touched, ops = h.moe_case(tokens, 4, 1)
+            sec, touched, ops = h.moe_case(tokens, 20, 4)
             print(json.dumps({"pmc_pass": True, "copy_bytes": nbytes, "moe_tokens": tokens, "expert_bytes": touched,
                               "int8_ops": ops}))
             return
         if args.pmc_shape.startswith("mmq,"):
             _, pq, pm, pk, pn = args.pmc_shape.split(",")
-            sec, ops = h.mmq_case(pq, int(pm), int(pk), int(pn), 4, 1)
+            sec, ops = h.mmq_case(pq, int(pm), int(pk), int(pn), 20, 4)
             print(json.dumps({"pmc_pass": True, "copy_bytes": nbytes, "mmq": args.pmc_shape, "int8_ops": ops}))
             return
         if args.pmc_shape:

@@ -60,10 +60,15 @@ __global__ void __launch_bounds__(Tile::THREADS, MIN_WAVES) mmq_q4_k_ds4_kernel(
 }
 
 template <class Tile, bool PREFETCH, int MIN_WAVES>
-void launch_q4_tile(const MmqArgs& a, hipStream_t stream) {
+int launch_q4_tile(const MmqArgs& a, hipStream_t stream) {
+  if (sizeof(typename Tile::Smem) > 65536) {   // the LDS limit is raised at set-up
+    const int rc = ensure_init();
+    if (rc != static_cast<int>(hipSuccess)) return rc;
+  }
   const dim3 grid(static_cast<unsigned>((a.M + Tile::BM - 1) / Tile::BM), static_cast<unsigned>((a.N + Tile::BN - 1) / Tile::BN));
   hipLaunchKernelGGL((mmq_q4_k_ds4_kernel<Tile, PREFETCH, MIN_WAVES>), grid, dim3(Tile::THREADS), sizeof(typename Tile::Smem),
                      stream, a);
+  return static_cast<int>(hipGetLastError());
 }
 
 // Verification: the same tile engine, which also writes every int32 sub-block dot to dots[M, N, K/32].
@@ -97,11 +102,7 @@ int launch_q4(const void* xq, const uint8_t* w, void* out, int out_kind, int64_t
   }
   MmqArgs a{static_cast<const uint8_t*>(xq), w, out, out_kind, static_cast<int>(M), static_cast<int>(K),
             static_cast<int>(N)};
-  switch (variant) {
-    case 1: launch_q4_tile<DenseQ4, false, 2>(a, stream); break;
-    default: launch_q4_tile<DenseQ4, true, 2>(a, stream); break;
-  }
-  return static_cast<int>(hipGetLastError());
+  return variant == 1 ? launch_q4_tile<DenseQ4, false, 2>(a, stream) : launch_q4_tile<DenseQ4, true, 2>(a, stream);
 }
 
 // --------------------------------------------------------------------------
@@ -249,8 +250,7 @@ int launch_q5(const void* xq, const uint8_t* w, void* out, int out_kind, int64_t
             static_cast<int>(N)};
   // without the register prefetch of the next step: with it this format spills 20 registers in the K loop
   // (752 us against 666 at M = 2048, 17408x5120)
-  launch_q4_tile<DenseQ5, false, 2>(a, stream);
-  return static_cast<int>(hipGetLastError());
+  return launch_q4_tile<DenseQ5, false, 2>(a, stream);
 }
 
 #define DEFINE_MMQ_Q5(SYMBOL, OKIND)                                                                        \
@@ -303,6 +303,8 @@ extern "C" int hipengine_gfx950_gguf_mmq_dots_i32(int32_t ggml_type, const void*
   const dim3 grid(static_cast<unsigned>((rows + BM - 1) / BM), static_cast<unsigned>((out_features + BN - 1) / BN));
   if (ggml_type == GGML_Q4_K) {
     if ((out_features % 32) != 0) return static_cast<int>(hipErrorInvalidValue);
+    const int rc = ensure_init();   // the LDS limit of this kernel
+    if (rc != static_cast<int>(hipSuccess)) return rc;
     hipLaunchKernelGGL(mmq_tile_dump_kernel<DenseQ4>, grid, dim3(THREADS), sizeof(DenseQ4::Smem), stream, a, dots);
   } else if (ggml_type == GGML_Q5_K) {
     if ((out_features % 32) != 0) return static_cast<int>(hipErrorInvalidValue);
@@ -439,6 +441,14 @@ int hipengine_gfx950::prefill_bf16_library_buffer(int ggml_type, const void* x, 
 }
 
 int hipengine_gfx950::mmq_load() {
+  // the Q4_K tile engine holds two copies of a K step's images: more than the 64 KiB a kernel may use unasked
+  for (const void* fn : {reinterpret_cast<const void*>(mmq_q4_k_ds4_kernel<DenseQ4, false, 2>),
+                         reinterpret_cast<const void*>(mmq_q4_k_ds4_kernel<DenseQ4, true, 2>),
+                         reinterpret_cast<const void*>(mmq_tile_dump_kernel<DenseQ4>)}) {
+    const hipError_t e = hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize,
+                                             static_cast<int>(sizeof(DenseQ4::Smem)));
+    if (e != hipSuccess) return static_cast<int>(e);
+  }
   hipFuncAttributes attr;
   return static_cast<int>(hipFuncGetAttributes(&attr, reinterpret_cast<const void*>(mmq_q6_k_d4s4_kernel<false, 128>)));
 }

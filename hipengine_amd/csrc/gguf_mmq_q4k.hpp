@@ -72,16 +72,21 @@ struct Q4Tile {
   static constexpr int W_PER = (W_CHUNKS + THREADS - 1) / THREADS;
   static constexpr int H_PER = (H_ITEMS + THREADS - 1) / THREADS;
 
+  // Two copies of everything a K step stages, so a step's images are written while slower waves still read the
+  // step before: one barrier per step.  What belongs to a step (values, nibbles, activation scales) alternates with
+  // the step; what belongs to a weight block of two steps (scales, mins, activation sums) with the block.
+  static constexpr int NBUF = Q5 ? 1 : 2;   // Q5_K x D4S4 images are too large to hold twice with two workgroups
+                                            // on a CU: one copy, and a second barrier per step
   struct Smem {
-    uint8_t xa[BM * A_STRIDE];   // DS4 blocks of the step, as stored
-    uint8_t wq[BN * W_STRIDE];   // 64 nibble bytes per column
-    float sw[8][BN];             // d*sc of the eight sub-blocks of the current weight block, by column (decoded at
-    float cw[8][BN];             // -MAGIC * sw                          the block's first K step, used by both)
-    float xd[4][BM];             // activation scale per sub-block of the step, by row
-    float dmin[BN];
-    _Float16 mnh[BN][8];         // 6-bit mins as fp16
-    _Float16 xsh[BM][8];         // activation sums of the weight block (fp16 in the DS4 block already; D4S4: high part)
-    _Float16 xsl[Q5 ? BM : 1][8];   // D4S4: low part of the float32 sums
+    uint8_t xa[NBUF][BM * A_STRIDE];   // DS4 blocks of the step, as stored
+    uint8_t wq[NBUF][BN * W_STRIDE];   // 64 nibble bytes per column
+    float sw[NBUF][8][BN];             // d*sc of the eight sub-blocks of the weight block, by column (decoded at the
+                                    // block's first K step, used by both)
+    float xd[NBUF][4][BM];             // activation scale per sub-block of the step, by row
+    float dmin[NBUF][BN];
+    _Float16 mnh[NBUF][BN][8];         // 6-bit mins as fp16
+    _Float16 xsh[NBUF][BM][8];         // activation sums of the weight block (fp16 in the DS4 block already; D4S4: high part)
+    _Float16 xsl[NBUF][Q5 ? BM : 1][8];   // D4S4: low part of the float32 sums
   };
 
   // Registers of one K step in flight between global memory and LDS.
@@ -136,22 +141,30 @@ struct Q4Tile {
   // tile column c read; rows and columns outside the problem are mapped to any
   // valid one by the caller (their results are not stored).
   template <bool WIDE>
-  static __device__ __forceinline__ void load(const uint8_t* xq, const uint8_t* w, int step, int tid,
-                                              const Offsets<WIDE>& o, Regs& r) {
+  static __device__ __forceinline__ void load_w(const uint8_t* w, int step, int tid, const Offsets<WIDE>& o,
+                                                u32x4 (&pw)[W_PER]) {
+    const int kb = step >> 1, h = step & 1;
+    const uint8_t* wb = w + static_cast<int64_t>(kb) * W_BLOCK;           // uniform
+#pragma unroll
+    for (int i = 0; i < W_PER; ++i) {
+      if constexpr (Q5) {
+        const int part = min(tid + i * THREADS, W_CHUNKS - 1) % W_PARTS;
+        pw[i] = *reinterpret_cast<const u32x4*>(wb + o.w[i] + (part < 4 ? h * 64 : 0));
+      } else {
+        pw[i] = *reinterpret_cast<const u32x4*>(wb + h * 64 + o.w[i]);
+      }
+    }
+  }
+
+  // activation chunks and the headers of both sides
+  template <bool WIDE>
+  static __device__ __forceinline__ void load_ah(const uint8_t* xq, const uint8_t* w, int step, int tid,
+                                                 const Offsets<WIDE>& o, Regs& r) {
     const int kb = step >> 1, h = step & 1;
     const uint8_t* xs = xq + static_cast<int64_t>(step) * A_BYTES;        // uniform
     const uint8_t* wb = w + static_cast<int64_t>(kb) * W_BLOCK;           // uniform
 #pragma unroll
     for (int i = 0; i < A_PER; ++i) r.pa[i] = *reinterpret_cast<const u32x4*>(xs + o.a[i]);
-#pragma unroll
-    for (int i = 0; i < W_PER; ++i) {
-      if constexpr (Q5) {
-        const int part = min(tid + i * THREADS, W_CHUNKS - 1) % W_PARTS;
-        r.pw[i] = *reinterpret_cast<const u32x4*>(wb + o.w[i] + (part < 4 ? h * 64 : 0));
-      } else {
-        r.pw[i] = *reinterpret_cast<const u32x4*>(wb + h * 64 + o.w[i]);
-      }
-    }
 #pragma unroll
     for (int i = 0; i < H_PER; ++i) {
       const int item = min(tid + i * THREADS, H_ITEMS - 1);
@@ -164,24 +177,31 @@ struct Q4Tile {
     }
   }
 
-  static __device__ __forceinline__ void store(Smem& s, int step, int tid, const Regs& r) {
-    const int h = step & 1;
+  template <bool WIDE>
+  static __device__ __forceinline__ void load(const uint8_t* xq, const uint8_t* w, int step, int tid,
+                                              const Offsets<WIDE>& o, Regs& r) {
+    load_w(w, step, tid, o, r.pw);
+    load_ah(xq, w, step, tid, o, r);
+  }
+
+  static __device__ __forceinline__ void store(Smem& s, int step, int tid, const Regs& r, const u32x4 (&pw)[W_PER]) {
+    const int h = step & 1, sb = step & (NBUF - 1), bb = (step >> 1) & (NBUF - 1);   // step half, step copy, block copy
 #pragma unroll
     for (int i = 0; i < A_PER; ++i) {
       const int c = tid + i * THREADS;           // DS4: 144-byte rows are contiguous in LDS, offset c*16
       if (c < A_CHUNKS) {
         if constexpr (Q5) {
           const int row = c / A_PARTS, part = c - row * A_PARTS;
-          *reinterpret_cast<u32x4*>(s.xa + row * A_STRIDE + part * 16) = r.pa[i];
+          *reinterpret_cast<u32x4*>(s.xa[sb] + row * A_STRIDE + part * 16) = r.pa[i];
         } else {
-          *reinterpret_cast<u32x4*>(s.xa + c * 16) = r.pa[i];
+          *reinterpret_cast<u32x4*>(s.xa[sb] + c * 16) = r.pa[i];
         }
       }
     }
 #pragma unroll
     for (int i = 0; i < W_PER; ++i) {
       const int c = tid + i * THREADS;
-      if (c < W_CHUNKS) *reinterpret_cast<u32x4*>(s.wq + (c / W_PARTS) * W_STRIDE + (c % W_PARTS) * 16) = r.pw[i];
+      if (c < W_CHUNKS) *reinterpret_cast<u32x4*>(s.wq[sb] + (c / W_PARTS) * W_STRIDE + (c % W_PARTS) * 16) = pw[i];
     }
 #pragma unroll
     for (int i = 0; i < H_PER; ++i) {
@@ -194,14 +214,13 @@ struct Q4Tile {
 #pragma unroll
           for (int j = 0; j < 8; ++j) {
             const float sw = d * static_cast<float>(((j < 4 ? u.sc_lo : u.sc_hi) >> (8 * (j & 3))) & 0xFFu);
-            s.sw[j][item] = sw;
-            s.cw[j][item] = -MMQ_MAGIC * sw;
+            s.sw[bb][j][item] = sw;
           }
-          s.dmin[item] = f16_bits_to_float(ph.x >> 16);
+          s.dmin[bb][item] = f16_bits_to_float(ph.x >> 16);
 #pragma unroll
           for (int j = 0; j < 8; ++j) {
             const uint32_t mn = ((j < 4 ? u.mn_lo : u.mn_hi) >> (8 * (j & 3))) & 0xFFu;
-            s.mnh[item][j] = static_cast<_Float16>(static_cast<float>(mn));
+            s.mnh[bb][item][j] = static_cast<_Float16>(static_cast<float>(mn));
           }
         }
       } else if (item < H_ITEMS) {
@@ -209,14 +228,14 @@ struct Q4Tile {
 #pragma unroll
         for (int j = 0; j < 4; ++j) {
           if constexpr (Q5) {
-            s.xd[j][row] = bits_to_float(ph[j]);
+            s.xd[sb][j][row] = bits_to_float(ph[j]);
             const float sum = bits_to_float(r.ph2[i][j]);
             const _Float16 hi = static_cast<_Float16>(sum);
-            s.xsh[row][4 * h + j] = hi;
-            s.xsl[row][4 * h + j] = static_cast<_Float16>(sum - static_cast<float>(hi));
+            s.xsh[bb][row][4 * h + j] = hi;
+            s.xsl[bb][row][4 * h + j] = static_cast<_Float16>(sum - static_cast<float>(hi));
           } else {
-            s.xd[j][row] = f16_bits_to_float(ph[j] & 0xFFFFu);
-            s.xsh[row][4 * h + j] = __builtin_bit_cast(_Float16, static_cast<uint16_t>(ph[j] >> 16));
+            s.xd[sb][j][row] = f16_bits_to_float(ph[j] & 0xFFFFu);
+            s.xsh[bb][row][4 * h + j] = __builtin_bit_cast(_Float16, static_cast<uint16_t>(ph[j] >> 16));
           }
         }
       }
@@ -228,7 +247,7 @@ struct Q4Tile {
   template <bool DUMP = false, class Dump = int>
   static __device__ __forceinline__ void compute(const Smem& s, int step, int wm, int wn, int lc, int g,
                                                  float (&acc)[NT][MT][16], Dump dump = 0) {
-    const int h = step & 1;
+    const int h = step & 1, sb = step & (NBUF - 1), bb = (step >> 1) & (NBUF - 1);
     v16i c0;
 #pragma unroll
     for (int v = 0; v < 16; ++v) c0[v] = static_cast<int>(MMQ_MAGIC_BITS);
@@ -238,14 +257,14 @@ struct Q4Tile {
 #pragma unroll
       for (int nt = 0; nt < NT; ++nt) {
         const int col = (wn * NT + nt) * 32 + lc;
-        const u32x4 qs = *reinterpret_cast<const u32x4*>(s.wq + col * W_STRIDE + sp * 32 + 16 * g);
+        const u32x4 qs = *reinterpret_cast<const u32x4*>(s.wq[sb] + col * W_STRIDE + sp * 32 + 16 * g);
         wlo[nt] = v4i{static_cast<int>(q4k_low(qs.x)), static_cast<int>(q4k_low(qs.y)),
                       static_cast<int>(q4k_low(qs.z)), static_cast<int>(q4k_low(qs.w))};
         whi[nt] = v4i{static_cast<int>(q4k_high(qs.x)), static_cast<int>(q4k_high(qs.y)),
                       static_cast<int>(q4k_high(qs.z)), static_cast<int>(q4k_high(qs.w))};
         if constexpr (Q5) {
           // values 16g..16g+15 of sub-blocks s0 = 4h + 2sp (low nibbles) and s0 + 1 (high): bit 4 is bit s of qh[l]
-          const u32x4 qh = *reinterpret_cast<const u32x4*>(s.wq + col * W_STRIDE + 64 + 16 * g);
+          const u32x4 qh = *reinterpret_cast<const u32x4*>(s.wq[sb] + col * W_STRIDE + 64 + 16 * g);
           const int s0 = 4 * h + 2 * sp;
 #pragma unroll
           for (int e = 0; e < 4; ++e) {
@@ -262,7 +281,7 @@ struct Q4Tile {
       for (int half = 0; half < 2; ++half)
 #pragma unroll
         for (int mt = 0; mt < MT; ++mt)
-          xop[half][mt] = *reinterpret_cast<const v4i*>(s.xa + ((wm * MT + mt) * 32 + lc) * A_STRIDE + A_QS +
+          xop[half][mt] = *reinterpret_cast<const v4i*>(s.xa[sb] + ((wm * MT + mt) * 32 + lc) * A_STRIDE + A_QS +
                                                         (2 * sp + half) * 32 + 16 * g);
       auto issue = [&](int i) {
         const int half = i / (MT * NT), mt = (i / NT) % MT, nt = i % NT;
@@ -278,13 +297,13 @@ struct Q4Tile {
         PairOps o;
 #pragma unroll
         for (int j = 0; j < 4; ++j) {
-          const float4 t = *reinterpret_cast<const float4*>(&s.xd[sl][rbase + 8 * j + 4 * g]);
+          const float4 t = *reinterpret_cast<const float4*>(&s.xd[sb][sl][rbase + 8 * j + 4 * g]);
           o.xdv[4 * j] = t.x; o.xdv[4 * j + 1] = t.y; o.xdv[4 * j + 2] = t.z; o.xdv[4 * j + 3] = t.w;
         }
 #pragma unroll
         for (int nt = 0; nt < NT; ++nt) {
           const int col = (wn * NT + nt) * 32 + lc;
-          o.sw[nt] = s.sw[4 * h + sl][col]; o.cw[nt] = s.cw[4 * h + sl][col];
+          o.sw[nt] = s.sw[bb][4 * h + sl][col]; o.cw[nt] = -MMQ_MAGIC * o.sw[nt];
         }
         return o;
       };
@@ -319,20 +338,20 @@ struct Q4Tile {
 #pragma unroll
       for (int mt = 0; mt < MT; ++mt) {
         const int arow = (wm * MT + mt) * 32 + lc;
-        const v4h xs = *reinterpret_cast<const v4h*>(&s.xsh[arow][4 * g]);
+        const v4h xs = *reinterpret_cast<const v4h*>(&s.xsh[bb][arow][4 * g]);
 #pragma unroll
         for (int nt = 0; nt < NT; ++nt) {
           const int col = (wn * NT + nt) * 32 + lc;
-          const v4h mn = *reinterpret_cast<const v4h*>(&s.mnh[col][4 * g]);
+          const v4h mn = *reinterpret_cast<const v4h*>(&s.mnh[bb][col][4 * g]);
           v16f z;
 #pragma unroll
           for (int v = 0; v < 16; ++v) z[v] = 0.0f;
           v16f t = __builtin_amdgcn_mfma_f32_32x32x8f16(xs, mn, z, 0, 0, 0);
           if constexpr (Q5) {
-            const v4h xl = *reinterpret_cast<const v4h*>(&s.xsl[arow][4 * g]);
+            const v4h xl = *reinterpret_cast<const v4h*>(&s.xsl[bb][arow][4 * g]);
             t = __builtin_amdgcn_mfma_f32_32x32x8f16(xl, mn, t, 0, 0, 0);
           }
-          const float nd = -s.dmin[col];
+          const float nd = -s.dmin[bb][col];
 #pragma unroll
           for (int v = 0; v < 16; ++v) acc[nt][mt][v] = __builtin_fmaf(nd, t[v], acc[nt][mt][v]);
         }
@@ -360,20 +379,25 @@ struct Q4Tile {
 
     const Offsets<WIDE_ROWS> offs = offsets<WIDE_ROWS>(x_row_bytes, w_row_bytes, tid, row_of, col_of);
     Regs regs;
-    if (PREFETCH) load(xq, w, 0, tid, offs, regs);
-    for (int step = 0; step < steps; ++step) {
-      if (!PREFETCH) load(xq, w, step, tid, offs, regs);
-      store(s, step, tid, regs);
-      __syncthreads();
-      // The loads of the next step are issued before this step is computed, so
-      // their latency hides behind the MFMA/FMA work.
-      if (PREFETCH && step + 1 < steps) load(xq, w, step + 1, tid, offs, regs);
+    auto work = [&](int step) {
       if constexpr (DUMP) {
         compute<true>(s, step, wm, wn, lc, g, acc, [&](int row, int col, int sb, int dot) { dump(row, col, 4 * step + sb, dot); });
       } else {
         compute(s, step, wm, wn, lc, g, acc);
       }
-      __syncthreads();   // the next step overwrites the tiles
+    };
+    if (PREFETCH) load(xq, w, 0, tid, offs, regs);
+    for (int step = 0; step < steps; ++step) {
+      if (!PREFETCH) load(xq, w, step, tid, offs, regs);
+      store(s, step, tid, regs, regs.pw);
+      __syncthreads();
+      // The loads of the next step are issued before this step is computed, so
+      // their latency hides behind the MFMA/FMA work.
+      if (PREFETCH && step + 1 < steps) load(xq, w, step + 1, tid, offs, regs);
+      work(step);
+      // two copies: no barrier here.  The next step writes the other copy, and whoever writes this copy again
+      // (two steps on) has passed the next step's barrier, which every wave reaches only after this compute
+      if constexpr (NBUF == 1) __syncthreads();
     }
 
     // lane holds column lc of each n tile and rows 8*(v/4) + 4*g + v%4 of each m tile

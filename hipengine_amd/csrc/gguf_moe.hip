@@ -995,6 +995,10 @@ int launch_moe_mmq(const void* xq, const int64_t* compact_to_source, const int64
       expert_stride_rows < 0 || out_kind < KIND_F32 || out_kind > KIND_F16) {
     return static_cast<int>(hipErrorInvalidValue);
   }
+  if (sizeof(typename Tile::Smem) > 65536) {   // the LDS limit is raised at set-up
+    const int rc = ensure_init();
+    if (rc != static_cast<int>(hipSuccess)) return rc;
+  }
   MoeMmqArgs a;
   a.xq = static_cast<const uint8_t*>(xq);
   a.compact_to_source = compact_to_source;
@@ -2168,6 +2172,11 @@ extern "C" int hipengine_qwen35_router_select(const float* logits, int64_t* sele
 }
 
 int hipengine_gfx950::moe_load() {
+  // the Q4_K tile engine holds two copies of a K step's images: more than the 64 KiB a kernel may use unasked
+  const hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(moe_mmq_kernel<MoeQ4>),
+                                           hipFuncAttributeMaxDynamicSharedMemorySize,
+                                           static_cast<int>(sizeof(MoeQ4::Smem) + MoeQ4::BM * sizeof(int)));
+  if (e != hipSuccess) return static_cast<int>(e);
   hipFuncAttributes attr;
   return static_cast<int>(hipFuncGetAttributes(&attr, reinterpret_cast<const void*>(moe_tile_map_kernel)));
 }
