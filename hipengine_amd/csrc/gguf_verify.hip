@@ -126,7 +126,7 @@ extern "C" int hipengine_gfx950_read_probe_grid(const void* src, int64_t bytes, 
 
 static int read_probe_launch(const void* src, int64_t bytes, int32_t waves_per_workgroup, int32_t loads_in_flight,
                              int32_t workgroups, void* sink, hipStream_t stream) {
-  if (!src || (reinterpret_cast<uintptr_t>(src) & 15) != 0 || bytes < 1024 || waves_per_workgroup < 1 || waves_per_workgroup > 16 ||
+  if (!src || (reinterpret_cast<uintptr_t>(src) & 1) != 0 || bytes < 1024 || waves_per_workgroup < 1 || waves_per_workgroup > 16 ||
       (loads_in_flight != 1 && loads_in_flight != 2 && loads_in_flight != 4)) {
     return static_cast<int>(hipErrorInvalidValue);
   }

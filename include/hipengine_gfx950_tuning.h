@@ -106,7 +106,9 @@ int hipengine_gfx950_gguf_q4_k_mmq_tuned(const void* xq, const uint8_t* qweight,
  * each with loads_in_flight (2 or 4) wave-wide 16-byte-per-lane loads in flight, consecutive 1 KB pieces dealt
  * to consecutive waves.  Nothing is computed or written (sink, [256 * waves_per_workgroup] uint32 or null, is
  * there to keep the loads alive).  The time of this launch is what a decode GEMV over a weight of that size
- * could reach if its arithmetic, its activations and its stores were free.  Measurement only.  New here. */
+ * could reach if its arithmetic, its activations and its stores were free.  src may be any even address: a base
+ * that is 2 mod 4 shows what 16-byte loads from such addresses cost (every other 210-byte Q6_K block starts at one).
+ * Measurement only.  New here. */
 int hipengine_gfx950_read_probe(const void* src, int64_t bytes, int32_t waves_per_workgroup, int32_t loads_in_flight,
                                 void* sink, hipengine_stream_t stream);
 
