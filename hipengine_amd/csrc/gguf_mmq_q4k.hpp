@@ -10,7 +10,10 @@
 // four 32-wide sub-blocks) per column.
 //   * The step's activation blocks and weight nibbles are copied to LDS with
 //     16-byte loads; with PREFETCH the loads of step s+1 are issued into
-//     registers before step s is computed.
+//     registers before step s is computed.  A thread's byte offsets are
+//     computed once per tile, a weight block's header is decoded once per
+//     block, and the Q4_K format keeps two LDS copies of a step's images, so
+//     the K loop has one barrier per step.
 //   * A wave reads MFMA operands straight from those LDS images: the int8
 //     activation bytes as they are, the weight nibbles split in registers.
 //     v_mfma_i32_32x32x32_i8 spans exactly one sub-block, so every int32
@@ -26,7 +29,7 @@
 //     fp16, mn_j <= 63), scaled by dmin[n] once per block.
 //
 // The float32 epilogue (2 VALU ops per output element per sub-block, 64 lanes
-// per CU-cycle) bounds this formulation at about a quarter of the int8 MFMA
+// per CU-cycle) bounds this formulation at about a fifth of the int8 MFMA
 // peak: the MFMA pipe itself is mostly idle.
 #pragma once
 
