@@ -215,6 +215,61 @@ def test_wrappers_validate_before_touching_the_library():
     assert Q.ds4_workspace_nbytes(2048, 5120) == 2048 * 40 * 144
 
 
+class _RecordingFunction:
+    """Stands in for a configured C function: records its arguments, returns a chosen hipError_t."""
+
+    def __init__(self, code=0):
+        self.code, self.calls, self.argtypes, self.restype = code, [], None, None
+
+    def __call__(self, *args):
+        self.calls.append(args)
+        return self.code
+
+
+class _RecordingLibrary:
+    def __init__(self, code=0):
+        self._code, self.functions = code, {}
+
+    def __getattr__(self, name):
+        if name.startswith("hipengine_"):
+            return self.functions.setdefault(name, _RecordingFunction(self._code))
+        raise AttributeError(name)
+
+
+def test_validation_flag_and_lean_launcher_reach_the_c_function_with_the_c_signature():
+    """The launch path of a decode loop: with validation on the wrapper refuses bad shapes before the library is
+    touched; with it off the same call goes straight to the C function (whose own checks remain); the lean
+    launcher is that C function with its argument types set once."""
+    from hipengine_amd.kernels.hip_gfx950 import _launch
+    from hipengine_amd.kernels.hip_gfx950.quant import gguf_q8_1_gemv as G
+
+    lib = _RecordingLibrary()
+    fn = G.FUSED[("q4_k", "f32", "f32")]
+    symbol = "hipengine_gguf_q4_k_q8_1_fused_gemv_f32_f32_out"
+    fn(16, 32, 48, 1, 5120, 17408, library=lib)
+    assert lib.functions[symbol].calls == [(16, 32, 48, 1, 5120, 17408, 128, 0)]
+    assert len(lib.functions[symbol].argtypes) == 8
+    with pytest.raises(ValueError):
+        fn(16, 32, 48, 1, 100, 8, library=lib)
+    assert len(lib.functions[symbol].calls) == 1                     # refused before the library was touched
+    assert _launch.VALIDATE is True
+    try:
+        _launch.set_validation(False)
+        fn(16, 32, 48, 1, 100, 8, library=lib)                       # not checked here: the C entry point's job
+        assert lib.functions[symbol].calls[-1] == (16, 32, 48, 1, 100, 8, 128, 0)
+    finally:
+        _launch.set_validation(True)
+    assert _launch.VALIDATE is True
+    lean = G.lean_fused("q4_k", "f32", "f32", library=lib)
+    assert lean is lib.functions[symbol]                             # the configured function itself
+    assert lean(16, 32, 48, 1, 5120, 17408, 128, 0) == 0
+    # a non-zero hipError_t from the C function surfaces as an error of the wrapper
+    bad = _RecordingLibrary(code=1)
+    with pytest.raises(Exception) as err:
+        fn(16, 32, 48, 1, 5120, 17408, library=bad)
+    assert "1" in str(err.value) or "invalid" in str(err.value).lower()
+
+
 def test_host_package_is_torch_free():
     """Importing the package, the wrappers and bench.py's harness must not import torch."""
     code = ("import sys; sys.path.insert(0, %r); import hipengine_amd, hipengine_amd.quant, "
