@@ -135,7 +135,9 @@ HIPENGINE_GFX950_DECLARE_FUSED_ALL(q8_0)
  * (loading/qwen35_gguf_consumer_surface.py:134-144,527-530).  Same argument list; here they run the fused
  * kernels above, so the arithmetic is q8_1 activations x integer weights (what hipEngine's dp4a kernels
  * compute), not the float-activation arithmetic of hipEngine's kernels of the same name.  Any rows >= 1:
- * batches of up to 8 rows per launch.
+ * batches of up to 8 rows per launch; from 32 rows of bf16 activations on, the MMQ GEMM instead, in chunks of at
+ * most 512 rows packed into a buffer the library holds (two regions per device used in turn: calls that overlap
+ * on one device may not number more than two; results then follow the MMQ's DS4 / D4S4 activation format).
  * Replace gguf_q4_k_gemv.hip:2483-2611 (Q4_K) and gguf_k_gemv.hip:5504-5545 (Q5_K, Q6_K, Q8_0). */
 #define HIPENGINE_GFX950_DECLARE_DENSE(q, a, o)                                                          \
   int hipengine_gguf_##q##_gemv_##a##_##o##_out(                                                         \
@@ -407,10 +409,11 @@ int hipengine_gguf_q8_0_mmq32_q8_1_d4s4_f32_bf16_bf16_out(const void* xq, const 
  * hipengine_gfx950_gguf_prefill_workspace_bytes reports = rows * in_features/128 * 144 or 160) and the MMQ
  * above runs on it: two launches.  ggml_type 12 (Q4_K), 13 (Q5_K; both out_features % 32 == 0), 14 (Q6_K) or 8
  * (Q8_0, in_features % 128 == 0); out_kind 0
- * float32, 1 bf16, 2 fp16.  This is what a ("linear", quant, "prefill_bf16_*_out") caller with 32 or more
- * rows should reach: hipEngine's prefill signature has no workspace argument, so the Python wrappers of the
- * prefill keys take it as an optional keyword and fall back to batches of 8 rows through the GEMV without
- * it.  New here. */
+ * float32, 1 bf16, 2 fp16.  The dense names above reach the same GEMM from 32 rows on through the library's own
+ * pack buffer (hipEngine's prefill signature has no workspace argument); this entry is for a caller that wants
+ * all rows packed at once into memory of its own - no limit on overlapping calls, one GEMM launch - and the
+ * Python wrappers of the prefill keys take such a workspace as an optional keyword.  Same bits either way.
+ * New here. */
 int hipengine_gfx950_gguf_prefill_workspace_bytes(int32_t ggml_type, int64_t rows, int64_t in_features,
                                                   int64_t* bytes);
 int hipengine_gfx950_gguf_prefill_bf16(int32_t ggml_type, const void* x, const uint8_t* qweight, void* out,
