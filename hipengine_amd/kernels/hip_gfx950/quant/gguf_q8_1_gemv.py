@@ -121,10 +121,12 @@ def _make_dense(quant: str, family: str, act: str, out: str):
     wrapper.__name__ = f"gguf_{quant}_{family}_{act}_{out}_out"
     wrapper.__doc__ = (
         f"hipEngine's dense {family} entry for {quant.upper()} (C symbol ``{symbol}``): {act} activations, quantized to "
-        f"q8_1 inside the kernel, {out} output; any number of rows, 8 per launch."
+        f"q8_1 inside the kernel, {out} output; any number of rows, 8 per launch"
+        + ("; from 32 rows of bf16 activations on the C entry runs the int8-MFMA MMQ over chunks of 512 rows packed "
+           "into a buffer the library holds (at most two such calls in flight per device)." if act == "bf16" else ".")
         + (" With ``workspace_ptr`` / ``workspace_bytes`` (see ``gguf_prefill_workspace_bytes``) and 32 rows or more, "
-           "bf16 activations are packed into the workspace and the int8-MFMA MMQ runs instead."
-           if family == "prefill" else ""))
+           "bf16 activations are packed into the caller's workspace instead and the MMQ runs once over all rows "
+           "(same bits)." if family == "prefill" else ""))
     return wrapper
 
 
