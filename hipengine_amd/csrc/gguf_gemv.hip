@@ -208,7 +208,9 @@ bool dslab_preferred(int qt, int chunk, int64_t K, int64_t N, const void* w) {
   // room, and measures slower than the phased slab: 17.3 against 14.7 us at 5120x5120, batch 8)
   if (chunk < (qt == GGML_Q8_0 ? 5 : 3) || K <= 6144) return false;
   const DslabPlan dp = default_dslab_plan(qt, chunk, K, N, w);
-  return dp.ok && dp.ksplit > 1;
+  // K parts of equal length only (K = 17408 in 4, 12288 and 8192 in 2: what has been run on hardware); a row whose
+  // blocks do not divide (K = 11008: 43 blocks) keeps its older form.  The explicit-layout entry takes any split.
+  return dp.ok && dp.ksplit > 1 && (K / QK_K) % dp.ksplit == 0;
 }
 
 GemvForm pick_form(int qt, int& chunk, int64_t K, int64_t N, const void* w) {

@@ -75,7 +75,8 @@ int hipengine_gfx950_gguf_q8_1_fused_gemv_pslab_tuned(int32_t ggml_type, const v
  * library holds (eight regions taken in turn by successive launches: more than eight such launches in flight at
  * once on one device share a region and race) and are added in part order by the workgroup that arrives last;
  * `workgroups` = row groups x k_parts.  rows <= 8, weights 2-byte aligned and < 4 GiB.  The default dispatch
- * takes this form for batches of 3 to 8 where K has to be split (in_features >= 6400 for Q4_K / Q6_K).  New here. */
+ * takes this form for batches of 3 to 8 where K has to be split (in_features >= 6400 for Q4_K / Q6_K) and splits
+ * into parts of equal length.  New here. */
 int hipengine_gfx950_gguf_q8_1_fused_gemv_dslab_tuned(int32_t ggml_type, const void* x, int32_t x_kind,
                                                       const uint8_t* qweight, void* out, int32_t out_kind,
                                                       int64_t rows, int64_t in_features, int64_t out_features,

@@ -105,3 +105,36 @@ def test_abi_version_and_host_only_entry_points(library):
     assert pf(14, 16, 16, None, 0, 64, 1024, 40, 16, big, None) == 1           # no output
     assert pf(14, 16, 16, 16, 7, 64, 1024, 40, 16, big, None) == 1             # output kind
     assert pf(8, 16, 16, 16, 0, 64, 1024, (1 << 24) + 1, 16, big, None) == 1   # out_features out of range
+
+
+def test_form_picks_hold_their_invariants_over_many_shapes(library):
+    """Host only: whatever the shape, the dispatcher names a form that exists, starts with 1..8 rows of the batch
+    (never more than asked), streams batch 1-2 wherever a matrix gives every CU a group of blocks, and takes the direct
+    slab form only for the types and row lengths it is built for."""
+    import random
+
+    ff = library.hipengine_gfx950_gguf_gemv_default_form
+    ff.argtypes = [ctypes.c_int32, ctypes.c_int64, ctypes.c_int64, ctypes.c_int64, ctypes.POINTER(ctypes.c_int32)]
+    form = (ctypes.c_int32 * 2)()
+    rng = random.Random(7)
+    seen = set()
+    shapes = [(qt, rows, 256 * nb, n) for qt in (8, 12, 13, 14) for rows in (1, 2, 3, 5, 8, 11, 64)
+              for nb in (1, 2, 16, 17, 20, 24, 25, 68, 96) for n in (1, 33, 1024, 5120, 17408)]
+    shapes += [(rng.choice((8, 12, 13, 14)), rng.randint(1, 40), 256 * rng.randint(1, 80), rng.randint(1, 200000))
+               for _ in range(2000)]
+    for qt, rows, k, n in shapes:
+        assert ff(qt, rows, k, n, form) == 0, (qt, rows, k, n)
+        kind, first = form[0], form[1]
+        seen.add(kind)
+        assert 0 <= kind <= 5 and 1 <= first <= min(rows, 8), (qt, rows, k, n, kind, first)
+        if first <= 2 and k >= 4096 and n * (k // 256) >= 16 * 256:
+            assert kind == 2, (qt, rows, k, n, kind, first)               # a group of 16 blocks per CU or more: the stream form
+        if kind == 3:
+            assert qt == 12 and k <= 6144                                 # (batch 1-2 only where a matrix is too small to stream)
+        if kind == 5:
+            assert qt in (8, 12, 14) and k > 6144 and first >= (5 if qt == 8 else 3)
+            assert (k // 256) % 2 == 0, (qt, rows, k, n)                   # K parts of equal length only
+        if kind == 4:
+            assert k % 512 == 0, (qt, rows, k, n)                          # the phased slab takes K blocks in pairs
+    assert seen == {0, 1, 2, 3, 4, 5}
+    assert ff(12, 0, 5120, 64, form) == 1 and ff(12, 1, 5120, 0, form) == 1 and ff(12, 1, 5000, 64, form) == 1
