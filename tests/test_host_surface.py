@@ -490,3 +490,24 @@ def test_gguf_reader_on_a_container_packed_without_this_package(tmp_path):
         assert probe.read_bytes() == golden.read_bytes()
     finally:
         probe.unlink(missing_ok=True)
+
+
+def test_bench_refuses_more_than_one_gpu_and_fails_loudly_without_one():
+    """bench.py is a one-GPU measurement: --gpus above 1 exits with a message that says so, and without a HIP
+    device it stops with an error instead of timing anything else."""
+    import subprocess
+    import sys
+    from pathlib import Path
+
+    root = Path(__file__).resolve().parents[1]
+    two = subprocess.run([sys.executable, str(root / "bench.py"), "--gpus", "2"], capture_output=True, text=True, timeout=120)
+    assert two.returncode != 0 and "one GPU" in (two.stderr + two.stdout)
+    try:
+        from hipengine_amd.core.hip import get_hip_runtime
+        has_gpu = get_hip_runtime().device_count() > 0
+    except Exception:
+        has_gpu = False
+    if not has_gpu:
+        one = subprocess.run([sys.executable, str(root / "bench.py"), "--steps", "2", "--warmup", "1"], capture_output=True,
+                             text=True, timeout=120)
+        assert one.returncode != 0 and "metric" not in one.stdout
